@@ -1,0 +1,264 @@
+"""Lazy tensors: operations build a graph, `realize()` runs it on the default
+device.
+
+Host-side mirror of the reference's `src/tensor/`: `tensor.rs:58-160`
+(constructors), `ops.rs` (elementwise `:21-160`, reductions `:178-245`,
+views `:336-450`, `scale`/`ones_like`/`zeros_like` `:699-725`),
+`realize.rs` (`realize` `:134-247`, `to_vec` `:268-298`, `set_data`
+`:322-359`, constant buffers for nodes named ones/zeros/scalar `:391-421`).
+Reference behaviours kept as they are: `scale(f)` multiplies by a tensor of
+ones and ignores `f`; `mean` returns `sum`; `pow` is `exp(ln(x))`.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import graph as G
+from .ast import DType, F32
+from .device import allocate_buffer_on_default_device, has_default_device
+from .executor import ExecutionError, execute_graph
+
+_NP = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "i64": np.int64,
+       "u8": np.uint8, "bool": np.uint8, "i8": np.int8, "i16": np.int16,
+       "u16": np.uint16, "u32": np.uint32, "u64": np.uint64, "f16": np.float16}
+
+# set_data() registers buffers here so any graph that uses the input can find
+# them (INPUT_BUFFER_CACHE, realize.rs:30-31); values keep their node alive.
+_INPUT_BUFFER_CACHE: Dict[int, tuple] = {}
+
+
+class Tensor:
+    def __init__(self, graph: G.GraphNode):
+        self.graph = graph
+        self.buffer = None
+        self._requires_grad = False
+        self._grad: Optional["Tensor"] = None
+
+    # -- constructors -------------------------------------------------------
+    @staticmethod
+    def from_graph(graph: G.GraphNode) -> "Tensor":
+        return Tensor(graph)
+
+    @staticmethod
+    def input(shape: Sequence[int], dtype: DType = F32) -> "Tensor":
+        return Tensor(G.input(list(shape), dtype))
+
+    @staticmethod
+    def named_input(name: str, shape: Sequence[int], dtype: DType = F32) -> "Tensor":
+        return Tensor(G.named_input(name, list(shape), dtype))
+
+    @staticmethod
+    def zeros(shape, dtype: DType = F32) -> "Tensor":
+        return Tensor(G.zeros(list(shape), dtype))
+
+    @staticmethod
+    def ones(shape, dtype: DType = F32) -> "Tensor":
+        return Tensor(G.ones(list(shape), dtype))
+
+    @staticmethod
+    def ones_like(other: "Tensor") -> "Tensor":
+        return Tensor(G.ones(other.shape(), other.dtype()))
+
+    @staticmethod
+    def zeros_like(other: "Tensor") -> "Tensor":
+        return Tensor(G.zeros(other.shape(), other.dtype()))
+
+    @staticmethod
+    def from_numpy(arr: np.ndarray) -> "Tensor":
+        """Convenience: input + set_data (needs a default device)."""
+        dt = {v: k for k, v in _NP.items() if k != "bool"}[arr.dtype.type]
+        t = Tensor.input(arr.shape, DType(dt))
+        t.set_data(arr)
+        return t
+
+    # -- accessors ------------------------------------------------------------
+    def shape(self) -> List[int]:
+        return [int(e.evaluate()) for e in self.graph.shape()]
+
+    def ndim(self) -> int:
+        return self.graph.ndim()
+
+    def dtype(self) -> DType:
+        return self.graph.dtype
+
+    def numel(self) -> int:
+        n = 1
+        for s in self.shape():
+            n *= s
+        return n
+
+    def with_name(self, name: str) -> "Tensor":
+        return Tensor(self.graph.with_name(name))
+
+    # -- elementwise --------------------------------------------------------------
+    def add(self, o): return Tensor(self.graph + o.graph)
+    def mul(self, o): return Tensor(self.graph * o.graph)
+    def sub(self, o): return Tensor(self.graph - o.graph)
+    def div(self, o): return Tensor(self.graph / o.graph)
+    __add__, __mul__, __sub__, __truediv__ = add, mul, sub, div
+
+    def maximum(self, o): return Tensor(self.graph.maximum(o.graph))
+    def minimum(self, o): return Tensor(self.graph.minimum(o.graph))
+    def neg(self): return Tensor(-self.graph)
+    __neg__ = neg
+    def recip(self): return Tensor(self.graph.recip())
+    def sqrt(self): return Tensor(self.graph.sqrt())
+    def ln(self): return Tensor(self.graph.ln())
+    def log2(self): return Tensor(self.graph.log2())
+    def exp(self): return Tensor(self.graph.exp())
+    def exp2(self): return Tensor(self.graph.exp2())
+    def sin(self): return Tensor(self.graph.sin())
+    def cos(self): return Tensor(self.graph.cos())
+    def floor(self): return Tensor(self.graph.floor())
+    def abs(self): return Tensor(self.graph.abs())
+    def square(self): return self.mul(self)
+    def pow(self, _exp: float): return self.ln().exp()
+
+    def lt(self, o): return Tensor(self.graph.lt(o.graph))
+    def gt(self, o): return Tensor(self.graph.gt(o.graph))
+    def le(self, o): return Tensor(self.graph.le(o.graph))
+    def ge(self, o): return Tensor(self.graph.ge(o.graph))
+    def eq(self, o): return Tensor(self.graph.eq_node(o.graph))
+    def ne(self, o): return Tensor(self.graph.ne_node(o.graph))
+
+    def where_cond(self, cond, other):
+        return Tensor(self.graph.where_cond(cond.graph, other.graph))
+
+    def cast(self, dtype: DType): return Tensor(self.graph.cast(dtype))
+
+    def scale(self, _factor: float) -> "Tensor":
+        return self.mul(Tensor.ones_like(self))
+
+    # -- reductions (the reduced axis is squeezed away) ------------------------------
+    def _check_axis(self, axis):
+        if not 0 <= axis < self.ndim():
+            raise IndexError(f"Axis {axis} out of bounds for {self.ndim()}D tensor")
+
+    def sum(self, axis):
+        self._check_axis(axis)
+        return Tensor(self.graph.sum(axis).squeeze(axis))
+
+    def max(self, axis):
+        self._check_axis(axis)
+        return Tensor(self.graph.max(axis).squeeze(axis))
+
+    def min(self, axis):
+        self._check_axis(axis)
+        return Tensor(self.graph.min(axis).squeeze(axis))
+
+    def prod(self, axis):
+        self._check_axis(axis)
+        return Tensor(self.graph.prod(axis).squeeze(axis))
+
+    def mean(self, axis): return self.sum(axis)
+
+    def cumsum(self, axis): return Tensor(self.graph.cumsum(axis))
+    def cumprod(self, axis): return Tensor(self.graph.cumprod(axis))
+    def cummax(self, axis): return Tensor(self.graph.cummax(axis))
+
+    # -- views ---------------------------------------------------------------------------
+    def unsqueeze(self, axis): return Tensor(self.graph.unsqueeze(axis))
+    def squeeze(self, axis): return Tensor(self.graph.squeeze(axis))
+    def permute(self, axes): return Tensor(self.graph.permute(list(axes)))
+    def contiguous(self): return Tensor(self.graph.contiguous())
+    def expand(self, axis, size): return Tensor(self.graph.expand(axis, size))
+
+    def t(self):
+        n = self.ndim()
+        axes = list(range(n))
+        axes[n - 2], axes[n - 1] = axes[n - 1], axes[n - 2]
+        return self.permute(axes)
+
+    def reshape(self, shape):
+        n = 1
+        for s in shape:
+            n *= s
+        if n != self.numel():
+            raise ValueError(f"Cannot reshape tensor of {self.numel()} elements to {n} elements")
+        return Tensor(self.graph.reshape(list(shape)))
+
+    def flatten(self): return self.reshape([self.numel()])
+
+    def pad(self, padding): return Tensor(self.graph.pad(list(padding), "zero"))
+
+    def unfold(self, axes, sizes, strides, dilations):
+        return Tensor(self.graph.unfold(axes, sizes, strides, dilations))
+
+    def fold(self, output_shape, axes, sizes, strides, dilations):
+        return Tensor(self.graph.fold(output_shape, axes, sizes, strides, dilations))
+
+    # -- realisation -------------------------------------------------------------------------
+    def is_realized(self) -> bool:
+        return self.buffer is not None
+
+    def set_data(self, data) -> None:
+        if not has_default_device():
+            raise ExecutionError("NoDevice")
+        arr = np.ascontiguousarray(np.asarray(data, dtype=_NP[self.dtype().name]))
+        if arr.size != self.numel():
+            raise ExecutionError(f"ShapeMismatch: Data size {arr.size} doesn't match "
+                                 f"tensor size {self.numel()}")
+        buf = allocate_buffer_on_default_device(self.shape(), self.dtype())
+        buf.write_from_host(arr.tobytes())
+        _INPUT_BUFFER_CACHE[id(self.graph)] = (self.graph, buf.clone_buffer())
+        self.buffer = buf
+
+    def realize(self) -> "Tensor":
+        if self.is_realized():
+            return self
+        if not has_default_device():
+            raise ExecutionError("NoDevice")
+        g = self.graph
+        if g.is_external():
+            hit = _INPUT_BUFFER_CACHE.get(id(g))
+            if hit is None:
+                raise ExecutionError("MissingInput: Input tensor has no data. "
+                                     "Call set_data() first.")
+            self.buffer = hit[1].clone_buffer()
+            return self
+        input_buffers = {}
+        for node in G.collect_inputs([g]):
+            hit = _INPUT_BUFFER_CACHE.get(id(node))
+            if hit is not None:
+                input_buffers[id(node)] = hit[1].clone_buffer()
+                continue
+            const = _create_constant_buffer(node)
+            if const is None:
+                raise ExecutionError(f"MissingInput: Input tensor "
+                                     f"'{node.name or hex(id(node))}' has no data. "
+                                     f"Call set_data() first.")
+            input_buffers[id(node)] = const
+        res = execute_graph([g], input_buffers)
+        if not res or res[0] is None:
+            raise ExecutionError("Internal: No output buffer returned from execution")
+        self.buffer = res[0]
+        return self
+
+    def to_numpy(self) -> np.ndarray:
+        """Flat array of the buffer's elements (to_vec, realize.rs:268-298)."""
+        if not self.is_realized():
+            raise ExecutionError("NotRealized")
+        raw = self.buffer.read_to_host()
+        return np.frombuffer(raw, dtype=_NP[self.dtype().name]).copy()
+
+    def to_vec(self) -> list:
+        return self.to_numpy().tolist()
+
+    def clear_buffer(self) -> None:
+        self.buffer = None
+
+
+def _create_constant_buffer(node: G.GraphNode):
+    fill = {"ones": 1.0, "zeros": 0.0, "scalar": 1.0}.get(node.name)
+    if fill is None:
+        return None
+    shape = [int(e.evaluate()) for e in node.shape()]
+    buf = allocate_buffer_on_default_device(shape, node.dtype)
+    n = 1
+    for s in shape:
+        n *= s
+    buf.write_from_host(np.full(n, fill, dtype=_NP[node.dtype.name]).tobytes())
+    return buf
