@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the eclat kernel path on one MI355X.
+
+A step is one pass of the hot path (execute the compiled Program) over one batch
+of synthetic input.  The headline workload is BASELINE config 2 -- row softmax of
+fp32 [4096, 4096], compiled from the reference's five-kernel lowering into one
+fused launch -- reported as HBM GB/s of algorithmic traffic (one read + one
+write).  The same JSON line carries config 3 (4096^3 fp32 matmul, TFLOP/s on the
+FP32 MFMA schedule) and config 1 under "extra", a roofline object per dominant
+kernel, and the CPU baseline (the oracle's C kernels, unfused, on host cores).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--options key=value,...]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix peak
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build(dev, hb, wl, name, shapes, options):
+    inputs_fn, graph_fn = wl.CONFIGS[name]
+    prog_ast, arg_names, out_name, const_inputs, _ = wl.lower_with_table(shapes, graph_fn)
+    prog = hb.HipProgram(dev, prog_ast, options)
+    return prog, arg_names, out_name, const_inputs
+
+
+def make_sets(dev, hb, prog, arg_names, const_inputs, arrays, nsets):
+    """`nsets` independent bindings so consecutive steps do not re-read lines
+    the previous step left in the last-level cache."""
+    sets = []
+    for _ in range(nsets):
+        named = {}
+        for b in prog.buffers:
+            if b["elided"]:
+                continue
+            if b["role"] == "temp":
+                continue                   # kept by the program itself
+            hbuf = hb.HipBuffer(dev, [b["bytes"]], None, nbytes=b["bytes"])
+            if b["name"] in arg_names:
+                hbuf.write_array(np.ascontiguousarray(arrays[arg_names.index(b["name"])]))
+            elif b["name"] in const_inputs:
+                fill = {"ones": 1.0, "zeros": 0.0, "scalar": 1.0}[const_inputs[b["name"]]]
+                hbuf.write_array(np.full(b["bytes"] // 4, fill, dtype=np.float32))
+            named[b["name"]] = hbuf
+        sets.append((prog.bind(named), named))
+    return sets
+
+
+def time_steps(dev, hb, prog, sets, steps, warmup):
+    """W untimed steps, then exactly K steps between two events on the launch
+    stream, with a device sync on both sides.  Returns (event ms, wall ms) per step."""
+    for i in range(warmup):
+        prog.run(sets[i % len(sets)][0], sync=False)
+    dev.sync()
+    e0, e1 = hb.Event(dev), hb.Event(dev)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        prog.run(sets[i % len(sets)][0], sync=False)
+    e1.record()
+    e1.sync()
+    dev.sync()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_ms(e1) / steps, wall / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--options", default="")
+    ap.add_argument("--sets", type=int, default=4)
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 (default: all)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU (every kernel here works on one GPU's "
+                 "share at its real shape); run with --gpus 1")
+    if args.steps < 1 or args.warmup < 0:
+        sys.exit("bench.py: --steps must be >= 1 and --warmup >= 0")
+
+    from harp_amd import backend as hb
+    from harp_amd import workloads as wl
+    if hb.device_count() == 0:
+        sys.exit("bench.py: no HIP device present; the HIP backend has no CPU path")
+    dev = hb.HipDevice(0)
+    props = dev.props
+    log(f"[bench] device: {props['name']} {props['arch']} CUs={props['compute_units']} "
+        f"clock={props['clock_khz'] / 1e6:.2f} GHz LDS/CU={props['local_memory_size']}")
+    options = args.options or None
+    want = lambda n: not args.only or args.only == n
+    result_extra = {}
+
+    # ---- config 2: row softmax 4096 x 4096 (headline) --------------------------------
+    softmax = None
+    if want("softmax"):
+        shapes = [(4096, 4096)]
+        arrays = wl.config2_inputs()
+        prog, arg_names, out_name, consts = build(dev, hb, wl, "config2_softmax", shapes, options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
+        ms, wall_ms = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
+        algo = sum(l["algo_bytes"] for l in prog.launches)
+        softmax = {"ms": ms, "wall_ms": wall_ms, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
+                   "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
+        log(f"[bench] softmax 4096^2: {ms * 1e3:.1f} us/step -> {softmax['gbs']:.0f} GB/s "
+            f"({softmax['gbs'] / HBM_PEAK_GBS:.1%} of 8 TB/s); {softmax['launches']}")
+        if not args.no_check:
+            got = sets[0][1][out_name].read_array(np.float32, (4096, 4096))
+            x = arrays[0].astype(np.float64)
+            e = np.exp(x[:64] - x[:64].max(1, keepdims=True))
+            assert np.allclose(got[:64], e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12), \
+                "softmax result check failed"
+            assert np.allclose(got.sum(1), 1.0, atol=1e-5), "softmax rows do not sum to 1"
+        del sets
+
+    # ---- config 3: 4096^3 fp32 matmul --------------------------------------------------
+    matmul = None
+    if want("matmul"):
+        shapes = [(4096, 4096), (4096, 4096)]
+        arrays = wl.config3_inputs()
+        prog, arg_names, out_name, consts = build(dev, hb, wl, "config3_matmul", shapes, options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 2)
+        k = max(5, min(args.steps, 50))
+        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 5))
+        flops = sum(l["flops"] for l in prog.launches)
+        matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k,
+                  "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
+        log(f"[bench] matmul 4096^3: {ms:.3f} ms/step -> {matmul['tflops']:.1f} TFLOP/s "
+            f"({matmul['tflops'] / FP32_MFMA_PEAK_TFLOPS:.1%} of FP32 MFMA peak); {matmul['launches']}")
+        if not args.no_check:
+            got = sets[0][1][out_name].read_array(np.float32, (4096, 4096))
+            a, b = arrays
+            ref = a[:32].astype(np.float64) @ b.astype(np.float64)
+            scale = np.abs(a[:32]).astype(np.float64) @ np.abs(b).astype(np.float64)
+            assert np.all(np.abs(got[:32] - ref) <= 1e-3 * scale), "matmul result check failed"
+        del sets
+
+    # ---- config 1: fused elementwise + reduce, 1024 x 1024 ------------------------------
+    cfg1 = None
+    if want("config1"):
+        shapes = [(1024, 1024)] * 3
+        arrays = wl.config1_inputs()
+        prog, arg_names, out_name, consts = build(dev, hb, wl, "config1_relu_sum", shapes, options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
+        ms, _ = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
+        algo = sum(l["algo_bytes"] for l in prog.launches)
+        cfg1 = {"us": ms * 1e3, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
+                "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
+        log(f"[bench] config1 relu-sum 1024^2: {cfg1['us']:.1f} us/step -> {cfg1['gbs']:.0f} GB/s")
+        del sets
+
+    # ---- CPU baseline: the oracle's unfused C kernels on host cores -------------------------
+    cpu = None
+    if not args.no_cpu_baseline and softmax is not None:
+        from oracle import baseline
+        arrays = wl.config2_inputs()
+        sec, reps, _ = baseline.time_graph(wl.config2_graph, arrays, min_seconds=8.0, max_reps=40)
+        cpu = {"value": softmax["algo_bytes"] / sec / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": f"full 4096x4096 softmax, unfused R,E,E,R,E kernels (gcc -O3 -ffast-math), "
+                         f"median of {reps} passes, {sec * 1e3:.0f} ms/pass"}
+        log(f"[bench] cpu baseline softmax: {sec * 1e3:.0f} ms/pass -> {cpu['value']:.2f} GB/s (1 core)")
+        if matmul is not None:
+            a, b = wl.config3_inputs()
+            sub = 8
+            sec_m, reps_m, _ = baseline.time_graph(wl.config3_graph, [a[:sub].copy(), b],
+                                                   min_seconds=4.0, max_reps=10)
+            gflops = 2.0 * sub * 4096 * 4096 / sec_m / 1e9
+            result_extra["cpu_baseline_matmul"] = {
+                "value": gflops / 1e3, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": f"{sub} of 4096 rows of A through the reference's ijk kernel "
+                          f"(gcc -O3 -ffast-math), median of {reps_m} passes, {sec_m * 1e3:.0f} ms/pass"}
+            log(f"[bench] cpu baseline matmul: {gflops:.2f} GFLOP/s (1 core, {sub}-row sample)")
+
+    head = softmax
+    out = {
+        "metric": "fused-kernel HBM GB/s (softmax 4096^2)" + (" + fp32 matmul TFLOP/s (4096^3)" if matmul else ""),
+        "value": round(head["gbs"], 1) if head else None,
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["ms"], 6) if head else None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic (seeded N(0, std 2) fp32 [4096,4096])",
+        "config": {"workload": "config2: row softmax fp32 [4096,4096], one fused launch",
+                   "buffer_sets": args.sets, "options": args.options},
+    }
+    if head:
+        out["roofline"] = {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
+                           "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                           "kernel": head["launches"][0][0], "schedule": head["launches"][0][1]}
+    if cpu:
+        out["cpu_baseline"] = cpu
+    if matmul:
+        result_extra["matmul_4096"] = {
+            "value": round(matmul["tflops"], 2), "unit": "TFLOP/s", "ms_per_step": round(matmul["ms"], 4),
+            "steps": matmul["steps"], "dtype": "f32",
+            "roofline": {"bound": "mfma", "achieved": round(matmul["tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(matmul["tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
+                         "traffic": None, "kernel": matmul["launches"][0][0],
+                         "schedule": matmul["launches"][0][1]}}
+    if cfg1:
+        result_extra["config1_relu_sum_1024"] = {"us_per_step": round(cfg1["us"], 2),
+                                                 "value": round(cfg1["gbs"], 1), "unit": "GB/s",
+                                                 "schedule": cfg1["launches"][0][1]}
+    result_extra["device"] = {"name": props["name"], "arch": props["arch"],
+                              "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
+    out["extra"] = result_extra
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

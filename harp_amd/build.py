@@ -1,0 +1,93 @@
+"""Builds libeclat_hip.so in-tree: wraps the kernel templates into string
+literals, compiles the host C++ with hipcc (host pass only; device code is
+generated at run time and compiled by hiprtc), and checks that each kernel
+template also compiles for gfx950 on its own.
+
+    python -m harp_amd.build            # build the library
+    python -m harp_amd.build --check    # additionally hipcc-compile the templates for gfx950
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libeclat_hip.so")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+SOURCES = ["ast.cpp", "analysis.cpp", "codegen.cpp", "gemm.cpp", "backend.cpp", "capi.cpp"]
+TEMPLATES = ["kernels/gemm_f32_mfma.hip"]
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-ffp-contract=off",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
+    return r
+
+
+def wrap_templates() -> None:
+    for t in TEMPLATES:
+        src = os.path.join(CSRC, t)
+        with open(src) as f:
+            text = f.read()
+        if ')EHK"' in text:
+            raise RuntimeError(f"{t} contains the raw-string terminator")
+        out = src + ".inc"
+        new = 'R"EHK(' + text + ')EHK"\n'
+        old = open(out).read() if os.path.exists(out) else None
+        if old != new:
+            with open(out, "w") as f:
+                f.write(new)
+
+
+def check_templates() -> None:
+    """Device compile of every template with its default parameters."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    with tempfile.TemporaryDirectory() as tmp:
+        for t in TEMPLATES:
+            out = os.path.join(tmp, os.path.basename(t) + ".hsaco")
+            _run([hipcc, "--genco"] + DEVICE_FLAGS + ["-o", out, os.path.join(CSRC, t)])
+
+
+def build(check: bool = False, force: bool = True) -> str:
+    wrap_templates()
+    srcs = [os.path.join(CSRC, s) for s in SOURCES]
+    if not force and os.path.exists(LIB):
+        newest = max(os.path.getmtime(p) for p in srcs + [os.path.join(CSRC, t) for t in TEMPLATES]
+                     + [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".hpp")])
+        if os.path.getmtime(LIB) >= newest:
+            return LIB
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    objs = []
+    with tempfile.TemporaryDirectory() as tmp:
+        procs = []
+        for s in srcs:
+            o = os.path.join(tmp, os.path.basename(s) + ".o")
+            objs.append(o)
+            cmd = [hipcc, "-x", "c++", "-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra",
+                   "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(ROCM, "include"),
+                   "-c", s, "-o", o]
+            procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE,
+                                                stderr=subprocess.PIPE, text=True)))
+        for cmd, p in procs:
+            out, err = p.communicate()
+            if p.returncode != 0:
+                raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), out, err))
+            if err.strip():
+                sys.stderr.write(err)
+        _run([hipcc, "-shared", "-o", LIB] + objs +
+             ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lhiprtc",
+              "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    if check:
+        check_templates()
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(check="--check" in sys.argv))

@@ -1,0 +1,405 @@
+#include "backend.hpp"
+
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+#include <unordered_map>
+
+namespace eh {
+
+namespace {
+
+void check(hipError_t e, const char* what) {
+  if (e != hipSuccess)
+    throw Error(std::string(what) + ": " + hipGetErrorString(e) + " (hip error " + std::to_string(static_cast<int>(e)) + ")");
+}
+
+uint64_t fnv1a(const std::string& s, uint64_t h) {
+  for (unsigned char c : s) {
+    h ^= c;
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+std::string hash_hex(const std::string& s) {
+  char buf[40];
+  snprintf(buf, sizeof buf, "%016llx%016llx", static_cast<unsigned long long>(fnv1a(s, 14695981039346656037ull)),
+           static_cast<unsigned long long>(fnv1a(s, 0x9e3779b97f4a7c15ull)));
+  return buf;
+}
+
+void mkdirs(const std::string& path) {
+  std::string cur;
+  for (size_t i = 0; i < path.size(); ++i) {
+    cur += path[i];
+    if (path[i] == '/' || i + 1 == path.size()) ::mkdir(cur.c_str(), 0755);
+  }
+}
+
+std::mutex g_bin_mu;
+std::unordered_map<std::string, std::shared_ptr<Binary>> g_bin_cache;
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// HipCompiler
+// ---------------------------------------------------------------------------------------------
+
+std::vector<std::string> HipCompiler::options(const std::string& arch) {
+  // fp-contract off: `a*b` followed by `+c` in separate graph nodes must round twice, as the C
+  // backend's output does.  The target feature keeps packed-fp32 instructions out of the code.
+  return {"--offload-arch=" + arch, "-O3", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops"};
+}
+
+bool HipCompiler::disk_cache_enabled() { return std::getenv("HARP_NO_DISK_CACHE") == nullptr; }
+
+std::string HipCompiler::cache_dir() {
+  std::string base;
+  if (const char* d = std::getenv("HARP_CACHE_DIR")) base = d;
+  else if (const char* h = std::getenv("HOME")) base = std::string(h) + "/.cache/harp";
+  else base = "/tmp/harp-cache";
+  return base + "/kernels/Hip";
+}
+
+Binary HipCompiler::compile(const std::string& source, const std::string& arch, bool use_disk_cache) {
+  std::vector<std::string> opts = options(arch);
+  int maj = 0, min = 0;
+  hiprtcVersion(&maj, &min);
+  std::string key_text = source;
+  for (const auto& o : opts) key_text += "\n" + o;
+  key_text += "\nhiprtc " + std::to_string(maj) + "." + std::to_string(min);
+  const std::string key = hash_hex(key_text);
+  {
+    std::lock_guard<std::mutex> lk(g_bin_mu);
+    auto it = g_bin_cache.find(key);
+    if (it != g_bin_cache.end()) return *it->second;
+  }
+  const bool disk = use_disk_cache && disk_cache_enabled();
+  const std::string path = cache_dir() + "/" + key + ".bin";
+  Binary out;
+  if (disk) {
+    std::ifstream f(path, std::ios::binary);
+    if (f) {
+      out.code.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+      out.from_cache = !out.code.empty();
+    }
+  }
+  if (!out.from_cache) {
+    hiprtcProgram prog;
+    if (hiprtcCreateProgram(&prog, source.c_str(), "eclat_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+      throw Error("hiprtcCreateProgram failed");
+    std::vector<const char*> copts;
+    for (const auto& o : opts) copts.push_back(o.c_str());
+    hiprtcResult r = hiprtcCompileProgram(prog, static_cast<int>(copts.size()), copts.data());
+    size_t ls = 0;
+    hiprtcGetProgramLogSize(prog, &ls);
+    if (ls > 1) {
+      out.log.resize(ls);
+      hiprtcGetProgramLog(prog, &out.log[0]);
+    }
+    if (r != HIPRTC_SUCCESS) {
+      hiprtcDestroyProgram(&prog);
+      throw Error(std::string("hiprtc compilation failed: ") + hiprtcGetErrorString(r) + "\n" + out.log);
+    }
+    size_t cs = 0;
+    hiprtcGetCodeSize(prog, &cs);
+    out.code.resize(cs);
+    hiprtcGetCode(prog, out.code.data());
+    hiprtcDestroyProgram(&prog);
+    if (disk) {
+      mkdirs(cache_dir());
+      const std::string tmp = path + ".tmp" + std::to_string(reinterpret_cast<uintptr_t>(&out) & 0xffff);
+      std::ofstream f(tmp, std::ios::binary);
+      if (f) {
+        f.write(out.code.data(), static_cast<std::streamsize>(out.code.size()));
+        f.close();
+        std::rename(tmp.c_str(), path.c_str());
+        std::ofstream meta(cache_dir() + "/" + key + ".json");
+        meta << "{\"arch\": \"" << arch << "\", \"hiprtc\": \"" << maj << "." << min << "\", \"bytes\": "
+             << out.code.size() << "}\n";
+      }
+    }
+  }
+  {
+    std::lock_guard<std::mutex> lk(g_bin_mu);
+    g_bin_cache[key] = std::make_shared<Binary>(out);
+  }
+  return out;
+}
+
+// ---------------------------------------------------------------------------------------------
+// HipDevice / HipBuffer / HipKernel
+// ---------------------------------------------------------------------------------------------
+
+int HipDevice::count() {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+HipDevice::HipDevice(int index) : index_(index) {
+  int n = count();
+  if (n == 0) throw Error("no HIP device is present (hipGetDeviceCount found none)");
+  if (index < 0 || index >= n)
+    throw Error("device index " + std::to_string(index) + " out of range (" + std::to_string(n) + " device(s))");
+  check(hipSetDevice(index), "hipSetDevice");
+  hipDeviceProp_t p;
+  check(hipGetDeviceProperties(&p, index), "hipGetDeviceProperties");
+  profile_.name = p.name;
+  profile_.arch = p.gcnArchName;
+  profile_.arch = profile_.arch.substr(0, profile_.arch.find(':'));
+  profile_.compute_units = p.multiProcessorCount;
+  profile_.warp_size = p.warpSize;
+  profile_.max_work_group_size = p.maxThreadsPerBlock;
+  profile_.local_memory_size = p.maxSharedMemoryPerMultiProcessor ? p.maxSharedMemoryPerMultiProcessor : p.sharedMemPerBlock;
+  profile_.global_memory_size = p.totalGlobalMem;
+  profile_.clock_khz = p.clockRate;
+  profile_.memory_clock_khz = p.memoryClockRate;
+  profile_.memory_bus_bits = p.memoryBusWidth;
+  profile_.l2_bytes = p.l2CacheSize;
+  check(hipStreamCreate(&stream_), "hipStreamCreate");
+}
+
+HipDevice::~HipDevice() {
+  if (stream_) {
+    (void)hipSetDevice(index_);
+    (void)hipStreamSynchronize(stream_);
+    (void)hipStreamDestroy(stream_);
+  }
+}
+
+void HipDevice::make_current() const { check(hipSetDevice(index_), "hipSetDevice"); }
+
+void HipDevice::synchronize() const {
+  make_current();
+  check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+}
+
+std::shared_ptr<HipKernel> HipDevice::load(const Binary& bin, const std::string& entry) {
+  return std::make_shared<HipKernel>(this, bin, entry);
+}
+
+HipBuffer::HipBuffer(HipDevice* dev, size_t bytes) : dev_(dev), bytes_(bytes) {
+  dev_->make_current();
+  if (bytes_ == 0) return;
+  check(hipMalloc(&ptr_, bytes_), "hipMalloc");
+  hipError_t e = hipMemsetAsync(ptr_, 0, bytes_, dev_->stream());
+  if (e != hipSuccess) {
+    (void)hipFree(ptr_);
+    check(e, "hipMemsetAsync");
+  }
+}
+
+HipBuffer::~HipBuffer() {
+  if (ptr_) {
+    (void)hipSetDevice(dev_->index());
+    (void)hipStreamSynchronize(dev_->stream());
+    (void)hipFree(ptr_);
+  }
+}
+
+void HipBuffer::write_from_host(const void* src, size_t bytes) {
+  if (bytes != bytes_)
+    throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(bytes));
+  if (!bytes_) return;
+  dev_->make_current();
+  check(hipMemcpyAsync(ptr_, src, bytes_, hipMemcpyHostToDevice, dev_->stream()), "hipMemcpyAsync(H2D)");
+  check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
+}
+
+void HipBuffer::read_to_host(void* dst, size_t bytes) const {
+  if (bytes != bytes_)
+    throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(bytes));
+  if (!bytes_) return;
+  dev_->make_current();
+  check(hipMemcpyAsync(dst, ptr_, bytes_, hipMemcpyDeviceToHost, dev_->stream()), "hipMemcpyAsync(D2H)");
+  check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
+}
+
+void HipBuffer::copy_from(const HipBuffer& src) {
+  if (src.bytes_ != bytes_)
+    throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(src.bytes_));
+  if (!bytes_) return;
+  dev_->make_current();
+  check(hipMemcpyAsync(ptr_, src.ptr_, bytes_, hipMemcpyDeviceToDevice, dev_->stream()), "hipMemcpyAsync(D2D)");
+}
+
+HipKernel::HipKernel(HipDevice* dev, const Binary& bin, const std::string& entry)
+    : dev_(dev), binary_(bin.code), entry_(entry) {
+  dev_->make_current();
+  check(hipModuleLoadData(&module_, binary_.data()), "hipModuleLoadData");
+  hipError_t e = hipModuleGetFunction(&fn_, module_, entry.c_str());
+  if (e != hipSuccess) {
+    (void)hipModuleUnload(module_);
+    module_ = nullptr;
+    throw Error("entry point '" + entry + "' not found in the code object: " + hipGetErrorString(e));
+  }
+}
+
+HipKernel::~HipKernel() {
+  if (module_) {
+    (void)hipSetDevice(dev_->index());
+    (void)hipStreamSynchronize(dev_->stream());
+    (void)hipModuleUnload(module_);
+  }
+}
+
+void HipKernel::launch(const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
+                       const std::vector<void*>& device_ptrs) const {
+  std::vector<void*> vals = device_ptrs;
+  std::vector<void*> params(vals.size());
+  for (size_t i = 0; i < vals.size(); ++i) params[i] = &vals[i];
+  check(hipModuleLaunchKernel(fn_, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, dev_->stream(),
+                              params.data(), nullptr),
+        ("launch of " + entry_).c_str());
+}
+
+// ---------------------------------------------------------------------------------------------
+// HipProgram
+// ---------------------------------------------------------------------------------------------
+
+GenOptions parse_options(const char* text) {
+  GenOptions o;
+  if (const char* env = std::getenv("ECLAT_HIP_ARCH")) o.arch = env;
+  if (!text) return o;
+  std::stringstream ss(text);
+  std::string item;
+  while (std::getline(ss, item, ',')) {
+    if (item.empty()) continue;
+    size_t eq = item.find('=');
+    if (eq == std::string::npos) throw Error("option '" + item + "' is not key=value");
+    std::string k = item.substr(0, eq), v = item.substr(eq + 1);
+    auto as_int = [&]() {
+      try {
+        return std::stoi(v);
+      } catch (const std::logic_error&) {
+        throw Error("option '" + k + "' needs an integer, got '" + v + "'");
+      }
+    };
+    if (k == "arch") o.arch = v;
+    else if (k == "fuse") o.fuse = as_int() != 0;
+    else if (k == "vectorize") o.vectorize = as_int() != 0;
+    else if (k == "row_threads") o.row_threads = as_int();
+    else if (k == "row_elems") o.row_elems = std::max(1, as_int());
+    else if (k == "flat_block") o.flat_block = as_int();
+    else if (k == "flat_iters") o.flat_iters = std::max(1, as_int());
+    else if (k == "gemm") o.gemm = as_int() != 0;
+    else if (k == "gemm_bm") o.gemm_bm = as_int();
+    else if (k == "gemm_bn") o.gemm_bn = as_int();
+    else if (k == "gemm_bk") o.gemm_bk = as_int();
+    else if (k == "gemm_wm") o.gemm_wm = as_int();
+    else if (k == "gemm_wn") o.gemm_wn = as_int();
+    else if (k == "nontemporal") o.nontemporal = as_int() != 0;
+    else throw Error("unknown option '" + k + "'");
+  }
+  if (o.flat_block < 64 || o.flat_block > 1024 || (o.flat_block & (o.flat_block - 1)))
+    throw Error("flat_block must be a power of two in [64, 1024]");
+  if (o.row_threads < 0 || o.row_threads > 1024 || (o.row_threads & (o.row_threads - 1)))
+    throw Error("row_threads must be 0 or a power of two up to 1024");
+  return o;
+}
+
+HipProgram::HipProgram(HipDevice* dev, const std::string& ast_text, const GenOptions& opt) : dev_(dev) {
+  NodePtr ast = parse_ast(ast_text);
+  if (ast->op == Op::Kernel) ast = make(Op::Program, {ast});
+  GenOptions o = opt;
+  if (dev_->profile().arch.rfind("gfx", 0) == 0) o.arch = dev_->profile().arch;
+  plan_ = plan_program(*ast, o);
+  for (size_t i = 0; i < plan_.buffers.size(); ++i) index_[plan_.buffers[i].name] = i;
+  temps_.assign(plan_.buffers.size(), nullptr);
+  for (const auto& ls : plan_.launches) {
+    for (const auto& a : ls.arg_bufs)
+      if (!index_.count(a)) throw Error("launch '" + ls.entry + "' binds unknown buffer '" + a + "'");
+    Binary bin = HipCompiler::compile(ls.source, o.arch);
+    kernels_.push_back(dev_->load(bin, ls.entry));
+  }
+}
+
+HipProgram::~HipProgram() {
+  for (HipBuffer* b : temps_)
+    if (b && b->release()) delete b;
+}
+
+void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
+  if (n != plan_.buffers.size())
+    throw Error("program binds " + std::to_string(plan_.buffers.size()) + " buffers, " + std::to_string(n) + " given");
+  std::lock_guard<std::mutex> lk(mu_);
+  dev_->make_current();
+  std::vector<HipBuffer*> bound(n, nullptr);
+  for (size_t i = 0; i < n; ++i) {
+    const BufferInfo& bi = plan_.buffers[i];
+    if (plan_.elided.count(bi.name)) continue;
+    HipBuffer* b = bufs[i];
+    if (!b) {
+      if (bi.role != "temp")
+        throw Error("MissingInput: buffer '" + bi.name + "' (" + bi.role + ") was not provided");
+      if (!temps_[i]) temps_[i] = new HipBuffer(dev_, bi.bytes());
+      b = temps_[i];
+    }
+    if (b->device() != dev_) throw Error("buffer '" + bi.name + "' lives on another device");
+    if (!bi.shape.empty() || bi.role == "temp") {
+      if (b->byte_len() < bi.bytes())
+        throw Error("Buffer size mismatch: '" + bi.name + "' needs " + std::to_string(bi.bytes()) + " bytes, has " +
+                    std::to_string(b->byte_len()));
+    }
+    bound[i] = b;
+  }
+  for (size_t l = 0; l < plan_.launches.size(); ++l) {
+    const LaunchSpec& ls = plan_.launches[l];
+    std::vector<void*> ptrs;
+    for (size_t a = 0; a < ls.arg_bufs.size(); ++a) {
+      size_t bi = index_.at(ls.arg_bufs[a]);
+      HipBuffer* b = bound[bi];
+      if (!b) throw Error("launch '" + ls.entry + "' needs buffer '" + ls.arg_bufs[a] + "', which is not bound");
+      if (a < ls.arg_min_bytes.size() && b->byte_len() < ls.arg_min_bytes[a])
+        throw Error("Buffer size mismatch: '" + ls.arg_bufs[a] + "' needs at least " +
+                    std::to_string(ls.arg_min_bytes[a]) + " bytes for '" + ls.entry + "', has " +
+                    std::to_string(b->byte_len()));
+      ptrs.push_back(b->device_ptr());
+    }
+    kernels_[l]->launch(ls.grid, ls.block, ls.lds_bytes, ptrs);
+  }
+  if (sync) dev_->synchronize();
+}
+
+void HipProgram::execute_positional(HipBuffer* const* inputs, size_t n_in, HipBuffer* const* outputs, size_t n_out,
+                                    bool sync) {
+  std::vector<HipBuffer*> bufs(plan_.buffers.size(), nullptr);
+  size_t ii = 0, oi = 0;
+  for (size_t i = 0; i < plan_.buffers.size(); ++i) {
+    const std::string& role = plan_.buffers[i].role;
+    if (role == "input") {
+      if (ii >= n_in) throw Error("kernel takes more inputs than the " + std::to_string(n_in) + " given");
+      bufs[i] = inputs[ii++];
+    } else if (role == "output") {
+      if (oi >= n_out) throw Error("kernel takes more outputs than the " + std::to_string(n_out) + " given");
+      bufs[i] = outputs[oi++];
+    }
+  }
+  if (ii != n_in || oi != n_out)
+    throw Error("kernel takes " + std::to_string(ii) + " inputs and " + std::to_string(oi) + " outputs, got " +
+                std::to_string(n_in) + " and " + std::to_string(n_out));
+  execute(bufs.data(), bufs.size(), sync);
+}
+
+std::vector<std::string> HipBackendRegistry::list_devices() {
+  std::vector<std::string> out;
+  int n = HipDevice::count();
+  for (int i = 0; i < n; ++i) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, i) == hipSuccess) out.push_back(std::string(p.name) + " (" + p.gcnArchName + ")");
+  }
+  return out;
+}
+
+}  // namespace eh

@@ -1,0 +1,147 @@
+// The backend proper: device, buffers, compiler, kernels, registry -- the C++ counterparts of
+// the traits a reference backend crate implements (src/backend/traits.rs: Device :273-306,
+// Buffer :455-482, Kernel :531-587, Compiler :592-607; src/backend/device.rs:83-171
+// BackendRegistry), shaped after crates/backend-c/src/{device,buffer,compiler,kernel,lib}.rs.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <atomic>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "ast.hpp"
+#include "codegen.hpp"
+
+namespace eh {
+
+struct DeviceProfile {
+  std::string name, arch;
+  int compute_units = 0, warp_size = 64, max_work_group_size = 1024;
+  size_t local_memory_size = 0, global_memory_size = 0;
+  int clock_khz = 0, memory_clock_khz = 0, memory_bus_bits = 0, l2_bytes = 0;
+};
+
+class HipKernel;
+
+// Code object produced by hiprtc (or read back from the disk cache).
+struct Binary {
+  std::vector<char> code;
+  std::string log;
+  bool from_cache = false;
+};
+
+class HipCompiler {
+ public:
+  // HIP C -> gfx950 code object.  Needs no device.  Throws eh::Error carrying the hiprtc log.
+  static Binary compile(const std::string& source, const std::string& arch, bool use_disk_cache = true);
+  static std::vector<std::string> options(const std::string& arch);
+  static std::string cache_dir();      // HARP_CACHE_DIR or ~/.cache/harp, + /kernels/Hip
+  static bool disk_cache_enabled();    // HARP_NO_DISK_CACHE unset
+};
+
+class HipDevice {
+ public:
+  static int count();                  // 0 when no GPU/driver is present
+  static bool is_available() { return count() > 0; }
+  explicit HipDevice(int index);
+  ~HipDevice();
+  HipDevice(const HipDevice&) = delete;
+  HipDevice& operator=(const HipDevice&) = delete;
+
+  int index() const { return index_; }
+  hipStream_t stream() const { return stream_; }
+  const DeviceProfile& profile() const { return profile_; }
+  void make_current() const;
+  void synchronize() const;
+
+  // Loads a code object and resolves one entry point; modules are shared per (binary, entry).
+  std::shared_ptr<HipKernel> load(const Binary& bin, const std::string& entry);
+
+ private:
+  int index_;
+  hipStream_t stream_ = nullptr;
+  DeviceProfile profile_;
+};
+
+class HipBuffer {
+ public:
+  HipBuffer(HipDevice* dev, size_t bytes);   // zero-filled, as the reference's buffers are
+  ~HipBuffer();
+  HipBuffer(const HipBuffer&) = delete;
+  HipBuffer& operator=(const HipBuffer&) = delete;
+
+  size_t byte_len() const { return bytes_; }
+  void* device_ptr() const { return ptr_; }
+  HipDevice* device() const { return dev_; }
+  void write_from_host(const void* src, size_t bytes);   // size must match exactly
+  void read_to_host(void* dst, size_t bytes) const;
+  void copy_from(const HipBuffer& src);                   // clone_buffer
+  void retain() { refs_.fetch_add(1); }
+  bool release() { return refs_.fetch_sub(1) == 1; }      // true when the last reference went
+
+ private:
+  HipDevice* dev_;
+  void* ptr_ = nullptr;
+  size_t bytes_;
+  std::atomic<int> refs_{1};
+};
+
+// One loaded entry point.
+class HipKernel {
+ public:
+  HipKernel(HipDevice* dev, const Binary& bin, const std::string& entry);
+  ~HipKernel();
+  void launch(const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
+              const std::vector<void*>& device_ptrs) const;
+  const std::vector<char>& binary() const { return binary_; }   // Kernel::get_binary
+  const std::string& entry() const { return entry_; }
+
+ private:
+  HipDevice* dev_;
+  hipModule_t module_ = nullptr;
+  hipFunction_t fn_ = nullptr;
+  std::vector<char> binary_;
+  std::string entry_;
+};
+
+// A Program compiled for a device: the launches in order plus the buffers they bind.
+class HipProgram {
+ public:
+  HipProgram(HipDevice* dev, const std::string& ast_text, const GenOptions& opt);
+  ~HipProgram();
+
+  const ProgramPlan& plan() const { return plan_; }
+  // `bufs[i]` binds plan().buffers[i]; entries for elided buffers are ignored, missing temps are
+  // allocated once and kept.  Launches go to the device's stream; `sync` waits for them.
+  void execute(HipBuffer* const* bufs, size_t n, bool sync);
+  // Positional form (Kernel::execute): immutable pointer parameters, then mutable ones.
+  void execute_positional(HipBuffer* const* inputs, size_t n_in, HipBuffer* const* outputs, size_t n_out, bool sync);
+  const HipKernel& kernel(size_t launch) const { return *kernels_.at(launch); }
+  HipDevice* device() const { return dev_; }
+
+ private:
+  HipDevice* dev_;
+  ProgramPlan plan_;
+  std::vector<std::shared_ptr<HipKernel>> kernels_;
+  std::map<std::string, size_t> index_;          // buffer name -> table index
+  std::vector<HipBuffer*> temps_;                // owned, by table index (nullptr if unused)
+  std::mutex mu_;
+};
+
+GenOptions parse_options(const char* text);       // "key=value,key=value" -> GenOptions
+
+class HipBackendRegistry {
+ public:
+  static const char* kind() { return "hip"; }
+  static const char* name() { return "HIP (gfx950)"; }
+  static bool is_available() { return HipDevice::is_available(); }
+  static bool supports_runtime() { return true; }
+  static bool supports_binary_cache() { return true; }
+  static std::vector<std::string> list_devices();
+};
+
+}  // namespace eh

@@ -1,0 +1,1154 @@
+#include "codegen.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <sstream>
+
+#include "gemm.hpp"
+
+namespace eh {
+
+// ---------------------------------------------------------------------------------------------
+// preamble shared by every generated translation unit
+// ---------------------------------------------------------------------------------------------
+
+const std::string& preamble() {
+  static const std::string s = R"EHP(
+// wave64 helpers for gfx950
+template <typename T> struct alignas(sizeof(T) * 4) EhV4 { T v[4]; };
+
+struct EhSum  { template <class T> __device__ __forceinline__ static T f(T a, T b) { return a + b; } };
+struct EhProd { template <class T> __device__ __forceinline__ static T f(T a, T b) { return a * b; } };
+struct EhMax {
+  __device__ __forceinline__ static float f(float a, float b) { return fmaxf(a, b); }
+  __device__ __forceinline__ static double f(double a, double b) { return fmax(a, b); }
+  template <class T> __device__ __forceinline__ static T f(T a, T b) { return a > b ? a : b; }
+};
+struct EhMin { template <class T> __device__ __forceinline__ static T f(T a, T b) { return a < b ? a : b; } };
+
+template <int CTRL> __device__ __forceinline__ float eh_dpp(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+// Combines W adjacent lanes (W a power of two, at most 64); every lane of a group ends with
+// the group's result.  fp32: DPP quad permutes and row mirrors inside a row of 16 lanes,
+// ds_swizzle across rows, readlane across the two halves of the wave.
+template <class Op, int W> __device__ __forceinline__ float eh_lanes_reduce(float v) {
+  if (W >= 2) v = Op::f(v, eh_dpp<0xB1>(v));    // quad_perm [1,0,3,2]
+  if (W >= 4) v = Op::f(v, eh_dpp<0x4E>(v));    // quad_perm [2,3,0,1]
+  if (W >= 8) v = Op::f(v, eh_dpp<0x141>(v));   // row_half_mirror
+  if (W >= 16) v = Op::f(v, eh_dpp<0x140>(v));  // row_mirror
+  if (W >= 32) v = Op::f(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));
+  if (W >= 64) {
+    float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    v = Op::f(lo, hi);
+  }
+  return v;
+}
+template <class Op, int W, class T> __device__ __forceinline__ T eh_lanes_reduce(T v) {
+#pragma unroll
+  for (int m = 1; m < W; m <<= 1) v = Op::f(v, __shfl_xor(v, m, 64));
+  return v;
+}
+
+// Reduction over the T threads that share a row.  T <= 64: lanes only.  T > 64: one row per
+// workgroup, per-wave partials staged through LDS (one slot array per reduction, one barrier).
+template <class Op, int T, class V> __device__ __forceinline__ V eh_row_reduce(V v, V* lds, int lr) {
+  if (T <= 64) return eh_lanes_reduce<Op, T>(v);
+  v = eh_lanes_reduce<Op, 64>(v);
+  constexpr int NW = T / 64 > 0 ? T / 64 : 1;
+  if ((lr & 63) == 0) lds[lr >> 6] = v;
+  __syncthreads();
+  V r = lds[0];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) r = Op::f(r, lds[w]);
+  return r;
+}
+)EHP";
+  return s;
+}
+
+// ---------------------------------------------------------------------------------------------
+// types and literals
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+std::string ctype(const DType& d) {
+  switch (d.ty) {
+    case Ty::Void: return "void";
+    case Ty::Bool: case Ty::U8: return "unsigned char";
+    case Ty::I8: return "signed char";
+    case Ty::I16: return "short";
+    case Ty::I32: return "int";
+    case Ty::I64: case Ty::Int: return "long long";
+    case Ty::U16: return "unsigned short";
+    case Ty::U32: return "unsigned int";
+    case Ty::U64: return "unsigned long long";
+    case Ty::F16: return "_Float16";
+    case Ty::BF16: return "__bf16";
+    case Ty::F32: return "float";
+    case Ty::F64: return "double";
+    case Ty::Ptr: return ctype(*d.inner) + "*";
+    default: throw Error("no HIP type for dtype " + d.name());
+  }
+}
+
+std::string literal(const Node& n) {
+  char buf[64];
+  switch (n.dtype.ty) {
+    case Ty::F32: case Ty::F16: case Ty::BF16: {
+      std::string cast = n.dtype.ty == Ty::F32 ? "" : "(" + ctype(n.dtype) + ")";
+      if (std::isnan(n.fval)) return cast + "__builtin_nanf(\"\")";
+      if (std::isinf(n.fval)) return cast + (n.fval > 0 ? "__builtin_inff()" : "(-__builtin_inff())");
+      float f = static_cast<float>(n.fval);
+      if (f == std::floor(f) && std::fabs(f) < 1e6f) snprintf(buf, sizeof buf, "%.1ff", f);
+      else snprintf(buf, sizeof buf, "%af", f);           // hex float: exact
+      return cast + buf;
+    }
+    case Ty::F64:
+      if (std::isnan(n.fval)) return "__builtin_nan(\"\")";
+      if (std::isinf(n.fval)) return n.fval > 0 ? "__builtin_inf()" : "(-__builtin_inf())";
+      snprintf(buf, sizeof buf, "%a", n.fval);
+      return buf;
+    case Ty::Bool: return n.ival ? "1" : "0";
+    case Ty::U8: case Ty::U16: case Ty::U32:
+      return std::to_string(static_cast<unsigned long long>(n.ival)) + "u";
+    case Ty::U64:
+      return std::to_string(static_cast<unsigned long long>(n.ival)) + "ull";
+    case Ty::I64: case Ty::Int:
+      if (n.ival == INT64_MIN) return "(-9223372036854775807ll - 1)";
+      if (n.ival > INT32_MAX || n.ival < INT32_MIN) return std::to_string(n.ival) + "ll";
+      return std::to_string(n.ival);
+    case Ty::I32:
+      if (n.ival == INT32_MIN) return "(-2147483647 - 1)";
+      return std::to_string(n.ival);
+    default:
+      return std::to_string(n.ival);
+  }
+}
+
+// Result type of an expression, as far as rendering needs it.
+Ty infer_ty(const Node& n, const std::map<std::string, Ty>* vars = nullptr) {
+  switch (n.op) {
+    case Op::Const: return n.dtype.ty;
+    case Op::Load: case Op::SharedLoad: case Op::Cast: return n.dtype.ty;
+    case Op::Lt: case Op::And: case Op::Not: return Ty::Bool;
+    case Op::Recip: case Op::Sqrt: case Op::Log2: case Op::Exp2: case Op::Sin: case Op::Floor: {
+      Ty t = infer_ty(*n.args[0], vars);
+      return t == Ty::F64 ? Ty::F64 : Ty::F32;
+    }
+    case Op::Select: return infer_ty(*n.args[1], vars);
+    case Op::Fma: return infer_ty(*n.args[0], vars);
+    case Op::Var:
+      if (vars) {
+        auto it = vars->find(n.name);
+        if (it != vars->end()) return it->second;
+      }
+      return Ty::I64;
+    case Op::Rand: return Ty::F32;
+    case Op::AtomicAdd: case Op::AtomicMax: return n.dtype.ty;
+    default:
+      if (n.args.empty()) return Ty::Unknown;
+      {
+        Ty a = infer_ty(*n.args[0], vars);
+        if (n.args.size() > 1) {
+          Ty b = infer_ty(*n.args[1], vars);
+          auto rank = [](Ty t) { return t == Ty::F64 ? 4 : t == Ty::F32 ? 3 : (t == Ty::F16 || t == Ty::BF16) ? 2 : 1; };
+          return rank(b) > rank(a) ? b : a;
+        }
+        return a;
+      }
+  }
+}
+
+const char* infix(Op op) {
+  switch (op) {
+    case Op::Add: return "+";
+    case Op::Mul: return "*";
+    case Op::Rem: return "%";
+    case Op::Idiv: return "/";
+    case Op::Lt: return "<";
+    case Op::And: return "&&";
+    case Op::BitAnd: return "&";
+    case Op::BitOr: return "|";
+    case Op::BitXor: return "^";
+    case Op::Shl: return "<<";
+    case Op::Shr: return ">>";
+    default: return nullptr;
+  }
+}
+
+using LoadHook = std::function<bool(const Node& load, std::string* out)>;
+
+struct ExprRenderer {
+  LoadHook load_hook;
+  const std::map<std::string, Ty>* var_types = nullptr;
+
+  std::string math1(const char* f32, const char* f64, const Node& n) const {
+    bool dbl = infer_ty(*n.args[0], var_types) == Ty::F64;
+    return std::string(dbl ? f64 : f32) + "(" + expr(*n.args[0]) + ")";
+  }
+
+  std::string expr(const Node& n) const {
+    if (const char* s = infix(n.op)) return "(" + expr(*n.args[0]) + " " + s + " " + expr(*n.args[1]) + ")";
+    switch (n.op) {
+      case Op::Const: return literal(n);
+      case Op::Var: case Op::Wildcard: return n.name;
+      case Op::Max: {
+        Ty t = infer_ty(n, var_types);
+        std::string a = expr(*n.args[0]), b = expr(*n.args[1]);
+        if (t == Ty::F32 || t == Ty::F16 || t == Ty::BF16) return "fmaxf(" + a + ", " + b + ")";
+        if (t == Ty::F64) return "fmax(" + a + ", " + b + ")";
+        return "((" + a + ") > (" + b + ") ? (" + a + ") : (" + b + "))";
+      }
+      case Op::Recip:
+        return infer_ty(*n.args[0], var_types) == Ty::F64 ? "(1.0 / " + expr(*n.args[0]) + ")"
+                                                         : "(1.0f / " + expr(*n.args[0]) + ")";
+      case Op::Sqrt: return math1("sqrtf", "sqrt", n);
+      case Op::Log2: return math1("log2f", "log2", n);
+      case Op::Exp2: return math1("exp2f", "exp2", n);
+      case Op::Sin: return math1("sinf", "sin", n);
+      case Op::Floor: return math1("floorf", "floor", n);
+      case Op::Not: return "(!" + expr(*n.args[0]) + ")";
+      case Op::BitNot: return "(~" + expr(*n.args[0]) + ")";
+      case Op::Cast: return "(" + ctype(n.dtype) + ")(" + expr(*n.args[0]) + ")";
+      case Op::Fma: {
+        bool dbl = infer_ty(n, var_types) == Ty::F64;
+        return std::string(dbl ? "fma(" : "fmaf(") + expr(*n.args[0]) + ", " + expr(*n.args[1]) + ", " +
+               expr(*n.args[2]) + ")";
+      }
+      case Op::Select:
+        return "(" + expr(*n.args[0]) + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
+      case Op::Load: {
+        std::string s;
+        if (load_hook && load_hook(n, &s)) return s;
+        if (n.count == 1) return expr(*n.args[0]) + "[" + expr(*n.args[1]) + "]";
+        return "*reinterpret_cast<const " + ctype(n.dtype) + "*>(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "])";
+      }
+      case Op::SharedLoad: return expr(*n.args[0]) + "[" + expr(*n.args[1]) + "]";
+      case Op::Rand: return "0.5f /* rand is not available in device code */";
+      case Op::Call: {
+        std::string s = n.name + "(";
+        for (size_t i = 0; i < n.args.size(); ++i) s += (i ? ", " : "") + expr(*n.args[i]);
+        return s + ")";
+      }
+      case Op::AtomicAdd:
+        return "atomicAdd(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "], " + expr(*n.args[2]) + ")";
+      case Op::AtomicMax:
+        if (n.dtype.ty == Ty::F32)
+          return "eh_atomic_max_f32(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "], " + expr(*n.args[2]) + ")";
+        return "atomicMax(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "], " + expr(*n.args[2]) + ")";
+      default:
+        throw Error(std::string("cannot render '") + op_name(n.op) + "' as an expression");
+    }
+  }
+};
+
+std::string hdr(const GenOptions&) {
+  return "// generated for gfx950 by eclat backend-hip\n#ifndef __HIPCC_RTC__\n#include <hip/hip_runtime.h>\n#endif\n" +
+         preamble();
+}
+
+// ---------------------------------------------------------------------------------------------
+// statement-by-statement rendering (kernels no schedule recognises)
+// ---------------------------------------------------------------------------------------------
+
+struct StmtRenderer {
+  ExprRenderer er;
+  int level = 1;
+  std::string ind() const { return std::string(static_cast<size_t>(level) * 2, ' '); }
+
+  std::string stmt(const Node& n) {
+    switch (n.op) {
+      case Op::Store:
+        return ind() + er.expr(*n.args[0]) + "[" + er.expr(*n.args[1]) + "] = " + er.expr(*n.args[2]) + ";\n";
+      case Op::Assign:
+        return ind() + n.name + " = " + er.expr(*n.args[0]) + ";\n";
+      case Op::Block: {
+        std::string s;
+        for (const auto& d : n.decls) s += ind() + ctype(d.second) + " " + d.first + ";\n";
+        for (const auto& a : n.args) s += stmt(*a);
+        return s;
+      }
+      case Op::Range: {
+        std::string s = ind() + "for (long long " + n.name + " = " + er.expr(*n.args[0]) + "; " + n.name + " < " +
+                        er.expr(*n.args[2]) + "; " + n.name + " += " + er.expr(*n.args[1]) + ") {\n";
+        ++level;
+        s += stmt(*n.args[3]);
+        --level;
+        return s + ind() + "}\n";
+      }
+      case Op::If: {
+        std::string s = ind() + "if (" + er.expr(*n.args[0]) + ") {\n";
+        ++level;
+        s += stmt(*n.args[1]);
+        --level;
+        s += ind() + "}";
+        if (n.args.size() > 2) {
+          s += " else {\n";
+          ++level;
+          s += stmt(*n.args[2]);
+          --level;
+          s += ind() + "}";
+        }
+        return s + "\n";
+      }
+      case Op::Barrier: return ind() + "__syncthreads();\n";
+      case Op::Return: return ind() + "return " + er.expr(*n.args[0]) + ";\n";
+      case Op::SharedAlloc:
+        return ind() + "__shared__ " + ctype(n.dtype) + " " + n.name + "[" + er.expr(*n.args[0]) + "];\n";
+      case Op::SharedStore:
+        return ind() + er.expr(*n.args[0]) + "[" + er.expr(*n.args[1]) + "] = " + er.expr(*n.args[2]) + ";\n";
+      case Op::WmmaMatmul:
+        throw Error("WmmaMatmul (f16 16x16x16 tiles) is not part of the fp32 path of this backend");
+      default:
+        return ind() + er.expr(n) + ";\n";
+    }
+  }
+};
+
+int64_t const_int(const Node& n, int64_t dflt) {
+  if (n.op == Op::Const && !n.dtype.is_float()) return n.ival;
+  return dflt;
+}
+
+const char* kAtomicMaxF32 = R"EHA(
+__device__ inline float eh_atomic_max_f32(float* addr, float v) {
+  unsigned int* a = reinterpret_cast<unsigned int*>(addr);
+  unsigned int old = *a, assumed;
+  do {
+    assumed = old;
+    if (__uint_as_float(assumed) >= v) break;
+    old = atomicCAS(a, assumed, __float_as_uint(v));
+  } while (assumed != old);
+  return __uint_as_float(old);
+}
+)EHA";
+
+}  // namespace
+
+std::string render_expr_text(const Node& e) {
+  ExprRenderer er;
+  return er.expr(e);
+}
+
+LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
+  if (k.op != Op::Kernel) throw Error("expected a kernel node");
+  LaunchSpec ls;
+  ls.entry = k.name;
+  ls.kernels = {k.name};
+  ls.schedule = "as-written";
+  std::ostringstream os;
+  os << hdr(opt) << kAtomicMaxF32;
+  os << "extern \"C\" __global__ void " << k.name << "(";
+  bool first = true;
+  std::string decls;
+  static const char* dim[] = {"x", "y", "z"};
+  for (const auto& p : k.params) {
+    if (p.kind == VarKind::Normal) {
+      if (!p.dtype.is_ptr())
+        throw Error("kernel '" + k.name + "' takes the shape variable '" + p.name +
+                    "'; only static shapes are supported on this path");
+      os << (first ? "" : ", ") << (p.mut_ ? "" : "const ") << ctype(p.dtype.elem()) << "* __restrict__ " << p.name;
+      first = false;
+      ls.arg_bufs.push_back(p.name);
+    } else {
+      const char* src = p.kind == VarKind::GroupId ? "blockIdx" : p.kind == VarKind::LocalId ? "threadIdx"
+                        : p.kind == VarKind::GroupSize ? "blockDim" : "gridDim";
+      if (p.axis < 0 || p.axis > 2) throw Error("bad axis on parameter " + p.name);
+      decls += "  const long long " + p.name + " = " + src + "." + dim[p.axis] +
+               (p.kind == VarKind::GridSize ? std::string(" * blockDim.") + dim[p.axis] : std::string()) + ";\n";
+    }
+  }
+  os << ") {\n" << decls;
+  StmtRenderer sr;
+  os << sr.stmt(*k.args[0]) << "}\n";
+  ls.source = os.str();
+  for (int i = 0; i < 3; ++i) {
+    int64_t g = k.grid.size() == 3 ? const_int(*k.grid[i], 1) : 1;
+    int64_t t = k.tg.size() == 3 ? const_int(*k.tg[i], 1) : 1;
+    if (g < 1 || t < 1 || t > 1024) throw Error("kernel '" + k.name + "' has an unusable dispatch size");
+    ls.block[i] = static_cast<unsigned>(t);
+    ls.grid[i] = static_cast<unsigned>(g);   // the AST's grid size counts workgroups
+  }
+  return ls;
+}
+
+// ---------------------------------------------------------------------------------------------
+// canonical stages and grouping
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+enum class StageKind { Wide, Reduce, Scalar };
+
+struct Stage {
+  StageKind kind = StageKind::Wide;
+  std::string kname;
+  NodePtr value;             // over canonical variables r0.. and c
+  ReduceKind rk = ReduceKind::None;
+  NodePtr identity;
+  DType acc_dtype;
+  std::string out_buf;
+  Affine out_aff;
+  DType out_dtype;
+  bool store = true;
+};
+
+struct Group {
+  std::vector<int64_t> rows;   // extents of the row loops (all > 1)
+  int64_t C = 1;               // extent of the column loop
+  std::vector<Stage> stages;
+  bool has_reduce() const {
+    for (const auto& s : stages)
+      if (s.kind == StageKind::Reduce) return true;
+    return false;
+  }
+  int64_t R() const {
+    int64_t r = 1;
+    for (auto e : rows) r *= e;
+    return r;
+  }
+  const Stage* producer(const std::string& buf) const {
+    for (const auto& s : stages)
+      if (s.out_buf == buf) return &s;
+    return nullptr;
+  }
+};
+
+NodePtr rename(const NodePtr& n, const std::map<std::string, NodePtr>& m) {
+  if (n->op == Op::Var) {
+    auto it = m.find(n->name);
+    return it == m.end() ? n : it->second;
+  }
+  bool changed = false;
+  std::vector<NodePtr> args;
+  args.reserve(n->args.size());
+  for (const auto& a : n->args) {
+    NodePtr r = rename(a, m);
+    changed = changed || r != a;
+    args.push_back(std::move(r));
+  }
+  if (!changed) return n;
+  auto c = std::make_shared<Node>(*n);
+  c->args = std::move(args);
+  return c;
+}
+
+// Canonical form of a kernel: `nrows` of its non-trivial loops are rows, then (for Wide) one
+// column loop; a reduce kernel's column is its reduce loop.
+bool canonicalise(const NestKernel& k, StageKind kind, std::vector<int64_t>* rows, int64_t* C, Stage* out) {
+  std::vector<Loop> live;
+  std::map<std::string, NodePtr> m;
+  for (const auto& l : k.loops) {
+    if (l.extent == 0) return false;
+    if (l.extent == 1) m[l.var] = make_i64(0);
+    else live.push_back(l);
+  }
+  rows->clear();
+  size_t nrow = live.size();
+  if (kind == StageKind::Wide) {
+    if (live.empty()) {
+      *C = 1;
+    } else {
+      nrow = live.size() - 1;
+      *C = live.back().extent;
+      m[live.back().var] = make_var("c");
+    }
+  } else if (kind == StageKind::Reduce) {
+    if (k.rloop.extent == 0) return false;
+    *C = k.rloop.extent;
+    m[k.rloop.var] = k.rloop.extent == 1 ? make_i64(0) : make_var("c");
+  }
+  for (size_t i = 0; i < nrow; ++i) {
+    rows->push_back(live[i].extent);
+    m[live[i].var] = make_var("r" + std::to_string(i));
+  }
+  out->kind = kind;
+  out->kname = k.name;
+  out->value = rename(k.value, m);
+  out->rk = k.rkind;
+  out->identity = k.identity;
+  out->acc_dtype = k.acc_dtype;
+  out->out_buf = k.out_buf;
+  out->out_dtype = k.out_dtype;
+  auto oa = affine_of(*rename(k.out_index, m));
+  if (!oa) return false;
+  out->out_aff = *oa;
+  return true;
+}
+
+// A reduce kernel is a row program candidate when its reduce loop walks memory contiguously
+// for at least one operand (otherwise lanes along the loop would not coalesce).
+bool reduce_is_rowwise(const NestKernel& k) {
+  std::vector<LoadRef> loads;
+  collect_loads(*k.value, loads);
+  bool any_unit = false, any_dep = false;
+  for (const auto& lr : loads) {
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a) continue;
+    int64_t c = a->of(k.rloop.var);
+    if (c != 0) any_dep = true;
+    if (c == 1 || c == -1) any_unit = true;
+  }
+  return any_unit || !any_dep;
+}
+
+// Loads of buffers produced inside the group must hit exactly the element the producer wrote.
+bool aligned_with_group(const Group& g, const Stage& s) {
+  std::vector<LoadRef> loads;
+  collect_loads(*s.value, loads);
+  for (const auto& lr : loads) {
+    const Stage* p = g.producer(lr.load->args[0]->name);
+    if (!p) continue;
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a || !(*a == p->out_aff)) return false;
+    if (s.kind == StageKind::Scalar && p->kind == StageKind::Wide) return false;
+  }
+  return true;
+}
+
+struct Canon {
+  bool ok = false;
+  Stage stage;
+  std::vector<int64_t> rows;
+  int64_t C = 1;
+};
+
+Canon canon_as(const NestKernel& k, StageKind kind) {
+  Canon c;
+  c.ok = canonicalise(k, kind, &c.rows, &c.C, &c.stage);
+  return c;
+}
+
+}  // namespace
+
+// The emitters live below; declared here so plan_program reads top-down.
+namespace {
+LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& buf_elems);
+LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt);
+}  // namespace
+
+ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
+  if (program.op != Op::Program) throw Error("expected a program node");
+  ProgramPlan plan;
+  std::vector<const Node*> kernels;
+  for (const auto& f : program.args) {
+    if (f->op == Op::Kernel) kernels.push_back(f.get());
+    else if (f->op == Op::Function) throw Error("helper functions in a program are not supported by this backend");
+  }
+  if (kernels.empty()) throw Error("program holds no kernel");
+
+  // buffer table: given, or synthesised from the kernels' pointer parameters
+  plan.buffers = program.buffers;
+  std::map<std::string, size_t> elems;
+  bool have_table = !plan.buffers.empty();
+  if (have_table) {
+    for (const auto& b : plan.buffers) elems[b.name] = b.numel();
+  } else {
+    std::set<std::string> seen;
+    for (const Node* k : kernels)
+      for (const auto& p : k->params)
+        if (p.dtype.is_ptr() && seen.insert(p.name).second) {
+          BufferInfo bi;
+          bi.name = p.name;
+          bi.dtype = p.dtype.elem();
+          bi.role = p.mut_ ? "output" : "input";
+          plan.buffers.push_back(bi);
+        } else if (p.dtype.is_ptr() && p.mut_) {
+          for (auto& b : plan.buffers)
+            if (b.name == p.name) b.role = "output";
+        }
+  }
+  auto role_of = [&](const std::string& name) -> std::string {
+    for (const auto& b : plan.buffers)
+      if (b.name == name) return b.role;
+    throw Error("kernel parameter '" + name + "' is missing from the program's buffer table");
+  };
+  for (const Node* k : kernels)
+    for (const auto& p : k->params)
+      if (p.dtype.is_ptr()) role_of(p.name);
+
+  // consumers per buffer (kernel indices)
+  std::map<std::string, std::vector<size_t>> readers;
+  for (size_t i = 0; i < kernels.size(); ++i)
+    for (const auto& p : kernels[i]->params)
+      if (p.dtype.is_ptr() && !p.mut_) readers[p.name].push_back(i);
+
+  std::vector<std::optional<NestKernel>> nests;
+  for (const Node* k : kernels) nests.push_back(extract_nest(*k));
+
+  size_t i = 0;
+  while (i < kernels.size()) {
+    if (!nests[i]) {
+      plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+      ++i;
+      continue;
+    }
+    const NestKernel& k0 = *nests[i];
+    // contraction (matmul-shaped reduce) -> MFMA schedule
+    if (k0.rkind == ReduceKind::Sum && opt.gemm) {
+      if (auto ls = try_emit_gemm(k0, opt)) {
+        plan.launches.push_back(*ls);
+        ++i;
+        continue;
+      }
+    }
+    if (k0.rkind != ReduceKind::None && !reduce_is_rowwise(k0)) {
+      plan.launches.push_back(emit_serial_reduce(k0, opt));
+      ++i;
+      continue;
+    }
+    // start a group with kernel i and extend it while the next kernels fit
+    Group g;
+    size_t first = i;
+    {
+      Canon c = canon_as(k0, k0.rkind == ReduceKind::None ? StageKind::Wide : StageKind::Reduce);
+      if (!c.ok) {
+        plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+        ++i;
+        continue;
+      }
+      g.rows = c.rows;
+      g.C = c.C;
+      g.stages.push_back(c.stage);
+    }
+    ++i;
+    while (opt.fuse && i < kernels.size() && nests[i]) {
+      const NestKernel& k = *nests[i];
+      if (k.rkind == ReduceKind::Sum && opt.gemm && gemm_shaped(k, opt)) break;
+      Canon pick;
+      if (k.rkind != ReduceKind::None) {
+        if (!reduce_is_rowwise(k)) break;
+        Canon c = canon_as(k, StageKind::Reduce);
+        if (c.ok && c.rows == g.rows && c.C == g.C) pick = c;
+      } else {
+        Canon w = canon_as(k, StageKind::Wide);
+        if (w.ok && w.rows == g.rows && w.C == g.C) pick = w;
+        else {
+          Canon s = canon_as(k, StageKind::Scalar);
+          if (s.ok && s.rows == g.rows && g.has_reduce()) pick = s;
+        }
+      }
+      if (!pick.ok || !aligned_with_group(g, pick.stage)) break;
+      // a buffer may be written once per group
+      if (g.producer(pick.stage.out_buf)) break;
+      g.stages.push_back(pick.stage);
+      ++i;
+    }
+    // which stage outputs must reach memory
+    for (size_t s = 0; s < g.stages.size(); ++s) {
+      Stage& st = g.stages[s];
+      bool needed = role_of(st.out_buf) != "temp";
+      for (size_t r : readers[st.out_buf])
+        if (r < first || r >= i) needed = true;
+      st.store = needed;
+      if (!needed) plan.elided.insert(st.out_buf);
+    }
+    plan.launches.push_back(emit_group(g, opt, elems));
+  }
+  return plan;
+}
+
+// ---------------------------------------------------------------------------------------------
+// emitters
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+const char* op_struct(ReduceKind k) {
+  switch (k) {
+    case ReduceKind::Sum: return "EhSum";
+    case ReduceKind::Max: return "EhMax";
+    case ReduceKind::Min: return "EhMin";
+    case ReduceKind::Prod: return "EhProd";
+    default: return "?";
+  }
+}
+
+std::string combine_text(ReduceKind k, const DType& t, const std::string& acc, const std::string& v) {
+  switch (k) {
+    case ReduceKind::Sum: return "(" + acc + " + " + v + ")";
+    case ReduceKind::Prod: return "(" + acc + " * " + v + ")";
+    case ReduceKind::Max:
+      if (t.ty == Ty::F32) return "fmaxf(" + acc + ", " + v + ")";
+      if (t.ty == Ty::F64) return "fmax(" + acc + ", " + v + ")";
+      return "(" + acc + " > " + v + " ? " + acc + " : " + v + ")";
+    case ReduceKind::Min: return "(" + acc + " < " + v + " ? " + acc + " : " + v + ")";
+    default: return acc;
+  }
+}
+
+bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+int64_t pow2_ceil(int64_t v) {
+  int64_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// One distinct external access: buffer + affine index over canonical vars.
+struct ExtLoad {
+  std::string buf;
+  Affine aff;
+  DType dtype;
+  int id = 0;
+  bool cached = false;   // held in registers for the whole row
+};
+
+struct GroupEmitter {
+  const Group& g;
+  const GenOptions& opt;
+  std::vector<ExtLoad> ext;          // distinct affine external loads eligible for caching/vectorising
+  std::vector<std::string> in_bufs;  // external buffers read, parameter order
+  std::map<std::string, DType> in_dtype;
+  bool idx64 = false;
+  int V = 1;
+  std::map<std::string, int64_t> need;   // elements each bound buffer must hold (max index + 1)
+
+  GroupEmitter(const Group& grp, const GenOptions& o) : g(grp), opt(o) {}
+
+  std::string sname(const std::string& buf) const { return "s_" + buf; }
+
+  int find_ext(const std::string& buf, const Affine& a) const {
+    for (const auto& e : ext)
+      if (e.buf == buf && e.aff == a) return e.id;
+    return -1;
+  }
+
+  // Collect external loads (recursing through nothing: stage values only reference buffers).
+  void scan() {
+    int64_t reach = 0;
+    std::vector<Loop> loops;
+    for (size_t i = 0; i < g.rows.size(); ++i) loops.push_back({"r" + std::to_string(i), g.rows[i]});
+    Loop cl{"c", g.C};
+    for (const auto& st : g.stages) {
+      std::vector<LoadRef> loads;
+      collect_loads(*st.value, loads);
+      for (const auto& lr : loads) {
+        const std::string& b = lr.load->args[0]->name;
+        if (g.producer(b) && g.producer(b) != &st) {
+          // only earlier stages can be producers; a later stage writing a buffer read here is external
+          bool earlier = false;
+          for (const auto& p : g.stages) {
+            if (&p == &st) break;
+            if (p.out_buf == b) earlier = true;
+          }
+          if (earlier) continue;
+        }
+        if (std::find(in_bufs.begin(), in_bufs.end(), b) == in_bufs.end()) {
+          in_bufs.push_back(b);
+          in_dtype[b] = lr.load->dtype;
+        }
+        auto a = affine_of(*lr.load->args[1]);
+        if (!a) { idx64 = true; continue; }     // opaque index: stay in 64-bit to be safe
+        const int64_t top = max_abs_index(*a, loads_loops(loops), &cl);
+        reach = std::max(reach, top);
+        need[b] = std::max(need[b], top + 1);
+        if (!lr.guarded && a->of("c") == 1 && find_ext(b, *a) < 0) {
+          ExtLoad e;
+          e.buf = b;
+          e.aff = *a;
+          e.dtype = lr.load->dtype;
+          e.id = static_cast<int>(ext.size());
+          ext.push_back(e);
+        }
+      }
+      if (st.store) {
+        const int64_t top = max_abs_index(st.out_aff, loops, &cl);
+        reach = std::max(reach, top);
+        need[st.out_buf] = std::max(need[st.out_buf], top + 1);
+      }
+    }
+    if (reach >= (int64_t{1} << 31) - 8 || g.R() * g.C >= (int64_t{1} << 31) - 8) idx64 = true;
+  }
+  static const std::vector<Loop>& loads_loops(const std::vector<Loop>& l) { return l; }
+
+  // 128-bit accesses need every vectorised access to start on a 4-element boundary.
+  bool aligned4(const Affine& a) const {
+    if (a.c % 4) return false;
+    for (const auto& kv : a.coef)
+      if (kv.first != "c" && kv.second % 4) return false;
+    return true;
+  }
+
+  void choose_vector() {
+    V = 1;
+    if (!opt.vectorize || g.C % 4) return;
+    for (const auto& e : ext)
+      if (!aligned4(e.aff) || e.dtype.itemsize() != 4) return;
+    for (const auto& st : g.stages)
+      if (st.kind == StageKind::Wide && st.store &&
+          (st.out_aff.of("c") != 1 || !aligned4(st.out_aff) || st.out_dtype.itemsize() != 4))
+        return;
+    V = 4;
+  }
+
+  std::string affine_text(const Affine& a, const std::string& cvar) const {
+    std::string s;
+    auto term = [&](const std::string& t) { s += s.empty() ? t : " + " + t; };
+    for (const auto& kv : a.coef) {
+      std::string v = kv.first == "c" ? cvar : kv.first;
+      if (kv.second == 1) term(v);
+      else term(v + " * " + std::to_string(kv.second) + (idx64 ? "ll" : ""));
+    }
+    if (a.c != 0 || s.empty()) term(std::to_string(a.c));
+    return "(" + s + ")";
+  }
+
+  // Value of a stage for the element whose column variable is `c` (declared in scope).
+  // `ld` maps a cached/vectorised external load id to the text that yields its value.
+  std::string value_text(const Stage& st, const std::function<std::string(int)>& ld) const {
+    ExprRenderer er;
+    er.load_hook = [&](const Node& load, std::string* out) {
+      const std::string& b = load.args[0]->name;
+      const Stage* p = nullptr;
+      for (const auto& q : g.stages) {
+        if (&q == &st) break;
+        if (q.out_buf == b) p = &q;
+      }
+      if (p) {
+        if (p->kind == StageKind::Wide) {
+          *out = "((" + ctype(p->out_dtype) + ")(" + value_text(*p, ld) + "))";
+        } else {
+          *out = sname(b);
+        }
+        return true;
+      }
+      auto a = affine_of(*load.args[1]);
+      if (a) {
+        int id = find_ext(b, *a);
+        if (id >= 0) {
+          std::string t = ld(id);
+          if (!t.empty()) { *out = t; return true; }
+        }
+        *out = b + "[" + affine_text(*a, "c") + "]";
+        return true;
+      }
+      return false;   // opaque index: rendered from the tree with canonical variable names
+    };
+    return er.expr(*st.value);
+  }
+
+  std::string params_text(std::vector<std::string>* order) const {
+    std::string s;
+    for (const auto& b : in_bufs) {
+      bool also_out = false;
+      for (const auto& st : g.stages) also_out = also_out || (st.store && st.out_buf == b);
+      if (also_out) throw Error("buffer '" + b + "' is both read as an input and written in one fused launch");
+      s += (s.empty() ? "" : ", ") + std::string("const ") + ctype(in_dtype.at(b)) + "* __restrict__ " + b;
+      order->push_back(b);
+    }
+    for (const auto& st : g.stages)
+      if (st.store) {
+        s += (s.empty() ? "" : ", ") + ctype(st.out_dtype) + "* __restrict__ " + st.out_buf;
+        order->push_back(st.out_buf);
+      }
+    return s;
+  }
+
+  std::string row_decode(const std::string& rowvar) const {
+    // row -> r0..rn-1 (row-major over the row loops)
+    std::string s;
+    if (g.rows.empty()) return s;
+    if (g.rows.size() == 1) return "  const idx_t r0 = " + rowvar + ";\n";
+    s += "  idx_t eh_rem = " + rowvar + ";\n";
+    for (size_t i = g.rows.size(); i-- > 0;) {
+      if (i == 0) s += "  const idx_t r0 = eh_rem;\n";
+      else {
+        s += "  const idx_t r" + std::to_string(i) + " = eh_rem % " + std::to_string(g.rows[i]) + ";\n";
+        s += "  eh_rem /= " + std::to_string(g.rows[i]) + ";\n";
+      }
+    }
+    return s;
+  }
+
+  void fill_min_bytes(LaunchSpec* ls) const {
+    for (const auto& b : ls->arg_bufs) {
+      size_t item = 4;
+      auto it = in_dtype.find(b);
+      if (it != in_dtype.end()) item = it->second.itemsize();
+      for (const auto& st : g.stages)
+        if (st.store && st.out_buf == b) item = st.out_dtype.itemsize();
+      auto n = need.find(b);
+      ls->arg_min_bytes.push_back(n == need.end() ? 0 : static_cast<size_t>(n->second) * item);
+    }
+  }
+
+  double algo_bytes(const std::map<std::string, size_t>& elems) const {
+    double b = 0;
+    for (const auto& n : in_bufs) {
+      auto it = elems.find(n);
+      double cnt = it != elems.end() ? static_cast<double>(it->second) : static_cast<double>(g.R() * g.C);
+      b += cnt * static_cast<double>(in_dtype.at(n).itemsize());
+    }
+    for (const auto& st : g.stages)
+      if (st.store)
+        b += static_cast<double>(st.kind == StageKind::Wide ? g.R() * g.C : g.R()) *
+             static_cast<double>(st.out_dtype.itemsize());
+    return b;
+  }
+
+  // ---- flat: no reductions; a grid-stride loop over 4-element vectors --------------------
+  LaunchSpec emit_flat(const std::map<std::string, size_t>& elems) {
+    LaunchSpec ls;
+    const int64_t N = g.R() * g.C;
+    const int64_t NVEC = N / V;
+    const int block = opt.flat_block;
+    int64_t want = (NVEC + static_cast<int64_t>(block) * opt.flat_iters - 1) / (static_cast<int64_t>(block) * opt.flat_iters);
+    int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(want, 1 << 20));
+    ls.entry = "ehk_" + g.stages.front().kname;
+    ls.schedule = "flat(V=" + std::to_string(V) + ",block=" + std::to_string(block) + ")";
+    ls.grid[0] = static_cast<unsigned>(blocks);
+    ls.block[0] = static_cast<unsigned>(block);
+    std::ostringstream os;
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "("
+       << params_text(&ls.arg_bufs) << ") {\n";
+    os << "  const idx_t eh_nvec = " << NVEC << ";\n";
+    os << "  const idx_t eh_stride = (idx_t)gridDim.x * " << block << ";\n";
+    os << "  for (idx_t eh_g = (idx_t)blockIdx.x * " << block << " + threadIdx.x; eh_g < eh_nvec; eh_g += eh_stride) {\n";
+    os << "  const idx_t eh_p = eh_g * " << V << ";\n";
+    if (!g.rows.empty()) {
+      os << "  const idx_t eh_row = eh_p / " << g.C << ";\n  const idx_t c0 = eh_p % " << g.C << ";\n";
+      os << row_decode("eh_row");
+    } else {
+      os << "  const idx_t c0 = eh_p;\n";
+    }
+    // vector loads
+    auto ld = [&](int id) -> std::string {
+      return V == 4 ? "ld" + std::to_string(id) + ".v[v]" : std::string();
+    };
+    if (V == 4)
+      for (const auto& e : ext)
+        os << "  const EhV4<" << ctype(e.dtype) << "> ld" << e.id << " = *reinterpret_cast<const EhV4<" << ctype(e.dtype)
+           << ">*>(" << e.buf << " + " << affine_text(e.aff, "c0") << ");\n";
+    for (const auto& st : g.stages) {
+      if (!st.store) continue;
+      std::string T = ctype(st.out_dtype);
+      if (V == 4) {
+        os << "  { EhV4<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o.v[v] = ("
+           << T << ")(" << value_text(st, ld) << "); }\n";
+        os << "  *reinterpret_cast<EhV4<" << T << ">*>(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ") = o; }\n";
+      } else {
+        os << "  { const idx_t c = c0; " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << T << ")("
+           << value_text(st, ld) << "); }\n";
+      }
+    }
+    os << "  }\n}\n";
+    ls.source = os.str();
+    ls.algo_bytes = algo_bytes(elems);
+    fill_min_bytes(&ls);
+    for (const auto& st : g.stages) ls.kernels.push_back(st.kname);
+    return ls;
+  }
+
+  // ---- row program: T threads per row, DPP/LDS reductions ---------------------------------
+  LaunchSpec emit_rows(const std::map<std::string, size_t>& elems) {
+    LaunchSpec ls;
+    const int64_t R = g.R(), C = g.C;
+    int64_t T = opt.row_threads > 0 ? opt.row_threads : pow2_ceil((C + opt.row_elems - 1) / opt.row_elems);
+    T = std::max<int64_t>(1, std::min<int64_t>(T, 1024));
+    if (!pow2(T)) T = pow2_ceil(T);
+    while (T * V > pow2_ceil(C) && T > 1) T >>= 1;          // no more threads than vectors in a row
+    const int64_t per_iter = T * V;
+    const int64_t NV = (C + per_iter - 1) / per_iter;
+    const bool reg = NV * V <= 64;                           // whole row of a thread fits registers
+    const bool tail = (C % per_iter) != 0;
+    const int64_t block = T >= 256 ? T : 256;
+    const int64_t RPB = block / T;
+    const int64_t blocks = (R + RPB - 1) / RPB;
+    if (blocks >= (int64_t{1} << 31)) throw Error("too many rows for one launch");
+    int nred = 0;
+    for (const auto& st : g.stages) nred += st.kind == StageKind::Reduce;
+    ls.entry = "ehk_" + g.stages.front().kname;
+    ls.schedule = "row(T=" + std::to_string(T) + ",V=" + std::to_string(V) + ",NV=" + std::to_string(NV) +
+                  (reg ? ",reg" : ",stream") + ",rows/block=" + std::to_string(RPB) + ")";
+    ls.grid[0] = static_cast<unsigned>(blocks);
+    ls.block[0] = static_cast<unsigned>(block);
+    for (auto& e : ext) e.cached = reg;
+
+    std::ostringstream os;
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "("
+       << params_text(&ls.arg_bufs) << ") {\n";
+    os << "  constexpr int T = " << T << ", V = " << V << ", NV = " << NV << ";\n";
+    os << "  constexpr idx_t C = " << C << ", R = " << R << ";\n";
+    os << "  const int lr = threadIdx.x % T;\n";
+    os << "  idx_t eh_row = (idx_t)blockIdx.x * " << RPB << " + threadIdx.x / T;\n";
+    os << "  const bool eh_row_ok = eh_row < R;\n  if (!eh_row_ok) eh_row = R - 1;\n";
+    os << row_decode("eh_row");
+    if (T > 64 && nred > 0) {
+      // LDS slots typed per reduction
+      int r = 0;
+      for (const auto& st : g.stages)
+        if (st.kind == StageKind::Reduce)
+          os << "  __shared__ " << ctype(st.acc_dtype) << " eh_red" << r++ << "[" << T / 64 << "];\n";
+    }
+    const std::string iter_open = std::string(reg ? "#pragma unroll\n" : "") +
+                                  "  for (int k = 0; k < NV; ++k) {\n    const idx_t c0 = (idx_t)(k * T + lr) * V;\n";
+    const std::string guard_open = tail ? "    if (c0 < C) {\n" : "    {\n";
+    // preload the row slices every stage shares
+    if (reg) {
+      for (const auto& e : ext) os << "  " << ctype(e.dtype) << " xc" << e.id << "[NV * V];\n";
+      if (!ext.empty()) {
+        os << iter_open << guard_open;
+        for (const auto& e : ext) {
+          if (V == 4) {
+            os << "      const EhV4<" << ctype(e.dtype) << "> t" << e.id << " = *reinterpret_cast<const EhV4<"
+               << ctype(e.dtype) << ">*>(" << e.buf << " + " << affine_text(e.aff, "c0") << ");\n";
+            os << "#pragma unroll\n      for (int v = 0; v < 4; ++v) xc" << e.id << "[k * 4 + v] = t" << e.id << ".v[v];\n";
+          } else {
+            os << "      xc" << e.id << "[k] = " << e.buf << "[" << affine_text(e.aff, "c0") << "];\n";
+          }
+        }
+        os << "    }\n  }\n";
+      }
+    }
+    auto ld = [&](int id) -> std::string {
+      if (reg) return "xc" + std::to_string(id) + "[k * V + v]";
+      return std::string();
+    };
+    int red_i = 0;
+    for (const auto& st : g.stages) {
+      const std::string T_out = ctype(st.out_dtype);
+      os << "  // " << st.kname << "\n";
+      if (st.kind == StageKind::Reduce) {
+        const std::string TA = ctype(st.acc_dtype);
+        const std::string acc = "acc" + std::to_string(red_i);
+        os << "  " << TA << " " << acc << " = " << literal(*st.identity) << ";\n";
+        os << iter_open << guard_open;
+        os << "#pragma unroll\n      for (int v = 0; v < V; ++v) { const idx_t c = c0 + v; " << acc << " = "
+           << combine_text(st.rk, st.acc_dtype, acc, "(" + TA + ")(" + value_text(st, ld) + ")") << "; }\n";
+        os << "    }\n  }\n";
+        os << "  const " << TA << " " << sname(st.out_buf) << " = eh_row_reduce<" << op_struct(st.rk) << ", T>(" << acc
+           << ", " << (T > 64 ? "eh_red" + std::to_string(red_i) : std::string("(" + TA + "*)nullptr")) << ", lr);\n";
+        if (st.store)
+          os << "  if (lr == 0 && eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "0") << "] = ("
+             << T_out << ")" << sname(st.out_buf) << ";\n";
+        ++red_i;
+      } else if (st.kind == StageKind::Scalar) {
+        // per-row value; loads of wide operands cannot occur here
+        auto none = [](int) { return std::string(); };
+        os << "  const " << T_out << " " << sname(st.out_buf) << " = (" << T_out << ")(" << value_text(st, none) << ");\n";
+        if (st.store)
+          os << "  if (lr == 0 && eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "0") << "] = "
+             << sname(st.out_buf) << ";\n";
+      } else if (st.store) {
+        os << iter_open << guard_open;
+        if (V == 4) {
+          os << "      EhV4<" << T_out << "> o;\n#pragma unroll\n      for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o.v[v] = ("
+             << T_out << ")(" << value_text(st, ld) << "); }\n";
+          os << "      if (eh_row_ok) *reinterpret_cast<EhV4<" << T_out << ">*>(" << st.out_buf << " + "
+             << affine_text(st.out_aff, "c0") << ") = o;\n";
+        } else {
+          os << "      const int v = 0; const idx_t c = c0; const " << T_out << " o = (" << T_out << ")(" << value_text(st, ld)
+             << ");\n      if (eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = o;\n";
+        }
+        os << "    }\n  }\n";
+      }
+    }
+    os << "}\n";
+    ls.source = os.str();
+    ls.algo_bytes = algo_bytes(elems);
+    fill_min_bytes(&ls);
+    for (const auto& st : g.stages) ls.kernels.push_back(st.kname);
+    return ls;
+  }
+};
+
+LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& elems) {
+  GroupEmitter ge(g, opt);
+  ge.scan();
+  ge.choose_vector();
+  bool any_store = false;
+  for (const auto& st : g.stages) any_store = any_store || st.store;
+  if (!any_store) throw Error("fused group starting at '" + g.stages.front().kname + "' produces nothing");
+  if (!g.has_reduce()) return ge.emit_flat(elems);
+  return ge.emit_rows(elems);
+}
+
+// One thread per output element, the reduce loop runs serially inside it.  Used when the
+// reduce axis is not the contiguous one: adjacent threads then read adjacent addresses.
+LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt) {
+  LaunchSpec ls;
+  std::vector<Loop> live;
+  std::map<std::string, NodePtr> zero;
+  for (const auto& l : k.loops) {
+    if (l.extent == 0) throw Error("kernel '" + k.name + "' has an empty loop");
+    if (l.extent == 1) zero[l.var] = make_i64(0);
+    else live.push_back(l);
+  }
+  if (k.rloop.extent == 0) throw Error("kernel '" + k.name + "' reduces over an empty axis");
+  int64_t N = 1;
+  for (const auto& l : live) N *= l.extent;
+  bool idx64 = false;
+  {
+    std::vector<LoadRef> loads;
+    collect_loads(*k.value, loads);
+    int64_t reach = max_abs_index(*k.out_aff, k.loops, &k.rloop);
+    for (const auto& lr : loads) {
+      auto a = affine_of(*lr.load->args[1]);
+      if (!a) { idx64 = true; break; }
+      reach = std::max(reach, max_abs_index(*a, k.loops, &k.rloop));
+    }
+    if (reach >= (int64_t{1} << 31) - 8 || N >= (int64_t{1} << 31) - 8) idx64 = true;
+  }
+  const int block = 256;
+  const int64_t blocks = (N + block - 1) / block;
+  if (blocks >= (int64_t{1} << 31)) throw Error("too many outputs for one launch");
+  ls.entry = "ehk_" + k.name;
+  ls.kernels = {k.name};
+  ls.schedule = "serial-reduce(block=256)";
+  ls.grid[0] = static_cast<unsigned>(blocks);
+  ls.block[0] = block;
+  std::ostringstream os;
+  os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+  os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(";
+  bool first = true;
+  for (const auto& p : k.params) {
+    os << (first ? "" : ", ") << (p.mut_ ? "" : "const ") << ctype(p.dtype.elem()) << "* __restrict__ " << p.name;
+    first = false;
+    ls.arg_bufs.push_back(p.name);
+  }
+  os << ") {\n  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
+  os << "  idx_t eh_rem = eh_o;\n";
+  for (size_t i = live.size(); i-- > 0;) {
+    os << "  const idx_t " << live[i].var << " = eh_rem % " << live[i].extent << ";\n";
+    if (i) os << "  eh_rem /= " << live[i].extent << ";\n";
+  }
+  for (const auto& z : zero) os << "  const idx_t " << z.first << " = 0;\n";
+  ExprRenderer er;
+  const std::string TA = ctype(k.acc_dtype);
+  os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+  os << "  for (idx_t " << k.rloop.var << " = 0; " << k.rloop.var << " < " << k.rloop.extent << "; ++" << k.rloop.var << ") {\n";
+  os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
+  NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
+  os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
+  ls.source = os.str();
+  {
+    std::map<std::string, int64_t> need;
+    std::vector<LoadRef> loads;
+    collect_loads(*k.value, loads);
+    bool opaque = false;
+    for (const auto& lr : loads) {
+      auto a = affine_of(*lr.load->args[1]);
+      if (!a) { opaque = true; continue; }
+      auto& n = need[lr.load->args[0]->name];
+      n = std::max(n, max_abs_index(*a, k.loops, &k.rloop) + 1);
+    }
+    need[k.out_buf] = max_abs_index(*k.out_aff, k.loops, nullptr) + 1;
+    for (const auto& p : k.params) {
+      auto it = need.find(p.name);
+      ls.arg_min_bytes.push_back(it == need.end() || (opaque && !p.mut_) ? 0 : static_cast<size_t>(it->second) * p.dtype.elem().itemsize());
+    }
+  }
+  return ls;
+}
+
+}  // namespace
+
+}  // namespace eh

@@ -1,0 +1,65 @@
+// AST -> HIP C for gfx950 (CDNA4).  Takes the place the reference gives a backend's Renderer
+// (src/backend/renderer.rs:20-35, 69-159; crates/backend-cuda/src/renderer.rs for the GPU
+// shape of it), but chooses a wave64 schedule from the kernel's structure instead of
+// replaying its loops: flat 128-bit elementwise, row programs with DPP + LDS reductions,
+// per-output serial reductions, FP32 MFMA contractions.
+#pragma once
+
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "analysis.hpp"
+#include "ast.hpp"
+
+namespace eh {
+
+struct GenOptions {
+  std::string arch = "gfx950";
+  bool fuse = true;          // merge compatible kernels of a Program into one launch
+  bool vectorize = true;     // 128-bit accesses where alignment allows
+  int row_threads = 0;       // threads cooperating on one row; 0 = choose from the row length
+  int row_elems = 16;        // target elements per thread per row when choosing row_threads
+  int flat_block = 256;
+  int flat_iters = 4;        // vectors handled by one thread of a flat kernel
+  int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
+  bool gemm = true;          // use the MFMA contraction schedule when the shape allows
+  bool nontemporal = false;  // streaming stores for outputs
+};
+
+struct LaunchSpec {
+  std::string entry;
+  std::string source;        // complete translation unit for hiprtc
+  std::string schedule;      // human-readable schedule tag, e.g. "row(T=256,V=4,reg)"
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {1, 1, 1};
+  unsigned lds_bytes = 0;
+  std::vector<std::string> arg_bufs;   // buffer name per kernel parameter, in order
+  std::vector<size_t> arg_min_bytes;   // smallest buffer each parameter may bind (0 = unknown)
+  std::vector<std::string> kernels;    // names of the lowered kernels this launch covers
+  double algo_bytes = 0;               // bytes of each distinct external buffer touched once
+  double flops = 0;
+};
+
+struct ProgramPlan {
+  std::vector<LaunchSpec> launches;
+  std::vector<BufferInfo> buffers;     // table (possibly synthesised from kernel params)
+  std::set<std::string> elided;        // temp buffers that never reach memory
+};
+
+// Plans a whole Program (one or more kernels, executed in order).  When the program carries no
+// buffer table every mutable pointer parameter is an output and nothing is elided.
+ProgramPlan plan_program(const Node& program, const GenOptions& opt);
+
+// Statement-by-statement rendering of one kernel, as written (one work-item unless the kernel
+// already carries group/local id parameters).  Used for forms no schedule recognises.
+LaunchSpec render_kernel_as_written(const Node& kernel, const GenOptions& opt);
+
+// Expression text in HIP C (math calls, literals); exposed for tests.
+std::string render_expr_text(const Node& e);
+
+// Shared preamble (vector type, cross-lane reductions).
+const std::string& preamble();
+
+}  // namespace eh

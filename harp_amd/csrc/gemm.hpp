@@ -1,0 +1,34 @@
+// FP32 MFMA schedule for contraction-shaped reduce kernels:
+//   for i, j: acc = 0; for k: acc += A[i,k] * B[k,j]; C[i,j] = acc
+// which is how the reference lowers matmul / linear layers for fp32
+// (src/lowerer/lower.rs:525-571 on the expand-mul-sum graph of examples/matmul_demo.rs:43-60
+// and crates/nn/src/functional/linear.rs:27-56; its own MatMul node only fires for f16,
+// src/opt/graph/suggesters/matmul.rs:60-65).
+#pragma once
+
+#include <optional>
+
+#include "analysis.hpp"
+#include "codegen.hpp"
+
+namespace eh {
+
+struct GemmShape {
+  int64_t M = 0, N = 0, K = 0, batch = 1;
+  std::string a_buf, b_buf, c_buf;
+  int64_t a_m = 0, a_k = 0, a_b = 0, a_off = 0;   // element strides / offset of A
+  int64_t b_k = 0, b_n = 0, b_b = 0, b_off = 0;
+  int64_t c_m = 0, c_n = 0, c_b = 0, c_off = 0;
+};
+
+// Recognises the contraction and returns its strides; nullopt otherwise.
+std::optional<GemmShape> match_gemm(const NestKernel& k);
+
+// True when match_gemm succeeds and the sizes fit one of the tile configurations.
+bool gemm_shaped(const NestKernel& k, const GenOptions& opt);
+
+// HIP source + dispatch for the kernel, or nullopt when it is not a contraction the MFMA
+// schedule covers (the caller then falls back to another schedule).
+std::optional<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt);
+
+}  // namespace eh

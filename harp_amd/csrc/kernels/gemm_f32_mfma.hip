@@ -1,0 +1,186 @@
+// FP32 contraction C[m,n] = sum_k A[m,k] * B[k,n] on CDNA4 matrix cores (gfx950).
+//
+// One workgroup owns a BM x BN tile of C and walks K in steps of BK.  Each wave owns a WM x WN
+// sub-tile as (WM/32) x (WN/32) accumulators of v_mfma_f32_32x32x2_f32.  A and B tiles are
+// staged in LDS k-major ([k][m] and [k][n], rows padded by 4 floats): the MFMA operand for
+// lane l is row k = 2*step + l/32, column l%32 of the wave's slice, so every half-wave reads
+// 32 consecutive floats.  Global loads are 128-bit along whichever axis of the operand is
+// contiguous; an operand whose contiguous axis is k is transposed on its way into LDS.
+// Two LDS buffers: the loads of tile t+1 are in flight while tile t is multiplied, one
+// barrier per step.  Workgroup ids are remapped so that each XCD (ids congruent mod 8) works
+// on a compact block of tiles and shares A/B panels through its own L2.
+//
+// The generator defines the EH_* macros; the defaults below make the file compile on its own.
+#ifndef __HIPCC_RTC__
+#include <hip/hip_runtime.h>
+#endif
+
+#ifndef EH_ENTRY
+#define EH_ENTRY ehk_gemm_default
+#define EH_M 4096
+#define EH_N 4096
+#define EH_K 4096
+#define EH_BATCH 1
+#define EH_BM 128
+#define EH_BN 128
+#define EH_BK 32
+#define EH_WM 64
+#define EH_WN 64
+#define EH_A_KCONTIG 1
+#define EH_B_NCONTIG 1
+#define EH_LDA 4096
+#define EH_LDB 4096
+#define EH_LDC 4096
+#define EH_A_OFF 0
+#define EH_B_OFF 0
+#define EH_C_OFF 0
+#define EH_A_BS 0
+#define EH_B_BS 0
+#define EH_C_BS 0
+#define EH_GROUP_M 8
+#endif
+
+typedef float eh_f16v __attribute__((ext_vector_type(16)));
+typedef float eh_f4v __attribute__((ext_vector_type(4)));
+
+namespace {
+constexpr int BM = EH_BM, BN = EH_BN, BK = EH_BK, WM = EH_WM, WN = EH_WN;
+constexpr int NWM = BM / WM, NWN = BN / WN, NT = NWM * NWN * 64;
+constexpr int AS = BM + 4, BS = BN + 4;            // padded LDS row lengths
+constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 128-bit loads per thread per tile
+constexpr int IB = WM / 32, JB = WN / 32;
+constexpr int TM = EH_M / BM, TN = EH_N / BN, NTILES = TM * TN, KT = EH_K / BK;
+static_assert(EH_M % BM == 0 && EH_N % BN == 0 && EH_K % BK == 0, "sizes must be multiples of the tile");
+static_assert(BM * BK % (4 * NT) == 0 && BN * BK % (4 * NT) == 0 && AV >= 1 && BV >= 1, "tile does not split over the threads");
+static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 2 == 0, "wave tile must be built from 32x32x2 MFMAs");
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restrict__ A,
+                                                          const float* __restrict__ B,
+                                                          float* __restrict__ C) {
+  __shared__ float As[2][BK * AS];
+  __shared__ float Bs[2][BK * BS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wid = tid >> 6;
+  const int wm = wid / NWN, wn = wid % NWN;
+  const int l32 = lane & 31, kh = lane >> 5;
+
+  // workgroup -> tile: compact per XCD, then grouped along M so neighbours share B panels
+  int tile = blockIdx.x;
+  if (NTILES % 8 == 0) tile = (tile % 8) * (NTILES / 8) + tile / 8;
+  constexpr int GM = EH_GROUP_M < TM ? EH_GROUP_M : TM;
+  const int group = tile / (GM * TN);
+  const int first_m = group * GM;
+  const int gsz = (TM - first_m) < GM ? (TM - first_m) : GM;
+  const int in_g = tile - group * GM * TN;
+  const int tm = first_m + in_g % gsz;
+  const int tn = in_g / gsz;
+  const long long m0 = (long long)tm * BM, n0 = (long long)tn * BN;
+
+  const long long bz = blockIdx.z;
+  const float* Ab = A + EH_A_OFF + bz * EH_A_BS;
+  const float* Bb = B + EH_B_OFF + bz * EH_B_BS;
+  float* Cb = C + EH_C_OFF + bz * EH_C_BS;
+
+  eh_f4v ra[AV], rb[BV];
+
+  auto gload = [&](int kt) {
+    const long long k0 = (long long)kt * BK;
+#pragma unroll
+    for (int i = 0; i < AV; ++i) {
+      const int q = tid + i * NT;
+#if EH_A_KCONTIG
+      const int m = q / (BK / 4), kq = q % (BK / 4);
+      ra[i] = *reinterpret_cast<const eh_f4v*>(Ab + (m0 + m) * EH_LDA + k0 + kq * 4);
+#else
+      const int k = q / (BM / 4), mq = q % (BM / 4);
+      ra[i] = *reinterpret_cast<const eh_f4v*>(Ab + (k0 + k) * EH_LDA + m0 + mq * 4);
+#endif
+    }
+#pragma unroll
+    for (int i = 0; i < BV; ++i) {
+      const int q = tid + i * NT;
+#if EH_B_NCONTIG
+      const int k = q / (BN / 4), nq = q % (BN / 4);
+      rb[i] = *reinterpret_cast<const eh_f4v*>(Bb + (k0 + k) * EH_LDB + n0 + nq * 4);
+#else
+      const int n = q / (BK / 4), kq = q % (BK / 4);
+      rb[i] = *reinterpret_cast<const eh_f4v*>(Bb + (n0 + n) * EH_LDB + k0 + kq * 4);
+#endif
+    }
+  };
+
+  auto sstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < AV; ++i) {
+      const int q = tid + i * NT;
+#if EH_A_KCONTIG
+      const int m = q / (BK / 4), kq = q % (BK / 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) As[buf][(kq * 4 + e) * AS + m] = ra[i][e];
+#else
+      const int k = q / (BM / 4), mq = q % (BM / 4);
+      *reinterpret_cast<eh_f4v*>(&As[buf][k * AS + mq * 4]) = ra[i];
+#endif
+    }
+#pragma unroll
+    for (int i = 0; i < BV; ++i) {
+      const int q = tid + i * NT;
+#if EH_B_NCONTIG
+      const int k = q / (BN / 4), nq = q % (BN / 4);
+      *reinterpret_cast<eh_f4v*>(&Bs[buf][k * BS + nq * 4]) = rb[i];
+#else
+      const int n = q / (BK / 4), kq = q % (BK / 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) Bs[buf][(kq * 4 + e) * BS + n] = rb[i][e];
+#endif
+    }
+  };
+
+  eh_f16v acc[IB][JB];
+#pragma unroll
+  for (int i = 0; i < IB; ++i)
+#pragma unroll
+    for (int j = 0; j < JB; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  gload(0);
+  sstore(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) gload(kt + 1);
+    const float* as = &As[buf][wm * WM + l32];
+    const float* bs = &Bs[buf][wn * WN + l32];
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float a[IB], b[JB];
+#pragma unroll
+      for (int i = 0; i < IB; ++i) a[i] = as[(kk + kh) * AS + i * 32];
+#pragma unroll
+      for (int j = 0; j < JB; ++j) b[j] = bs[(kk + kh) * BS + j * 32];
+#pragma unroll
+      for (int i = 0; i < IB; ++i)
+#pragma unroll
+        for (int j = 0; j < JB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) sstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
+#pragma unroll
+  for (int i = 0; i < IB; ++i)
+#pragma unroll
+    for (int j = 0; j < JB; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const long long row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
+        const long long col = n0 + wn * WN + j * 32 + l32;
+        Cb[row * EH_LDC + col] = acc[i][j][r];
+      }
+}

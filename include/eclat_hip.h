@@ -1,0 +1,144 @@
+/* C ABI of libeclat_hip: the MI355X (gfx950) kernel backend for the eclat tensor compiler.
+ *
+ * These entry points are what a `crates/backend-hip` in the reference workspace binds to
+ * implement the reference's backend traits; each group cites the trait methods it stands for
+ * (paths relative to the reference repository).  All functions are thread-safe, return 0 on
+ * success and a non-zero EH_ERR_* code otherwise; eh_last_error() then gives the message of the
+ * calling thread's most recent failure.  Handles are opaque.  No function takes or returns a
+ * framework tensor type: only plain pointers, sizes and NUL-terminated strings.
+ *
+ * Kernel ASTs travel as text, e.g.
+ *   (program (kernel "E_4_0" (params ("buf0" (ptr f32 global) imm normal) ...) (grid ...) (tg ...)
+ *     (range "ridx0" (const i64 0) (const i64 1) (const i64 4) (store (var "buf4") ... ) sequential)))
+ * one s-expression per reference `AstNode` variant (src/ast/mod.rs:107-385).
+ */
+#ifndef ECLAT_HIP_H
+#define ECLAT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EH_OK 0
+#define EH_ERR_INVALID 1   /* bad argument / handle */
+#define EH_ERR_PARSE 2     /* malformed AST text or options */
+#define EH_ERR_UNSUPPORTED 3
+#define EH_ERR_COMPILE 4   /* hiprtc rejected generated or given source */
+#define EH_ERR_DEVICE 5    /* HIP runtime error, or no device */
+#define EH_ERR_SIZE 6      /* buffer size mismatch */
+
+typedef struct eh_device eh_device;
+typedef struct eh_buffer eh_buffer;
+typedef struct eh_program eh_program;   /* one or more launches compiled from a Program AST */
+typedef struct eh_plan eh_plan;         /* rendered sources + dispatch, no device involved */
+typedef struct eh_event eh_event;
+
+/* ---- library ---------------------------------------------------------------------------- */
+int eh_version(void);                   /* 100 * major + minor */
+const char* eh_last_error(void);        /* valid until the calling thread's next failing call */
+void eh_free(void* p);                  /* releases memory handed out by eh_compile_source */
+
+/* ---- BackendRegistry: kind/name/is_available/list_devices/create_device
+ *      (src/backend/device.rs:83-131), Device::profile (src/backend/traits.rs:273-306) ------- */
+typedef struct eh_device_props {
+  char name[128];
+  char arch[32];                        /* "gfx950" */
+  int compute_units;
+  int warp_size;                        /* 64 */
+  int max_work_group_size;
+  size_t local_memory_size;             /* LDS bytes per compute unit */
+  size_t global_memory_size;
+  int clock_khz;
+  int memory_clock_khz;
+  int memory_bus_bits;
+  int l2_bytes;
+} eh_device_props;
+
+int eh_device_count(int* count);        /* 0 devices is not an error */
+int eh_device_open(int index, eh_device** out);
+int eh_device_close(eh_device* dev);    /* buffers and programs of the device must be gone */
+int eh_device_get_props(eh_device* dev, eh_device_props* out);
+int eh_device_sync(eh_device* dev);     /* waits for everything queued on the device's stream */
+
+/* ---- Buffer: allocate (zero-filled), byte_len, write_from_host (size must match exactly),
+ *      read_to_host, clone_buffer (src/backend/traits.rs:455-482;
+ *      crates/backend-c/src/buffer.rs:84-131); BackendRegistry::allocate_buffer
+ *      (src/backend/device.rs:132-134) -------------------------------------------------------- */
+int eh_buffer_alloc(eh_device* dev, size_t bytes, eh_buffer** out);
+int eh_buffer_retain(eh_buffer* buf);
+int eh_buffer_release(eh_buffer* buf);
+int eh_buffer_bytes(eh_buffer* buf, size_t* bytes);
+int eh_buffer_write(eh_buffer* buf, const void* src, size_t bytes);
+int eh_buffer_read(eh_buffer* buf, void* dst, size_t bytes);
+int eh_buffer_copy(eh_buffer* dst, eh_buffer* src);        /* device-to-device, same size */
+int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
+
+/* ---- Renderer: AST -> source + dispatch sizes, no device needed
+ *      (src/backend/renderer.rs:20-35; KernelSourceRenderer and extract_kernel_config,
+ *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
+ *      arch, fuse, vectorize, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
+ *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, nontemporal. ---------------------------------------- */
+typedef struct eh_launch_info {
+  const char* entry;                    /* kernel symbol */
+  const char* source;                   /* HIP C translation unit */
+  const char* schedule;                 /* e.g. "row(T=256,V=4,NV=4,reg,rows/block=1)" */
+  unsigned grid[3];                     /* workgroups */
+  unsigned block[3];                    /* work-items per workgroup */
+  unsigned lds_bytes;                   /* dynamic LDS */
+  int n_args;                           /* pointer parameters, see eh_plan_launch_arg */
+  int n_kernels;                        /* lowered kernels covered by this launch */
+  double algo_bytes;                    /* each distinct external buffer counted once */
+  double flops;                         /* 2*M*N*K for contractions, else 0 */
+} eh_launch_info;
+
+int eh_render_program(const char* ast_text, const char* options, eh_plan** out);
+int eh_plan_num_launches(eh_plan* plan, int* n);
+int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out);    /* strings live as long as the plan */
+int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name);
+int eh_plan_launch_kernel(eh_plan* plan, int launch, int k, const char** kernel_name);
+int eh_plan_num_buffers(eh_plan* plan, int* n);
+int eh_plan_buffer(eh_plan* plan, int i, const char** name, const char** role, size_t* bytes, int* elided);
+int eh_plan_release(eh_plan* plan);
+
+/* ---- Compiler: source -> code object with hiprtc for `arch` (NULL = gfx950), no device needed
+ *      (Compiler::compile, src/backend/traits.rs:592-607; crates/backend-c/src/compiler.rs:101-165).
+ *      *blob is released with eh_free. ----------------------------------------------------------- */
+int eh_compile_source(const char* source, const char* arch, void** blob, size_t* len);
+
+/* ---- BackendRegistry::compile_ast + Kernel (src/backend/device.rs:136-160;
+ *      src/backend/traits.rs:531-587): compile a Program AST for a device and run it.
+ *      A program made of one kernel without a buffer table is the per-kernel drop-in:
+ *      eh_program_execute_positional == Kernel::execute(inputs, outputs).  A program with a
+ *      buffer table `(buffers ("name" dtype (shape ...) input|output|temp) ...)` is compiled
+ *      as a whole: kernels are fused where possible and temps that never reach memory are
+ *      reported as elided. ------------------------------------------------------------------------ */
+int eh_program_compile(eh_device* dev, const char* ast_text, const char* options, eh_program** out);
+int eh_program_release(eh_program* prog);
+int eh_program_num_buffers(eh_program* prog, int* n);
+int eh_program_buffer(eh_program* prog, int i, const char** name, const char** role, size_t* bytes, int* elided);
+int eh_program_num_launches(eh_program* prog, int* n);
+int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
+/* bufs[i] binds buffer i of the table; NULL is allowed for elided buffers and for temps (the
+ * program then keeps its own).  sync != 0 waits for completion (the reference's kernels are
+ * synchronous); sync == 0 only queues the launches on the device's stream. */
+int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
+int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,
+                                  eh_buffer* const* outputs, int n_outputs, int sync);
+/* Kernel::get_binary / BackendRegistry::compile_from_binary (src/backend/traits.rs:576-586,
+ * src/backend/device.rs:161-170): the gfx950 code object of one launch. */
+int eh_program_binary(eh_program* prog, int launch, const void** blob, size_t* len);
+
+/* ---- timing on the device's stream (HIP events) ------------------------------------------------ */
+int eh_event_create(eh_device* dev, eh_event** out);
+int eh_event_record(eh_event* ev);          /* on the device's stream */
+int eh_event_sync(eh_event* ev);
+int eh_event_elapsed_ms(eh_event* start, eh_event* stop, float* ms);
+int eh_event_release(eh_event* ev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ECLAT_HIP_H */

@@ -125,6 +125,7 @@ class CBackend:
     def __init__(self, openmp: bool = False):
         self.kind = "openmp" if openmp else "c"
         self.openmp = openmp
+        self._devices = {}
 
     def name(self) -> str:
         return "OpenMP (oracle)" if self.openmp else "C (oracle)"
@@ -133,7 +134,7 @@ class CBackend:
         return True
 
     def create_device(self, index: int):
-        return ("cpu", index)
+        return self._devices.setdefault(index, ("cpu", index))
 
     def list_devices(self) -> List[str]:
         return ["cpu"]

@@ -1,0 +1,226 @@
+"""Parity of the HIP backend with the CPU oracle on identical seeded inputs.
+Every case goes through the C ABI (ctypes -> libeclat_hip.so).
+
+Tolerance classes (written where they are applied):
+  * add / mul / max / select / compare / cast / copies / indexing: bit-exact
+    (up to the sign of zero and flushed denormals: the oracle is gcc -ffast-math);
+  * recip / sqrt / exp2 / log2 / sin: 4 ulp-class, rtol 1e-6 (libm vs device libm);
+  * reductions (incl. softmax): rtol 1e-5;
+  * K=4096 MFMA matmul: rtol 1e-3 of the row scale.
+"""
+
+import numpy as np
+import pytest
+
+from conftest import bits_equal_mod_zero, realize_on
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng
+
+
+def both(fe, build, arrays, fuse=True):
+    ref = realize_on(fe, "c", build, arrays)
+    got = realize_on(fe, "hip", build, arrays, fuse=fuse)
+    return ref, got
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_reference_known_answers(frontend, hip, fuse):
+    a = np.array([1, 2, 3, 4], dtype=np.float32)
+    b = np.array([5, 6, 7, 8], dtype=np.float32)
+    assert realize_on(frontend, "hip", lambda x, y: x + y, [a, b], fuse=fuse).tolist() == [6, 8, 10, 12]
+    b2 = np.array([2, 3, 4, 5], dtype=np.float32)
+    assert realize_on(frontend, "hip", lambda x, y: x * y, [a, b2], fuse=fuse).tolist() == [2, 6, 12, 20]
+    m1 = np.array([[1, 2], [3, 4]], dtype=np.float32)
+    m2 = np.array([[5, 6], [7, 8]], dtype=np.float32)
+    out = realize_on(frontend, "hip", lambda x, y: frontend.nn.matmul(x, y), [m1, m2], fuse=fuse)
+    assert out.tolist() == [19, 22, 43, 50]
+
+
+ELEMENTWISE = {
+    "mul_add": lambda a, b, c: a * b + c,
+    "relu_chain": lambda a, b, c: (a * b + c).maximum(c) - a,
+    "neg_min": lambda a, b, c: (-a).minimum(b) * c,
+    "where": lambda a, b, c: a.where_cond(a.lt(b), c),
+    "abs": lambda a, b, c: a.abs() + b * c,
+}
+
+
+@pytest.mark.parametrize("shape", [(1,), (7,), (37, 53), (64, 128), (3, 5, 8), (1000, 1024)])
+@pytest.mark.parametrize("name", sorted(ELEMENTWISE))
+@pytest.mark.parametrize("fuse", [False, True])
+def test_elementwise_bit_exact(frontend, hip, shape, name, fuse):
+    rng = RNG(hash((shape, name)) % 2**32)
+    arrs = [rng.normal(0, 1, shape).astype(np.float32) for _ in range(3)]
+    ref, got = both(frontend, ELEMENTWISE[name], arrs, fuse)
+    assert bits_equal_mod_zero(ref, got)
+
+
+@pytest.mark.parametrize("op", ["sqrt", "recip", "exp", "ln", "sin", "cos", "exp2", "log2"])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_transcendental_elementwise(frontend, hip, op, fuse):
+    x = RNG(5).uniform(0.1, 9.0, (33, 65)).astype(np.float32)
+    ref, got = both(frontend, lambda t: getattr(t, op)(), [x], fuse)
+    assert np.allclose(got, ref, rtol=1e-6, atol=1e-6)
+
+
+def test_floor_and_cast_bit_exact(frontend, hip):
+    x = RNG(6).normal(0, 50, (17, 19)).astype(np.float32)
+    ref, got = both(frontend, lambda t: t.floor(), [x])
+    assert bits_equal_mod_zero(ref, got)
+
+
+@pytest.mark.parametrize("shape,axis", [((8, 10), 1), ((33, 1000), 1), ((16, 4096), 1), ((5, 7, 64), 2),
+                                        ((64, 48), 0), ((9, 130, 6), 1), ((1, 17), 1), ((17, 1), 1),
+                                        ((300, 70000), 1)])
+@pytest.mark.parametrize("op", ["sum", "max", "min", "prod"])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_reductions(frontend, hip, shape, axis, op, fuse):
+    rng = RNG(hash((shape, axis, op)) % 2**32)
+    if op == "prod":
+        x = rng.uniform(0.97, 1.03, shape).astype(np.float32)
+    else:
+        x = rng.normal(0, 1, shape).astype(np.float32)
+    ref, got = both(frontend, lambda t: getattr(t, op)(axis), [x], fuse)
+    if op in ("max", "min"):
+        assert bits_equal_mod_zero(ref, got)          # order-independent, exact
+    else:
+        scale = np.abs(x).sum(axis).ravel() if op == "sum" else np.abs(ref)
+        assert np.all(np.abs(got - ref) <= 1e-5 * np.maximum(scale, 1e-30))   # rel-err 1e-5
+
+
+@pytest.mark.parametrize("shape", [(8, 10), (33, 1000), (128, 4096), (4, 6, 50), (2, 100000)])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_softmax_and_log_softmax(frontend, hip, shape, fuse):
+    x = RNG(len(shape) * 1000 + shape[-1]).normal(0, 2, shape).astype(np.float32)
+    ax = len(shape) - 1
+    ref, got = both(frontend, lambda t: frontend.nn.softmax(t, ax), [x], fuse)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-9)             # reduction class
+    assert np.allclose(got.reshape(-1, shape[-1]).sum(1), 1.0, atol=1e-5)
+    ref, got = both(frontend, lambda t: frontend.nn.log_softmax(t, ax), [x], fuse)
+    assert np.allclose(got, ref, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_config1_fused_elementwise_reduce(frontend, hip, fuse):
+    """BASELINE config 1: s = sum(relu(a*b + c), -1), fp32 [1024,1024], N(0,1)."""
+    rng = RNG(1234)
+    a, b, c = (rng.normal(0, 1, (1024, 1024)).astype(np.float32) for _ in range(3))
+    ref, got = both(frontend, lambda x, y, z: frontend.nn.relu(x * y + z).sum(1), [a, b, c], fuse)
+    assert np.allclose(got, ref, rtol=1e-5)
+    assert np.all(got >= 0)
+
+
+def test_config2_row_softmax_full_size(frontend, hip):
+    """BASELINE config 2: row softmax of fp32 [4096,4096], N(0, std 2)."""
+    x = RNG(1235).normal(0, 2, (4096, 4096)).astype(np.float32)
+    ref, got = both(frontend, lambda t: frontend.nn.softmax(t, 1), [x])
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-12)
+    got2 = got.reshape(4096, 4096)
+    assert np.allclose(got2.sum(1), 1.0, atol=1e-5)
+    assert np.array_equal(got2.argmax(1), x.argmax(1))
+
+
+@pytest.mark.parametrize("m,k,n", [(4, 3, 2), (64, 64, 64), (128, 256, 128), (256, 96, 192), (100, 60, 36),
+                                   (512, 1024, 256)])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_matmul_small(frontend, hip, m, k, n, fuse):
+    rng = RNG(m * 7 + k * 3 + n)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    ref, got = both(frontend, lambda x, y: frontend.nn.matmul(x, y), [a, b], fuse)
+    scale = (np.abs(a) @ np.abs(b)).ravel()
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale + 1e-30)
+
+
+@pytest.mark.parametrize("batch,kin,kout", [(8, 12, 5), (256, 128, 64), (128, 320, 192)])
+def test_linear_layer(frontend, hip, batch, kin, kout):
+    rng = RNG(batch + kin + kout)
+    x = rng.uniform(-1, 1, (batch, kin)).astype(np.float32)
+    w = rng.uniform(-1, 1, (kout, kin)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (kout,)).astype(np.float32)
+    ref, got = both(frontend, lambda t, u, v: frontend.nn.linear(t, u, v), [x, w, bias])
+    scale = (np.abs(x) @ np.abs(w.T) + np.abs(bias)).ravel()
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale)
+
+
+def test_config3_matmul_4096(frontend, hip):
+    """BASELINE config 3: C = A@B, fp32 4096^3, U(-1,1).  The C oracle runs a row subset
+    (64 rows of A, 2 GFLOP); float64 numpy covers every row."""
+    rng = RNG(1236)
+    a = rng.uniform(-1, 1, (4096, 4096)).astype(np.float32)
+    b = rng.uniform(-1, 1, (4096, 4096)).astype(np.float32)
+    got = realize_on(frontend, "hip", lambda x, y: frontend.nn.matmul(x, y), [a, b]).reshape(4096, 4096)
+    rows = np.sort(rng.choice(4096, 64, replace=False))
+    ref_rows = realize_on(frontend, "c", lambda x, y: frontend.nn.matmul(x, y), [a[rows].copy(), b])
+    ref_rows = ref_rows.reshape(64, 4096)
+    scale = np.abs(a[rows]) @ np.abs(b)
+    assert np.all(np.abs(got[rows] - ref_rows) <= 1e-3 * scale)                   # north-star bound
+    assert np.max(np.abs(got[rows] - ref_rows) / scale) < 1e-5                    # what is observed
+    ref64 = a.astype(np.float64) @ b.astype(np.float64)
+    err = np.abs(got - ref64) / (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64))
+    assert err.max() < 1e-5
+
+
+INDEX_FORMS = {
+    "transpose": lambda t: t.permute([1, 0]).contiguous(),
+    "broadcast": lambda t: t.unsqueeze(0).expand(0, 3).contiguous(),
+    "pad": lambda t: t.pad([(1, 2), (0, 1)]).contiguous(),
+    "reshape_sum": lambda t: t.reshape([3, 8]).sum(1),
+    "cumsum": lambda t: t.cumsum(1),
+    "cummax": lambda t: t.cummax(0),
+    "unfold": lambda t: t.unfold([0, 1], [2, 3], [1, 1], [1, 1]).contiguous(),
+    "fold_unfold": lambda t: t.unfold([0, 1], [2, 2], [2, 2], [1, 1]).fold([4, 6], [0, 1], [2, 2], [2, 2], [1, 1]),
+    "neg_transposed": lambda t: (-t.permute([1, 0])).contiguous(),
+}
+
+
+@pytest.mark.parametrize("name", sorted(INDEX_FORMS))
+@pytest.mark.parametrize("fuse", [False, True])
+def test_index_forms_bit_exact(frontend, hip, name, fuse):
+    x = RNG(11).normal(0, 1, (4, 6)).astype(np.float32)
+    ref, got = both(frontend, INDEX_FORMS[name], [x], fuse)
+    if name in ("cumsum",):
+        assert np.allclose(got, ref, rtol=1e-6)
+    else:
+        assert bits_equal_mod_zero(ref, got)
+
+
+def test_buffer_roundtrip_and_size_check(hip):
+    dev = hip.HipDevice(0)
+    from harp_amd.frontend import F32
+    buf = hip.HipBuffer(dev, [5, 3], F32)
+    assert buf.read_array(np.float32).tolist() == [0.0] * 15            # zero-filled
+    data = np.arange(15, dtype=np.float32)
+    buf.write_from_host(data.tobytes())
+    assert np.array_equal(buf.read_array(np.float32), data)
+    clone = buf.clone_buffer()
+    assert np.array_equal(clone.read_array(np.float32), data)
+    with pytest.raises(hip.EhError) as e:
+        buf.write_from_host(b"\0" * 8)
+    assert "Buffer size mismatch" in str(e.value)
+    assert dev.props["arch"].startswith("gfx9") and dev.props["warp_size"] == 64
+
+
+def test_undersized_buffer_is_rejected_before_launch(frontend, hip):
+    dev = hip.HipDevice(0)
+    a = frontend.Tensor.input([64, 64])
+    prog, _, _ = frontend.lower_graph([(a + a).graph])
+    k = hip.HipKernel(dev, prog)
+    small = hip.HipBuffer(dev, [16], frontend.F32)
+    full = hip.HipBuffer(dev, [64, 64], frontend.F32)
+    with pytest.raises(hip.EhError) as e:
+        k.execute([small], [full])
+    assert "Buffer size mismatch" in str(e.value)
+    with pytest.raises(hip.EhError):
+        k.execute([full, full], [full])                      # wrong argument count
+
+
+def test_kernel_binary_round_trip(frontend, hip):
+    dev = hip.HipDevice(0)
+    a = frontend.Tensor.input([256])
+    prog, _, _ = frontend.lower_graph([(a * a).graph])
+    k = hip.HipKernel(dev, prog)
+    blob = k.get_binary()
+    assert blob[:4] == b"\x7fELF" and len(blob) > 1000

@@ -1,0 +1,216 @@
+"""Host-side checks that need no GPU: the C ABI exports what the header declares, the AST
+reader, the renderer's schedules for the BASELINE configs, hiprtc compilation for gfx950,
+and the front end's lowering structure."""
+
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from harp_amd import _lib
+    with open(os.path.join(ROOT, "include", "eclat_hip.h")) as f:
+        header = f.read()
+    declared = set(re.findall(r"\b(eh_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found"
+    for name in sorted(declared):
+        assert hasattr(_lib.lib, name), f"{name} declared in eclat_hip.h but not exported"
+    assert declared == set(_lib.EXPORTED)
+    assert _lib.lib.eh_version() >= 100
+
+
+def _program_with_table(fe, tensor):
+    from harp_amd.frontend.executor import buffer_table
+    from harp_amd.frontend.graph import collect_inputs
+    prog, lw, _ = fe.lower_graph([tensor.graph])
+    ins = [lw.lookup_buffer_name(n) for n in collect_inputs([tensor.graph])]
+    outs = [p.name for k in prog.args for p in k.attrs["params"] if p.mutable]
+    last = max(outs, key=lambda s: int(s[3:]))
+    return fe.AstNode.program(prog.args, buffers=buffer_table(prog, lw, ins, [last]))
+
+
+def test_config2_softmax_is_one_row_kernel(frontend):
+    from harp_amd import backend as hb
+    x = frontend.Tensor.input([4096, 4096])
+    plan = hb.render_program(_program_with_table(frontend, frontend.nn.softmax(x, 1)))
+    assert len(plan.launches) == 1
+    l = plan.launches[0]
+    assert l["schedule"].startswith("row(") and "V=4" in l["schedule"] and "reg" in l["schedule"]
+    assert l["kernels"] == ["R_4096_1_0", "E_4096_4096_1", "E_4096_4096_2", "R_4096_1_3", "E_4096_4096_4"]
+    assert l["algo_bytes"] == 2 * 4096 * 4096 * 4                 # one read + one write
+    assert l["grid"][0] * (l["block"][0] // int(re.search(r"T=(\d+)", l["schedule"]).group(1))) >= 4096
+    assert sum(b["elided"] for b in plan.buffers) == 4            # max, shifted, exp, sum never reach HBM
+    assert "eh_row_reduce<EhMax" in l["source"] and "eh_row_reduce<EhSum" in l["source"]
+    assert len(hb.compile_source(l["source"])) > 1000             # hiprtc -> gfx950 code object
+
+
+def test_config1_fuses_into_one_launch(frontend):
+    from harp_amd import backend as hb
+    a, b, c = (frontend.Tensor.input([1024, 1024]) for _ in range(3))
+    plan = hb.render_program(_program_with_table(frontend, frontend.nn.relu(a * b + c).sum(1)))
+    assert len(plan.launches) == 1 and plan.launches[0]["kernels"][-1].startswith("R_1024_1")
+    # separate graph nodes keep separate roundings: no fused multiply-add in the text
+    assert "fmaf" not in plan.launches[0]["source"]
+    assert len(hb.compile_source(plan.launches[0]["source"])) > 1000
+
+
+def test_config3_matmul_takes_the_mfma_schedule(frontend):
+    from harp_amd import backend as hb
+    a, b = frontend.Tensor.input([4096, 4096]), frontend.Tensor.input([4096, 4096])
+    plan = hb.render_program(_program_with_table(frontend, frontend.nn.matmul(a, b)))
+    assert len(plan.launches) == 1
+    l = plan.launches[0]
+    assert l["schedule"].startswith("mfma32x32x2(") and l["flops"] == 2.0 * 4096 ** 3
+    assert "__builtin_amdgcn_mfma_f32_32x32x2f32" in l["source"]
+    assert len(hb.compile_source(l["source"])) > 1000
+    # option fuse=0 / gemm=0 fall back to other schedules and still compile
+    plan2 = hb.render_program(_program_with_table(frontend, frontend.nn.matmul(a, b)), {"gemm": 0})
+    assert not plan2.launches[0]["schedule"].startswith("mfma")
+
+
+def test_unfused_per_kernel_rendering(frontend):
+    from harp_amd import backend as hb
+    x = frontend.Tensor.input([64, 100])
+    prog, _, _ = frontend.lower_graph([frontend.nn.softmax(x, 1).graph])
+    assert [k.attrs["name"][0] for k in prog.args] == ["R", "E", "E", "R", "E"]
+    for k in prog.args:                                          # what compile_ast receives
+        plan = hb.render_program(frontend.AstNode.program([k]))
+        assert len(plan.launches) == 1
+        assert len(hb.compile_source(plan.launches[0]["source"])) > 500
+
+
+def test_as_written_rendering_of_scatter_and_scan(frontend):
+    from harp_amd import backend as hb
+    x = frontend.Tensor.input([4, 4])
+    y = x.unfold([0, 1], [2, 2], [2, 2], [1, 1]).fold([4, 4], [0, 1], [2, 2], [2, 2], [1, 1])
+    prog, _, _ = frontend.lower_graph([y.graph])
+    names = [k.attrs["name"] for k in prog.args]
+    assert names[0].startswith("C_") and names[1].startswith("S_")
+    plan = hb.render_program(prog)
+    assert plan.launches[1]["schedule"] == "as-written" and "atomicAdd" in plan.launches[1]["source"]
+    for l in plan.launches:
+        hb.compile_source(l["source"])
+    prog2, _, _ = frontend.lower_graph([x.cumsum(1).graph])
+    plan2 = hb.render_program(prog2)
+    assert plan2.launches[0]["schedule"] == "as-written"
+    hb.compile_source(plan2.launches[0]["source"])
+
+
+@pytest.mark.parametrize("text,needle", [
+    ("(program", "missing ')'"),
+    ("(program (kernel \"k\" (params) (frobnicate)))", "frobnicate"),
+    ("(bogus 1 2)", "unknown AST node"),
+    ("(program)", "no kernel"),
+    ("(add (const f32 1.0))", "takes 2 operands"),
+])
+def test_malformed_ast_is_reported(text, needle):
+    from harp_amd import backend as hb
+    with pytest.raises(hb.EhError) as e:
+        hb.render_program(text)
+    assert needle in str(e.value)
+
+
+def test_bad_options_and_bad_source_are_reported(frontend):
+    from harp_amd import backend as hb
+    a = frontend.Tensor.input([8])
+    prog, _, _ = frontend.lower_graph([(a + a).graph])
+    with pytest.raises(hb.EhError) as e:
+        hb.render_program(prog, "no_such_option=1")
+    assert "unknown option" in str(e.value)
+    with pytest.raises(hb.EhError) as e:
+        hb.render_program(prog, "row_threads=100")
+    assert "power of two" in str(e.value)
+    with pytest.raises(hb.EhError) as e:
+        hb.compile_source("this is not HIP")
+    assert e.value.code == 4 and "hiprtc" in str(e.value)
+
+
+def test_no_device_is_an_error_not_a_fallback():
+    from harp_amd import backend as hb
+    if hb.device_count() > 0:
+        pytest.skip("a GPU is present")
+    with pytest.raises(hb.EhError) as e:
+        hb.HipDevice(0)
+    assert "no HIP device" in str(e.value)
+    assert not hb.HipBackendRegistry().is_available()
+
+
+def test_lowering_structure(frontend):
+    # src/lowerer/lower.rs:1335-1441: kernel name prefixes, parameter order
+    a = frontend.Tensor.input([32, 64])
+    b = frontend.Tensor.input([32, 64])
+    prog, lw, _ = frontend.lower_graph([(a + b).graph])
+    (k,) = prog.args
+    assert k.attrs["name"] == "E_32_64_0"
+    ps = k.attrs["params"]
+    assert [p.mutable for p in ps] == [False, False, True]
+    assert [p.name for p in ps] == ["buf0", "buf2", "buf4"]      # counter advances by two
+    prog, _, _ = frontend.lower_graph([a.sum(1).graph])
+    assert prog.args[0].attrs["name"].startswith("R_32_1_")
+    # a view with two consumers is materialised by a copy kernel, a single-consumer view is inlined
+    t = a.permute([1, 0])
+    prog, _, _ = frontend.lower_graph([(t + t).graph])
+    assert [k.attrs["name"][0] for k in prog.args] == ["C", "E"]
+    prog, _, _ = frontend.lower_graph([(a.permute([1, 0]) + b.permute([1, 0])).graph])
+    assert [k.attrs["name"][0] for k in prog.args] == ["E"]
+
+
+def test_view_algebra(frontend):
+    # spot checks mirroring src/graph/shape/view.rs tests
+    V, E = frontend.View, frontend.Expr
+    v = V.contiguous([3, 4])
+    assert v.strides == [E.const(4), E.const(1)] and v.is_contiguous()
+    p = v.permute([1, 0])
+    assert p.shape() == [E.const(4), E.const(3)] and p.strides == [E.const(1), E.const(4)]
+    assert not p.is_contiguous() and not p.is_innermost_contiguous()
+    u = v.unsqueeze(0)
+    assert u.shape()[0] == E.const(1) and u.strides[0] == E.const(0)
+    assert u.squeeze(0) == v
+    ex = u.expand(0, 5)
+    assert ex.shape()[0] == E.const(5) and ex.strides[0] == E.const(0)
+    pd = V.padded(v, [(1, 1), (1, 1)], "zero")
+    assert pd.shape() == [E.const(5), E.const(6)] and pd.has_bounds()
+    un = V.contiguous([2, 3, 8, 10]).unfold([2, 3], [3, 3], [1, 1], [1, 1])
+    assert [d.evaluate() for d in un.shape()] == [2, 3, 6, 8, 3, 3]
+    assert V.contiguous([6, 4]).reshape([2, 12]).is_contiguous()
+    with pytest.raises(AssertionError):
+        p.reshape([12])
+
+
+def test_tensor_api_errors(frontend):
+    frontend.clear_default_device()
+    t = frontend.Tensor.input([4])
+    with pytest.raises(frontend.ExecutionError) as e:
+        t.set_data([1, 2, 3, 4])
+    assert "NoDevice" in str(e.value)
+    frontend.set_device_str("c")
+    with pytest.raises(frontend.ExecutionError) as e:
+        t.set_data([1, 2, 3])
+    assert "ShapeMismatch" in str(e.value)
+    u = frontend.Tensor.input([4])
+    with pytest.raises(frontend.ExecutionError) as e:
+        (t + u).realize()
+    assert "MissingInput" in str(e.value)
+    with pytest.raises(frontend.ExecutionError):
+        u.to_vec()
+    with pytest.raises(frontend.DeviceError):
+        frontend.set_device_str("nosuchbackend")
+
+
+def test_kernel_cache_counts(frontend):
+    # crates/backend-c/src/lib.rs:246-297: second realize of the same graph hits the cache
+    frontend.set_device_str("c")
+    frontend.clear_cache()
+    import numpy as np
+    from conftest import realize_on
+    a = np.ones(16, dtype=np.float32)
+    realize_on(frontend, "c", lambda x: x + x, [a])
+    s1 = frontend.cache_stats()
+    realize_on(frontend, "c", lambda x: x + x, [a])
+    s2 = frontend.cache_stats()
+    assert s1["misses"] == 1 and s1["hits"] == 0
+    assert s2["misses"] == 1 and s2["hits"] == 1 and s2["entries"] == 1
