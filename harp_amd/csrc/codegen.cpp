@@ -747,7 +747,8 @@ struct GroupEmitter {
         if (!a) { idx64 = true; continue; }     // opaque index: stay in 64-bit to be safe
         const int64_t top = max_abs_index(*a, loads_loops(loops), &cl);
         reach = std::max(reach, top);
-        need[b] = std::max(need[b], top + 1);
+        // a load under a Select only happens where its bounds condition holds
+        if (!lr.guarded) need[b] = std::max(need[b], top + 1);
         if (!lr.guarded && a->of("c") == 1 && find_ext(b, *a) < 0) {
           ExtLoad e;
           e.buf = b;

