@@ -87,7 +87,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 (default: all)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | copy (default: all but copy)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -130,6 +130,17 @@ def main():
                 "softmax result check failed"
             assert np.allclose(got.sum(1), 1.0, atol=1e-5), "softmax rows do not sum to 1"
         del sets
+
+    # ---- calibration: plain copy of the same size (for counter scaling, not a result) ------
+    if args.only == "copy":
+        wl.CONFIGS["copy"] = (wl.config2_inputs, lambda x: x.contiguous())
+        arrays = wl.config2_inputs()
+        prog, arg_names, out_name, consts = build(dev, hb, wl, "copy", [(4096, 4096)], options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
+        ms, _ = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
+        log(f"[bench] copy 4096^2 ({prog.launches[0]['entry']}, {prog.launches[0]['schedule']}): "
+            f"{ms * 1e3:.1f} us/step -> {2 * 4096 * 4096 * 4 / (ms * 1e-3) / 1e9:.0f} GB/s")
+        return
 
     # ---- config 3: 4096^3 fp32 matmul --------------------------------------------------
     matmul = None

@@ -299,7 +299,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_bk") o.gemm_bk = as_int();
     else if (k == "gemm_wm") o.gemm_wm = as_int();
     else if (k == "gemm_wn") o.gemm_wn = as_int();
-    else if (k == "nontemporal") o.nontemporal = as_int() != 0;
+    else if (k == "nontemporal") o.nontemporal = as_int();
     else throw Error("unknown option '" + k + "'");
   }
   if (o.flat_block < 64 || o.flat_block > 1024 || (o.flat_block & (o.flat_block - 1)))

@@ -17,7 +17,15 @@ namespace eh {
 const std::string& preamble() {
   static const std::string s = R"EHP(
 // wave64 helpers for gfx950
-template <typename T> struct alignas(sizeof(T) * 4) EhV4 { T v[4]; };
+template <typename T> using EhV4 = T __attribute__((ext_vector_type(4)));
+template <bool NT, typename T> __device__ __forceinline__ EhV4<T> eh_load4(const T* p) {
+  if (NT) return __builtin_nontemporal_load(reinterpret_cast<const EhV4<T>*>(p));
+  return *reinterpret_cast<const EhV4<T>*>(p);
+}
+template <bool NT, typename T> __device__ __forceinline__ void eh_store4(T* p, EhV4<T> v) {
+  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<EhV4<T>*>(p));
+  else *reinterpret_cast<EhV4<T>*>(p) = v;
+}
 
 struct EhSum  { template <class T> __device__ __forceinline__ static T f(T a, T b) { return a + b; } };
 struct EhProd { template <class T> __device__ __forceinline__ static T f(T a, T b) { return a * b; } };
@@ -867,6 +875,17 @@ struct GroupEmitter {
     return s;
   }
 
+  // Streaming (non-temporal) hints.  By default only stores of outputs too large to be
+  // re-read from cache by a following kernel are streamed.
+  bool nt_stores() const {
+    if (opt.nontemporal >= 0) return opt.nontemporal >= 1;
+    int64_t bytes = 0;
+    for (const auto& st : g.stages)
+      if (st.store && st.kind == StageKind::Wide) bytes += g.R() * g.C * static_cast<int64_t>(st.out_dtype.itemsize());
+    return bytes >= (int64_t{32} << 20);
+  }
+  bool nt_loads() const { return opt.nontemporal >= 2; }
+
   void fill_min_bytes(LaunchSpec* ls) const {
     for (const auto& b : ls->arg_bufs) {
       size_t item = 4;
@@ -901,8 +920,11 @@ struct GroupEmitter {
     const int block = opt.flat_block;
     int64_t want = (NVEC + static_cast<int64_t>(block) * opt.flat_iters - 1) / (static_cast<int64_t>(block) * opt.flat_iters);
     int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(want, 1 << 20));
+    const char* nt = nt_loads() ? "true" : "false";
+    const char* nts = nt_stores() ? "true" : "false";
     ls.entry = "ehk_" + g.stages.front().kname;
-    ls.schedule = "flat(V=" + std::to_string(V) + ",block=" + std::to_string(block) + ")";
+    ls.schedule = "flat(V=" + std::to_string(V) + ",block=" + std::to_string(block) + (nt_stores() ? ",nt-store" : "") +
+                  (nt_loads() ? ",nt-load" : "") + ")";
     ls.grid[0] = static_cast<unsigned>(blocks);
     ls.block[0] = static_cast<unsigned>(block);
     std::ostringstream os;
@@ -921,19 +943,19 @@ struct GroupEmitter {
     }
     // vector loads
     auto ld = [&](int id) -> std::string {
-      return V == 4 ? "ld" + std::to_string(id) + ".v[v]" : std::string();
+      return V == 4 ? "ld" + std::to_string(id) + "[v]" : std::string();
     };
     if (V == 4)
       for (const auto& e : ext)
-        os << "  const EhV4<" << ctype(e.dtype) << "> ld" << e.id << " = *reinterpret_cast<const EhV4<" << ctype(e.dtype)
-           << ">*>(" << e.buf << " + " << affine_text(e.aff, "c0") << ");\n";
+        os << "  const EhV4<" << ctype(e.dtype) << "> ld" << e.id << " = eh_load4<" << nt << ">(" << e.buf << " + "
+           << affine_text(e.aff, "c0") << ");\n";
     for (const auto& st : g.stages) {
       if (!st.store) continue;
       std::string T = ctype(st.out_dtype);
       if (V == 4) {
-        os << "  { EhV4<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o.v[v] = ("
+        os << "  { EhV4<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o[v] = ("
            << T << ")(" << value_text(st, ld) << "); }\n";
-        os << "  *reinterpret_cast<EhV4<" << T << ">*>(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ") = o; }\n";
+        os << "  eh_store4<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ", o); }\n";
       } else {
         os << "  { const idx_t c = c0; " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << T << ")("
            << value_text(st, ld) << "); }\n";
@@ -954,6 +976,9 @@ struct GroupEmitter {
     int64_t T = opt.row_threads > 0 ? opt.row_threads : pow2_ceil((C + opt.row_elems - 1) / opt.row_elems);
     T = std::max<int64_t>(1, std::min<int64_t>(T, 1024));
     if (!pow2(T)) T = pow2_ceil(T);
+    // two waves per row would pay for an LDS exchange and a barrier; one wave with twice the
+    // elements per lane is faster for rows this short
+    if (opt.row_threads == 0 && T == 128) T = 64;
     while (T * V > pow2_ceil(C) && T > 1) T >>= 1;          // no more threads than vectors in a row
     const int64_t per_iter = T * V;
     const int64_t NV = (C + per_iter - 1) / per_iter;
@@ -965,9 +990,12 @@ struct GroupEmitter {
     if (blocks >= (int64_t{1} << 31)) throw Error("too many rows for one launch");
     int nred = 0;
     for (const auto& st : g.stages) nred += st.kind == StageKind::Reduce;
+    const char* nt = nt_loads() ? "true" : "false";
+    const char* nts = nt_stores() ? "true" : "false";
     ls.entry = "ehk_" + g.stages.front().kname;
     ls.schedule = "row(T=" + std::to_string(T) + ",V=" + std::to_string(V) + ",NV=" + std::to_string(NV) +
-                  (reg ? ",reg" : ",stream") + ",rows/block=" + std::to_string(RPB) + ")";
+                  (reg ? ",reg" : ",stream") + ",rows/block=" + std::to_string(RPB) + (nt_stores() ? ",nt-store" : "") +
+                  (nt_loads() ? ",nt-load" : "") + ")";
     ls.grid[0] = static_cast<unsigned>(blocks);
     ls.block[0] = static_cast<unsigned>(block);
     for (auto& e : ext) e.cached = reg;
@@ -999,9 +1027,9 @@ struct GroupEmitter {
         os << iter_open << guard_open;
         for (const auto& e : ext) {
           if (V == 4) {
-            os << "      const EhV4<" << ctype(e.dtype) << "> t" << e.id << " = *reinterpret_cast<const EhV4<"
-               << ctype(e.dtype) << ">*>(" << e.buf << " + " << affine_text(e.aff, "c0") << ");\n";
-            os << "#pragma unroll\n      for (int v = 0; v < 4; ++v) xc" << e.id << "[k * 4 + v] = t" << e.id << ".v[v];\n";
+            os << "      const EhV4<" << ctype(e.dtype) << "> t" << e.id << " = eh_load4<" << nt << ">(" << e.buf << " + "
+               << affine_text(e.aff, "c0") << ");\n";
+            os << "#pragma unroll\n      for (int v = 0; v < 4; ++v) xc" << e.id << "[k * 4 + v] = t" << e.id << "[v];\n";
           } else {
             os << "      xc" << e.id << "[k] = " << e.buf << "[" << affine_text(e.aff, "c0") << "];\n";
           }
@@ -1041,10 +1069,10 @@ struct GroupEmitter {
       } else if (st.store) {
         os << iter_open << guard_open;
         if (V == 4) {
-          os << "      EhV4<" << T_out << "> o;\n#pragma unroll\n      for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o.v[v] = ("
+          os << "      EhV4<" << T_out << "> o;\n#pragma unroll\n      for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o[v] = ("
              << T_out << ")(" << value_text(st, ld) << "); }\n";
-          os << "      if (eh_row_ok) *reinterpret_cast<EhV4<" << T_out << ">*>(" << st.out_buf << " + "
-             << affine_text(st.out_aff, "c0") << ") = o;\n";
+          os << "      if (eh_row_ok) eh_store4<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0")
+             << ", o);\n";
         } else {
           os << "      const int v = 0; const idx_t c = c0; const " << T_out << " o = (" << T_out << ")(" << value_text(st, ld)
              << ");\n      if (eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = o;\n";

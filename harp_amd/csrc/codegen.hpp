@@ -20,12 +20,12 @@ struct GenOptions {
   bool fuse = true;          // merge compatible kernels of a Program into one launch
   bool vectorize = true;     // 128-bit accesses where alignment allows
   int row_threads = 0;       // threads cooperating on one row; 0 = choose from the row length
-  int row_elems = 16;        // target elements per thread per row when choosing row_threads
+  int row_elems = 8;         // target elements per thread per row when choosing row_threads
   int flat_block = 256;
   int flat_iters = 4;        // vectors handled by one thread of a flat kernel
   int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
-  bool nontemporal = false;  // streaming stores for outputs
+  int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores
 };
 
 struct LaunchSpec {

@@ -17,7 +17,7 @@ struct Tile {
 };
 
 // Largest first.  Each uses 256 threads (four waves).
-const Tile kTiles[] = {{128, 128, 32, 64, 64}, {64, 64, 32, 32, 32}};
+const Tile kTiles[] = {{128, 128, 16, 64, 64}, {64, 64, 16, 32, 32}};
 
 bool pick_tile(const GemmShape& s, const GenOptions& opt, Tile* out) {
   auto fits = [&](const Tile& t) {
