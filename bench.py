@@ -33,6 +33,16 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch from the committed counter summary (rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE, scaled by a copy kernel of known size); None when the kernel is not in it."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)["kernels"][kernel]["traffic_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def build(dev, hb, wl, name, shapes, options):
     inputs_fn, graph_fn = wl.CONFIGS[name]
     prog_ast, arg_names, out_name, const_inputs, _ = wl.lower_with_table(shapes, graph_fn)
@@ -214,7 +224,9 @@ def main():
     }
     if head:
         out["roofline"] = {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                           "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
+                           "traffic": measured_traffic(head["launches"][0][0]) if not args.options else None,
+                           "algorithmic_bytes": head["algo_bytes"],
                            "kernel": head["launches"][0][0], "schedule": head["launches"][0][1]}
     if cpu:
         out["cpu_baseline"] = cpu
@@ -224,7 +236,8 @@ def main():
             "steps": matmul["steps"], "dtype": "f32",
             "roofline": {"bound": "mfma", "achieved": round(matmul["tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(matmul["tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
-                         "traffic": None, "kernel": matmul["launches"][0][0],
+                         "traffic": measured_traffic(matmul["launches"][0][0]) if not args.options else None,
+                         "kernel": matmul["launches"][0][0],
                          "schedule": matmul["launches"][0][1]}}
     if cfg1:
         result_extra["config1_relu_sum_1024"] = {"us_per_step": round(cfg1["us"], 2),
