@@ -1,0 +1,197 @@
+//! Eclat backend for AMD MI355X (gfx950) -- binds `libeclat_hip` to the backend traits.
+//!
+//! SOURCE ONLY: the pipeline that produced this crate has no Rust toolchain; it has never been
+//! compiled or run.  It shows which trait method each C entry point serves.
+//!
+//! The AST is serialised to the s-expression text `eh_program_compile` reads (one form per
+//! `AstNode` variant, see `ser.rs`); rendering, hiprtc compilation, caching of code objects
+//! and launching all happen behind the C ABI.
+
+mod ffi;
+mod ser;
+
+use std::any::Any;
+use std::ffi::CString;
+use std::sync::Arc;
+
+use eclat::ast::{AstNode, DType};
+use eclat::backend::device::{BackendRegistry, DeviceError};
+use eclat::backend::global::DeviceKind;
+use eclat::backend::traits::{Buffer, Kernel, KernelConfig};
+use eclat::backend::KernelSignature;
+
+type DynErr = Box<dyn std::error::Error + Send + Sync>;
+
+fn check(code: i32) -> Result<(), DynErr> {
+    if code == 0 { Ok(()) } else { Err(ffi::last_error().into()) }
+}
+
+pub struct HipDevice { raw: *mut ffi::eh_device }
+unsafe impl Send for HipDevice {}
+unsafe impl Sync for HipDevice {}
+impl Drop for HipDevice { fn drop(&mut self) { unsafe { ffi::eh_device_close(self.raw); } } }
+
+pub struct HipBuffer { raw: *mut ffi::eh_buffer, dev: Arc<HipDevice>, shape: Vec<usize>, dtype: DType, bytes: usize }
+unsafe impl Send for HipBuffer {}
+unsafe impl Sync for HipBuffer {}
+impl Drop for HipBuffer { fn drop(&mut self) { unsafe { ffi::eh_buffer_release(self.raw); } } }
+
+impl HipBuffer {
+    fn allocate(dev: &Arc<HipDevice>, shape: Vec<usize>, dtype: DType) -> Result<Self, DynErr> {
+        let bytes = shape.iter().product::<usize>() * dtype.size_in_bytes();
+        let mut raw = std::ptr::null_mut();
+        check(unsafe { ffi::eh_buffer_alloc(dev.raw, bytes, &mut raw) })?;   // zero-filled
+        Ok(Self { raw, dev: dev.clone(), shape, dtype, bytes })
+    }
+}
+
+impl Buffer for HipBuffer {
+    fn shape(&self) -> &[usize] { &self.shape }
+    fn dtype(&self) -> DType { self.dtype.clone() }
+    fn byte_len(&self) -> usize { self.bytes }
+    fn read_to_host(&self) -> Result<Vec<u8>, DynErr> {
+        let mut v = vec![0u8; self.bytes];
+        check(unsafe { ffi::eh_buffer_read(self.raw, v.as_mut_ptr().cast(), self.bytes) })?;
+        Ok(v)
+    }
+    fn write_from_host(&mut self, data: &[u8]) -> Result<(), DynErr> {
+        // the library rejects a length different from byte_len(), as CBuffer does
+        check(unsafe { ffi::eh_buffer_write(self.raw, data.as_ptr().cast(), data.len()) })
+    }
+    fn clone_buffer(&self) -> Box<dyn Buffer> {
+        let b = HipBuffer::allocate(&self.dev, self.shape.clone(), self.dtype.clone()).expect("allocation failed");
+        unsafe { ffi::eh_buffer_copy(b.raw, self.raw); }
+        Box::new(b)
+    }
+    fn as_any(&self) -> &dyn Any { self }
+    fn as_any_mut(&mut self) -> &mut dyn Any { self }
+}
+
+enum Loaded { Program(*mut ffi::eh_program), Module(*mut ffi::eh_module) }
+
+pub struct HipKernel { loaded: Loaded, config: KernelConfig, ast_text: Option<Arc<String>>, dev: Arc<HipDevice> }
+unsafe impl Send for HipKernel {}
+unsafe impl Sync for HipKernel {}
+impl Drop for HipKernel {
+    fn drop(&mut self) {
+        unsafe {
+            match self.loaded {
+                Loaded::Program(p) => { ffi::eh_program_release(p); }
+                Loaded::Module(m) => { ffi::eh_module_release(m); }
+            }
+        }
+    }
+}
+
+fn raw_buffers(bufs: &[&dyn Buffer]) -> Vec<*mut ffi::eh_buffer> {
+    bufs.iter().map(|b| b.as_any().downcast_ref::<HipBuffer>().expect("buffer is not a HipBuffer").raw).collect()
+}
+
+impl Kernel for HipKernel {
+    fn clone_kernel(&self) -> Box<dyn Kernel> {
+        // recompile from the AST text; the library's code-object cache makes this a lookup
+        let text = self.ast_text.as_ref().expect("kernels loaded from a binary cannot be cloned");
+        Box::new(compile_text(&self.dev, text.clone(), self.config.clone()).expect("recompile failed"))
+    }
+    fn config(&self) -> &KernelConfig { &self.config }
+    fn device_kind(&self) -> DeviceKind { DeviceKind::Hip }
+    fn execute(&self, inputs: &[&dyn Buffer], outputs: &mut [&mut dyn Buffer]) -> Result<(), DynErr> {
+        let ins = raw_buffers(inputs);
+        let outs: Vec<_> = outputs.iter().map(|b| b.as_any().downcast_ref::<HipBuffer>()
+            .expect("buffer is not a HipBuffer").raw).collect();
+        match self.loaded {
+            Loaded::Program(p) => check(unsafe {
+                ffi::eh_program_execute_positional(p, ins.as_ptr(), ins.len() as i32, outs.as_ptr(), outs.len() as i32, 1)
+            }),
+            Loaded::Module(_) => {
+                let g = self.config.global_work_size;
+                let l = self.config.local_work_size.unwrap_or([1, 1, 1]);
+                self.execute_with_sizes(inputs, outputs, g, l)
+            }
+        }
+    }
+    fn execute_with_sizes(&self, inputs: &[&dyn Buffer], outputs: &mut [&mut dyn Buffer],
+                          grid_size: [usize; 3], local_size: [usize; 3]) -> Result<(), DynErr> {
+        // `grid_size` is the global size here; the library wants workgroup counts
+        let Loaded::Module(m) = self.loaded else { return self.execute(inputs, outputs); };
+        let mut args = raw_buffers(inputs);
+        args.extend(outputs.iter().map(|b| b.as_any().downcast_ref::<HipBuffer>().expect("not a HipBuffer").raw));
+        let block = local_size.map(|v| v.max(1) as u32);
+        let grid = [0, 1, 2].map(|i| (grid_size[i].max(1) as u32).div_ceil(block[i]));
+        check(unsafe { ffi::eh_module_launch(m, grid.as_ptr(), block.as_ptr(), 0, args.as_ptr(), args.len() as i32, 1) })
+    }
+    fn as_any(&self) -> &dyn Any { self }
+    fn supports_binary_cache(&self) -> bool { matches!(self.loaded, Loaded::Program(_)) }
+    fn get_binary(&self) -> Option<Vec<u8>> {
+        let Loaded::Program(p) = self.loaded else { return None; };
+        let (mut blob, mut len) = (std::ptr::null(), 0usize);
+        if unsafe { ffi::eh_program_binary(p, 0, &mut blob, &mut len) } != 0 { return None; }
+        Some(unsafe { std::slice::from_raw_parts(blob.cast::<u8>(), len) }.to_vec())
+    }
+}
+
+fn compile_text(dev: &Arc<HipDevice>, text: Arc<String>, config: KernelConfig) -> Result<HipKernel, DynErr> {
+    let c = CString::new(text.as_str())?;
+    let mut raw = std::ptr::null_mut();
+    check(unsafe { ffi::eh_program_compile(dev.raw, c.as_ptr(), std::ptr::null(), &mut raw) })?;
+    Ok(HipKernel { loaded: Loaded::Program(raw), config, ast_text: Some(text), dev: dev.clone() })
+}
+
+struct HipBackendRegistry;
+
+fn device_of(device: &dyn Any) -> Result<&Arc<HipDevice>, DeviceError> {
+    device.downcast_ref::<Arc<HipDevice>>()
+        .ok_or_else(|| DeviceError::InitializationError("Invalid device type: expected HipDevice".into()))
+}
+
+impl BackendRegistry for HipBackendRegistry {
+    fn kind(&self) -> DeviceKind { DeviceKind::Hip }
+    fn name(&self) -> &str { "HIP (gfx950)" }
+    fn is_available(&self) -> bool {
+        let mut n = 0;
+        unsafe { ffi::eh_device_count(&mut n) == 0 && n > 0 }
+    }
+    fn create_device(&self, index: usize) -> Result<Arc<dyn Any + Send + Sync>, DeviceError> {
+        let mut raw = std::ptr::null_mut();
+        if unsafe { ffi::eh_device_open(index as i32, &mut raw) } != 0 {
+            return Err(DeviceError::InitializationError(ffi::last_error()));
+        }
+        Ok(Arc::new(Arc::new(HipDevice { raw })))
+    }
+    fn list_devices(&self) -> Vec<String> {
+        let mut n = 0;
+        unsafe { ffi::eh_device_count(&mut n); }
+        (0..n).map(|i| format!("hip:{i}")).collect()
+    }
+    fn supports_runtime(&self) -> bool { true }
+    fn allocate_buffer(&self, device: &dyn Any, shape: Vec<usize>, dtype: DType) -> Result<Box<dyn Buffer>, DeviceError> {
+        let dev = device_of(device)?;
+        HipBuffer::allocate(dev, shape, dtype).map(|b| Box::new(b) as Box<dyn Buffer>)
+            .map_err(|e| DeviceError::InitializationError(format!("Failed to allocate HIP buffer: {e}")))
+    }
+    fn compile_ast(&self, device: &dyn Any, program: AstNode, _signature: KernelSignature)
+                   -> Result<Box<dyn Kernel>, DeviceError> {
+        let dev = device_of(device)?;
+        let entry = ser::first_kernel_name(&program).unwrap_or_else(|| "kernel".to_string());
+        let text = Arc::new(ser::to_text(&program));
+        compile_text(dev, text, KernelConfig::new(entry)).map(|k| Box::new(k) as Box<dyn Kernel>)
+            .map_err(|e| DeviceError::InitializationError(format!("Failed to compile AST: {e}")))
+    }
+    fn supports_binary_cache(&self) -> bool { true }
+    fn compile_from_binary(&self, device: &dyn Any, binary: &[u8], config: KernelConfig)
+                           -> Result<Box<dyn Kernel>, DeviceError> {
+        let dev = device_of(device)?;
+        let entry = CString::new(config.entry_point.as_str()).map_err(|e| DeviceError::InitializationError(e.to_string()))?;
+        let mut raw = std::ptr::null_mut();
+        if unsafe { ffi::eh_module_load(dev.raw, binary.as_ptr().cast(), binary.len(), entry.as_ptr(), &mut raw) } != 0 {
+            return Err(DeviceError::InitializationError(ffi::last_error()));
+        }
+        Ok(Box::new(HipKernel { loaded: Loaded::Module(raw), config, ast_text: None, dev: dev.clone() }))
+    }
+}
+
+/// Registers the backend (called at program start when the crate is linked).
+pub fn init() { eclat::backend::register_backend(Box::new(HipBackendRegistry)); }
+
+#[ctor::ctor]
+fn auto_init() { init(); }

@@ -86,6 +86,9 @@ _SIGS = {
     "eh_program_execute": ([_P, POINTER(_P), c_int, c_int], c_int),
     "eh_program_execute_positional": ([_P, POINTER(_P), c_int, POINTER(_P), c_int, c_int], c_int),
     "eh_program_binary": ([_P, c_int, POINTER(_P), POINTER(c_size_t)], c_int),
+    "eh_module_load": ([_P, _P, c_size_t, c_char_p, POINTER(_P)], c_int),
+    "eh_module_launch": ([_P, POINTER(c_uint), POINTER(c_uint), c_uint, POINTER(_P), c_int, c_int], c_int),
+    "eh_module_release": ([_P], c_int),
     "eh_event_create": ([_P, POINTER(_P)], c_int),
     "eh_event_record": ([_P], c_int),
     "eh_event_sync": ([_P], c_int),

@@ -246,6 +246,27 @@ class HipKernel:
         return self._prog.launches
 
 
+class HipModule:
+    """One entry point of a code object (`compile_from_binary` + `execute_with_sizes`)."""
+
+    def __init__(self, device: HipDevice, blob: bytes, entry: str):
+        self.device = device
+        self._h = c_void_p()
+        buf = (ctypes.c_char * len(blob)).from_buffer_copy(blob)
+        check(lib.eh_module_load(device._h, buf, len(blob), entry.encode(), byref(self._h)))
+
+    def launch(self, grid, block, args: Sequence[HipBuffer], lds_bytes: int = 0, sync: bool = True):
+        g = (ctypes.c_uint * 3)(*grid)
+        b = (ctypes.c_uint * 3)(*block)
+        a = (c_void_p * max(len(args), 1))(*[x._h for x in args])
+        check(lib.eh_module_launch(self._h, g, b, lds_bytes, a, len(args), 1 if sync else 0))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib.eh_module_release(h)
+
+
 class Event:
     def __init__(self, device: HipDevice):
         self._h = c_void_p()

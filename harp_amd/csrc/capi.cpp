@@ -26,6 +26,10 @@ struct eh_program {
 struct eh_plan {
   ProgramPlan plan;
 };
+struct eh_module {
+  HipDevice* dev;
+  std::shared_ptr<HipKernel> kernel;
+};
 struct eh_event {
   HipDevice* dev;
   hipEvent_t ev;
@@ -334,6 +338,42 @@ int eh_program_binary(eh_program* prog, int launch, const void** blob, size_t* l
   *blob = b.data();
   *len = b.size();
   return EH_OK;
+}
+
+int eh_module_load(eh_device* dev, const void* blob, size_t len, const char* entry, eh_module** out) {
+  REQUIRE(dev && blob && len > 0 && entry && out, "device, blob, entry or out is NULL");
+  return guard([&] {
+    Binary b;
+    b.code.assign(static_cast<const char*>(blob), static_cast<const char*>(blob) + len);
+    if (len < 4 || std::memcmp(b.code.data(), "\x7f" "ELF", 4) != 0)
+      throw Error("code object does not start with an ELF header");
+    *out = new eh_module{&dev->dev, dev->dev.load(b, entry)};
+  });
+}
+
+int eh_module_launch(eh_module* mod, const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
+                     eh_buffer* const* args, int n_args, int sync) {
+  REQUIRE(mod && grid && block && n_args >= 0 && (args || n_args == 0), "bad arguments");
+  return guard([&] {
+    unsigned long long threads = 1ull * block[0] * block[1] * block[2];
+    if (threads == 0 || threads > 1024 || grid[0] == 0 || grid[1] == 0 || grid[2] == 0)
+      throw Error("dispatch size out of range (block of " + std::to_string(threads) + " work-items)");
+    if (lds_bytes > 160 * 1024) throw Error("dynamic LDS request exceeds 160 KiB");
+    std::vector<void*> ptrs;
+    for (int i = 0; i < n_args; ++i) {
+      if (!args[i]) throw Error("argument " + std::to_string(i) + " is NULL");
+      if (args[i]->buf.device() != mod->dev) throw Error("argument " + std::to_string(i) + " lives on another device");
+      ptrs.push_back(args[i]->buf.device_ptr());
+    }
+    mod->dev->make_current();
+    mod->kernel->launch(grid, block, lds_bytes, ptrs);
+    if (sync) mod->dev->synchronize();
+  });
+}
+
+int eh_module_release(eh_module* mod) {
+  REQUIRE(mod, "module is NULL");
+  return guard([&] { delete mod; });
 }
 
 int eh_event_create(eh_device* dev, eh_event** out) {

@@ -35,6 +35,7 @@ typedef struct eh_buffer eh_buffer;
 typedef struct eh_program eh_program;   /* one or more launches compiled from a Program AST */
 typedef struct eh_plan eh_plan;         /* rendered sources + dispatch, no device involved */
 typedef struct eh_event eh_event;
+typedef struct eh_module eh_module;     /* one entry point of a loaded code object */
 
 /* ---- library ---------------------------------------------------------------------------- */
 int eh_version(void);                   /* 100 * major + minor */
@@ -130,6 +131,16 @@ int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, in
 /* Kernel::get_binary / BackendRegistry::compile_from_binary (src/backend/traits.rs:576-586,
  * src/backend/device.rs:161-170): the gfx950 code object of one launch. */
 int eh_program_binary(eh_program* prog, int launch, const void** blob, size_t* len);
+
+/* ---- Thin module layer: load a gfx950 code object (from eh_compile_source, eh_program_binary or
+ *      the disk cache) and launch one entry point with buffer arguments.  This is
+ *      BackendRegistry::compile_from_binary + Kernel::execute_with_sizes
+ *      (src/backend/device.rs:161-170, src/backend/traits.rs:556-566); `grid` counts
+ *      workgroups, `block` work-items per workgroup. -------------------------------------------- */
+int eh_module_load(eh_device* dev, const void* blob, size_t len, const char* entry, eh_module** out);
+int eh_module_launch(eh_module* mod, const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
+                     eh_buffer* const* args, int n_args, int sync);
+int eh_module_release(eh_module* mod);
 
 /* ---- timing on the device's stream (HIP events) ------------------------------------------------ */
 int eh_event_create(eh_device* dev, eh_event** out);

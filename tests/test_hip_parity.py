@@ -227,3 +227,15 @@ def test_kernel_binary_round_trip(frontend, hip):
     k = hip.HipKernel(dev, prog)
     blob = k.get_binary()
     assert blob[:4] == b"\x7fELF" and len(blob) > 1000
+    # compile_from_binary: load the code object again and launch it with explicit sizes
+    l = k.launches[0]
+    mod = hip.HipModule(dev, blob, l["entry"])
+    x = np.arange(256, dtype=np.float32)
+    src, dst = hip.HipBuffer(dev, [256], frontend.F32), hip.HipBuffer(dev, [256], frontend.F32)
+    src.write_array(x)
+    mod.launch(l["grid"], l["block"], [src, dst])
+    assert np.array_equal(dst.read_array(np.float32), x * x)
+    with pytest.raises(hip.EhError):
+        hip.HipModule(dev, b"not a code object", "k")
+    with pytest.raises(hip.EhError):
+        hip.HipModule(dev, blob, "no_such_entry")
