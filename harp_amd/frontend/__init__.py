@@ -14,3 +14,4 @@ from .lowerer import Lowerer, all_fusions, lower_graph
 from .tensor import Tensor
 from .view import View
 from . import nn
+from .config import exact_mode

@@ -51,10 +51,18 @@ def buffer_table(program: AstNode, lowerer, input_names: Sequence[str],
     return table
 
 
-def _root_buffer_name(root: GraphNode, lowerer, available: Sequence[str]):
+def _root_buffer_name(root: GraphNode, lowerer, available: Sequence[str], opt_root=None):
     name = lowerer.lookup_buffer_name(root)
     if name is not None and name in available:
         return name
+    # the optimised graph's root (graph passes rebuild nodes), or -- when that root is a view
+    # that was inlined -- the node whose buffer it views
+    n = opt_root
+    while n is not None:
+        name = lowerer.lookup_buffer_name(n)
+        if name is not None and name in available:
+            return name
+        n = n.src[0] if (n.op.kind == "view" and n.src) else None
     best = None
     for k in available:
         if k.startswith("buf") and k[3:].isdigit():
@@ -72,7 +80,7 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
         raise ExecutionError("NoDevice")
     if not roots:
         return []
-    program, lowerer, _ = lower_graph(roots)
+    program, lowerer, opt_roots = lower_graph(roots)
     kernels = [k for k in program.args if k.op == "kernel"]
 
     input_nodes = collect_inputs(roots)
@@ -89,8 +97,8 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
                     if p.dtype.is_ptr() and p.mutable]
         all_names = list(buffer_map.keys()) + produced
         out_names = []
-        for r in roots:
-            nm = _root_buffer_name(r, lowerer, all_names)
+        for r, o in zip(roots, opt_roots):
+            nm = _root_buffer_name(r, lowerer, all_names, o)
             if nm is not None and nm not in out_names:
                 out_names.append(nm)
         table = buffer_table(program, lowerer, list(buffer_map.keys()), out_names)
@@ -125,7 +133,7 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
                 buffer_map[p.name] = b
 
     results = []
-    for r in roots:
-        nm = _root_buffer_name(r, lowerer, list(buffer_map.keys()))
-        results.append(buffer_map.pop(nm) if nm is not None else None)
+    for r, o in zip(roots, opt_roots):
+        nm = _root_buffer_name(r, lowerer, list(buffer_map.keys()), o)
+        results.append(buffer_map.get(nm) if nm is not None else None)
     return results

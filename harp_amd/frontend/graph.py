@@ -78,16 +78,19 @@ class GraphOp:
 
 
 class GraphNode:
-    __slots__ = ("src", "view", "op", "dtype", "name", "buffer_id", "__weakref__")
+    __slots__ = ("src", "view", "op", "dtype", "name", "buffer_id", "hint", "__weakref__")
 
     def __init__(self, src: Sequence["GraphNode"], view: View, op: GraphOp, dtype: DType,
-                 buffer_id: Optional[int] = None, name: Optional[str] = None):
+                 buffer_id: Optional[int] = None, name: Optional[str] = None, hint=None):
         self.src = list(src)
         self.view = view
         self.op = op
         self.dtype = dtype
         self.name = name
         self.buffer_id = buffer_id
+        # which view transformation built this node, e.g. ("permute", [1, 0]); the reference
+        # keeps no such record -- only the exact-gradient mode reads it
+        self.hint = hint
 
     # -- accessors ---------------------------------------------------------
     def shape(self) -> List[Expr]:
@@ -103,31 +106,35 @@ class GraphNode:
         return self.buffer_id is not None
 
     def with_name(self, name: str) -> "GraphNode":
-        return GraphNode(self.src, self.view, self.op, self.dtype, self.buffer_id, name)
+        return GraphNode(self.src, self.view, self.op, self.dtype, self.buffer_id, name, self.hint)
 
     def with_new_sources(self, src) -> "GraphNode":
-        return GraphNode(src, self.view, self.op, self.dtype, self.buffer_id, self.name)
+        return GraphNode(src, self.view, self.op, self.dtype, self.buffer_id, self.name, self.hint)
 
     def __repr__(self):
         return f"GraphNode(name={self.name}, dtype={self.dtype}, shape={self.shape()}, op={self.op.kind})"
 
     # -- view transformations (node.rs:325-480): op holds the SOURCE view ----
-    def _view_node(self, new_view: View) -> "GraphNode":
-        return GraphNode([self], new_view, GraphOp("view", view=self.view), self.dtype)
+    def _view_node(self, new_view: View, hint=None) -> "GraphNode":
+        return GraphNode([self], new_view, GraphOp("view", view=self.view), self.dtype, hint=hint)
 
-    def permute(self, axes): return self._view_node(self.view.permute(list(axes)))
-    def unsqueeze(self, axis): return self._view_node(self.view.unsqueeze(axis))
-    def squeeze(self, axis): return self._view_node(self.view.squeeze(axis))
-    def expand(self, axis, size): return self._view_node(self.view.expand(axis, size))
-    def reshape(self, shape): return self._view_node(self.view.reshape(shape))
-    def flip(self, axis): return self._view_node(self.view.flip(axis))
-    def repeat(self, axis, times): return self._view_node(self.view.repeat(axis, times))
+    def permute(self, axes):
+        return self._view_node(self.view.permute(list(axes)), ("permute", list(axes)))
+
+    def unsqueeze(self, axis): return self._view_node(self.view.unsqueeze(axis), ("unsqueeze", axis))
+    def squeeze(self, axis): return self._view_node(self.view.squeeze(axis), ("squeeze", axis))
+    def expand(self, axis, size): return self._view_node(self.view.expand(axis, size), ("expand", axis))
+    def reshape(self, shape): return self._view_node(self.view.reshape(shape), ("reshape",))
+    def flip(self, axis): return self._view_node(self.view.flip(axis), ("flip", axis))
+    def repeat(self, axis, times): return self._view_node(self.view.repeat(axis, times), ("expand", axis))
 
     def slice_axis(self, axis, start, length):
-        return self._view_node(self.view.slice_axis(axis, start, length))
+        return self._view_node(self.view.slice_axis(axis, start, length),
+                               ("slice", axis, Expr.of(start)))
 
     def pad(self, padding, value: str = "zero"):
-        return self._view_node(View.padded(self.view, list(padding), value))
+        padding = [(Expr.of(b), Expr.of(a)) for b, a in padding]
+        return self._view_node(View.padded(self.view, padding, value), ("pad", padding))
 
     def contiguous(self) -> "GraphNode":
         return GraphNode([self], View.contiguous(self.shape()),

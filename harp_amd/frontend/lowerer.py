@@ -401,10 +401,39 @@ class Lowerer:
         return self.make_kernel(name, m_loop, inputs, output)
 
 
-def lower_graph(roots: Sequence[GraphNode], optimize: bool = True):
+def unshare_views(roots: Sequence[GraphNode]) -> List[GraphNode]:
+    """Gives every consumer its own copy of each View node it reads, so that all views have
+    one consumer and are inlined.  Not in the reference: there a view with several consumers
+    is materialised contiguously by a copy kernel but still indexed through its own
+    (possibly strided) view by the readers (`lower.rs:209-224` vs `:452-455`), which is only
+    right for contiguous views.  Used by the exact mode."""
+    memo: Dict[int, GraphNode] = {}
+    order = topological_sort(roots)
+
+    def fresh(n: GraphNode) -> GraphNode:
+        # a private copy of a view chain, down to the first node that computes something
+        if n.op.kind == "view" and not n.is_external() and n.src:
+            return GraphNode([fresh(n.src[0])], n.view, n.op, n.dtype, None, n.name, n.hint)
+        return memo[id(n)]
+
+    for n in order:
+        if n.op.kind == "view" and not n.is_external() and n.src:
+            continue                      # rebuilt on demand by fresh()
+        new_src = [fresh(s) for s in n.src]
+        changed = any(a is not b for a, b in zip(new_src, n.src))
+        memo[id(n)] = n.with_new_sources(new_src) if changed else n
+    return [fresh(r) for r in roots]
+
+
+def lower_graph(roots: Sequence[GraphNode], optimize: bool = True, exact_views: bool = None):
     """`CompilationPipeline::lower_with_lowerer` (compile.rs:227-244) with the
     level-0 graph optimisation (`AllFusions`, compile.rs:366-371).  Returns
     (program AST, lowerer, optimised roots)."""
+    from . import config
+    if exact_views is None:
+        exact_views = config.EXACT
+    if exact_views:
+        roots = unshare_views(roots)
     opt_roots = all_fusions(roots) if optimize else list(roots)
     lw = Lowerer()
     program = lw.lower(opt_roots)

@@ -132,6 +132,12 @@ class Tensor:
     def scale(self, _factor: float) -> "Tensor":
         return self.mul(Tensor.ones_like(self))
 
+    def scale_exact(self, factor: float) -> "Tensor":
+        """x * factor as a literal in the map (not in the reference, whose `scale`
+        ignores the factor)."""
+        from .ast import AstNode
+        return Tensor(self.graph.unary_op(lambda x: AstNode.mul(x, AstNode.const_f32(factor))))
+
     # -- reductions (the reduced axis is squeezed away) ------------------------------
     def _check_axis(self, axis):
         if not 0 <= axis < self.ndim():
@@ -189,6 +195,48 @@ class Tensor:
 
     def fold(self, output_shape, axes, sizes, strides, dilations):
         return Tensor(self.graph.fold(output_shape, axes, sizes, strides, dilations))
+
+    # -- autograd (src/tensor/autograd.rs:83-340) ------------------------------------------------
+    def requires_grad_(self, flag: bool = True) -> "Tensor":
+        self._requires_grad = bool(flag)
+        return self
+
+    def requires_grad(self) -> bool:
+        return self._requires_grad
+
+    def grad(self) -> Optional["Tensor"]:
+        return self._grad
+
+    def set_grad(self, grad: "Tensor") -> None:
+        self._grad = grad
+
+    def zero_grad(self) -> None:
+        self._grad = None
+
+    def detach(self) -> "Tensor":
+        t = Tensor(self.graph)
+        t.buffer = self.buffer
+        return t
+
+    def backward(self):
+        raise ExecutionError("NoParams: backward() requires explicit parameters. Use "
+                             "backward_with_params([tensor1, tensor2, ...]) instead.")
+
+    def backward_with_params(self, params: Sequence["Tensor"], exact: bool = None) -> None:
+        """Builds the gradient graphs and stores them on the parameters; nothing
+        runs until a gradient is realized.  `exact=True` uses mathematically correct
+        VJPs instead of the reference's rules as written."""
+        from .grad import backward as compute_backward
+        from . import config
+        if exact is None:
+            exact = config.EXACT
+        if not params:
+            raise ExecutionError("NoParams: No parameters provided for backward pass.")
+        res = compute_backward(self.graph, [p.graph for p in params], exact=exact)
+        for p in params:
+            g = res.get(p.graph)
+            if g is not None:
+                p.set_grad(Tensor(g))
 
     # -- realisation -------------------------------------------------------------------------
     def is_realized(self) -> bool:

@@ -129,3 +129,138 @@ def test_index_forms_brute_force(frontend, fn, ref):
     x = np.random.default_rng(11).normal(0, 1, (4, 6)).astype(np.float32)
     out = realize_on(frontend, "c", fn, [x])
     assert np.allclose(out, np.asarray(ref(x)).ravel(), rtol=1e-6, atol=1e-6)
+
+
+def _grads_on(fe, kind, build_loss, arrays):
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    fe.set_device_str(kind)
+    try:
+        ts = []
+        for a in arrays:
+            t = fe.Tensor.input(list(a.shape))
+            t.requires_grad_(True)
+            t.set_data(a)
+            ts.append(t)
+        loss = build_loss(*ts)
+        loss.backward_with_params(ts)
+        out = []
+        for t in ts:
+            g = t.grad()
+            assert g is not None
+            g.realize()
+            out.append(g.to_numpy())
+        return out
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+
+
+def test_autograd_known_answers(frontend):
+    # crates/backend-metal/src/lib.rs:262-368
+    x = np.array([1, 2, 3, 4], dtype=np.float32)
+    (gx,) = _grads_on(frontend, "c", lambda t: (t * t).sum(0), [x])
+    assert gx.tolist() == [2, 4, 6, 8]
+    a = np.array([1, 2, 3, 4], dtype=np.float32)
+    b = np.array([5, 6, 7, 8], dtype=np.float32)
+    ga, gb = _grads_on(frontend, "c", lambda s, t: (s * t).sum(0), [a, b])
+    assert ga.tolist() == [5, 6, 7, 8] and gb.tolist() == [1, 2, 3, 4]
+    (g2,) = _grads_on(frontend, "c", lambda t: (t + t).sum(0), [x])
+    assert g2.tolist() == [2, 2, 2, 2]
+
+
+def test_autograd_rules_as_written(frontend):
+    """The VJP dispatcher classifies a map by its top node (src/grad/rules.rs:736-778):
+    a - b passes +g to b, a / b uses the product rule, exp(x) differentiates as exp2(x)."""
+    a = np.array([1.0, 2.0, 3.0], dtype=np.float32)
+    b = np.array([4.0, 5.0, 8.0], dtype=np.float32)
+    def sq_diff(s, t):
+        u = s - t
+        return (u * u).sum(0)
+    ga, gb = _grads_on(frontend, "c", sq_diff, [a, b])
+    assert np.allclose(ga, 2 * (a - b)) and np.allclose(gb, 2 * (a - b))      # same sign for both
+    # a gradient that is only a view of the seed (no kernel to run) cannot be realized,
+    # as in the reference (src/tensor/realize.rs:239-242)
+    with pytest.raises(frontend.ExecutionError):
+        _grads_on(frontend, "c", lambda s, t: (s - t).sum(0), [a, b])
+    ga, gb = _grads_on(frontend, "c", lambda s, t: (s / t).sum(0), [a, b])
+    assert np.allclose(ga, b) and np.allclose(gb, a)
+    (gx,) = _grads_on(frontend, "c", lambda t: t.exp().sum(0), [a])
+    assert np.allclose(gx, np.exp2(a), rtol=1e-6)
+    # relu: gradient flows where x >= 0
+    x = np.array([-1.0, 0.5, 2.0, -3.0], dtype=np.float32)
+    w = np.array([3.0, 5.0, 7.0, 9.0], dtype=np.float32)
+    gr, _ = _grads_on(frontend, "c", lambda t, u: (frontend.nn.relu(t) * u).sum(0), [x, w])
+    assert gr.tolist() == [0, 5, 7, 0]
+    # where_cond writes through the view of its `self` operand (src/graph/ops.rs:452-462): when
+    # the upstream gradient is a broadcast (stride-0) view every element lands on index 0
+    (gr0,) = _grads_on(frontend, "c", lambda t: frontend.nn.relu(t).sum(0), [x])
+    assert gr0.tolist() == [0, 0, 0, 0]
+    # linear layer: the broadcast in expand-mul-sum has a different element count than its
+    # source, so the view rule treats it as padding and slices instead of summing
+    # (src/grad/rules.rs:586-612); the gradient tensor is then a [2,3] view of a [2,3,4]
+    # buffer, which is what to_vec returns -- the reference's optimiser rejects exactly this
+    # length mismatch (crates/nn/src/optim/optimizer.rs:118-125)
+    xm = np.arange(6, dtype=np.float32).reshape(2, 3)
+    w = (np.arange(12, dtype=np.float32).reshape(4, 3) - 5) / 4
+    gx, gw = _grads_on(frontend, "c",
+                       lambda t, u: frontend.nn.linear(t, u).sum(1).sum(0), [xm, w])
+    assert gx.size == 24 and np.allclose(gx.reshape(2, 3, 4), np.broadcast_to(w.T, (2, 3, 4)))
+    # the weight's gradient keeps only batch row 0 (slice, not sum) and reaches [4,3] by a
+    # reshape of the [3,4] product instead of a transpose
+    assert gw.size == 12 and np.array_equal(gw, np.repeat(xm[0], 4))
+
+
+def _exact_grads_on(fe, kind, build_loss, arrays):
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    fe.set_device_str(kind)
+    try:
+        ts = []
+        for a in arrays:
+            t = fe.Tensor.input(list(a.shape))
+            t.set_data(a)
+            ts.append(t)
+        with fe.exact_mode():
+            loss = build_loss(*ts)
+            loss.backward_with_params(ts)
+            out = []
+            for t in ts:
+                g = t.grad().contiguous()          # a gradient may be a pure view
+                g.realize()
+                out.append(g.to_numpy().reshape(t.shape()))
+        return out
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+
+
+def test_exact_gradients_match_calculus(frontend):
+    """The exact mode (not in the reference) against closed-form derivatives."""
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-1, 1, (5, 3)).astype(np.float32)
+    w = rng.uniform(-1, 1, (4, 3)).astype(np.float32)
+    b = rng.uniform(-1, 1, (4,)).astype(np.float32)
+    t = rng.uniform(-1, 1, (5, 4)).astype(np.float32)
+
+    def loss(xt, wt, bt, tt):
+        d = frontend.nn.linear(xt, wt, bt) - tt
+        return (d * d).sum(1).sum(0)
+    gx, gw, gb, gt = _exact_grads_on(frontend, "c", loss, [x, w, b, t])
+    d = x @ w.T + b - t
+    assert np.allclose(gx, 2 * d @ w, rtol=1e-5, atol=1e-6)
+    assert np.allclose(gw, 2 * d.T @ x, rtol=1e-5, atol=1e-6)
+    assert np.allclose(gb, 2 * d.sum(0), rtol=1e-5, atol=1e-6)
+    assert np.allclose(gt, -2 * d, rtol=1e-5, atol=1e-6)
+
+    a = rng.uniform(0.5, 2.0, (6,)).astype(np.float32)
+    c = rng.uniform(0.5, 2.0, (6,)).astype(np.float32)
+    ga, gc = _exact_grads_on(frontend, "c", lambda s, u: ((s / u).exp() * s.ln()).sum(0), [a, c])
+    e = np.exp(a / c)
+    assert np.allclose(ga, e / c * np.log(a) + e / a, rtol=1e-5)
+    assert np.allclose(gc, -e * a / c ** 2 * np.log(a), rtol=1e-5)
+    (gr,) = _exact_grads_on(frontend, "c", lambda s: frontend.nn.relu(s - s.exp2()).sum(0), [a - 1.2])
+    z = (a - 1.2) - np.exp2(a - 1.2)
+    assert np.allclose(gr, (z >= 0) * (1 - np.exp2(a - 1.2) * np.log(2)), rtol=1e-5, atol=1e-6)
+    m = rng.normal(0, 1, (4, 7)).astype(np.float32)
+    (gm,) = _exact_grads_on(frontend, "c", lambda s: (frontend.nn.softmax(s, 1) * s).sum(1).sum(0), [m])
+    p = np.exp(m - m.max(1, keepdims=True))
+    p /= p.sum(1, keepdims=True)
+    ref = p + p * (m - (p * m).sum(1, keepdims=True))
+    assert np.allclose(gm, ref, rtol=1e-4, atol=1e-5)
