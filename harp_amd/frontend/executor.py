@@ -58,7 +58,7 @@ def _root_buffer_name(root: GraphNode, lowerer, available: Sequence[str], opt_ro
     # the optimised graph's root (graph passes rebuild nodes), or -- when that root is a view
     # that was inlined -- the node whose buffer it views
     n = opt_root
-    while n is not None:
+    while n is not None and not n.is_external():
         name = lowerer.lookup_buffer_name(n)
         if name is not None and name in available:
             return name
