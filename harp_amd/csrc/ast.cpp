@@ -363,8 +363,9 @@ NodePtr to_node(const SX& s) {
               bi.shape.push_back(v);
             }
             bi.role = b.items[3].atom;
-            if (bi.role != "input" && bi.role != "output" && bi.role != "temp")
-              fail(b, "role must be input, output or temp");
+            if (bi.role != "input" && bi.role != "output" && bi.role != "temp" && bi.role != "ones" &&
+                bi.role != "zeros")
+              fail(b, "role must be input, output, temp, ones or zeros");
             n->buffers.push_back(std::move(bi));
           }
         } else {

@@ -378,7 +378,7 @@ void HipProgram::execute_positional(HipBuffer* const* inputs, size_t n_in, HipBu
   size_t ii = 0, oi = 0;
   for (size_t i = 0; i < plan_.buffers.size(); ++i) {
     const std::string& role = plan_.buffers[i].role;
-    if (role == "input") {
+    if (role == "input" || role == "ones" || role == "zeros") {
       if (ii >= n_in) throw Error("kernel takes more inputs than the " + std::to_string(n_in) + " given");
       bufs[i] = inputs[ii++];
     } else if (role == "output") {

@@ -538,7 +538,7 @@ Canon canon_as(const NestKernel& k, StageKind kind) {
 // The emitters live below; declared here so plan_program reads top-down.
 namespace {
 LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& buf_elems);
-LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt);
+void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan);
 }  // namespace
 
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
@@ -587,8 +587,50 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     for (const auto& p : kernels[i]->params)
       if (p.dtype.is_ptr() && !p.mut_) readers[p.name].push_back(i);
 
+  // inputs the executor itself fills with a constant (role ones / zeros): reads of them are
+  // folded into literals wherever a kernel is recognised, so they cost no memory traffic
+  std::map<std::string, double> consts;
+  for (const auto& b : plan.buffers) {
+    if (b.role == "ones") consts[b.name] = 1.0;
+    if (b.role == "zeros") consts[b.name] = 0.0;
+  }
+  std::function<NodePtr(const NodePtr&)> fold = [&](const NodePtr& n) -> NodePtr {
+    if (n->op == Op::Load && n->args[0]->op == Op::Var && consts.count(n->args[0]->name) && n->count == 1) {
+      auto c = std::make_shared<Node>(Op::Const);
+      c->dtype = n->dtype;
+      c->fval = consts.at(n->args[0]->name);
+      c->ival = static_cast<int64_t>(c->fval);
+      return c;
+    }
+    bool changed = false;
+    std::vector<NodePtr> args;
+    for (const auto& a : n->args) {
+      NodePtr r = fold(a);
+      changed = changed || r != a;
+      args.push_back(std::move(r));
+    }
+    if (!changed) return n;
+    auto c = std::make_shared<Node>(*n);
+    c->args = std::move(args);
+    return c;
+  };
+
   std::vector<std::optional<NestKernel>> nests;
-  for (const Node* k : kernels) nests.push_back(extract_nest(*k));
+  for (const Node* k : kernels) {
+    nests.push_back(extract_nest(*k));
+    if (nests.back() && !consts.empty()) {
+      NestKernel& nk = *nests.back();
+      nk.value = fold(nk.value);
+      std::vector<LoadRef> loads;
+      collect_loads(*nk.value, loads);
+      std::set<std::string> used;
+      for (const auto& lr : loads) used.insert(lr.load->args[0]->name);
+      std::vector<Param> kept;
+      for (const auto& p : nk.params)
+        if (p.mut_ || used.count(p.name) || !consts.count(p.name)) kept.push_back(p);
+      nk.params = kept;
+    }
+  }
 
   size_t i = 0;
   while (i < kernels.size()) {
@@ -607,7 +649,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       }
     }
     if (k0.rkind != ReduceKind::None && !reduce_is_rowwise(k0)) {
-      plan.launches.push_back(emit_serial_reduce(k0, opt));
+      emit_serial_reduce(k0, opt, &plan);
       ++i;
       continue;
     }
@@ -658,6 +700,13 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (!needed) plan.elided.insert(st.out_buf);
     }
     plan.launches.push_back(emit_group(g, opt, elems));
+  }
+  // constant inputs no launch binds any more need not exist
+  for (const auto& c : consts) {
+    bool bound = false;
+    for (const auto& ls : plan.launches)
+      for (const auto& a : ls.arg_bufs) bound = bound || a == c.first;
+    if (!bound) plan.elided.insert(c.first);
   }
   return plan;
 }
@@ -1100,22 +1149,28 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
   return ge.emit_rows(elems);
 }
 
-// One thread per output element, the reduce loop runs serially inside it.  Used when the
-// reduce axis is not the contiguous one: adjacent threads then read adjacent addresses.
-LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt) {
-  LaunchSpec ls;
+// Reductions over a non-contiguous axis that are not contractions.  One thread per output
+// element, adjacent threads on adjacent outputs (so loads along the fastest output axis
+// coalesce), the reduce loop serial inside the thread.  When there are few outputs and a long
+// reduce axis the axis is split over gridDim.y: each workgroup (64 outputs x 4 row phases)
+// reduces one chunk into a scratch buffer [chunks][outputs] and a second launch combines the
+// chunks -- deterministic, no atomics.
+struct SerialReduce {
+  const NestKernel& k;
+  const GenOptions& opt;
   std::vector<Loop> live;
   std::map<std::string, NodePtr> zero;
-  for (const auto& l : k.loops) {
-    if (l.extent == 0) throw Error("kernel '" + k.name + "' has an empty loop");
-    if (l.extent == 1) zero[l.var] = make_i64(0);
-    else live.push_back(l);
-  }
-  if (k.rloop.extent == 0) throw Error("kernel '" + k.name + "' reduces over an empty axis");
   int64_t N = 1;
-  for (const auto& l : live) N *= l.extent;
   bool idx64 = false;
-  {
+
+  SerialReduce(const NestKernel& kk, const GenOptions& o) : k(kk), opt(o) {
+    for (const auto& l : k.loops) {
+      if (l.extent == 0) throw Error("kernel '" + k.name + "' has an empty loop");
+      if (l.extent == 1) zero[l.var] = make_i64(0);
+      else live.push_back(l);
+    }
+    if (k.rloop.extent == 0) throw Error("kernel '" + k.name + "' reduces over an empty axis");
+    for (const auto& l : live) N *= l.extent;
     std::vector<LoadRef> loads;
     collect_loads(*k.value, loads);
     int64_t reach = max_abs_index(*k.out_aff, k.loops, &k.rloop);
@@ -1126,39 +1181,29 @@ LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt) {
     }
     if (reach >= (int64_t{1} << 31) - 8 || N >= (int64_t{1} << 31) - 8) idx64 = true;
   }
-  const int block = 256;
-  const int64_t blocks = (N + block - 1) / block;
-  if (blocks >= (int64_t{1} << 31)) throw Error("too many outputs for one launch");
-  ls.entry = "ehk_" + k.name;
-  ls.kernels = {k.name};
-  ls.schedule = "serial-reduce(block=256)";
-  ls.grid[0] = static_cast<unsigned>(blocks);
-  ls.block[0] = block;
-  std::ostringstream os;
-  os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
-  os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(";
-  bool first = true;
-  for (const auto& p : k.params) {
-    os << (first ? "" : ", ") << (p.mut_ ? "" : "const ") << ctype(p.dtype.elem()) << "* __restrict__ " << p.name;
-    first = false;
-    ls.arg_bufs.push_back(p.name);
+
+  std::string params(LaunchSpec* ls, bool with_out, const std::string& extra) const {
+    std::string t;
+    for (const auto& p : k.params) {
+      if (p.mut_ && !with_out) continue;
+      t += (t.empty() ? "" : ", ") + std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + p.name;
+      ls->arg_bufs.push_back(p.name);
+    }
+    if (!extra.empty()) t += (t.empty() ? "" : ", ") + extra;
+    return t;
   }
-  os << ") {\n  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
-  os << "  idx_t eh_rem = eh_o;\n";
-  for (size_t i = live.size(); i-- > 0;) {
-    os << "  const idx_t " << live[i].var << " = eh_rem % " << live[i].extent << ";\n";
-    if (i) os << "  eh_rem /= " << live[i].extent << ";\n";
+
+  std::string decode(const std::string& ovar) const {
+    std::string t = "  idx_t eh_rem = " + ovar + ";\n";
+    for (size_t i = live.size(); i-- > 0;) {
+      t += "  const idx_t " + live[i].var + " = eh_rem % " + std::to_string(live[i].extent) + ";\n";
+      if (i) t += "  eh_rem /= " + std::to_string(live[i].extent) + ";\n";
+    }
+    for (const auto& z : zero) t += "  const idx_t " + z.first + " = 0;\n";
+    return t;
   }
-  for (const auto& z : zero) os << "  const idx_t " << z.first << " = 0;\n";
-  ExprRenderer er;
-  const std::string TA = ctype(k.acc_dtype);
-  os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
-  os << "  for (idx_t " << k.rloop.var << " = 0; " << k.rloop.var << " < " << k.rloop.extent << "; ++" << k.rloop.var << ") {\n";
-  os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
-  NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
-  os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
-  ls.source = os.str();
-  {
+
+  void min_bytes(LaunchSpec* ls) const {
     std::map<std::string, int64_t> need;
     std::vector<LoadRef> loads;
     collect_loads(*k.value, loads);
@@ -1166,16 +1211,132 @@ LaunchSpec emit_serial_reduce(const NestKernel& k, const GenOptions& opt) {
     for (const auto& lr : loads) {
       auto a = affine_of(*lr.load->args[1]);
       if (!a) { opaque = true; continue; }
+      if (lr.guarded) continue;
       auto& n = need[lr.load->args[0]->name];
       n = std::max(n, max_abs_index(*a, k.loops, &k.rloop) + 1);
     }
     need[k.out_buf] = max_abs_index(*k.out_aff, k.loops, nullptr) + 1;
-    for (const auto& p : k.params) {
-      auto it = need.find(p.name);
-      ls.arg_min_bytes.push_back(it == need.end() || (opaque && !p.mut_) ? 0 : static_cast<size_t>(it->second) * p.dtype.elem().itemsize());
+    for (const auto& b : ls->arg_bufs) {
+      size_t item = 4;
+      bool is_out = false;
+      for (const auto& p : k.params)
+        if (p.name == b) { item = p.dtype.elem().itemsize(); is_out = p.mut_; }
+      auto it = need.find(b);
+      ls->arg_min_bytes.push_back(it == need.end() || (opaque && !is_out) ? 0 : static_cast<size_t>(it->second) * item);
     }
   }
-  return ls;
+
+  LaunchSpec single() const {
+    LaunchSpec ls;
+    const int block = 256;
+    const int64_t blocks = (N + block - 1) / block;
+    if (blocks >= (int64_t{1} << 31)) throw Error("too many outputs for one launch");
+    ls.entry = "ehk_" + k.name;
+    ls.kernels = {k.name};
+    ls.schedule = "serial-reduce(block=256)";
+    ls.grid[0] = static_cast<unsigned>(blocks);
+    ls.block[0] = block;
+    std::ostringstream os;
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << params(&ls, true, "") << ") {\n";
+    os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
+    os << decode("eh_o");
+    ExprRenderer er;
+    const std::string TA = ctype(k.acc_dtype);
+    os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+    os << "  for (idx_t " << k.rloop.var << " = 0; " << k.rloop.var << " < " << k.rloop.extent << "; ++" << k.rloop.var << ") {\n";
+    os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
+    NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
+    os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
+    ls.source = os.str();
+    min_bytes(&ls);
+    return ls;
+  }
+
+  bool wants_split() const { return k.rloop.extent >= 512 && N <= (1 << 18); }
+
+  // Two launches and one scratch buffer (appended to `buffers`).
+  std::vector<LaunchSpec> split(std::vector<BufferInfo>* buffers) const {
+    const int64_t K = k.rloop.extent;
+    const int64_t cols = (N + 63) / 64;
+    int64_t S = std::max<int64_t>(1, std::min<int64_t>((2048 + cols - 1) / cols, K / 64));
+    const int64_t CH = (K + S - 1) / S;
+    S = (K + CH - 1) / CH;
+    const std::string TA = ctype(k.acc_dtype);
+    const std::string scratch = "eh_part_" + k.name;
+    BufferInfo sb;
+    sb.name = scratch;
+    sb.dtype = k.acc_dtype;
+    sb.shape = {S, N};
+    sb.role = "temp";
+    buffers->push_back(sb);
+    ExprRenderer er;
+    std::vector<LaunchSpec> out(2);
+    {
+      LaunchSpec& ls = out[0];
+      ls.entry = "ehk_" + k.name + "_part";
+      ls.kernels = {k.name};
+      ls.schedule = "split-reduce(chunks=" + std::to_string(S) + ",rows/chunk=" + std::to_string(CH) + ")";
+      ls.grid[0] = static_cast<unsigned>(cols);
+      ls.grid[1] = static_cast<unsigned>(S);
+      ls.block[0] = 256;
+      std::ostringstream os;
+      os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+      os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "("
+         << params(&ls, false, TA + "* __restrict__ " + scratch) << ") {\n";
+      ls.arg_bufs.push_back(scratch);
+      os << "  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;\n";
+      os << "  const idx_t eh_oo = (idx_t)blockIdx.x * 64 + tx;\n  const bool eh_ok = eh_oo < " << N << ";\n";
+      os << "  const idx_t eh_o = eh_ok ? eh_oo : " << N - 1 << ";\n";
+      os << decode("eh_o");
+      os << "  const idx_t eh_r0 = (idx_t)blockIdx.y * " << CH << ";\n";
+      os << "  const idx_t eh_r1 = eh_r0 + " << CH << " < " << K << " ? eh_r0 + " << CH << " : " << K << ";\n";
+      os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+      os << "  for (idx_t " << k.rloop.var << " = eh_r0 + ty; " << k.rloop.var << " < eh_r1; " << k.rloop.var << " += 4) {\n";
+      os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
+      os << "  __shared__ " << TA << " eh_sm[4][64];\n  eh_sm[ty][tx] = acc;\n  __syncthreads();\n";
+      os << "  if (ty == 0 && eh_ok) {\n    " << TA << " r = eh_sm[0][tx];\n";
+      for (int q = 1; q < 4; ++q)
+        os << "    r = " << combine_text(k.rkind, k.acc_dtype, "r", "eh_sm[" + std::to_string(q) + "][tx]") << ";\n";
+      os << "    " << scratch << "[(idx_t)blockIdx.y * " << N << " + eh_oo] = r;\n  }\n}\n";
+      ls.source = os.str();
+      min_bytes(&ls);
+      ls.arg_min_bytes.back() = static_cast<size_t>(S * N) * k.acc_dtype.itemsize();
+    }
+    {
+      LaunchSpec& ls = out[1];
+      ls.entry = "ehk_" + k.name;
+      ls.kernels = {k.name};
+      ls.schedule = "split-reduce-final(chunks=" + std::to_string(S) + ")";
+      ls.grid[0] = static_cast<unsigned>((N + 255) / 256);
+      ls.block[0] = 256;
+      std::ostringstream os;
+      os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+      os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(const " << TA << "* __restrict__ "
+         << scratch << ", " << ctype(k.out_dtype) << "* __restrict__ " << k.out_buf << ") {\n";
+      ls.arg_bufs = {scratch, k.out_buf};
+      os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
+      os << decode("eh_o");
+      os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+      os << "  for (idx_t s = 0; s < " << S << "; ++s) acc = "
+         << combine_text(k.rkind, k.acc_dtype, "acc", scratch + "[s * " + std::to_string(N) + " + eh_o]") << ";\n";
+      NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
+      os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
+      ls.source = os.str();
+      ls.arg_min_bytes = {static_cast<size_t>(S * N) * k.acc_dtype.itemsize(),
+                          static_cast<size_t>(max_abs_index(*k.out_aff, k.loops, nullptr) + 1) * k.out_dtype.itemsize()};
+    }
+    return out;
+  }
+};
+
+void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan) {
+  SerialReduce sr(k, opt);
+  if (sr.wants_split()) {
+    for (auto& ls : sr.split(&plan->buffers)) plan->launches.push_back(std::move(ls));
+  } else {
+    plan->launches.push_back(sr.single());
+  }
 }
 
 }  // namespace

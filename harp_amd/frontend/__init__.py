@@ -11,7 +11,7 @@ from .executor import ExecutionError, execute_graph
 from .expr import Expr
 from .graph import GraphNode, GraphOp
 from .lowerer import Lowerer, all_fusions, lower_graph
-from .tensor import Tensor
+from .tensor import Tensor, realize_many
 from .view import View
 from . import nn
 from .config import exact_mode

@@ -32,9 +32,11 @@ def _const_shape(shape) -> List[int]:
 
 
 def buffer_table(program: AstNode, lowerer, input_names: Sequence[str],
-                 output_names: Sequence[str]) -> List[dict]:
-    """Name, dtype, shape and role (input | output | temp) of every buffer
-    the program's kernels touch, in first-use order."""
+                 output_names: Sequence[str], constants: Dict[str, str] = None) -> List[dict]:
+    """Name, dtype, shape and role (input | output | temp | ones | zeros) of every
+    buffer the program's kernels touch, in first-use order.  `constants` names the inputs
+    the executor itself filled with 1.0 / 0.0."""
+    constants = constants or {}
     seen, table = set(), []
     for kern in program.args:
         for p in kern.attrs["params"]:
@@ -44,7 +46,8 @@ def buffer_table(program: AstNode, lowerer, input_names: Sequence[str],
             info = lowerer.get_buffer_info_by_name(p.name)
             if info is None:
                 raise ExecutionError(f"no shape known for buffer '{p.name}'")
-            role = ("input" if p.name in input_names
+            role = (constants[p.name] if p.name in constants
+                    else "input" if p.name in input_names
                     else "output" if p.name in output_names else "temp")
             table.append({"name": p.name, "dtype": info[1],
                           "shape": _const_shape(info[0]), "role": role})
@@ -73,8 +76,10 @@ def _root_buffer_name(root: GraphNode, lowerer, available: Sequence[str], opt_ro
 
 
 def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
-                  fuse_program: bool = None):
-    """Returns one buffer per root (None where the reference finds none)."""
+                  fuse_program: bool = None, constant_inputs: Dict[int, str] = None):
+    """Returns one buffer per root (None where the reference finds none).
+    `constant_inputs` maps id(input node) -> "ones" | "zeros" for inputs whose buffer
+    the caller synthesised (realize.rs:391-421); a whole-program backend may fold them."""
     dev = get_default_device()
     if dev is None:
         raise ExecutionError("NoDevice")
@@ -101,7 +106,12 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
             nm = _root_buffer_name(r, lowerer, all_names, o)
             if nm is not None and nm not in out_names:
                 out_names.append(nm)
-        table = buffer_table(program, lowerer, list(buffer_map.keys()), out_names)
+        consts = {}
+        for n in input_nodes:
+            kind = (constant_inputs or {}).get(id(n))
+            if kind:
+                consts[lowerer.lookup_buffer_name(n)] = kind
+        table = buffer_table(program, lowerer, list(buffer_map.keys()), out_names, consts)
         prog_ast = AstNode.program(kernels, buffers=table)
         compiled = dev.compile_program(prog_ast)
         outs = compiled.execute({k: v for k, v in buffer_map.items()})

@@ -354,8 +354,8 @@ def compute_vjp_exact(node: GraphNode, g: GraphNode) -> List[Optional[GraphNode]
             nw = node.unsqueeze(axis) if node.ndim() < x.ndim() else node
             full = nw.repeat(axis, size)
             if rop in ("max", "min"):
-                return [_dense(ge) * x.eq_node(full).cast(x.dtype)]
-            return [(_dense(ge) * full) / x]
+                return [ge * x.eq_node(full).cast(x.dtype)]
+            return [(ge * full) / x]
         raise NotImplementedError("exact VJP of a reduce with a fused map: differentiate before fusion")
     if op.kind == "map_reduce":
         return _elementwise_vjp_exact(node, g, op.map)
@@ -364,7 +364,8 @@ def compute_vjp_exact(node: GraphNode, g: GraphNode) -> List[Optional[GraphNode]
 
 def _elementwise_vjp_exact(node, g, m) -> List[Optional[GraphNode]]:
     ins = node.src
-    g = _dense(g)
+    # g may be a broadcast view; unary results inherit that view (stored compactly), which
+    # every reader then indexes consistently, so only selects need a dense operand
     if m.op == "add" and _is_w(m.args[0], 0) and m.args[1].op == "mul" and \
             _is_w(m.args[1].args[0], 1) and _is_f32(m.args[1].args[1], -1.0):
         return [g, -g]                                   # a - b

@@ -343,14 +343,21 @@ def collect_inputs(roots: Sequence[GraphNode]) -> List[GraphNode]:
 
 
 def apply_transform(transform: Callable[[GraphNode], Optional[GraphNode]],
-                    roots: Sequence[GraphNode]) -> List[GraphNode]:
+                    roots: Sequence[GraphNode], share_cache: bool = False) -> List[GraphNode]:
     """GraphTransform::apply (traversal.rs:197-245): bottom-up, a fresh cache
-    per root, nodes rebuilt only when a source changed."""
+    per root, nodes rebuilt only when a source changed.  `share_cache` keeps one cache
+    for all roots, so nodes common to several roots stay common (the reference rebuilds
+    them once per root)."""
     out = []
+    shared: Dict[int, GraphNode] = {}
+    keep = []
     for root in roots:
-        cache: Dict[int, GraphNode] = {}
+        cache: Dict[int, GraphNode] = shared if share_cache else {}
         order = topological_sort([root])
+        keep.append(order)
         for node in order:
+            if id(node) in cache:
+                continue
             new_src = [cache[id(s)] for s in node.src]
             changed = any(a is not b for a, b in zip(new_src, node.src))
             cur = node.with_new_sources(new_src) if changed else node

@@ -54,12 +54,15 @@ def _elementwise_reduce_fusion(node: GraphNode) -> Optional[GraphNode]:
     return None
 
 
-def fuse_views(roots): return apply_transform(_view_fusion, roots)
-def fuse_elementwise_reduce(roots): return apply_transform(_elementwise_reduce_fusion, roots)
+def fuse_views(roots, share=False): return apply_transform(_view_fusion, roots, share)
 
 
-def all_fusions(roots: Sequence[GraphNode]) -> List[GraphNode]:
-    return fuse_elementwise_reduce(fuse_views(roots))
+def fuse_elementwise_reduce(roots, share=False):
+    return apply_transform(_elementwise_reduce_fusion, roots, share)
+
+
+def all_fusions(roots: Sequence[GraphNode], share: bool = False) -> List[GraphNode]:
+    return fuse_elementwise_reduce(fuse_views(roots, share), share)
 
 
 # --------------------------------------------------------------------------
@@ -434,7 +437,7 @@ def lower_graph(roots: Sequence[GraphNode], optimize: bool = True, exact_views: 
         exact_views = config.EXACT
     if exact_views:
         roots = unshare_views(roots)
-    opt_roots = all_fusions(roots) if optimize else list(roots)
+    opt_roots = all_fusions(roots, share=exact_views) if optimize else list(roots)
     lw = Lowerer()
     program = lw.lower(opt_roots)
     return program, lw, opt_roots

@@ -268,6 +268,7 @@ class Tensor:
             self.buffer = hit[1].clone_buffer()
             return self
         input_buffers = {}
+        constant_inputs = {}
         for node in G.collect_inputs([g]):
             hit = _INPUT_BUFFER_CACHE.get(id(node))
             if hit is not None:
@@ -279,7 +280,8 @@ class Tensor:
                                      f"'{node.name or hex(id(node))}' has no data. "
                                      f"Call set_data() first.")
             input_buffers[id(node)] = const
-        res = execute_graph([g], input_buffers)
+            constant_inputs[id(node)] = "zeros" if node.name == "zeros" else "ones"
+        res = execute_graph([g], input_buffers, constant_inputs=constant_inputs)
         if not res or res[0] is None:
             raise ExecutionError("Internal: No output buffer returned from execution")
         self.buffer = res[0]
@@ -297,6 +299,37 @@ class Tensor:
 
     def clear_buffer(self) -> None:
         self.buffer = None
+
+
+def realize_many(tensors: Sequence[Tensor]) -> None:
+    """Realizes several tensors with one `execute_graph` call (`execute_graph` takes a slice
+    of roots, executor.rs:149-152), so work they share is done once."""
+    todo = [t for t in tensors if not t.is_realized() and not t.graph.is_external()]
+    for t in tensors:
+        if t.graph.is_external():
+            t.realize()
+    if not todo:
+        return
+    if not has_default_device():
+        raise ExecutionError("NoDevice")
+    roots = [t.graph for t in todo]
+    input_buffers, constant_inputs = {}, {}
+    for node in G.collect_inputs(roots):
+        hit = _INPUT_BUFFER_CACHE.get(id(node))
+        if hit is not None:
+            input_buffers[id(node)] = hit[1].clone_buffer()
+            continue
+        const = _create_constant_buffer(node)
+        if const is None:
+            raise ExecutionError(f"MissingInput: Input tensor '{node.name or hex(id(node))}' "
+                                 f"has no data. Call set_data() first.")
+        input_buffers[id(node)] = const
+        constant_inputs[id(node)] = "zeros" if node.name == "zeros" else "ones"
+    res = execute_graph(roots, input_buffers, constant_inputs=constant_inputs)
+    for t, b in zip(todo, res):
+        if b is None:
+            raise ExecutionError("Internal: No output buffer returned from execution")
+        t.buffer = b
 
 
 def _create_constant_buffer(node: G.GraphNode):

@@ -65,7 +65,77 @@ def lower_with_table(shapes: List[Tuple[int, ...]], graph_fn: Callable):
     numbered = [n for n in produced if n.startswith("buf") and n[3:].isdigit()]
     out = max(numbered, key=lambda s: int(s[3:]))
     all_inputs = list(by_id.values())
-    table = buffer_table(prog, lw, all_inputs, [out])
     const_inputs = {by_id[id(n)]: n.name for n in collect_inputs([y.graph])
                     if by_id[id(n)] not in arg_names}
+    table = buffer_table(prog, lw, all_inputs, [out],
+                         {k: ("zeros" if v == "zeros" else "ones") for k, v in const_inputs.items()})
     return AstNode.program(list(prog.args), buffers=table), arg_names, out, const_inputs, prog
+
+
+# ---------------------------------------------------------------------------
+# config 4: MLP training step (exact gradients; see harp_amd/frontend/config.py)
+# ---------------------------------------------------------------------------
+
+def tanh_exact(x: Tensor) -> Tensor:
+    """tanh(x) = 2*sigmoid(2x) - 1 with the factors actually applied (the reference's
+    `nn::tanh` loses them because `Tensor::scale` ignores its argument)."""
+    sig = nn.sigmoid(x.scale_exact(2.0))
+    return sig.scale_exact(2.0) - Tensor.ones_like(x)
+
+
+def mlp_sizes(full: bool = True):
+    return (8192, [1024, 4096, 4096, 1024]) if full else (64, [32, 64, 64, 32])
+
+
+def config4_inputs(batch: int = 8192, dims=(1024, 4096, 4096, 1024), seed: int = 1237):
+    """x ~ U(-pi, pi), target sin(x) (first/last width must match), W ~ U(+-1/sqrt(fan_in))."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-np.pi, np.pi, (batch, dims[0])).astype(np.float32)
+    t = np.sin(x[:, :dims[-1]]).astype(np.float32)
+    params = []
+    for fan_in, fan_out in zip(dims[:-1], dims[1:]):
+        k = 1.0 / np.sqrt(fan_in)
+        params.append(rng.uniform(-k, k, (fan_out, fan_in)).astype(np.float32))
+        params.append(rng.uniform(-k, k, (fan_out,)).astype(np.float32))
+    return [x, t] + params
+
+
+def config4_graph(x: Tensor, t: Tensor, *params: Tensor, lr: float = 1e-3):
+    """One SGD step as a single graph: forward, mean-squared error, exact backward,
+    p - lr*grad for every parameter.  Returns [new parameters..., loss]."""
+    from .frontend import exact_mode
+    with exact_mode():
+        h = x
+        n_layers = len(params) // 2
+        for i in range(n_layers):
+            h = nn.linear(h, params[2 * i], params[2 * i + 1])
+            if i + 1 < n_layers:
+                h = tanh_exact(h)
+        d = h - t
+        n = 1
+        for s in d.shape():
+            n *= s
+        loss = (d * d).sum(1).sum(0).scale_exact(1.0 / n)
+        loss.backward_with_params(list(params))
+        new_params = [p - p.grad().scale_exact(lr) for p in params]
+    return new_params + [loss]
+
+
+def lower_multi(tensors_in, roots):
+    """Lowers several roots into one Program with a buffer table.  Returns (program AST,
+    input buffer names in the order of `tensors_in`, output buffer name per root, constant
+    inputs {buffer name: "ones" | "zeros"})."""
+    from .frontend import exact_mode
+    from .frontend.executor import _root_buffer_name
+    with exact_mode():
+        prog, lw, opt_roots = lower_graph([r.graph for r in roots])
+    all_inputs = collect_inputs([r.graph for r in roots])
+    by_id = {id(n): lw.lookup_buffer_name(n) for n in all_inputs}
+    arg_names = [by_id[id(t.graph)] for t in tensors_in]
+    produced = [p.name for k in prog.args for p in k.attrs["params"] if p.dtype.is_ptr() and p.mutable]
+    avail = list(by_id.values()) + produced
+    outs = [_root_buffer_name(r.graph, lw, avail, o) for r, o in zip(roots, opt_roots)]
+    consts = {by_id[id(n)]: n.name for n in all_inputs if by_id[id(n)] not in arg_names}
+    table = buffer_table(prog, lw, list(by_id.values()), outs,
+                         {k: ("zeros" if v == "zeros" else "ones") for k, v in consts.items()})
+    return AstNode.program(list(prog.args), buffers=table), arg_names, outs, consts, prog

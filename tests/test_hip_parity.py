@@ -239,3 +239,68 @@ def test_kernel_binary_round_trip(frontend, hip):
         hip.HipModule(dev, b"not a code object", "k")
     with pytest.raises(hip.EhError):
         hip.HipModule(dev, blob, "no_such_entry")
+
+
+def _train_step_on(fe, kind, arrays, fuse=True):
+    """Config 4 graph (forward, MSE, exact backward, SGD update) realized with one
+    execute_graph call; returns [new parameters..., loss] as flat arrays."""
+    import os
+    from harp_amd import workloads as wl
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    fe.set_device_str(kind)
+    old = os.environ.get("ECLAT_HIP_FUSE")
+    os.environ["ECLAT_HIP_FUSE"] = "1" if fuse else "0"
+    try:
+        with fe.exact_mode():
+            ts = []
+            for a in arrays:
+                t = fe.Tensor.input(list(a.shape))
+                t.set_data(a)
+                ts.append(t)
+            roots = wl.config4_graph(*ts)
+            fe.realize_many(roots)
+            return [r.to_numpy() for r in roots]
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+        if old is None:
+            os.environ.pop("ECLAT_HIP_FUSE", None)
+        else:
+            os.environ["ECLAT_HIP_FUSE"] = old
+
+
+@pytest.mark.parametrize("batch,dims", [(64, (32, 64, 64, 32)), (256, (128, 256, 128, 128)), (50, (12, 20, 12))])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_config4_mlp_training_step(frontend, hip, batch, dims, fuse):
+    """BASELINE config 4 at oracle-sized shapes: every updated parameter and the loss match
+    the C oracle running the same graph; the step also matches a float64 numpy MLP."""
+    from harp_amd import workloads as wl
+    arrays = wl.config4_inputs(batch, dims, seed=99)
+    if dims[0] != dims[-1]:
+        arrays[1] = arrays[1][:, :dims[-1]]
+    ref = _train_step_on(frontend, "c", arrays)
+    got = _train_step_on(frontend, "hip", arrays, fuse)
+    for r, g, a in zip(ref, got, arrays[2:] + [np.zeros(1, np.float32)]):
+        assert r.shape == g.shape
+        # gradients are sums over the batch of products: reduction class, scaled by |param|+lr*|grad|
+        assert np.allclose(g, r, rtol=1e-5, atol=1e-6 * max(1.0, float(np.abs(r).max())))
+    # numpy float64 reference of the whole step
+    x, t = arrays[0].astype(np.float64), arrays[1].astype(np.float64)
+    ps = [p.astype(np.float64) for p in arrays[2:]]
+    hs, pre = [x], []
+    nl = len(ps) // 2
+    for i in range(nl):
+        z = hs[-1] @ ps[2 * i].T + ps[2 * i + 1]
+        pre.append(z)
+        hs.append(np.tanh(z) if i + 1 < nl else z)
+    d = hs[-1] - t
+    loss = (d * d).mean()
+    gz = 2 * d / d.size
+    grads = [None] * len(ps)
+    for i in range(nl - 1, -1, -1):
+        grads[2 * i] = gz.T @ hs[i]
+        grads[2 * i + 1] = gz.sum(0)
+        if i > 0:
+            gz = (gz @ ps[2 * i]) * (1 - np.tanh(pre[i - 1]) ** 2)
+    assert abs(float(got[-1][0]) - loss) <= 1e-4 * abs(loss)
+    for p, gr, g in zip(ps, grads, got[:-1]):
+        assert np.allclose(g.reshape(p.shape), p - 1e-3 * gr, rtol=1e-4, atol=1e-6)
