@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | copy (default: all but copy)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | copy (default: all but copy)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -188,6 +188,44 @@ def main():
         log(f"[bench] config1 relu-sum 1024^2: {cfg1['us']:.1f} us/step -> {cfg1['gbs']:.0f} GB/s")
         del sets
 
+    # ---- config 4: MLP 1024-4096-4096-1024, batch 8192, forward + backward + SGD ---------
+    mlp = None
+    if want("mlp"):
+        batch, dims = wl.mlp_sizes(True)
+        arrays = wl.config4_inputs(batch, dims)
+        from harp_amd.frontend import Tensor
+        ts = [Tensor.input(list(a.shape)) for a in arrays]
+        roots = wl.config4_graph(*ts)
+        prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
+        prog = hb.HipProgram(dev, prog_ast, options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 1)
+        k = max(3, min(args.steps, 20))
+        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 3))
+        flops = sum(l["flops"] for l in prog.launches)
+        algo = sum(l["algo_bytes"] for l in prog.launches)
+        mlp = {"ms": ms, "steps": k, "flops": flops, "algo_bytes": algo,
+               "lowered_kernels": len(plain.args), "launches": len(prog.launches),
+               "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
+        log(f"[bench] mlp step (batch {batch}, {dims}): {ms:.2f} ms/step -> {flops / ms / 1e9:.1f} TFLOP/s, "
+            f"{batch / ms * 1e3:.0f} samples/s; {mlp['lowered_kernels']} kernels -> {mlp['launches']} launches")
+        if not args.no_check:
+            named = sets[0][1]
+            x, t, params = arrays[0], arrays[1], arrays[2:]
+            h = x
+            for i in range(len(params) // 2):
+                h = h @ params[2 * i].T + params[2 * i + 1]
+                if i + 1 < len(params) // 2:
+                    h = np.tanh(h)
+            d = h.astype(np.float64) - t
+            loss = float((d * d).mean())
+            got_loss = float(named[outs[-1]].read_array(np.float32, (1,))[0])
+            assert abs(got_loss - loss) <= 1e-3 * abs(loss), f"mlp loss check failed: {got_loss} vs {loss}"
+            nb = params[-1].astype(np.float64) - 1e-3 * (2.0 * d / d.size).sum(0)
+            got_b = named[outs[-2]].read_array(np.float32, (dims[-1],))
+            assert np.allclose(got_b, nb, rtol=1e-4, atol=1e-7), "mlp bias update check failed"
+            mlp["loss"] = got_loss
+        del sets
+
     # ---- CPU baseline: the oracle's unfused C kernels on host cores -------------------------
     cpu = None
     if not args.no_cpu_baseline and softmax is not None:
@@ -209,6 +247,19 @@ def main():
                 "sample": f"{sub} of 4096 rows of A through the reference's ijk kernel "
                           f"(gcc -O3 -ffast-math), median of {reps_m} passes, {sec_m * 1e3:.0f} ms/pass"}
             log(f"[bench] cpu baseline matmul: {gflops:.2f} GFLOP/s (1 core, {sub}-row sample)")
+
+        if mlp is not None:
+            from harp_amd.frontend import exact_mode
+            sub = 4
+            arrays = wl.config4_inputs(sub, wl.mlp_sizes(True)[1])
+            with exact_mode():
+                sec_p, reps_p, _ = baseline.time_graph(lambda *ts: wl.config4_graph(*ts), arrays,
+                                                       min_seconds=4.0, max_reps=3)
+            result_extra["cpu_baseline_mlp"] = {
+                "value": sub / sec_p, "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": f"batch {sub} of 8192 through the same lowered kernels, unfused "
+                          f"(gcc -O3 -ffast-math), median of {reps_p} passes, {sec_p * 1e3:.0f} ms/pass"}
+            log(f"[bench] cpu baseline mlp: {sub / sec_p:.2f} samples/s (1 core, batch {sub})")
 
     head = softmax
     out = {
@@ -243,6 +294,13 @@ def main():
         result_extra["config1_relu_sum_1024"] = {"us_per_step": round(cfg1["us"], 2),
                                                  "value": round(cfg1["gbs"], 1), "unit": "GB/s",
                                                  "schedule": cfg1["launches"][0][1]}
+    if mlp:
+        result_extra["config4_mlp_step"] = {
+            "value": round(8192 / mlp["ms"] * 1e3, 1), "unit": "samples/s", "ms_per_step": round(mlp["ms"], 3),
+            "steps": mlp["steps"], "tflops": round(mlp["flops"] / mlp["ms"] / 1e9, 2),
+            "algorithmic_bytes": mlp["algo_bytes"], "lowered_kernels": mlp["lowered_kernels"],
+            "launches": mlp["launches"], "gemm_launches": mlp["gemm_launches"], "loss": mlp.get("loss"),
+            "workload": "MLP 1024-4096-4096-1024, batch 8192: forward, MSE, exact backward, SGD update, one Program"}
     result_extra["device"] = {"name": props["name"], "arch": props["arch"],
                               "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
     out["extra"] = result_extra

@@ -61,7 +61,8 @@ struct BufferInfo {
   std::string name;
   DType dtype;
   std::vector<int64_t> shape;
-  std::string role;  // input | output | temp
+  std::string role;  // input | output | temp | ones | zeros
+  bool shape_known = true;  // false when the program came without a buffer table
   size_t numel() const {
     size_t n = 1;
     for (auto d : shape) n *= static_cast<size_t>(d);

@@ -347,7 +347,7 @@ void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
       b = temps_[i];
     }
     if (b->device() != dev_) throw Error("buffer '" + bi.name + "' lives on another device");
-    if (!bi.shape.empty() || bi.role == "temp") {
+    if (bi.shape_known) {
       if (b->byte_len() < bi.bytes())
         throw Error("Buffer size mismatch: '" + bi.name + "' needs " + std::to_string(bi.bytes()) + " bytes, has " +
                     std::to_string(b->byte_len()));

@@ -89,7 +89,7 @@ int buffer_entry(const ProgramPlan& p, int i, const char** name, const char** ro
   const BufferInfo& b = p.buffers[static_cast<size_t>(i)];
   if (name) *name = b.name.c_str();
   if (role) *role = b.role.c_str();
-  if (bytes) *bytes = b.shape.empty() && b.role != "temp" ? 0 : b.bytes();
+  if (bytes) *bytes = b.shape_known ? b.bytes() : 0;
   if (elided) *elided = p.elided.count(b.name) ? 1 : 0;
   return EH_OK;
 }

@@ -566,6 +566,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           bi.name = p.name;
           bi.dtype = p.dtype.elem();
           bi.role = p.mut_ ? "output" : "input";
+          bi.shape_known = false;
           plan.buffers.push_back(bi);
         } else if (p.dtype.is_ptr() && p.mut_) {
           for (auto& b : plan.buffers)

@@ -27,10 +27,11 @@ def prepare(graph_fn: Callable, arrays: Sequence[np.ndarray], openmp: bool = Fal
     from harp_amd.frontend.graph import collect_inputs
     tensors = [Tensor.input(list(a.shape)) for a in arrays]
     y = graph_fn(*tensors)
-    prog, lw, _ = lower_graph([y.graph])
+    roots = [r.graph for r in y] if isinstance(y, (list, tuple)) else [y.graph]
+    prog, lw, _ = lower_graph(roots)
     bufs: Dict[str, CBuffer] = {}
     by_id = {id(t.graph): a for t, a in zip(tensors, arrays)}
-    for n in collect_inputs([y.graph]):
+    for n in collect_inputs(roots):
         name = lw.lookup_buffer_name(n)
         b = CBuffer([int(e.evaluate()) for e in n.shape()], n.dtype.name)
         if id(n) in by_id:

@@ -214,3 +214,29 @@ def test_kernel_cache_counts(frontend):
     s2 = frontend.cache_stats()
     assert s1["misses"] == 1 and s1["hits"] == 0
     assert s2["misses"] == 1 and s2["hits"] == 1 and s2["entries"] == 1
+
+
+def test_config4_training_step_plan(frontend):
+    """The MLP step (forward, loss, exact backward, SGD) lowers to one multi-root Program whose
+    matmuls all take the MFMA schedule, whose bias gradients take the two-launch column
+    reduce, and whose synthesised ones/zeros inputs never become device buffers."""
+    from harp_amd import backend as hb, workloads as wl
+    batch, dims = 256, (128, 256, 128, 128)
+    shapes = [(batch, dims[0]), (batch, dims[-1])]
+    for a, b in zip(dims[:-1], dims[1:]):
+        shapes += [(b, a), (b,)]
+    ts = [frontend.Tensor.input(list(s)) for s in shapes]
+    roots = wl.config4_graph(*ts)
+    prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
+    assert len(outs) == len(set(outs)) == 7 and len(arg_names) == 8
+    plan = hb.render_program(prog_ast)
+    assert len(plan.launches) < len(plain.args) // 2
+    scheds = [l["schedule"] for l in plan.launches]
+    assert sum(s.startswith("mfma32x32x2(") for s in scheds) == 8      # 3 forward, 3 dW, 2 dX
+    assert sum("-reduce(" in s for s in scheds) == 3                   # bias gradients (column sums)
+    by_name = {b["name"]: b for b in plan.buffers}
+    assert by_name[outs[-1]]["bytes"] == 4 and by_name[outs[-1]]["role"] == "output"   # scalar loss
+    for name in consts:
+        assert by_name[name]["elided"], name
+    for src in {l["source"] for l in plan.launches}:
+        assert len(hb.compile_source(src)) > 1000
