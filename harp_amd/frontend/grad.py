@@ -359,7 +359,9 @@ def compute_vjp_exact(node: GraphNode, g: GraphNode) -> List[Optional[GraphNode]
         raise NotImplementedError("exact VJP of a reduce with a fused map: differentiate before fusion")
     if op.kind == "map_reduce":
         return _elementwise_vjp_exact(node, g, op.map)
-    return compute_vjp(node, g)                          # unfold / scatter / scan / matmul
+    if op.kind == "unfold":
+        return [_unfold_adjoint(g, op)]
+    return compute_vjp(node, g)                          # scatter / scan / matmul
 
 
 def _elementwise_vjp_exact(node, g, m) -> List[Optional[GraphNode]]:
@@ -392,6 +394,47 @@ def _elementwise_vjp_exact(node, g, m) -> List[Optional[GraphNode]]:
         z = _zeros_like(g)
         return [None, _select_dense(ins[0], g, z), _select_dense(ins[0], z, g)]
     return _elementwise_vjp(node, g, m)                  # add, mul, neg, recip, sqrt, ln, sin, ...
+
+
+def _unfold_adjoint(g: GraphNode, op) -> GraphNode:
+    """Adjoint of a sliding-window unfold as a gather (no scatter, no atomics): every input
+    position sums the window slots that read it.  g: [preserved..., out_0.., k_0..].
+
+    Windows that tile the axis (stride == size, dilation 1) are a pure re-indexing:
+    interleave (out_i, k_i) and merge.  Unit-stride windows are a sum over the window
+    offsets of g's slice at that offset, zero-padded back to the input extent."""
+    in_shape = [int(e.evaluate()) for e in op.input_shape]
+    sizes = [int(e.evaluate()) for e in op.sizes]
+    strides = [int(e.evaluate()) for e in op.strides]
+    dils = [int(e.evaluate()) for e in op.dilations]
+    axes, nu = list(op.axes), len(op.axes)
+    npres = len(in_shape) - nu
+    if axes != list(range(npres, npres + nu)):
+        raise NotImplementedError("exact unfold adjoint: windowed axes must be the trailing ones")
+    outs = [int(e.evaluate()) for e in g.shape()[npres:npres + nu]]
+    if all(s == k and d == 1 for s, k, d in zip(strides, sizes, dils)):
+        perm = list(range(npres))
+        for i in range(nu):
+            perm += [npres + i, npres + nu + i]
+        merged = g.permute(perm).contiguous().reshape(
+            in_shape[:npres] + [o * k for o, k in zip(outs, sizes)])
+        padding = [(0, 0)] * npres + [(0, n - o * k) for n, o, k in zip(in_shape[npres:], outs, sizes)]
+        return merged.pad(padding, "zero") if any(a for _, a in padding) else merged
+    if all(s == 1 for s in strides):
+        import itertools
+        total = None
+        for ks in itertools.product(*[range(k) for k in sizes]):
+            term = g
+            for i in range(nu - 1, -1, -1):                      # drop the window axes, last first
+                term = term.slice_axis(npres + nu + i, ks[i], 1).squeeze(npres + nu + i)
+            padding = [(0, 0)] * npres
+            for i in range(nu):
+                before = ks[i] * dils[i]
+                padding.append((before, in_shape[npres + i] - outs[i] - before))
+            term = term.pad(padding, "zero")
+            total = term if total is None else total + term
+        return total
+    raise NotImplementedError("exact unfold adjoint: strided overlapping windows")
 
 
 def _select_dense(cond: GraphNode, a: GraphNode, b: GraphNode) -> GraphNode:

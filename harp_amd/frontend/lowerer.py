@@ -409,18 +409,27 @@ def unshare_views(roots: Sequence[GraphNode]) -> List[GraphNode]:
     one consumer and are inlined.  Not in the reference: there a view with several consumers
     is materialised contiguously by a copy kernel but still indexed through its own
     (possibly strided) view by the readers (`lower.rs:209-224` vs `:452-455`), which is only
-    right for contiguous views.  Used by the exact mode."""
+    right for contiguous views.  Used by the exact mode.
+
+    Unfold nodes become plain views here as well: the reference materialises an unfold into
+    a contiguous window buffer and then lets its readers index that buffer through the
+    unfold's own (input-space) view (`lower.rs:344-348` vs `:221-224`), which reads the
+    wrong elements; as an inlined view the windows are read straight from the input."""
     memo: Dict[int, GraphNode] = {}
     order = topological_sort(roots)
 
+    def is_view(n: GraphNode) -> bool:
+        return n.op.kind in ("view", "unfold") and not n.is_external() and bool(n.src)
+
     def fresh(n: GraphNode) -> GraphNode:
         # a private copy of a view chain, down to the first node that computes something
-        if n.op.kind == "view" and not n.is_external() and n.src:
-            return GraphNode([fresh(n.src[0])], n.view, n.op, n.dtype, None, n.name, n.hint)
+        if is_view(n):
+            op = n.op if n.op.kind == "view" else GraphOp("view", view=n.src[0].view)
+            return GraphNode([fresh(n.src[0])], n.view, op, n.dtype, None, n.name, n.hint)
         return memo[id(n)]
 
     for n in order:
-        if n.op.kind == "view" and not n.is_external() and n.src:
+        if is_view(n):
             continue                      # rebuilt on demand by fresh()
         new_src = [fresh(s) for s in n.src]
         changed = any(a is not b for a, b in zip(new_src, n.src))

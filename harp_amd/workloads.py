@@ -121,6 +121,52 @@ def config4_graph(x: Tensor, t: Tensor, *params: Tensor, lr: float = 1e-3):
     return new_params + [loss]
 
 
+# ---------------------------------------------------------------------------
+# config 5: MNIST-shaped CNN, forward + backward (exact gradients)
+# ---------------------------------------------------------------------------
+
+def cnn_sizes(full: bool = True):
+    """(batch, image side, conv1 channels, conv2 channels, hidden width, classes)."""
+    return (256, 28, 32, 64, 128, 10) if full else (4, 8, 4, 8, 16, 10)
+
+
+def config5_inputs(batch=256, side=28, c1=32, c2=64, hidden=128, classes=10, seed: int = 1238):
+    """images ~ U(0,1) [batch,1,side,side]; one-hot of uniform labels; conv and fc parameters
+    ~ U(+-1/sqrt(fan_in)).  Returns [x, one_hot, w1, b1, w2, b2, w3, b3, w4, b4]."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 1, (batch, 1, side, side)).astype(np.float32)
+    labels = rng.integers(0, classes, batch)
+    one_hot = np.zeros((batch, classes), np.float32)
+    one_hot[np.arange(batch), labels] = 1.0
+    flat = c2 * (side // 4) ** 2
+    params = []
+    for shape, fan_in in (((c1, 1, 3, 3), 9), ((c2, c1, 3, 3), 9 * c1),
+                          ((hidden, flat), flat), ((classes, hidden), hidden)):
+        k = 1.0 / np.sqrt(fan_in)
+        params.append(rng.uniform(-k, k, shape).astype(np.float32))
+        params.append(rng.uniform(-k, k, (shape[0],)).astype(np.float32))
+    return [x, one_hot] + params
+
+
+def config5_graph(x: Tensor, one_hot: Tensor, *params: Tensor):
+    """conv3x3(pad 1)+relu+maxpool2 twice, fc+relu, fc, cross-entropy; exact backward.
+    Returns [gradient of every parameter..., loss]."""
+    from .frontend import exact_mode
+    w1, b1, w2, b2, w3, b3, w4, b4 = params
+    with exact_mode():
+        h = nn.max_pool2d(nn.relu(nn.conv2d(x, w1, b1, padding=(1, 1))), (2, 2))
+        h = nn.max_pool2d(nn.relu(nn.conv2d(h, w2, b2, padding=(1, 1))), (2, 2))
+        n = h.shape()[0]
+        h = h.reshape([n, h.numel() // n])
+        h = nn.relu(nn.linear(h, w3, b3))
+        logits = nn.linear(h, w4, b4)
+        loss = nn.cross_entropy_loss(logits, one_hot, exact=True)
+        loss.backward_with_params(list(params))
+        # a gradient may come out as a view (the weight's is a permute); roots must own buffers
+        grads = [p.grad().contiguous() for p in params]
+    return grads + [loss]
+
+
 def lower_multi(tensors_in, roots):
     """Lowers several roots into one Program with a buffer table.  Returns (program AST,
     input buffer names in the order of `tensors_in`, output buffer name per root, constant

@@ -304,3 +304,48 @@ def test_config4_mlp_training_step(frontend, hip, batch, dims, fuse):
     assert abs(float(got[-1][0]) - loss) <= 1e-4 * abs(loss)
     for p, gr, g in zip(ps, grads, got[:-1]):
         assert np.allclose(g.reshape(p.shape), p - 1e-3 * gr, rtol=1e-4, atol=1e-6)
+
+
+def _cnn_step_on(fe, kind, arrays, fuse=True):
+    import os
+    from harp_amd import workloads as wl
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    fe.set_device_str(kind)
+    old = os.environ.get("ECLAT_HIP_FUSE")
+    os.environ["ECLAT_HIP_FUSE"] = "1" if fuse else "0"
+    try:
+        with fe.exact_mode():
+            ts = []
+            for a in arrays:
+                t = fe.Tensor.input(list(a.shape))
+                t.set_data(a)
+                ts.append(t)
+            roots = wl.config5_graph(*ts)
+            fe.realize_many(roots)
+            return [r.to_numpy() for r in roots]
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+        if old is None:
+            os.environ.pop("ECLAT_HIP_FUSE", None)
+        else:
+            os.environ["ECLAT_HIP_FUSE"] = old
+
+
+@pytest.mark.parametrize("sizes", [(4, 8, 4, 8, 16, 10), (8, 28, 32, 64, 128, 10)])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_config5_cnn_training_step(frontend, hip, sizes, fuse):
+    """BASELINE config 5 (second case: the real channel/image sizes at batch 8): every
+    parameter gradient and the loss match the C oracle running the same exact-mode graph,
+    and a float64 numpy CNN."""
+    from harp_amd import workloads as wl
+    from cnn_reference import cnn_step
+    arrays = wl.config5_inputs(*sizes, seed=77)
+    ref = _cnn_step_on(frontend, "c", arrays)
+    got = _cnn_step_on(frontend, "hip", arrays, fuse)
+    loss, grads = cnn_step(arrays[0], arrays[1], arrays[2:])
+    assert abs(float(got[-1][0]) - float(ref[-1][0])) <= 1e-5 * abs(float(ref[-1][0]))
+    assert abs(float(got[-1][0]) - loss) <= 1e-5 * abs(loss)
+    for g, r, n in zip(got[:-1], ref[:-1], grads):
+        scale = max(float(np.abs(r).max()), 1e-6)
+        assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
+        assert np.allclose(g.reshape(n.shape), n, rtol=1e-3, atol=1e-5 * scale)

@@ -264,3 +264,42 @@ def test_exact_gradients_match_calculus(frontend):
     p /= p.sum(1, keepdims=True)
     ref = p + p * (m - (p * m).sum(1, keepdims=True))
     assert np.allclose(gm, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_exact_unfold_views_and_cnn_step(frontend):
+    """Exact mode: unfold windows are read from the input (not through the reference's
+    double-applied view), and the config-5 CNN step built from conv2d / max_pool2d /
+    cross_entropy_loss plus exact VJPs matches a float64 numpy CNN."""
+    from harp_amd import workloads as wl
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    from cnn_reference import cnn_step
+    frontend.set_device_str("c")
+    x = np.arange(2 * 2 * 4 * 4, dtype=np.float32).reshape(2, 2, 4, 4)
+    win = np.empty((2, 2, 2, 2, 3, 3), np.float32)
+    for i in range(3):
+        for j in range(3):
+            win[..., i, j] = x[:, :, i:i + 2, j:j + 2]
+    with frontend.exact_mode():
+        got = realize_on(frontend, "c", lambda t: t.unfold([2, 3], [3, 3], [1, 1], [1, 1]).contiguous(), [x])
+    assert np.array_equal(got.reshape(win.shape), win)
+    # as written the reader indexes the materialised windows through the unfold view again
+    got_ref = realize_on(frontend, "c", lambda t: t.unfold([2, 3], [3, 3], [1, 1], [1, 1]).contiguous(), [x])
+    assert not np.array_equal(got_ref.reshape(win.shape), win)
+
+    arrays = wl.config5_inputs(*wl.cnn_sizes(False))
+    try:
+        with frontend.exact_mode():
+            ts = []
+            for a in arrays:
+                t = frontend.Tensor.input(list(a.shape))
+                t.set_data(a)
+                ts.append(t)
+            roots = wl.config5_graph(*ts)
+            frontend.realize_many(roots)
+            got = [r.to_numpy() for r in roots]
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+    loss, grads = cnn_step(arrays[0], arrays[1], arrays[2:])
+    assert abs(float(got[-1][0]) - loss) <= 1e-6 * abs(loss)
+    for g, r in zip(got[:-1], grads):
+        assert np.allclose(g.reshape(r.shape), r, rtol=1e-4, atol=1e-7)
