@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | copy (default: all but copy)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy (default: all but copy)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -226,6 +226,32 @@ def main():
             mlp["loss"] = got_loss
         del sets
 
+    # ---- config 5: MNIST-shaped CNN, batch 256, forward + backward -------------------------
+    cnn = None
+    if want("cnn"):
+        sizes = wl.cnn_sizes(True)
+        arrays = wl.config5_inputs(*sizes)
+        from harp_amd.frontend import Tensor
+        ts = [Tensor.input(list(a.shape)) for a in arrays]
+        roots = wl.config5_graph(*ts)
+        prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
+        prog = hb.HipProgram(dev, prog_ast, options)
+        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 1)
+        k = max(3, min(args.steps, 50))
+        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 5))
+        cnn = {"ms": ms, "steps": k, "flops": sum(l["flops"] for l in prog.launches),
+               "algo_bytes": sum(l["algo_bytes"] for l in prog.launches),
+               "lowered_kernels": len(plain.args), "launches": len(prog.launches),
+               "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
+        log(f"[bench] cnn step (batch {sizes[0]}): {ms:.3f} ms/step -> {sizes[0] / ms * 1e3:.0f} images/s; "
+            f"{cnn['lowered_kernels']} kernels -> {cnn['launches']} launches ({cnn['gemm_launches']} MFMA)")
+        if not args.no_check:
+            named = sets[0][1]
+            got_loss = float(named[outs[-1]].read_array(np.float32, (1,))[0])
+            assert np.isfinite(got_loss) and abs(got_loss - np.log(10.0)) < 0.5, f"cnn loss {got_loss}"
+            cnn["loss"] = got_loss
+        del sets
+
     # ---- CPU baseline: the oracle's unfused C kernels on host cores -------------------------
     cpu = None
     if not args.no_cpu_baseline and softmax is not None:
@@ -301,6 +327,14 @@ def main():
             "algorithmic_bytes": mlp["algo_bytes"], "lowered_kernels": mlp["lowered_kernels"],
             "launches": mlp["launches"], "gemm_launches": mlp["gemm_launches"], "loss": mlp.get("loss"),
             "workload": "MLP 1024-4096-4096-1024, batch 8192: forward, MSE, exact backward, SGD update, one Program"}
+    if cnn:
+        result_extra["config5_cnn_step"] = {
+            "value": round(256 / cnn["ms"] * 1e3, 1), "unit": "images/s", "ms_per_step": round(cnn["ms"], 4),
+            "steps": cnn["steps"], "algorithmic_bytes": cnn["algo_bytes"],
+            "lowered_kernels": cnn["lowered_kernels"], "launches": cnn["launches"],
+            "gemm_launches": cnn["gemm_launches"], "loss": cnn.get("loss"),
+            "workload": "CNN 1x28x28: conv3x3(32)+relu+pool, conv3x3(64)+relu+pool, fc 3136-128-10, "
+                        "cross-entropy; batch 256 forward + exact backward, one Program"}
     result_extra["device"] = {"name": props["name"], "arch": props["arch"],
                               "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
     out["extra"] = result_extra
