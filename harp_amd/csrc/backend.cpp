@@ -299,6 +299,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_bk") o.gemm_bk = as_int();
     else if (k == "gemm_wm") o.gemm_wm = as_int();
     else if (k == "gemm_wn") o.gemm_wn = as_int();
+    else if (k == "gemm_split_k") o.gemm_split_k = as_int();
     else if (k == "nontemporal") o.nontemporal = as_int();
     else throw Error("unknown option '" + k + "'");
   }

@@ -643,8 +643,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     const NestKernel& k0 = *nests[i];
     // contraction (matmul-shaped reduce) -> MFMA schedule
     if (k0.rkind == ReduceKind::Sum && opt.gemm) {
-      if (auto ls = try_emit_gemm(k0, opt)) {
-        plan.launches.push_back(*ls);
+      auto gl = try_emit_gemm(k0, opt, &plan.buffers);
+      if (!gl.empty()) {
+        for (auto& ls : gl) plan.launches.push_back(std::move(ls));
         ++i;
         continue;
       }

@@ -1,5 +1,6 @@
 #include "gemm.hpp"
 
+#include <algorithm>
 #include <sstream>
 
 namespace eh {
@@ -16,41 +17,77 @@ struct Tile {
   int bm, bn, bk, wm, wn;
 };
 
-// Largest first.  Each uses 256 threads (four waves).
-const Tile kTiles[] = {{128, 128, 16, 64, 64}, {64, 64, 16, 32, 32}};
+// Each uses 256 threads (four waves).
+const Tile kBig = {128, 128, 16, 64, 64}, kSmall = {64, 64, 16, 32, 32};
 
-bool pick_tile(const GemmShape& s, const GenOptions& opt, Tile* out) {
-  auto fits = [&](const Tile& t) {
-    if (s.M % t.bm || s.N % t.bn || s.K % t.bk) return false;
-    if (t.bm % t.wm || t.bn % t.wn || t.wm % 32 || t.wn % 32) return false;
-    int nt = (t.bm / t.wm) * (t.bn / t.wn) * 64;
-    if (nt > 1024 || (t.bm * t.bk) % (4 * nt) || (t.bn * t.bk) % (4 * nt)) return false;
-    size_t lds = 2ull * static_cast<size_t>(t.bk) * (t.bm + 4 + t.bn + 4) * 4;
-    return lds <= 160 * 1024;
-  };
-  if (opt.gemm_bm > 0) {
-    Tile t{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
-    if (fits(t)) { *out = t; return true; }
-    return false;
-  }
-  for (const auto& t : kTiles)
-    if (fits(t)) {
-      // prefer the small tile when the big one cannot fill the chip
-      if (t.bm == 128 && (s.M / 128) * (s.N / 128) * s.batch < 256 && fits(kTiles[1])) continue;
-      *out = t;
-      return true;
-    }
-  return false;
+bool tile_valid(const Tile& t) {
+  if (t.bm <= 0 || t.bn <= 0 || t.bk <= 0 || t.wm <= 0 || t.wn <= 0) return false;
+  if (t.bm % t.wm || t.bn % t.wn || t.wm % 32 || t.wn % 32 || t.bk % 4) return false;
+  int nt = (t.bm / t.wm) * (t.bn / t.wn) * 64;
+  if (nt > 1024 || (t.bm * t.bk) % (4 * nt) || (t.bn * t.bk) % (4 * nt)) return false;
+  size_t lds = 2ull * static_cast<size_t>(t.bk) * (t.bm + 4 + t.bn + 4) * 4;
+  return lds <= 160 * 1024;
 }
 
-// 128-bit global loads need every row start on a 4-float boundary.
-bool vector_ok(const GemmShape& s) {
-  bool a_k = s.a_k == 1, a_m = s.a_m == 1;
-  bool b_n = s.b_n == 1, b_k = s.b_k == 1;
-  if (!(a_k || a_m) || !(b_n || b_k)) return false;
-  int64_t lda = a_k ? s.a_m : s.a_k, ldb = b_n ? s.b_k : s.b_n;
-  if (lda % 4 || ldb % 4 || s.a_off % 4 || s.b_off % 4 || s.a_b % 4 || s.b_b % 4) return false;
-  return s.c_n == 1;
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+struct Choice {
+  Tile tile;
+  int split_k = 1;
+};
+
+// Tile and K split.  The big tile halves LDS traffic per flop but needs enough tiles to
+// put several workgroups on each of the 256 CUs; when even the small tile leaves CUs
+// idle and K is long, K is split over blockIdx.y.
+bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
+  if (s.K < 16 || s.M < 2 || s.N < 2) return false;
+  Choice c;
+  if (opt.gemm_bm > 0) {
+    c.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
+    if (!tile_valid(c.tile)) return false;
+  } else {
+    int64_t big = ceil_div(s.M, 128) * ceil_div(s.N, 128) * s.batch;
+    bool waste_ok = s.M >= 96 && s.N >= 96;
+    c.tile = (big >= 512 && waste_ok) ? kBig : kSmall;
+  }
+  int64_t tiles = ceil_div(s.M, c.tile.bm) * ceil_div(s.N, c.tile.bn) * s.batch;
+  int64_t ksteps = ceil_div(s.K, c.tile.bk);
+  if (opt.gemm_split_k > 0) {
+    c.split_k = static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps));
+  } else if (opt.gemm_split_k < 0 && tiles < 256 && ksteps >= 32) {
+    int64_t want = ceil_div(1024, tiles);
+    c.split_k = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(want, ksteps / 8)));
+  }
+  *out = c;
+  return true;
+}
+
+// Whether an operand can be read with aligned 128-bit loads along its unit-stride axis.
+bool vec_ok(int64_t unit_extent, int64_t s_unit, int64_t s_other, int64_t off, int64_t bs) {
+  return s_unit == 1 && unit_extent % 4 == 0 && s_other % 4 == 0 && off % 4 == 0 && bs % 4 == 0;
+}
+
+struct VarUse {
+  std::string var;
+  int64_t extent;
+};
+
+// Merges neighbouring loop variables (outer, inner) that every given affine index walks as
+// one longer axis: stride(outer) == extent(inner) * stride(inner).
+void collapse(std::vector<VarUse>* vars, const std::vector<Affine*>& affs) {
+  for (size_t i = 0; i + 1 < vars->size();) {
+    const VarUse &o = (*vars)[i], &in = (*vars)[i + 1];
+    bool ok = true;
+    for (const Affine* a : affs) ok = ok && a->of(o.var) == in.extent * a->of(in.var);
+    if (!ok) {
+      ++i;
+      continue;
+    }
+    // the merged axis keeps the inner variable's name and stride
+    for (Affine* a : affs) a->coef.erase(o.var);
+    (*vars)[i + 1].extent *= o.extent;
+    vars->erase(vars->begin() + static_cast<long>(i));
+  }
 }
 
 }  // namespace
@@ -66,41 +103,47 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
   auto aa = affine_of(*la->args[1]);
   auto ab = affine_of(*lb->args[1]);
   if (!aa || !ab || !k.out_aff) return std::nullopt;
+  Affine ac = *k.out_aff;
   const std::string& kv = k.rloop.var;
   if (aa->of(kv) <= 0 || ab->of(kv) <= 0 || k.rloop.extent < 2) return std::nullopt;
-  std::string mvar, nvar, bvar;
-  int64_t M = 0, N = 0, batch = 1;
+  // output loops by which operands they index: A only -> rows, B only -> columns, both -> batch
+  std::vector<VarUse> mv, nv, bv;
   for (const auto& l : k.loops) {
     if (l.extent == 1) continue;
     bool in_a = aa->of(l.var) != 0, in_b = ab->of(l.var) != 0;
-    if (in_a && !in_b) {
-      if (!mvar.empty()) return std::nullopt;
-      mvar = l.var;
-      M = l.extent;
-    } else if (in_b && !in_a) {
-      if (!nvar.empty()) return std::nullopt;
-      nvar = l.var;
-      N = l.extent;
-    } else if (in_a && in_b) {
-      if (!bvar.empty()) return std::nullopt;
-      bvar = l.var;
-      batch = l.extent;
-    } else {
-      return std::nullopt;
-    }
+    if (ac.of(l.var) <= 0) return std::nullopt;
+    if (in_a && aa->of(l.var) < 0) return std::nullopt;
+    if (in_b && ab->of(l.var) < 0) return std::nullopt;
+    if (in_a && !in_b) mv.push_back({l.var, l.extent});
+    else if (in_b && !in_a) nv.push_back({l.var, l.extent});
+    else if (in_a && in_b) bv.push_back({l.var, l.extent});
+    else return std::nullopt;
   }
-  if (mvar.empty() || nvar.empty()) return std::nullopt;
-  // operands may come in either order; make `A` the one indexed by the output's row variable
+  collapse(&mv, {&*aa, &ac});
+  collapse(&nv, {&*ab, &ac});
+  collapse(&bv, {&*aa, &*ab, &ac});
+  // a leftover outer row (column) axis can ride on the batch axis: the other operand simply
+  // does not move with it
+  if (bv.empty() && mv.size() == 2) {
+    bv.push_back(mv[0]);
+    mv.erase(mv.begin());
+  } else if (bv.empty() && nv.size() == 2) {
+    bv.push_back(nv[0]);
+    nv.erase(nv.begin());
+  }
+  if (mv.size() != 1 || nv.size() != 1 || bv.size() > 1) return std::nullopt;
+  const std::string &mvar = mv[0].var, &nvar = nv[0].var;
   GemmShape s;
-  s.M = M; s.N = N; s.K = k.rloop.extent; s.batch = batch;
+  s.M = mv[0].extent; s.N = nv[0].extent; s.K = k.rloop.extent;
   s.a_buf = la->args[0]->name; s.b_buf = lb->args[0]->name; s.c_buf = k.out_buf;
   s.a_m = aa->of(mvar); s.a_k = aa->of(kv); s.a_off = aa->c;
   s.b_n = ab->of(nvar); s.b_k = ab->of(kv); s.b_off = ab->c;
-  s.c_m = k.out_aff->of(mvar); s.c_n = k.out_aff->of(nvar); s.c_off = k.out_aff->c;
-  if (!bvar.empty()) {
-    s.a_b = aa->of(bvar); s.b_b = ab->of(bvar); s.c_b = k.out_aff->of(bvar);
+  s.c_m = ac.of(mvar); s.c_n = ac.of(nvar); s.c_off = ac.c;
+  if (!bv.empty()) {
+    s.batch = bv[0].extent;
+    s.a_b = aa->of(bv[0].var); s.b_b = ab->of(bv[0].var); s.c_b = ac.of(bv[0].var);
   }
-  if (s.a_m <= 0 || s.b_n <= 0 || s.c_m <= 0 || s.c_n <= 0) return std::nullopt;
+  if (s.a_off < 0 || s.b_off < 0 || s.c_off < 0) return std::nullopt;
   if (s.c_n != 1 && s.c_m == 1) {
     // C is column-major: compute C^T = B^T A^T instead, which is row-major
     GemmShape t = s;
@@ -116,19 +159,26 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
 
 bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
   auto s = match_gemm(k);
-  Tile t;
-  return s && vector_ok(*s) && pick_tile(*s, opt, &t);
+  Choice c;
+  return s && choose(*s, opt, &c);
 }
 
-std::optional<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt) {
+std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers) {
   auto s = match_gemm(k);
-  Tile t;
-  if (!s || !vector_ok(*s) || !pick_tile(*s, opt, &t)) return std::nullopt;
-  const bool a_kc = s->a_k == 1, b_nc = s->b_n == 1;
-  LaunchSpec ls;
-  ls.entry = "ehk_" + k.name;
+  Choice ch;
+  if (!s || !choose(*s, opt, &ch)) return {};
+  const Tile& t = ch.tile;
+  // each thread fetches four elements along the operand's faster axis
+  const bool a_kc = s->a_k <= s->a_m, b_nc = s->b_n <= s->b_k;
+  const bool a_vec = a_kc ? vec_ok(s->K, s->a_k, s->a_m, s->a_off, s->a_b) : vec_ok(s->M, s->a_m, s->a_k, s->a_off, s->a_b);
+  const bool b_vec = b_nc ? vec_ok(s->N, s->b_n, s->b_k, s->b_off, s->b_b) : vec_ok(s->K, s->b_k, s->b_n, s->b_off, s->b_b);
+  const int S = ch.split_k;
+  std::vector<LaunchSpec> out(S > 1 ? 2 : 1);
+  LaunchSpec& ls = out[0];
+  ls.entry = "ehk_" + k.name + (S > 1 ? "_part" : "");
   ls.kernels = {k.name};
   const int nt = (t.bm / t.wm) * (t.bn / t.wn) * 64;
+  const std::string scratch = "eh_part_" + k.name;
   std::ostringstream os;
   os << "// generated for gfx950 by eclat backend-hip: MFMA contraction\n";
   os << "#define EH_ENTRY " << ls.entry << "\n";
@@ -137,30 +187,67 @@ std::optional<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& o
   os << "#define EH_BM " << t.bm << "\n#define EH_BN " << t.bn << "\n#define EH_BK " << t.bk << "\n#define EH_WM "
      << t.wm << "\n#define EH_WN " << t.wn << "\n";
   os << "#define EH_A_KCONTIG " << (a_kc ? 1 : 0) << "\n#define EH_B_NCONTIG " << (b_nc ? 1 : 0) << "\n";
-  os << "#define EH_LDA " << (a_kc ? s->a_m : s->a_k) << "LL\n#define EH_LDB " << (b_nc ? s->b_k : s->b_n)
-     << "LL\n#define EH_LDC " << s->c_m << "LL\n";
+  os << "#define EH_A_VEC " << (a_vec ? 1 : 0) << "\n#define EH_B_VEC " << (b_vec ? 1 : 0) << "\n";
+  os << "#define EH_A_SM " << s->a_m << "LL\n#define EH_A_SK " << s->a_k << "LL\n";
+  os << "#define EH_B_SK " << s->b_k << "LL\n#define EH_B_SN " << s->b_n << "LL\n";
+  os << "#define EH_C_SM " << s->c_m << "LL\n#define EH_C_SN " << s->c_n << "LL\n";
   os << "#define EH_A_OFF " << s->a_off << "LL\n#define EH_B_OFF " << s->b_off << "LL\n#define EH_C_OFF " << s->c_off
      << "LL\n";
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
+  os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
   os << kGemmSource;
   ls.source = os.str();
+  const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;
   ls.schedule = "mfma32x32x2(tile=" + std::to_string(t.bm) + "x" + std::to_string(t.bn) + "x" + std::to_string(t.bk) +
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
-                (b_nc ? ",B:n" : ",B:k") + ")";
-  ls.grid[0] = static_cast<unsigned>((s->M / t.bm) * (s->N / t.bn));
+                (a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") + (b_vec ? "" : "/scalar") +
+                (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") + ")";
+  ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
+  ls.grid[1] = static_cast<unsigned>(S);
   ls.grid[2] = static_cast<unsigned>(s->batch);
   ls.block[0] = static_cast<unsigned>(nt);
-  ls.arg_bufs = {s->a_buf, s->b_buf, s->c_buf};
+  const size_t c_elems =
+      static_cast<size_t>(s->c_off + (s->M - 1) * s->c_m + (s->N - 1) * s->c_n + (s->batch - 1) * s->c_b + 1);
+  const size_t part_elems = static_cast<size_t>(S) * static_cast<size_t>(s->batch * s->M * s->N);
+  ls.arg_bufs = {s->a_buf, s->b_buf, S > 1 ? scratch : s->c_buf};
   ls.arg_min_bytes = {
       4 * static_cast<size_t>(s->a_off + (s->M - 1) * s->a_m + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
       4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1),
-      4 * static_cast<size_t>(s->c_off + (s->M - 1) * s->c_m + (s->N - 1) * s->c_n + (s->batch - 1) * s->c_b + 1)};
+      4 * (S > 1 ? part_elems : c_elems)};
   ls.flops = 2.0 * static_cast<double>(s->M) * static_cast<double>(s->N) * static_cast<double>(s->K) *
              static_cast<double>(s->batch);
   ls.algo_bytes = 4.0 * static_cast<double>(s->batch) *
                   (static_cast<double>(s->M) * s->K + static_cast<double>(s->K) * s->N + static_cast<double>(s->M) * s->N);
-  return ls;
+  if (S > 1) {
+    BufferInfo sb;
+    sb.name = scratch;
+    sb.dtype = k.out_dtype;
+    sb.shape = {S, s->batch, s->M, s->N};
+    sb.role = "temp";
+    buffers->push_back(sb);
+    // second launch: C[b,m,n] = sum over splits, in split order (deterministic)
+    LaunchSpec& fin = out[1];
+    fin.entry = "ehk_" + k.name;
+    fin.kernels = {k.name};
+    fin.schedule = "split-k-final(chunks=" + std::to_string(S) + ")";
+    const int64_t total = s->batch * s->M * s->N;
+    fin.grid[0] = static_cast<unsigned>(ceil_div(total, 256));
+    fin.block[0] = 256;
+    fin.arg_bufs = {scratch, s->c_buf};
+    fin.arg_min_bytes = {4 * part_elems, 4 * c_elems};
+    std::ostringstream fs;
+    fs << "// generated for gfx950 by eclat backend-hip: sum of split-K partial tiles\n";
+    fs << "extern \"C\" __global__ void __launch_bounds__(256) " << fin.entry
+       << "(const float* __restrict__ P, float* __restrict__ C) {\n";
+    fs << "  const long long o = (long long)blockIdx.x * 256 + threadIdx.x;\n  if (o >= " << total << "LL) return;\n";
+    fs << "  float acc = 0.0f;\n  for (int s = 0; s < " << S << "; ++s) acc += P[(long long)s * " << total << "LL + o];\n";
+    fs << "  const long long n = o % " << s->N << "LL, m = (o / " << s->N << "LL) % " << s->M << "LL, b = o / "
+       << (s->M * s->N) << "LL;\n";
+    fs << "  C[" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n << "LL] = acc;\n}\n";
+    fin.source = fs.str();
+  }
+  return out;
 }
 
 }  // namespace eh

@@ -24,11 +24,12 @@ struct GemmShape {
 // Recognises the contraction and returns its strides; nullopt otherwise.
 std::optional<GemmShape> match_gemm(const NestKernel& k);
 
-// True when match_gemm succeeds and the sizes fit one of the tile configurations.
+// True when match_gemm succeeds and the contraction is large enough for the MFMA schedule.
 bool gemm_shaped(const NestKernel& k, const GenOptions& opt);
 
-// HIP source + dispatch for the kernel, or nullopt when it is not a contraction the MFMA
-// schedule covers (the caller then falls back to another schedule).
-std::optional<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt);
+// HIP source + dispatch for the kernel; empty when it is not a contraction the MFMA schedule
+// covers (the caller then falls back to another schedule).  One launch, or two when K is
+// split: partial tiles into a scratch buffer appended to `buffers`, then their sum.
+std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers);
 
 }  // namespace eh

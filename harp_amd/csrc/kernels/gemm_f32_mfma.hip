@@ -9,6 +9,9 @@
 // Two LDS buffers: the loads of tile t+1 are in flight while tile t is multiplied, one
 // barrier per step.  Workgroup ids are remapped so that each XCD (ids congruent mod 8) works
 // on a compact block of tiles and shares A/B panels through its own L2.
+// Sizes need not be multiples of the tile (edge tiles load zeros and skip stores), operands
+// that cannot be read as aligned 128-bit vectors are read element by element, and a long K
+// with few output tiles can be split over blockIdx.y into partial sums.
 //
 // The generator defines the EH_* macros; the defaults below make the file compile on its own.
 #ifndef __HIPCC_RTC__
@@ -23,20 +26,26 @@
 #define EH_BATCH 1
 #define EH_BM 128
 #define EH_BN 128
-#define EH_BK 32
+#define EH_BK 16
 #define EH_WM 64
 #define EH_WN 64
 #define EH_A_KCONTIG 1
 #define EH_B_NCONTIG 1
-#define EH_LDA 4096
-#define EH_LDB 4096
-#define EH_LDC 4096
+#define EH_A_VEC 1
+#define EH_B_VEC 1
+#define EH_A_SM 4096LL
+#define EH_A_SK 1LL
+#define EH_B_SK 4096LL
+#define EH_B_SN 1LL
+#define EH_C_SM 4096LL
+#define EH_C_SN 1LL
 #define EH_A_OFF 0
 #define EH_B_OFF 0
 #define EH_C_OFF 0
 #define EH_A_BS 0
 #define EH_B_BS 0
 #define EH_C_BS 0
+#define EH_SPLITK 1
 #define EH_GROUP_M 8
 #endif
 
@@ -47,12 +56,39 @@ namespace {
 constexpr int BM = EH_BM, BN = EH_BN, BK = EH_BK, WM = EH_WM, WN = EH_WN;
 constexpr int NWM = BM / WM, NWN = BN / WN, NT = NWM * NWN * 64;
 constexpr int AS = BM + 4, BS = BN + 4;            // padded LDS row lengths
-constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 128-bit loads per thread per tile
+constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 4-element loads per thread per tile
 constexpr int IB = WM / 32, JB = WN / 32;
-constexpr int TM = EH_M / BM, TN = EH_N / BN, NTILES = TM * TN, KT = EH_K / BK;
-static_assert(EH_M % BM == 0 && EH_N % BN == 0 && EH_K % BK == 0, "sizes must be multiples of the tile");
+constexpr long long M = EH_M, N = EH_N, K = EH_K;
+constexpr int TM = (EH_M + BM - 1) / BM, TN = (EH_N + BN - 1) / BN, NTILES = TM * TN;
+constexpr int KT_ALL = (EH_K + BK - 1) / BK;
+constexpr int KT = (KT_ALL + EH_SPLITK - 1) / EH_SPLITK;      // k-steps per split
+// Ragged sizes: rows/columns past the end are loaded as zero and never stored.
+constexpr bool EDGE_M = EH_M % BM != 0, EDGE_N = EH_N % BN != 0;
+constexpr bool EDGE_K = EH_K % BK != 0 || KT_ALL % EH_SPLITK != 0;
 static_assert(BM * BK % (4 * NT) == 0 && BN * BK % (4 * NT) == 0 && AV >= 1 && BV >= 1, "tile does not split over the threads");
-static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 2 == 0, "wave tile must be built from 32x32x2 MFMAs");
+static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 4 == 0, "wave tile must be built from 32x32x2 MFMAs");
+// 128-bit loads need the four elements to be in range together
+static_assert(!EH_A_VEC || (EH_A_KCONTIG ? EH_K % 4 == 0 : EH_M % 4 == 0), "A cannot be loaded as vectors");
+static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B cannot be loaded as vectors");
+
+// Four elements of an operand starting at (r, k) and running along its fast axis; elements
+// outside [0,R) x [0,kend) read as zero.  `along_k` says which axis the four run along.
+template <bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
+__device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long r, long long k,
+                                              long long R, long long kend) {
+  eh_f4v v = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (VEC) {
+    const bool ok = (!EDGE_R || r < R) && (!EDGE_K || k < kend);
+    if (ok) v = *reinterpret_cast<const eh_f4v*>(p + r * SR + k * SK);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const long long rr = ALONG_K ? r : r + e, kk = ALONG_K ? k + e : k;
+      if (rr < R && kk < kend) v[e] = p[rr * SR + kk * SK];
+    }
+  }
+  return v;
+}
 }  // namespace
 
 extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restrict__ A,
@@ -81,21 +117,31 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
   const long long bz = blockIdx.z;
   const float* Ab = A + EH_A_OFF + bz * EH_A_BS;
   const float* Bb = B + EH_B_OFF + bz * EH_B_BS;
+#if EH_SPLITK > 1
+  // partial sums go to a dense [split][batch][M][N] scratch; a second launch adds them up
+  const long long kbeg = (long long)blockIdx.y * KT * BK;
+  const long long kend = (kbeg + (long long)KT * BK) < K ? (kbeg + (long long)KT * BK) : K;
+  float* Cb = C + ((long long)blockIdx.y * EH_BATCH + bz) * (M * N);
+  constexpr long long CSM = N, CSN = 1;
+#else
+  const long long kbeg = 0, kend = K;
   float* Cb = C + EH_C_OFF + bz * EH_C_BS;
+  constexpr long long CSM = EH_C_SM, CSN = EH_C_SN;
+#endif
 
   eh_f4v ra[AV], rb[BV];
 
   auto gload = [&](int kt) {
-    const long long k0 = (long long)kt * BK;
+    const long long k0 = kbeg + (long long)kt * BK;
 #pragma unroll
     for (int i = 0; i < AV; ++i) {
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
-      ra[i] = *reinterpret_cast<const eh_f4v*>(Ab + (m0 + m) * EH_LDA + k0 + kq * 4);
+      ra[i] = eh_tile_load<EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(Ab, m0 + m, k0 + kq * 4, M, kend);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
-      ra[i] = *reinterpret_cast<const eh_f4v*>(Ab + (k0 + k) * EH_LDA + m0 + mq * 4);
+      ra[i] = eh_tile_load<EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(Ab, m0 + mq * 4, k0 + k, M, kend);
 #endif
     }
 #pragma unroll
@@ -103,10 +149,10 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
       const int q = tid + i * NT;
 #if EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
-      rb[i] = *reinterpret_cast<const eh_f4v*>(Bb + (k0 + k) * EH_LDB + n0 + nq * 4);
+      rb[i] = eh_tile_load<EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(Bb, n0 + nq * 4, k0 + k, N, kend);
 #else
       const int n = q / (BK / 4), kq = q % (BK / 4);
-      rb[i] = *reinterpret_cast<const eh_f4v*>(Bb + (n0 + n) * EH_LDB + k0 + kq * 4);
+      rb[i] = eh_tile_load<EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(Bb, n0 + n, k0 + kq * 4, N, kend);
 #endif
     }
   };
@@ -181,6 +227,6 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
       for (int r = 0; r < 16; ++r) {
         const long long row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
         const long long col = n0 + wn * WN + j * 32 + l32;
-        Cb[row * EH_LDC + col] = acc[i][j][r];
+        if ((!EDGE_M || row < M) && (!EDGE_N || col < N)) Cb[row * CSM + col * CSN] = acc[i][j][r];
       }
 }

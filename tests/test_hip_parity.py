@@ -349,3 +349,80 @@ def test_config5_cnn_training_step(frontend, hip, sizes, fuse):
         scale = max(float(np.abs(r).max()), 1e-6)
         assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
         assert np.allclose(g.reshape(n.shape), n, rtol=1e-3, atol=1e-5 * scale)
+
+
+def _run_program(fe, hb, graph_fn, arrays, options=None):
+    """Lowers graph_fn with a buffer table, compiles it as one HIP program with `options`,
+    runs it and returns (flat result, launch schedules)."""
+    from harp_amd import workloads as wl
+    dev = hb.HipDevice(0)
+    prog_ast, arg_names, out, consts, _ = wl.lower_with_table([a.shape for a in arrays], graph_fn)
+    prog = hb.HipProgram(dev, prog_ast, options)
+    named = {}
+    for name, a in zip(arg_names, arrays):
+        b = hb.HipBuffer(dev, list(a.shape), fe.F32)
+        b.write_array(np.ascontiguousarray(a))
+        named[name] = b
+    for b in prog.buffers:
+        if b["name"] in consts and not b["elided"]:
+            cb = hb.HipBuffer(dev, [b["bytes"] // 4], fe.F32)
+            cb.write_array(np.full(b["bytes"] // 4, 0.0 if consts[b["name"]] == "zeros" else 1.0, np.float32))
+            named[b["name"]] = cb
+    outs = prog.execute(named)
+    return outs[out].read_array(np.float32), [l["schedule"] for l in prog.launches]
+
+
+def _contract(fe, kind):
+    """Contractions as the front end writes them (unsqueeze/expand, multiply, sum)."""
+    if kind == "matmul":                      # a [M,K] @ b [K,N]
+        return lambda a, b: fe.nn.matmul(a, b)
+    if kind == "linear":                      # x [B,K] . w [O,K]
+        return lambda x, w: fe.nn.linear(x, w)
+    if kind == "rows3d":                      # x [G,R,K] . w [O,K] -> [G,R,O]: (G,R) walk as one axis
+        return lambda x, w: (x.unsqueeze(2) * w.unsqueeze(0).unsqueeze(0)).sum(3)
+    if kind == "per_group":                   # g [G,R,O], c [G,R,K] -> [G,O,K], reduce over R
+        return lambda g, c: (g.unsqueeze(3) * c.unsqueeze(2)).sum(1)
+    raise KeyError(kind)
+
+
+CONTRACTIONS = [
+    # kind, shapes, options, expected in schedule
+    ("matmul", [(100, 60), (60, 36)], None, "edges"),
+    ("matmul", [(70, 50), (50, 30)], None, "/scalar"),
+    ("matmul", [(64, 2048), (2048, 64)], None, "split-k="),
+    ("matmul", [(96, 1000), (1000, 40)], None, "split-k="),
+    ("matmul", [(256, 512), (512, 256)], {"gemm_split_k": 3}, "split-k=3"),
+    ("matmul", [(192, 160), (160, 320)], {"gemm_bm": 128, "gemm_bn": 128, "gemm_bk": 16, "gemm_wm": 64, "gemm_wn": 64}, "tile=128x128x16"),
+    ("linear", [(130, 72), (50, 72)], None, "edges"),
+    ("linear", [(33, 18), (7, 18)], None, "/scalar"),
+    ("rows3d", [(6, 50, 36), (20, 36)], None, "mfma"),
+    ("rows3d", [(4, 49, 288), (64, 288)], None, "mfma"),
+    ("per_group", [(6, 50, 20), (6, 50, 36)], None, "mfma"),
+    ("per_group", [(3, 196, 64), (3, 196, 288)], None, "mfma"),
+]
+
+
+@pytest.mark.parametrize("kind,shapes,options,expect", CONTRACTIONS)
+def test_contraction_variants_on_mfma(frontend, hip, kind, shapes, options, expect):
+    """Ragged sizes, operands that cannot be read as 128-bit vectors, K split over
+    workgroups, row axes that merge, and per-group contractions all take the MFMA schedule
+    and match the C oracle (sum order differs: reduction tolerance) and float64 numpy."""
+    rng = RNG(sum(sum(s) for s in shapes))
+    arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
+    fn = _contract(frontend, kind)
+    got, scheds = _run_program(frontend, hip, fn, arrays, options)
+    assert any(s.startswith("mfma32x32x2(") and expect in s for s in scheds), scheds
+    ref = realize_on(frontend, "c", fn, arrays)
+    a64 = [a.astype(np.float64) for a in arrays]
+    if kind == "matmul":
+        exact, scale = a64[0] @ a64[1], np.abs(a64[0]) @ np.abs(a64[1])
+    elif kind == "linear":
+        exact, scale = a64[0] @ a64[1].T, np.abs(a64[0]) @ np.abs(a64[1]).T
+    elif kind == "rows3d":
+        exact, scale = a64[0] @ a64[1].T, np.abs(a64[0]) @ np.abs(a64[1]).T
+    else:
+        exact = np.einsum("gro,grk->gok", a64[0], a64[1])
+        scale = np.einsum("gro,grk->gok", np.abs(a64[0]), np.abs(a64[1]))
+    assert got.shape == ref.shape == (exact.size,)
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale.ravel() + 1e-30)
+    assert np.all(np.abs(got - exact.ravel()) <= 1e-5 * scale.ravel() + 1e-30)
