@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy (default: all but copy)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak (default: all but copy)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -150,6 +150,44 @@ def main():
         ms, _ = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
         log(f"[bench] copy 4096^2 ({prog.launches[0]['entry']}, {prog.launches[0]['schedule']}): "
             f"{ms * 1e3:.1f} us/step -> {2 * 4096 * 4096 * 4 / (ms * 1e-3) / 1e9:.0f} GB/s")
+        return
+
+    # ---- calibration: MFMA issue rate with operands in registers (not a result) -------------
+    if args.only == "mfma_peak":
+        iters, waves_per_cu = 4096, 8
+        src = """
+typedef float f16v __attribute__((ext_vector_type(16)));
+extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
+  f16v acc[4];
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  float a = threadIdx.x * 1e-3f, b = blockIdx.x * 1e-3f;
+  for (int it = 0; it < %d; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+  }
+  float s = 0.0f;
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += acc[i][r];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+""" % iters
+        blocks = props["compute_units"] * waves_per_cu // 4
+        mod = hb.HipModule(dev, hb.compile_source(src), "eh_mfma_peak")
+        out = hb.HipBuffer(dev, [blocks * 256 * 4], None, nbytes=blocks * 256 * 4)
+        for _ in range(3):
+            mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+        dev.sync()
+        e0, e1 = hb.Event(dev), hb.Event(dev)
+        e0.record()
+        reps = 20
+        for _ in range(reps):
+            mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+        e1.record()
+        e1.sync()
+        ms = e0.elapsed_ms(e1) / reps
+        flops = blocks * 4 * iters * 4 * (32 * 32 * 2 * 2)
+        log(f"[bench] MFMA f32 32x32x2 issue-rate ceiling: {flops / ms / 1e9:.1f} TFLOP/s "
+            f"({flops / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS:.1%} of the published {FP32_MFMA_PEAK_TFLOPS}); "
+            f"{blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
         return
 
     # ---- config 3: 4096^3 fp32 matmul --------------------------------------------------

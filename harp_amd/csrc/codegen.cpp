@@ -1256,6 +1256,46 @@ struct SerialReduce {
   }
 
   bool wants_split() const { return k.rloop.extent >= 512 && N <= (1 << 18); }
+  bool wants_columns() const { return k.rloop.extent >= 32 && N <= (1 << 16); }
+
+  // One launch; a workgroup owns 64 outputs and RG threads share each output's reduction
+  // (interleaved rows, partials combined through LDS in a fixed order).  For reductions too
+  // short to split over workgroups but long enough that one thread per output would spend
+  // its time waiting on dependent loads.
+  LaunchSpec columns() const {
+    const int64_t K = k.rloop.extent;
+    const int RG = K >= 128 ? 16 : 4;
+    const int block = 64 * RG;
+    LaunchSpec ls;
+    ls.entry = "ehk_" + k.name;
+    ls.kernels = {k.name};
+    ls.schedule = "column-reduce(block=" + std::to_string(block) + ",threads/output=" + std::to_string(RG) + ")";
+    ls.grid[0] = static_cast<unsigned>((N + 63) / 64);
+    ls.block[0] = static_cast<unsigned>(block);
+    const std::string TA = ctype(k.acc_dtype);
+    ExprRenderer er;
+    std::ostringstream os;
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "(" << params(&ls, true, "")
+       << ") {\n";
+    os << "  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;\n";
+    os << "  const idx_t eh_oo = (idx_t)blockIdx.x * 64 + tx;\n  const bool eh_ok = eh_oo < " << N << ";\n";
+    os << "  const idx_t eh_o = eh_ok ? eh_oo : " << N - 1 << ";\n";
+    os << decode("eh_o");
+    os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+    os << "#pragma unroll 4\n";
+    os << "  for (idx_t " << k.rloop.var << " = ty; " << k.rloop.var << " < " << K << "; " << k.rloop.var << " += " << RG
+       << ") {\n";
+    os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
+    os << "  __shared__ " << TA << " eh_sm[" << RG << "][64];\n  eh_sm[ty][tx] = acc;\n  __syncthreads();\n";
+    os << "  if (ty == 0 && eh_ok) {\n    " << TA << " r = eh_sm[0][tx];\n";
+    os << "    for (int q = 1; q < " << RG << "; ++q) r = " << combine_text(k.rkind, k.acc_dtype, "r", "eh_sm[q][tx]") << ";\n";
+    NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
+    os << "    " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")r;\n  }\n}\n";
+    ls.source = os.str();
+    min_bytes(&ls);
+    return ls;
+  }
 
   // Two launches and one scratch buffer (appended to `buffers`).
   std::vector<LaunchSpec> split(std::vector<BufferInfo>* buffers) const {
@@ -1336,6 +1376,8 @@ void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan*
   SerialReduce sr(k, opt);
   if (sr.wants_split()) {
     for (auto& ls : sr.split(&plan->buffers)) plan->launches.push_back(std::move(ls));
+  } else if (sr.wants_columns()) {
+    plan->launches.push_back(sr.columns());
   } else {
     plan->launches.push_back(sr.single());
   }

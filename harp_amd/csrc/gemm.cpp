@@ -40,7 +40,7 @@ struct Choice {
 // put several workgroups on each of the 256 CUs; when even the small tile leaves CUs
 // idle and K is long, K is split over blockIdx.y.
 bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
-  if (s.K < 16 || s.M < 2 || s.N < 2) return false;
+  if (s.K < 8 || s.M < 2 || s.N < 2) return false;
   Choice c;
   if (opt.gemm_bm > 0) {
     c.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
