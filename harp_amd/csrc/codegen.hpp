@@ -24,6 +24,8 @@ struct GenOptions {
   int flat_block = 256;
   int flat_iters = 4;        // vectors handled by one thread of a flat kernel
   int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
+  int gemm_setprio = 0;               // wave priority during the multiply loop
+  int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
   int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores

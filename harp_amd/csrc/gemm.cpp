@@ -17,12 +17,23 @@ struct Tile {
   int bm, bn, bk, wm, wn;
 };
 
-// Each uses 256 threads (four waves).
-const Tile kBig = {128, 128, 16, 64, 64}, kSmall = {64, 64, 16, 32, 32};
+// Candidate tiles: {bm, bn, bk, wm, wn}, workgroups one CU holds at once (registers and LDS),
+// sustained TFLOP/s with the chip full (measured on 4096^3), and the share of a full CU's
+// rate that a single resident workgroup reaches.
+struct Candidate {
+  Tile tile;
+  int wgs_per_cu;
+  double rate, alone;
+};
+const Candidate kCandidates[] = {
+    {{256, 256, 16, 64, 64}, 1, 133.0, 1.0},   // 16 waves
+    {{128, 128, 16, 64, 64}, 4, 124.0, 0.4},   // 4 waves
+    {{64, 64, 16, 32, 32}, 8, 105.0, 0.25},    // 4 waves
+};
 
 bool tile_valid(const Tile& t) {
   if (t.bm <= 0 || t.bn <= 0 || t.bk <= 0 || t.wm <= 0 || t.wn <= 0) return false;
-  if (t.bm % t.wm || t.bn % t.wn || t.wm % 32 || t.wn % 32 || t.bk % 4) return false;
+  if (t.bm % t.wm || t.bn % t.wn || t.wm % 32 || t.wn % 32 || t.bk % 16) return false;
   int nt = (t.bm / t.wm) * (t.bn / t.wn) * 64;
   if (nt > 1024 || (t.bm * t.bk) % (4 * nt) || (t.bn * t.bk) % (4 * nt)) return false;
   size_t lds = 2ull * static_cast<size_t>(t.bk) * (t.bm + 4 + t.bn + 4) * 4;
@@ -36,30 +47,60 @@ struct Choice {
   int split_k = 1;
 };
 
-// Tile and K split.  The big tile halves LDS traffic per flop but needs enough tiles to
-// put several workgroups on each of the 256 CUs; when even the small tile leaves CUs
-// idle and K is long, K is split over blockIdx.y.
+// Estimated microseconds for one tile shape and K split: whole rounds of resident
+// workgroups at the tile's sustained rate, a last partial round no faster than a lone
+// workgroup allows, plus writing and re-reading the partial tiles when K is split.
+double estimate_us(const GemmShape& s, const Candidate& c, int split) {
+  const double cus = 256.0;
+  const int64_t wgs = ceil_div(s.M, c.tile.bm) * ceil_div(s.N, c.tile.bn) * s.batch * split;
+  const int64_t ksteps = ceil_div(ceil_div(s.K, c.tile.bk), split);
+  const double wg_flops = 2.0 * c.tile.bm * c.tile.bn * static_cast<double>(ksteps) * c.tile.bk;
+  const double slots = cus * c.wgs_per_cu;
+  const double round_us = slots * wg_flops / (c.rate * 1e6);
+  const int64_t full = wgs / static_cast<int64_t>(slots);
+  const int64_t rest = wgs - full * static_cast<int64_t>(slots);
+  double us = static_cast<double>(full) * round_us;
+  if (rest > 0) {
+    double per_cu = static_cast<double>(ceil_div(rest, static_cast<int64_t>(cus))) / c.wgs_per_cu;
+    us += round_us * std::max(per_cu, c.alone / c.wgs_per_cu * 1.0);
+  }
+  us += 2.0;   // prologue, epilogue, launch
+  if (split > 1) us += 3.0 + (split + 1.0) * 4.0 * static_cast<double>(s.batch * s.M * s.N) / 4e6;
+  return us;
+}
+
+// Tile and K split for a contraction.
 bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
   if (s.K < 8 || s.M < 2 || s.N < 2) return false;
-  Choice c;
+  Choice best;
   if (opt.gemm_bm > 0) {
-    c.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
-    if (!tile_valid(c.tile)) return false;
-  } else {
-    int64_t big = ceil_div(s.M, 128) * ceil_div(s.N, 128) * s.batch;
-    bool waste_ok = s.M >= 96 && s.N >= 96;
-    c.tile = (big >= 512 && waste_ok) ? kBig : kSmall;
+    best.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
+    if (!tile_valid(best.tile)) return false;
+    int64_t ksteps = ceil_div(s.K, best.tile.bk);
+    if (opt.gemm_split_k > 1) best.split_k = static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps));
+    *out = best;
+    return true;
   }
-  int64_t tiles = ceil_div(s.M, c.tile.bm) * ceil_div(s.N, c.tile.bn) * s.batch;
-  int64_t ksteps = ceil_div(s.K, c.tile.bk);
-  if (opt.gemm_split_k > 0) {
-    c.split_k = static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps));
-  } else if (opt.gemm_split_k < 0 && tiles < 256 && ksteps >= 32) {
-    int64_t want = ceil_div(1024, tiles);
-    c.split_k = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(want, ksteps / 8)));
+  double best_us = 0;
+  bool have = false;
+  for (const auto& c : kCandidates) {
+    const int64_t ksteps = ceil_div(s.K, c.tile.bk);
+    for (int split : {1, 2, 4, 8, 16, 32}) {
+      if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
+      if (opt.gemm_split_k > 1 && split != 1) break;
+      int sp = opt.gemm_split_k > 1 ? static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps)) : split;
+      if (sp > 1 && ksteps / sp < 8) break;
+      double us = estimate_us(s, c, sp);
+      if (!have || us < best_us) {
+        have = true;
+        best_us = us;
+        best.tile = c.tile;
+        best.split_k = sp;
+      }
+    }
   }
-  *out = c;
-  return true;
+  *out = best;
+  return have;
 }
 
 // Whether an operand can be read with aligned 128-bit loads along its unit-stride axis.
@@ -196,6 +237,13 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
   os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
+  {
+    // a 256-thread workgroup puts one wave on each SIMD; four resident workgroups per CU need
+    // 128 registers per lane or fewer, larger workgroups get proportionally fewer
+    int waves = opt.gemm_waves > 0 ? opt.gemm_waves : std::max(1, 4 / std::max(1, nt / 256)) * std::max(1, nt / 256);
+    os << "#define EH_WAVES_PER_SIMD " << std::min(8, waves) << "\n";
+  }
+  os << "#define EH_SETPRIO " << std::max(0, std::min(3, opt.gemm_setprio)) << "\n";
   os << kGemmSource;
   ls.source = os.str();
   const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;

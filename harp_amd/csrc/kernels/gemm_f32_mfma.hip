@@ -1,14 +1,24 @@
 // FP32 contraction C[m,n] = sum_k A[m,k] * B[k,n] on CDNA4 matrix cores (gfx950).
 //
 // One workgroup owns a BM x BN tile of C and walks K in steps of BK.  Each wave owns a WM x WN
-// sub-tile as (WM/32) x (WN/32) accumulators of v_mfma_f32_32x32x2_f32.  A and B tiles are
-// staged in LDS k-major ([k][m] and [k][n], rows padded by 4 floats): the MFMA operand for
-// lane l is row k = 2*step + l/32, column l%32 of the wave's slice, so every half-wave reads
-// 32 consecutive floats.  Global loads are 128-bit along whichever axis of the operand is
-// contiguous; an operand whose contiguous axis is k is transposed on its way into LDS.
-// Two LDS buffers: the loads of tile t+1 are in flight while tile t is multiplied, one
-// barrier per step.  Workgroup ids are remapped so that each XCD (ids congruent mod 8) works
-// on a compact block of tiles and shares A/B panels through its own L2.
+// sub-tile as (WM/32) x (WN/32) accumulators of v_mfma_f32_32x32x2_f32.
+//
+// LDS holds each operand tile in the layout its global layout allows to be written with one
+// 128-bit store per thread, so nothing is transposed on the way in:
+//   * an operand whose contiguous axis is k is kept as [k/4][row][4]: a thread's four
+//     consecutive k values of one row are one LDS element, and a lane later reads the four
+//     with one ds_read_b128;
+//   * an operand whose contiguous axis is the row (m for A, n for B) is kept as [k][row].
+// The sum over k does not care which k value goes to which MFMA, so inside a block of eight
+// k values MFMA e (e = 0..3) multiplies k = 8j+e on lanes 0-31 and k = 8j+4+e on lanes 32-63:
+// that is what makes the four-k element usable as is.  Rows are padded by four floats
+// (elements) so that stores and reads spread over the banks.
+//
+// Two LDS buffers; the global loads of tile t+1 are issued before tile t is multiplied, the
+// LDS operands of k-block j+1 are fetched while block j is multiplied, and the last block of a
+// tile step is multiplied after the next tile has been published (store, barrier) and its
+// first operands requested.  Workgroup ids are remapped so that each XCD (ids congruent mod
+// 8) works on a compact block of tiles and shares A/B panels through its own L2.
 // Sizes need not be multiples of the tile (edge tiles load zeros and skip stores), operands
 // that cannot be read as aligned 128-bit vectors are read element by element, and a long K
 // with few output tiles can be split over blockIdx.y into partial sums.
@@ -48,6 +58,9 @@
 #define EH_SPLITK 1
 #define EH_GROUP_M 8
 #endif
+#ifndef EH_SETPRIO
+#define EH_SETPRIO 0     // wave priority while multiplying
+#endif
 
 typedef float eh_f16v __attribute__((ext_vector_type(16)));
 typedef float eh_f4v __attribute__((ext_vector_type(4)));
@@ -55,9 +68,10 @@ typedef float eh_f4v __attribute__((ext_vector_type(4)));
 namespace {
 constexpr int BM = EH_BM, BN = EH_BN, BK = EH_BK, WM = EH_WM, WN = EH_WN;
 constexpr int NWM = BM / WM, NWN = BN / WN, NT = NWM * NWN * 64;
-constexpr int AS = BM + 4, BS = BN + 4;            // padded LDS row lengths
+constexpr int AS = BM + 4, BS = BN + 4;            // padded row counts / row lengths in LDS
 constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 4-element loads per thread per tile
 constexpr int IB = WM / 32, JB = WN / 32;
+constexpr int NBLK = BK / 8;                       // blocks of eight k values per tile step
 constexpr long long M = EH_M, N = EH_N, K = EH_K;
 constexpr int TM = (EH_M + BM - 1) / BM, TN = (EH_N + BN - 1) / BN, NTILES = TM * TN;
 constexpr int KT_ALL = (EH_K + BK - 1) / BK;
@@ -66,13 +80,13 @@ constexpr int KT = (KT_ALL + EH_SPLITK - 1) / EH_SPLITK;      // k-steps per spl
 constexpr bool EDGE_M = EH_M % BM != 0, EDGE_N = EH_N % BN != 0;
 constexpr bool EDGE_K = EH_K % BK != 0 || KT_ALL % EH_SPLITK != 0;
 static_assert(BM * BK % (4 * NT) == 0 && BN * BK % (4 * NT) == 0 && AV >= 1 && BV >= 1, "tile does not split over the threads");
-static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 4 == 0, "wave tile must be built from 32x32x2 MFMAs");
+static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "wave tile must be built from 32x32x2 MFMAs, k in pairs of blocks of eight");
 // 128-bit loads need the four elements to be in range together
 static_assert(!EH_A_VEC || (EH_A_KCONTIG ? EH_K % 4 == 0 : EH_M % 4 == 0), "A cannot be loaded as vectors");
 static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B cannot be loaded as vectors");
 
 // Four elements of an operand starting at (r, k) and running along its fast axis; elements
-// outside [0,R) x [0,kend) read as zero.  `along_k` says which axis the four run along.
+// outside [0,R) x [0,kend) read as zero.  ALONG_K says which axis the four run along.
 template <bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
 __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long r, long long k,
                                               long long R, long long kend) {
@@ -89,13 +103,38 @@ __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long
   }
   return v;
 }
+
+// One operand tile in LDS (RS = padded number of rows).  KC: [k/4][row][4], else [k][row].
+template <bool KC, int RS>
+struct EhTile {
+  // where a thread's four elements go: (row r, k0..k0+3) for KC, (k, rows r0..r0+3) otherwise
+  __device__ __forceinline__ static void put(float* t, int r, int k, eh_f4v v) {
+    if (KC) *reinterpret_cast<eh_f4v*>(&t[((k >> 2) * RS + r) * 4]) = v;
+    else *reinterpret_cast<eh_f4v*>(&t[k * RS + r]) = v;
+  }
+  // the four operand values of one lane for k-block j: element e feeds MFMA e
+  __device__ __forceinline__ static eh_f4v get(const float* t, int j, int kh, int r) {
+    if (KC) return *reinterpret_cast<const eh_f4v*>(&t[((2 * j + kh) * RS + r) * 4]);
+    eh_f4v v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = t[(8 * j + 4 * kh + e) * RS + r];
+    return v;
+  }
+};
+using ATile = EhTile<EH_A_KCONTIG != 0, AS>;
+using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restrict__ A,
+#ifndef EH_WAVES_PER_SIMD
+#define EH_WAVES_PER_SIMD 4   // register budget: 512 / this many VGPRs+AGPRs per lane
+#endif
+
+extern "C" __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(EH_WAVES_PER_SIMD, EH_WAVES_PER_SIMD)))
+EH_ENTRY(const float* __restrict__ A,
                                                           const float* __restrict__ B,
                                                           float* __restrict__ C) {
-  __shared__ float As[2][BK * AS];
-  __shared__ float Bs[2][BK * BS];
+  __shared__ __attribute__((aligned(16))) float As[2][BK * AS];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * BS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wid = tid >> 6;
@@ -131,6 +170,8 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
 
   eh_f4v ra[AV], rb[BV];
 
+  // thread q of the tile owns four elements: along k at (row q / (BK/4), k 4*(q % (BK/4))) for
+  // a k-contiguous operand, along the row at (k q / (rows/4), row 4*(q % (rows/4))) otherwise
   auto gload = [&](int kt) {
     const long long k0 = kbeg + (long long)kt * BK;
 #pragma unroll
@@ -162,24 +203,18 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
     for (int i = 0; i < AV; ++i) {
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
-      const int m = q / (BK / 4), kq = q % (BK / 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) As[buf][(kq * 4 + e) * AS + m] = ra[i][e];
+      ATile::put(As[buf], q / (BK / 4), (q % (BK / 4)) * 4, ra[i]);
 #else
-      const int k = q / (BM / 4), mq = q % (BM / 4);
-      *reinterpret_cast<eh_f4v*>(&As[buf][k * AS + mq * 4]) = ra[i];
+      ATile::put(As[buf], (q % (BM / 4)) * 4, q / (BM / 4), ra[i]);
 #endif
     }
 #pragma unroll
     for (int i = 0; i < BV; ++i) {
       const int q = tid + i * NT;
 #if EH_B_NCONTIG
-      const int k = q / (BN / 4), nq = q % (BN / 4);
-      *reinterpret_cast<eh_f4v*>(&Bs[buf][k * BS + nq * 4]) = rb[i];
+      BTile::put(Bs[buf], (q % (BN / 4)) * 4, q / (BN / 4), rb[i]);
 #else
-      const int n = q / (BK / 4), kq = q % (BK / 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) Bs[buf][(kq * 4 + e) * BS + n] = rb[i][e];
+      BTile::put(Bs[buf], q / (BK / 4), (q % (BK / 4)) * 4, rb[i]);
 #endif
     }
   };
@@ -196,26 +231,53 @@ extern "C" __global__ void __launch_bounds__(NT) EH_ENTRY(const float* __restric
   sstore(0);
   __syncthreads();
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) gload(kt + 1);
-    const float* as = &As[buf][wm * WM + l32];
-    const float* bs = &Bs[buf][wn * WN + l32];
+  // two register slots of operands: block j+1 is fetched while block j is multiplied
+  eh_f4v a[2][IB], b[2][JB];
+  auto fetch = [&](int buf, int j, int slot) {
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float a[IB], b[JB];
+    for (int i = 0; i < IB; ++i) a[slot][i] = ATile::get(As[buf], j, kh, wm * WM + i * 32 + l32);
 #pragma unroll
-      for (int i = 0; i < IB; ++i) a[i] = as[(kk + kh) * AS + i * 32];
+    for (int jj = 0; jj < JB; ++jj) b[slot][jj] = BTile::get(Bs[buf], j, kh, wn * WN + jj * 32 + l32);
+  };
+  auto multiply = [&](int slot) {
 #pragma unroll
-      for (int j = 0; j < JB; ++j) b[j] = bs[(kk + kh) * BS + j * 32];
+    for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int i = 0; i < IB; ++i)
 #pragma unroll
-        for (int j = 0; j < JB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int jj = 0; jj < JB; ++jj)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[slot][i][e], b[slot][jj][e], acc[i][jj], 0, 0, 0);
+  };
+
+  fetch(0, 0, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    const bool more = kt + 1 < KT;
+    if (more) {
+      gload(kt + 1);
+      // keep the global loads up here: their latency is hidden by the whole multiply loop only
+      // if they are issued before it (the compiler would otherwise sink them to their use)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (kt + 1 < KT) sstore(buf ^ 1);
+#if EH_SETPRIO
+    __builtin_amdgcn_s_setprio(EH_SETPRIO);
+#endif
+#pragma unroll
+    for (int j = 0; j < NBLK - 1; ++j) {
+      fetch(buf, j + 1, (j + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);   // reads of the next block stay ahead of these MFMAs
+      multiply(j & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#if EH_SETPRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
+    if (more) sstore(buf ^ 1);
     __syncthreads();
+    if (more) fetch(buf ^ 1, 0, NBLK & 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply((NBLK - 1) & 1);
   }
 
   // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
