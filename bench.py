@@ -300,6 +300,17 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
                "sample": f"full 4096x4096 softmax, unfused R,E,E,R,E kernels (gcc -O3 -ffast-math), "
                          f"median of {reps} passes, {sec * 1e3:.0f} ms/pass"}
         log(f"[bench] cpu baseline softmax: {sec * 1e3:.0f} ms/pass -> {cpu['value']:.2f} GB/s (1 core)")
+        # the OpenMP variant of the same kernels on the cores this process may use
+        cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+        cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+        os.environ["OMP_NUM_THREADS"] = str(cores)
+        sec_o, reps_o, _ = baseline.time_graph(wl.config2_graph, arrays, min_seconds=4.0, max_reps=40, openmp=True)
+        result_extra["cpu_baseline_openmp"] = {
+            "value": softmax["algo_bytes"] / sec_o / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"full 4096x4096 softmax, the same five kernels with '#pragma omp parallel for' on the "
+                      f"outer loop (gcc -O3 -ffast-math -fopenmp), median of {reps_o} passes, {sec_o * 1e3:.1f} ms/pass"}
+        log(f"[bench] cpu baseline softmax, OpenMP: {sec_o * 1e3:.1f} ms/pass -> "
+            f"{result_extra['cpu_baseline_openmp']['value']:.1f} GB/s ({cores} cores)")
         if matmul is not None:
             a, b = wl.config3_inputs()
             sub = 8

@@ -541,6 +541,77 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan);
 }  // namespace
 
+// An elementwise kernel as a function of the linear index of its (dense, row-major) output, for
+// contractions that evaluate it in their tile loader.  Only kernels reading one f32 buffer.
+std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems) {
+  if (k.rkind != ReduceKind::None || k.out_dtype.ty != Ty::F32 || !k.out_aff || k.out_aff->c != 0) return std::nullopt;
+  int64_t stride = 1, numel = 1;
+  std::vector<int64_t> strides(k.loops.size(), 0);
+  size_t used = 0;
+  for (size_t i = k.loops.size(); i-- > 0;) {
+    const Loop& l = k.loops[i];
+    if (l.extent <= 0) return std::nullopt;
+    strides[i] = stride;
+    if (l.extent > 1) {
+      if (k.out_aff->of(l.var) != stride) return std::nullopt;
+      ++used;
+    }
+    stride *= l.extent;
+    numel *= l.extent;
+  }
+  for (const auto& kv : k.out_aff->coef) {
+    bool live = false;
+    for (const auto& l : k.loops) live = live || (l.var == kv.first && l.extent > 1);
+    if (kv.second != 0 && !live) return std::nullopt;
+  }
+  (void)used;
+  std::vector<LoadRef> loads;
+  collect_loads(*k.value, loads);
+  if (loads.empty()) return std::nullopt;
+  const std::string src = loads[0].load->args[0]->name;
+  for (const auto& lr : loads) {
+    if (lr.load->args[0]->op != Op::Var || lr.load->args[0]->name != src) return std::nullopt;
+    if (lr.load->dtype.ty != Ty::F32 || lr.load->count != 1) return std::nullopt;
+  }
+  if (src == k.out_buf) return std::nullopt;
+  // pure gathers only (a load, possibly under an index-only guard with a constant default):
+  // anything that computes is cheaper done once than once per tile that reads it
+  {
+    const Node* v = k.value.get();
+    if (v->op == Op::Select && v->args[2]->op == Op::Const) {
+      std::vector<LoadRef> in_cond;
+      collect_loads(*v->args[0], in_cond);
+      if (!in_cond.empty()) return std::nullopt;
+      v = v->args[1].get();
+    }
+    if (v->op != Op::Load) return std::nullopt;
+  }
+  auto it = elems.find(src);
+  const bool small = it != elems.end() && it->second < (size_t{1} << 30) && numel < (int64_t{1} << 30);
+  FoldedOperand f;
+  f.src = src;
+  f.src_bytes = it == elems.end() ? 0.0 : 4.0 * static_cast<double>(it->second);
+  std::ostringstream os;
+  os << "// element eh_L of what kernel " << k.name << " would have written\n";
+  os << "__device__ __forceinline__ float EH_FOLD_FN(const float* __restrict__ " << src << ", long long eh_L) {\n";
+  os << "  typedef " << (small ? "int" : "long long") << " eh_fold_idx;\n  const eh_fold_idx eh_l = (eh_fold_idx)eh_L;\n";
+  for (size_t i = 0; i < k.loops.size(); ++i) {
+    const Loop& l = k.loops[i];
+    if (l.extent == 1) {
+      os << "  const eh_fold_idx " << l.var << " = 0;\n";
+    } else {
+      os << "  const eh_fold_idx " << l.var << " = (eh_l / " << strides[i] << ") % " << l.extent << ";\n";
+    }
+  }
+  ExprRenderer er;
+  os << "  return (float)(" << er.expr(*k.value) << ");\n}\n";
+  f.function = os.str();
+  if (auto a = affine_of(*loads[0].load->args[1]))
+    for (size_t i = 0; i < k.loops.size(); ++i)
+      if (k.loops[i].extent > 1) f.src_stride[strides[i]] = a->of(k.loops[i].var);
+  return f;
+}
+
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
   ProgramPlan plan;
@@ -633,8 +704,38 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // gather / copy kernels read only by contractions are evaluated inside those contractions'
+  // tile loaders (implicit GEMM): no launch, no buffer
+  FoldMap folded;
+  std::set<size_t> folded_kernels;
+  if (opt.gemm && opt.gemm_fold && have_table) {
+    for (size_t p = 0; p < kernels.size(); ++p) {
+      if (!nests[p] || nests[p]->rkind != ReduceKind::None) continue;
+      const NestKernel& pk = *nests[p];
+      if (role_of(pk.out_buf) != "temp") continue;
+      auto rd = readers.find(pk.out_buf);
+      if (rd == readers.end() || rd->second.empty()) continue;
+      bool ok = true;
+      for (size_t r : rd->second) {
+        if (r <= p || !nests[r] || !gemm_shaped(*nests[r], opt)) { ok = false; break; }
+        auto g = match_gemm(*nests[r]);
+        if (!g || (g->a_buf == pk.out_buf) == (g->b_buf == pk.out_buf)) { ok = false; break; }
+      }
+      if (!ok) continue;
+      auto f = make_fold(pk, elems);
+      if (!f || folded.count(f->src)) continue;
+      folded[pk.out_buf] = *f;
+      folded_kernels.insert(p);
+      plan.elided.insert(pk.out_buf);
+    }
+  }
+
   size_t i = 0;
   while (i < kernels.size()) {
+    if (folded_kernels.count(i)) {
+      ++i;
+      continue;
+    }
     if (!nests[i]) {
       plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
       ++i;
@@ -643,7 +744,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     const NestKernel& k0 = *nests[i];
     // contraction (matmul-shaped reduce) -> MFMA schedule
     if (k0.rkind == ReduceKind::Sum && opt.gemm) {
-      auto gl = try_emit_gemm(k0, opt, &plan.buffers);
+      auto gl = try_emit_gemm(k0, opt, &plan.buffers, &folded);
       if (!gl.empty()) {
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
         ++i;
@@ -670,7 +771,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       g.stages.push_back(c.stage);
     }
     ++i;
-    while (opt.fuse && i < kernels.size() && nests[i]) {
+    while (opt.fuse && i < kernels.size() && nests[i] && !folded_kernels.count(i)) {
       const NestKernel& k = *nests[i];
       if (k.rkind == ReduceKind::Sum && opt.gemm && gemm_shaped(k, opt)) break;
       Canon pick;

@@ -1,6 +1,7 @@
 #include "gemm.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <sstream>
 
 namespace eh {
@@ -204,15 +205,33 @@ bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
   return s && choose(*s, opt, &c);
 }
 
-std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers) {
+std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers,
+                                      const FoldMap* folded) {
   auto s = match_gemm(k);
   Choice ch;
   if (!s || !choose(*s, opt, &ch)) return {};
   const Tile& t = ch.tile;
+  const FoldedOperand* fa = nullptr;
+  const FoldedOperand* fb = nullptr;
+  if (folded) {
+    auto ia = folded->find(s->a_buf), ib = folded->find(s->b_buf);
+    if (ia != folded->end()) fa = &ia->second;
+    if (ib != folded->end()) fb = &ib->second;
+  }
   // each thread fetches four elements along the operand's faster axis
-  const bool a_kc = s->a_k <= s->a_m, b_nc = s->b_n <= s->b_k;
-  const bool a_vec = a_kc ? vec_ok(s->K, s->a_k, s->a_m, s->a_off, s->a_b) : vec_ok(s->M, s->a_m, s->a_k, s->a_off, s->a_b);
-  const bool b_vec = b_nc ? vec_ok(s->N, s->b_n, s->b_k, s->b_off, s->b_b) : vec_ok(s->K, s->b_k, s->b_n, s->b_off, s->b_b);
+  bool a_kc = s->a_k <= s->a_m, b_nc = s->b_n <= s->b_k;
+  // a computed operand is walked along whichever of its axes is contiguous in the memory its
+  // producer reads (rows when both are or neither is known)
+  auto along_k = [](const FoldedOperand& f, int64_t s_row, int64_t s_k) {
+    auto ir = f.src_stride.find(s_row), ik = f.src_stride.find(s_k);
+    int64_t r = ir == f.src_stride.end() ? 0 : std::llabs(ir->second);
+    int64_t kk = ik == f.src_stride.end() ? 0 : std::llabs(ik->second);
+    return kk != 0 && (r == 0 || kk < r);
+  };
+  if (fa) a_kc = along_k(*fa, s->a_m, s->a_k);
+  if (fb) b_nc = !along_k(*fb, s->b_n, s->b_k);
+  const bool a_vec = !fa && (a_kc ? vec_ok(s->K, s->a_k, s->a_m, s->a_off, s->a_b) : vec_ok(s->M, s->a_m, s->a_k, s->a_off, s->a_b));
+  const bool b_vec = !fb && (b_nc ? vec_ok(s->N, s->b_n, s->b_k, s->b_off, s->b_b) : vec_ok(s->K, s->b_k, s->b_n, s->b_off, s->b_b));
   const int S = ch.split_k;
   std::vector<LaunchSpec> out(S > 1 ? 2 : 1);
   LaunchSpec& ls = out[0];
@@ -237,6 +256,15 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
   os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
+  auto emit_fold = [&](const FoldedOperand* f, const char* macro, const char* fn) {
+    if (!f) return;
+    std::string text = f->function;
+    const std::string ph = "EH_FOLD_FN";
+    for (size_t at = text.find(ph); at != std::string::npos; at = text.find(ph, at)) text.replace(at, ph.size(), fn);
+    os << "#define " << macro << " 1\n" << text;
+  };
+  emit_fold(fa, "EH_A_FOLD", "eh_a_elem");
+  emit_fold(fb, "EH_B_FOLD", "eh_b_elem");
   {
     // a 256-thread workgroup puts one wave on each SIMD; four resident workgroups per CU need
     // 128 registers per lane or fewer, larger workgroups get proportionally fewer
@@ -249,7 +277,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;
   ls.schedule = "mfma32x32x2(tile=" + std::to_string(t.bm) + "x" + std::to_string(t.bn) + "x" + std::to_string(t.bk) +
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
-                (a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") + (b_vec ? "" : "/scalar") +
+                (fa ? "/folded" : a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") +
+                (fb ? "/folded" : b_vec ? "" : "/scalar") +
                 (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
   ls.grid[1] = static_cast<unsigned>(S);
@@ -258,15 +287,23 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   const size_t c_elems =
       static_cast<size_t>(s->c_off + (s->M - 1) * s->c_m + (s->N - 1) * s->c_n + (s->batch - 1) * s->c_b + 1);
   const size_t part_elems = static_cast<size_t>(S) * static_cast<size_t>(s->batch * s->M * s->N);
-  ls.arg_bufs = {s->a_buf, s->b_buf, S > 1 ? scratch : s->c_buf};
+  ls.arg_bufs = {fa ? fa->src : s->a_buf, fb ? fb->src : s->b_buf, S > 1 ? scratch : s->c_buf};
+  // a folded operand binds the producer's source, whose size the buffer table already fixes
   ls.arg_min_bytes = {
-      4 * static_cast<size_t>(s->a_off + (s->M - 1) * s->a_m + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
-      4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1),
+      fa ? 0 : 4 * static_cast<size_t>(s->a_off + (s->M - 1) * s->a_m + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
+      fb ? 0 : 4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1),
       4 * (S > 1 ? part_elems : c_elems)};
   ls.flops = 2.0 * static_cast<double>(s->M) * static_cast<double>(s->N) * static_cast<double>(s->K) *
              static_cast<double>(s->batch);
-  ls.algo_bytes = 4.0 * static_cast<double>(s->batch) *
-                  (static_cast<double>(s->M) * s->K + static_cast<double>(s->K) * s->N + static_cast<double>(s->M) * s->N);
+  {
+    // an operand the batch does not move (stride 0) is read once, not once per batch
+    const double nb = static_cast<double>(s->batch);
+    double a_bytes = 4.0 * static_cast<double>(s->M) * s->K * (s->a_b == 0 ? 1.0 : nb);
+    double b_bytes = 4.0 * static_cast<double>(s->K) * s->N * (s->b_b == 0 ? 1.0 : nb);
+    if (fa && fa->src_bytes > 0) a_bytes = fa->src_bytes;
+    if (fb && fb->src_bytes > 0) b_bytes = fb->src_bytes;
+    ls.algo_bytes = a_bytes + b_bytes + 4.0 * nb * static_cast<double>(s->M) * s->N;
+  }
   if (S > 1) {
     BufferInfo sb;
     sb.name = scratch;

@@ -6,6 +6,7 @@
 // src/opt/graph/suggesters/matmul.rs:60-65).
 #pragma once
 
+#include <map>
 #include <optional>
 
 #include "analysis.hpp"
@@ -21,6 +22,22 @@ struct GemmShape {
   int64_t c_m = 0, c_n = 0, c_b = 0, c_off = 0;
 };
 
+// An elementwise producer (im2col gather, layout copy, padding ...) whose dense output a
+// contraction would read: the tile loader evaluates it per element instead, so the buffer is
+// never written.  `function` is the text of
+//   __device__ float EH_FOLD_FN(const float* __restrict__ <src>, long long eh_L)
+// returning element eh_L of the producer's output.
+struct FoldedOperand {
+  std::string src;        // the one buffer the producer reads
+  std::string function;
+  double src_bytes = 0;   // 0 = unknown
+  // for each loop of the producer: its stride in the producer's output -> its stride in the
+  // source (only when the source index is affine); tells which operand axis is contiguous in
+  // the memory actually read
+  std::map<int64_t, int64_t> src_stride;
+};
+using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer
+
 // Recognises the contraction and returns its strides; nullopt otherwise.
 std::optional<GemmShape> match_gemm(const NestKernel& k);
 
@@ -30,6 +47,7 @@ bool gemm_shaped(const NestKernel& k, const GenOptions& opt);
 // HIP source + dispatch for the kernel; empty when it is not a contraction the MFMA schedule
 // covers (the caller then falls back to another schedule).  One launch, or two when K is
 // split: partial tiles into a scratch buffer appended to `buffers`, then their sum.
-std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers);
+std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers,
+                                      const FoldMap* folded = nullptr);
 
 }  // namespace eh

@@ -19,6 +19,9 @@
 // tile step is multiplied after the next tile has been published (store, barrier) and its
 // first operands requested.  Workgroup ids are remapped so that each XCD (ids congruent mod
 // 8) works on a compact block of tiles and shares A/B panels through its own L2.
+// An operand can also be computed instead of loaded: when a gather or copy kernel (im2col,
+// a layout change, padding) would have produced it, the generator passes that kernel as a
+// function of the element index and the tile loader calls it (implicit GEMM).
 // Sizes need not be multiples of the tile (edge tiles load zeros and skip stores), operands
 // that cannot be read as aligned 128-bit vectors are read element by element, and a long K
 // with few output tiles can be split over blockIdx.y into partial sums.
@@ -85,20 +88,41 @@ static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "wave tile must be b
 static_assert(!EH_A_VEC || (EH_A_KCONTIG ? EH_K % 4 == 0 : EH_M % 4 == 0), "A cannot be loaded as vectors");
 static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B cannot be loaded as vectors");
 
+// How element i of an operand is obtained: from memory, or (EH_A_FOLD / EH_B_FOLD) by
+// evaluating the elementwise kernel that would have produced it, on that kernel's own source.
+struct EhFromMemory {
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return p[i]; }
+};
+#ifdef EH_A_FOLD
+struct EhAElem {
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return eh_a_elem(p, i); }
+};
+#else
+using EhAElem = EhFromMemory;
+#endif
+#ifdef EH_B_FOLD
+struct EhBElem {
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return eh_b_elem(p, i); }
+};
+#else
+using EhBElem = EhFromMemory;
+#endif
+
 // Four elements of an operand starting at (r, k) and running along its fast axis; elements
-// outside [0,R) x [0,kend) read as zero.  ALONG_K says which axis the four run along.
-template <bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
-__device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long r, long long k,
+// outside [0,R) x [0,kend) read as zero.  ALONG_K says which axis the four run along; `base`
+// is the operand's offset plus the batch offset.
+template <class ELEM, bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
+__device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long base, long long r, long long k,
                                               long long R, long long kend) {
   eh_f4v v = {0.0f, 0.0f, 0.0f, 0.0f};
   if (VEC) {
     const bool ok = (!EDGE_R || r < R) && (!EDGE_K || k < kend);
-    if (ok) v = *reinterpret_cast<const eh_f4v*>(p + r * SR + k * SK);
+    if (ok) v = *reinterpret_cast<const eh_f4v*>(p + base + r * SR + k * SK);
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const long long rr = ALONG_K ? r : r + e, kk = ALONG_K ? k + e : k;
-      if (rr < R && kk < kend) v[e] = p[rr * SR + kk * SK];
+      if (rr < R && kk < kend) v[e] = ELEM::at(p, base + rr * SR + kk * SK);
     }
   }
   return v;
@@ -154,8 +178,7 @@ EH_ENTRY(const float* __restrict__ A,
   const long long m0 = (long long)tm * BM, n0 = (long long)tn * BN;
 
   const long long bz = blockIdx.z;
-  const float* Ab = A + EH_A_OFF + bz * EH_A_BS;
-  const float* Bb = B + EH_B_OFF + bz * EH_B_BS;
+  const long long a_base = EH_A_OFF + bz * EH_A_BS, b_base = EH_B_OFF + bz * EH_B_BS;
 #if EH_SPLITK > 1
   // partial sums go to a dense [split][batch][M][N] scratch; a second launch adds them up
   const long long kbeg = (long long)blockIdx.y * KT * BK;
@@ -179,10 +202,10 @@ EH_ENTRY(const float* __restrict__ A,
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
-      ra[i] = eh_tile_load<EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(Ab, m0 + m, k0 + kq * 4, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, m0 + m, k0 + kq * 4, M, kend);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
-      ra[i] = eh_tile_load<EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(Ab, m0 + mq * 4, k0 + k, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, m0 + mq * 4, k0 + k, M, kend);
 #endif
     }
 #pragma unroll
@@ -190,10 +213,10 @@ EH_ENTRY(const float* __restrict__ A,
       const int q = tid + i * NT;
 #if EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
-      rb[i] = eh_tile_load<EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(Bb, n0 + nq * 4, k0 + k, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, n0 + nq * 4, k0 + k, N, kend);
 #else
       const int n = q / (BK / 4), kq = q % (BK / 4);
-      rb[i] = eh_tile_load<EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(Bb, n0 + n, k0 + kq * 4, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, n0 + n, k0 + kq * 4, N, kend);
 #endif
     }
   };
