@@ -51,43 +51,13 @@ def build(dev, hb, wl, name, shapes, options):
 
 
 def make_sets(dev, hb, prog, arg_names, const_inputs, arrays, nsets):
-    """`nsets` independent bindings so consecutive steps do not re-read lines
-    the previous step left in the last-level cache."""
-    sets = []
-    for _ in range(nsets):
-        named = {}
-        for b in prog.buffers:
-            if b["elided"]:
-                continue
-            if b["role"] == "temp":
-                continue                   # kept by the program itself
-            hbuf = hb.HipBuffer(dev, [b["bytes"]], None, nbytes=b["bytes"])
-            if b["name"] in arg_names:
-                hbuf.write_array(np.ascontiguousarray(arrays[arg_names.index(b["name"])]))
-            elif b["name"] in const_inputs:
-                fill = {"ones": 1.0, "zeros": 0.0, "scalar": 1.0}[const_inputs[b["name"]]]
-                hbuf.write_array(np.full(b["bytes"] // 4, fill, dtype=np.float32))
-            named[b["name"]] = hbuf
-        sets.append((prog.bind(named), named))
-    return sets
+    from harp_amd import measure
+    return measure.make_sets(dev, prog, arg_names, const_inputs, arrays, nsets)
 
 
 def time_steps(dev, hb, prog, sets, steps, warmup):
-    """W untimed steps, then exactly K steps between two events on the launch
-    stream, with a device sync on both sides.  Returns (event ms, wall ms) per step."""
-    for i in range(warmup):
-        prog.run(sets[i % len(sets)][0], sync=False)
-    dev.sync()
-    e0, e1 = hb.Event(dev), hb.Event(dev)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        prog.run(sets[i % len(sets)][0], sync=False)
-    e1.record()
-    e1.sync()
-    dev.sync()
-    wall = (time.perf_counter() - t0) * 1e3
-    return e0.elapsed_ms(e1) / steps, wall / steps
+    from harp_amd import measure
+    return measure.time_steps(dev, prog, sets, steps, warmup)
 
 
 def main():

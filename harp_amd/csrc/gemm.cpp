@@ -266,9 +266,11 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   emit_fold(fa, "EH_A_FOLD", "eh_a_elem");
   emit_fold(fb, "EH_B_FOLD", "eh_b_elem");
   {
-    // a 256-thread workgroup puts one wave on each SIMD; four resident workgroups per CU need
-    // 128 registers per lane or fewer, larger workgroups get proportionally fewer
-    int waves = opt.gemm_waves > 0 ? opt.gemm_waves : std::max(1, 4 / std::max(1, nt / 256)) * std::max(1, nt / 256);
+    // register budget: 512 lanes' registers per SIMD shared by the resident waves; a wave needs
+    // its accumulators (wm*wn/64) plus about 56 for operands, staging and addresses
+    int waves = 8;
+    while (waves > 1 && 512 / waves < t.wm * t.wn / 64 + 56) waves /= 2;
+    if (opt.gemm_waves > 0) waves = opt.gemm_waves;
     os << "#define EH_WAVES_PER_SIMD " << std::min(8, waves) << "\n";
   }
   os << "#define EH_SETPRIO " << std::max(0, std::min(3, opt.gemm_setprio)) << "\n";

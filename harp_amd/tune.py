@@ -1,0 +1,207 @@
+"""Beam search over the HIP generator's gfx950 schedule space, with the device as the estimator.
+
+The reference optimises every lowered AST with `BeamSearchOptimizer`
+(`src/opt/ast/optimizer/beam_search.rs:34-66, 235-410`): a beam of candidate ASTs, suggesters
+that propose rewrites (tiling, vectorisation, parallelisation: `src/opt/ast/suggesters/`), a
+static cost estimator (`src/opt/ast/estimator.rs`) that ranks them, stop after `max_steps` or
+when nothing improves.  This backend does not rewrite ASTs: its generator picks a schedule
+from the kernel's structure, and what remains open is the schedule's parameters.  The search
+here keeps the reference's shape -- states, suggesters proposing neighbours, a beam, early
+stop -- over that parameter space (contraction tile, wave tile, waves per SIMD, K split;
+threads and elements per row; block size, vectors per thread, streaming stores), and ranks
+states by running them: event-timed launches of the compiled Program on the GPU.
+
+    python -m harp_amd.tune --config config3_matmul [--beam 3] [--steps 4]
+
+prints the best options as the "key=value,..." string `eh_program_compile` takes.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import backend as hb
+from . import measure
+
+Options = Tuple[Tuple[str, int], ...]          # sorted (key, value) pairs: hashable state
+
+
+def _freeze(d: Dict[str, int]) -> Options:
+    return tuple(sorted(d.items()))
+
+
+def options_string(opts: Options) -> str:
+    return ",".join(f"{k}={v}" for k, v in opts)
+
+
+# -- suggesters: each proposes neighbours of a state, given the schedules the plan uses ----------
+
+GEMM_TILES = [  # (bm, bn, bk, wm, wn): macro tile, k step, wave tile; LDS 2*bk*(bm+bn+8)*4 <= 160 KiB
+    (256, 256, 16, 64, 64), (256, 256, 16, 128, 64), (256, 128, 16, 64, 64), (128, 256, 16, 64, 64),
+    (128, 128, 16, 64, 64), (128, 128, 16, 32, 64), (128, 128, 32, 64, 64), (128, 64, 16, 64, 32),
+    (64, 64, 16, 32, 32), (64, 64, 32, 32, 32),
+]
+
+
+def suggest_gemm(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """Tile shapes, register budget (waves per SIMD) and K split of the MFMA contraction."""
+    if not any(s.startswith("mfma") for s in schedules):
+        return
+    cur = tuple(state.get(k, 0) for k in ("gemm_bm", "gemm_bn", "gemm_bk", "gemm_wm", "gemm_wn"))
+    for t in GEMM_TILES:
+        if t != cur:
+            yield {**state, **dict(zip(("gemm_bm", "gemm_bn", "gemm_bk", "gemm_wm", "gemm_wn"), t))}
+    if state.get("gemm_bm", 0):
+        threads = (state["gemm_bm"] // state["gemm_wm"]) * (state["gemm_bn"] // state["gemm_wn"]) * 64
+        per_simd = max(1, threads // 256)
+        for w in (per_simd, 2 * per_simd, 4 * per_simd):
+            if w <= 8 and w != state.get("gemm_waves", 0):
+                yield {**state, "gemm_waves": w}
+        for sk in (1, 2, 4, 8):
+            if sk != state.get("gemm_split_k", 1):
+                yield {**state, "gemm_split_k": sk}
+    for p in (0, 1):
+        if p != state.get("gemm_setprio", 0):
+            yield {**state, "gemm_setprio": p}
+
+
+def suggest_row(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """Threads cooperating on a row and elements per thread of row programs."""
+    if not any(s.startswith("row(") for s in schedules):
+        return
+    for t in (32, 64, 128, 256, 512, 1024):
+        if t != state.get("row_threads", 0):
+            yield {**state, "row_threads": t}
+    for e in (4, 8, 16):
+        if e != state.get("row_elems", 8) and not state.get("row_threads", 0):
+            yield {**state, "row_elems": e}
+
+
+def suggest_flat(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """Block size and vectors per thread of flat elementwise kernels."""
+    if not any(s.startswith("flat(") for s in schedules):
+        return
+    for b in (128, 256, 512, 1024):
+        if b != state.get("flat_block", 256):
+            yield {**state, "flat_block": b}
+    for it in (1, 2, 4, 8):
+        if it != state.get("flat_iters", 4):
+            yield {**state, "flat_iters": it}
+
+
+def suggest_streaming(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """Non-temporal stores / loads for the memory-bound schedules."""
+    if not any(s.startswith(("row(", "flat(")) for s in schedules):
+        return
+    for nt in (0, 1, 2):
+        if nt != state.get("nontemporal", -1):
+            yield {**state, "nontemporal": nt}
+
+
+SUGGESTERS: List[Callable] = [suggest_gemm, suggest_row, suggest_flat, suggest_streaming]
+
+
+# -- the search --------------------------------------------------------------------------------
+
+class MeasuredEstimator:
+    """Cost of a state = event-timed milliseconds per launch of the Program compiled with it.
+    States the generator or hiprtc rejects cost infinity."""
+
+    def __init__(self, dev, prog_ast, arg_names, consts, arrays, steps=20, warmup=3, sets=2):
+        self.dev, self.ast = dev, prog_ast
+        self.arg_names, self.consts, self.arrays = arg_names, consts, arrays
+        self.steps, self.warmup, self.nsets = steps, warmup, sets
+        self.cache: Dict[Options, float] = {}
+
+    def schedules(self, opts: Options) -> List[str]:
+        return [l["schedule"] for l in hb.render_program(self.ast, dict(opts) or None).launches]
+
+    def cost(self, opts: Options) -> float:
+        if opts in self.cache:
+            return self.cache[opts]
+        try:
+            prog = hb.HipProgram(self.dev, self.ast, dict(opts) or None)
+            sets = measure.make_sets(self.dev, prog, self.arg_names, self.consts, self.arrays, self.nsets)
+            ms, _ = measure.time_steps(self.dev, prog, sets, self.steps, self.warmup)
+        except hb.EhError:
+            ms = float("inf")
+        self.cache[opts] = ms
+        return ms
+
+
+def beam_search(estimator, start: Optional[Dict[str, int]] = None, beam_width: int = 3, max_steps: int = 4,
+                no_improvement_limit: int = 1, suggesters: Sequence[Callable] = SUGGESTERS, log=None):
+    """Returns (best options, best cost, history).  history: [(step, options string, cost)]
+    for every state measured, in measurement order."""
+    first = _freeze(start or {})
+    beam = [(estimator.cost(first), first)]
+    history = [(0, options_string(first), beam[0][0])]
+    best_cost, best = beam[0]
+    stale = 0
+    seen = {first}
+    for step in range(1, max_steps + 1):
+        candidates = []
+        for _, state in beam:
+            schedules = estimator.schedules(state)
+            for sg in suggesters:
+                for nxt in sg(dict(state), schedules):
+                    f = _freeze(nxt)
+                    if f in seen:
+                        continue
+                    seen.add(f)
+                    c = estimator.cost(f)
+                    history.append((step, options_string(f), c))
+                    if log:
+                        log(f"[tune] step {step}: {options_string(f) or '(defaults)'} -> {c:.4f} ms")
+                    candidates.append((c, f))
+        if not candidates:
+            break
+        beam = sorted(beam + candidates)[:beam_width]
+        if beam[0][0] < best_cost * 0.995:
+            best_cost, best = beam[0]
+            stale = 0
+        else:
+            stale += 1
+            if stale >= no_improvement_limit:
+                break
+    return best, best_cost, history
+
+
+def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None):
+    """Searches the options of one of `workloads.CONFIGS` on device 0."""
+    from . import workloads as wl
+    default_shapes = {"config1_relu_sum": [(1024, 1024)] * 3, "config2_softmax": [(4096, 4096)],
+                      "config3_matmul": [(4096, 4096)] * 2}
+    shapes = shapes or default_shapes[name]
+    inputs_fn, graph_fn = wl.CONFIGS[name]
+    rng = np.random.default_rng(7)
+    arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
+    prog_ast, arg_names, _out, consts, _ = wl.lower_with_table(shapes, graph_fn)
+    dev = hb.HipDevice(0)
+    est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps)
+    return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--config", default="config3_matmul")
+    ap.add_argument("--beam", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=4, help="search steps (beam expansions)")
+    ap.add_argument("--launches", type=int, default=20, help="timed launches per state")
+    args = ap.parse_args(argv)
+    if hb.device_count() == 0:
+        sys.exit("tune: no HIP device present")
+    best, cost, history = tune_config(args.config, beam_width=args.beam, max_steps=args.steps,
+                                      steps=args.launches, log=lambda m: print(m, file=sys.stderr, flush=True))
+    print(json.dumps({"config": args.config, "options": options_string(best), "ms": cost,
+                      "default_ms": history[0][2], "states_measured": len(history)}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

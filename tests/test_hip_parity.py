@@ -454,3 +454,21 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
     for g, r in zip(got[:-1], ref[:-1]):
         scale = max(float(np.abs(r).max()), 1e-6)
         assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
+
+
+def test_measured_option_search(frontend, hip):
+    """One expansion of the beam search on a 512^3 matmul: every proposed state compiles or is
+    rejected cleanly, the winner is no slower than the defaults, and it computes the same C."""
+    from harp_amd import tune
+    msgs = []
+    best, cost, history = tune.tune_config("config3_matmul", shapes=[(512, 512), (512, 512)],
+                                           beam_width=2, max_steps=1, steps=10, log=msgs.append)
+    assert len(history) > 5 and history[0][1] == ""
+    assert cost <= history[0][2] * 1.02 and np.isfinite(cost)
+    rng = RNG(5)
+    a = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    b = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    got, scheds = _run_program(frontend, hip, lambda x, y: frontend.nn.matmul(x, y), [a, b], dict(best) or None)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert np.all(np.abs(got.reshape(512, 512) - exact) <= 1e-5 * scale)

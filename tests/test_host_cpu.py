@@ -240,3 +240,37 @@ def test_config4_training_step_plan(frontend):
         assert by_name[name]["elided"], name
     for src in {l["source"] for l in plan.launches}:
         assert len(hb.compile_source(src)) > 1000
+
+
+def test_option_beam_search_on_a_synthetic_cost():
+    """The schedule search without a device: suggesters propose neighbours by the schedules in
+    the plan, the beam keeps the cheapest states, the search stops when nothing improves."""
+    from harp_amd import tune
+
+    class Fake:
+        def __init__(self):
+            self.calls = 0
+
+        def schedules(self, opts):
+            return ["mfma32x32x2(tile=...)", "row(T=64)"]
+
+        def cost(self, opts):
+            self.calls += 1
+            d = dict(opts)
+            c = 10.0
+            c -= 3.0 if (d.get("gemm_bm"), d.get("gemm_bn")) == (256, 256) else 0.0
+            c -= 1.0 if d.get("gemm_waves") == 4 else 0.0
+            c -= 0.5 if d.get("row_threads") == 512 else 0.0
+            return c
+
+    est = Fake()
+    best, cost, history = tune.beam_search(est, beam_width=2, max_steps=6)
+    d = dict(best)
+    assert (d["gemm_bm"], d["gemm_bn"]) == (256, 256) and d["gemm_waves"] == 4 and d["row_threads"] == 512
+    assert cost == 5.5 and history[0] == (0, "", 10.0)
+    assert len({h[1] for h in history}) == len(history)              # no state measured twice
+    # flat-only plans get no contraction or row proposals
+    assert list(tune.suggest_gemm({}, ["flat(V=4,block=256)"])) == []
+    assert all("flat_" in k or k == "nontemporal" for sg in (tune.suggest_flat, tune.suggest_streaming)
+               for st in sg({}, ["flat(V=4,block=256)"]) for k in st)
+    assert tune.options_string(tune._freeze({"b": 2, "a": 1})) == "a=1,b=2"
