@@ -387,6 +387,177 @@ LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// outer-parallel rendering of kernels no schedule recognises (scan, scatter-add, ...)
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+struct WriteRef {
+  std::string buf;
+  const Node* index;
+};
+
+void collect_writes(const Node& n, std::vector<WriteRef>& writes, std::set<std::string>& read_bufs,
+                    std::map<std::string, int64_t>& inner_extents, bool* ok) {
+  if (n.op == Op::Store || n.op == Op::AtomicAdd || n.op == Op::AtomicMax) {
+    if (n.args[0]->op != Op::Var) *ok = false;
+    else writes.push_back({n.args[0]->name, n.args[1].get()});
+  }
+  if (n.op == Op::Load) {
+    if (n.args[0]->op == Op::Var) read_bufs.insert(n.args[0]->name);
+    else *ok = false;
+  }
+  if (n.op == Op::Range) {
+    if (n.args[0]->op != Op::Const || n.args[1]->op != Op::Const || n.args[2]->op != Op::Const) *ok = false;
+    else inner_extents[n.name] = n.args[2]->ival - n.args[0]->ival;
+  }
+  if (n.op == Op::Barrier || n.op == Op::SharedAlloc || n.op == Op::SharedStore || n.op == Op::WmmaMatmul ||
+      n.op == Op::Return)
+    *ok = false;
+  for (const auto& a : n.args) collect_writes(*a, writes, read_bufs, inner_extents, ok);
+}
+
+// True when distinct value tuples of `vars` (each 0 <= v < extent) give distinct indices:
+// sorted by |coefficient|, every coefficient exceeds the reach of all smaller ones.
+bool injective(const Affine& a, const std::vector<Loop>& vars) {
+  std::vector<std::pair<int64_t, int64_t>> ce;   // (|coef|, extent)
+  for (const auto& v : vars) {
+    if (v.extent <= 1) continue;
+    int64_t c = std::llabs(a.of(v.var));
+    if (c == 0) return false;
+    ce.push_back({c, v.extent});
+  }
+  std::sort(ce.begin(), ce.end());
+  int64_t reach = 0;
+  for (const auto& p : ce) {
+    if (p.first <= reach) return false;
+    reach += p.first * (p.second - 1);
+  }
+  return true;
+}
+
+}  // namespace
+
+// Kernels outside the canonical forms arrive as sequential loop nests for one work-item
+// (src/lowerer/lower.rs:580-735: prefix scans, zero-fill + scatter-add).  Each top-level nest
+// becomes its own launch, in order; the outer loops of a nest are spread over work-items when
+// their iterations cannot touch the same output element (every write index is affine and
+// injective in the loop variables, nothing written is read), each work-item then runs what is
+// left of the nest exactly as written, so sums keep the reference's order.  A nest that does
+// not qualify runs as written in one work-item.  Empty result: the kernel has a form this
+// does not cover (shape variables, hand-placed group/local ids, shared memory).
+std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOptions& opt) {
+  std::vector<LaunchSpec> out;
+  if (k.op != Op::Kernel) return out;
+  for (const auto& p : k.params)
+    if (p.kind != VarKind::Normal || !p.dtype.is_ptr()) return {};
+  for (int i = 0; i < 3; ++i) {
+    if (k.grid.size() == 3 && const_int(*k.grid[i], 1) != 1) return {};
+    if (k.tg.size() == 3 && const_int(*k.tg[i], 1) != 1) return {};
+  }
+  const Node& body = *k.args[0];
+  std::vector<const Node*> tops;
+  if (body.op == Op::Block) {
+    if (!body.decls.empty()) return {};
+    for (const auto& a : body.args) tops.push_back(a.get());
+  } else {
+    tops.push_back(&body);
+  }
+  if (tops.empty()) return {};
+  // buffers written anywhere in the kernel must not be read by a nest that is spread out
+  std::set<std::string> written_anywhere;
+  {
+    std::vector<WriteRef> w;
+    std::set<std::string> r;
+    std::map<std::string, int64_t> e;
+    bool ok = true;
+    collect_writes(body, w, r, e, &ok);
+    if (!ok) return {};
+    for (const auto& x : w) written_anywhere.insert(x.buf);
+  }
+  std::string sig;
+  std::vector<std::string> arg_bufs;
+  for (const auto& p : k.params) {
+    sig += (sig.empty() ? "" : ", ") + std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + p.name;
+    arg_bufs.push_back(p.name);
+  }
+  bool any_parallel = false;
+  for (size_t t = 0; t < tops.size(); ++t) {
+    if (tops[t]->op != Op::Range) return {};
+    // the perfect nest at the top of this statement
+    std::vector<Loop> loops;
+    const Node* cur = tops[t];
+    while (cur->op == Op::Range && cur->args[0]->op == Op::Const && cur->args[0]->ival == 0 &&
+           cur->args[1]->op == Op::Const && cur->args[1]->ival == 1 && cur->args[2]->op == Op::Const &&
+           cur->args[2]->ival >= 1) {
+      loops.push_back({cur->name, cur->args[2]->ival});
+      const Node* b = cur->args[3].get();
+      if (b->op == Op::Block && b->decls.empty() && b->args.size() == 1) b = b->args[0].get();
+      cur = b;
+      if (cur->op != Op::Range) break;
+    }
+    const Node* inner = cur;
+    if (loops.empty()) return {};
+    if (inner->op == Op::Range) {
+      // the walk stopped at a loop it cannot spread (non-constant bounds): keep it inside
+    }
+    std::vector<WriteRef> writes;
+    std::set<std::string> reads;
+    std::map<std::string, int64_t> inner_extents;
+    bool ok = true;
+    collect_writes(*inner, writes, reads, inner_extents, &ok);
+    if (!ok) return {};
+    bool spread = !writes.empty();
+    for (const auto& r : reads) spread = spread && !written_anywhere.count(r);
+    for (const auto& w : writes) {
+      auto a = affine_of(*w.index);
+      if (!a) { spread = false; break; }
+      std::vector<Loop> vars = loops;
+      for (const auto& kv : a->coef)
+        if (kv.second != 0) {
+          bool is_outer = false;
+          for (const auto& l : loops) is_outer = is_outer || l.var == kv.first;
+          if (is_outer) continue;
+          auto ie = inner_extents.find(kv.first);
+          if (ie == inner_extents.end()) { spread = false; break; }
+          vars.push_back({kv.first, ie->second});
+        }
+      if (!spread || !injective(*a, vars)) { spread = false; break; }
+    }
+    LaunchSpec ls;
+    ls.entry = k.name + "_n" + std::to_string(t);
+    ls.kernels = {k.name};
+    ls.arg_bufs = arg_bufs;
+    std::ostringstream os;
+    os << hdr(opt) << kAtomicMaxF32;
+    StmtRenderer sr;
+    if (spread) {
+      int64_t total = 1;
+      for (const auto& l : loops) total *= l.extent;
+      if (total >= (int64_t{1} << 40)) return {};
+      os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << sig << ") {\n";
+      os << "  long long eh_r = (long long)blockIdx.x * 256 + threadIdx.x;\n  if (eh_r >= " << total << "ll) return;\n";
+      for (size_t i = loops.size(); i-- > 0;) {
+        os << "  const long long " << loops[i].var << " = eh_r % " << loops[i].extent << ";\n";
+        if (i) os << "  eh_r /= " << loops[i].extent << ";\n";
+      }
+      os << sr.stmt(*inner) << "}\n";
+      ls.grid[0] = static_cast<unsigned>((total + 255) / 256);
+      ls.block[0] = 256;
+      ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + ")";
+      any_parallel = true;
+    } else {
+      os << "extern \"C\" __global__ void " << ls.entry << "(" << sig << ") {\n" << sr.stmt(*tops[t]) << "}\n";
+      ls.schedule = "as-written";
+    }
+    ls.source = os.str();
+    out.push_back(std::move(ls));
+  }
+  if (!any_parallel) return {};
+  return out;
+}
+
+// ---------------------------------------------------------------------------------------------
 // canonical stages and grouping
 // ---------------------------------------------------------------------------------------------
 
@@ -737,7 +908,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       continue;
     }
     if (!nests[i]) {
-      plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+      auto spread = render_kernel_outer_parallel(*kernels[i], opt);
+      if (spread.empty()) plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+      else for (auto& ls : spread) plan.launches.push_back(std::move(ls));
       ++i;
       continue;
     }

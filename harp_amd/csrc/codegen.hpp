@@ -60,6 +60,10 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt);
 // already carries group/local id parameters).  Used for forms no schedule recognises.
 LaunchSpec render_kernel_as_written(const Node& kernel, const GenOptions& opt);
 
+// One launch per top-level loop nest of such a kernel, the outer loops of a nest spread over
+// work-items where their iterations cannot collide; empty when the kernel's form is not covered.
+std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& kernel, const GenOptions& opt);
+
 // Expression text in HIP C (math calls, literals); exposed for tests.
 std::string render_expr_text(const Node& e);
 

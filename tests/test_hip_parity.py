@@ -472,3 +472,35 @@ def test_measured_option_search(frontend, hip):
     exact = a.astype(np.float64) @ b.astype(np.float64)
     scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
     assert np.all(np.abs(got.reshape(512, 512) - exact) <= 1e-5 * scale)
+
+
+SPREAD_FORMS = {
+    # name: (shape, graph, schedule expected somewhere in the plan, sums keep the oracle's order)
+    "cumsum_rows": ((300, 257), lambda t: t.cumsum(1), "outer-parallel(work-items=300)"),
+    # as lowered, the accumulator of a mid-axis scan runs on over the inner axis too: only axis 0 is free
+    "cumprod_mid": ((6, 50, 9), lambda t: t.cumprod(1), "outer-parallel(work-items=6)"),
+    "cummax_rows": ((128, 1000), lambda t: t.cummax(1), "outer-parallel(work-items=128)"),
+    "fold_tiles": ((64, 96), lambda t: t.unfold([0, 1], [2, 3], [2, 3], [1, 1])
+                   .fold([64, 96], [0, 1], [2, 3], [2, 3], [1, 1]), "outer-parallel(work-items=6144)"),
+    "fold_overlapping": ((20, 30), lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1])
+                         .fold([20, 30], [0, 1], [3, 3], [1, 1], [1, 1]), "as-written"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(SPREAD_FORMS))
+def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
+    """Prefix scans run one work-item per scanned line, scatter-adds one per element where
+    windows do not overlap (else as written, one work-item): bit-exact with the oracle either
+    way, because every sum keeps the sequential order (running sums and products are held to
+    the reduction tolerance, as everywhere)."""
+    shape, fn, expect = SPREAD_FORMS[name]
+    x = RNG(len(name)).uniform(0.5, 1.5, shape).astype(np.float32)
+    t = frontend.Tensor.input(list(shape))
+    prog, _, _ = frontend.lower_graph([fn(t).graph])
+    scheds = [l["schedule"] for l in hip.render_program(prog).launches]
+    assert expect in scheds, scheds
+    ref, got = both(frontend, fn, [x], False)
+    if name.startswith(("cumsum", "cumprod")):       # the C compiler may contract or reorder: reduction class
+        assert np.allclose(got, ref, rtol=1e-6)
+    else:
+        assert bits_equal_mod_zero(ref, got)

@@ -83,7 +83,7 @@ def test_unfused_per_kernel_rendering(frontend):
         assert len(hb.compile_source(plan.launches[0]["source"])) > 500
 
 
-def test_as_written_rendering_of_scatter_and_scan(frontend):
+def test_rendering_of_scatter_and_scan(frontend):
     from harp_amd import backend as hb
     x = frontend.Tensor.input([4, 4])
     y = x.unfold([0, 1], [2, 2], [2, 2], [1, 1]).fold([4, 4], [0, 1], [2, 2], [2, 2], [1, 1])
@@ -91,13 +91,23 @@ def test_as_written_rendering_of_scatter_and_scan(frontend):
     names = [k.attrs["name"] for k in prog.args]
     assert names[0].startswith("C_") and names[1].startswith("S_")
     plan = hb.render_program(prog)
-    assert plan.launches[1]["schedule"] == "as-written" and "atomicAdd" in plan.launches[1]["source"]
+    # zero-fill and scatter-add nests become two launches; tiling windows cannot collide, so
+    # both are spread over work-items (16 outputs, 16 window slots)
+    assert [l["schedule"] for l in plan.launches[1:]] == ["outer-parallel(work-items=16)"] * 2
+    assert "atomicAdd" in plan.launches[2]["source"]
     for l in plan.launches:
         hb.compile_source(l["source"])
+    # overlapping windows could collide: that nest stays one work-item, as written
+    z = x.unfold([0, 1], [2, 2], [1, 1], [1, 1]).fold([4, 4], [0, 1], [2, 2], [1, 1], [1, 1])
+    plan_z = hb.render_program(frontend.lower_graph([z.graph])[0])
+    assert [l["schedule"] for l in plan_z.launches[1:]] == ["outer-parallel(work-items=16)", "as-written"]
     prog2, _, _ = frontend.lower_graph([x.cumsum(1).graph])
     plan2 = hb.render_program(prog2)
-    assert plan2.launches[0]["schedule"] == "as-written"
+    assert plan2.launches[0]["schedule"] == "outer-parallel(work-items=4)"
     hb.compile_source(plan2.launches[0]["source"])
+    # a scan over axis 0 is lowered with one accumulator for the whole tensor: nothing to spread
+    plan3 = hb.render_program(frontend.lower_graph([x.cummax(0).graph])[0])
+    assert plan3.launches[0]["schedule"] == "as-written"
 
 
 @pytest.mark.parametrize("text,needle", [
