@@ -2,7 +2,7 @@
 """Benchmark of the eclat kernel path on one MI355X.
 
 A step is one pass of the hot path (execute the compiled Program) over one batch
-of synthetic input.  The headline workload is BASELINE config 2 -- row softmax of
+of synthetic input.  The headline workload is benchmark configuration 2 -- row softmax of
 fp32 [4096, 4096], compiled from the reference's five-kernel lowering into one
 fused launch -- reported as HBM GB/s of algorithmic traffic (one read + one
 write).  The same JSON line carries config 3 (4096^3 fp32 matmul, TFLOP/s on the
@@ -305,6 +305,20 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
                 "sample": f"batch {sub} of 8192 through the same lowered kernels, unfused "
                           f"(gcc -O3 -ffast-math), median of {reps_p} passes, {sec_p * 1e3:.0f} ms/pass"}
             log(f"[bench] cpu baseline mlp: {sub / sec_p:.2f} samples/s (1 core, batch {sub})")
+
+        if cnn is not None:
+            from harp_amd.frontend import exact_mode
+            sub = 64
+            sizes = wl.cnn_sizes(True)
+            arrays = wl.config5_inputs(sub, *sizes[1:])
+            with exact_mode():
+                sec_c, reps_c, _ = baseline.time_graph(lambda *ts: wl.config5_graph(*ts), arrays,
+                                                       min_seconds=4.0, max_reps=10)
+            result_extra["cpu_baseline_cnn"] = {
+                "value": sub / sec_c, "unit": "images/s", "cores": 1, "kind": "port",
+                "sample": f"batch {sub} of 256 through the same lowered kernels, unfused "
+                          f"(gcc -O3 -ffast-math), median of {reps_c} passes, {sec_c * 1e3:.0f} ms/pass"}
+            log(f"[bench] cpu baseline cnn: {sub / sec_c:.1f} images/s (1 core, batch {sub})")
 
     head = softmax
     out = {

@@ -1,4 +1,4 @@
-"""The BASELINE configurations as front-end graphs with seeded synthetic inputs.
+"""The benchmark configurations as front-end graphs with seeded synthetic inputs.
 
 Used by the benchmark, the smoke check and the parity tests so that all three
 run the same graphs on the same data.

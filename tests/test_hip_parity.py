@@ -107,7 +107,7 @@ def test_softmax_and_log_softmax(frontend, hip, shape, fuse):
 
 @pytest.mark.parametrize("fuse", [False, True])
 def test_config1_fused_elementwise_reduce(frontend, hip, fuse):
-    """BASELINE config 1: s = sum(relu(a*b + c), -1), fp32 [1024,1024], N(0,1)."""
+    """benchmark configuration 1: s = sum(relu(a*b + c), -1), fp32 [1024,1024], N(0,1)."""
     rng = RNG(1234)
     a, b, c = (rng.normal(0, 1, (1024, 1024)).astype(np.float32) for _ in range(3))
     ref, got = both(frontend, lambda x, y, z: frontend.nn.relu(x * y + z).sum(1), [a, b, c], fuse)
@@ -116,7 +116,7 @@ def test_config1_fused_elementwise_reduce(frontend, hip, fuse):
 
 
 def test_config2_row_softmax_full_size(frontend, hip):
-    """BASELINE config 2: row softmax of fp32 [4096,4096], N(0, std 2)."""
+    """benchmark configuration 2: row softmax of fp32 [4096,4096], N(0, std 2)."""
     x = RNG(1235).normal(0, 2, (4096, 4096)).astype(np.float32)
     ref, got = both(frontend, lambda t: frontend.nn.softmax(t, 1), [x])
     assert np.allclose(got, ref, rtol=1e-5, atol=1e-12)
@@ -149,7 +149,7 @@ def test_linear_layer(frontend, hip, batch, kin, kout):
 
 
 def test_config3_matmul_4096(frontend, hip):
-    """BASELINE config 3: C = A@B, fp32 4096^3, U(-1,1).  The C oracle runs a row subset
+    """benchmark configuration 3: C = A@B, fp32 4096^3, U(-1,1).  The C oracle runs a row subset
     (64 rows of A, 2 GFLOP); float64 numpy covers every row."""
     rng = RNG(1236)
     a = rng.uniform(-1, 1, (4096, 4096)).astype(np.float32)
@@ -271,7 +271,7 @@ def _train_step_on(fe, kind, arrays, fuse=True):
 @pytest.mark.parametrize("batch,dims", [(64, (32, 64, 64, 32)), (256, (128, 256, 128, 128)), (50, (12, 20, 12))])
 @pytest.mark.parametrize("fuse", [False, True])
 def test_config4_mlp_training_step(frontend, hip, batch, dims, fuse):
-    """BASELINE config 4 at oracle-sized shapes: every updated parameter and the loss match
+    """benchmark configuration 4 at oracle-sized shapes: every updated parameter and the loss match
     the C oracle running the same graph; the step also matches a float64 numpy MLP."""
     from harp_amd import workloads as wl
     arrays = wl.config4_inputs(batch, dims, seed=99)
@@ -334,7 +334,7 @@ def _cnn_step_on(fe, kind, arrays, fuse=True):
 @pytest.mark.parametrize("sizes", [(4, 8, 4, 8, 16, 10), (8, 28, 32, 64, 128, 10)])
 @pytest.mark.parametrize("fuse", [False, True])
 def test_config5_cnn_training_step(frontend, hip, sizes, fuse):
-    """BASELINE config 5 (second case: the real channel/image sizes at batch 8): every
+    """benchmark configuration 5 (second case: the real channel/image sizes at batch 8): every
     parameter gradient and the loss match the C oracle running the same exact-mode graph,
     and a float64 numpy CNN."""
     from harp_amd import workloads as wl

@@ -1,5 +1,5 @@
 """Host-side checks that need no GPU: the C ABI exports what the header declares, the AST
-reader, the renderer's schedules for the BASELINE configs, hiprtc compilation for gfx950,
+reader, the renderer's schedules for the benchmark configurations, hiprtc compilation for gfx950,
 and the front end's lowering structure."""
 
 import os
