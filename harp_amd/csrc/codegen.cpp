@@ -712,6 +712,28 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan);
 }  // namespace
 
+// Row-major strides of a kernel's loops when its output index is exactly the dense linear index
+// of those loops (coefficient of each live loop = product of the inner extents, no offset).
+std::optional<std::vector<int64_t>> dense_strides(const NestKernel& k, int64_t* numel) {
+  if (!k.out_aff || k.out_aff->c != 0) return std::nullopt;
+  int64_t stride = 1;
+  std::vector<int64_t> strides(k.loops.size(), 0);
+  for (size_t i = k.loops.size(); i-- > 0;) {
+    const Loop& l = k.loops[i];
+    if (l.extent <= 0) return std::nullopt;
+    strides[i] = stride;
+    if (l.extent > 1 && k.out_aff->of(l.var) != stride) return std::nullopt;
+    stride *= l.extent;
+  }
+  for (const auto& kv : k.out_aff->coef) {
+    bool live = false;
+    for (const auto& l : k.loops) live = live || (l.var == kv.first && l.extent > 1);
+    if (kv.second != 0 && !live) return std::nullopt;
+  }
+  *numel = stride;
+  return strides;
+}
+
 // An elementwise kernel as a function of the linear index of its (dense, row-major) output, for
 // contractions that evaluate it in their tile loader.  Only kernels reading one f32 buffer.
 std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems) {
@@ -917,12 +939,134 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     const NestKernel& k0 = *nests[i];
     // contraction (matmul-shaped reduce) -> MFMA schedule
     if (k0.rkind == ReduceKind::Sum && opt.gemm) {
-      auto gl = try_emit_gemm(k0, opt, &plan.buffers, &folded);
+      // elementwise kernels that follow over the same dense index space and feed on the
+      // result become the contraction's epilogue
+      EpilogueSpec epi;
+      size_t after = i + 1;
+      bool have_epi = false;
+      if (opt.gemm_epilogue && opt.fuse && have_table && gemm_shaped(k0, opt)) {
+        auto gs = match_gemm(k0);
+        if (gs && gemm_output_dense(*gs)) {
+          const int64_t total = gs->batch * gs->M * gs->N;
+          const bool small = total < (int64_t{1} << 30);
+          std::map<std::string, DType> avail;          // values held in registers: C and stage outputs
+          avail[k0.out_buf] = k0.out_dtype;
+          std::vector<size_t> taken;
+          size_t j = i + 1;
+          for (; j < kernels.size(); ++j) {
+            if (!nests[j] || folded_kernels.count(j) || nests[j]->rkind != ReduceKind::None) break;
+            const NestKernel& sk = *nests[j];
+            int64_t numel = 0;
+            auto strides = dense_strides(sk, &numel);
+            if (!strides || numel != total || avail.count(sk.out_buf)) break;
+            std::vector<LoadRef> loads;
+            collect_loads(*sk.value, loads);
+            bool feeds = false, ok = true;
+            for (const auto& lr : loads) {
+              if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
+              if (!avail.count(lr.load->args[0]->name)) continue;
+              auto a = affine_of(*lr.load->args[1]);
+              if (!a || !(*a == *sk.out_aff)) { ok = false; break; }   // must read the element it is computing
+              feeds = true;
+            }
+            if (!ok || !feeds) break;
+            avail[sk.out_buf] = sk.out_dtype;
+            taken.push_back(j);
+          }
+          if (!taken.empty()) {
+            after = taken.back() + 1;
+            auto needed = [&](const std::string& buf) {
+              if (role_of(buf) != "temp") return true;
+              for (size_t r : readers[buf])
+                if (r <= i || r >= after) return true;
+              return false;
+            };
+            std::ostringstream fn, body;
+            std::vector<std::string> ext_order;
+            std::map<std::string, std::pair<std::string, size_t>> ext;   // name -> (declaration, min bytes)
+            epi.store_c = needed(k0.out_buf);
+            if (!epi.store_c) plan.elided.insert(k0.out_buf);
+            const std::string IT = small ? "int" : "long long";
+            body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
+            body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
+            if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
+            for (size_t j2 : taken) {
+              const NestKernel& sk = *nests[j2];
+              int64_t numel = 0;
+              auto strides = *dense_strides(sk, &numel);
+              epi.kernels.push_back(sk.name);
+              body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
+              for (size_t li = 0; li < sk.loops.size(); ++li) {
+                const Loop& l = sk.loops[li];
+                if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
+                else body << "    const " << IT << " " << l.var << " = (eh_l / " << strides[li] << ") % " << l.extent << ";\n";
+              }
+              ExprRenderer er;
+              er.load_hook = [&](const Node& ld, std::string* out) {
+                const std::string& b = ld.args[0]->name;
+                if (!avail.count(b)) return false;
+                *out = "eh_v_" + b;
+                return true;
+              };
+              std::vector<LoadRef> loads;
+              collect_loads(*sk.value, loads);
+              for (const auto& lr : loads) {
+                const std::string& b = lr.load->args[0]->name;
+                if (avail.count(b) || ext.count(b)) {
+                  if (ext.count(b) && !lr.guarded) {
+                    if (auto a = affine_of(*lr.load->args[1]))
+                      ext[b].second = std::max(ext[b].second, static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) *
+                                                                   lr.load->dtype.itemsize());
+                  }
+                  continue;
+                }
+                size_t mb = 0;
+                if (!lr.guarded)
+                  if (auto a = affine_of(*lr.load->args[1]))
+                    mb = static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) * lr.load->dtype.itemsize();
+                DType et = lr.load->dtype;
+                for (const auto& pp : sk.params)
+                  if (pp.name == b) et = pp.dtype.elem();
+                ext[b] = {"const " + ctype(et) + "* __restrict__ " + b, mb};
+                ext_order.push_back(b);
+                epi.bytes += static_cast<double>(elems.count(b) ? elems.at(b) : 0) * et.itemsize();
+              }
+              body << "    eh_v_" << sk.out_buf << " = (" << ctype(sk.out_dtype) << ")(" << er.expr(*sk.value) << ");\n";
+              if (needed(sk.out_buf)) {
+                body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
+                ext[sk.out_buf] = {ctype(sk.out_dtype) + "* __restrict__ " + sk.out_buf,
+                                   static_cast<size_t>(total) * sk.out_dtype.itemsize()};
+                ext_order.push_back(sk.out_buf);
+                epi.bytes += static_cast<double>(total) * sk.out_dtype.itemsize();
+              } else {
+                plan.elided.insert(sk.out_buf);
+              }
+              body << "  }\n";
+            }
+            for (const auto& b : ext_order) {
+              epi.params += ", " + ext[b].first;
+              epi.args += ", " + b;
+              epi.bufs.push_back(b);
+              epi.min_bytes.push_back(ext[b].second);
+            }
+            fn << "// what kernels";
+            for (const auto& n : epi.kernels) fn << " " << n;
+            fn << " do to element eh_e of " << k0.out_buf << "\n";
+            fn << "__device__ __forceinline__ void eh_epilogue(long long eh_e, float eh_acc"
+               << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params
+               << ") {\n" << body.str() << "}\n";
+            epi.function = fn.str();
+            have_epi = true;
+          }
+        }
+      }
+      auto gl = try_emit_gemm(k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
       if (!gl.empty()) {
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
-        ++i;
+        i = have_epi ? after : i + 1;
         continue;
       }
+      if (have_epi) throw Error("internal: contraction '" + k0.name + "' matched but could not be emitted");
     }
     if (k0.rkind != ReduceKind::None && !reduce_is_rowwise(k0)) {
       emit_serial_reduce(k0, opt, &plan);

@@ -199,6 +199,10 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
   return s;
 }
 
+bool gemm_output_dense(const GemmShape& s) {
+  return s.c_off == 0 && s.c_n == 1 && s.c_m == s.N && (s.batch == 1 || s.c_b == s.M * s.N);
+}
+
 bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
   auto s = match_gemm(k);
   Choice c;
@@ -206,7 +210,7 @@ bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
 }
 
 std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers,
-                                      const FoldMap* folded) {
+                                      const FoldMap* folded, const EpilogueSpec* epilogue) {
   auto s = match_gemm(k);
   Choice ch;
   if (!s || !choose(*s, opt, &ch)) return {};
@@ -263,6 +267,13 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     for (size_t at = text.find(ph); at != std::string::npos; at = text.find(ph, at)) text.replace(at, ph.size(), fn);
     os << "#define " << macro << " 1\n" << text;
   };
+  const bool epi_here = epilogue && S == 1;     // with K split the epilogue runs in the summing launch
+  if (epi_here) {
+    os << "#define EH_EPILOGUE 1\n#define EH_EPI_PARAMS " << epilogue->params << "\n#define EH_EPI_ARGS " << epilogue->args
+       << "\n";
+    if (!epilogue->store_c) os << "#define EH_NO_C 1\n";
+    os << epilogue->function;
+  }
   emit_fold(fa, "EH_A_FOLD", "eh_a_elem");
   emit_fold(fb, "EH_B_FOLD", "eh_b_elem");
   {
@@ -281,7 +292,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
                 (fa ? "/folded" : a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") +
                 (fb ? "/folded" : b_vec ? "" : "/scalar") +
-                (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") + ")";
+                (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
+                (epi_here ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
   ls.grid[1] = static_cast<unsigned>(S);
   ls.grid[2] = static_cast<unsigned>(s->batch);
@@ -289,12 +301,22 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   const size_t c_elems =
       static_cast<size_t>(s->c_off + (s->M - 1) * s->c_m + (s->N - 1) * s->c_n + (s->batch - 1) * s->c_b + 1);
   const size_t part_elems = static_cast<size_t>(S) * static_cast<size_t>(s->batch * s->M * s->N);
-  ls.arg_bufs = {fa ? fa->src : s->a_buf, fb ? fb->src : s->b_buf, S > 1 ? scratch : s->c_buf};
+  ls.arg_bufs = {fa ? fa->src : s->a_buf, fb ? fb->src : s->b_buf};
   // a folded operand binds the producer's source, whose size the buffer table already fixes
   ls.arg_min_bytes = {
       fa ? 0 : 4 * static_cast<size_t>(s->a_off + (s->M - 1) * s->a_m + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
-      fb ? 0 : 4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1),
-      4 * (S > 1 ? part_elems : c_elems)};
+      fb ? 0 : 4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1)};
+  if (!(epi_here && !epilogue->store_c)) {
+    ls.arg_bufs.push_back(S > 1 ? scratch : s->c_buf);
+    ls.arg_min_bytes.push_back(4 * (S > 1 ? part_elems : c_elems));
+  }
+  if (epi_here) {
+    for (size_t i = 0; i < epilogue->bufs.size(); ++i) {
+      ls.arg_bufs.push_back(epilogue->bufs[i]);
+      ls.arg_min_bytes.push_back(epilogue->min_bytes[i]);
+    }
+    for (const auto& n : epilogue->kernels) ls.kernels.push_back(n);
+  }
   ls.flops = 2.0 * static_cast<double>(s->M) * static_cast<double>(s->N) * static_cast<double>(s->K) *
              static_cast<double>(s->batch);
   {
@@ -304,7 +326,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     double b_bytes = 4.0 * static_cast<double>(s->K) * s->N * (s->b_b == 0 ? 1.0 : nb);
     if (fa && fa->src_bytes > 0) a_bytes = fa->src_bytes;
     if (fb && fb->src_bytes > 0) b_bytes = fb->src_bytes;
-    ls.algo_bytes = a_bytes + b_bytes + 4.0 * nb * static_cast<double>(s->M) * s->N;
+    const double c_bytes = 4.0 * nb * static_cast<double>(s->M) * s->N;
+    ls.algo_bytes = a_bytes + b_bytes + (epilogue && !epilogue->store_c ? 0.0 : c_bytes) + (epilogue ? epilogue->bytes : 0.0);
   }
   if (S > 1) {
     BufferInfo sb;
@@ -321,17 +344,36 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     const int64_t total = s->batch * s->M * s->N;
     fin.grid[0] = static_cast<unsigned>(ceil_div(total, 256));
     fin.block[0] = 256;
-    fin.arg_bufs = {scratch, s->c_buf};
-    fin.arg_min_bytes = {4 * part_elems, 4 * c_elems};
+    const bool fin_c = !(epilogue && !epilogue->store_c);
+    fin.arg_bufs = {scratch};
+    fin.arg_min_bytes = {4 * part_elems};
+    if (fin_c) {
+      fin.arg_bufs.push_back(s->c_buf);
+      fin.arg_min_bytes.push_back(4 * c_elems);
+    }
     std::ostringstream fs;
     fs << "// generated for gfx950 by eclat backend-hip: sum of split-K partial tiles\n";
-    fs << "extern \"C\" __global__ void __launch_bounds__(256) " << fin.entry
-       << "(const float* __restrict__ P, float* __restrict__ C) {\n";
+    if (epilogue) {
+      fs << "#ifndef __HIPCC_RTC__\n#include <hip/hip_runtime.h>\n#endif\n" << epilogue->function;
+      for (size_t i = 0; i < epilogue->bufs.size(); ++i) {
+        fin.arg_bufs.push_back(epilogue->bufs[i]);
+        fin.arg_min_bytes.push_back(epilogue->min_bytes[i]);
+      }
+      for (const auto& n : epilogue->kernels) fin.kernels.push_back(n);
+      fin.schedule = "split-k-final(chunks=" + std::to_string(S) + ",epilogue=" + std::to_string(epilogue->kernels.size()) + ")";
+    }
+    fs << "extern \"C\" __global__ void __launch_bounds__(256) " << fin.entry << "(const float* __restrict__ P"
+       << (fin_c ? ", float* __restrict__ C" : "") << (epilogue ? epilogue->params : std::string()) << ") {\n";
     fs << "  const long long o = (long long)blockIdx.x * 256 + threadIdx.x;\n  if (o >= " << total << "LL) return;\n";
     fs << "  float acc = 0.0f;\n  for (int s = 0; s < " << S << "; ++s) acc += P[(long long)s * " << total << "LL + o];\n";
     fs << "  const long long n = o % " << s->N << "LL, m = (o / " << s->N << "LL) % " << s->M << "LL, b = o / "
        << (s->M * s->N) << "LL;\n";
-    fs << "  C[" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n << "LL] = acc;\n}\n";
+    if (epilogue) {
+      // the epilogue is written for dense C: element o is (b*M + m)*N + n
+      fs << "  (void)n; (void)m; (void)b;\n  eh_epilogue(o, acc" << (epilogue->store_c ? ", C" : "") << epilogue->args << ");\n}\n";
+    } else {
+      fs << "  C[" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n << "LL] = acc;\n}\n";
+    }
     fin.source = fs.str();
   }
   return out;

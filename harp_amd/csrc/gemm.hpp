@@ -38,6 +38,25 @@ struct FoldedOperand {
 };
 using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer
 
+// Elementwise kernels that follow a contraction over the same dense index space, run on each
+// output element while it is still in the accumulator (bias, activation, saved intermediates).
+// `function` is the text of
+//   __device__ void eh_epilogue(long long eh_e, float eh_acc <params>)
+// which stores whatever has to reach memory, C itself included when `store_c`.
+struct EpilogueSpec {
+  std::string function;
+  std::string params;                  // ", const float* __restrict__ buf3, float* __restrict__ buf9"
+  std::string args;                    // ", buf3, buf9"
+  std::vector<std::string> bufs;       // the extra parameters' buffers, in order
+  std::vector<size_t> min_bytes;
+  std::vector<std::string> kernels;    // names of the kernels taken in
+  bool store_c = true;
+  double bytes = 0;                    // algorithmic bytes of the extra parameters
+};
+
+// True when element (b, m, n) of C sits at (b*M + m)*N + n, the index an epilogue is written for.
+bool gemm_output_dense(const GemmShape& s);
+
 // Recognises the contraction and returns its strides; nullopt otherwise.
 std::optional<GemmShape> match_gemm(const NestKernel& k);
 
@@ -48,6 +67,6 @@ bool gemm_shaped(const NestKernel& k, const GenOptions& opt);
 // covers (the caller then falls back to another schedule).  One launch, or two when K is
 // split: partial tiles into a scratch buffer appended to `buffers`, then their sum.
 std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers,
-                                      const FoldMap* folded = nullptr);
+                                      const FoldMap* folded = nullptr, const EpilogueSpec* epilogue = nullptr);
 
 }  // namespace eh

@@ -149,14 +149,27 @@ using ATile = EhTile<EH_A_KCONTIG != 0, AS>;
 using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
 }  // namespace
 
+// Epilogue: elementwise kernels that follow the contraction over the same dense index space
+// run on each element while it is in the accumulator; eh_epilogue stores what must reach memory
+// (C itself only if something else still reads it: EH_NO_C drops the parameter).
+#ifndef EH_EPILOGUE
+#define EH_EPI_PARAMS
+#define EH_EPI_ARGS
+#endif
+#ifdef EH_NO_C
+#define EH_C_PARAM
+#define EH_C_ARG
+#else
+#define EH_C_PARAM , float* __restrict__ C
+#define EH_C_ARG , C
+#endif
+
 #ifndef EH_WAVES_PER_SIMD
 #define EH_WAVES_PER_SIMD 4   // register budget: 512 / this many VGPRs+AGPRs per lane
 #endif
 
 extern "C" __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(EH_WAVES_PER_SIMD, EH_WAVES_PER_SIMD)))
-EH_ENTRY(const float* __restrict__ A,
-                                                          const float* __restrict__ B,
-                                                          float* __restrict__ C) {
+EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_EPI_PARAMS) {
   __shared__ __attribute__((aligned(16))) float As[2][BK * AS];
   __shared__ __attribute__((aligned(16))) float Bs[2][BK * BS];
 
@@ -185,6 +198,8 @@ EH_ENTRY(const float* __restrict__ A,
   const long long kend = (kbeg + (long long)KT * BK) < K ? (kbeg + (long long)KT * BK) : K;
   float* Cb = C + ((long long)blockIdx.y * EH_BATCH + bz) * (M * N);
   constexpr long long CSM = N, CSN = 1;
+#elif defined(EH_EPILOGUE)
+  const long long kbeg = 0, kend = K;
 #else
   const long long kbeg = 0, kend = K;
   float* Cb = C + EH_C_OFF + bz * EH_C_BS;
@@ -312,6 +327,12 @@ EH_ENTRY(const float* __restrict__ A,
       for (int r = 0; r < 16; ++r) {
         const long long row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
         const long long col = n0 + wn * WN + j * 32 + l32;
-        if ((!EDGE_M || row < M) && (!EDGE_N || col < N)) Cb[row * CSM + col * CSN] = acc[i][j][r];
+        if ((!EDGE_M || row < M) && (!EDGE_N || col < N)) {
+#if defined(EH_EPILOGUE) && EH_SPLITK == 1
+          eh_epilogue((bz * M + row) * N + col, acc[i][j][r] EH_C_ARG EH_EPI_ARGS);
+#else
+          Cb[row * CSM + col * CSN] = acc[i][j][r];
+#endif
+        }
       }
 }

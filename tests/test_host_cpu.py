@@ -244,6 +244,12 @@ def test_config4_training_step_plan(frontend):
     scheds = [l["schedule"] for l in plan.launches]
     assert sum(s.startswith("mfma32x32x2(") for s in scheds) == 8      # 3 forward, 3 dW, 2 dX
     assert sum("-reduce(" in s for s in scheds) == 3                   # bias gradients (column sums)
+    # bias add and activation chains ride on the forward contractions' accumulators
+    epi = [l for l in plan.launches if "epilogue=" in l["schedule"]]
+    assert len(epi) >= 3 and all("eh_epilogue(" in l["source"] for l in epi)
+    assert any(len(l["kernels"]) >= 6 for l in epi)
+    off = hb.render_program(prog_ast, {"gemm_epilogue": 0})
+    assert not any("epilogue=" in l["schedule"] for l in off.launches) and len(off.launches) > len(plan.launches)
     by_name = {b["name"]: b for b in plan.buffers}
     assert by_name[outs[-1]]["bytes"] == 4 and by_name[outs[-1]]["role"] == "output"   # scalar loss
     for name in consts:
