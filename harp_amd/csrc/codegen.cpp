@@ -805,6 +805,60 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   return f;
 }
 
+// C of contraction `g` is dense; consumer `sk` (dense output) reads it at `read` (affine over
+// sk's loops), a bijection between the two index spaces.  Returns g's output index rewritten
+// so that each element lands at the consumer's own linear index, or nullopt when the consumer's
+// loops do not regroup into g's loops.
+std::optional<Affine> relayout(const NestKernel& g, const NestKernel& sk, const Affine& read) {
+  if (read.c != 0 || !g.out_aff || !sk.out_aff) return std::nullopt;
+  struct CV { int64_t read, out, extent; };
+  std::vector<CV> cv;
+  int64_t reach = 0;
+  for (const auto& l : sk.loops) {
+    if (l.extent <= 1) continue;
+    int64_t r = read.of(l.var);
+    if (r <= 0) return std::nullopt;
+    cv.push_back({r, sk.out_aff->of(l.var), l.extent});
+    reach += r * (l.extent - 1);
+  }
+  for (const auto& kv : read.coef) {
+    bool live = false;
+    for (const auto& l : sk.loops) live = live || (l.var == kv.first && l.extent > 1);
+    if (kv.second != 0 && !live) return std::nullopt;
+  }
+  std::sort(cv.begin(), cv.end(), [](const CV& a, const CV& b) { return a.read > b.read; });
+  struct GV { std::string var; int64_t stride, extent; };
+  std::vector<GV> gv;
+  int64_t total = 1;
+  for (const auto& l : g.loops) {
+    if (l.extent <= 1) continue;
+    gv.push_back({l.var, g.out_aff->of(l.var), l.extent});
+    total *= l.extent;
+  }
+  if (reach != total - 1) return std::nullopt;
+  std::sort(gv.begin(), gv.end(), [](const GV& a, const GV& b) { return a.stride > b.stride; });
+  Affine out;
+  size_t ci = 0;
+  for (const auto& v : gv) {
+    // consumer loops that together walk this loop of the contraction: same span of C, and
+    // walking as one axis in the consumer's output too
+    int64_t covered = 1;
+    size_t first = ci;
+    while (ci < cv.size() && covered < v.extent) {
+      covered *= cv[ci].extent;
+      ++ci;
+    }
+    if (covered != v.extent || ci == first) return std::nullopt;
+    if (cv[ci - 1].read != v.stride) return std::nullopt;
+    for (size_t q = first; q + 1 < ci; ++q)
+      if (cv[q].read != cv[q + 1].read * cv[q + 1].extent || cv[q].out != cv[q + 1].out * cv[q + 1].extent)
+        return std::nullopt;
+    out.coef[v.var] = cv[ci - 1].out;
+  }
+  if (ci != cv.size()) return std::nullopt;
+  return out;
+}
+
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
   ProgramPlan plan;
@@ -944,6 +998,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       EpilogueSpec epi;
       size_t after = i + 1;
       bool have_epi = false;
+      NestKernel k0r = k0;          // k0 with C laid out as its consumer wants it, when that applies
       if (opt.gemm_epilogue && opt.fuse && have_table && gemm_shaped(k0, opt)) {
         auto gs = match_gemm(k0);
         if (gs && gemm_output_dense(*gs)) {
@@ -951,6 +1006,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           const bool small = total < (int64_t{1} << 30);
           std::map<std::string, DType> avail;          // values held in registers: C and stage outputs
           avail[k0.out_buf] = k0.out_dtype;
+          bool c_relaid = false;
           std::vector<size_t> taken;
           size_t j = i + 1;
           for (; j < kernels.size(); ++j) {
@@ -962,14 +1018,35 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             std::vector<LoadRef> loads;
             collect_loads(*sk.value, loads);
             bool feeds = false, ok = true;
+            std::optional<Affine> relaid;
             for (const auto& lr : loads) {
               if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
               if (!avail.count(lr.load->args[0]->name)) continue;
               auto a = affine_of(*lr.load->args[1]);
-              if (!a || !(*a == *sk.out_aff)) { ok = false; break; }   // must read the element it is computing
+              if (!a) { ok = false; break; }
+              if (!(*a == *sk.out_aff)) {
+                // The first consumer may read C through a permutation (a transposed weight
+                // gradient, NHWC -> NCHW after a convolution).  If C has no other reader the
+                // contraction can write C's elements where this consumer wants them: lay C out
+                // in the consumer's index space and the read becomes the aligned one.
+                bool sole = taken.empty() && !c_relaid && role_of(k0.out_buf) == "temp" &&
+                            lr.load->args[0]->name == k0.out_buf;
+                for (size_t r : readers[k0.out_buf]) sole = sole && r == j;
+                auto na = sole ? relayout(k0, sk, *a) : std::nullopt;
+                if (!na || (relaid && !(*relaid == *na))) { ok = false; break; }
+                relaid = na;
+              } else if (relaid) {
+                ok = false;   // the same stage reads C both ways
+                break;
+              }
               feeds = true;
             }
             if (!ok || !feeds) break;
+            if (relaid) {
+              k0r.out_aff = *relaid;
+              c_relaid = true;
+              if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; c_relaid = false; break; }
+            }
             avail[sk.out_buf] = sk.out_dtype;
             taken.push_back(j);
           }
@@ -1060,7 +1137,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           }
         }
       }
-      auto gl = try_emit_gemm(k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
+      auto gl = try_emit_gemm(have_epi ? k0r : k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
       if (!gl.empty()) {
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
         i = have_epi ? after : i + 1;

@@ -369,8 +369,9 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     fs << "  const long long n = o % " << s->N << "LL, m = (o / " << s->N << "LL) % " << s->M << "LL, b = o / "
        << (s->M * s->N) << "LL;\n";
     if (epilogue) {
-      // the epilogue is written for dense C: element o is (b*M + m)*N + n
-      fs << "  (void)n; (void)m; (void)b;\n  eh_epilogue(o, acc" << (epilogue->store_c ? ", C" : "") << epilogue->args << ");\n}\n";
+      // the epilogue takes the address of the element in C's layout
+      fs << "  eh_epilogue(" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n
+         << "LL, acc" << (epilogue->store_c ? ", C" : "") << epilogue->args << ");\n}\n";
     } else {
       fs << "  C[" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n << "LL] = acc;\n}\n";
     }

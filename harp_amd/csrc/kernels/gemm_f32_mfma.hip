@@ -329,7 +329,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
         const long long col = n0 + wn * WN + j * 32 + l32;
         if ((!EDGE_M || row < M) && (!EDGE_N || col < N)) {
 #if defined(EH_EPILOGUE) && EH_SPLITK == 1
-          eh_epilogue((bz * M + row) * N + col, acc[i][j][r] EH_C_ARG EH_EPI_ARGS);
+          eh_epilogue(EH_C_OFF + bz * EH_C_BS + row * EH_C_SM + col * EH_C_SN, acc[i][j][r] EH_C_ARG EH_EPI_ARGS);
 #else
           Cb[row * CSM + col * CSN] = acc[i][j][r];
 #endif
