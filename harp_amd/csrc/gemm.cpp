@@ -1,6 +1,7 @@
 #include "gemm.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <sstream>
 
@@ -25,11 +26,12 @@ struct Candidate {
   Tile tile;
   int wgs_per_cu;
   double rate, alone;
+  double step_us;   // time one k-step of a workgroup takes when nothing hides its load latency
 };
 const Candidate kCandidates[] = {
-    {{256, 256, 16, 64, 64}, 1, 133.0, 1.0},   // 16 waves
-    {{128, 128, 16, 64, 64}, 4, 124.0, 0.4},   // 4 waves
-    {{64, 64, 16, 32, 32}, 8, 105.0, 0.25},    // 4 waves
+    {{256, 256, 16, 64, 64}, 1, 133.0, 1.0, 1.2},    // 16 waves
+    {{128, 128, 16, 64, 64}, 4, 124.0, 0.4, 1.0},    // 4 waves
+    {{64, 64, 16, 32, 32}, 8, 105.0, 0.25, 0.8},     // 4 waves
 };
 
 bool tile_valid(const Tile& t) {
@@ -65,6 +67,10 @@ double estimate_us(const GemmShape& s, const Candidate& c, int split) {
     double per_cu = static_cast<double>(ceil_div(rest, static_cast<int64_t>(cus))) / c.wgs_per_cu;
     us += round_us * std::max(per_cu, c.alone / c.wgs_per_cu * 1.0);
   }
+  // a workgroup cannot finish faster than its k-steps' dependent load latencies allow
+  // (measured: 49 steps of a lone 64x64 workgroup take 40 us)
+  const double rounds = std::ceil(static_cast<double>(wgs) / slots);
+  us = std::max(us, rounds * static_cast<double>(ksteps) * c.step_us);
   us += 2.0;   // prologue, epilogue, launch
   if (split > 1) us += 3.0 + (split + 1.0) * 4.0 * static_cast<double>(s.batch * s.M * s.N) / 4e6;
   return us;
