@@ -190,6 +190,34 @@ def test_index_forms_bit_exact(frontend, hip, name, fuse):
         assert bits_equal_mod_zero(ref, got)
 
 
+GATHER_FORMS = {
+    "transpose": lambda t: t.permute([1, 0]).contiguous(),
+    "pad": lambda t: t.pad([(1, 2), (3, 1)]).contiguous(),
+    "windows": lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1]).contiguous(),
+    "tiles_interleaved": lambda t: t.unfold([0, 1], [2, 2], [2, 2], [1, 1]).permute([0, 2, 1, 3]).contiguous(),
+    "flip_neg": lambda t: (-t.flip(1)).contiguous(),
+    "repeat_rows": lambda t: t.unsqueeze(0).expand(0, 5).contiguous(),
+}
+
+
+@pytest.mark.parametrize("name", sorted(GATHER_FORMS))
+@pytest.mark.parametrize("shape", [(64, 96), (50, 82)])
+def test_gathering_copies_bit_exact(frontend, hip, name, shape):
+    """Copies through permuted, padded, windowed and repeated views, thousands of elements
+    (several workgroups of the flat schedule, ragged last block)."""
+    if name == "flip_neg" and not hasattr(frontend.Tensor, "flip"):
+        pytest.skip("no flip in the tensor API")
+    x = RNG(shape[0]).normal(0, 1, shape).astype(np.float32)
+    fn = GATHER_FORMS[name]
+    t = frontend.Tensor.input(list(shape))
+    with frontend.exact_mode():
+        prog, _, _ = frontend.lower_graph([fn(t).graph])
+        scheds = [l["schedule"] for l in hip.render_program(prog).launches]
+        ref, got = both(frontend, fn, [x], True)
+    assert any(s.startswith("flat(") for s in scheds), scheds
+    assert bits_equal_mod_zero(ref, got)
+
+
 def test_buffer_roundtrip_and_size_check(hip):
     dev = hip.HipDevice(0)
     from harp_amd.frontend import F32
