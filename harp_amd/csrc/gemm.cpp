@@ -250,6 +250,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   const int nt = (t.bm / t.wm) * (t.bn / t.wn) * 64;
   const std::string scratch = "eh_part_" + k.name;
   std::ostringstream os;
+  std::string dma_tag;
   os << "// generated for gfx950 by eclat backend-hip: MFMA contraction\n";
   os << "#define EH_ENTRY " << ls.entry << "\n";
   os << "#define EH_M " << s->M << "\n#define EH_N " << s->N << "\n#define EH_K " << s->K << "\n#define EH_BATCH "
@@ -258,6 +259,14 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
      << t.wm << "\n#define EH_WN " << t.wn << "\n";
   os << "#define EH_A_KCONTIG " << (a_kc ? 1 : 0) << "\n#define EH_B_NCONTIG " << (b_nc ? 1 : 0) << "\n";
   os << "#define EH_A_VEC " << (a_vec ? 1 : 0) << "\n#define EH_B_VEC " << (b_vec ? 1 : 0) << "\n";
+  {
+    // direct-to-LDS loads: row-contiguous operand, 128-bit loads, no guards needed on its tile
+    const bool k_exact = s->K % t.bk == 0 && ((s->K / t.bk) % ch.split_k) == 0;
+    const bool a_dma = opt.gemm_dma && !a_kc && a_vec && k_exact && s->M % t.bm == 0;
+    const bool b_dma = opt.gemm_dma && b_nc && b_vec && k_exact && s->N % t.bn == 0;
+    os << "#define EH_A_DMA " << (a_dma ? 1 : 0) << "\n#define EH_B_DMA " << (b_dma ? 1 : 0) << "\n";
+    dma_tag = std::string(a_dma ? ",A>lds" : "") + (b_dma ? ",B>lds" : "");
+  }
   os << "#define EH_A_SM " << s->a_m << "LL\n#define EH_A_SK " << s->a_k << "LL\n";
   os << "#define EH_B_SK " << s->b_k << "LL\n#define EH_B_SN " << s->b_n << "LL\n";
   os << "#define EH_C_SM " << s->c_m << "LL\n#define EH_C_SN " << s->c_n << "LL\n";
@@ -298,7 +307,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
                 (fa ? "/folded" : a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") +
                 (fb ? "/folded" : b_vec ? "" : "/scalar") +
-                (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
+                dma_tag + (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
                 (epi_here ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
   ls.grid[1] = static_cast<unsigned>(S);

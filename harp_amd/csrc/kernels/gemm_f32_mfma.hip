@@ -71,7 +71,19 @@ typedef float eh_f4v __attribute__((ext_vector_type(4)));
 namespace {
 constexpr int BM = EH_BM, BN = EH_BN, BK = EH_BK, WM = EH_WM, WN = EH_WN;
 constexpr int NWM = BM / WM, NWN = BN / WN, NT = NWM * NWN * 64;
-constexpr int AS = BM + 4, BS = BN + 4;            // padded row counts / row lengths in LDS
+// A row-contiguous operand whose tile needs no guards goes from global memory straight into
+// LDS (global_load_lds_dwordx4: lane i of a wave writes its 16 bytes at base + 16*i): work-item
+// q's four elements are element q of the unpadded [k][row] tile, so a wave's 64 loads fill
+// 1 KiB of consecutive LDS and neither registers nor ds_write are involved.  (For a
+// k-contiguous operand the lanes would have to take one row each, 16 bytes per cache line:
+// measured 7 % slower than staging it through registers.)
+#ifndef EH_A_DMA
+#define EH_A_DMA 0
+#endif
+#ifndef EH_B_DMA
+#define EH_B_DMA 0
+#endif
+constexpr int AS = BM + (EH_A_DMA ? 0 : 4), BS = BN + (EH_B_DMA ? 0 : 4);   // (padded) rows per k in LDS
 constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 4-element loads per thread per tile
 constexpr int IB = WM / 32, JB = WN / 32;
 constexpr int NBLK = BK / 8;                       // blocks of eight k values per tile step
@@ -145,6 +157,8 @@ struct EhTile {
     return v;
   }
 };
+template <bool V> struct EhBool { static constexpr bool value = V; };
+struct EhFlag { bool value; };
 using ATile = EhTile<EH_A_KCONTIG != 0, AS>;
 using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
 }  // namespace
@@ -170,8 +184,19 @@ using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
 
 extern "C" __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(EH_WAVES_PER_SIMD, EH_WAVES_PER_SIMD)))
 EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_EPI_PARAMS) {
+  // two tiles per operand, as separate arrays: the compiler then knows that a direct-to-LDS
+  // load into one does not touch what is being read from the other
+#if EH_A_DMA || EH_B_DMA
+  __shared__ __attribute__((aligned(16))) float As0[BK * AS];
+  __shared__ __attribute__((aligned(16))) float As1[BK * AS];
+  __shared__ __attribute__((aligned(16))) float Bs0[BK * BS];
+  __shared__ __attribute__((aligned(16))) float Bs1[BK * BS];
+#else
   __shared__ __attribute__((aligned(16))) float As[2][BK * AS];
   __shared__ __attribute__((aligned(16))) float Bs[2][BK * BS];
+  float* const As0 = As[0];
+  float* const Bs0 = Bs[0];
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wid = tid >> 6;
@@ -210,12 +235,21 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 
   // thread q of the tile owns four elements: along k at (row q / (BK/4), k 4*(q % (BK/4))) for
   // a k-contiguous operand, along the row at (k q / (rows/4), row 4*(q % (rows/4))) otherwise
-  auto gload = [&](int kt) {
+  auto to_lds = [&](const float* gp, float* tile, int q_wave) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gp,
+                                     (__attribute__((address_space(3))) void*)(tile + q_wave * 4), 16, 0, 0);
+  };
+  auto gload = [&](int kt, float* a_tile, float* b_tile) {
+    (void)a_tile;
+    (void)b_tile;
     const long long k0 = kbeg + (long long)kt * BK;
 #pragma unroll
     for (int i = 0; i < AV; ++i) {
       const int q = tid + i * NT;
-#if EH_A_KCONTIG
+#if EH_A_DMA
+      const int k = q / (BM / 4), mq = q % (BM / 4);
+      to_lds(A + a_base + (k0 + k) * EH_A_SK + (m0 + mq * 4) * EH_A_SM, a_tile, (tid & ~63) + i * NT);
+#elif EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
       ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, m0 + m, k0 + kq * 4, M, kend);
 #else
@@ -226,7 +260,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #pragma unroll
     for (int i = 0; i < BV; ++i) {
       const int q = tid + i * NT;
-#if EH_B_NCONTIG
+#if EH_B_DMA
+      const int k = q / (BN / 4), nq = q % (BN / 4);
+      to_lds(B + b_base + (k0 + k) * EH_B_SK + (n0 + nq * 4) * EH_B_SN, b_tile, (tid & ~63) + i * NT);
+#elif EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
       rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, n0 + nq * 4, k0 + k, N, kend);
 #else
@@ -236,25 +273,34 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
     }
   };
 
-  auto sstore = [&](int buf) {
+  auto sstore = [&](float* a_tile, float* b_tile) {
+    (void)a_tile;
+    (void)b_tile;
+#if !EH_A_DMA
 #pragma unroll
     for (int i = 0; i < AV; ++i) {
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
-      ATile::put(As[buf], q / (BK / 4), (q % (BK / 4)) * 4, ra[i]);
+      ATile::put(a_tile, q / (BK / 4), (q % (BK / 4)) * 4, ra[i]);
 #else
-      ATile::put(As[buf], (q % (BM / 4)) * 4, q / (BM / 4), ra[i]);
+      ATile::put(a_tile, (q % (BM / 4)) * 4, q / (BM / 4), ra[i]);
 #endif
     }
+#endif
+#if !EH_B_DMA
 #pragma unroll
     for (int i = 0; i < BV; ++i) {
       const int q = tid + i * NT;
 #if EH_B_NCONTIG
-      BTile::put(Bs[buf], (q % (BN / 4)) * 4, q / (BN / 4), rb[i]);
+      BTile::put(b_tile, (q % (BN / 4)) * 4, q / (BN / 4), rb[i]);
 #else
-      BTile::put(Bs[buf], q / (BK / 4), (q % (BK / 4)) * 4, rb[i]);
+      BTile::put(b_tile, q / (BK / 4), (q % (BK / 4)) * 4, rb[i]);
 #endif
     }
+#endif
+#if EH_A_DMA || EH_B_DMA
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's direct-to-LDS loads have landed
+#endif
   };
 
   eh_f16v acc[IB][JB];
@@ -265,17 +311,17 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  gload(0);
-  sstore(0);
+  gload(0, As0, Bs0);
+  sstore(As0, Bs0);
   __syncthreads();
 
   // two register slots of operands: block j+1 is fetched while block j is multiplied
   eh_f4v a[2][IB], b[2][JB];
-  auto fetch = [&](int buf, int j, int slot) {
+  auto fetch = [&](const float* a_tile, const float* b_tile, int j, int slot) {
 #pragma unroll
-    for (int i = 0; i < IB; ++i) a[slot][i] = ATile::get(As[buf], j, kh, wm * WM + i * 32 + l32);
+    for (int i = 0; i < IB; ++i) a[slot][i] = ATile::get(a_tile, j, kh, wm * WM + i * 32 + l32);
 #pragma unroll
-    for (int jj = 0; jj < JB; ++jj) b[slot][jj] = BTile::get(Bs[buf], j, kh, wn * WN + jj * 32 + l32);
+    for (int jj = 0; jj < JB; ++jj) b[slot][jj] = BTile::get(b_tile, j, kh, wn * WN + jj * 32 + l32);
   };
   auto multiply = [&](int slot) {
 #pragma unroll
@@ -286,13 +332,12 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
         for (int jj = 0; jj < JB; ++jj)
           acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[slot][i][e], b[slot][jj][e], acc[i][jj], 0, 0, 0);
   };
-
-  fetch(0, 0, 0);
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    const bool more = kt + 1 < KT;
+  // one tile step: multiply the tile in (a_cur, b_cur) while the next one travels to (a_nxt, b_nxt)
+  // (`more`: a next tile exists; a compile-time tag so that the loop body has no branches)
+  auto step = [&](int kt, float* a_cur, float* b_cur, float* a_nxt, float* b_nxt, auto more_tag) {
+    const bool more = more_tag.value;
     if (more) {
-      gload(kt + 1);
+      gload(kt + 1, a_nxt, b_nxt);
       // keep the global loads up here: their latency is hidden by the whole multiply loop only
       // if they are issued before it (the compiler would otherwise sink them to their use)
       asm volatile("" ::: "memory");
@@ -303,7 +348,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #endif
 #pragma unroll
     for (int j = 0; j < NBLK - 1; ++j) {
-      fetch(buf, j + 1, (j + 1) & 1);
+      fetch(a_cur, b_cur, j + 1, (j + 1) & 1);
       __builtin_amdgcn_sched_barrier(0);   // reads of the next block stay ahead of these MFMAs
       multiply(j & 1);
       __builtin_amdgcn_sched_barrier(0);
@@ -311,12 +356,34 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #if EH_SETPRIO
     __builtin_amdgcn_s_setprio(0);
 #endif
-    if (more) sstore(buf ^ 1);
+    if (more) sstore(a_nxt, b_nxt);
     __syncthreads();
-    if (more) fetch(buf ^ 1, 0, NBLK & 1);
+    if (more) fetch(a_nxt, b_nxt, 0, NBLK & 1);
     __builtin_amdgcn_sched_barrier(0);
     multiply((NBLK - 1) & 1);
+  };
+
+  fetch(As0, Bs0, 0, 0);
+#if !(EH_A_DMA || EH_B_DMA)
+  // one loop body, buffers chosen by the step's parity
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    step(kt, As[buf], Bs[buf], As[buf ^ 1], Bs[buf ^ 1], EhFlag{kt + 1 < KT});
   }
+#else
+  // unrolled by two so that each direct-to-LDS load names its destination array statically
+  int kt = 0;
+  for (; kt + 2 < KT; kt += 2) {
+    step(kt, As0, Bs0, As1, Bs1, EhBool<true>{});
+    step(kt + 1, As1, Bs1, As0, Bs0, EhBool<true>{});
+  }
+  if (kt + 2 == KT) {
+    step(kt, As0, Bs0, As1, Bs1, EhBool<true>{});
+    step(kt + 1, As1, Bs1, As0, Bs0, EhBool<false>{});
+  } else {
+    step(kt, As0, Bs0, As1, Bs1, EhBool<false>{});
+  }
+#endif
 
   // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32
 #pragma unroll
