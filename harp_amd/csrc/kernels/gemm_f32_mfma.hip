@@ -157,8 +157,6 @@ struct EhTile {
     return v;
   }
 };
-template <bool V> struct EhBool { static constexpr bool value = V; };
-struct EhFlag { bool value; };
 using ATile = EhTile<EH_A_KCONTIG != 0, AS>;
 using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
 }  // namespace
@@ -333,9 +331,8 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
           acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[slot][i][e], b[slot][jj][e], acc[i][jj], 0, 0, 0);
   };
   // one tile step: multiply the tile in (a_cur, b_cur) while the next one travels to (a_nxt, b_nxt)
-  // (`more`: a next tile exists; a compile-time tag so that the loop body has no branches)
-  auto step = [&](int kt, float* a_cur, float* b_cur, float* a_nxt, float* b_nxt, auto more_tag) {
-    const bool more = more_tag.value;
+  // (`more`: a next tile exists; a literal in the unrolled loop, uniform otherwise)
+  auto step = [&](int kt, float* a_cur, float* b_cur, float* a_nxt, float* b_nxt, const bool more) {
     if (more) {
       gload(kt + 1, a_nxt, b_nxt);
       // keep the global loads up here: their latency is hidden by the whole multiply loop only
@@ -368,20 +365,20 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   // one loop body, buffers chosen by the step's parity
   for (int kt = 0; kt < KT; ++kt) {
     const int buf = kt & 1;
-    step(kt, As[buf], Bs[buf], As[buf ^ 1], Bs[buf ^ 1], EhFlag{kt + 1 < KT});
+    step(kt, As[buf], Bs[buf], As[buf ^ 1], Bs[buf ^ 1], kt + 1 < KT);
   }
 #else
   // unrolled by two so that each direct-to-LDS load names its destination array statically
   int kt = 0;
   for (; kt + 2 < KT; kt += 2) {
-    step(kt, As0, Bs0, As1, Bs1, EhBool<true>{});
-    step(kt + 1, As1, Bs1, As0, Bs0, EhBool<true>{});
+    step(kt, As0, Bs0, As1, Bs1, true);
+    step(kt + 1, As1, Bs1, As0, Bs0, true);
   }
   if (kt + 2 == KT) {
-    step(kt, As0, Bs0, As1, Bs1, EhBool<true>{});
-    step(kt + 1, As1, Bs1, As0, Bs0, EhBool<false>{});
+    step(kt, As0, Bs0, As1, Bs1, true);
+    step(kt + 1, As1, Bs1, As0, Bs0, false);
   } else {
-    step(kt, As0, Bs0, As1, Bs1, EhBool<false>{});
+    step(kt, As0, Bs0, As1, Bs1, false);
   }
 #endif
 

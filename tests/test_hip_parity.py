@@ -420,6 +420,8 @@ CONTRACTIONS = [
     ("matmul", [(64, 2048), (2048, 64)], None, "split-k="),
     ("matmul", [(96, 1000), (1000, 40)], None, "split-k="),
     ("matmul", [(256, 512), (512, 256)], {"gemm_split_k": 3}, "split-k=3"),
+    ("matmul", [(256, 64), (64, 128)], {"gemm_dma": 1}, "B>lds"),
+    ("per_group", [(3, 64, 64), (3, 64, 128)], {"gemm_dma": 1}, "A>lds,B>lds"),
     ("matmul", [(192, 160), (160, 320)], {"gemm_bm": 128, "gemm_bn": 128, "gemm_bk": 16, "gemm_wm": 64, "gemm_wn": 64}, "tile=128x128x16"),
     ("linear", [(130, 72), (50, 72)], None, "edges"),
     ("linear", [(33, 18), (7, 18)], None, "/scalar"),
