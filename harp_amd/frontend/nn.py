@@ -73,7 +73,7 @@ def conv2d(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None, stride=(1, 
     h_out = (h + 2 * ph - dh * (kh - 1) - 1) // sh + 1
     w_out = (w + 2 * pw - dw * (kw - 1) - 1) // sw + 1
     padded = x.pad([(0, 0), (0, 0), (ph, ph), (pw, pw)])
-    unfolded = padded.unfold([2, 3], [kh, kw], [sh, sw], [dh, dw])
+    unfolded = padded.unfold_2d((kh, kw), (sh, sw), (dh, dw))
     cols = unfolded.permute([0, 2, 3, 1, 4, 5]).contiguous().reshape([n, h_out * w_out, cin * kh * kw])
     weight_flat = weight.reshape([cout, cin * kh * kw])
     product = cols.unsqueeze(2) * weight_flat.unsqueeze(0).unsqueeze(0)
@@ -93,7 +93,7 @@ def max_pool2d(x: Tensor, kernel_size, stride=None, padding=(0, 0), dilation=(1,
     h_out = (h + 2 * ph - dh * (kh - 1) - 1) // sh + 1
     w_out = (w + 2 * pw - dw * (kw - 1) - 1) // sw + 1
     padded = x.pad([(0, 0), (0, 0), (ph, ph), (pw, pw)]) if (ph > 0 or pw > 0) else x
-    unfolded = padded.unfold([2, 3], [kh, kw], [sh, sw], [dh, dw])
+    unfolded = padded.unfold_2d((kh, kw), (sh, sw), (dh, dw))
     return unfolded.contiguous().reshape([n, c, h_out, w_out, kh * kw]).max(4)
 
 

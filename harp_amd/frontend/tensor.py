@@ -67,6 +67,23 @@ class Tensor:
         return Tensor(G.zeros(other.shape(), other.dtype()))
 
     @staticmethod
+    def scalar(_value=0.0, dtype: DType = F32) -> "Tensor":
+        """A rank-0 constant node.  The value is not recorded (tensor.rs:332-337): realize
+        fills every synthesised constant that is not `zeros` with 1.0 (realize.rs:391-421)."""
+        return Tensor(G.scalar(dtype))
+
+    @staticmethod
+    def from_shape_data(shape: Sequence[int], data) -> "Tensor":
+        """Checks that `data` has the shape's element count and returns a plain input: the
+        reference does not attach the data either (tensor.rs:186-200); call set_data()."""
+        n = 1
+        for d in shape:
+            n *= int(d)
+        if len(data) != n:
+            raise ValueError(f"Data length {len(data)} doesn't match shape {list(shape)} (numel={n})")
+        return Tensor.input(shape)
+
+    @staticmethod
     def from_numpy(arr: np.ndarray) -> "Tensor":
         """Convenience: input + set_data (needs a default device)."""
         dt = {v: k for k, v in _NP.items() if k != "bool"}[arr.dtype.type]
@@ -193,6 +210,18 @@ class Tensor:
     def unfold(self, axes, sizes, strides, dilations):
         return Tensor(self.graph.unfold(axes, sizes, strides, dilations))
 
+    def unfold_1d(self, kernel_size, stride, dilation):
+        """[N,C,L] -> [N,C,L_out,K] (ops.rs:592-598)."""
+        return self.unfold([2], [kernel_size], [stride], [dilation])
+
+    def unfold_2d(self, kernel_size, stride, dilation):
+        """[N,C,H,W] -> [N,C,H_out,W_out,kH,kW] (ops.rs:566-580)."""
+        return self.unfold([2, 3], list(kernel_size), list(stride), list(dilation))
+
+    def unfold_3d(self, kernel_size, stride, dilation):
+        """[N,C,D,H,W] -> [N,C,D_out,H_out,W_out,kD,kH,kW] (ops.rs:611-624)."""
+        return self.unfold([2, 3, 4], list(kernel_size), list(stride), list(dilation))
+
     def fold(self, output_shape, axes, sizes, strides, dilations):
         return Tensor(self.graph.fold(output_shape, axes, sizes, strides, dilations))
 
@@ -212,6 +241,14 @@ class Tensor:
 
     def zero_grad(self) -> None:
         self._grad = None
+
+    def accumulate_grad(self, grad: "Tensor") -> None:
+        """Adds to the stored gradient graph, or stores the first one (autograd.rs:200-209)."""
+        self._grad = grad if self._grad is None else Tensor(self._grad.graph + grad.graph)
+
+    def try_buffer(self):
+        """The realized buffer or None (realize.rs:97-104)."""
+        return self.buffer
 
     def detach(self) -> "Tensor":
         t = Tensor(self.graph)

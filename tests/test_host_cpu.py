@@ -211,6 +211,26 @@ def test_tensor_api_errors(frontend):
         frontend.set_device_str("nosuchbackend")
 
 
+def test_tensor_constructors_and_small_api(frontend):
+    T = frontend.Tensor
+    assert T.scalar(3.5).shape() == [] and T.scalar(3.5).graph.name == "scalar"     # value not recorded
+    t = T.from_shape_data([2, 3], [0.0] * 6)
+    assert t.shape() == [2, 3] and not t.is_realized() and t.try_buffer() is None     # data not attached
+    with pytest.raises(ValueError):
+        T.from_shape_data([2, 3], [0.0] * 5)
+    x = T.input([2, 3, 10])
+    assert x.unfold_1d(3, 1, 1).shape() == [2, 3, 8, 3]
+    y = T.input([2, 3, 8, 9])
+    assert y.unfold_2d((3, 2), (1, 1), (1, 1)).shape() == [2, 3, 6, 8, 3, 2]
+    z = T.input([1, 2, 5, 6, 7])
+    assert z.unfold_3d((2, 2, 2), (1, 2, 1), (1, 1, 1)).shape() == [1, 2, 4, 3, 6, 2, 2, 2]
+    p = T.input([4])
+    p.accumulate_grad(T.ones([4]))
+    first = p.grad()
+    p.accumulate_grad(T.ones([4]))
+    assert p.grad() is not first and p.grad().graph.op.kind == "map_reduce" and p.grad().shape() == [4]
+
+
 def test_kernel_cache_counts(frontend):
     # crates/backend-c/src/lib.rs:246-297: second realize of the same graph hits the cache
     frontend.set_device_str("c")
