@@ -783,22 +783,12 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   const bool small = it != elems.end() && it->second < (size_t{1} << 30) && numel < (int64_t{1} << 30);
   FoldedOperand f;
   f.src = src;
+  f.kernel = k.name;
+  f.small = small;
   f.src_bytes = it == elems.end() ? 0.0 : 4.0 * static_cast<double>(it->second);
-  std::ostringstream os;
-  os << "// element eh_L of what kernel " << k.name << " would have written\n";
-  os << "__device__ __forceinline__ float EH_FOLD_FN(const float* __restrict__ " << src << ", long long eh_L) {\n";
-  os << "  typedef " << (small ? "int" : "long long") << " eh_fold_idx;\n  const eh_fold_idx eh_l = (eh_fold_idx)eh_L;\n";
-  for (size_t i = 0; i < k.loops.size(); ++i) {
-    const Loop& l = k.loops[i];
-    if (l.extent == 1) {
-      os << "  const eh_fold_idx " << l.var << " = 0;\n";
-    } else {
-      os << "  const eh_fold_idx " << l.var << " = (eh_l / " << strides[i] << ") % " << l.extent << ";\n";
-    }
-  }
+  for (size_t i = 0; i < k.loops.size(); ++i) f.loops.push_back({k.loops[i].var, k.loops[i].extent, strides[i]});
   ExprRenderer er;
-  os << "  return (float)(" << er.expr(*k.value) << ");\n}\n";
-  f.function = os.str();
+  f.expr = er.expr(*k.value);
   if (auto a = affine_of(*loads[0].load->args[1]))
     for (size_t i = 0; i < k.loops.size(); ++i)
       if (k.loops[i].extent > 1) f.src_stride[strides[i]] = a->of(k.loops[i].var);

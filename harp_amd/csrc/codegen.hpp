@@ -28,7 +28,7 @@ struct GenOptions {
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
   bool gemm_epilogue = true;          // run elementwise consumers of a contraction on its accumulators
-  bool gemm_fold = false;             // evaluate gather/copy producers inside the tile loader (implicit GEMM)
+  bool gemm_fold = true;              // evaluate gather/copy producers inside the tile loader (implicit GEMM)
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
   int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores

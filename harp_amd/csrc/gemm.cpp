@@ -275,12 +275,43 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
   os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
-  auto emit_fold = [&](const FoldedOperand* f, const char* macro, const char* fn) {
+  // A computed operand's element (row r, k) sits at off + bz*bs + r*sr + k*sk of the producer's
+  // output.  Split that index at Q (a boundary between the producer's loops): when the row part
+  // only moves the quotient and the k part only the remainder (mode 1), or the other way round
+  // (mode 2), the part that belongs to the row is the same for every k step, and the compiler
+  // hoists its decode out of the k loop; no division by Q is needed either.
+  auto emit_fold = [&](const FoldedOperand* f, const char* X, const char* fn, int64_t off, int64_t bs, int64_t sr,
+                       int64_t sk, int64_t rows, int64_t kext) {
     if (!f) return;
-    std::string text = f->function;
-    const std::string ph = "EH_FOLD_FN";
-    for (size_t at = text.find(ph); at != std::string::npos; at = text.find(ph, at)) text.replace(at, ph.size(), fn);
-    os << "#define " << macro << " 1\n" << text;
+    int64_t total = 1;
+    for (const auto& l : f->loops) total *= l.extent;
+    auto boundary = [&](int64_t q) {
+      for (const auto& l : f->loops)
+        if (l.stride == q) return true;
+      return q == total;
+    };
+    int mode = 0;
+    int64_t Q = total;
+    if (sr > 0 && boundary(sr) && off % sr == 0 && bs % sr == 0 && kext * sk <= sr) {
+      mode = 1;
+      Q = sr;
+    } else if (sk > 0 && boundary(sk) && off % sk == 0 && bs % sk == 0 && rows * sr <= sk) {
+      mode = 2;
+      Q = sk;
+    }
+    const std::string IT = f->small ? "int" : "long long";
+    os << "#define EH_" << X << "_FOLD 1\n#define EH_" << X << "_FOLD_MODE " << mode << "\n#define EH_" << X << "_FOLD_Q " << Q
+       << "LL\n";
+    os << "// element (eh_U * " << Q << " + eh_I) of what kernel " << f->kernel << " would have written\n";
+    os << "__device__ __forceinline__ float " << fn << "(const float* __restrict__ " << f->src
+       << ", long long eh_U64, long long eh_I64) {\n";
+    os << "  const " << IT << " eh_U = (" << IT << ")eh_U64, eh_I = (" << IT << ")eh_I64;\n";
+    for (const auto& l : f->loops) {
+      if (l.extent == 1) os << "  const " << IT << " " << l.name << " = 0;\n";
+      else if (l.stride >= Q) os << "  const " << IT << " " << l.name << " = (eh_U / " << l.stride / Q << ") % " << l.extent << ";\n";
+      else os << "  const " << IT << " " << l.name << " = (eh_I / " << l.stride << ") % " << l.extent << ";\n";
+    }
+    os << "  return (float)(" << f->expr << ");\n}\n";
   };
   const bool epi_here = epilogue && S == 1;     // with K split the epilogue runs in the summing launch
   if (epi_here) {
@@ -289,8 +320,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     if (!epilogue->store_c) os << "#define EH_NO_C 1\n";
     os << epilogue->function;
   }
-  emit_fold(fa, "EH_A_FOLD", "eh_a_elem");
-  emit_fold(fb, "EH_B_FOLD", "eh_b_elem");
+  emit_fold(fa, "A", "eh_a_elem", s->a_off, s->a_b, s->a_m, s->a_k, s->M, s->K);
+  emit_fold(fb, "B", "eh_b_elem", s->b_off, s->b_b, s->b_n, s->b_k, s->N, s->K);
   {
     // register budget: 512 lanes' registers per SIMD shared by the resident waves; a wave needs
     // its accumulators (wm*wn/64) plus about 56 for operands, staging and addresses

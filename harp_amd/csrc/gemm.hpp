@@ -24,16 +24,23 @@ struct GemmShape {
 
 // An elementwise producer (im2col gather, layout copy, padding ...) whose dense output a
 // contraction would read: the tile loader evaluates it per element instead, so the buffer is
-// never written.  `function` is the text of
-//   __device__ float EH_FOLD_FN(const float* __restrict__ <src>, long long eh_L)
-// returning element eh_L of the producer's output.
+// never written.  The contraction builds a device function from this: the producer's loop
+// variables are decoded from the element's index in the producer's output (loops with a
+// stride of at least Q from the quotient, the others from the remainder, Q chosen so that one
+// of the two parts does not change along the contraction's k loop) and `expr` is returned.
 struct FoldedOperand {
   std::string src;        // the one buffer the producer reads
-  std::string function;
-  double src_bytes = 0;   // 0 = unknown
-  // for each loop of the producer: its stride in the producer's output -> its stride in the
-  // source (only when the source index is affine); tells which operand axis is contiguous in
-  // the memory actually read
+  std::string kernel;     // the producer's name (for comments)
+  std::string expr;       // C expression over the loop variables and `src`
+  struct LoopVar {
+    std::string name;
+    int64_t extent, stride;   // stride in the producer's dense output
+  };
+  std::vector<LoopVar> loops;   // outermost first
+  bool small = true;            // 32-bit index arithmetic suffices
+  double src_bytes = 0;         // 0 = unknown
+  // loop stride in the producer's output -> that loop's stride in the source (only when the
+  // source index is affine); tells which operand axis is contiguous in the memory actually read
   std::map<int64_t, int64_t> src_stride;
 };
 using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer

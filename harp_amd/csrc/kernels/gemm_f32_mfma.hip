@@ -100,32 +100,57 @@ static_assert(WM % 32 == 0 && WN % 32 == 0 && BK % 16 == 0, "wave tile must be b
 static_assert(!EH_A_VEC || (EH_A_KCONTIG ? EH_K % 4 == 0 : EH_M % 4 == 0), "A cannot be loaded as vectors");
 static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B cannot be loaded as vectors");
 
-// How element i of an operand is obtained: from memory, or (EH_A_FOLD / EH_B_FOLD) by
-// evaluating the elementwise kernel that would have produced it, on that kernel's own source.
+// How an operand's element (batch bz, row r, k) is obtained: from memory at
+// off + bz*bs + r*sr + k*sk, or (EH_A_FOLD / EH_B_FOLD) by evaluating the elementwise kernel
+// that would have produced that element, on that kernel's own source.  The generated function
+// takes the element's index split at Q into (quotient, remainder); in mode 1 the row decides
+// the quotient and k the remainder, in mode 2 the other way round, so whatever is decoded from
+// the row's part is loop-invariant along k.
+template <long long OFF, long long BS, long long SR, long long SK>
 struct EhFromMemory {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return p[i]; }
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
+    return p[OFF + bz * BS + r * SR + k * SK];
+  }
 };
 #ifdef EH_A_FOLD
 struct EhAElem {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return eh_a_elem(p, i); }
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
+    constexpr long long Q = EH_A_FOLD_Q;
+#if EH_A_FOLD_MODE == 1
+    return eh_a_elem(p, EH_A_OFF / Q + bz * (EH_A_BS / Q) + r * (EH_A_SM / Q), k * EH_A_SK);
+#elif EH_A_FOLD_MODE == 2
+    return eh_a_elem(p, EH_A_OFF / Q + bz * (EH_A_BS / Q) + k * (EH_A_SK / Q), r * EH_A_SM);
+#else
+    return eh_a_elem(p, 0, EH_A_OFF + bz * EH_A_BS + r * EH_A_SM + k * EH_A_SK);
+#endif
+  }
 };
 #else
-using EhAElem = EhFromMemory;
+using EhAElem = EhFromMemory<EH_A_OFF, EH_A_BS, EH_A_SM, EH_A_SK>;
 #endif
 #ifdef EH_B_FOLD
 struct EhBElem {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long i) { return eh_b_elem(p, i); }
+  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
+    constexpr long long Q = EH_B_FOLD_Q;
+#if EH_B_FOLD_MODE == 1
+    return eh_b_elem(p, EH_B_OFF / Q + bz * (EH_B_BS / Q) + r * (EH_B_SN / Q), k * EH_B_SK);
+#elif EH_B_FOLD_MODE == 2
+    return eh_b_elem(p, EH_B_OFF / Q + bz * (EH_B_BS / Q) + k * (EH_B_SK / Q), r * EH_B_SN);
+#else
+    return eh_b_elem(p, 0, EH_B_OFF + bz * EH_B_BS + r * EH_B_SN + k * EH_B_SK);
+#endif
+  }
 };
 #else
-using EhBElem = EhFromMemory;
+using EhBElem = EhFromMemory<EH_B_OFF, EH_B_BS, EH_B_SN, EH_B_SK>;
 #endif
 
 // Four elements of an operand starting at (r, k) and running along its fast axis; elements
 // outside [0,R) x [0,kend) read as zero.  ALONG_K says which axis the four run along; `base`
-// is the operand's offset plus the batch offset.
+// is the operand's offset plus the batch offset (used by the 128-bit path).
 template <class ELEM, bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
-__device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long base, long long r, long long k,
-                                              long long R, long long kend) {
+__device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long base, long long bz, long long r,
+                                              long long k, long long R, long long kend) {
   eh_f4v v = {0.0f, 0.0f, 0.0f, 0.0f};
   if (VEC) {
     const bool ok = (!EDGE_R || r < R) && (!EDGE_K || k < kend);
@@ -134,7 +159,7 @@ __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const long long rr = ALONG_K ? r : r + e, kk = ALONG_K ? k + e : k;
-      if (rr < R && kk < kend) v[e] = ELEM::at(p, base + rr * SR + kk * SK);
+      if (rr < R && kk < kend) v[e] = ELEM::at(p, bz, rr, kk);
     }
   }
   return v;
@@ -249,10 +274,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(A + a_base + (k0 + k) * EH_A_SK + (m0 + mq * 4) * EH_A_SM, a_tile, (tid & ~63) + i * NT);
 #elif EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, m0 + m, k0 + kq * 4, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, m0 + mq * 4, k0 + k, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend);
 #endif
     }
 #pragma unroll
@@ -263,10 +288,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(B + b_base + (k0 + k) * EH_B_SK + (n0 + nq * 4) * EH_B_SN, b_tile, (tid & ~63) + i * NT);
 #elif EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, n0 + nq * 4, k0 + k, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend);
 #else
       const int n = q / (BK / 4), kq = q % (BK / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, n0 + n, k0 + kq * 4, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + n, k0 + kq * 4, N, kend);
 #endif
     }
   };

@@ -459,27 +459,31 @@ def test_contraction_variants_on_mfma(frontend, hip, kind, shapes, options, expe
 
 
 def test_config5_with_implicit_gemm_loader(frontend, hip):
-    """Option gemm_fold=1: im2col gathers and layout copies that only contractions read are
-    evaluated inside the contractions' tile loaders (no launch, no buffer).  Same results."""
+    """im2col gathers and layout copies that only contractions read are evaluated inside the
+    contractions' tile loaders (no launch, no buffer); option gemm_fold=0 materialises them.
+    Same results either way."""
     from harp_amd import workloads as wl
     from harp_amd.frontend.device import _BACKENDS
     sizes = (8, 28, 32, 64, 128, 10)
     arrays = wl.config5_inputs(*sizes, seed=78)
     ts = [frontend.Tensor.input(list(a.shape)) for a in arrays]
     prog_ast = wl.lower_multi(ts, wl.config5_graph(*ts))[0]
-    plain = hip.render_program(prog_ast)
-    folded = hip.render_program(prog_ast, {"gemm_fold": 1})
+    plain = hip.render_program(prog_ast, {"gemm_fold": 0})
+    folded = hip.render_program(prog_ast)
     assert len(folded.launches) < len(plain.launches)
     assert sum("/folded" in l["schedule"] for l in folded.launches) >= 3
     assert sum(b["elided"] for b in folded.buffers) > sum(b["elided"] for b in plain.buffers)
     ref = _cnn_step_on(frontend, "c", arrays)
     reg = _BACKENDS["hip"]
     old = reg.options
-    reg.options = {"gemm_fold": 1}
+    reg.options = {"gemm_fold": 0}
     try:
-        got = _cnn_step_on(frontend, "hip", arrays, True)
+        got_plain = _cnn_step_on(frontend, "hip", arrays, True)
     finally:
         reg.options = old
+    got = _cnn_step_on(frontend, "hip", arrays, True)
+    for g, p in zip(got, got_plain):
+        assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
     assert abs(float(got[-1][0]) - float(ref[-1][0])) <= 1e-5 * abs(float(ref[-1][0]))
     for g, r in zip(got[:-1], ref[:-1]):
         scale = max(float(np.abs(r).max()), 1e-6)
