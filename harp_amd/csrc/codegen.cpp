@@ -941,6 +941,77 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // A contraction per batch element whose results the next kernel sums over the batch (the
+  // weight gradient of a convolution: per-image products, then a sum over images) is one
+  // contraction with the batch folded into k, when both operands walk (batch, k) as one axis.
+  // The summing kernel disappears, and so does the per-batch result buffer.
+  std::set<size_t> absorbed;
+  std::map<size_t, std::string> absorbed_name;
+  if (opt.gemm && opt.gemm_merge_batch && have_table) {
+    for (size_t i = 0; i + 1 < kernels.size(); ++i) {
+      if (!nests[i] || !nests[i + 1]) continue;
+      const NestKernel& g0 = *nests[i];
+      const NestKernel& r2 = *nests[i + 1];
+      if (g0.rkind != ReduceKind::Sum || r2.rkind != ReduceKind::Sum || !gemm_shaped(g0, opt)) continue;
+      auto gs = match_gemm(g0);
+      if (!gs || gs->batch <= 1 || gs->a_b != gs->K * gs->a_k || gs->b_b != gs->K * gs->b_k) continue;
+      if (role_of(g0.out_buf) != "temp" || readers[g0.out_buf] != std::vector<size_t>{i + 1}) continue;
+      if (!r2.identity || r2.identity->fval != 0.0 || r2.acc_dtype.ty != Ty::F32 || r2.out_dtype.ty != Ty::F32) continue;
+      const Node& v = *r2.value;
+      if (v.op != Op::Load || v.args[0]->op != Op::Var || v.args[0]->name != g0.out_buf || v.count != 1) continue;
+      auto ra = affine_of(*v.args[1]);
+      if (!ra || !r2.out_aff || !g0.out_aff || ra->c != g0.out_aff->c) continue;
+      // the batch loop of g0: the one both operands move with
+      std::string bvar;
+      {
+        const Node& gv = *g0.value;
+        auto aa = affine_of(*gv.args[0]->args[1]);
+        auto ab = affine_of(*gv.args[1]->args[1]);
+        if (!aa || !ab) continue;
+        int nb = 0;
+        for (const auto& l : g0.loops)
+          if (l.extent > 1 && aa->of(l.var) != 0 && ab->of(l.var) != 0) { bvar = l.var; ++nb; }
+        if (nb != 1) continue;
+      }
+      // r2 must sum exactly that axis and keep the others: match loops by their stride in C
+      if (r2.rloop.extent != gs->batch || ra->of(r2.rloop.var) != g0.out_aff->of(bvar)) continue;
+      std::map<std::string, NodePtr> to_g0;     // r2's loop variables in terms of g0's
+      bool ok = true;
+      size_t matched = 0;
+      for (const auto& l2 : r2.loops) {
+        if (l2.extent <= 1) { to_g0[l2.var] = make_i64(0); continue; }
+        const Loop* hit = nullptr;
+        for (const auto& l0 : g0.loops)
+          if (l0.var != bvar && l0.extent == l2.extent && g0.out_aff->of(l0.var) == ra->of(l2.var)) hit = &l0;
+        if (!hit) { ok = false; break; }
+        to_g0[l2.var] = make_var(hit->var);
+        ++matched;
+      }
+      size_t live0 = 0;
+      for (const auto& l0 : g0.loops) live0 += (l0.extent > 1 && l0.var != bvar);
+      if (!ok || matched != live0) continue;
+      NestKernel m = g0;
+      m.value = rename(g0.value, {{bvar, make_i64(0)}});
+      m.rloop.extent = g0.rloop.extent * gs->batch;
+      for (auto& l : m.loops)
+        if (l.var == bvar) l.extent = 1;
+      m.out_buf = r2.out_buf;
+      m.out_dtype = r2.out_dtype;
+      m.out_index = rename(rename(r2.out_index, {{r2.rloop.var, make_i64(0)}}), to_g0);
+      m.out_aff = affine_of(*m.out_index);
+      for (const auto& p : r2.params)
+        if (p.mut_) {
+          for (auto& q : m.params)
+            if (q.mut_) q = p;
+        }
+      if (!m.out_aff || !gemm_shaped(m, opt)) continue;
+      plan.elided.insert(g0.out_buf);      // (g0 refers to nests[i]: use it before the assignment)
+      absorbed_name[i] = r2.name;
+      absorbed.insert(i + 1);
+      nests[i] = m;
+    }
+  }
+
   // gather / copy kernels read only by contractions are evaluated inside those contractions'
   // tile loaders (implicit GEMM): no launch, no buffer
   FoldMap folded;
@@ -969,7 +1040,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
 
   size_t i = 0;
   while (i < kernels.size()) {
-    if (folded_kernels.count(i)) {
+    if (folded_kernels.count(i) || absorbed.count(i)) {
       ++i;
       continue;
     }
@@ -1000,6 +1071,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           std::vector<size_t> taken;
           size_t j = i + 1;
           for (; j < kernels.size(); ++j) {
+            if (absorbed.count(j)) continue;
             if (!nests[j] || folded_kernels.count(j) || nests[j]->rkind != ReduceKind::None) break;
             const NestKernel& sk = *nests[j];
             int64_t numel = 0;
@@ -1129,6 +1201,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       }
       auto gl = try_emit_gemm(have_epi ? k0r : k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
       if (!gl.empty()) {
+        if (absorbed_name.count(i)) gl.back().kernels.push_back(absorbed_name[i]);
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
         i = have_epi ? after : i + 1;
         continue;

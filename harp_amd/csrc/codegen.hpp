@@ -27,6 +27,7 @@ struct GenOptions {
   int gemm_setprio = 0;               // wave priority during the multiply loop
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
+  bool gemm_merge_batch = false;      // per-batch contractions summed over the batch become one contraction
   bool gemm_epilogue = true;          // run elementwise consumers of a contraction on its accumulators
   bool gemm_fold = true;              // evaluate gather/copy producers inside the tile loader (implicit GEMM)
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks

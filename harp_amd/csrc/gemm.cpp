@@ -92,7 +92,7 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
   bool have = false;
   for (const auto& c : kCandidates) {
     const int64_t ksteps = ceil_div(s.K, c.tile.bk);
-    for (int split : {1, 2, 4, 8, 16, 32}) {
+    for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
       if (opt.gemm_split_k > 1 && split != 1) break;
       int sp = opt.gemm_split_k > 1 ? static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps)) : split;

@@ -82,7 +82,7 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
  *      arch, fuse, vectorize, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
- *      gemm_epilogue, gemm_dma, nontemporal. ----------------------------------------------- */
+ *      gemm_epilogue, gemm_dma, gemm_merge_batch, nontemporal. ----------------------------- */
 typedef struct eh_launch_info {
   const char* entry;                    /* kernel symbol */
   const char* source;                   /* HIP C translation unit */

@@ -482,6 +482,18 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
     got = _cnn_step_on(frontend, "hip", arrays, True)
     for g, p in zip(got, got_plain):
         assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
+    # option gemm_merge_batch=1: per-image weight-gradient contractions and the sum over images
+    # that follows become one contraction with the batch folded into k
+    merged = hip.render_program(prog_ast, {"gemm_merge_batch": 1})
+    assert len(merged.launches) < len(folded.launches)
+    reg.options = {"gemm_merge_batch": 1}
+    try:
+        got_merged = _cnn_step_on(frontend, "hip", arrays, True)
+    finally:
+        reg.options = old
+    for g, r in zip(got_merged[:-1], ref[:-1]):
+        scale = max(float(np.abs(r).max()), 1e-6)
+        assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
     assert abs(float(got[-1][0]) - float(ref[-1][0])) <= 1e-5 * abs(float(ref[-1][0]))
     for g, r in zip(got[:-1], ref[:-1]):
         scale = max(float(np.abs(r).max()), 1e-6)
