@@ -95,7 +95,10 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
     for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
       if (opt.gemm_split_k > 1 && split != 1) break;
-      int sp = opt.gemm_split_k > 1 ? static_cast<int>(std::min<int64_t>(opt.gemm_split_k, ksteps)) : split;
+      // a requested split is capped so that every chunk keeps at least eight k-steps
+      int sp = opt.gemm_split_k > 1
+                   ? static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(opt.gemm_split_k, ksteps / 8)))
+                   : split;
       if (sp > 1 && ksteps / sp < 8) break;
       double us = estimate_us(s, c, sp);
       if (!have || us < best_us) {
