@@ -1,0 +1,94 @@
+"""Seeded random tensor graphs for differential testing (HIP backend against the C oracle).
+
+Each graph is a short chain over one or two inputs drawn from the tensor API the benchmark
+configurations use: elementwise arithmetic and math, broadcasts, views (permute, reshape, pad,
+expand), reductions over any axis, row-wise normalisations and small contractions.  Values stay
+in a range where every op is well conditioned (no division by ~0, no overflow), so the
+tolerance classes of the parity tests apply.
+"""
+
+import numpy as np
+
+
+def _unary(rng, fe, t):
+    k = rng.integers(0, 7)
+    if k == 0:
+        return t.neg()
+    if k == 1:
+        return (t * t + fe.Tensor.ones_like(t)).sqrt()
+    if k == 2:
+        return (t * t + fe.Tensor.ones_like(t)).recip()
+    if k == 3:
+        return t.sin()
+    if k == 4:
+        return fe.nn.relu(t)
+    if k == 5:
+        return fe.nn.sigmoid(t)
+    return t.maximum(t.neg())
+
+
+def _binary(rng, a, b):
+    k = rng.integers(0, 5)
+    if k == 0:
+        return a + b
+    if k == 1:
+        return a * b
+    if k == 2:
+        return a - b
+    if k == 3:
+        return a.maximum(b)
+    return a.minimum(b)
+
+
+def build(seed: int, fe):
+    """Returns (input shapes, function of input tensors -> output tensor, description)."""
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(1, 4))
+    shape = [int(rng.choice([1, 2, 3, 5, 8, 13, 32, 64, 100])) for _ in range(nd)]
+    kind = int(rng.integers(0, 8))
+    has_y = bool(rng.integers(0, 2))
+    has_w = kind == 4 and nd >= 2
+
+    def fn(*ins):
+        x = ins[0]
+        y = ins[1] if has_y else None
+        r = np.random.default_rng(seed + 1)
+        t = x if y is None else _binary(r, x, y)       # every input is used
+        for _ in range(int(r.integers(1, 4))):
+            t = _unary(r, fe, t) if (y is None or r.integers(0, 2)) else _binary(r, t, y)
+        if kind == 0:                                   # reduce over a random axis
+            ax = int(r.integers(0, t.ndim()))
+            t = [t.sum, t.max, t.min][int(r.integers(0, 3))](ax)
+        elif kind == 1 and t.ndim() >= 2:               # permute then elementwise (gathering copy)
+            perm = list(r.permutation(t.ndim()))
+            t = _unary(r, fe, t.permute([int(p) for p in perm]).contiguous())
+        elif kind == 2:                                 # softmax / log-softmax over the last axis
+            ax = t.ndim() - 1
+            t = fe.nn.softmax(t, ax) if r.integers(0, 2) else fe.nn.log_softmax(t, ax)
+        elif kind == 3:                                 # pad, then reduce over the last axis
+            pads = [(int(r.integers(0, 3)), int(r.integers(0, 3))) for _ in range(t.ndim())]
+            t = t.pad(pads).contiguous()
+            t = t.sum(t.ndim() - 1)
+        elif kind == 4 and t.ndim() >= 2:               # contraction with a second operand
+            a = t.reshape([t.numel() // t.shape()[-1], t.shape()[-1]])
+            w = ins[-1]
+            t = fe.nn.linear(a, w)
+            t = _unary(r, fe, t)
+        elif kind == 5:                                 # broadcast against a row vector
+            v = t.sum(0).unsqueeze(0) if t.ndim() >= 2 else t
+            t = _binary(r, t, v.expand(0, t.shape()[0])) if t.ndim() >= 2 else _unary(r, fe, t)
+        elif kind == 6:                                 # reduce, then elementwise on the result
+            t = _unary(r, fe, t.sum(t.ndim() - 1))
+        else:                                           # reshape to rows of a different length
+            n = t.numel()
+            cols = [c for c in (1, 2, 4, 5, 8, 10, 16, 25) if n % c == 0]
+            c = int(r.choice(cols))
+            t = _unary(r, fe, t.reshape([n // c, c])).sum(1)
+        return t
+
+    shapes = [tuple(shape)]
+    if has_y:
+        shapes.append(tuple(shape))
+    if has_w:
+        shapes.append((int(rng.choice([3, 10, 33, 64])), shape[-1]))
+    return shapes, fn, f"seed {seed}: shape {shape}, kind {kind}"

@@ -548,3 +548,18 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
         assert np.allclose(got, ref, rtol=1e-6)
     else:
         assert bits_equal_mod_zero(ref, got)
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_graphs_match_the_oracle(frontend, hip, seed):
+    """Differential test on seeded random graphs (tests/graph_fuzz.py): elementwise chains,
+    views, reductions over any axis, row normalisations, small contractions.  Held to the
+    reduction tolerance (every graph may contain a sum)."""
+    import graph_fuzz
+    shapes, fn, desc = graph_fuzz.build(seed, frontend)
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    ref, got = both(frontend, fn, arrays, True)
+    assert ref.shape == got.shape, desc
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), desc
