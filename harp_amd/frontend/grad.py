@@ -393,7 +393,14 @@ def _elementwise_vjp_exact(node, g, m) -> List[Optional[GraphNode]]:
     if m.op == "select" and len(ins) == 3:
         z = _zeros_like(g)
         return [None, _select_dense(ins[0], g, z), _select_dense(ins[0], z, g)]
-    return _elementwise_vjp(node, g, m)                  # add, mul, neg, recip, sqrt, ln, sin, ...
+    if m.op == "select" and len(ins) == 2 and m.args[0].op == "lt" and _is_w(m.args[0].args[0], 0) and \
+            _is_w(m.args[0].args[1], 1) and _is_w(m.args[1], 0) and _is_w(m.args[2], 1):
+        z = _zeros_like(g)                               # minimum(a, b) = a < b ? a : b
+        cond = ins[0].lt(ins[1])
+        return [_select_dense(cond, g, z), _select_dense(cond, z, g)]
+    if categorize_map(m) not in ("add", "mul", "neg", "recip", "sqrt", "log", "sin", "floor", "cast", "comparison"):
+        raise NotImplementedError(f"no exact VJP for the elementwise map {m.to_sexpr()}")
+    return _elementwise_vjp(node, g, m)                  # rules that are right as written
 
 
 def _unfold_adjoint(g: GraphNode, op) -> GraphNode:

@@ -46,6 +46,7 @@ def build(seed: int, fe):
     nd = int(rng.integers(1, 4))
     shape = [int(rng.choice([1, 2, 3, 5, 8, 13, 32, 64, 100])) for _ in range(nd)]
     kind = int(rng.integers(0, 8))
+    red = int(rng.integers(0, 3))                        # kind 0: sum, max or min
     has_y = bool(rng.integers(0, 2))
     has_w = kind == 4 and nd >= 2
 
@@ -58,7 +59,7 @@ def build(seed: int, fe):
             t = _unary(r, fe, t) if (y is None or r.integers(0, 2)) else _binary(r, t, y)
         if kind == 0:                                   # reduce over a random axis
             ax = int(r.integers(0, t.ndim()))
-            t = [t.sum, t.max, t.min][int(r.integers(0, 3))](ax)
+            t = [t.sum, t.max, t.min][red](ax)
         elif kind == 1 and t.ndim() >= 2:               # permute then elementwise (gathering copy)
             perm = list(r.permutation(t.ndim()))
             t = _unary(r, fe, t.permute([int(p) for p in perm]).contiguous())
@@ -91,4 +92,5 @@ def build(seed: int, fe):
         shapes.append(tuple(shape))
     if has_w:
         shapes.append((int(rng.choice([3, 10, 33, 64])), shape[-1]))
-    return shapes, fn, f"seed {seed}: shape {shape}, kind {kind}"
+    what = f"kind {kind}" + (f" ({['sum', 'max', 'min'][red]})" if kind == 0 else "")
+    return shapes, fn, f"seed {seed}: shape {shape}, {what}"

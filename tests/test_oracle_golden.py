@@ -303,3 +303,82 @@ def test_exact_unfold_views_and_cnn_step(frontend):
     assert abs(float(got[-1][0]) - loss) <= 1e-6 * abs(loss)
     for g, r in zip(got[:-1], grads):
         assert np.allclose(g.reshape(r.shape), r, rtol=1e-4, atol=1e-7)
+
+
+def _one(t):
+    return type(t).ones_like(t)
+
+
+def _nn():
+    from harp_amd.frontend import nn
+    return nn
+
+
+def _tanh(t):
+    from harp_amd.workloads import tanh_exact
+    return tanh_exact(t)
+
+
+VJP_CASES = {
+    # name: (function of the input tensors, input shapes, finite-difference step)
+    "sub_mul": (lambda a, b: (a - b) * a, [(12, 7)] * 2, 1e-2),
+    "div": (lambda a, b: a / (b * b + _one(b)), [(12, 7)] * 2, 1e-2),
+    "sqrt_recip": (lambda a: (a * a + _one(a)).sqrt() * (a * a + _one(a)).recip(), [(12, 7)], 1e-2),
+    "exp_ln": (lambda a: a.exp() + (a * a + _one(a)).ln(), [(12, 7)], 1e-2),
+    "exp2_log2": (lambda a: a.exp2() + (a * a + _one(a)).log2(), [(12, 7)], 1e-2),
+    "sin_cos": (lambda a: a.sin() * a.cos(), [(12, 7)], 1e-2),
+    "maximum_minimum": (lambda a, b: a.maximum(b) + a.minimum(b) * a, [(12, 7)] * 2, 1e-3),
+    "reduce_sum_max_min": (lambda a: a.sum(1) * a.max(1) + a.min(0).sum(0).unsqueeze(0).expand(0, 12), [(12, 7)], 1e-3),
+    "prod": (lambda a: a.prod(1), [(6, 4)], 1e-3),
+    "views": (lambda a: (a.permute([1, 0]).contiguous().reshape([4, 21]) * a.reshape([4, 21])).sum(1), [(12, 7)], 1e-2),
+    "pad_unsqueeze_expand": (lambda a: a.pad([(1, 2), (0, 1)]).contiguous() * a.sum(0).unsqueeze(0).expand(0, 12).pad([(1, 2), (0, 1)]),
+                             [(12, 7)], 1e-2),
+    "softmax": (lambda a: _nn().softmax(a, 1) * a, [(12, 7)], 1e-2),
+    "log_softmax": (lambda a: _nn().log_softmax(a, 1) * a, [(12, 7)], 1e-2),
+    "linear_tanh": (lambda a, w, b: _tanh(_nn().linear(a, w, b)), [(12, 7), (5, 7), (5,)], 1e-2),
+    "unfold_windows": (lambda a: a.unfold([0, 1], [3, 3], [1, 1], [1, 1]).contiguous() *
+                       a.unfold([0, 1], [3, 3], [1, 1], [1, 1]).contiguous(), [(8, 7)], 1e-2),
+    "unfold_tiles": (lambda a: a.unfold([0, 1], [2, 3], [2, 3], [1, 1]).contiguous().reshape([4, 2, 6]).max(2),
+                     [(8, 6)], 1e-3),
+}
+
+
+@pytest.mark.parametrize("name", sorted(VJP_CASES))
+def test_exact_vjps_against_finite_differences(frontend, name):
+    """The exact-mode gradient rules are not the reference's, so nothing of the reference pins
+    them; calculus does: the directional derivative of sum(f) along a random direction, from
+    central differences of the oracle's own forward results, must equal <gradient, direction>."""
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    fn, shapes, h = VJP_CASES[name]
+    rng = np.random.default_rng(sum(map(ord, name)))
+    arrays = [(rng.uniform(0.3, 1.5, s) * rng.choice([-1.0, 1.0], s)).astype(np.float32) for s in shapes]
+    dirs = [rng.normal(0, 1, s).astype(np.float32) for s in shapes]
+
+    def total(*ts):
+        out = fn(*ts)
+        while out.ndim() > 0:
+            out = out.sum(out.ndim() - 1)
+        return out
+
+    def value(arrs):
+        with frontend.exact_mode():
+            return float(realize_on(frontend, "c", total, arrs)[0])
+
+    frontend.set_device_str("c")
+    try:
+        with frontend.exact_mode():
+            ts = []
+            for a in arrays:
+                t = frontend.Tensor.input(list(a.shape))
+                t.set_data(a)
+                ts.append(t)
+            loss = total(*ts)
+            loss.backward_with_params(ts)
+            grads = [t.grad().contiguous() for t in ts]
+            frontend.realize_many(grads)
+            grads = [g.to_numpy().astype(np.float64) for g in grads]
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+    numeric = (value([a + h * d for a, d in zip(arrays, dirs)]) - value([a - h * d for a, d in zip(arrays, dirs)])) / (2 * h)
+    analytic = sum(float((g.reshape(d.shape) * d).sum()) for g, d in zip(grads, dirs))
+    assert abs(numeric - analytic) <= 2e-2 * max(1.0, abs(numeric), abs(analytic)), (numeric, analytic)
