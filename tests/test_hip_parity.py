@@ -71,6 +71,60 @@ def test_floor_and_cast_bit_exact(frontend, hip):
     assert bits_equal_mod_zero(ref, got)
 
 
+OTHER_TYPES = {
+    # name: (graph, numpy dtype, value range, exact?)
+    "i32_mul_add": (lambda a, b: a * b + a, np.int32, 1000, True),
+    "i32_row_sum": (lambda a, b: (a * b).sum(1), np.int32, 1000, True),
+    "i32_max": (lambda a, b: a.maximum(b).max(1), np.int32, 1000, True),
+    "i64_add": (lambda a, b: a + b, np.int64, 2 ** 40, True),
+    "f64_mul_add": (lambda a, b: a * b + a, np.float64, 3.0, True),
+    "f64_row_sum": (lambda a, b: (a * b).sum(1), np.float64, 3.0, False),
+    # the C renderer names the float functions whatever the element type
+    # (crates/backend-c/src/renderer.rs:182-201), so the oracle's double sqrt and max go
+    # through single precision; the device code uses the double forms
+    "f64_sqrt": (lambda a, b: (a * a + b * b).sqrt(), np.float64, 3.0, False),
+    "f64_max": (lambda a, b: a.maximum(b), np.float64, 3.0, False),
+}
+
+
+@pytest.mark.parametrize("shape", [(5, 7), (64, 128), (33, 1000)])
+@pytest.mark.parametrize("name", sorted(OTHER_TYPES))
+def test_other_element_types(frontend, hip, name, shape):
+    """i32, i64 and f64 tensors through the same schedules (the benchmark configurations
+    are all fp32).  Integer results and double add/mul are bit-exact; what the oracle
+    computes in single precision, or sums in another order, is held to 1e-6."""
+    fn, dt, lim, exact = OTHER_TYPES[name]
+    rng = RNG(hash((name, shape)) % 2**32)
+    if np.issubdtype(dt, np.integer):
+        arrs = [rng.integers(-lim, lim, shape).astype(dt) for _ in range(2)]
+    else:
+        arrs = [rng.uniform(-lim, lim, shape).astype(dt) for _ in range(2)]
+    for fuse in (False, True):
+        ref, got = both(frontend, fn, arrs, fuse)
+        assert got.dtype == ref.dtype == dt
+        if exact:
+            assert np.array_equal(got, ref), (name, fuse)
+        else:
+            assert np.allclose(got, ref, rtol=1e-6, atol=1e-6), (name, fuse)
+
+
+def test_double_contraction_keeps_double_precision(frontend, hip):
+    """The MFMA schedule is fp32 only: a double contraction takes a generic reduce schedule
+    and keeps double accuracy."""
+    rng = RNG(9)
+    a, b = rng.uniform(-1, 1, (37, 64)), rng.uniform(-1, 1, (64, 29))
+    ref, got = both(frontend, lambda x, y: frontend.nn.matmul(x, y), [a, b])
+    assert got.dtype == np.float64
+    assert np.allclose(got, ref, rtol=1e-12, atol=1e-13)
+    assert np.allclose(got.reshape(37, 29), a @ b, rtol=1e-12, atol=1e-13)
+
+
+def test_cast_round_trip_bit_exact(frontend, hip):
+    x = RNG(8).normal(0, 50, (64, 96)).astype(np.float32)
+    ref, got = both(frontend, lambda t: t.cast(frontend.I32).cast(frontend.F32), [x])
+    assert np.array_equal(got, ref) and np.array_equal(got.reshape(x.shape), np.trunc(x))
+
+
 @pytest.mark.parametrize("shape,axis", [((8, 10), 1), ((33, 1000), 1), ((16, 4096), 1), ((5, 7, 64), 2),
                                         ((64, 48), 0), ((9, 130, 6), 1), ((1, 17), 1), ((17, 1), 1),
                                         ((300, 70000), 1)])
@@ -103,6 +157,33 @@ def test_softmax_and_log_softmax(frontend, hip, shape, fuse):
     assert np.allclose(got.reshape(-1, shape[-1]).sum(1), 1.0, atol=1e-5)
     ref, got = both(frontend, lambda t: frontend.nn.log_softmax(t, ax), [x], fuse)
     assert np.allclose(got, ref, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("shape", [(32, 512), (7, 33), (512, 4096)])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_layer_norm_rows(frontend, hip, shape, fuse):
+    """The graph of `crates/cli/examples/layer_norm.ecl`: two row sums, a square root and an
+    affine map.  The tensor API has no scalar constants, so 1/C and eps come in as vectors.
+    Fused, the ten lowered kernels are one row launch."""
+    R, C = shape
+    rng = RNG(R * 100 + C)
+    x = rng.normal(0.5, 2, shape).astype(np.float32)
+    gamma, beta = (rng.normal(1, 0.2, (C,)).astype(np.float32) for _ in range(2))
+    inv = np.full((R,), 1.0 / C, np.float32)
+    eps = np.full((R,), 1e-5, np.float32)
+
+    def layer_norm(t, g, b, inv_n, e):
+        mean = t.sum(1) * inv_n
+        centred = t - mean.unsqueeze(1).expand(1, C)
+        var = (centred * centred).sum(1) * inv_n
+        std = (var + e).sqrt()
+        return centred / std.unsqueeze(1).expand(1, C) * g.unsqueeze(0).expand(0, R) + b.unsqueeze(0).expand(0, R)
+
+    ref, got = both(frontend, layer_norm, [x, gamma, beta, inv, eps], fuse)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5)             # reduction class
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5) * gamma + beta
+    assert np.allclose(got.reshape(shape), want, rtol=1e-4, atol=1e-4)
 
 
 @pytest.mark.parametrize("fuse", [False, True])
