@@ -7,6 +7,21 @@ use std::ffi::{c_char, c_int, c_uint, c_void};
 #[repr(C)] pub struct eh_buffer { _p: [u8; 0] }
 #[repr(C)] pub struct eh_program { _p: [u8; 0] }
 #[repr(C)] pub struct eh_module { _p: [u8; 0] }
+#[repr(C)] pub struct eh_plan { _p: [u8; 0] }
+
+#[repr(C)]
+pub struct eh_launch_info {
+    pub entry: *const c_char,
+    pub source: *const c_char,
+    pub schedule: *const c_char,
+    pub grid: [c_uint; 3],
+    pub block: [c_uint; 3],
+    pub lds_bytes: c_uint,
+    pub n_args: c_int,
+    pub n_kernels: c_int,
+    pub algo_bytes: f64,
+    pub flops: f64,
+}
 
 #[repr(C)]
 pub struct eh_device_props {
@@ -25,6 +40,13 @@ pub struct eh_device_props {
 
 unsafe extern "C" {
     pub fn eh_last_error() -> *const c_char;
+    pub fn eh_free(p: *mut c_void);
+    pub fn eh_render_program(ast_text: *const c_char, options: *const c_char, out: *mut *mut eh_plan) -> c_int;
+    pub fn eh_plan_num_launches(plan: *mut eh_plan, n: *mut c_int) -> c_int;
+    pub fn eh_plan_launch(plan: *mut eh_plan, launch: c_int, out: *mut eh_launch_info) -> c_int;
+    pub fn eh_plan_release(plan: *mut eh_plan) -> c_int;
+    pub fn eh_compile_source(source: *const c_char, arch: *const c_char, blob: *mut *mut c_void,
+                             len: *mut usize) -> c_int;
     pub fn eh_device_count(count: *mut c_int) -> c_int;
     pub fn eh_device_open(index: c_int, out: *mut *mut eh_device) -> c_int;
     pub fn eh_device_close(dev: *mut eh_device) -> c_int;

@@ -17,7 +17,11 @@ use std::sync::Arc;
 use eclat::ast::{AstNode, DType};
 use eclat::backend::device::{BackendRegistry, DeviceError};
 use eclat::backend::global::DeviceKind;
-use eclat::backend::traits::{Buffer, Kernel, KernelConfig};
+use eclat::backend::renderer::Renderer;
+use eclat::backend::traits::{
+    Buffer, Compiler, Device, DeviceFeature, DeviceInstruction, DeviceProfile, DeviceType, Kernel, KernelConfig,
+    MatrixCapability, OpKind, SimdCapability,
+};
 use eclat::backend::KernelSignature;
 
 type DynErr = Box<dyn std::error::Error + Send + Sync>;
@@ -26,21 +30,87 @@ fn check(code: i32) -> Result<(), DynErr> {
     if code == 0 { Ok(()) } else { Err(ffi::last_error().into()) }
 }
 
-pub struct HipDevice { raw: *mut ffi::eh_device }
-unsafe impl Send for HipDevice {}
-unsafe impl Sync for HipDevice {}
-impl Drop for HipDevice { fn drop(&mut self) { unsafe { ffi::eh_device_close(self.raw); } } }
+struct DeviceHandle { raw: *mut ffi::eh_device }
+unsafe impl Send for DeviceHandle {}
+unsafe impl Sync for DeviceHandle {}
+impl Drop for DeviceHandle { fn drop(&mut self) { unsafe { ffi::eh_device_close(self.raw); } } }
 
-pub struct HipBuffer { raw: *mut ffi::eh_buffer, dev: Arc<HipDevice>, shape: Vec<usize>, dtype: DType, bytes: usize }
+/// One opened GPU; clones share the handle, which closes when the last clone (a device, a
+/// buffer or a kernel holds one each) is dropped.
+#[derive(Clone)]
+pub struct HipDevice { handle: Arc<DeviceHandle> }
+
+impl HipDevice {
+    pub fn open(index: usize) -> Result<Self, DynErr> {
+        let mut raw = std::ptr::null_mut();
+        check(unsafe { ffi::eh_device_open(index as i32, &mut raw) })?;
+        Ok(Self { handle: Arc::new(DeviceHandle { raw }) })
+    }
+    fn raw(&self) -> *mut ffi::eh_device { self.handle.raw }
+    fn props(&self) -> Option<ffi::eh_device_props> {
+        let mut p = std::mem::MaybeUninit::<ffi::eh_device_props>::zeroed();
+        if unsafe { ffi::eh_device_get_props(self.raw(), p.as_mut_ptr()) } != 0 { return None; }
+        Some(unsafe { p.assume_init() })
+    }
+}
+
+/// `Device` (src/backend/traits.rs:273-306).  The profile describes gfx950 as the library
+/// reports it; the AST-level parallelisation and matrix features are declined on purpose:
+/// this backend takes the kernels as lowered (sequential `Range` nests) and picks the
+/// work-item mapping, LDS staging and MFMA tiling itself while rendering.
+impl Device for HipDevice {
+    fn is_available() -> bool {
+        let mut n = 0;
+        unsafe { ffi::eh_device_count(&mut n) == 0 && n > 0 }
+    }
+    fn profile(&self) -> DeviceProfile {
+        let (cus, wave, max_wg, lds) = match self.props() {
+            Some(p) => (p.compute_units as usize, p.warp_size as usize, p.max_work_group_size as usize, p.local_memory_size),
+            None => (256, 64, 1024, 160 * 1024),
+        };
+        let mut simd = Vec::new();
+        for op in [OpKind::Add, OpKind::Mul, OpKind::Fma, OpKind::Compare, OpKind::Load, OpKind::Store] {
+            simd.push(SimdCapability::new(DType::F32, op, 4));      // 16-byte global accesses
+        }
+        DeviceProfile {
+            device_type: DeviceType::DiscreteGpu,
+            compute_units: cus,
+            max_work_group_size: max_wg,
+            preferred_work_group_size_range: (wave, 256),
+            local_memory_size: lds,
+            warp_size: wave,
+            preferred_tile_sizes: vec![16, 32, 64, 128, 256],
+            simd_capabilities: simd,
+            // v_mfma_f32_32x32x2_f32 and v_mfma_f32_16x16x4_f32
+            matrix_capabilities: vec![MatrixCapability::new(DType::F32, DType::F32, 32, 32, 2),
+                                      MatrixCapability::new(DType::F32, DType::F32, 16, 16, 4)],
+        }
+    }
+    fn supports_feature(&self, feature: DeviceFeature) -> bool {
+        match feature {
+            DeviceFeature::FastMath | DeviceFeature::HalfPrecision | DeviceFeature::DoublePrecision
+            | DeviceFeature::LocalMemory | DeviceFeature::AtomicOperations | DeviceFeature::SubgroupOperations => true,
+            DeviceFeature::ParallelKernel | DeviceFeature::MatrixOperations => false,
+        }
+    }
+    fn supports_instruction(&self, instruction: DeviceInstruction) -> bool {
+        match instruction {
+            DeviceInstruction::Fma | DeviceInstruction::Rsqrt | DeviceInstruction::AtomicAddFloat
+            | DeviceInstruction::NativeDiv | DeviceInstruction::NativeExpLog => true,
+        }
+    }
+}
+
+pub struct HipBuffer { raw: *mut ffi::eh_buffer, dev: HipDevice, shape: Vec<usize>, dtype: DType, bytes: usize }
 unsafe impl Send for HipBuffer {}
 unsafe impl Sync for HipBuffer {}
 impl Drop for HipBuffer { fn drop(&mut self) { unsafe { ffi::eh_buffer_release(self.raw); } } }
 
 impl HipBuffer {
-    fn allocate(dev: &Arc<HipDevice>, shape: Vec<usize>, dtype: DType) -> Result<Self, DynErr> {
+    fn allocate(dev: &HipDevice, shape: Vec<usize>, dtype: DType) -> Result<Self, DynErr> {
         let bytes = shape.iter().product::<usize>() * dtype.size_in_bytes();
         let mut raw = std::ptr::null_mut();
-        check(unsafe { ffi::eh_buffer_alloc(dev.raw, bytes, &mut raw) })?;   // zero-filled
+        check(unsafe { ffi::eh_buffer_alloc(dev.raw(), bytes, &mut raw) })?;   // zero-filled
         Ok(Self { raw, dev: dev.clone(), shape, dtype, bytes })
     }
 }
@@ -69,7 +139,7 @@ impl Buffer for HipBuffer {
 
 enum Loaded { Program(*mut ffi::eh_program), Module(*mut ffi::eh_module) }
 
-pub struct HipKernel { loaded: Loaded, config: KernelConfig, ast_text: Option<Arc<String>>, dev: Arc<HipDevice> }
+pub struct HipKernel { loaded: Loaded, config: KernelConfig, ast_text: Option<Arc<String>>, dev: HipDevice }
 unsafe impl Send for HipKernel {}
 unsafe impl Sync for HipKernel {}
 impl Drop for HipKernel {
@@ -130,17 +200,78 @@ impl Kernel for HipKernel {
     }
 }
 
-fn compile_text(dev: &Arc<HipDevice>, text: Arc<String>, config: KernelConfig) -> Result<HipKernel, DynErr> {
+fn compile_text(dev: &HipDevice, text: Arc<String>, config: KernelConfig) -> Result<HipKernel, DynErr> {
     let c = CString::new(text.as_str())?;
     let mut raw = std::ptr::null_mut();
-    check(unsafe { ffi::eh_program_compile(dev.raw, c.as_ptr(), std::ptr::null(), &mut raw) })?;
+    check(unsafe { ffi::eh_program_compile(dev.raw(), c.as_ptr(), std::ptr::null(), &mut raw) })?;
     Ok(HipKernel { loaded: Loaded::Program(raw), config, ast_text: Some(text), dev: dev.clone() })
+}
+
+/// `Renderer` (src/backend/renderer.rs:20-35): AST -> HIP C, no device involved.  The text is
+/// every launch's translation unit in launch order; dispatch sizes come with the plan
+/// (`eh_plan_launch`), not from the AST's grid fields.
+#[derive(Default)]
+pub struct HipRenderer { options: Option<String> }
+
+impl Renderer for HipRenderer {
+    type CodeRepr = String;
+    type Option = String;          // "key=value,..." as `eh_render_program` takes it
+    fn render(&self, program: &AstNode) -> String {
+        let Ok(text) = CString::new(ser::to_text(program)) else { return String::new(); };
+        let opts = self.options.as_ref().and_then(|o| CString::new(o.as_str()).ok());
+        let mut plan = std::ptr::null_mut();
+        let optr = opts.as_ref().map_or(std::ptr::null(), |o| o.as_ptr());
+        if unsafe { ffi::eh_render_program(text.as_ptr(), optr, &mut plan) } != 0 {
+            return format!("/* {} */", ffi::last_error());
+        }
+        let mut out = String::new();
+        let mut n = 0;
+        unsafe {
+            ffi::eh_plan_num_launches(plan, &mut n);
+            for i in 0..n {
+                let mut info = std::mem::MaybeUninit::<ffi::eh_launch_info>::zeroed();
+                if ffi::eh_plan_launch(plan, i, info.as_mut_ptr()) == 0 {
+                    out.push_str(&std::ffi::CStr::from_ptr(info.assume_init().source).to_string_lossy());
+                    out.push('\n');
+                }
+            }
+            ffi::eh_plan_release(plan);
+        }
+        out
+    }
+    fn is_available(&self) -> bool { true }     // rendering needs no GPU
+    fn with_option(&mut self, option: String) { self.options = Some(option); }
+}
+
+/// `Compiler` (src/backend/traits.rs:592-607): HIP C source -> gfx950 code object with hiprtc,
+/// loaded as one entry point; `config` carries the entry name and the dispatch sizes.
+pub struct HipCompiler;
+
+impl Compiler for HipCompiler {
+    type Dev = HipDevice;
+    type Kernel = HipKernel;
+    type Error = std::io::Error;
+    fn new() -> Self { HipCompiler }
+    fn compile(&self, device: &HipDevice, source: &str, config: KernelConfig) -> Result<HipKernel, std::io::Error> {
+        let err = |m: String| std::io::Error::new(std::io::ErrorKind::Other, m);
+        let src = CString::new(source).map_err(|e| err(e.to_string()))?;
+        let entry = CString::new(config.entry_point.as_str()).map_err(|e| err(e.to_string()))?;
+        let (mut blob, mut len) = (std::ptr::null_mut(), 0usize);
+        if unsafe { ffi::eh_compile_source(src.as_ptr(), std::ptr::null(), &mut blob, &mut len) } != 0 {
+            return Err(err(ffi::last_error()));
+        }
+        let mut raw = std::ptr::null_mut();
+        let rc = unsafe { ffi::eh_module_load(device.raw(), blob, len, entry.as_ptr(), &mut raw) };
+        unsafe { ffi::eh_free(blob); }
+        if rc != 0 { return Err(err(ffi::last_error())); }
+        Ok(HipKernel { loaded: Loaded::Module(raw), config, ast_text: None, dev: device.clone() })
+    }
 }
 
 struct HipBackendRegistry;
 
-fn device_of(device: &dyn Any) -> Result<&Arc<HipDevice>, DeviceError> {
-    device.downcast_ref::<Arc<HipDevice>>()
+fn device_of(device: &dyn Any) -> Result<&HipDevice, DeviceError> {
+    device.downcast_ref::<HipDevice>()
         .ok_or_else(|| DeviceError::InitializationError("Invalid device type: expected HipDevice".into()))
 }
 
@@ -152,11 +283,8 @@ impl BackendRegistry for HipBackendRegistry {
         unsafe { ffi::eh_device_count(&mut n) == 0 && n > 0 }
     }
     fn create_device(&self, index: usize) -> Result<Arc<dyn Any + Send + Sync>, DeviceError> {
-        let mut raw = std::ptr::null_mut();
-        if unsafe { ffi::eh_device_open(index as i32, &mut raw) } != 0 {
-            return Err(DeviceError::InitializationError(ffi::last_error()));
-        }
-        Ok(Arc::new(Arc::new(HipDevice { raw })))
+        HipDevice::open(index).map(|d| Arc::new(d) as Arc<dyn Any + Send + Sync>)
+            .map_err(|e| DeviceError::InitializationError(e.to_string()))
     }
     fn list_devices(&self) -> Vec<String> {
         let mut n = 0;
@@ -183,7 +311,7 @@ impl BackendRegistry for HipBackendRegistry {
         let dev = device_of(device)?;
         let entry = CString::new(config.entry_point.as_str()).map_err(|e| DeviceError::InitializationError(e.to_string()))?;
         let mut raw = std::ptr::null_mut();
-        if unsafe { ffi::eh_module_load(dev.raw, binary.as_ptr().cast(), binary.len(), entry.as_ptr(), &mut raw) } != 0 {
+        if unsafe { ffi::eh_module_load(dev.raw(), binary.as_ptr().cast(), binary.len(), entry.as_ptr(), &mut raw) } != 0 {
             return Err(DeviceError::InitializationError(ffi::last_error()));
         }
         Ok(Box::new(HipKernel { loaded: Loaded::Module(raw), config, ast_text: None, dev: dev.clone() }))
