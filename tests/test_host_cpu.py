@@ -23,6 +23,26 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib.eh_version() >= 100
 
 
+def test_rust_binding_names_only_declared_symbols():
+    """The Rust shim (never compiled here) may only bind what the header declares, with the
+    same number of parameters."""
+    with open(os.path.join(ROOT, "include", "eclat_hip.h")) as f:
+        header = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    with open(os.path.join(ROOT, "crates", "backend-hip", "src", "ffi.rs")) as f:
+        ffi = f.read()
+
+    def arity(params):
+        params = params.strip()
+        return 0 if params in ("", "void") else params.count(",") + 1
+
+    declared = {m.group(1): arity(m.group(2)) for m in re.finditer(r"\b(eh_[a-z_0-9]+)\s*\(([^)]*)\)", header)}
+    bound = {m.group(1): arity(m.group(2)) for m in re.finditer(r"pub fn (eh_[a-z_0-9]+)\(([^)]*)\)", ffi)}
+    assert len(bound) >= 15
+    for name, n in bound.items():
+        assert name in declared, f"{name} bound in ffi.rs but not declared in eclat_hip.h"
+        assert declared[name] == n, f"{name}: {n} parameters in ffi.rs, {declared[name]} in the header"
+
+
 def _program_with_table(fe, tensor):
     from harp_amd.frontend.executor import buffer_table
     from harp_amd.frontend.graph import collect_inputs
