@@ -1316,6 +1316,11 @@ struct ExtLoad {
   bool cached = false;   // held in registers for the whole row
 };
 
+// Index arithmetic is done in 32-bit `int` while every index, every loop counter and the
+// grid-stride increments added to them (a grid's worth of work-items times the vector width)
+// stay well below 2^31; from 2^30 reachable elements on, kernels use 64-bit indices.
+constexpr int64_t kIndex32Limit = int64_t{1} << 30;
+
 struct GroupEmitter {
   const Group& g;
   const GenOptions& opt;
@@ -1381,7 +1386,7 @@ struct GroupEmitter {
         need[st.out_buf] = std::max(need[st.out_buf], top + 1);
       }
     }
-    if (reach >= (int64_t{1} << 31) - 8 || g.R() * g.C >= (int64_t{1} << 31) - 8) idx64 = true;
+    if (reach >= kIndex32Limit || g.R() * g.C >= kIndex32Limit) idx64 = true;
   }
   static const std::vector<Loop>& loads_loops(const std::vector<Loop>& l) { return l; }
 
@@ -1739,7 +1744,7 @@ struct SerialReduce {
       if (!a) { idx64 = true; break; }
       reach = std::max(reach, max_abs_index(*a, k.loops, &k.rloop));
     }
-    if (reach >= (int64_t{1} << 31) - 8 || N >= (int64_t{1} << 31) - 8) idx64 = true;
+    if (reach >= kIndex32Limit || N >= kIndex32Limit) idx64 = true;
   }
 
   std::string params(LaunchSpec* ls, bool with_out, const std::string& extra) const {

@@ -297,6 +297,25 @@ def test_gathering_copies_bit_exact(frontend, hip, name, shape):
     assert bits_equal_mod_zero(ref, got)
 
 
+def test_tensor_beyond_32_bit_indices(frontend, hip):
+    """2^31 + 262 144 elements (8.6 GB of fp32): element and row indices leave the 32-bit
+    range, so the generated kernels must switch to 64-bit index arithmetic.  Elementwise
+    result bit-exact, row maxima exact, row sums in the reduction class."""
+    rows, cols = 65544, 32768
+    block = RNG(31).normal(0, 1, (rows // 8, cols)).astype(np.float32)
+    x = np.tile(block, (8, 1))
+    del block
+    ref, got = both(frontend, lambda t: t * t + t, [x])
+    assert got.size == rows * cols > 2 ** 31
+    assert bits_equal_mod_zero(ref, got)
+    assert np.array_equal(got[-cols:], (x[-1] * x[-1] + x[-1]))          # the very last row
+    del ref, got
+    ref, got = both(frontend, lambda t: t.max(1), [x])
+    assert np.array_equal(ref, got) and np.array_equal(got, x.max(1))
+    ref, got = both(frontend, lambda t: t.sum(1), [x])
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(x[:64]).sum(1).max())
+
+
 def test_buffer_roundtrip_and_size_check(hip):
     dev = hip.HipDevice(0)
     from harp_amd.frontend import F32
