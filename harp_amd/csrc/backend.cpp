@@ -2,12 +2,16 @@
 
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
+#include <unistd.h>
 
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <list>
+#include <mutex>
 #include <sstream>
+#include <thread>
 #include <unordered_map>
 
 namespace eh {
@@ -42,8 +46,40 @@ void mkdirs(const std::string& path) {
   }
 }
 
-std::mutex g_bin_mu;
-std::unordered_map<std::string, std::shared_ptr<Binary>> g_bin_cache;
+// In-memory code objects, least recently used first out; the capacity is the reference's
+// kernel-cache capacity (src/backend/cache/store.rs:116-168).
+class BinaryCache {
+ public:
+  static constexpr size_t kCapacity = 1024;
+  std::shared_ptr<Binary> find(const std::string& key) {
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = index_.find(key);
+    if (it == index_.end()) return nullptr;
+    order_.splice(order_.begin(), order_, it->second);      // now the most recently used
+    return it->second->second;
+  }
+  void insert(const std::string& key, std::shared_ptr<Binary> bin) {
+    std::lock_guard<std::mutex> lk(mu_);
+    auto it = index_.find(key);
+    if (it != index_.end()) {
+      it->second->second = std::move(bin);
+      order_.splice(order_.begin(), order_, it->second);
+      return;
+    }
+    order_.emplace_front(key, std::move(bin));
+    index_[key] = order_.begin();
+    while (order_.size() > kCapacity) {
+      index_.erase(order_.back().first);
+      order_.pop_back();
+    }
+  }
+
+ private:
+  std::mutex mu_;
+  std::list<std::pair<std::string, std::shared_ptr<Binary>>> order_;
+  std::unordered_map<std::string, std::list<std::pair<std::string, std::shared_ptr<Binary>>>::iterator> index_;
+};
+BinaryCache g_bin_cache;
 
 }  // namespace
 
@@ -76,11 +112,7 @@ Binary HipCompiler::compile(const std::string& source, const std::string& arch, 
   for (const auto& o : opts) key_text += "\n" + o;
   key_text += "\nhiprtc " + std::to_string(maj) + "." + std::to_string(min);
   const std::string key = hash_hex(key_text);
-  {
-    std::lock_guard<std::mutex> lk(g_bin_mu);
-    auto it = g_bin_cache.find(key);
-    if (it != g_bin_cache.end()) return *it->second;
-  }
+  if (auto hit = g_bin_cache.find(key)) return *hit;
   const bool disk = use_disk_cache && disk_cache_enabled();
   const std::string path = cache_dir() + "/" + key + ".bin";
   Binary out;
@@ -115,7 +147,9 @@ Binary HipCompiler::compile(const std::string& source, const std::string& arch, 
     hiprtcDestroyProgram(&prog);
     if (disk) {
       mkdirs(cache_dir());
-      const std::string tmp = path + ".tmp" + std::to_string(reinterpret_cast<uintptr_t>(&out) & 0xffff);
+      // private name, then an atomic rename: concurrent writers of one key never share a file
+      const std::string tmp = path + ".tmp" + std::to_string(static_cast<long>(::getpid())) + "_" +
+                              std::to_string(std::hash<std::thread::id>{}(std::this_thread::get_id()) & 0xffffff);
       std::ofstream f(tmp, std::ios::binary);
       if (f) {
         f.write(out.code.data(), static_cast<std::streamsize>(out.code.size()));
@@ -127,10 +161,7 @@ Binary HipCompiler::compile(const std::string& source, const std::string& arch, 
       }
     }
   }
-  {
-    std::lock_guard<std::mutex> lk(g_bin_mu);
-    g_bin_cache[key] = std::make_shared<Binary>(out);
-  }
+  g_bin_cache.insert(key, std::make_shared<Binary>(out));
   return out;
 }
 
