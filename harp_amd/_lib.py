@@ -58,6 +58,7 @@ _SIGS = {
     "eh_device_close": ([_P], c_int),
     "eh_device_get_props": ([_P, POINTER(DeviceProps)], c_int),
     "eh_device_sync": ([_P], c_int),
+    "eh_device_trim": ([_P, POINTER(c_size_t)], c_int),
     "eh_buffer_alloc": ([_P, c_size_t, POINTER(_P)], c_int),
     "eh_buffer_retain": ([_P], c_int),
     "eh_buffer_release": ([_P], c_int),

@@ -114,6 +114,12 @@ class HipDevice:
     def sync(self) -> None:
         check(lib.eh_device_sync(self._h))
 
+    def trim(self) -> int:
+        """Returns the memory of released buffers to the driver; gives the bytes that were kept."""
+        kept = c_size_t(0)
+        check(lib.eh_device_trim(self._h, byref(kept)))
+        return kept.value
+
     def alloc(self, nbytes: int) -> "HipBuffer":
         return HipBuffer(self, [nbytes], None, nbytes=nbytes)
 
@@ -141,6 +147,11 @@ class HipBuffer:
 
     def byte_len(self) -> int:
         return self._nbytes
+
+    def device_ptr(self) -> int:
+        p = c_void_p()
+        check(lib.eh_buffer_device_ptr(self._h, byref(p)))
+        return p.value or 0
 
     def write_from_host(self, raw) -> None:
         raw = bytes(raw) if not isinstance(raw, (bytes, bytearray)) else raw

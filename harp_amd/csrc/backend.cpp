@@ -199,14 +199,63 @@ HipDevice::HipDevice(int index) : index_(index) {
   profile_.memory_bus_bits = p.memoryBusWidth;
   profile_.l2_bytes = p.l2CacheSize;
   check(hipStreamCreate(&stream_), "hipStreamCreate");
+  pool_limit_ = std::getenv("ECLAT_HIP_NO_POOL") ? 0 : profile_.global_memory_size / 4;
 }
 
 HipDevice::~HipDevice() {
   if (stream_) {
     (void)hipSetDevice(index_);
     (void)hipStreamSynchronize(stream_);
+    for (auto& kv : pool_) (void)hipFree(kv.second);
     (void)hipStreamDestroy(stream_);
   }
+}
+
+void* HipDevice::allocate(size_t bytes) {
+  {
+    std::lock_guard<std::mutex> lk(pool_mu_);
+    auto it = pool_.find(bytes);
+    if (it != pool_.end()) {
+      void* p = it->second;
+      pool_.erase(it);
+      pooled_bytes_ -= bytes;
+      return p;
+    }
+  }
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes);
+  if (e == hipErrorOutOfMemory) {      // give the kept blocks back and try once more
+    (void)hipGetLastError();
+    trim();
+    e = hipMalloc(&p, bytes);
+  }
+  check(e, "hipMalloc");
+  return p;
+}
+
+void HipDevice::release(void* ptr, size_t bytes) {
+  {
+    std::lock_guard<std::mutex> lk(pool_mu_);
+    if (pooled_bytes_ + bytes <= pool_limit_) {
+      pool_.emplace(bytes, ptr);
+      pooled_bytes_ += bytes;
+      return;
+    }
+  }
+  (void)hipStreamSynchronize(stream_);
+  (void)hipFree(ptr);
+}
+
+void HipDevice::trim() {
+  std::multimap<size_t, void*> blocks;
+  {
+    std::lock_guard<std::mutex> lk(pool_mu_);
+    blocks.swap(pool_);
+    pooled_bytes_ = 0;
+  }
+  if (blocks.empty()) return;
+  (void)hipStreamSynchronize(stream_);
+  for (auto& kv : blocks) (void)hipFree(kv.second);
 }
 
 void HipDevice::make_current() const { check(hipSetDevice(index_), "hipSetDevice"); }
@@ -223,10 +272,10 @@ std::shared_ptr<HipKernel> HipDevice::load(const Binary& bin, const std::string&
 HipBuffer::HipBuffer(HipDevice* dev, size_t bytes) : dev_(dev), bytes_(bytes) {
   dev_->make_current();
   if (bytes_ == 0) return;
-  check(hipMalloc(&ptr_, bytes_), "hipMalloc");
+  ptr_ = dev_->allocate(bytes_);
   hipError_t e = hipMemsetAsync(ptr_, 0, bytes_, dev_->stream());
   if (e != hipSuccess) {
-    (void)hipFree(ptr_);
+    dev_->release(ptr_, bytes_);
     check(e, "hipMemsetAsync");
   }
 }
@@ -234,8 +283,7 @@ HipBuffer::HipBuffer(HipDevice* dev, size_t bytes) : dev_(dev), bytes_(bytes) {
 HipBuffer::~HipBuffer() {
   if (ptr_) {
     (void)hipSetDevice(dev_->index());
-    (void)hipStreamSynchronize(dev_->stream());
-    (void)hipFree(ptr_);
+    dev_->release(ptr_, bytes_);
   }
 }
 

@@ -61,10 +61,23 @@ class HipDevice {
   // Loads a code object and resolves one entry point; modules are shared per (binary, entry).
   std::shared_ptr<HipKernel> load(const Binary& bin, const std::string& entry);
 
+  // Device memory for buffers.  Released blocks are kept (up to a quarter of the device's
+  // memory) and handed out again to requests of the same size without a hipMalloc/hipFree
+  // pair and its device-wide wait: every use of a block is queued on this device's one
+  // stream, so the next owner's work runs after the previous owner's.  ECLAT_HIP_NO_POOL
+  // set in the environment turns the reuse off.
+  void* allocate(size_t bytes);
+  void release(void* ptr, size_t bytes);
+  void trim();                         // returns every kept block to the driver
+  size_t pooled_bytes() const { return pooled_bytes_; }
+
  private:
   int index_;
   hipStream_t stream_ = nullptr;
   DeviceProfile profile_;
+  std::mutex pool_mu_;
+  std::multimap<size_t, void*> pool_;  // size -> free block
+  size_t pooled_bytes_ = 0, pool_limit_ = 0;
 };
 
 class HipBuffer {

@@ -144,6 +144,14 @@ int eh_device_sync(eh_device* dev) {
   return guard([&] { dev->dev.synchronize(); });
 }
 
+int eh_device_trim(eh_device* dev, size_t* kept_bytes) {
+  REQUIRE(dev, "device is NULL");
+  return guard([&] {
+    if (kept_bytes) *kept_bytes = dev->dev.pooled_bytes();
+    dev->dev.trim();
+  });
+}
+
 int eh_buffer_alloc(eh_device* dev, size_t bytes, eh_buffer** out) {
   REQUIRE(dev && out, "device or out is NULL");
   return guard([&] { *out = new eh_buffer(&dev->dev, bytes); });

@@ -68,6 +68,12 @@ int eh_device_sync(eh_device* dev);     /* waits for everything queued on the de
  *      read_to_host, clone_buffer (src/backend/traits.rs:455-482;
  *      crates/backend-c/src/buffer.rs:84-131); BackendRegistry::allocate_buffer
  *      (src/backend/device.rs:132-134) -------------------------------------------------------- */
+/* Released buffers' memory is kept by the device (up to a quarter of its memory) and reused by
+ * later allocations of the same size, so the executor's allocate-per-kernel pattern
+ * (src/backend/executor.rs:313-332) costs no hipMalloc/hipFree after the first pass.
+ * eh_device_trim gives the kept blocks back to the driver; *kept_bytes (may be NULL) receives
+ * how much was kept before.  ECLAT_HIP_NO_POOL in the environment turns the reuse off. */
+int eh_device_trim(eh_device* dev, size_t* kept_bytes);
 int eh_buffer_alloc(eh_device* dev, size_t bytes, eh_buffer** out);
 int eh_buffer_retain(eh_buffer* buf);
 int eh_buffer_release(eh_buffer* buf);

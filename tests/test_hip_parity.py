@@ -332,6 +332,25 @@ def test_buffer_roundtrip_and_size_check(hip):
     assert dev.props["arch"].startswith("gfx9") and dev.props["warp_size"] == 64
 
 
+def test_released_memory_is_reused_and_zero_filled(hip):
+    """A released buffer's block serves the next allocation of the same size; the new buffer
+    is zero-filled all the same.  Trimming hands the kept blocks back."""
+    dev = hip.HipDevice(0)
+    dev.trim()
+    n = 1 << 20
+    a = dev.alloc(n)
+    a.write_array(np.full(n, 0xAB, np.uint8))
+    ptr = a.device_ptr()
+    del a
+    b = dev.alloc(n)
+    assert b.device_ptr() == ptr
+    assert not b.read_array(np.uint8).any()
+    c = dev.alloc(n)                      # b still lives: another block
+    assert c.device_ptr() != ptr
+    del b, c
+    assert dev.trim() == 2 * n and dev.trim() == 0
+
+
 def test_undersized_buffer_is_rejected_before_launch(frontend, hip):
     dev = hip.HipDevice(0)
     a = frontend.Tensor.input([64, 64])
