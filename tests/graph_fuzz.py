@@ -40,11 +40,15 @@ def _binary(rng, a, b):
     return a.minimum(b)
 
 
-def build(seed: int, fe):
+SMALL_DIMS = (1, 2, 3, 5, 8, 13, 32, 64, 100)
+LARGE_DIMS = (1, 4, 31, 128, 257, 1000, 2048)      # with at most two axes: up to 4 Mi elements
+
+
+def build(seed: int, fe, dims=SMALL_DIMS, max_rank=3):
     """Returns (input shapes, function of input tensors -> output tensor, description)."""
     rng = np.random.default_rng(seed)
-    nd = int(rng.integers(1, 4))
-    shape = [int(rng.choice([1, 2, 3, 5, 8, 13, 32, 64, 100])) for _ in range(nd)]
+    nd = int(rng.integers(1, max_rank + 1))
+    shape = [int(rng.choice(dims)) for _ in range(nd)]
     kind = int(rng.integers(0, 8))
     red = int(rng.integers(0, 3))                        # kind 0: sum, max or min
     has_y = bool(rng.integers(0, 2))

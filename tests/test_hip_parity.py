@@ -684,6 +684,21 @@ def test_random_graphs_match_the_oracle(frontend, hip, seed):
     assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), desc
 
 
+@pytest.mark.parametrize("seed", range(5000, 5012))
+def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
+    """The same generator with one or two axes of up to 2048 elements: vectorised accesses,
+    rows held in registers or LDS, multi-block reductions, MFMA contractions with edges."""
+    import graph_fuzz
+    shapes, fn, desc = graph_fuzz.build(seed, frontend, dims=graph_fuzz.LARGE_DIMS, max_rank=2)
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    for fuse in (True, False):
+        ref, got = both(frontend, fn, arrays, fuse)
+        assert ref.shape == got.shape, desc
+        scale = max(1.0, float(np.abs(ref).max()))
+        assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
+
+
 def _grads_on(fe, kind, shapes, fn, arrays):
     """Exact-mode gradients of sum(fn(inputs)) with respect to every input, plus the sum,
     realized together.  Returns None when the graph uses an op without an exact VJP."""
