@@ -98,3 +98,33 @@ def build(seed: int, fe, dims=SMALL_DIMS, max_rank=3):
         shapes.append((int(rng.choice([3, 10, 33, 64])), shape[-1]))
     what = f"kind {kind}" + (f" ({['sum', 'max', 'min'][red]})" if kind == 0 else "")
     return shapes, fn, f"seed {seed}: shape {shape}, {what}"
+
+
+def build_cnn(seed: int, fe):
+    """A random small convolutional classifier: conv (1x1, 2x2 or 3x3, optional padding and
+    bias) + relu, optional 2x2 max-pool, flatten, linear, log-softmax.  Returns
+    (input shapes, function -> [batch, classes] log-probabilities, description)."""
+    rng = np.random.default_rng(seed)
+    b, cin = int(rng.choice([1, 2, 5])), int(rng.choice([1, 3, 4]))
+    h, w = int(rng.choice([6, 8, 12])), int(rng.choice([6, 9, 12]))
+    cout, k = int(rng.choice([2, 5, 8, 33])), int(rng.choice([1, 2, 3]))
+    pad = int(rng.integers(0, 2)) if k == 3 else 0
+    use_bias = bool(rng.integers(0, 2))
+    ho, wo = h + 2 * pad - k + 1, w + 2 * pad - k + 1
+    pool = bool(rng.integers(0, 2)) and ho % 2 == 0 and wo % 2 == 0
+    hp, wp = (ho // 2, wo // 2) if pool else (ho, wo)
+    feat, classes = cout * hp * wp, int(rng.choice([3, 10]))
+
+    def fn(x, w1, w2, b2, *rest):
+        y = fe.nn.relu(fe.nn.conv2d(x, w1, rest[0] if use_bias else None, padding=(pad, pad)))
+        if pool:
+            y = fe.nn.max_pool2d(y, (2, 2))
+        y = y.contiguous().reshape([b, feat])
+        return fe.nn.log_softmax(fe.nn.linear(y, w2, b2), 1)
+
+    shapes = [(b, cin, h, w), (cout, cin, k, k), (classes, feat), (classes,)]
+    if use_bias:
+        shapes.append((cout,))
+    desc = (f"seed {seed}: x {shapes[0]}, conv {cout}x{cin}x{k}x{k} pad {pad} bias {use_bias}, "
+            f"pool {pool}, classes {classes}")
+    return shapes, fn, desc

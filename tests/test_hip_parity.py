@@ -699,6 +699,29 @@ def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
         assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
 
 
+@pytest.mark.parametrize("seed", range(400, 412))
+def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
+    """Random conv + pool + linear classifiers (tests/graph_fuzz.py): forward with the fused
+    and the per-kernel path, then every gradient of the summed output in exact mode."""
+    import graph_fuzz
+    shapes, fn, desc = graph_fuzz.build_cnn(seed, frontend)
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
+    for fuse in (True, False):
+        ref, got = both(frontend, fn, arrays, fuse)
+        assert ref.shape == got.shape, desc
+        assert np.allclose(got, ref, rtol=2e-5, atol=2e-5), (desc, fuse)
+    ref = _grads_on(frontend, "c", shapes, fn, arrays)
+    got = _grads_on(frontend, "hip", shapes, fn, arrays)
+    assert ref is not None and len(ref) == len(got) == len(shapes) + 1, desc
+    for r, g in zip(ref, got):
+        assert r.shape == g.shape, desc
+        scale = max(1.0, float(np.abs(r).max()))
+        close = np.isclose(g, r, rtol=1e-4, atol=1e-5 * scale)
+        # a relu or max-pool tie that falls differently moves one window's gradient
+        assert int((~close).sum()) <= (2 if "pool True" in desc else 0), desc
+
+
 def _grads_on(fe, kind, shapes, fn, arrays):
     """Exact-mode gradients of sum(fn(inputs)) with respect to every input, plus the sum,
     realized together.  Returns None when the graph uses an op without an exact VJP."""
