@@ -89,5 +89,20 @@ def build(check: bool = False, force: bool = True) -> str:
     return LIB
 
 
+CLIENT_SRC = os.path.join(os.path.dirname(HERE), "tests", "capi_client.c")
+CLIENT = os.path.join(os.path.dirname(HERE), "tests", "capi_client.bin")
+
+
+def build_capi_client() -> str:
+    """The plain-C client of the C ABI (tests/capi_client.c), strict C99, linked against the
+    built library with a relative run path so it runs from any checkout."""
+    _run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-O1",
+          "-I" + os.path.join(os.path.dirname(HERE), "include"), CLIENT_SRC, "-o", CLIENT,
+          "-L" + HERE, "-l:libeclat_hip.so", "-Wl,-rpath,$ORIGIN/../harp_amd",
+          "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return CLIENT
+
+
 if __name__ == "__main__":
     print(build(check="--check" in sys.argv))
+    print(build_capi_client())

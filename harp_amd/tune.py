@@ -12,6 +12,7 @@ threads and elements per row; block size, vectors per thread, streaming stores),
 states by running them: event-timed launches of the compiled Program on the GPU.
 
     python -m harp_amd.tune --config config3_matmul [--beam 3] [--steps 4]
+    python -m harp_amd.tune --config config5_cnn_step
 
 prints the best options as the "key=value,..." string `eh_program_compile` takes.
 """
@@ -173,8 +174,20 @@ def beam_search(estimator, start: Optional[Dict[str, int]] = None, beam_width: i
 
 
 def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None):
-    """Searches the options of one of `workloads.CONFIGS` on device 0."""
+    """Searches the options of one benchmark configuration on device 0: one of
+    `workloads.CONFIGS`, or a whole training step (`config4_mlp_step`, `config5_cnn_step`),
+    where one option set serves every launch of the step."""
     from . import workloads as wl
+    from .frontend import Tensor
+    dev = hb.HipDevice(0)
+    if name in ("config4_mlp_step", "config5_cnn_step"):
+        mlp = name == "config4_mlp_step"
+        arrays = wl.config4_inputs(*wl.mlp_sizes(True)) if mlp else wl.config5_inputs(*wl.cnn_sizes(True))
+        ts = [Tensor.input(list(a.shape)) for a in arrays]
+        roots = wl.config4_graph(*ts) if mlp else wl.config5_graph(*ts)
+        prog_ast, arg_names, _outs, consts, _ = wl.lower_multi(ts, roots)
+        est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps, sets=1)
+        return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
     default_shapes = {"config1_relu_sum": [(1024, 1024)] * 3, "config2_softmax": [(4096, 4096)],
                       "config3_matmul": [(4096, 4096)] * 2}
     shapes = shapes or default_shapes[name]
@@ -182,7 +195,6 @@ def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log
     rng = np.random.default_rng(7)
     arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
     prog_ast, arg_names, _out, consts, _ = wl.lower_with_table(shapes, graph_fn)
-    dev = hb.HipDevice(0)
     est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps)
     return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
 

@@ -316,6 +316,19 @@ def test_tensor_beyond_32_bit_indices(frontend, hip):
     assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(x[:64]).sum(1).max())
 
 
+def test_c_client_runs_the_known_answer(hip):
+    """The plain-C client (tests/capi_client.c, built with the library) computes the
+    reference's [1,2,3,4] + [5,6,7,8] through the C ABI alone, from the compiled program and
+    again from its binary."""
+    import os
+    import subprocess
+    from harp_amd import build as hb_build
+    exe = hb_build.CLIENT if os.path.exists(hb_build.CLIENT) else hb_build.build_capi_client()
+    r = subprocess.run([exe, "run"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert "run ok" in r.stdout
+
+
 def test_buffer_roundtrip_and_size_check(hip):
     dev = hip.HipDevice(0)
     from harp_amd.frontend import F32

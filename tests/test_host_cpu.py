@@ -43,6 +43,17 @@ def test_rust_binding_names_only_declared_symbols():
         assert declared[name] == n, f"{name}: {n} parameters in ffi.rs, {declared[name]} in the header"
 
 
+def test_c_client_renders_and_compiles_without_a_gpu():
+    """tests/capi_client.c is strict C99 against include/eclat_hip.h: it builds with -Werror
+    and renders + compiles a kernel for gfx950 with no Python and no device involved."""
+    import subprocess
+    from harp_amd import build as hb_build
+    exe = hb_build.build_capi_client()
+    r = subprocess.run([exe, "render"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert "render ok: ehk_E_4_0" in r.stdout and "gfx950" in r.stdout
+
+
 def _program_with_table(fe, tensor):
     from harp_amd.frontend.executor import buffer_table
     from harp_amd.frontend.graph import collect_inputs
