@@ -316,6 +316,44 @@ def test_tensor_beyond_32_bit_indices(frontend, hip):
     assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(x[:64]).sum(1).max())
 
 
+def test_concurrent_compile_and_execute(frontend, hip):
+    """Four threads share one device handle; each compiles its own programs and runs them on
+    its own buffers while the others do the same (ctypes drops the interpreter lock inside
+    every call).  Every result must equal the single-threaded one."""
+    import threading
+    from harp_amd import measure, workloads as wl
+    dev = hip.HipDevice(0)
+    jobs = []
+    for i in range(4):                      # lowering shares front-end counters: do it up front
+        shape = (200 + 37 * i, 96 + 8 * i)
+        x = RNG(i).normal(0, 1, shape).astype(np.float32)
+        ast, names, out, consts, _ = wl.lower_with_table([shape], lambda t: frontend.nn.softmax(t * t, 1))
+        e = np.exp((x * x) - (x * x).max(1, keepdims=True))
+        jobs.append((ast, names, out, consts, x, e / e.sum(1, keepdims=True)))
+    errors = []
+
+    def work(job):
+        ast, names, out, consts, x, want = job
+        try:
+            for _ in range(3):
+                prog = hip.HipProgram(dev, ast, None)
+                (binding, named), = measure.make_sets(dev, prog, names, consts, [x], 1)
+                for _ in range(10):
+                    prog.run(binding, sync=True)
+                got = named[out].read_array(np.float32, want.shape)
+                if not np.allclose(got, want, rtol=1e-5, atol=1e-7):
+                    errors.append("wrong result")
+        except Exception as exc:            # noqa: BLE001 - reported below
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_c_client_runs_the_known_answer(hip):
     """The plain-C client (tests/capi_client.c, built with the library) computes the
     reference's [1,2,3,4] + [5,6,7,8] through the C ABI alone, from the compiled program and
