@@ -395,13 +395,14 @@ namespace {
 struct WriteRef {
   std::string buf;
   const Node* index;
+  bool atomic;      // AtomicAdd / AtomicMax: safe from any number of work-items at once
 };
 
 void collect_writes(const Node& n, std::vector<WriteRef>& writes, std::set<std::string>& read_bufs,
                     std::map<std::string, int64_t>& inner_extents, bool* ok) {
   if (n.op == Op::Store || n.op == Op::AtomicAdd || n.op == Op::AtomicMax) {
     if (n.args[0]->op != Op::Var) *ok = false;
-    else writes.push_back({n.args[0]->name, n.args[1].get()});
+    else writes.push_back({n.args[0]->name, n.args[1].get(), n.op != Op::Store});
   }
   if (n.op == Op::Load) {
     if (n.args[0]->op == Op::Var) read_bufs.insert(n.args[0]->name);
@@ -443,8 +444,10 @@ bool injective(const Affine& a, const std::vector<Loop>& vars) {
 // becomes its own launch, in order; the outer loops of a nest are spread over work-items when
 // their iterations cannot touch the same output element (every write index is affine and
 // injective in the loop variables, nothing written is read), each work-item then runs what is
-// left of the nest exactly as written, so sums keep the reference's order.  A nest that does
-// not qualify runs as written in one work-item.  Empty result: the kernel has a form this
+// left of the nest exactly as written, so sums keep the reference's order.  Writes the AST
+// marks atomic (the scatter-add of overlapping windows) may collide: the device's atomics
+// make that safe, and only the order of the additions is left open.  A nest that does not
+// qualify runs as written in one work-item.  Empty result: the kernel has a form this
 // does not cover (shape variables, hand-placed group/local ids, shared memory).
 std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOptions& opt) {
   std::vector<LaunchSpec> out;
@@ -508,10 +511,15 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
     collect_writes(*inner, writes, reads, inner_extents, &ok);
     if (!ok) return {};
     bool spread = !writes.empty();
+    bool colliding = false;
     for (const auto& r : reads) spread = spread && !written_anywhere.count(r);
     for (const auto& w : writes) {
       auto a = affine_of(*w.index);
-      if (!a) { spread = false; break; }
+      if (!a) {
+        if (w.atomic) { colliding = true; continue; }
+        spread = false;
+        break;
+      }
       std::vector<Loop> vars = loops;
       for (const auto& kv : a->coef)
         if (kv.second != 0) {
@@ -522,7 +530,11 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
           if (ie == inner_extents.end()) { spread = false; break; }
           vars.push_back({kv.first, ie->second});
         }
-      if (!spread || !injective(*a, vars)) { spread = false; break; }
+      if (!spread) break;
+      if (!injective(*a, vars)) {
+        if (w.atomic) colliding = true;
+        else { spread = false; break; }
+      }
     }
     LaunchSpec ls;
     ls.entry = k.name + "_n" + std::to_string(t);
@@ -544,7 +556,7 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       os << sr.stmt(*inner) << "}\n";
       ls.grid[0] = static_cast<unsigned>((total + 255) / 256);
       ls.block[0] = 256;
-      ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + ")";
+      ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + (colliding ? ",atomics)" : ")");
       any_parallel = true;
     } else {
       os << "extern \"C\" __global__ void " << ls.entry << "(" << sig << ") {\n" << sr.stmt(*tops[t]) << "}\n";

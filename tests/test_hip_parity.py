@@ -697,16 +697,19 @@ SPREAD_FORMS = {
     "fold_tiles": ((64, 96), lambda t: t.unfold([0, 1], [2, 3], [2, 3], [1, 1])
                    .fold([64, 96], [0, 1], [2, 3], [2, 3], [1, 1]), "outer-parallel(work-items=6144)"),
     "fold_overlapping": ((20, 30), lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1])
-                         .fold([20, 30], [0, 1], [3, 3], [1, 1], [1, 1]), "as-written"),
+                         .fold([20, 30], [0, 1], [3, 3], [1, 1], [1, 1]), "outer-parallel(work-items=4536,atomics)"),
+    "fold_overlapping_large": ((300, 500), lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1])
+                               .fold([300, 500], [0, 1], [3, 3], [1, 1], [1, 1]),
+                               "outer-parallel(work-items=1335636,atomics)"),
 }
 
 
 @pytest.mark.parametrize("name", sorted(SPREAD_FORMS))
 def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
-    """Prefix scans run one work-item per scanned line, scatter-adds one per element where
-    windows do not overlap (else as written, one work-item): bit-exact with the oracle either
-    way, because every sum keeps the sequential order (running sums and products are held to
-    the reduction tolerance, as everywhere)."""
+    """Prefix scans run one work-item per scanned line, scatter-adds one per window element:
+    bit-exact with the oracle where every sum keeps the sequential order; running sums and
+    products, and the atomic additions of overlapping windows (whose order is open), are held
+    to the reduction tolerance, as everywhere."""
     shape, fn, expect = SPREAD_FORMS[name]
     x = RNG(len(name)).uniform(0.5, 1.5, shape).astype(np.float32)
     t = frontend.Tensor.input(list(shape))
@@ -714,7 +717,7 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
     scheds = [l["schedule"] for l in hip.render_program(prog).launches]
     assert expect in scheds, scheds
     ref, got = both(frontend, fn, [x], False)
-    if name.startswith(("cumsum", "cumprod")):       # the C compiler may contract or reorder: reduction class
+    if name.startswith(("cumsum", "cumprod", "fold_overlapping")):   # order of the additions is open: reduction class
         assert np.allclose(got, ref, rtol=1e-6)
     else:
         assert bits_equal_mod_zero(ref, got)

@@ -128,10 +128,11 @@ def test_rendering_of_scatter_and_scan(frontend):
     assert "atomicAdd" in plan.launches[2]["source"]
     for l in plan.launches:
         hb.compile_source(l["source"])
-    # overlapping windows could collide: that nest stays one work-item, as written
+    # overlapping windows collide: the AST's atomic adds become device atomics
     z = x.unfold([0, 1], [2, 2], [1, 1], [1, 1]).fold([4, 4], [0, 1], [2, 2], [1, 1], [1, 1])
     plan_z = hb.render_program(frontend.lower_graph([z.graph])[0])
-    assert [l["schedule"] for l in plan_z.launches[1:]] == ["outer-parallel(work-items=16)", "as-written"]
+    assert [l["schedule"] for l in plan_z.launches[1:]] == ["outer-parallel(work-items=16)",
+                                                           "outer-parallel(work-items=36,atomics)"]
     prog2, _, _ = frontend.lower_graph([x.cumsum(1).graph])
     plan2 = hb.render_program(prog2)
     assert plan2.launches[0]["schedule"] == "outer-parallel(work-items=4)"
