@@ -316,6 +316,46 @@ def test_tensor_beyond_32_bit_indices(frontend, hip):
     assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(x[:64]).sum(1).max())
 
 
+GROUP_PARALLEL_ADD = """
+(program (kernel "E_1000_0" (params ("gidx0" i64 imm (group_id 0)) ("buf0" (ptr f32 global) imm normal)
+    ("buf2" (ptr f32 global) imm normal) ("buf4" (ptr f32 global) mut normal))
+  (grid (const i64 1000) (const i64 1) (const i64 1)) (tg (const i64 1) (const i64 1) (const i64 1))
+  (block (decls) (store (var "buf4") (var "gidx0")
+     (add (load (var "buf0") (var "gidx0") 1 f32) (load (var "buf2") (var "gidx0") 1 f32))))))
+"""
+
+GROUP_AND_LOCAL_ADD = """
+(program (kernel "E_1000_0" (params ("gidx0" i64 imm (group_id 0)) ("lidx0" i64 imm (local_id 0))
+    ("buf0" (ptr f32 global) imm normal) ("buf2" (ptr f32 global) imm normal) ("buf4" (ptr f32 global) mut normal))
+  (grid (const i64 16) (const i64 1) (const i64 1)) (tg (const i64 64) (const i64 1) (const i64 1))
+  (block (decls)
+    (if (lt (add (mul (var "gidx0") (const i64 64)) (var "lidx0")) (const i64 1000))
+      (store (var "buf4") (add (mul (var "gidx0") (const i64 64)) (var "lidx0"))
+        (add (load (var "buf0") (add (mul (var "gidx0") (const i64 64)) (var "lidx0")) 1 f32)
+             (load (var "buf2") (add (mul (var "gidx0") (const i64 64)) (var "lidx0")) 1 f32)))))))
+"""
+
+
+@pytest.mark.parametrize("text,grid,block", [(GROUP_PARALLEL_ADD, [1000, 1, 1], [1, 1, 1]),
+                                             (GROUP_AND_LOCAL_ADD, [16, 1, 1], [64, 1, 1])])
+def test_kernels_parallelised_by_the_reference_run_as_written(hip, text, grid, block):
+    """Kernels the reference's own suggesters have already parallelised carry group / local id
+    parameters and their dispatch size (`src/opt/ast/suggesters/parallelization.rs:186-232`:
+    one workgroup per iteration, then a local axis with a bounds check).  They are launched
+    with exactly that size, ids bound to blockIdx / threadIdx."""
+    dev = hip.HipDevice(0)
+    k = hip.HipKernel(dev, text)
+    l, = k.launches
+    assert l["schedule"] == "as-written" and l["grid"] == grid and l["block"] == block
+    rng = RNG(3)
+    a, b = (rng.normal(0, 1, 1000).astype(np.float32) for _ in range(2))
+    bufs = [dev.alloc(4000) for _ in range(3)]
+    bufs[0].write_array(a)
+    bufs[1].write_array(b)
+    k.execute(bufs[:2], bufs[2:])
+    assert np.array_equal(bufs[2].read_array(np.float32), a + b)
+
+
 def test_concurrent_compile_and_execute(frontend, hip):
     """Four threads share one device handle; each compiles its own programs and runs them on
     its own buffers while the others do the same (ctypes drops the interpreter lock inside
