@@ -316,6 +316,20 @@ def test_tensor_beyond_32_bit_indices(frontend, hip):
     assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(x[:64]).sum(1).max())
 
 
+@pytest.mark.parametrize("name", ["attention", "attention_masked", "avg_pool2d", "conv1d", "elu", "gelu",
+                                  "leaky_relu", "prelu", "silu"])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_nn_functions(frontend, hip, name, fuse):
+    """Activations, 1-D convolution, average pooling and scaled dot-product attention
+    (tests/nn_cases.py): HIP against the oracle, and against the formula in float64."""
+    import nn_cases
+    fn, arrays, want = nn_cases.cases(frontend)[name]
+    with frontend.exact_mode():
+        ref, got = both(frontend, fn, arrays, fuse)
+    assert np.allclose(got, ref, rtol=2e-5, atol=2e-6)
+    assert np.allclose(got.reshape(want.shape), want, rtol=1e-4, atol=1e-5)
+
+
 GROUP_PARALLEL_ADD = """
 (program (kernel "E_1000_0" (params ("gidx0" i64 imm (group_id 0)) ("buf0" (ptr f32 global) imm normal)
     ("buf2" (ptr f32 global) imm normal) ("buf4" (ptr f32 global) mut normal))

@@ -382,3 +382,18 @@ def test_exact_vjps_against_finite_differences(frontend, name):
     numeric = (value([a + h * d for a, d in zip(arrays, dirs)]) - value([a - h * d for a, d in zip(arrays, dirs)])) / (2 * h)
     analytic = sum(float((g.reshape(d.shape) * d).sum()) for g, d in zip(grads, dirs))
     assert abs(numeric - analytic) <= 2e-2 * max(1.0, abs(numeric), abs(analytic)), (numeric, analytic)
+
+
+NN_CASE_NAMES = ["attention", "attention_masked", "avg_pool2d", "conv1d", "elu", "gelu", "leaky_relu", "prelu",
+                 "silu"]
+
+
+@pytest.mark.parametrize("name", NN_CASE_NAMES)
+def test_nn_functions_match_their_mathematics(frontend, name):
+    """The op trees of the remaining `crates/nn/src/functional` mirrors, evaluated by the
+    oracle, against float64 numpy of the formula each function documents."""
+    import nn_cases
+    fn, arrays, want = nn_cases.cases(frontend)[name]
+    with frontend.exact_mode():
+        got = realize_on(frontend, "c", fn, arrays)
+    assert np.allclose(got.reshape(want.shape), want, rtol=2e-5, atol=2e-6)
