@@ -14,4 +14,5 @@ from .lowerer import Lowerer, all_fusions, lower_graph
 from .tensor import Tensor, realize_many
 from .view import View
 from . import nn
+from . import layers, optim
 from .config import exact_mode

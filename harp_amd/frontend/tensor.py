@@ -291,6 +291,19 @@ class Tensor:
         _INPUT_BUFFER_CACHE[id(self.graph)] = (self.graph, buf.clone_buffer())
         self.buffer = buf
 
+    def set_buffer(self, buf) -> None:
+        """Binds an input tensor to a buffer that is already on the device (the realized buffer
+        of another tensor of this size).  Not in the reference, whose only way to give an input
+        its data is `set_data` from host memory."""
+        if not self.graph.is_external():
+            raise ExecutionError("NotAnInput: set_buffer() needs an input tensor")
+        want = self.numel() * np.dtype(_NP[self.dtype().name]).itemsize
+        if buf is None or buf.byte_len() != want:
+            raise ExecutionError(f"ShapeMismatch: buffer of {None if buf is None else buf.byte_len()} bytes "
+                                 f"for a tensor of {want}")
+        _INPUT_BUFFER_CACHE[id(self.graph)] = (self.graph, buf)
+        self.buffer = buf
+
     def realize(self) -> "Tensor":
         if self.is_realized():
             return self

@@ -330,6 +330,20 @@ def test_nn_functions(frontend, hip, name, fuse):
     assert np.allclose(got.reshape(want.shape), want, rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("optimizer", ["sgd", "momentum", "adam"])
+def test_training_loop_on_the_device(frontend, hip, optimizer):
+    """Six optimizer steps of a small MLP (tests/train_loop.py); every step is one Program
+    (forward, exact backward, update of parameters and optimizer state), the new parameters
+    stay on the device.  HIP against the oracle and against float64 numpy."""
+    import train_loop
+    ref_losses, ref_params = train_loop.run(frontend, "c", optimizer, 6)
+    losses, params = train_loop.run(frontend, "hip", optimizer, 6)
+    np_losses, np_params = train_loop.run_numpy(frontend, optimizer, 6)
+    assert np.allclose(losses, ref_losses, rtol=1e-5) and np.allclose(losses, np_losses, rtol=1e-4)
+    for a, b, c in zip(params, ref_params, np_params):
+        assert np.allclose(a, b, rtol=1e-4, atol=1e-6) and np.allclose(a, c, rtol=1e-3, atol=1e-5)
+
+
 GROUP_PARALLEL_ADD = """
 (program (kernel "E_1000_0" (params ("gidx0" i64 imm (group_id 0)) ("buf0" (ptr f32 global) imm normal)
     ("buf2" (ptr f32 global) imm normal) ("buf4" (ptr f32 global) mut normal))

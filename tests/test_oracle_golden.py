@@ -397,3 +397,38 @@ def test_nn_functions_match_their_mathematics(frontend, name):
     with frontend.exact_mode():
         got = realize_on(frontend, "c", fn, arrays)
     assert np.allclose(got.reshape(want.shape), want, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("optimizer", ["sgd", "momentum", "adam"])
+def test_training_loop_matches_numpy(frontend, optimizer):
+    """Layers + optimizer mirrors (tests/train_loop.py): six steps on the oracle follow the
+    float64 numpy loop of the same arithmetic (`sgd.rs:73-103`, `adam.rs:70-110`)."""
+    import train_loop
+    losses, params = train_loop.run(frontend, "c", optimizer, 6)
+    ref_losses, ref_params = train_loop.run_numpy(frontend, optimizer, 6)
+    assert np.allclose(losses, ref_losses, rtol=1e-5)
+    for a, b in zip(params, ref_params):
+        assert np.allclose(a, b, rtol=1e-4, atol=1e-6)
+    assert losses[-1] < losses[0]
+
+
+def test_parameter_and_layer_api(frontend):
+    """`Parameter` (parameter.rs:31-214) and the deterministic layer initialisation
+    (`linear.rs:57-68`: sin(0.1 i) * sqrt(1/in), zero bias)."""
+    from harp_amd.frontend.layers import Linear, Parameter, ParameterError
+    frontend.set_device_str("c")
+    lin = Linear(4, 3)
+    w = lin.weight.to_numpy()
+    assert w.shape == (3, 4) and np.allclose(w.ravel(), np.sin(0.1 * np.arange(12)) * 0.5, atol=1e-7)
+    assert not lin.bias.to_numpy().any() and lin.weight.has_data()
+    p = Parameter.from_data("p", [1, 2, 3, 4, 5, 6], [2, 3])
+    assert p.shape() == [2, 3] and p.numel() == 6 and p.to_vec() == [1, 2, 3, 4, 5, 6]
+    assert p.tensor().requires_grad() and p.grad() is None
+    p.update_data([6, 5, 4, 3, 2, 1])
+    assert p.tensor().to_vec() == [6, 5, 4, 3, 2, 1]
+    with pytest.raises(ParameterError):
+        p.update_data([1, 2, 3])
+    with pytest.raises(ParameterError):
+        Parameter.from_data("q", [1, 2, 3], [2, 2])
+    with pytest.raises(frontend.optim.OptimError):
+        frontend.optim.SGD([p], 0.1).step()              # no gradient yet
