@@ -154,9 +154,8 @@ class HipBuffer:
         return p.value or 0
 
     def write_from_host(self, raw) -> None:
-        raw = bytes(raw) if not isinstance(raw, (bytes, bytearray)) else raw
-        buf = (ctypes.c_char * len(raw)).from_buffer_copy(raw) if raw else None
-        check(lib.eh_buffer_write(self._h, buf, len(raw)))
+        raw = raw if isinstance(raw, bytes) else bytes(raw)
+        check(lib.eh_buffer_write(self._h, raw if raw else None, len(raw)))     # read in place
 
     def write_array(self, arr) -> None:
         """Zero-copy upload of a C-contiguous numpy array."""

@@ -36,6 +36,7 @@ _tls = threading.local()
 # kernel cache (cache/store.rs:116-168): LRU of 1024 compiled kernels
 _CACHE_CAPACITY = 1024
 _kernel_cache: "OrderedDict[Tuple[str, str, int], object]" = OrderedDict()
+_program_cache: "OrderedDict[tuple, object]" = OrderedDict()
 _cache_stats = {"hits": 0, "misses": 0, "entries": 0, "evictions": 0}
 
 
@@ -152,6 +153,33 @@ def compile_ast_with_cache(program, signature=None):
     return kernel
 
 
+_PROGRAM_CACHE_CAPACITY = 64          # whole programs keep their temporaries resident
+
+
+def compile_program_with_cache(program):
+    """Whole-program counterpart of `compile_ast_with_cache`, same key.  A training loop
+    realizes the same Program every step: a hit skips rendering, module loading and the
+    allocation of the program's temporaries.  Hits and misses count in the same statistics."""
+    d = get_default_device()
+    if d is None:
+        raise DeviceError("No default device set")
+    key = ("program", program.to_sexpr(), d.kind, id(d.device))
+    with _lock:
+        hit = _program_cache.get(key)
+        if hit is not None:
+            _program_cache.move_to_end(key)
+            _cache_stats["hits"] += 1
+            return hit
+        _cache_stats["misses"] += 1
+    compiled = d.compile_program(program)
+    with _lock:
+        _program_cache[key] = compiled
+        while len(_program_cache) > _PROGRAM_CACHE_CAPACITY:
+            _program_cache.popitem(last=False)
+            _cache_stats["evictions"] += 1
+    return compiled
+
+
 def cache_stats() -> Dict[str, int]:
     with _lock:
         return dict(_cache_stats)
@@ -160,5 +188,6 @@ def cache_stats() -> Dict[str, int]:
 def clear_cache() -> None:
     with _lock:
         _kernel_cache.clear()
+        _program_cache.clear()
         for k in _cache_stats:
             _cache_stats[k] = 0

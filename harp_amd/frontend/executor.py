@@ -18,7 +18,8 @@ import os
 from typing import Dict, List, Sequence
 
 from .ast import AstNode
-from .device import (DeviceError, compile_ast_with_cache, get_default_device)
+from .device import (DeviceError, compile_ast_with_cache, compile_program_with_cache,
+                     get_default_device)
 from .graph import GraphNode, collect_inputs
 from .lowerer import lower_graph
 
@@ -113,7 +114,7 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
                 consts[lowerer.lookup_buffer_name(n)] = kind
         table = buffer_table(program, lowerer, list(buffer_map.keys()), out_names, consts)
         prog_ast = AstNode.program(kernels, buffers=table)
-        compiled = dev.compile_program(prog_ast)
+        compiled = compile_program_with_cache(prog_ast)
         outs = compiled.execute({k: v for k, v in buffer_map.items()})
         buffer_map.update(outs)
     else:

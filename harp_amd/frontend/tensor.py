@@ -12,6 +12,7 @@ ones and ignores `f`; `mean` returns `sum`; `pow` is `exp(ln(x))`.
 
 from __future__ import annotations
 
+from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -287,7 +288,10 @@ class Tensor:
             raise ExecutionError(f"ShapeMismatch: Data size {arr.size} doesn't match "
                                  f"tensor size {self.numel()}")
         buf = allocate_buffer_on_default_device(self.shape(), self.dtype())
-        buf.write_from_host(arr.tobytes())
+        if hasattr(buf, "write_array"):
+            buf.write_array(arr)                       # straight from the array's memory
+        else:
+            buf.write_from_host(arr.tobytes())
         _INPUT_BUFFER_CACHE[id(self.graph)] = (self.graph, buf.clone_buffer())
         self.buffer = buf
 
@@ -382,14 +386,32 @@ def realize_many(tensors: Sequence[Tensor]) -> None:
         t.buffer = b
 
 
+_CONSTANT_BUFFERS: "OrderedDict[tuple, object]" = OrderedDict()
+_CONSTANT_BUFFERS_MAX = 32
+
+
 def _create_constant_buffer(node: G.GraphNode):
+    """Buffer for a ones / zeros tensor (realize.rs:391-421).  The filled buffers are kept per
+    device, shape and value: a training loop asks for the same ones every step, and the
+    executor only ever reads them (it clones its inputs)."""
     fill = {"ones": 1.0, "zeros": 0.0, "scalar": 1.0}.get(node.name)
     if fill is None:
         return None
     shape = [int(e.evaluate()) for e in node.shape()]
+    from .device import get_default_device
+    dev = get_default_device()
+    key = (id(dev.device) if dev is not None else None, tuple(shape), node.dtype.name, fill)
+    hit = _CONSTANT_BUFFERS.get(key)
+    if hit is not None:
+        _CONSTANT_BUFFERS.move_to_end(key)
+        return hit
     buf = allocate_buffer_on_default_device(shape, node.dtype)
-    n = 1
-    for s in shape:
-        n *= s
-    buf.write_from_host(np.full(n, fill, dtype=_NP[node.dtype.name]).tobytes())
+    if fill != 0.0:                                   # a fresh buffer is zero-filled already
+        n = 1
+        for s in shape:
+            n *= s
+        buf.write_from_host(np.full(n, fill, dtype=_NP[node.dtype.name]).tobytes())
+    _CONSTANT_BUFFERS[key] = buf
+    while len(_CONSTANT_BUFFERS) > _CONSTANT_BUFFERS_MAX:
+        _CONSTANT_BUFFERS.popitem(last=False)
     return buf

@@ -821,7 +821,7 @@ def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
         assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
 
 
-@pytest.mark.parametrize("seed", range(400, 412))
+@pytest.mark.parametrize("seed", range(400, 408))
 def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
     """Random conv + pool + linear classifiers (tests/graph_fuzz.py): forward with the fused
     and the per-kernel path, then every gradient of the summed output in exact mode."""
