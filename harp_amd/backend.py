@@ -10,6 +10,7 @@ buffers (`Buffer`, `src/backend/traits.rs:455-482`) and compiled kernels
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import byref, c_char_p, c_float, c_int, c_size_t, c_void_p
 from typing import Dict, List, Optional, Sequence
 
@@ -219,7 +220,10 @@ class HipProgram:
         check(lib.eh_program_execute(self._h, binding[0], len(self.buffers), 1 if sync else 0))
 
     def execute(self, inputs: Dict[str, HipBuffer]) -> Dict[str, HipBuffer]:
-        """Binds inputs by name, allocates the outputs, runs, returns the outputs."""
+        """Binds inputs by name, allocates the outputs, queues the launches, returns the
+        outputs.  Nothing waits here: reads, later programs and the reuse of released memory
+        are all ordered behind these launches on the device's stream, so the host can build the
+        next step meanwhile.  ECLAT_HIP_SYNC=1 in the environment waits after every program."""
         named = dict(inputs)
         outs = {}
         for b in self.buffers:
@@ -227,7 +231,7 @@ class HipProgram:
                 hb = HipBuffer(self.device, [b["bytes"]], None, nbytes=b["bytes"])
                 named[b["name"]] = hb
                 outs[b["name"]] = hb
-        self.run(self.bind(named), sync=True)
+        self.run(self.bind(named), sync=os.environ.get("ECLAT_HIP_SYNC", "0") == "1")
         return outs
 
     def binary(self, launch: int = 0) -> bytes:
