@@ -939,6 +939,27 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   std::vector<std::optional<NestKernel>> nests;
   for (const Node* k : kernels) {
     nests.push_back(extract_nest(*k));
+    if (nests.back() && nests.back()->rkind == ReduceKind::None) {
+      // An elementwise nest has no loop-carried dependence, so its loops may run in any order:
+      // walk the output in address order (largest stride outermost).  A kernel lowered through
+      // a transposing view otherwise strides through memory with its innermost loop, and it
+      // would not share an index space with the kernel that produced its operand.
+      NestKernel& nk = *nests.back();
+      const Affine& oa = *nk.out_aff;
+      bool all_used = true;
+      for (const auto& l : nk.loops) all_used = all_used && (l.extent == 1 || oa.of(l.var) != 0);
+      if (all_used) {
+        std::vector<Loop> wide;                       // loops of extent 1 keep their places
+        for (const auto& l : nk.loops)
+          if (l.extent > 1) wide.push_back(l);
+        std::stable_sort(wide.begin(), wide.end(), [&](const Loop& a, const Loop& b) {
+          return std::llabs(oa.of(a.var)) > std::llabs(oa.of(b.var));
+        });
+        size_t w = 0;
+        for (auto& l : nk.loops)
+          if (l.extent > 1) l = wide[w++];
+      }
+    }
     if (nests.back() && !consts.empty()) {
       NestKernel& nk = *nests.back();
       nk.value = fold(nk.value);
@@ -1080,6 +1101,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           std::map<std::string, DType> avail;          // values held in registers: C and stage outputs
           avail[k0.out_buf] = k0.out_dtype;
           bool c_relaid = false;
+          size_t relaid_pos = 0;                       // position in `taken` of the stage that reads through a permutation
+          Affine relaid_read;                          // ... and the index it reads at, over its own loops
+          std::set<std::string> old_space;             // values produced before that stage
           std::vector<size_t> taken;
           size_t j = i + 1;
           for (; j < kernels.size(); ++j) {
@@ -1092,34 +1116,45 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             std::vector<LoadRef> loads;
             collect_loads(*sk.value, loads);
             bool feeds = false, ok = true;
-            std::optional<Affine> relaid;
+            std::optional<Affine> permuted;            // the one index all values of the chain are read at, if not the aligned one
             for (const auto& lr : loads) {
               if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
-              if (!avail.count(lr.load->args[0]->name)) continue;
+              const std::string& b = lr.load->args[0]->name;
+              if (!avail.count(b)) continue;
               auto a = affine_of(*lr.load->args[1]);
               if (!a) { ok = false; break; }
-              if (!(*a == *sk.out_aff)) {
-                // The first consumer may read C through a permutation (a transposed weight
-                // gradient, NHWC -> NCHW after a convolution).  If C has no other reader the
-                // contraction can write C's elements where this consumer wants them: lay C out
-                // in the consumer's index space and the read becomes the aligned one.
-                bool sole = taken.empty() && !c_relaid && role_of(k0.out_buf) == "temp" &&
-                            lr.load->args[0]->name == k0.out_buf;
-                for (size_t r : readers[k0.out_buf]) sole = sole && r == j;
-                auto na = sole ? relayout(k0, sk, *a) : std::nullopt;
-                if (!na || (relaid && !(*relaid == *na))) { ok = false; break; }
-                relaid = na;
-              } else if (relaid) {
-                ok = false;   // the same stage reads C both ways
+              const bool aligned = *a == *sk.out_aff;
+              if (c_relaid && (old_space.count(b) || !aligned)) { ok = false; break; }
+              if (!aligned) {
+                if (feeds && !permuted) { ok = false; break; }          // the stage reads the chain both ways
+                if (permuted && !(*permuted == *a)) { ok = false; break; }
+                permuted = *a;
+              } else if (permuted) {
+                ok = false;
                 break;
               }
               feeds = true;
             }
             if (!ok || !feeds) break;
-            if (relaid) {
-              k0r.out_aff = *relaid;
+            if (permuted) {
+              // A consumer may read the chain's values through a permutation (a transposed weight
+              // gradient and its update, NHWC -> NCHW after a convolution).  If nothing computed so
+              // far is needed outside the chain, the contraction can put each element where this
+              // consumer wants it: C takes the consumer's index space, the stages before it are
+              // evaluated at the element's original position, and the read becomes the aligned one.
+              bool sole = true;
+              for (const auto& kv : avail) {
+                sole = sole && role_of(kv.first) == "temp";
+                for (size_t r : readers[kv.first]) sole = sole && r > i && r <= j;
+              }
+              auto na = sole ? relayout(k0, sk, *permuted) : std::nullopt;
+              if (!na) break;
+              k0r.out_aff = *na;
+              if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; break; }
               c_relaid = true;
-              if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; c_relaid = false; break; }
+              relaid_pos = taken.size();
+              relaid_read = *permuted;
+              for (const auto& kv : avail) old_space.insert(kv.first);
             }
             avail[sk.out_buf] = sk.out_dtype;
             taken.push_back(j);
@@ -1141,17 +1176,37 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
             body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
             if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
-            for (size_t j2 : taken) {
-              const NestKernel& sk = *nests[j2];
+            auto decode = [&](const NestKernel& sk, const std::string& from) {
               int64_t numel = 0;
               auto strides = *dense_strides(sk, &numel);
-              epi.kernels.push_back(sk.name);
-              body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
               for (size_t li = 0; li < sk.loops.size(); ++li) {
                 const Loop& l = sk.loops[li];
                 if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
-                else body << "    const " << IT << " " << l.var << " = (eh_l / " << strides[li] << ") % " << l.extent << ";\n";
+                else body << "    const " << IT << " " << l.var << " = (" << from << " / " << strides[li] << ") % " << l.extent << ";\n";
               }
+            };
+            if (c_relaid && relaid_pos > 0) {
+              // where this element sat before C took the later consumer's layout: the stages
+              // ahead of that consumer index their other operands with it
+              if (epi.store_c) throw Error("internal: relaid contraction '" + k0.name + "' must not store C");
+              body << "  " << IT << " eh_lo;\n  {\n";
+              decode(*nests[taken[relaid_pos]], "eh_l");
+              body << "    eh_lo = ";
+              bool first_term = true;
+              for (const auto& kv : relaid_read.coef) {
+                if (kv.second == 0) continue;
+                body << (first_term ? "" : " + ") << kv.first << " * " << kv.second;
+                first_term = false;
+              }
+              if (first_term) body << "0";
+              body << ";\n  }\n";
+            }
+            for (size_t ti = 0; ti < taken.size(); ++ti) {
+              const size_t j2 = taken[ti];
+              const NestKernel& sk = *nests[j2];
+              epi.kernels.push_back(sk.name);
+              body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
+              decode(sk, (c_relaid && ti < relaid_pos) ? "eh_lo" : "eh_l");
               ExprRenderer er;
               er.load_hook = [&](const Node& ld, std::string* out) {
                 const std::string& b = ld.args[0]->name;
