@@ -1104,6 +1104,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           size_t relaid_pos = 0;                       // position in `taken` of the stage that reads through a permutation
           Affine relaid_read;                          // ... and the index it reads at, over its own loops
           std::set<std::string> old_space;             // values produced before that stage
+          std::set<size_t> independent;                // taken stages that read no value of the chain
           std::vector<size_t> taken;
           size_t j = i + 1;
           for (; j < kernels.size(); ++j) {
@@ -1135,7 +1136,10 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
               }
               feeds = true;
             }
-            if (!ok || !feeds) break;
+            if (!ok) break;
+            // a stage over the same index space that reads nothing of the chain (the square of a
+            // saved activation, say) rides along when a later stage combines it with the chain
+            if (!feeds) independent.insert(j);
             if (permuted) {
               // A consumer may read the chain's values through a permutation (a transposed weight
               // gradient and its update, NHWC -> NCHW after a convolution).  If nothing computed so
@@ -1158,6 +1162,11 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             }
             avail[sk.out_buf] = sk.out_dtype;
             taken.push_back(j);
+          }
+          while (!taken.empty() && independent.count(taken.back())) {
+            avail.erase(nests[taken.back()]->out_buf);      // nothing after it uses the chain: leave it out
+            independent.erase(taken.back());
+            taken.pop_back();
           }
           if (!taken.empty()) {
             after = taken.back() + 1;
