@@ -283,7 +283,7 @@ def test_config4_training_step_plan(frontend):
     matmuls all take the MFMA schedule, whose bias gradients take the two-launch column
     reduce, and whose synthesised ones/zeros inputs never become device buffers."""
     from harp_amd import backend as hb, workloads as wl
-    batch, dims = 256, (128, 256, 128, 128)
+    batch, dims = 192, (128, 256, 128, 128)       # a batch no weight dimension equals
     shapes = [(batch, dims[0]), (batch, dims[-1])]
     for a, b in zip(dims[:-1], dims[1:]):
         shapes += [(b, a), (b,)]
@@ -300,6 +300,16 @@ def test_config4_training_step_plan(frontend):
     epi = [l for l in plan.launches if "epilogue=" in l["schedule"]]
     assert len(epi) >= 3 and all("eh_epilogue(" in l["source"] for l in epi)
     assert any(len(l["kernels"]) >= 6 for l in epi)
+    # every weight's SGD update (lr * dW, then W - that read through a transposing view) is
+    # part of its gradient contraction: no elementwise launch over a weight matrix is left,
+    # and the gradient itself never reaches memory
+    weight_kernels = {f"E_{b}_{a}" for a, b in zip(dims[:-1], dims[1:])} | {f"E_{a}_{b}" for a, b in zip(dims[:-1], dims[1:])}
+    for l in plan.launches:
+        if l["schedule"].startswith("flat("):
+            assert not any(k.rsplit("_", 1)[0] in weight_kernels for k in l["kernels"]), l["kernels"]
+    # the tanh' products of the backward pass (one stage squares a saved activation and reads
+    # nothing of the chain) ride on the dX contractions
+    assert sum(len(l["kernels"]) >= 8 for l in epi) >= 2
     off = hb.render_program(prog_ast, {"gemm_epilogue": 0})
     assert not any("epilogue=" in l["schedule"] for l in off.launches) and len(off.launches) > len(plan.launches)
     by_name = {b["name"]: b for b in plan.buffers}
