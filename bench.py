@@ -234,14 +234,14 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             mlp["loss"] = got_loss
         del sets
 
-    # ---- config 5: MNIST-shaped CNN, batch 256, forward + backward -------------------------
+    # ---- config 5: MNIST-shaped CNN, batch 256, forward + backward + SGD update ------------
     cnn = None
     if want("cnn"):
         sizes = wl.cnn_sizes(True)
         arrays = wl.config5_inputs(*sizes)
         from harp_amd.frontend import Tensor
         ts = [Tensor.input(list(a.shape)) for a in arrays]
-        roots = wl.config5_graph(*ts)
+        roots = wl.config5_graph(*ts, lr=1e-2)
         prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
         prog = hb.HipProgram(dev, prog_ast, options)
         sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 1)
@@ -312,7 +312,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             sizes = wl.cnn_sizes(True)
             arrays = wl.config5_inputs(sub, *sizes[1:])
             with exact_mode():
-                sec_c, reps_c, _ = baseline.time_graph(lambda *ts: wl.config5_graph(*ts), arrays,
+                sec_c, reps_c, _ = baseline.time_graph(lambda *ts: wl.config5_graph(*ts, lr=1e-2), arrays,
                                                        min_seconds=4.0, max_reps=10)
             result_extra["cpu_baseline_cnn"] = {
                 "value": sub / sec_c, "unit": "images/s", "cores": 1, "kind": "port",
@@ -367,7 +367,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             "lowered_kernels": cnn["lowered_kernels"], "launches": cnn["launches"],
             "gemm_launches": cnn["gemm_launches"], "loss": cnn.get("loss"),
             "workload": "CNN 1x28x28: conv3x3(32)+relu+pool, conv3x3(64)+relu+pool, fc 3136-128-10, "
-                        "cross-entropy; batch 256 forward + exact backward, one Program"}
+                        "cross-entropy; batch 256 forward + exact backward + SGD update, one Program"}
     result_extra["device"] = {"name": props["name"], "arch": props["arch"],
                               "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
     out["extra"] = result_extra

@@ -184,7 +184,7 @@ def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log
         mlp = name == "config4_mlp_step"
         arrays = wl.config4_inputs(*wl.mlp_sizes(True)) if mlp else wl.config5_inputs(*wl.cnn_sizes(True))
         ts = [Tensor.input(list(a.shape)) for a in arrays]
-        roots = wl.config4_graph(*ts) if mlp else wl.config5_graph(*ts)
+        roots = wl.config4_graph(*ts) if mlp else wl.config5_graph(*ts, lr=1e-2)
         prog_ast, arg_names, _outs, consts, _ = wl.lower_multi(ts, roots)
         est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps, sets=1)
         return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)

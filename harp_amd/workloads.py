@@ -148,9 +148,10 @@ def config5_inputs(batch=256, side=28, c1=32, c2=64, hidden=128, classes=10, see
     return [x, one_hot] + params
 
 
-def config5_graph(x: Tensor, one_hot: Tensor, *params: Tensor):
+def config5_graph(x: Tensor, one_hot: Tensor, *params: Tensor, lr: float = None):
     """conv3x3(pad 1)+relu+maxpool2 twice, fc+relu, fc, cross-entropy; exact backward.
-    Returns [gradient of every parameter..., loss]."""
+    Returns [gradient of every parameter..., loss], or with a learning rate the whole SGD
+    step [p - lr*gradient for every parameter..., loss]."""
     from .frontend import exact_mode
     w1, b1, w2, b2, w3, b3, w4, b4 = params
     with exact_mode():
@@ -163,6 +164,8 @@ def config5_graph(x: Tensor, one_hot: Tensor, *params: Tensor):
         loss = nn.cross_entropy_loss(logits, one_hot, exact=True)
         loss.backward_with_params(list(params))
         # a gradient may come out as a view (the weight's is a permute); roots must own buffers
+        if lr is not None:
+            return [p - p.grad().scale_exact(lr) for p in params] + [loss]
         grads = [p.grad().contiguous() for p in params]
     return grads + [loss]
 

@@ -570,7 +570,7 @@ def test_config4_mlp_training_step(frontend, hip, batch, dims, fuse):
         assert np.allclose(g.reshape(p.shape), p - 1e-3 * gr, rtol=1e-4, atol=1e-6)
 
 
-def _cnn_step_on(fe, kind, arrays, fuse=True):
+def _cnn_step_on(fe, kind, arrays, fuse=True, lr=None):
     import os
     from harp_amd import workloads as wl
     from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
@@ -584,7 +584,7 @@ def _cnn_step_on(fe, kind, arrays, fuse=True):
                 t = fe.Tensor.input(list(a.shape))
                 t.set_data(a)
                 ts.append(t)
-            roots = wl.config5_graph(*ts)
+            roots = wl.config5_graph(*ts, lr=lr)
             fe.realize_many(roots)
             return [r.to_numpy() for r in roots]
     finally:
@@ -613,6 +613,21 @@ def test_config5_cnn_training_step(frontend, hip, sizes, fuse):
         scale = max(float(np.abs(r).max()), 1e-6)
         assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
         assert np.allclose(g.reshape(n.shape), n, rtol=1e-3, atol=1e-5 * scale)
+
+
+def test_config5_cnn_step_with_sgd_update(frontend, hip):
+    """The form the benchmark times: the same step with p - lr * gradient for every parameter
+    as the roots (the updates ride on the gradient contractions where they can)."""
+    from harp_amd import workloads as wl
+    from cnn_reference import cnn_step
+    arrays = wl.config5_inputs(8, 28, 32, 64, 128, 10, seed=78)
+    ref = _cnn_step_on(frontend, "c", arrays, lr=0.05)
+    got = _cnn_step_on(frontend, "hip", arrays, lr=0.05)
+    loss, grads = cnn_step(arrays[0], arrays[1], arrays[2:])
+    assert abs(float(got[-1][0]) - loss) <= 1e-5 * abs(loss)
+    for g, r, p, n in zip(got[:-1], ref[:-1], arrays[2:], grads):
+        assert np.allclose(g, r, rtol=1e-5, atol=1e-6)
+        assert np.allclose(g.reshape(p.shape), p - 0.05 * n, rtol=1e-4, atol=1e-6)
 
 
 def _run_program(fe, hb, graph_fn, arrays, options=None):
