@@ -12,6 +12,7 @@ Tolerance classes (written where they are applied):
 import numpy as np
 import pytest
 
+import golden_ops
 from conftest import bits_equal_mod_zero, realize_on
 
 pytestmark = pytest.mark.gpu
@@ -36,6 +37,39 @@ def test_reference_known_answers(frontend, hip, fuse):
     m2 = np.array([[5, 6], [7, 8]], dtype=np.float32)
     out = realize_on(frontend, "hip", lambda x, y: frontend.nn.matmul(x, y), [m1, m2], fuse=fuse)
     assert out.tolist() == [19, 22, 43, 50]
+
+
+_FX = golden_ops.load()
+
+
+@pytest.mark.parametrize("case", _FX["forward"], ids=lambda c: c["id"])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_fixture_forward_known_answers(frontend, hip, case, fuse):
+    """The reference's own known answers (tests/golden/) through the HIP backend."""
+    arrays = [golden_ops.array(v, s) for v, s in zip(case["inputs"], case["shapes"])]
+    out = realize_on(frontend, "hip", golden_ops.graph(frontend, case["op"]), arrays, fuse=fuse)
+    golden_ops.check_forward(case, out)
+
+
+def test_fixture_gradients_and_properties(frontend, hip):
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    for case in _FX["properties"]:
+        arrays = [golden_ops.array(v, s) for v, s in zip(case["inputs"], case["shapes"])]
+        out = realize_on(frontend, "hip", golden_ops.graph(frontend, case["op"]), arrays)
+        assert out.size == case["length"] and abs(float(out.sum()) - case["sum"]) < case["atol"]
+    frontend.set_device_str("hip")
+    for case in _FX["gradients"]:
+        try:
+            ts = []
+            for v, s in zip(case["inputs"], case["shapes"]):
+                t = frontend.Tensor.input(s).requires_grad_(True)
+                t.set_data(golden_ops.array(v, s))
+                ts.append(t)
+            golden_ops.graph(frontend, case["op"])(*ts).backward_with_params(ts)
+            got = [t.grad().realize().to_numpy().tolist() for t in ts]
+        finally:
+            _INPUT_BUFFER_CACHE.clear()
+        assert got == [[float(v) for v in e] for e in case["expected"]], case["id"]
 
 
 ELEMENTWISE = {

@@ -4,7 +4,37 @@ assertions (no GPU)."""
 import numpy as np
 import pytest
 
+import golden_ops
 from conftest import realize_on
+
+_FX = golden_ops.load()
+
+
+@pytest.mark.parametrize("case", _FX["forward"], ids=lambda c: c["id"])
+def test_fixture_forward_known_answers(frontend, case):
+    """Every forward known answer in tests/golden/ on the oracle (both CPU flavours)."""
+    arrays = [golden_ops.array(v, s) for v, s in zip(case["inputs"], case["shapes"])]
+    for kind in ("c", "openmp"):
+        golden_ops.check_forward(case, realize_on(frontend, kind, golden_ops.graph(frontend, case["op"]), arrays))
+
+
+@pytest.mark.parametrize("case", _FX["properties"], ids=lambda c: c["id"])
+def test_fixture_properties(frontend, case):
+    arrays = [golden_ops.array(v, s) for v, s in zip(case["inputs"], case["shapes"])]
+    out = realize_on(frontend, "c", golden_ops.graph(frontend, case["op"]), arrays)
+    assert out.size == case["length"] and abs(float(out.sum()) - case["sum"]) < case["atol"]
+
+
+@pytest.mark.parametrize("case", _FX["shapes"], ids=lambda c: c["id"])
+def test_fixture_unfold_shapes(frontend, case):
+    t = frontend.Tensor.input(case["input_shape"])
+    assert t.unfold(*case["unfold"]).shape() == case["expected_shape"]
+
+
+@pytest.mark.parametrize("case", _FX["rendered_text"], ids=lambda c: c["expr"])
+def test_fixture_rendered_text(frontend, case):
+    from oracle.c_renderer import render_expr
+    assert render_expr(golden_ops.expr(frontend, case["expr"]).to_sexpr()) == case["text"]
 
 
 def test_rendered_expression_text(frontend):
@@ -32,50 +62,6 @@ def test_header_and_types(frontend):
     assert render_dtype("f32") == "float" and render_dtype("f64") == "double"
     assert render_dtype("i32") == "int" and render_dtype("i64") == "long long"
     assert render_dtype(["ptr", "f32", "global"]) == "float*"
-
-
-def test_add_mul_known_answers(frontend):
-    # crates/backend-c/src/lib.rs:183-245
-    a = np.array([1, 2, 3, 4], dtype=np.float32)
-    b = np.array([5, 6, 7, 8], dtype=np.float32)
-    assert realize_on(frontend, "c", lambda x, y: x + y, [a, b]).tolist() == [6, 8, 10, 12]
-    a2 = np.array([1, 2, 3, 4], dtype=np.float32)
-    b2 = np.array([2, 3, 4, 5], dtype=np.float32)
-    assert realize_on(frontend, "c", lambda x, y: x * y, [a2, b2]).tolist() == [2, 6, 12, 20]
-    a3 = np.arange(1, 7, dtype=np.float32).reshape(2, 3)
-    b3 = a3[::-1, ::-1].copy()
-    assert realize_on(frontend, "c", lambda x, y: x + y, [a3, b3]).tolist() == [7.0] * 6
-
-
-def test_large_add_openmp(frontend):
-    # crates/backend-openmp/src/lib.rs:205-230: 10 000 elements, a[i]=i, b[i]=10000-i
-    a = np.arange(10000, dtype=np.float32)
-    b = (10000 - np.arange(10000)).astype(np.float32)
-    out = realize_on(frontend, "openmp", lambda x, y: x + y, [a, b])
-    assert np.allclose(out, 10000.0, atol=1e-3)
-
-
-def test_matmul_2x2_known_answer(frontend):
-    # crates/backend-metal/src/compiler.rs:240-257
-    a = np.array([[1, 2], [3, 4]], dtype=np.float32)
-    b = np.array([[5, 6], [7, 8]], dtype=np.float32)
-    out = realize_on(frontend, "c", lambda x, y: frontend.nn.matmul(x, y), [a, b])
-    assert out.tolist() == [19, 22, 43, 50]
-
-
-def test_matmul_demo_shape(frontend):
-    # examples/matmul_demo.rs:114-129, 166-178: 4x3 @ 3x2 against the plain triple loop
-    a = (np.arange(12, dtype=np.float32) * 0.5 - 1).reshape(4, 3)
-    b = (np.arange(6, dtype=np.float32) * 0.25 + 1).reshape(3, 2)
-    out = realize_on(frontend, "c", lambda x, y: frontend.nn.matmul(x, y), [a, b]).reshape(4, 2)
-    ref = np.zeros((4, 2), dtype=np.float32)
-    for i in range(4):
-        for j in range(2):
-            s = np.float32(0)
-            for k in range(3):
-                s = np.float32(s + a[i, k] * b[k, j])
-            ref[i, j] = s
-    assert np.array_equal(out, ref)
 
 
 def test_fold_of_unfold_preserves_sum(frontend):
@@ -154,17 +140,11 @@ def _grads_on(fe, kind, build_loss, arrays):
         _INPUT_BUFFER_CACHE.clear()
 
 
-def test_autograd_known_answers(frontend):
-    # crates/backend-metal/src/lib.rs:262-368
-    x = np.array([1, 2, 3, 4], dtype=np.float32)
-    (gx,) = _grads_on(frontend, "c", lambda t: (t * t).sum(0), [x])
-    assert gx.tolist() == [2, 4, 6, 8]
-    a = np.array([1, 2, 3, 4], dtype=np.float32)
-    b = np.array([5, 6, 7, 8], dtype=np.float32)
-    ga, gb = _grads_on(frontend, "c", lambda s, t: (s * t).sum(0), [a, b])
-    assert ga.tolist() == [5, 6, 7, 8] and gb.tolist() == [1, 2, 3, 4]
-    (g2,) = _grads_on(frontend, "c", lambda t: (t + t).sum(0), [x])
-    assert g2.tolist() == [2, 2, 2, 2]
+@pytest.mark.parametrize("case", _FX["gradients"], ids=lambda c: c["id"])
+def test_fixture_gradient_known_answers(frontend, case):
+    arrays = [golden_ops.array(v, s) for v, s in zip(case["inputs"], case["shapes"])]
+    grads = _grads_on(frontend, "c", golden_ops.graph(frontend, case["op"]), arrays)
+    assert [g.tolist() for g in grads] == [[float(v) for v in e] for e in case["expected"]]
 
 
 def test_autograd_rules_as_written(frontend):
