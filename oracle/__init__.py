@@ -14,11 +14,15 @@ it; the product (`harp_amd`) never does and never falls back to it.
 What pins it (all without running the reference, whose Rust toolchain is not
 available): the rendered-text assertions the reference's own tests hold
 (`crates/backend-c/src/renderer.rs:262-296`, `src/backend/renderer.rs`
-literal forms), the reference's known-answer vectors (add/mul/2-D add,
-`crates/backend-c/src/lib.rs:183-245`; 2x2 matmul,
-`crates/backend-metal/src/compiler.rs:240-257`; fold-of-unfold sum,
-`crates/backend-c/src/lib.rs:299-340`), and numpy evaluation of the same
-graphs.  Parity unpinned: the reference's two AST beam searches may rewrite
+literal forms), the reference's known-answer vectors, kept as data in
+`tests/golden/reference_known_answers.json` (add/mul/2-D add,
+`crates/backend-c/src/lib.rs:181-246`; 10 000-element add,
+`crates/backend-openmp/src/lib.rs:207-230`; 2x2 matmul,
+`crates/backend-metal/src/compiler.rs:193-257`; the 4x3x2 matmul loop of
+`examples/matmul_demo.rs`; fold-of-unfold sum, `crates/backend-c/src/lib.rs:298-340`;
+three gradients, `crates/backend-metal/src/lib.rs:261-369`), and numpy evaluation
+of the same graphs (closed forms, finite differences for the exact VJPs,
+brute force over every index form).  Parity unpinned: the reference's two AST beam searches may rewrite
 `acc + a*b` into `fma(a, b, acc)` or re-tile loops before rendering; the
 oracle renders the AST as lowered, so reductions are compared within
 tolerance, never bit-for-bit.
