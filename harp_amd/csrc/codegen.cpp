@@ -319,9 +319,28 @@ struct StmtRenderer {
   }
 };
 
+// Value of a dispatch-size expression, evaluated as the reference's pipeline does
+// (`evaluate_ast_expr`, src/backend/pipeline.rs:505-553): constants, +, *, integer division and
+// remainder (a zero divisor gives 1 and 0), max.  Shape variables are not supported on this
+// path, so a variable or any other node is an error rather than the reference's silent 1.
 int64_t const_int(const Node& n, int64_t dflt) {
-  if (n.op == Op::Const && !n.dtype.is_float()) return n.ival;
-  return dflt;
+  (void)dflt;
+  switch (n.op) {
+    case Op::Const: return n.dtype.is_float() ? static_cast<int64_t>(n.fval) : n.ival;
+    case Op::Add: return const_int(*n.args[0], 1) + const_int(*n.args[1], 1);
+    case Op::Mul: return const_int(*n.args[0], 1) * const_int(*n.args[1], 1);
+    case Op::Idiv: {
+      const int64_t d = const_int(*n.args[1], 1);
+      return d != 0 ? const_int(*n.args[0], 1) / d : 1;
+    }
+    case Op::Rem: {
+      const int64_t d = const_int(*n.args[1], 1);
+      return d != 0 ? const_int(*n.args[0], 1) % d : 0;
+    }
+    case Op::Max: return std::max(const_int(*n.args[0], 1), const_int(*n.args[1], 1));
+    default:
+      throw Error(std::string("dispatch size uses '") + op_name(n.op) + "', which cannot be evaluated at compile time");
+  }
 }
 
 const char* kAtomicMaxF32 = R"EHA(

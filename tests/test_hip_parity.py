@@ -389,7 +389,8 @@ GROUP_PARALLEL_ADD = """
 GROUP_AND_LOCAL_ADD = """
 (program (kernel "E_1000_0" (params ("gidx0" i64 imm (group_id 0)) ("lidx0" i64 imm (local_id 0))
     ("buf0" (ptr f32 global) imm normal) ("buf2" (ptr f32 global) imm normal) ("buf4" (ptr f32 global) mut normal))
-  (grid (const i64 16) (const i64 1) (const i64 1)) (tg (const i64 64) (const i64 1) (const i64 1))
+  (grid (idiv (add (const i64 1000) (const i64 63)) (const i64 64)) (const i64 1) (const i64 1))
+  (tg (const i64 64) (const i64 1) (const i64 1))
   (block (decls)
     (if (lt (add (mul (var "gidx0") (const i64 64)) (var "lidx0")) (const i64 1000))
       (store (var "buf4") (add (mul (var "gidx0") (const i64 64)) (var "lidx0"))
@@ -403,8 +404,9 @@ GROUP_AND_LOCAL_ADD = """
 def test_kernels_parallelised_by_the_reference_run_as_written(hip, text, grid, block):
     """Kernels the reference's own suggesters have already parallelised carry group / local id
     parameters and their dispatch size (`src/opt/ast/suggesters/parallelization.rs:186-232`:
-    one workgroup per iteration, then a local axis with a bounds check).  They are launched
-    with exactly that size, ids bound to blockIdx / threadIdx."""
+    one workgroup per iteration, then a local axis with a bounds check and a `ceil_div` grid
+    size, evaluated as `src/backend/pipeline.rs:505-553` does).  They are launched with exactly
+    that size, ids bound to blockIdx / threadIdx."""
     dev = hip.HipDevice(0)
     k = hip.HipKernel(dev, text)
     l, = k.launches

@@ -171,6 +171,28 @@ def test_bad_options_and_bad_source_are_reported(frontend):
     assert e.value.code == 4 and "hiprtc" in str(e.value)
 
 
+@pytest.mark.parametrize("expr,value", [
+    ("(const i64 42)", 42),                                             # pipeline.rs:719-723
+    ("(mul (const i64 10) (const i64 20))", 200),                       # pipeline.rs:740-752
+    ("(add (const i64 10) (const i64 20))", 30),
+    ("(idiv (const i64 100) (const i64 10))", 10),
+    ("(idiv (add (const i64 1000) (const i64 63)) (const i64 64))", 16),   # ceil_div, parallelization_common.rs:575
+    ("(max (const i64 3) (rem (const i64 17) (const i64 5)))", 3),
+])
+def test_dispatch_size_expressions(expr, value):
+    """Grid sizes of kernels the reference has parallelised are expressions; they evaluate as
+    the reference's `evaluate_ast_expr` does (src/backend/pipeline.rs:505-553, cases of its
+    tests :718-752).  A shape variable is an error here, not a silent 1."""
+    from harp_amd import backend as hb
+    text = ('(program (kernel "k" (params ("g" i64 imm (group_id 0)) ("o" (ptr f32 global) mut normal)) '
+            f'(grid {expr} (const i64 1) (const i64 1)) (tg (const i64 1) (const i64 1) (const i64 1)) '
+            '(block (decls) (store (var "o") (var "g") (const f32 1.0)))))')
+    l, = hb.render_program(text).launches
+    assert l["schedule"] == "as-written" and l["grid"] == [value, 1, 1]
+    with pytest.raises(hb.EhError, match="cannot be evaluated"):
+        hb.render_program(text.replace(expr, '(var "n")'))
+
+
 def test_no_device_is_an_error_not_a_fallback():
     from harp_amd import backend as hb
     if hb.device_count() > 0:
