@@ -238,7 +238,10 @@ struct ExprRenderer {
         return "*reinterpret_cast<const " + ctype(n.dtype) + "*>(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "])";
       }
       case Op::SharedLoad: return expr(*n.args[0]) + "[" + expr(*n.args[1]) + "]";
-      case Op::Rand: return "0.5f /* rand is not available in device code */";
+      case Op::Rand:
+        // the C backend renders libc's rand() (src/backend/renderer.rs:313): host state, no
+        // device counterpart, and no graph operation produces the node
+        throw Error("the Rand node (libc rand() in the C backend) has no device implementation");
       case Op::Call: {
         std::string s = n.name + "(";
         for (size_t i = 0; i < n.args.size(); ++i) s += (i ? ", " : "") + expr(*n.args[i]);
@@ -323,21 +326,20 @@ struct StmtRenderer {
 // (`evaluate_ast_expr`, src/backend/pipeline.rs:505-553): constants, +, *, integer division and
 // remainder (a zero divisor gives 1 and 0), max.  Shape variables are not supported on this
 // path, so a variable or any other node is an error rather than the reference's silent 1.
-int64_t const_int(const Node& n, int64_t dflt) {
-  (void)dflt;
+int64_t dispatch_value(const Node& n) {
   switch (n.op) {
     case Op::Const: return n.dtype.is_float() ? static_cast<int64_t>(n.fval) : n.ival;
-    case Op::Add: return const_int(*n.args[0], 1) + const_int(*n.args[1], 1);
-    case Op::Mul: return const_int(*n.args[0], 1) * const_int(*n.args[1], 1);
+    case Op::Add: return dispatch_value(*n.args[0]) + dispatch_value(*n.args[1]);
+    case Op::Mul: return dispatch_value(*n.args[0]) * dispatch_value(*n.args[1]);
     case Op::Idiv: {
-      const int64_t d = const_int(*n.args[1], 1);
-      return d != 0 ? const_int(*n.args[0], 1) / d : 1;
+      const int64_t d = dispatch_value(*n.args[1]);
+      return d != 0 ? dispatch_value(*n.args[0]) / d : 1;
     }
     case Op::Rem: {
-      const int64_t d = const_int(*n.args[1], 1);
-      return d != 0 ? const_int(*n.args[0], 1) % d : 0;
+      const int64_t d = dispatch_value(*n.args[1]);
+      return d != 0 ? dispatch_value(*n.args[0]) % d : 0;
     }
-    case Op::Max: return std::max(const_int(*n.args[0], 1), const_int(*n.args[1], 1));
+    case Op::Max: return std::max(dispatch_value(*n.args[0]), dispatch_value(*n.args[1]));
     default:
       throw Error(std::string("dispatch size uses '") + op_name(n.op) + "', which cannot be evaluated at compile time");
   }
@@ -396,8 +398,8 @@ LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
   os << sr.stmt(*k.args[0]) << "}\n";
   ls.source = os.str();
   for (int i = 0; i < 3; ++i) {
-    int64_t g = k.grid.size() == 3 ? const_int(*k.grid[i], 1) : 1;
-    int64_t t = k.tg.size() == 3 ? const_int(*k.tg[i], 1) : 1;
+    int64_t g = k.grid.size() == 3 ? dispatch_value(*k.grid[i]) : 1;
+    int64_t t = k.tg.size() == 3 ? dispatch_value(*k.tg[i]) : 1;
     if (g < 1 || t < 1 || t > 1024) throw Error("kernel '" + k.name + "' has an unusable dispatch size");
     ls.block[i] = static_cast<unsigned>(t);
     ls.grid[i] = static_cast<unsigned>(g);   // the AST's grid size counts workgroups
@@ -474,8 +476,8 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
   for (const auto& p : k.params)
     if (p.kind != VarKind::Normal || !p.dtype.is_ptr()) return {};
   for (int i = 0; i < 3; ++i) {
-    if (k.grid.size() == 3 && const_int(*k.grid[i], 1) != 1) return {};
-    if (k.tg.size() == 3 && const_int(*k.tg[i], 1) != 1) return {};
+    if (k.grid.size() == 3 && dispatch_value(*k.grid[i]) != 1) return {};
+    if (k.tg.size() == 3 && dispatch_value(*k.tg[i]) != 1) return {};
   }
   const Node& body = *k.args[0];
   std::vector<const Node*> tops;
