@@ -110,6 +110,8 @@ bool mentions_var(const Node& n, const std::string& name) {
 }
 
 // acc = combine(acc, value): which reduction, and what is combined in.
+}  // namespace
+
 bool match_combine(const Node& e, const std::string& acc, ReduceKind* kind, NodePtr* value) {
   auto binary = [&](ReduceKind k) {
     if (is_var(*e.args[0], acc) && !mentions_var(*e.args[1], acc)) {
@@ -151,6 +153,8 @@ bool match_combine(const Node& e, const std::string& acc, ReduceKind* kind, Node
       return false;
   }
 }
+
+namespace {
 
 bool buffer_param(const std::vector<Param>& ps, const std::string& name, DType* elem) {
   for (const auto& p : ps)

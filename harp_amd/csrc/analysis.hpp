@@ -57,6 +57,10 @@ struct NestKernel {
 // or already parallelised kernels), which are rendered statement by statement instead.
 std::optional<NestKernel> extract_nest(const Node& kernel);
 
+// `e` as `combine(acc, value)` for one of the reference's reduce / scan operators
+// (src/graph/node.rs:63-77): sum, product, max, select-min, or the fused multiply-add form.
+bool match_combine(const Node& e, const std::string& acc, ReduceKind* kind, NodePtr* value);
+
 // Every Load in an expression, in evaluation order, with whether it sits under a Select branch.
 struct LoadRef {
   const Node* load;

@@ -419,6 +419,50 @@ struct WriteRef {
   bool atomic;      // AtomicAdd / AtomicMax: safe from any number of work-items at once
 };
 
+// A prefix scan along one line, as `LoopGenerator::generate_scan` writes it
+// (src/lowerer/lower.rs:691-735): acc = identity; for the inner loops { acc = combine(acc,
+// value); out[index] = acc }.
+struct ScanLine {
+  std::string acc;
+  DType acc_dtype;
+  NodePtr identity, value, out_ptr, out_index;
+  ReduceKind kind = ReduceKind::None;
+  std::vector<Loop> loops;     // the scanned loops, outermost first
+  int64_t length = 1;
+};
+
+std::optional<ScanLine> match_scan_line(const Node& n) {
+  if (n.op != Op::Block || n.decls.size() != 1 || n.args.size() != 2) return std::nullopt;
+  ScanLine sl;
+  sl.acc = n.decls[0].first;
+  sl.acc_dtype = n.decls[0].second;
+  const Node& init = *n.args[0];
+  if (init.op != Op::Assign || init.name != sl.acc || init.args[0]->op != Op::Const) return std::nullopt;
+  sl.identity = init.args[0];
+  const Node* cur = n.args[1].get();
+  while (cur->op == Op::Range && cur->args[0]->op == Op::Const && cur->args[0]->ival == 0 &&
+         cur->args[1]->op == Op::Const && cur->args[1]->ival == 1 && cur->args[2]->op == Op::Const &&
+         cur->args[2]->ival >= 1) {
+    sl.loops.push_back({cur->name, cur->args[2]->ival});
+    sl.length *= cur->args[2]->ival;
+    const Node* b = cur->args[3].get();
+    while (b->op == Op::Block && b->decls.empty() && b->args.size() == 1) b = b->args[0].get();
+    cur = b;
+  }
+  if (sl.loops.empty() || cur->op != Op::Block || !cur->decls.empty() || cur->args.size() != 2) return std::nullopt;
+  const Node& step = *cur->args[0];
+  const Node& store = *cur->args[1];
+  if (step.op != Op::Assign || step.name != sl.acc) return std::nullopt;
+  if (!match_combine(*step.args[0], sl.acc, &sl.kind, &sl.value)) return std::nullopt;
+  if (sl.kind != ReduceKind::Sum && sl.kind != ReduceKind::Prod && sl.kind != ReduceKind::Max) return std::nullopt;
+  if (store.op != Op::Store || store.args[2]->op != Op::Var || store.args[2]->name != sl.acc) return std::nullopt;
+  sl.out_ptr = store.args[0];
+  sl.out_index = store.args[1];
+  return sl;
+}
+
+std::string combine_text(ReduceKind k, const DType& t, const std::string& acc, const std::string& v);
+
 void collect_writes(const Node& n, std::vector<WriteRef>& writes, std::set<std::string>& read_bufs,
                     std::map<std::string, int64_t>& inner_extents, bool* ok) {
   if (n.op == Op::Store || n.op == Op::AtomicAdd || n.op == Op::AtomicMax) {
@@ -564,7 +608,67 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
     std::ostringstream os;
     os << hdr(opt) << kAtomicMaxF32;
     StmtRenderer sr;
-    if (spread) {
+    // A long scanned line gets a workgroup instead of a work-item: tiles of 256 x 4 elements,
+    // each thread scans its four, the wave and then the workgroup scan the thread totals, and
+    // the tile's total is carried into the next tile.  The combine order differs from the
+    // sequential one (exact for max, the reduction tolerance for sums and products).
+    std::optional<ScanLine> scan = spread ? match_scan_line(*inner) : std::nullopt;
+    if (scan && scan->length >= 512) {
+      int64_t lines = 1;
+      for (const auto& l : loops) lines *= l.extent;
+      if (lines >= (int64_t{1} << 31)) return {};
+      const std::string T = ctype(scan->acc_dtype);
+      const std::string ident = literal(*scan->identity);
+      ExprRenderer er;
+      auto comb = [&](const std::string& a, const std::string& b) { return combine_text(scan->kind, scan->acc_dtype, a, b); };
+      os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << sig << ") {\n";
+      os << "  long long eh_r = blockIdx.x;\n";
+      for (size_t i = loops.size(); i-- > 0;) {
+        os << "  const long long " << loops[i].var << " = eh_r % " << loops[i].extent << ";\n";
+        if (i) os << "  eh_r /= " << loops[i].extent << ";\n";
+      }
+      os << "  __shared__ " << T << " eh_wave_total[4];\n";
+      os << "  const int eh_lane = threadIdx.x & 63, eh_wave = threadIdx.x >> 6;\n";
+      os << "  " << T << " eh_carry = " << ident << ";\n";
+      os << "  for (long long eh_t0 = 0; eh_t0 < " << scan->length << "ll; eh_t0 += 1024) {\n";
+      os << "    " << T << " eh_v[4];\n";
+      os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+      os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
+      os << "      eh_v[eh_e] = " << ident << ";\n";
+      os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
+      for (size_t i = scan->loops.size(); i-- > 0;) {
+        os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
+        if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+      }
+      os << "        eh_v[eh_e] = (" << T << ")(" << er.expr(*scan->value) << ");\n      }\n";
+      os << "      if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n    }\n";
+      // inclusive scan of the thread totals across the wave, then across the four waves
+      os << "    " << T << " eh_inc = eh_v[3];\n";
+      os << "#pragma unroll\n    for (int eh_d = 1; eh_d < 64; eh_d <<= 1) {\n";
+      os << "      const " << T << " eh_o = __shfl_up(eh_inc, eh_d, 64);\n";
+      os << "      if (eh_lane >= eh_d) eh_inc = " << comb("eh_o", "eh_inc") << ";\n    }\n";
+      os << "    if (eh_lane == 63) eh_wave_total[eh_wave] = eh_inc;\n    __syncthreads();\n";
+      os << "    " << T << " eh_before = eh_carry;            // everything ahead of this thread's four\n";
+      os << "    for (int eh_w = 0; eh_w < eh_wave; ++eh_w) eh_before = " << comb("eh_before", "eh_wave_total[eh_w]") << ";\n";
+      os << "    const " << T << " eh_prev = __shfl_up(eh_inc, 1, 64);\n";
+      os << "    if (eh_lane) eh_before = " << comb("eh_before", "eh_prev") << ";\n";
+      os << "    " << T << " eh_all = eh_carry;\n";
+      os << "    for (int eh_w = 0; eh_w < 4; ++eh_w) eh_all = " << comb("eh_all", "eh_wave_total[eh_w]") << ";\n";
+      os << "    eh_carry = eh_all;\n";
+      os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+      os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
+      os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
+      for (size_t i = scan->loops.size(); i-- > 0;) {
+        os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
+        if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+      }
+      os << "        " << er.expr(*scan->out_ptr) << "[" << er.expr(*scan->out_index) << "] = " << comb("eh_before", "eh_v[eh_e]") << ";\n      }\n    }\n";
+      os << "    __syncthreads();\n  }\n}\n";
+      ls.grid[0] = static_cast<unsigned>(lines);
+      ls.block[0] = 256;
+      ls.schedule = "scan-row(lines=" + std::to_string(lines) + ",length=" + std::to_string(scan->length) + ")";
+      any_parallel = true;
+    } else if (spread) {
       int64_t total = 1;
       for (const auto& l : loops) total *= l.extent;
       if (total >= (int64_t{1} << 40)) return {};

@@ -812,7 +812,12 @@ SPREAD_FORMS = {
     "cumsum_rows": ((300, 257), lambda t: t.cumsum(1), "outer-parallel(work-items=300)"),
     # as lowered, the accumulator of a mid-axis scan runs on over the inner axis too: only axis 0 is free
     "cumprod_mid": ((6, 50, 9), lambda t: t.cumprod(1), "outer-parallel(work-items=6)"),
-    "cummax_rows": ((128, 1000), lambda t: t.cummax(1), "outer-parallel(work-items=128)"),
+    "cummax_rows": ((128, 300), lambda t: t.cummax(1), "outer-parallel(work-items=128)"),
+    # lines of 512 elements and more get a workgroup each: tiles of 1024, carry between tiles
+    "cummax_long": ((128, 1000), lambda t: t.cummax(1), "scan-row(lines=128,length=1000)"),
+    "cumsum_long": ((37, 5000), lambda t: t.cumsum(1), "scan-row(lines=37,length=5000)"),
+    "cumprod_long": ((8, 3001), lambda t: t.cumprod(1), "scan-row(lines=8,length=3001)"),
+    "cumsum_mid_long": ((3, 200, 9), lambda t: t.cumsum(1), "scan-row(lines=3,length=1800)"),
     "fold_tiles": ((64, 96), lambda t: t.unfold([0, 1], [2, 3], [2, 3], [1, 1])
                    .fold([64, 96], [0, 1], [2, 3], [2, 3], [1, 1]), "outer-parallel(work-items=6144)"),
     "fold_overlapping": ((20, 30), lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1])
@@ -830,14 +835,17 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
     products, and the atomic additions of overlapping windows (whose order is open), are held
     to the reduction tolerance, as everywhere."""
     shape, fn, expect = SPREAD_FORMS[name]
-    x = RNG(len(name)).uniform(0.5, 1.5, shape).astype(np.float32)
+    lo, hi = (0.995, 1.005) if name == "cumprod_long" else (0.5, 1.5)      # a long product must stay finite
+    x = RNG(len(name)).uniform(lo, hi, shape).astype(np.float32)
     t = frontend.Tensor.input(list(shape))
     prog, _, _ = frontend.lower_graph([fn(t).graph])
     scheds = [l["schedule"] for l in hip.render_program(prog).launches]
     assert expect in scheds, scheds
     ref, got = both(frontend, fn, [x], False)
     if name.startswith(("cumsum", "cumprod", "fold_overlapping")):   # order of the additions is open: reduction class
-        assert np.allclose(got, ref, rtol=1e-6)
+        assert np.allclose(got, ref, rtol=1e-5 if name.endswith("_long") else 1e-6)
+        if name == "cumsum_long":
+            assert np.allclose(got.reshape(shape), np.cumsum(x.astype(np.float64), 1), rtol=1e-5)
     else:
         assert bits_equal_mod_zero(ref, got)
 
