@@ -627,21 +627,61 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
         os << "  const long long " << loops[i].var << " = eh_r % " << loops[i].extent << ";\n";
         if (i) os << "  eh_r /= " << loops[i].extent << ";\n";
       }
+      // 128-bit accesses when the line is one loop walked with unit stride by every load and by
+      // the store, everything 16-byte aligned, four-byte elements
+      bool vec = scan->loops.size() == 1 && scan->length % 4 == 0 && scan->acc_dtype.itemsize() == 4;
+      const std::string sv = scan->loops[0].var;
+      std::vector<LoadRef> sloads;
+      collect_loads(*scan->value, sloads);
+      auto unit_aligned = [&](const Node& index) {
+        auto a = affine_of(index);
+        if (!a || a->of(sv) != 1 || a->c % 4) return false;
+        for (const auto& kv : a->coef)
+          if (kv.first != sv && kv.second % 4) return false;
+        return true;
+      };
+      for (const auto& lr : sloads)
+        vec = vec && !lr.guarded && lr.load->count == 1 && lr.load->dtype.itemsize() == 4 &&
+              lr.load->args[0]->op == Op::Var && unit_aligned(*lr.load->args[1]);
+      vec = vec && scan->out_ptr->op == Op::Var && unit_aligned(*scan->out_index);
       os << "  __shared__ " << T << " eh_wave_total[4];\n";
       os << "  const int eh_lane = threadIdx.x & 63, eh_wave = threadIdx.x >> 6;\n";
       os << "  " << T << " eh_carry = " << ident << ";\n";
       os << "  for (long long eh_t0 = 0; eh_t0 < " << scan->length << "ll; eh_t0 += 1024) {\n";
       os << "    " << T << " eh_v[4];\n";
-      os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
-      os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
-      os << "      eh_v[eh_e] = " << ident << ";\n";
-      os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
-      for (size_t i = scan->loops.size(); i-- > 0;) {
-        os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
-        if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+      if (vec) {
+        os << "    const long long eh_tb = eh_t0 + threadIdx.x * 4;\n    const bool eh_in = eh_tb < " << scan->length << "ll;\n";
+        os << "    {\n      const long long " << sv << " = eh_in ? eh_tb : 0;\n";
+        std::vector<std::string> seen;
+        for (const auto& lr : sloads) {
+          const std::string key = to_text(*lr.load);
+          if (std::find(seen.begin(), seen.end(), key) != seen.end()) continue;
+          os << "      const EhV4<" << ctype(lr.load->dtype) << "> eh_ld" << seen.size() << " = eh_load4<false>("
+             << lr.load->args[0]->name << " + " << er.expr(*lr.load->args[1]) << ");\n";
+          seen.push_back(key);
+        }
+        ExprRenderer ev;
+        ev.load_hook = [&](const Node& ld, std::string* out) {
+          const std::string key = to_text(ld);
+          for (size_t q = 0; q < seen.size(); ++q)
+            if (seen[q] == key) { *out = "eh_ld" + std::to_string(q) + "[eh_e]"; return true; }
+          return false;
+        };
+        os << "#pragma unroll\n      for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+        os << "        eh_v[eh_e] = eh_in ? (" << T << ")(" << ev.expr(*scan->value) << ") : " << ident << ";\n";
+        os << "        if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n      }\n    }\n";
+      } else {
+        os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+        os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
+        os << "      eh_v[eh_e] = " << ident << ";\n";
+        os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
+        for (size_t i = scan->loops.size(); i-- > 0;) {
+          os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
+          if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+        }
+        os << "        eh_v[eh_e] = (" << T << ")(" << er.expr(*scan->value) << ");\n      }\n";
+        os << "      if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n    }\n";
       }
-      os << "        eh_v[eh_e] = (" << T << ")(" << er.expr(*scan->value) << ");\n      }\n";
-      os << "      if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n    }\n";
       // inclusive scan of the thread totals across the wave, then across the four waves
       os << "    " << T << " eh_inc = eh_v[3];\n";
       os << "#pragma unroll\n    for (int eh_d = 1; eh_d < 64; eh_d <<= 1) {\n";
@@ -655,14 +695,20 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       os << "    " << T << " eh_all = eh_carry;\n";
       os << "    for (int eh_w = 0; eh_w < 4; ++eh_w) eh_all = " << comb("eh_all", "eh_wave_total[eh_w]") << ";\n";
       os << "    eh_carry = eh_all;\n";
-      os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
-      os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
-      os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
-      for (size_t i = scan->loops.size(); i-- > 0;) {
-        os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
-        if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+      if (vec) {
+        os << "    if (eh_in) {\n      const long long " << sv << " = eh_tb;\n      EhV4<" << T << "> eh_out;\n";
+        os << "#pragma unroll\n      for (int eh_e = 0; eh_e < 4; ++eh_e) eh_out[eh_e] = " << comb("eh_before", "eh_v[eh_e]") << ";\n";
+        os << "      eh_store4<false>(" << scan->out_ptr->name << " + " << er.expr(*scan->out_index) << ", eh_out);\n    }\n";
+      } else {
+        os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+        os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
+        os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
+        for (size_t i = scan->loops.size(); i-- > 0;) {
+          os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
+          if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+        }
+        os << "        " << er.expr(*scan->out_ptr) << "[" << er.expr(*scan->out_index) << "] = " << comb("eh_before", "eh_v[eh_e]") << ";\n      }\n    }\n";
       }
-      os << "        " << er.expr(*scan->out_ptr) << "[" << er.expr(*scan->out_index) << "] = " << comb("eh_before", "eh_v[eh_e]") << ";\n      }\n    }\n";
       os << "    __syncthreads();\n  }\n}\n";
       ls.grid[0] = static_cast<unsigned>(lines);
       ls.block[0] = 256;
