@@ -525,7 +525,15 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
   }
   const Node& body = *k.args[0];
   std::vector<const Node*> tops;
-  if (body.op == Op::Block) {
+  // a scan lowered with one accumulator for the whole tensor (axis 0) is a single line
+  bool whole_scan = false;
+  if (body.op == Op::Block && !body.decls.empty()) {
+    auto sl = match_scan_line(body);
+    whole_scan = sl && sl->length >= 512;        // a short one stays as written
+  }
+  if (whole_scan) {
+    tops.push_back(&body);
+  } else if (body.op == Op::Block) {
     if (!body.decls.empty()) return {};
     for (const auto& a : body.args) tops.push_back(a.get());
   } else {
@@ -551,7 +559,7 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
   }
   bool any_parallel = false;
   for (size_t t = 0; t < tops.size(); ++t) {
-    if (tops[t]->op != Op::Range) return {};
+    if (tops[t]->op != Op::Range && !whole_scan) return {};
     // the perfect nest at the top of this statement
     std::vector<Loop> loops;
     const Node* cur = tops[t];
@@ -565,7 +573,7 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       if (cur->op != Op::Range) break;
     }
     const Node* inner = cur;
-    if (loops.empty()) return {};
+    if (loops.empty() && !whole_scan) return {};
     if (inner->op == Op::Range) {
       // the walk stopped at a loop it cannot spread (non-constant bounds): keep it inside
     }

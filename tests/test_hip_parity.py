@@ -818,6 +818,8 @@ SPREAD_FORMS = {
     "cumsum_long": ((37, 5000), lambda t: t.cumsum(1), "scan-row(lines=37,length=5000)"),
     "cumprod_long": ((8, 3001), lambda t: t.cumprod(1), "scan-row(lines=8,length=3001)"),
     "cumsum_mid_long": ((3, 200, 9), lambda t: t.cumsum(1), "scan-row(lines=3,length=1800)"),
+    # a scan over axis 0 is lowered with one accumulator for the whole tensor: one long line
+    "cummax_axis0": ((300, 50), lambda t: t.cummax(0), "scan-row(lines=1,length=15000)"),
     "fold_tiles": ((64, 96), lambda t: t.unfold([0, 1], [2, 3], [2, 3], [1, 1])
                    .fold([64, 96], [0, 1], [2, 3], [2, 3], [1, 1]), "outer-parallel(work-items=6144)"),
     "fold_overlapping": ((20, 30), lambda t: t.unfold([0, 1], [3, 3], [1, 1], [1, 1])
