@@ -153,7 +153,14 @@ def compile_ast_with_cache(program, signature=None):
     return kernel
 
 
-_PROGRAM_CACHE_CAPACITY = 64          # whole programs keep their temporaries resident
+_PROGRAM_CACHE_CAPACITY = 64          # whole programs keep their temporaries resident,
+_PROGRAM_CACHE_BYTES = 32 << 30       # so the cache is also bounded by what they hold on the device
+
+
+def _resident_bytes(compiled) -> int:
+    """Device memory a cached program keeps between runs (its temporaries)."""
+    return sum(b["bytes"] for b in getattr(compiled, "buffers", ())
+               if b.get("role") == "temp" and not b.get("elided"))
 
 
 def compile_program_with_cache(program):
@@ -174,7 +181,9 @@ def compile_program_with_cache(program):
     compiled = d.compile_program(program)
     with _lock:
         _program_cache[key] = compiled
-        while len(_program_cache) > _PROGRAM_CACHE_CAPACITY:
+        while len(_program_cache) > 1 and (len(_program_cache) > _PROGRAM_CACHE_CAPACITY or
+                                           sum(_resident_bytes(p) for p in _program_cache.values())
+                                           > _PROGRAM_CACHE_BYTES):
             _program_cache.popitem(last=False)
             _cache_stats["evictions"] += 1
     return compiled
