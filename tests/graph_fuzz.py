@@ -44,12 +44,15 @@ SMALL_DIMS = (1, 2, 3, 5, 8, 13, 32, 64, 100)
 LARGE_DIMS = (1, 4, 31, 128, 257, 1000, 2048)      # with at most two axes: up to 4 Mi elements
 
 
-def build(seed: int, fe, dims=SMALL_DIMS, max_rank=3):
-    """Returns (input shapes, function of input tensors -> output tensor, description)."""
+def build(seed: int, fe, dims=SMALL_DIMS, max_rank=3, kinds=(0, 8)):
+    """Returns (input shapes, function of input tensors -> output tensor, description).
+    `kinds` is the half-open range the final stage is drawn from: 0-7 are reductions, gathering
+    copies, row normalisations, padding, contractions, broadcasts and reshapes; 8-11 prefix
+    scans, selects on comparisons, sliding windows and batched contractions."""
     rng = np.random.default_rng(seed)
     nd = int(rng.integers(1, max_rank + 1))
     shape = [int(rng.choice(dims)) for _ in range(nd)]
-    kind = int(rng.integers(0, 8))
+    kind = int(rng.integers(kinds[0], kinds[1]))
     red = int(rng.integers(0, 3))                        # kind 0: sum, max or min
     has_y = bool(rng.integers(0, 2))
     has_w = kind == 4 and nd >= 2
@@ -84,6 +87,25 @@ def build(seed: int, fe, dims=SMALL_DIMS, max_rank=3):
             t = _binary(r, t, v.expand(0, t.shape()[0])) if t.ndim() >= 2 else _unary(r, fe, t)
         elif kind == 6:                                 # reduce, then elementwise on the result
             t = _unary(r, fe, t.sum(t.ndim() - 1))
+        elif kind == 8:                                 # prefix scan over the last axis
+            ax = t.ndim() - 1
+            # nothing after it: a prefix sum's rounding depends on the order of its additions, and
+            # a steep function of the result would turn that into a large relative difference
+            t = [t.cumsum, t.cummax][int(r.integers(0, 2))](ax)
+        elif kind == 9:                                 # select on a comparison
+            other = _unary(r, fe, t)
+            cond = [t.lt, t.ge, t.gt, t.le][int(r.integers(0, 4))](other)
+            t = t.where_cond(cond, other * other)
+        elif kind == 10:                                # sliding windows over the last axis, reduced
+            n = t.shape()[-1]
+            k = 2 if n >= 2 else 1
+            stride = int(r.integers(1, 3))
+            w = t.unfold([t.ndim() - 1], [k], [stride], [1]).contiguous()
+            t = [w.max, w.sum][int(r.integers(0, 2))](w.ndim() - 1)
+        elif kind == 11 and t.ndim() == 3:              # batched contraction over the last axis
+            a = t.unsqueeze(2)                          # [B, M, 1, K]
+            b = _unary(r, fe, t).unsqueeze(1)           # [B, 1, M, K]
+            t = (a * b).sum(3)                          # [B, M, M]
         else:                                           # reshape to rows of a different length
             n = t.numel()
             cols = [c for c in (1, 2, 4, 5, 8, 10, 16, 25) if n % c == 0]

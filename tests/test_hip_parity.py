@@ -867,6 +867,40 @@ def test_random_graphs_match_the_oracle(frontend, hip, seed):
     assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), desc
 
 
+@pytest.mark.parametrize("seed", range(600, 632))
+def test_random_graphs_with_scans_selects_and_windows(frontend, hip, seed):
+    """The same generator ending in a prefix scan, a select on a comparison, sliding windows
+    (unfold) or a batched contraction; small and large axes alternate."""
+    import graph_fuzz
+    large = seed % 2 == 1
+    shapes, fn, desc = graph_fuzz.build(seed, frontend, kinds=(8, 12),
+                                        dims=graph_fuzz.LARGE_DIMS if large else graph_fuzz.SMALL_DIMS,
+                                        max_rank=2 if large else 3)
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    # Lowered in exact mode: as the reference lowers it, a reader of a materialised unfold
+    # indexes the window buffer with the unfold's input-space view and runs past its end
+    # (`lower.rs:344-348` vs `:221-224`); the HIP backend refuses such a launch on the host.
+    # A prefix sum near zero has lost the digits its terms cancelled: scans are held to the
+    # size of the largest prefix instead.
+    rtol = 2e-4 if "kind 8" in desc else 2e-5
+    with frontend.exact_mode():
+        for fuse in (True, False):
+            ref, got = both(frontend, fn, arrays, fuse)
+            assert ref.shape == got.shape, desc
+            scale = max(1.0, float(np.abs(ref).max()))
+            assert np.allclose(got, ref, rtol=rtol, atol=2e-6 * scale), (desc, fuse)
+
+
+def test_out_of_bounds_reader_of_a_materialised_unfold_is_refused(frontend, hip):
+    """Lowered as the reference does, max over sliding windows reads the contiguous window
+    buffer [257,128,2] through the unfold's own view (row stride 257) and would run 255
+    elements past its end; the launch is rejected on the host instead of faulting."""
+    x = RNG(1).normal(0, 1, (257, 257)).astype(np.float32)
+    with pytest.raises(hip.EhError, match="needs at least"):
+        realize_on(frontend, "hip", lambda t: t.unfold([1], [2], [2], [1]).contiguous().max(2), [x])
+
+
 @pytest.mark.parametrize("seed", range(5000, 5012))
 def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
     """The same generator with one or two axes of up to 2048 elements: vectorised accesses,
