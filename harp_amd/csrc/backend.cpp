@@ -104,7 +104,7 @@ std::string HipCompiler::cache_dir() {
   return base + "/kernels/Hip";
 }
 
-Binary HipCompiler::compile(const std::string& source, const std::string& arch, bool use_disk_cache) {
+Binary HipCompiler::compile(const std::string& source, const std::string& arch, bool use_disk_cache, bool refresh) {
   std::vector<std::string> opts = options(arch);
   int maj = 0, min = 0;
   hiprtcVersion(&maj, &min);
@@ -112,15 +112,24 @@ Binary HipCompiler::compile(const std::string& source, const std::string& arch, 
   for (const auto& o : opts) key_text += "\n" + o;
   key_text += "\nhiprtc " + std::to_string(maj) + "." + std::to_string(min);
   const std::string key = hash_hex(key_text);
-  if (auto hit = g_bin_cache.find(key)) return *hit;
+  if (!refresh)
+    if (auto hit = g_bin_cache.find(key)) return *hit;
   const bool disk = use_disk_cache && disk_cache_enabled();
   const std::string path = cache_dir() + "/" + key + ".bin";
   Binary out;
-  if (disk) {
+  const std::string meta_path = cache_dir() + "/" + key + ".json";
+  if (disk && !refresh) {
+    // a cached code object counts only if its side file vouches for it: same length, same hash
+    // (a truncated or half-written file must never reach the module loader)
     std::ifstream f(path, std::ios::binary);
-    if (f) {
+    std::ifstream m(meta_path);
+    if (f && m) {
+      std::string meta((std::istreambuf_iterator<char>(m)), std::istreambuf_iterator<char>());
       out.code.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
-      out.from_cache = !out.code.empty();
+      const std::string want = "\"fnv1a\": \"" + hash_hex(std::string(out.code.begin(), out.code.end())) + "\"";
+      const std::string len = "\"bytes\": " + std::to_string(out.code.size());
+      out.from_cache = !out.code.empty() && meta.find(want) != std::string::npos && meta.find(len) != std::string::npos;
+      if (!out.from_cache) out.code.clear();
     }
   }
   if (!out.from_cache) {
@@ -155,9 +164,10 @@ Binary HipCompiler::compile(const std::string& source, const std::string& arch, 
         f.write(out.code.data(), static_cast<std::streamsize>(out.code.size()));
         f.close();
         std::rename(tmp.c_str(), path.c_str());
-        std::ofstream meta(cache_dir() + "/" + key + ".json");
+        std::ofstream meta(meta_path);
         meta << "{\"arch\": \"" << arch << "\", \"hiprtc\": \"" << maj << "." << min << "\", \"bytes\": "
-             << out.code.size() << "}\n";
+             << out.code.size() << ", \"fnv1a\": \"" << hash_hex(std::string(out.code.begin(), out.code.end()))
+             << "\"}\n";
       }
     }
   }
@@ -407,7 +417,14 @@ HipProgram::HipProgram(HipDevice* dev, const std::string& ast_text, const GenOpt
     for (const auto& a : ls.arg_bufs)
       if (!index_.count(a)) throw Error("launch '" + ls.entry + "' binds unknown buffer '" + a + "'");
     Binary bin = HipCompiler::compile(ls.source, o.arch);
-    kernels_.push_back(dev_->load(bin, ls.entry));
+    try {
+      kernels_.push_back(dev_->load(bin, ls.entry));
+    } catch (...) {
+      // a cached code object the loader rejects: compile afresh, replace it, try once more
+      if (!bin.from_cache) throw;
+      bin = HipCompiler::compile(ls.source, o.arch, true, true);
+      kernels_.push_back(dev_->load(bin, ls.entry));
+    }
   }
 }
 

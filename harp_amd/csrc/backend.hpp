@@ -37,7 +37,10 @@ struct Binary {
 class HipCompiler {
  public:
   // HIP C -> gfx950 code object.  Needs no device.  Throws eh::Error carrying the hiprtc log.
-  static Binary compile(const std::string& source, const std::string& arch, bool use_disk_cache = true);
+  // `refresh` ignores what the caches hold for this source and overwrites it (used when a
+  // cached code object turns out not to load).
+  static Binary compile(const std::string& source, const std::string& arch, bool use_disk_cache = true,
+                        bool refresh = false);
   static std::vector<std::string> options(const std::string& arch);
   static std::string cache_dir();      // HARP_CACHE_DIR or ~/.cache/harp, + /kernels/Hip
   static bool disk_cache_enabled();    // HARP_NO_DISK_CACHE unset

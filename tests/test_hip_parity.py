@@ -458,6 +458,41 @@ def test_concurrent_compile_and_execute(frontend, hip):
     assert not errors, errors
 
 
+def test_corrupt_disk_cache_entry_is_replaced(frontend, hip, tmp_path, monkeypatch):
+    """A code object in the disk cache that does not load (truncated file) is compiled afresh
+    and overwritten instead of failing every later run."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import sys, os, numpy as np\n"
+        "sys.path.insert(0, %r)\n"
+        "from harp_amd import backend as hb, workloads as wl\n"
+        "ast, names, out, consts, _ = wl.lower_with_table([(64, 96)], lambda t: t * t + t)\n"
+        "dev = hb.HipDevice(0)\n"
+        "prog = hb.HipProgram(dev, ast, None)\n"
+        "x = np.arange(64 * 96, dtype=np.float32).reshape(64, 96) / 100\n"
+        "b = dev.alloc(x.nbytes); b.write_array(x)\n"
+        "res = prog.execute({names[0]: b})[out].read_array(np.float32, x.shape)\n"
+        "assert np.array_equal(res, x * x + x)\n"
+        "print('ok')\n") % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, HARP_CACHE_DIR=str(tmp_path))
+    env.pop("HARP_NO_DISK_CACHE", None)
+    run = lambda: subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    first = run()
+    assert first.returncode == 0, first.stderr
+    bins = [os.path.join(dp, f) for dp, _, fs in os.walk(tmp_path) for f in fs if f.endswith(".bin")]
+    assert bins, "nothing was cached"
+    sizes = {}
+    for path in bins:
+        sizes[path] = os.path.getsize(path)
+        with open(path, "r+b") as f:
+            f.truncate(100)
+    second = run()                                     # fresh process: only the disk cache is left
+    assert second.returncode == 0, second.stderr
+    assert all(os.path.getsize(p) == n for p, n in sizes.items())
+
+
 def test_c_client_runs_the_known_answer(hip):
     """The plain-C client (tests/capi_client.c, built with the library) computes the
     reference's [1,2,3,4] + [5,6,7,8] through the C ABI alone, from the compiled program and
