@@ -641,6 +641,50 @@ def test_config4_mlp_training_step(frontend, hip, batch, dims, fuse):
         assert np.allclose(g.reshape(p.shape), p - 1e-3 * gr, rtol=1e-4, atol=1e-6)
 
 
+def test_compiled_step_fed_back_matches_eager_steps(frontend, hip):
+    """`CompiledStep` lowers and compiles the MLP step once and is then called three times with
+    its own outputs (the updated parameters, still on the device) as the next inputs; the
+    oracle runs the same three steps through the eager path, re-lowering each time."""
+    from harp_amd import workloads as wl
+    from harp_amd.step import CompiledStep
+    arrays = wl.config4_inputs(64, (32, 64, 64, 32), seed=5)
+    step = CompiledStep(lambda *ts: wl.config4_graph(*ts, lr=0.05), [a.shape for a in arrays])
+    assert len(step.launches) < step.lowered_kernels // 2
+    bufs = [step.upload(a) for a in arrays]
+    ref_arrays = list(arrays)
+    for _ in range(3):
+        outs = step(*bufs)
+        bufs = bufs[:2] + outs[:-1]
+        frontend.set_device_str("c")
+        ref = _train_step_with_lr(frontend, ref_arrays, 0.05)
+        ref_arrays = ref_arrays[:2] + [r.reshape(a.shape) for r, a in zip(ref[:-1], arrays[2:])]
+        got_loss = float(outs[-1].read_array(np.float32)[0])
+        assert abs(got_loss - float(ref[-1][0])) <= 1e-5 * abs(float(ref[-1][0]))
+    for b, r in zip(bufs[2:], ref_arrays[2:]):
+        assert np.allclose(b.read_array(np.float32, r.shape), r, rtol=1e-4, atol=1e-6)
+    with pytest.raises(ValueError):
+        step(*bufs[:-1])
+    with pytest.raises(ValueError):
+        step(*(bufs[:-1] + [bufs[0]]))                  # wrong size for the last parameter
+
+
+def _train_step_with_lr(fe, arrays, lr):
+    from harp_amd import workloads as wl
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    try:
+        with fe.exact_mode():
+            ts = []
+            for a in arrays:
+                t = fe.Tensor.input(list(a.shape))
+                t.set_data(a)
+                ts.append(t)
+            roots = wl.config4_graph(*ts, lr=lr)
+            fe.realize_many(roots)
+            return [r.to_numpy() for r in roots]
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+
+
 def _cnn_step_on(fe, kind, arrays, fuse=True, lr=None):
     import os
     from harp_amd import workloads as wl
