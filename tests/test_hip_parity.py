@@ -931,7 +931,7 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
         assert bits_equal_mod_zero(ref, got)
 
 
-@pytest.mark.parametrize("seed", range(96))
+@pytest.mark.parametrize("seed", range(64))
 def test_random_graphs_match_the_oracle(frontend, hip, seed):
     """Differential test on seeded random graphs (tests/graph_fuzz.py): elementwise chains,
     views, reductions over any axis, row normalisations, small contractions.  Held to the
@@ -946,7 +946,7 @@ def test_random_graphs_match_the_oracle(frontend, hip, seed):
     assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), desc
 
 
-@pytest.mark.parametrize("seed", range(600, 632))
+@pytest.mark.parametrize("seed", range(600, 624))
 def test_random_graphs_with_scans_selects_and_windows(frontend, hip, seed):
     """The same generator ending in a prefix scan, a select on a comparison, sliding windows
     (unfold) or a batched contraction; small and large axes alternate."""
@@ -995,7 +995,7 @@ def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
         assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
 
 
-@pytest.mark.parametrize("seed", range(400, 408))
+@pytest.mark.parametrize("seed", range(400, 405))
 def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
     """Random conv + pool + linear classifiers (tests/graph_fuzz.py): forward with the fused
     and the per-kernel path, then every gradient of the summed output in exact mode."""
@@ -1044,7 +1044,7 @@ def _grads_on(fe, kind, shapes, fn, arrays):
         _INPUT_BUFFER_CACHE.clear()
 
 
-@pytest.mark.parametrize("seed", range(200, 248))
+@pytest.mark.parametrize("seed", range(200, 232))
 def test_random_graph_gradients_match_the_oracle(frontend, hip, seed):
     """The same random graphs, differentiated: loss = sum of the output, exact-mode VJPs,
     all gradients and the loss as roots of one Program.  HIP against the C oracle."""
