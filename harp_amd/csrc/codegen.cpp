@@ -2119,7 +2119,7 @@ struct SerialReduce {
   std::vector<LaunchSpec> split(std::vector<BufferInfo>* buffers) const {
     const int64_t K = k.rloop.extent;
     const int64_t cols = (N + 63) / 64;
-    int64_t S = std::max<int64_t>(1, std::min<int64_t>((2048 + cols - 1) / cols, K / 64));
+    int64_t S = std::max<int64_t>(1, std::min<int64_t>((2048 + cols - 1) / cols, K / 128));
     const int64_t CH = (K + S - 1) / S;
     S = (K + CH - 1) / CH;
     const std::string TA = ctype(k.acc_dtype);
@@ -2152,6 +2152,7 @@ struct SerialReduce {
       os << "  const idx_t eh_r0 = (idx_t)blockIdx.y * " << CH << ";\n";
       os << "  const idx_t eh_r1 = eh_r0 + " << CH << " < " << K << " ? eh_r0 + " << CH << " : " << K << ";\n";
       os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
+      os << "#pragma unroll 8\n";
       os << "  for (idx_t " << k.rloop.var << " = eh_r0 + ty; " << k.rloop.var << " < eh_r1; " << k.rloop.var << " += 4) {\n";
       os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
       os << "  __shared__ " << TA << " eh_sm[4][64];\n  eh_sm[ty][tx] = acc;\n  __syncthreads();\n";
