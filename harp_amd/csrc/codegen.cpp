@@ -1585,6 +1585,8 @@ struct GroupEmitter {
   bool idx64 = false;
   int V = 1;
   std::map<std::string, int64_t> need;   // elements each bound buffer must hold (max index + 1)
+  // lets a schedule serve some external loads from somewhere else (an LDS tile)
+  std::function<bool(const std::string& buf, const Affine& index, std::string* text)> load_override;
 
   GroupEmitter(const Group& grp, const GenOptions& o) : g(grp), opt(o) {}
 
@@ -1698,6 +1700,7 @@ struct GroupEmitter {
       }
       auto a = affine_of(*load.args[1]);
       if (a) {
+        if (load_override && load_override(b, *a, out)) return true;
         int id = find_ext(b, *a);
         if (id >= 0) {
           std::string t = ld(id);
@@ -1838,6 +1841,117 @@ struct GroupEmitter {
     return ls;
   }
 
+  // ---- transposing copies: a 64 x 64 tile through LDS ---------------------------------------
+  // Elementwise groups in which some operand is contiguous along a row loop while the output is
+  // contiguous along the column loop (permute + contiguous, NCHW <-> NHWC, x^T + y).  Read
+  // as written, such an operand is fetched with a stride between neighbouring work-items.
+  struct TransposedLoad { std::string buf; Affine aff; DType dtype; };
+
+  // every external load of the group, with whether a Select guards it
+  template <class F> void for_each_external_load(F&& f) const {
+    for (const auto& st : g.stages) {
+      std::vector<LoadRef> loads;
+      collect_loads(*st.value, loads);
+      for (const auto& lr : loads) {
+        const std::string& b = lr.load->args[0]->name;
+        bool earlier = false;
+        for (const auto& p : g.stages) {
+          if (&p == &st) break;
+          if (p.out_buf == b) earlier = true;
+        }
+        if (!earlier) f(lr);
+      }
+    }
+  }
+
+  // The row loop the strided operands are contiguous along, or -1 when the group is not of
+  // this form (or too small to bother).
+  int transposed_axis(std::vector<TransposedLoad>* tl) const {
+    if (g.has_reduce() || g.rows.empty() || g.C < 32 || g.R() * g.C < (1 << 16)) return -1;
+    for (const auto& st : g.stages)
+      if (st.store && st.out_aff.of("c") != 1) return -1;
+    int axis = -1;
+    bool ok = true;
+    for_each_external_load([&](const LoadRef& lr) {
+      auto a = affine_of(*lr.load->args[1]);
+      if (!a || lr.load->count != 1) { ok = false; return; }
+      if (a->of("c") == 1 || a->of("c") == 0) return;       // aligned with the output, or a broadcast
+      if (lr.guarded || std::llabs(a->of("c")) < 8) { ok = false; return; }
+      int t = -1;
+      for (size_t i = 0; i < g.rows.size(); ++i)
+        if (a->of("r" + std::to_string(i)) == 1) t = static_cast<int>(i);
+      if (t < 0 || (axis >= 0 && axis != t)) { ok = false; return; }
+      axis = t;
+      for (const auto& e : *tl)
+        if (e.buf == lr.load->args[0]->name && e.aff == *a) return;
+      tl->push_back({lr.load->args[0]->name, *a, lr.load->dtype});
+    });
+    if (!ok || axis < 0 || tl->empty() || tl->size() > 4 || g.rows[static_cast<size_t>(axis)] < 32) return -1;
+    return axis;
+  }
+
+  LaunchSpec emit_transposed(const std::map<std::string, size_t>& elems, int axis, const std::vector<TransposedLoad>& tl) {
+    LaunchSpec ls;
+    const size_t t = static_cast<size_t>(axis);
+    const int64_t Rt = g.rows[t], C = g.C;
+    const int64_t nrt = (Rt + 63) / 64, nct = (C + 63) / 64;
+    int64_t others = 1;
+    for (size_t i = 0; i < g.rows.size(); ++i)
+      if (i != t) others *= g.rows[i];
+    const int64_t blocks = nrt * nct * others;
+    if (blocks >= (int64_t{1} << 31)) throw Error("too many tiles for one launch");
+    const std::string rt = "r" + std::to_string(t);
+    ls.entry = "ehk_" + g.stages.front().kname;
+    ls.schedule = "transpose(tile=64x64,axis=" + std::to_string(axis) + ",operands=" + std::to_string(tl.size()) + ")";
+    ls.grid[0] = static_cast<unsigned>(blocks);
+    ls.block[0] = 256;
+    std::ostringstream os;
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << params_text(&ls.arg_bufs) << ") {\n";
+    for (size_t k = 0; k < tl.size(); ++k)
+      os << "  __shared__ " << ctype(tl[k].dtype) << " eh_tile" << k << "[64][65];\n";
+    os << "  const int eh_tx = threadIdx.x & 63, eh_ty = threadIdx.x >> 6;\n";
+    os << "  idx_t eh_b = blockIdx.x;\n";
+    os << "  const idx_t eh_c0 = (eh_b % " << nct << ") * 64;\n  eh_b /= " << nct << ";\n";
+    os << "  const idx_t eh_r0 = (eh_b % " << nrt << ") * 64;\n  eh_b /= " << nrt << ";\n";
+    for (size_t i = g.rows.size(); i-- > 0;) {
+      if (i == t) continue;
+      os << "  const idx_t r" << i << " = eh_b % " << g.rows[i] << ";\n  eh_b /= " << g.rows[i] << ";\n";
+    }
+    // phase 1: neighbouring work-items walk the operand's contiguous axis
+    os << "  {\n    const idx_t " << rt << " = eh_r0 + eh_tx;\n";
+    os << "#pragma unroll 4\n    for (int eh_cc = eh_ty; eh_cc < 64; eh_cc += 4) {\n      const idx_t c = eh_c0 + eh_cc;\n";
+    os << "      if (" << rt << " < " << Rt << " && c < " << C << ") {\n";
+    for (size_t k = 0; k < tl.size(); ++k)
+      os << "        eh_tile" << k << "[eh_cc][eh_tx] = " << tl[k].buf << "[" << affine_text(tl[k].aff, "c") << "];\n";
+    os << "      }\n    }\n  }\n  __syncthreads();\n";
+    // phase 2: neighbouring work-items walk the output's contiguous axis
+    load_override = [&](const std::string& buf, const Affine& a, std::string* text) {
+      for (size_t k = 0; k < tl.size(); ++k)
+        if (tl[k].buf == buf && tl[k].aff == a) {
+          *text = "eh_tile" + std::to_string(k) + "[eh_tx][eh_rr]";
+          return true;
+        }
+      return false;
+    };
+    auto none = [](int) { return std::string(); };
+    os << "  {\n    const idx_t c = eh_c0 + eh_tx;\n";
+    os << "#pragma unroll 4\n    for (int eh_rr = eh_ty; eh_rr < 64; eh_rr += 4) {\n      const idx_t " << rt << " = eh_r0 + eh_rr;\n";
+    os << "      if (" << rt << " < " << Rt << " && c < " << C << ") {\n";
+    for (const auto& st : g.stages) {
+      if (!st.store) continue;
+      os << "        " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << ctype(st.out_dtype) << ")("
+         << value_text(st, none) << ");\n";
+    }
+    os << "      }\n    }\n  }\n}\n";
+    load_override = nullptr;
+    ls.source = os.str();
+    ls.algo_bytes = algo_bytes(elems);
+    fill_min_bytes(&ls);
+    for (const auto& st : g.stages) ls.kernels.push_back(st.kname);
+    return ls;
+  }
+
   // ---- row program: T threads per row, DPP/LDS reductions ---------------------------------
   LaunchSpec emit_rows(const std::map<std::string, size_t>& elems) {
     LaunchSpec ls;
@@ -1965,7 +2079,11 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
   bool any_store = false;
   for (const auto& st : g.stages) any_store = any_store || st.store;
   if (!any_store) throw Error("fused group starting at '" + g.stages.front().kname + "' produces nothing");
-  if (!g.has_reduce()) return ge.emit_flat(elems);
+  if (!g.has_reduce()) {
+    std::vector<GroupEmitter::TransposedLoad> tl;
+    const int axis = opt.transpose ? ge.transposed_axis(&tl) : -1;
+    return axis >= 0 ? ge.emit_transposed(elems, axis, tl) : ge.emit_flat(elems);
+  }
   return ge.emit_rows(elems);
 }
 

@@ -19,6 +19,7 @@ struct GenOptions {
   std::string arch = "gfx950";
   bool fuse = true;          // merge compatible kernels of a Program into one launch
   bool vectorize = true;     // 128-bit accesses where alignment allows
+  bool transpose = true;     // transposing elementwise groups go through 64x64 LDS tiles
   int row_threads = 0;       // threads cooperating on one row; 0 = choose from the row length
   int row_elems = 8;         // target elements per thread per row when choosing row_threads
   int flat_block = 256;
