@@ -1864,13 +1864,21 @@ struct GroupEmitter {
     }
   }
 
-  // The row loop the strided operands are contiguous along, or -1 when the group is not of
-  // this form (or too small to bother).
-  int transposed_axis(std::vector<TransposedLoad>* tl) const {
-    if (g.has_reduce() || g.rows.empty() || g.C < 32 || g.R() * g.C < (1 << 16)) return -1;
+  // Which loops the tile spans.  `row_run`: adjacent row loops (outermost first) that every
+  // strided operand walks as one contiguous axis; `col_run`: row loops that, followed by the
+  // column loop, every store walks as one contiguous axis.  Empty row_run: not this form.
+  struct TransposePlan {
+    std::vector<size_t> row_run, col_run;
+    int64_t Rt = 1, Ct = 1;
+  };
+
+  TransposePlan transposed_axes(std::vector<TransposedLoad>* tl) const {
+    TransposePlan none;
+    if (g.has_reduce() || g.rows.empty() || g.R() * g.C < (1 << 16)) return none;
     for (const auto& st : g.stages)
-      if (st.store && st.out_aff.of("c") != 1) return -1;
-    int axis = -1;
+      if (st.store && st.out_aff.of("c") != 1) return none;
+    auto rv = [](size_t i) { return "r" + std::to_string(i); };
+    int inner = -1;
     bool ok = true;
     for_each_external_load([&](const LoadRef& lr) {
       auto a = affine_of(*lr.load->args[1]);
@@ -1879,30 +1887,56 @@ struct GroupEmitter {
       if (lr.guarded || std::llabs(a->of("c")) < 8) { ok = false; return; }
       int t = -1;
       for (size_t i = 0; i < g.rows.size(); ++i)
-        if (a->of("r" + std::to_string(i)) == 1) t = static_cast<int>(i);
-      if (t < 0 || (axis >= 0 && axis != t)) { ok = false; return; }
-      axis = t;
+        if (a->of(rv(i)) == 1) t = static_cast<int>(i);
+      if (t < 0 || (inner >= 0 && inner != t)) { ok = false; return; }
+      inner = t;
       for (const auto& e : *tl)
         if (e.buf == lr.load->args[0]->name && e.aff == *a) return;
       tl->push_back({lr.load->args[0]->name, *a, lr.load->dtype});
     });
-    if (!ok || axis < 0 || tl->empty() || tl->size() > 4 || g.rows[static_cast<size_t>(axis)] < 32) return -1;
-    return axis;
+    if (!ok || inner < 0 || tl->empty() || tl->size() > 4) return none;
+    TransposePlan tp;
+    // the column side: c, then the innermost row loops while every store keeps walking on
+    tp.Ct = g.C;
+    for (size_t i = g.rows.size(); i-- > 0;) {
+      if (static_cast<int>(i) == inner) break;
+      bool chains = true;
+      for (const auto& st : g.stages)
+        if (st.store) chains = chains && st.out_aff.of(rv(i)) == tp.Ct;
+      if (!chains) break;
+      tp.col_run.insert(tp.col_run.begin(), i);
+      tp.Ct *= g.rows[i];
+    }
+    // the row side: the operands' unit-stride loop, then the loops outside it while every
+    // strided operand keeps walking on
+    tp.row_run = {static_cast<size_t>(inner)};
+    tp.Rt = g.rows[static_cast<size_t>(inner)];
+    for (size_t i = static_cast<size_t>(inner); i-- > 0;) {
+      bool chains = true;
+      for (const auto& e : *tl) chains = chains && e.aff.of(rv(i)) == tp.Rt;
+      if (!chains) break;
+      tp.row_run.insert(tp.row_run.begin(), i);
+      tp.Rt *= g.rows[i];
+    }
+    if (tp.Rt < 32 || tp.Ct < 32) return none;
+    return tp;
   }
 
-  LaunchSpec emit_transposed(const std::map<std::string, size_t>& elems, int axis, const std::vector<TransposedLoad>& tl) {
+  LaunchSpec emit_transposed(const std::map<std::string, size_t>& elems, const TransposePlan& tp,
+                             const std::vector<TransposedLoad>& tl) {
     LaunchSpec ls;
-    const size_t t = static_cast<size_t>(axis);
-    const int64_t Rt = g.rows[t], C = g.C;
-    const int64_t nrt = (Rt + 63) / 64, nct = (C + 63) / 64;
+    const int64_t nrt = (tp.Rt + 63) / 64, nct = (tp.Ct + 63) / 64;
+    std::vector<bool> in_tile(g.rows.size(), false);
+    for (size_t i : tp.row_run) in_tile[i] = true;
+    for (size_t i : tp.col_run) in_tile[i] = true;
     int64_t others = 1;
     for (size_t i = 0; i < g.rows.size(); ++i)
-      if (i != t) others *= g.rows[i];
+      if (!in_tile[i]) others *= g.rows[i];
     const int64_t blocks = nrt * nct * others;
     if (blocks >= (int64_t{1} << 31)) throw Error("too many tiles for one launch");
-    const std::string rt = "r" + std::to_string(t);
     ls.entry = "ehk_" + g.stages.front().kname;
-    ls.schedule = "transpose(tile=64x64,axis=" + std::to_string(axis) + ",operands=" + std::to_string(tl.size()) + ")";
+    ls.schedule = "transpose(tile=64x64,rows=" + std::to_string(tp.Rt) + ",cols=" + std::to_string(tp.Ct) +
+                  ",operands=" + std::to_string(tl.size()) + ")";
     ls.grid[0] = static_cast<unsigned>(blocks);
     ls.block[0] = 256;
     std::ostringstream os;
@@ -1915,13 +1949,40 @@ struct GroupEmitter {
     os << "  const idx_t eh_c0 = (eh_b % " << nct << ") * 64;\n  eh_b /= " << nct << ";\n";
     os << "  const idx_t eh_r0 = (eh_b % " << nrt << ") * 64;\n  eh_b /= " << nrt << ";\n";
     for (size_t i = g.rows.size(); i-- > 0;) {
-      if (i == t) continue;
+      if (in_tile[i]) continue;
       os << "  const idx_t r" << i << " = eh_b % " << g.rows[i] << ";\n  eh_b /= " << g.rows[i] << ";\n";
     }
-    // phase 1: neighbouring work-items walk the operand's contiguous axis
-    os << "  {\n    const idx_t " << rt << " = eh_r0 + eh_tx;\n";
-    os << "#pragma unroll 4\n    for (int eh_cc = eh_ty; eh_cc < 64; eh_cc += 4) {\n      const idx_t c = eh_c0 + eh_cc;\n";
-    os << "      if (" << rt << " < " << Rt << " && c < " << C << ") {\n";
+    // position along the merged row axis -> its loops; along the merged column axis -> its loops and c
+    auto decode_rows = [&](const std::string& m, const std::string& ind) {
+      std::string t = ind + "idx_t eh_q = " + m + ";\n";
+      for (size_t q = tp.row_run.size(); q-- > 0;) {
+        const size_t i = tp.row_run[q];
+        if (q == 0) t += ind + "const idx_t r" + std::to_string(i) + " = eh_q;\n";
+        else {
+          t += ind + "const idx_t r" + std::to_string(i) + " = eh_q % " + std::to_string(g.rows[i]) + ";\n";
+          t += ind + "eh_q /= " + std::to_string(g.rows[i]) + ";\n";
+        }
+      }
+      return t;
+    };
+    auto decode_cols = [&](const std::string& m, const std::string& ind) {
+      std::string t = ind + "idx_t eh_p = " + m + ";\n";
+      if (tp.col_run.empty()) return t + ind + "const idx_t c = eh_p;\n";
+      t += ind + "const idx_t c = eh_p % " + std::to_string(g.C) + ";\n" + ind + "eh_p /= " + std::to_string(g.C) + ";\n";
+      for (size_t q = tp.col_run.size(); q-- > 0;) {
+        const size_t i = tp.col_run[q];
+        if (q == 0) t += ind + "const idx_t r" + std::to_string(i) + " = eh_p;\n";
+        else {
+          t += ind + "const idx_t r" + std::to_string(i) + " = eh_p % " + std::to_string(g.rows[i]) + ";\n";
+          t += ind + "eh_p /= " + std::to_string(g.rows[i]) + ";\n";
+        }
+      }
+      return t;
+    };
+    // phase 1: neighbouring work-items walk the operands' contiguous axis
+    os << "  if (eh_r0 + eh_tx < " << tp.Rt << ") {\n" << decode_rows("eh_r0 + eh_tx", "    ");
+    os << "#pragma unroll 4\n    for (int eh_cc = eh_ty; eh_cc < 64; eh_cc += 4) {\n";
+    os << "      if (eh_c0 + eh_cc < " << tp.Ct << ") {\n" << decode_cols("eh_c0 + eh_cc", "        ");
     for (size_t k = 0; k < tl.size(); ++k)
       os << "        eh_tile" << k << "[eh_cc][eh_tx] = " << tl[k].buf << "[" << affine_text(tl[k].aff, "c") << "];\n";
     os << "      }\n    }\n  }\n  __syncthreads();\n";
@@ -1935,9 +1996,9 @@ struct GroupEmitter {
       return false;
     };
     auto none = [](int) { return std::string(); };
-    os << "  {\n    const idx_t c = eh_c0 + eh_tx;\n";
-    os << "#pragma unroll 4\n    for (int eh_rr = eh_ty; eh_rr < 64; eh_rr += 4) {\n      const idx_t " << rt << " = eh_r0 + eh_rr;\n";
-    os << "      if (" << rt << " < " << Rt << " && c < " << C << ") {\n";
+    os << "  if (eh_c0 + eh_tx < " << tp.Ct << ") {\n" << decode_cols("eh_c0 + eh_tx", "    ");
+    os << "#pragma unroll 4\n    for (int eh_rr = eh_ty; eh_rr < 64; eh_rr += 4) {\n";
+    os << "      if (eh_r0 + eh_rr < " << tp.Rt << ") {\n" << decode_rows("eh_r0 + eh_rr", "        ");
     for (const auto& st : g.stages) {
       if (!st.store) continue;
       os << "        " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << ctype(st.out_dtype) << ")("
@@ -2081,8 +2142,9 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
   if (!any_store) throw Error("fused group starting at '" + g.stages.front().kname + "' produces nothing");
   if (!g.has_reduce()) {
     std::vector<GroupEmitter::TransposedLoad> tl;
-    const int axis = opt.transpose ? ge.transposed_axis(&tl) : -1;
-    return axis >= 0 ? ge.emit_transposed(elems, axis, tl) : ge.emit_flat(elems);
+    GroupEmitter::TransposePlan tp;
+    if (opt.transpose) tp = ge.transposed_axes(&tl);
+    return tp.row_run.empty() ? ge.emit_flat(elems) : ge.emit_transposed(elems, tp, tl);
   }
   return ge.emit_rows(elems);
 }

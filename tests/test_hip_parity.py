@@ -511,6 +511,9 @@ TRANSPOSING = {
     "swap_last_two_of_three": ((9, 130, 70), lambda t: t.permute([0, 2, 1]).contiguous()),
     "transpose_plus_aligned": ((257, 257), lambda t: (t.permute([1, 0]) + t) * t),
     "rotate_three_axes": ((40, 64, 96), lambda t: t.permute([2, 0, 1]).contiguous()),
+    # the contiguous axes are pairs of loops here: (h, w) of the operand, (h, w) of the output
+    "nchw_to_nhwc": ((9, 40, 14, 14), lambda t: t.permute([0, 2, 3, 1]).contiguous()),
+    "nhwc_to_nchw_relu": ((9, 14, 14, 40), lambda t: t.permute([0, 3, 1, 2]).maximum(t.permute([0, 3, 1, 2]) * t.permute([0, 3, 1, 2]))),
 }
 
 
