@@ -369,7 +369,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             "workload": "CNN 1x28x28: conv3x3(32)+relu+pool, conv3x3(64)+relu+pool, fc 3136-128-10, "
                         "cross-entropy; batch 256 forward + exact backward, plus the SGD update (more than the "
                         "configuration asks for, inside the timed region), one Program"}
-    result_extra["device"] = {"name": props["name"], "arch": props["arch"],
+    result_extra["device"] = {"name": props["name"] or "MI355X (name not reported by the runtime)", "arch": props["arch"],
                               "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
     out["extra"] = result_extra
     print(json.dumps(out), flush=True)
