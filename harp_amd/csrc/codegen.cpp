@@ -1040,6 +1040,136 @@ std::optional<Affine> relayout(const NestKernel& g, const NestKernel& sk, const 
   return out;
 }
 
+// ---------------------------------------------------------------------------------------------
+// few, very long reduce lines: split over workgroups before planning
+// ---------------------------------------------------------------------------------------------
+
+namespace {
+
+NodePtr make_range(const std::string& var, int64_t extent, NodePtr body) {
+  auto r = make(Op::Range, {make_i64(0), make_i64(1), make_i64(extent), std::move(body)});
+  r->name = var;
+  r->parallel = "sequential";
+  return r;
+}
+
+NodePtr make_combine(ReduceKind k, const NodePtr& acc, const NodePtr& v) {
+  switch (k) {
+    case ReduceKind::Sum: return make(Op::Add, {acc, v});
+    case ReduceKind::Prod: return make(Op::Mul, {acc, v});
+    case ReduceKind::Max: return make(Op::Max, {acc, v});
+    default: return make(Op::Select, {make(Op::Lt, {acc, v}), acc, v});     // min, as node.rs:63-77 writes it
+  }
+}
+
+NodePtr make_kernel(const std::string& name, std::vector<Param> params, NodePtr body) {
+  auto k = std::make_shared<Node>(Op::Kernel);
+  k->name = name;
+  k->params = std::move(params);
+  k->args = {std::move(body)};
+  for (int i = 0; i < 3; ++i) {
+    k->grid.push_back(make_i64(1));
+    k->tg.push_back(make_i64(1));
+  }
+  return k;
+}
+
+// acc = identity; for var in [0, extent): acc = combine(acc, value); out[index] = acc
+NodePtr make_reduce_block(const NestKernel& nk, const std::string& var, int64_t extent, const NodePtr& value,
+                          const std::string& out_buf, const NodePtr& out_index) {
+  auto acc = make_var("acc");
+  auto init = make(Op::Assign, {nk.identity});
+  init->name = "acc";
+  auto step = make(Op::Assign, {make_combine(nk.rkind, acc, value)});
+  step->name = "acc";
+  auto store = make(Op::Store, {make_var(out_buf), out_index, acc});
+  auto blk = make(Op::Block, {init, make_range(var, extent, step), store});
+  blk->decls.push_back({"acc", nk.acc_dtype});
+  return blk;
+}
+
+struct RowSplit {
+  NodePtr part, final_;      // the two kernels that replace the original
+  BufferInfo scratch;        // [lines * chunks] partial results
+};
+
+// A reduce whose lines are few and very long (a total over a whole tensor, a softmax over two
+// rows of millions) would occupy a handful of workgroups.  Rewritten as two reduces -- every
+// line cut into `chunks` pieces, then the pieces of a line combined -- both take the ordinary
+// row schedule, the first with lines * chunks rows.  The combine order changes (reduction
+// tolerance for sums and products, exact for max and min).
+std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
+  if (nk.rkind == ReduceKind::None || !nk.out_aff) return std::nullopt;
+  int64_t lines = 1;
+  for (const auto& l : nk.loops) lines *= l.extent;
+  const int64_t K = nk.rloop.extent;
+  if (lines > 16 || K < (int64_t{1} << 21)) return std::nullopt;
+  std::vector<LoadRef> loads;
+  collect_loads(*nk.value, loads);
+  bool unit = false;
+  for (const auto& lr : loads) {
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a || lr.load->args[0]->op != Op::Var) return std::nullopt;
+    const int64_t c = a->of(nk.rloop.var);
+    if (c != 0 && c != 1) return std::nullopt;
+    unit = unit || c == 1;
+  }
+  if (!unit) return std::nullopt;
+  int64_t chunks = 0;
+  for (int64_t align : {4, 1}) {           // chunks that start on a 16-byte boundary first
+    for (int64_t s = 4096 / lines; s >= 8 && !chunks; --s)
+      if (K % (s * align) == 0 && K / s >= 4096) chunks = s;
+  }
+  if (!chunks) return std::nullopt;
+  const int64_t CH = K / chunks;
+  RowSplit rs;
+  rs.scratch.name = "eh_rowpart_" + nk.name;
+  rs.scratch.dtype = nk.acc_dtype;
+  rs.scratch.shape = {lines * chunks};
+  rs.scratch.role = "temp";
+  // position of a line among the lines (row-major over the outer loops)
+  NodePtr line = make_i64(0);
+  for (const auto& l : nk.loops) line = make(Op::Add, {make(Op::Mul, {line, make_i64(l.extent)}), make_var(l.var)});
+  const std::string sv = "eh_chunk", kv = "eh_k";
+  auto part_index = make(Op::Add, {make(Op::Mul, {line, make_i64(chunks)}), make_var(sv)});
+  DType pt;
+  pt.ty = Ty::Ptr;
+  pt.inner = std::make_shared<DType>(nk.acc_dtype);
+  {
+    // value with the reduce variable replaced by chunk * CH + k
+    NodePtr pos = make(Op::Add, {make(Op::Mul, {make_var(sv), make_i64(CH)}), make_var(kv)});
+    NodePtr value = rename(nk.value, {{nk.rloop.var, pos}});
+    NodePtr body = make_range(sv, chunks, make_reduce_block(nk, kv, CH, value, rs.scratch.name, part_index));
+    for (size_t i = nk.loops.size(); i-- > 0;) body = make_range(nk.loops[i].var, nk.loops[i].extent, body);
+    std::vector<Param> params;
+    for (const auto& p : nk.params)
+      if (!p.mut_) params.push_back(p);
+    Param sp;
+    sp.name = rs.scratch.name;
+    sp.dtype = pt;
+    sp.mut_ = true;
+    params.push_back(sp);
+    rs.part = make_kernel(nk.name + "_rows", params, body);
+  }
+  {
+    auto ld = make(Op::Load, {make_var(rs.scratch.name), part_index});
+    ld->dtype = nk.acc_dtype;
+    NodePtr body = make_reduce_block(nk, sv, chunks, ld, nk.out_buf, nk.out_index);
+    for (size_t i = nk.loops.size(); i-- > 0;) body = make_range(nk.loops[i].var, nk.loops[i].extent, body);
+    std::vector<Param> params;
+    Param sp;
+    sp.name = rs.scratch.name;
+    sp.dtype = pt;
+    params.push_back(sp);
+    for (const auto& p : nk.params)
+      if (p.mut_) params.push_back(p);
+    rs.final_ = make_kernel(nk.name, params, body);
+  }
+  return rs;
+}
+
+}  // namespace
+
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
   ProgramPlan plan;
@@ -1052,6 +1182,21 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
 
   // buffer table: given, or synthesised from the kernels' pointer parameters
   plan.buffers = program.buffers;
+  std::vector<NodePtr> rewritten;          // owns the kernels that replace split ones
+  if (!plan.buffers.empty() && opt.fuse) {
+    std::vector<const Node*> out;
+    for (const Node* k : kernels) {
+      auto nk = extract_nest(*k);
+      auto rs = nk ? split_long_rows(*nk) : std::nullopt;
+      if (!rs) { out.push_back(k); continue; }
+      rewritten.push_back(rs->part);
+      rewritten.push_back(rs->final_);
+      out.push_back(rs->part.get());
+      out.push_back(rs->final_.get());
+      plan.buffers.push_back(rs->scratch);
+    }
+    kernels = out;
+  }
   std::map<std::string, size_t> elems;
   bool have_table = !plan.buffers.empty();
   if (have_table) {

@@ -959,6 +959,50 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
         assert bits_equal_mod_zero(ref, got)
 
 
+LONG_LINES = {
+    # name: (shape, graph, float64 statement of the same, entry of the kernel that cuts the lines)
+    "sum_4x10M": ((4, 10_000_000), lambda t: t.sum(1), lambda x: x.sum(1), "row"),
+    "sum_all_16M": ((1 << 24,), lambda t: t.sum(0), lambda x: x.sum(0, keepdims=True), "row"),
+    "max_2x4M": ((2, 1 << 22), lambda t: t.max(1), lambda x: x.max(1), "row"),
+    "min_3x2x2M": ((3, 2, 1 << 21), lambda t: t.min(2), lambda x: x.min(2), "row"),
+    "mean_sq_2x3M": ((2, 3 << 20), lambda t: (t * t).sum(1), lambda x: (x * x).sum(1), "row"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LONG_LINES))
+def test_few_very_long_reduce_lines_are_cut_over_workgroups(frontend, hip, name):
+    """A reduce with a handful of lines of millions of elements is planned as two reduces (pieces
+    of a line, then the pieces): max and min stay bit-exact with the oracle; a sum is held to
+    the reduction tolerance against float64, since the oracle's own sequential float32 sum of
+    10^7 terms is only good to about 1e-4."""
+    from harp_amd import workloads as wl
+    shape, fn, exact_fn, sched = LONG_LINES[name]
+    launches = hip.render_program(wl.lower_with_table([shape], fn)[0]).launches
+    cut = [l for l in launches if l["entry"].endswith("_rows")]
+    assert len(cut) == 1 and cut[0]["schedule"].startswith(sched) and cut[0]["grid"][0] >= 128, launches
+    x = RNG(len(name)).uniform(-1.0, 1.5, shape).astype(np.float32)
+    ref, got = both(frontend, fn, [x], True)
+    if name.startswith(("max", "min")):
+        assert bits_equal_mod_zero(ref, got)
+        return
+    x64 = x.astype(np.float64)
+    exact, scale = exact_fn(x64).ravel(), exact_fn(np.abs(x64)).ravel()
+    assert np.all(np.abs(got.ravel() - exact) <= 1e-5 * scale)
+    assert np.all(np.abs(ref.ravel() - exact) <= 1e-3 * scale)
+
+
+def test_softmax_over_two_rows_of_millions(frontend, hip):
+    """Row softmax whose rows are too long for one workgroup each: every reduce in it is cut."""
+    shape = (2, 1 << 22)
+    x = RNG(77).uniform(-3, 3, shape).astype(np.float32)
+    fn = lambda t: frontend.nn.softmax(t, 1)
+    ref, got = both(frontend, fn, [x], True)
+    e = np.exp(x.astype(np.float64) - x.max(1, keepdims=True))
+    exact = e / e.sum(1, keepdims=True)
+    assert np.allclose(got.reshape(shape), exact, rtol=1e-5, atol=0)
+    assert np.allclose(ref.reshape(shape), exact, rtol=1e-3, atol=0)
+
+
 @pytest.mark.parametrize("seed", range(64))
 def test_random_graphs_match_the_oracle(frontend, hip, seed):
     """Differential test on seeded random graphs (tests/graph_fuzz.py): elementwise chains,

@@ -342,6 +342,30 @@ def test_config4_training_step_plan(frontend):
         assert len(hb.compile_source(src)) > 1000
 
 
+def test_few_very_long_reduce_lines_are_planned_as_two_reduces(frontend):
+    """Four lines of ten million elements: the plan cuts every line into pieces that start on
+    a 16-byte boundary (one workgroup each), adds the scratch buffer for the pieces and then
+    reduces those; without the buffer table (nowhere to put the scratch) or with fusion off
+    the kernel stays whole, and lines of ordinary length are never cut."""
+    from harp_amd import backend as hb, workloads as wl
+    ast = wl.lower_with_table([(4, 10_000_000)], lambda t: t.sum(1))[0]
+    plan = hb.render_program(ast)
+    assert [l["entry"][-5:] for l in plan.launches][0] == "_rows" and len(plan.launches) == 2
+    part, final = plan.launches
+    assert part["schedule"].startswith("row(") and part["grid"][0] == 4000 and ",V=4," in part["schedule"]
+    scratch = [b for b in plan.buffers if b["name"].startswith("eh_rowpart_")]
+    assert len(scratch) == 1 and scratch[0]["bytes"] == 4 * 4000 and scratch[0]["role"] == "temp"
+    assert scratch[0]["name"] in part["args"] and scratch[0]["name"] in final["args"]
+    for src in (part["source"], final["source"]):
+        assert len(hb.compile_source(src)) > 1000
+    assert len(hb.render_program(ast, {"fuse": False}).launches) == 1
+    t = frontend.Tensor.input([4, 10_000_000])
+    bare = frontend.lower_graph([t.sum(1).graph])[0]
+    assert len(hb.render_program(bare).launches) == 1
+    short = wl.lower_with_table([(4, 1 << 20)], lambda t: t.sum(1))[0]
+    assert len(hb.render_program(short).launches) == 1
+
+
 def test_option_beam_search_on_a_synthetic_cost():
     """The schedule search without a device: suggesters propose neighbours by the schedules in
     the plan, the beam keeps the cheapest states, the search stops when nothing improves."""
