@@ -514,7 +514,8 @@ bool injective(const Affine& a, const std::vector<Loop>& vars) {
 // make that safe, and only the order of the additions is left open.  A nest that does not
 // qualify runs as written in one work-item.  Empty result: the kernel has a form this
 // does not cover (shape variables, hand-placed group/local ids, shared memory).
-std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOptions& opt) {
+std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOptions& opt,
+                                                     std::vector<BufferInfo>* extra_buffers) {
   std::vector<LaunchSpec> out;
   if (k.op != Op::Kernel) return out;
   for (const auto& p : k.params)
@@ -629,12 +630,6 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       const std::string ident = literal(*scan->identity);
       ExprRenderer er;
       auto comb = [&](const std::string& a, const std::string& b) { return combine_text(scan->kind, scan->acc_dtype, a, b); };
-      os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << sig << ") {\n";
-      os << "  long long eh_r = blockIdx.x;\n";
-      for (size_t i = loops.size(); i-- > 0;) {
-        os << "  const long long " << loops[i].var << " = eh_r % " << loops[i].extent << ";\n";
-        if (i) os << "  eh_r /= " << loops[i].extent << ";\n";
-      }
       // 128-bit accesses when the line is one loop walked with unit stride by every load and by
       // the store, everything 16-byte aligned, four-byte elements
       bool vec = scan->loops.size() == 1 && scan->length % 4 == 0 && scan->acc_dtype.itemsize() == 4;
@@ -652,44 +647,130 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
         vec = vec && !lr.guarded && lr.load->count == 1 && lr.load->dtype.itemsize() == 4 &&
               lr.load->args[0]->op == Op::Var && unit_aligned(*lr.load->args[1]);
       vec = vec && scan->out_ptr->op == Op::Var && unit_aligned(*scan->out_index);
-      os << "  __shared__ " << T << " eh_wave_total[4];\n";
-      os << "  const int eh_lane = threadIdx.x & 63, eh_wave = threadIdx.x >> 6;\n";
-      os << "  " << T << " eh_carry = " << ident << ";\n";
-      os << "  for (long long eh_t0 = 0; eh_t0 < " << scan->length << "ll; eh_t0 += 1024) {\n";
-      os << "    " << T << " eh_v[4];\n";
-      if (vec) {
-        os << "    const long long eh_tb = eh_t0 + threadIdx.x * 4;\n    const bool eh_in = eh_tb < " << scan->length << "ll;\n";
-        os << "    {\n      const long long " << sv << " = eh_in ? eh_tb : 0;\n";
-        std::vector<std::string> seen;
-        for (const auto& lr : sloads) {
-          const std::string key = to_text(*lr.load);
-          if (std::find(seen.begin(), seen.end(), key) != seen.end()) continue;
-          os << "      const EhV4<" << ctype(lr.load->dtype) << "> eh_ld" << seen.size() << " = eh_load4<false>("
-             << lr.load->args[0]->name << " + " << er.expr(*lr.load->args[1]) << ");\n";
-          seen.push_back(key);
-        }
-        ExprRenderer ev;
-        ev.load_hook = [&](const Node& ld, std::string* out) {
-          const std::string key = to_text(ld);
-          for (size_t q = 0; q < seen.size(); ++q)
-            if (seen[q] == key) { *out = "eh_ld" + std::to_string(q) + "[eh_e]"; return true; }
-          return false;
-        };
-        os << "#pragma unroll\n      for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
-        os << "        eh_v[eh_e] = eh_in ? (" << T << ")(" << ev.expr(*scan->value) << ") : " << ident << ";\n";
-        os << "        if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n      }\n    }\n";
-      } else {
-        os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
-        os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
-        os << "      eh_v[eh_e] = " << ident << ";\n";
-        os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
-        for (size_t i = scan->loops.size(); i-- > 0;) {
-          os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
-          if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
-        }
-        os << "        eh_v[eh_e] = (" << T << ")(" << er.expr(*scan->value) << ");\n      }\n";
-        os << "      if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n    }\n";
+      // A handful of very long lines (a scan over axis 0 is lowered as one line over the whole
+      // tensor) would occupy a handful of workgroups: cut every line into chunks of whole
+      // tiles, total each chunk in a first launch, and let the workgroup that scans a chunk
+      // start from the combined totals of the chunks ahead of it.
+      int64_t chunks = 1, chunk_len = scan->length;
+      if (extra_buffers && lines <= 16 && scan->length >= (int64_t{1} << 19)) {
+        const int64_t want = 2048 / lines;
+        chunk_len = std::max<int64_t>(4096, ((scan->length + want - 1) / want + 1023) / 1024 * 1024);
+        chunks = (scan->length + chunk_len - 1) / chunk_len;
       }
+      const std::string scratch = "eh_scanpart_" + k.name + "_n" + std::to_string(t);
+      // the four values of this thread in the tile at eh_t0, each combined with the ones before
+      // it in the thread: eh_v[3] is the thread's total
+      auto emit_tile_values = [&](std::ostringstream& os) {
+        os << "    " << T << " eh_v[4];\n";
+        if (vec) {
+          os << "    const long long eh_tb = eh_t0 + threadIdx.x * 4;\n    const bool eh_in = eh_tb < " << scan->length << "ll;\n";
+          os << "    {\n      const long long " << sv << " = eh_in ? eh_tb : 0;\n";
+          std::vector<std::string> seen;
+          for (const auto& lr : sloads) {
+            const std::string key = to_text(*lr.load);
+            if (std::find(seen.begin(), seen.end(), key) != seen.end()) continue;
+            os << "      const EhV4<" << ctype(lr.load->dtype) << "> eh_ld" << seen.size() << " = eh_load4<false>("
+               << lr.load->args[0]->name << " + " << er.expr(*lr.load->args[1]) << ");\n";
+            seen.push_back(key);
+          }
+          ExprRenderer ev;
+          ev.load_hook = [&](const Node& ld, std::string* out) {
+            const std::string key = to_text(ld);
+            for (size_t q = 0; q < seen.size(); ++q)
+              if (seen[q] == key) { *out = "eh_ld" + std::to_string(q) + "[eh_e]"; return true; }
+            return false;
+          };
+          os << "#pragma unroll\n      for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+          os << "        eh_v[eh_e] = eh_in ? (" << T << ")(" << ev.expr(*scan->value) << ") : " << ident << ";\n";
+          os << "        if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n      }\n    }\n";
+        } else {
+          os << "#pragma unroll\n    for (int eh_e = 0; eh_e < 4; ++eh_e) {\n";
+          os << "      const long long eh_t = eh_t0 + threadIdx.x * 4 + eh_e;\n";
+          os << "      eh_v[eh_e] = " << ident << ";\n";
+          os << "      if (eh_t < " << scan->length << "ll) {\n        long long eh_q = eh_t;\n";
+          for (size_t i = scan->loops.size(); i-- > 0;) {
+            os << "        const long long " << scan->loops[i].var << " = eh_q % " << scan->loops[i].extent << ";\n";
+            if (i) os << "        eh_q /= " << scan->loops[i].extent << ";\n";
+          }
+          os << "        eh_v[eh_e] = (" << T << ")(" << er.expr(*scan->value) << ");\n      }\n";
+          os << "      if (eh_e) eh_v[eh_e] = " << comb("eh_v[eh_e - 1]", "eh_v[eh_e]") << ";\n    }\n";
+        }
+      };
+      // entry, line variables, lane ids; with chunks also eh_chunk and the tile range of the chunk
+      auto emit_head = [&](std::ostringstream& os, const std::string& entry, const std::string& params) {
+        os << "extern \"C\" __global__ void __launch_bounds__(256) " << entry << "(" << params << ") {\n";
+        if (chunks > 1) {
+          os << "  const long long eh_chunk = blockIdx.x % " << chunks << ", eh_line = blockIdx.x / " << chunks << ";\n";
+          os << "  long long eh_r = eh_line;\n";
+          os << "  const long long eh_first = eh_chunk * " << chunk_len << "ll;\n";
+          os << "  const long long eh_last = eh_first + " << chunk_len << "ll < " << scan->length << "ll ? eh_first + "
+             << chunk_len << "ll : " << scan->length << "ll;\n";
+        } else {
+          os << "  long long eh_r = blockIdx.x;\n";
+          os << "  const long long eh_first = 0, eh_last = " << scan->length << "ll;\n";
+        }
+        for (size_t i = loops.size(); i-- > 0;) {
+          os << "  const long long " << loops[i].var << " = eh_r % " << loops[i].extent << ";\n";
+          if (i) os << "  eh_r /= " << loops[i].extent << ";\n";
+        }
+        os << "  __shared__ " << T << " eh_wave_total[4];\n";
+        os << "  const int eh_lane = threadIdx.x & 63, eh_wave = threadIdx.x >> 6;\n";
+      };
+      // eh_p of every thread combined over the workgroup into `dst` (same value in every thread)
+      auto emit_block_combine = [&](std::ostringstream& os, const std::string& dst) {
+        os << "#pragma unroll\n  for (int eh_d = 32; eh_d > 0; eh_d >>= 1) eh_p = " << comb("eh_p", "__shfl_xor(eh_p, eh_d, 64)") << ";\n";
+        os << "  if (eh_lane == 0) eh_wave_total[eh_wave] = eh_p;\n  __syncthreads();\n";
+        os << "  for (int eh_w = 0; eh_w < 4; ++eh_w) " << dst << " = " << comb(dst, "eh_wave_total[eh_w]") << ";\n";
+        os << "  __syncthreads();\n";
+      };
+      if (chunks > 1) {
+        // first launch: the total of every chunk
+        LaunchSpec lt;
+        lt.entry = ls.entry + "_tot";
+        lt.kernels = {k.name};
+        std::string tsig;
+        for (const auto& p : k.params) {
+          if (p.mut_) continue;
+          tsig += (tsig.empty() ? "" : ", ") + std::string("const ") + ctype(p.dtype.elem()) + "* __restrict__ " + p.name;
+          lt.arg_bufs.push_back(p.name);
+        }
+        tsig += (tsig.empty() ? "" : ", ") + T + "* __restrict__ " + scratch;
+        lt.arg_bufs.push_back(scratch);
+        std::ostringstream ot;
+        ot << hdr(opt);
+        emit_head(ot, lt.entry, tsig);
+        ot << "  " << T << " eh_p = " << ident << ";\n";
+        ot << "  for (long long eh_t0 = eh_first; eh_t0 < eh_last; eh_t0 += 1024) {\n";
+        emit_tile_values(ot);
+        ot << "    eh_p = " << comb("eh_p", "eh_v[3]") << ";\n  }\n";
+        ot << "  " << T << " eh_total = " << ident << ";\n";
+        emit_block_combine(ot, "eh_total");
+        ot << "  if (threadIdx.x == 0) " << scratch << "[blockIdx.x] = eh_total;\n}\n";
+        lt.source = ot.str();
+        lt.grid[0] = static_cast<unsigned>(lines * chunks);
+        lt.block[0] = 256;
+        lt.schedule = "scan-row-totals(lines=" + std::to_string(lines) + ",chunks=" + std::to_string(chunks) + ")";
+        out.push_back(std::move(lt));
+        BufferInfo sb;
+        sb.name = scratch;
+        sb.dtype = scan->acc_dtype;
+        sb.shape = {lines * chunks};
+        sb.role = "temp";
+        extra_buffers->push_back(sb);
+        ls.arg_bufs.push_back(scratch);
+      }
+      emit_head(os, ls.entry, chunks > 1 ? sig + ", const " + T + "* __restrict__ " + scratch : sig);
+      os << "  " << T << " eh_carry = " << ident << ";\n";
+      if (chunks > 1) {
+        // everything ahead of this chunk in its line
+        os << "  {\n  " << T << " eh_p = " << ident << ";\n";
+        os << "  for (long long eh_q = threadIdx.x; eh_q < eh_chunk; eh_q += 256) eh_p = "
+           << comb("eh_p", scratch + "[eh_line * " + std::to_string(chunks) + " + eh_q]") << ";\n";
+        emit_block_combine(os, "eh_carry");
+        os << "  }\n";
+      }
+      os << "  for (long long eh_t0 = eh_first; eh_t0 < eh_last; eh_t0 += 1024) {\n";
+      emit_tile_values(os);
       // inclusive scan of the thread totals across the wave, then across the four waves
       os << "    " << T << " eh_inc = eh_v[3];\n";
       os << "#pragma unroll\n    for (int eh_d = 1; eh_d < 64; eh_d <<= 1) {\n";
@@ -718,9 +799,10 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
         os << "        " << er.expr(*scan->out_ptr) << "[" << er.expr(*scan->out_index) << "] = " << comb("eh_before", "eh_v[eh_e]") << ";\n      }\n    }\n";
       }
       os << "    __syncthreads();\n  }\n}\n";
-      ls.grid[0] = static_cast<unsigned>(lines);
+      ls.grid[0] = static_cast<unsigned>(lines * chunks);
       ls.block[0] = 256;
-      ls.schedule = "scan-row(lines=" + std::to_string(lines) + ",length=" + std::to_string(scan->length) + ")";
+      ls.schedule = "scan-row(lines=" + std::to_string(lines) + ",length=" + std::to_string(scan->length) +
+                    (chunks > 1 ? ",chunks=" + std::to_string(chunks) : "") + ")";
       any_parallel = true;
     } else if (spread) {
       int64_t total = 1;
@@ -1402,7 +1484,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       continue;
     }
     if (!nests[i]) {
-      auto spread = render_kernel_outer_parallel(*kernels[i], opt);
+      auto spread = render_kernel_outer_parallel(*kernels[i], opt, have_table && opt.fuse ? &plan.buffers : nullptr);
       if (spread.empty()) plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
       else for (auto& ls : spread) plan.launches.push_back(std::move(ls));
       ++i;

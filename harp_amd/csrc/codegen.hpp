@@ -66,7 +66,10 @@ LaunchSpec render_kernel_as_written(const Node& kernel, const GenOptions& opt);
 
 // One launch per top-level loop nest of such a kernel, the outer loops of a nest spread over
 // work-items where their iterations cannot collide; empty when the kernel's form is not covered.
-std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& kernel, const GenOptions& opt);
+// `extra_buffers`: where a schedule that needs a scratch buffer may declare it (the Program's
+// buffer table); null when the caller has no table, and such schedules are then not used.
+std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& kernel, const GenOptions& opt,
+                                                     std::vector<BufferInfo>* extra_buffers = nullptr);
 
 // Expression text in HIP C (math calls, literals); exposed for tests.
 std::string render_expr_text(const Node& e);

@@ -991,6 +991,46 @@ def test_few_very_long_reduce_lines_are_cut_over_workgroups(frontend, hip, name)
     assert np.all(np.abs(ref.ravel() - exact) <= 1e-3 * scale)
 
 
+LONG_SCANS = {
+    # name: (shape, graph, float64 statement, schedule of the scanning launch)
+    "cummax_axis0": ((2048, 512), lambda t: t.cummax(0), None, "scan-row(lines=1,length=1048576,chunks=256)"),
+    "cumsum_ragged": ((3, 700001), lambda t: t.cumsum(1), lambda x: np.cumsum(x, 1), "scan-row(lines=3,length=700001,chunks=171)"),
+    "cumsum_2x1M": ((2, 1 << 20), lambda t: (t * t).cumsum(1), lambda x: np.cumsum(x * x, 1), "scan-row(lines=2,length=1048576,chunks=256)"),
+    "cumprod_1x600k": ((1, 600_000), lambda t: t.cumprod(1), lambda x: np.cumprod(x, 1), "scan-row(lines=1,length=600000,chunks=147)"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LONG_SCANS))
+def test_few_very_long_scan_lines_are_cut_over_workgroups(frontend, hip, name):
+    """A prefix scan with a handful of lines of a million elements: a first launch totals chunks
+    of whole tiles, the scanning launch starts every chunk from the totals ahead of it.  Max is
+    bit-exact with the oracle; sums and products are held to the reduction tolerance against
+    float64 (the oracle's sequential float32 scan over 10^6 terms is itself only good to about 1e-4)."""
+    from harp_amd import workloads as wl
+    shape, fn, exact_fn, sched = LONG_SCANS[name]
+    launches = hip.render_program(wl.lower_with_table([shape], fn)[0]).launches
+    scheds = [l["schedule"] for l in launches]
+    assert sched in scheds and any(s.startswith("scan-row-totals(") for s in scheds), scheds
+    x = RNG(len(name)).uniform(-1.0, 1.5, shape).astype(np.float32)
+    if name.startswith("cumprod"):
+        x = np.exp(RNG(len(name)).uniform(-0.05, 0.05, shape)).astype(np.float32)
+    ref, got = both(frontend, fn, [x], True)
+    if exact_fn is None:
+        assert bits_equal_mod_zero(ref, got)
+        return
+    x64 = x.astype(np.float64)
+    exact, scale = exact_fn(x64).ravel(), exact_fn(np.abs(x64)).ravel()
+    if name.startswith("cumprod"):
+        # every rounding of a product reaches the result at full weight, whatever the order:
+        # n roundings of 2^-24 each walk to about sqrt(n) * 2^-24 on either side
+        bound = 8 * np.sqrt(x.size) * 2.0 ** -24
+        assert np.all(np.abs(got.ravel() - exact) <= bound * scale)
+        assert np.all(np.abs(ref.ravel() - exact) <= bound * scale)
+        return
+    assert np.all(np.abs(got.ravel() - exact) <= 1e-5 * scale)
+    assert np.all(np.abs(ref.ravel() - exact) <= 1e-3 * scale)
+
+
 def test_softmax_over_two_rows_of_millions(frontend, hip):
     """Row softmax whose rows are too long for one workgroup each: every reduce in it is cut."""
     shape = (2, 1 << 22)

@@ -366,6 +366,29 @@ def test_few_very_long_reduce_lines_are_planned_as_two_reduces(frontend):
     assert len(hb.render_program(short).launches) == 1
 
 
+def test_few_very_long_scan_lines_are_planned_as_totals_then_scan(frontend):
+    """A scan over axis 0 is lowered with one accumulator for the whole tensor: one line of a
+    million elements.  With a buffer table the plan totals chunks of whole 1024-element tiles
+    first and scans every chunk from the totals ahead of it; without one it stays a single
+    workgroup per line."""
+    from harp_amd import backend as hb, workloads as wl
+    ast = wl.lower_with_table([(2048, 512)], lambda t: t.cumsum(0))[0]
+    plan = hb.render_program(ast)
+    assert [l["schedule"] for l in plan.launches] == ["scan-row-totals(lines=1,chunks=256)",
+                                                       "scan-row(lines=1,length=1048576,chunks=256)"]
+    tot, scan = plan.launches
+    scratch = [b for b in plan.buffers if b["name"].startswith("eh_scanpart_")]
+    assert len(scratch) == 1 and scratch[0]["bytes"] == 4 * 256 and scratch[0]["role"] == "temp"
+    assert tot["args"][-1] == scan["args"][-1] == scratch[0]["name"] and tot["grid"] == scan["grid"] == [256, 1, 1]
+    for l in plan.launches:
+        assert len(hb.compile_source(l["source"])) > 1000
+    assert [l["schedule"] for l in hb.render_program(ast, {"fuse": False}).launches] == ["scan-row(lines=1,length=1048576)"]
+    ragged = hb.render_program(wl.lower_with_table([(3, 700001)], lambda t: t.cummax(1))[0])
+    assert [l["schedule"] for l in ragged.launches][-1] == "scan-row(lines=3,length=700001,chunks=171)"
+    many = hb.render_program(wl.lower_with_table([(64, 1 << 19)], lambda t: t.cumsum(1))[0])
+    assert [l["schedule"] for l in many.launches] == ["scan-row(lines=64,length=524288)"]
+
+
 def test_option_beam_search_on_a_synthetic_cost():
     """The schedule search without a device: suggesters propose neighbours by the schedules in
     the plan, the beam keeps the cheapest states, the search stops when nothing improves."""
