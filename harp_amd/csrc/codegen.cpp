@@ -647,12 +647,12 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
         vec = vec && !lr.guarded && lr.load->count == 1 && lr.load->dtype.itemsize() == 4 &&
               lr.load->args[0]->op == Op::Var && unit_aligned(*lr.load->args[1]);
       vec = vec && scan->out_ptr->op == Op::Var && unit_aligned(*scan->out_index);
-      // A handful of very long lines (a scan over axis 0 is lowered as one line over the whole
-      // tensor) would occupy a handful of workgroups: cut every line into chunks of whole
+      // A few long lines (a scan over axis 0 is lowered as one line over the whole tensor)
+      // would occupy a few workgroups, each bound by the tile-to-tile dependency: cut every line into chunks of whole
       // tiles, total each chunk in a first launch, and let the workgroup that scans a chunk
       // start from the combined totals of the chunks ahead of it.
       int64_t chunks = 1, chunk_len = scan->length;
-      if (extra_buffers && lines <= 16 && scan->length >= (int64_t{1} << 19)) {
+      if (extra_buffers && lines <= 256 && scan->length >= (int64_t{1} << 14)) {
         const int64_t want = 2048 / lines;
         chunk_len = std::max<int64_t>(4096, ((scan->length + want - 1) / want + 1023) / 1024 * 1024);
         chunks = (scan->length + chunk_len - 1) / chunk_len;
@@ -1185,7 +1185,13 @@ std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
   int64_t lines = 1;
   for (const auto& l : nk.loops) lines *= l.extent;
   const int64_t K = nk.rloop.extent;
-  if (lines > 16 || K < (int64_t{1} << 21)) return std::nullopt;
+  {
+    // measured on MI355X: a workgroup streams its line at about 92 GB/s whatever the number of
+    // lines (up to one per CU); the two launches cost about 5.5 us plus the traffic
+    const double whole_us = 1.5 + double(K) * 4.0 / 92e3;
+    const double cut_us = 5.5 + double(lines) * double(K) * 4.0 / 10e6;
+    if (lines > 128 || K < (int64_t{1} << 17) || whole_us <= 1.2 * cut_us) return std::nullopt;
+  }
   std::vector<LoadRef> loads;
   collect_loads(*nk.value, loads);
   bool unit = false;

@@ -966,6 +966,8 @@ LONG_LINES = {
     "max_2x4M": ((2, 1 << 22), lambda t: t.max(1), lambda x: x.max(1), "row"),
     "min_3x2x2M": ((3, 2, 1 << 21), lambda t: t.min(2), lambda x: x.min(2), "row"),
     "mean_sq_2x3M": ((2, 3 << 20), lambda t: (t * t).sum(1), lambda x: (x * x).sum(1), "row"),
+    "max_32x256k": ((32, 1 << 18), lambda t: t.max(1), lambda x: x.max(1), "row"),
+    "sum_8x300k": ((8, 300_000), lambda t: t.sum(1), lambda x: x.sum(1), "row"),
 }
 
 
@@ -996,6 +998,8 @@ LONG_SCANS = {
     "cummax_axis0": ((2048, 512), lambda t: t.cummax(0), None, "scan-row(lines=1,length=1048576,chunks=256)"),
     "cumsum_ragged": ((3, 700001), lambda t: t.cumsum(1), lambda x: np.cumsum(x, 1), "scan-row(lines=3,length=700001,chunks=171)"),
     "cumsum_2x1M": ((2, 1 << 20), lambda t: (t * t).cumsum(1), lambda x: np.cumsum(x * x, 1), "scan-row(lines=2,length=1048576,chunks=256)"),
+    "cumsum_100x20k": ((100, 20_000), lambda t: t.cumsum(1), lambda x: np.cumsum(x, 1), "scan-row(lines=100,length=20000,chunks=5)"),
+    "cummax_mid_7x3000x11": ((7, 3000, 11), lambda t: t.cummax(1), None, "scan-row(lines=7,length=33000,chunks=9)"),
     "cumprod_1x600k": ((1, 600_000), lambda t: t.cumprod(1), lambda x: np.cumprod(x, 1), "scan-row(lines=1,length=600000,chunks=147)"),
 }
 

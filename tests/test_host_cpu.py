@@ -362,7 +362,7 @@ def test_few_very_long_reduce_lines_are_planned_as_two_reduces(frontend):
     t = frontend.Tensor.input([4, 10_000_000])
     bare = frontend.lower_graph([t.sum(1).graph])[0]
     assert len(hb.render_program(bare).launches) == 1
-    short = wl.lower_with_table([(4, 1 << 20)], lambda t: t.sum(1))[0]
+    short = wl.lower_with_table([(4, 1 << 16)], lambda t: t.sum(1))[0]
     assert len(hb.render_program(short).launches) == 1
 
 
@@ -385,8 +385,8 @@ def test_few_very_long_scan_lines_are_planned_as_totals_then_scan(frontend):
     assert [l["schedule"] for l in hb.render_program(ast, {"fuse": False}).launches] == ["scan-row(lines=1,length=1048576)"]
     ragged = hb.render_program(wl.lower_with_table([(3, 700001)], lambda t: t.cummax(1))[0])
     assert [l["schedule"] for l in ragged.launches][-1] == "scan-row(lines=3,length=700001,chunks=171)"
-    many = hb.render_program(wl.lower_with_table([(64, 1 << 19)], lambda t: t.cumsum(1))[0])
-    assert [l["schedule"] for l in many.launches] == ["scan-row(lines=64,length=524288)"]
+    many = hb.render_program(wl.lower_with_table([(512, 1 << 14)], lambda t: t.cumsum(1))[0])
+    assert [l["schedule"] for l in many.launches] == ["scan-row(lines=512,length=16384)"]
 
 
 def test_option_beam_search_on_a_synthetic_cost():
