@@ -940,14 +940,25 @@ bool reduce_is_rowwise(const NestKernel& k) {
   std::vector<LoadRef> loads;
   collect_loads(*k.value, loads);
   bool any_unit = false, any_dep = false;
+  // the operand with the largest footprint decides when operands disagree (a vector times a
+  // matrix: the vector is contiguous along the reduce axis, the matrix along the outputs)
+  int64_t widest = 0;
+  bool widest_unit = false;
   for (const auto& lr : loads) {
     auto a = affine_of(*lr.load->args[1]);
     if (!a) continue;
     int64_t c = a->of(k.rloop.var);
     if (c != 0) any_dep = true;
     if (c == 1 || c == -1) any_unit = true;
+    if (c == 0) continue;
+    int64_t foot = k.rloop.extent;
+    for (const auto& l : k.loops)
+      if (a->of(l.var) != 0) foot *= l.extent;
+    const bool unit = c == 1 || c == -1;
+    if (foot > widest || (foot == widest && unit)) { widest = foot; widest_unit = unit; }
   }
-  return any_unit || !any_dep;
+  if (!any_dep) return true;
+  return any_unit && widest_unit;
 }
 
 // Loads of buffers produced inside the group must hit exactly the element the producer wrote.

@@ -959,6 +959,26 @@ def test_scan_and_scatter_kernels_spread_over_work_items(frontend, hip, name):
         assert bits_equal_mod_zero(ref, got)
 
 
+@pytest.mark.parametrize("shapes,family", [(((1, 1000), (1000, 3000)), "-reduce("), (((3000, 1000), (1000, 1)), "row("),
+                                           (((1, 4096), (4096, 512)), "-reduce(")])
+def test_vector_times_matrix_follows_the_matrix_layout(frontend, hip, shapes, family):
+    """x[1,K] @ W[K,N]: the vector is contiguous along the reduce axis but the matrix, which is
+    all the traffic, is contiguous along the outputs, so the contraction is scheduled as a
+    reduce over a non-contiguous axis (coalesced rows of W); W[N,K] @ x[K,1] stays a row reduce."""
+    from harp_amd import workloads as wl
+    fn = lambda a, b: frontend.nn.matmul(a, b)
+    scheds = [l["schedule"] for l in hip.render_program(wl.lower_with_table(list(shapes), fn)[0]).launches]
+    assert scheds[0].split("(")[0] + "(" in (family, "split" + family, "column" + family, "serial" + family), scheds
+    rng = RNG(sum(shapes[0]))
+    a = rng.uniform(-1, 1, shapes[0]).astype(np.float32)
+    b = rng.uniform(-1, 1, shapes[1]).astype(np.float32)
+    ref, got = both(frontend, fn, [a, b], True)
+    exact = (a.astype(np.float64) @ b.astype(np.float64)).ravel()
+    scale = (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)).ravel()
+    assert np.all(np.abs(got.ravel() - exact) <= 1e-5 * scale)
+    assert np.all(np.abs(ref.ravel() - exact) <= 1e-5 * scale)
+
+
 LONG_LINES = {
     # name: (shape, graph, float64 statement of the same, entry of the kernel that cuts the lines)
     "sum_4x10M": ((4, 10_000_000), lambda t: t.sum(1), lambda x: x.sum(1), "row"),
