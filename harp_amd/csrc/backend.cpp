@@ -379,6 +379,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "fuse") o.fuse = as_int() != 0;
     else if (k == "vectorize") o.vectorize = as_int() != 0;
     else if (k == "transpose") o.transpose = as_int() != 0;
+    else if (k == "window") o.window = as_int() != 0;
     else if (k == "row_threads") o.row_threads = as_int();
     else if (k == "row_elems") o.row_elems = std::max(1, as_int());
     else if (k == "flat_block") o.flat_block = as_int();

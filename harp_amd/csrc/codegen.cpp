@@ -994,6 +994,8 @@ Canon canon_as(const NestKernel& k, StageKind kind) {
 namespace {
 LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& buf_elems);
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan);
+LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestKernel*>& chain, const GenOptions& opt,
+                              const std::map<std::string, size_t>& elems);
 }  // namespace
 
 // Row-major strides of a kernel's loops when its output index is exactly the dense linear index
@@ -1494,9 +1496,96 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // A short reduce over windows that pure gather kernels laid out for it (max-pool, avg-pool:
+  // unfold, copy, reduce over the window axis) reads the source through the gathers' index
+  // maps instead: the window buffers are never written.
+  std::map<size_t, std::vector<size_t>> windows;     // reduce kernel -> its gathers, nearest first
+  if (opt.fuse && opt.window && have_table) {
+    std::map<std::string, size_t> writer;
+    for (size_t q = 0; q < kernels.size(); ++q)
+      if (nests[q] && !folded_kernels.count(q) && !absorbed.count(q)) writer[nests[q]->out_buf] = q;
+    // a gather that reads `buf` stays inside it, and walks it almost contiguously as the
+    // innermost loop outside the window advances
+    auto gather_ok = [&](const NestKernel& g, int64_t K) {
+      if (!make_fold(g, elems)) return false;
+      std::vector<LoadRef> loads;
+      collect_loads(*g.value, loads);
+      int64_t tail = 1;
+      size_t t = g.loops.size();
+      while (t > 0 && tail < K) tail *= g.loops[--t].extent;
+      if (tail != K || t == 0) return false;
+      while (t > 0 && g.loops[t - 1].extent == 1) --t;
+      if (t == 0) return false;
+      const auto src_elems = elems.find(loads[0].load->args[0]->name);
+      for (const auto& lr : loads) {
+        auto a = affine_of(*lr.load->args[1]);
+        if (!a || std::llabs(a->of(g.loops[t - 1].var)) > 8) return false;
+        if (!lr.guarded && (src_elems == elems.end() ||
+                            max_abs_index(*a, g.loops, nullptr) >= static_cast<int64_t>(src_elems->second)))
+          return false;
+      }
+      return true;
+    };
+    for (size_t r = 0; r < kernels.size(); ++r) {
+      if (!nests[r] || folded_kernels.count(r) || absorbed.count(r)) continue;
+      const NestKernel& rk = *nests[r];
+      if (rk.rkind == ReduceKind::None || !rk.out_aff || rk.rloop.extent > 64 || rk.rloop.extent < 2) continue;
+      if (rk.acc_dtype.ty != Ty::F32 || rk.out_dtype.ty != Ty::F32 || gemm_shaped(rk, opt)) continue;
+      std::vector<LoadRef> loads;
+      collect_loads(*rk.value, loads);
+      std::string T;
+      bool ok = !loads.empty();
+      for (const auto& lr : loads) {
+        if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
+        const std::string& b = lr.load->args[0]->name;
+        auto w = writer.find(b);
+        if (role_of(b) != "temp" || w == writer.end() || w->second >= r) continue;
+        if (!T.empty() && T != b) { ok = false; break; }
+        T = b;
+      }
+      if (!ok || T.empty() || readers[T] != std::vector<size_t>{r}) continue;
+      const auto t_elems = elems.find(T);
+      for (const auto& lr : loads) {
+        if (lr.load->args[0]->name != T) continue;
+        auto a = affine_of(*lr.load->args[1]);
+        if (!a || a->of(rk.rloop.var) != 1 || t_elems == elems.end() ||
+            max_abs_index(*a, rk.loops, &rk.rloop) >= static_cast<int64_t>(t_elems->second))
+          ok = false;
+      }
+      if (!ok) continue;
+      std::vector<size_t> chain;
+      std::string buf = T;
+      while (chain.size() < 3) {
+        auto w = writer.find(buf);
+        if (w == writer.end() || role_of(buf) != "temp") break;
+        const size_t q = w->second;
+        if (nests[q]->rkind != ReduceKind::None || !gather_ok(*nests[q], rk.rloop.extent)) break;
+        if (!chain.empty() && readers[buf] != std::vector<size_t>{chain.back()}) break;
+        chain.push_back(q);
+        std::vector<LoadRef> gl;
+        collect_loads(*nests[q]->value, gl);
+        buf = gl[0].load->args[0]->name;
+      }
+      if (chain.empty()) continue;
+      windows[r] = chain;
+      for (size_t q : chain) {
+        folded_kernels.insert(q);
+        writer.erase(nests[q]->out_buf);
+        plan.elided.insert(nests[q]->out_buf);
+      }
+    }
+  }
+
   size_t i = 0;
   while (i < kernels.size()) {
     if (folded_kernels.count(i) || absorbed.count(i)) {
+      ++i;
+      continue;
+    }
+    if (auto w = windows.find(i); w != windows.end()) {
+      std::vector<const NestKernel*> chain;
+      for (size_t q : w->second) chain.push_back(&*nests[q]);
+      plan.launches.push_back(emit_window_reduce(*nests[i], chain, opt, elems));
       ++i;
       continue;
     }
@@ -2614,6 +2703,194 @@ struct SerialReduce {
     return out;
   }
 };
+
+// One work-item per output of a short reduce `r`; `chain` are the pure gathers between the
+// source and r's operand, nearest first (chain[0] wrote what r reads).  Each gather becomes a
+// device function of the element's position in its dense output: the loop variables are
+// decoded from the position and the gather's own expression is evaluated, with its load of
+// the previous gather's output turned into a call of that gather's function.
+LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestKernel*>& chain, const GenOptions& opt,
+                              const std::map<std::string, size_t>& elems) {
+  LaunchSpec ls;
+  ls.entry = "ehk_" + r.name;
+  ls.kernels = {};
+  for (size_t j = chain.size(); j-- > 0;) ls.kernels.push_back(chain[j]->name);
+  ls.kernels.push_back(r.name);
+  int64_t N = 1;
+  std::vector<Loop> live;
+  for (const auto& l : r.loops) {
+    N *= l.extent;
+    if (l.extent > 1) live.push_back(l);
+  }
+  if ((N + 255) / 256 >= (int64_t{1} << 31)) throw Error("too many outputs for one launch");
+  std::vector<LoadRef> deep;
+  collect_loads(*chain.back()->value, deep);
+  const std::string src = deep[0].load->args[0]->name;
+  bool idx64 = N >= kIndex32Limit;
+  auto big = [&](const std::string& b) {
+    auto it = elems.find(b);
+    return it == elems.end() || it->second >= static_cast<size_t>(kIndex32Limit);
+  };
+  idx64 = idx64 || big(src) || big(r.out_buf);
+  for (const auto* g : chain) idx64 = idx64 || big(g->out_buf);
+  std::vector<LoadRef> rloads;
+  collect_loads(*r.value, rloads);
+  for (const auto& lr : rloads) idx64 = idx64 || big(lr.load->args[0]->name);
+  std::ostringstream os;
+  os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+  auto fn_of = [](const std::string& buf) { return "eh_win_" + buf; };
+  // The arguments of gather g's function for the element at `index` of its dense output: one
+  // per loop of g, the digit (index / stride) % extent.  `index` is affine over the caller's
+  // loops, so most digits come out as one of those loops (or a constant after unrolling)
+  // without a division: terms whose coefficient is a multiple of stride * extent vanish,
+  // terms below the stride cannot carry when together they stay below it.
+  auto call_of = [&](const NestKernel& g, const Node& index, const std::vector<Loop>& caller) {
+    ExprRenderer plain;
+    const std::string whole = "((idx_t)(" + plain.expr(index) + "))";
+    auto a = affine_of(index);
+    std::string args;
+    // the index as a mixed-radix number over the caller's loops: coefficients ascending, each
+    // above everything the smaller terms can add up to
+    struct Term { int64_t c, ext; std::string var; };
+    std::vector<Term> terms;
+    bool nested = a.has_value() && a->c == 0;
+    if (nested) {
+      for (const auto& kv : a->coef) {
+        if (kv.second == 0) continue;
+        int64_t ext = 0;
+        for (const auto& l : caller)
+          if (l.var == kv.first) ext = l.extent;
+        if (kv.second < 0 || ext <= 0) { nested = false; break; }
+        if (ext > 1) terms.push_back({kv.second, ext, kv.first});
+      }
+      std::sort(terms.begin(), terms.end(), [](const Term& x, const Term& y) { return x.c < y.c; });
+      int64_t reach = 0;
+      for (const auto& t : terms) {
+        if (t.c <= reach) { nested = false; break; }
+        reach += t.c * (t.ext - 1);
+      }
+    }
+    int64_t stride = 1;
+    std::vector<std::string> digits(g.loops.size());
+    for (size_t q = g.loops.size(); q-- > 0;) {
+      const int64_t e = g.loops[q].extent;
+      std::string d;
+      if (e == 1) {
+        d = "0";
+      } else {
+        bool symbolic = nested;
+        int64_t dmax = 0;
+        std::string sum;
+        auto add = [&](const std::string& t, int64_t tmax) {
+          sum += (sum.empty() ? "" : " + ") + t;
+          dmax += tmax;
+        };
+        if (symbolic)
+          for (const auto& t : terms) {
+            if (t.c % (stride * e) == 0) continue;                       // vanishes modulo the extent
+            if (t.c >= stride) {
+              if (t.c % stride) { symbolic = false; break; }
+              const int64_t m = t.c / stride;
+              add(m == 1 ? t.var : t.var + " * " + std::to_string(m), m * (t.ext - 1));
+            } else if (t.c * (t.ext - 1) >= stride) {                      // reaches into this digit from below
+              if (stride % t.c) { symbolic = false; break; }
+              const int64_t dv = stride / t.c;
+              add("(" + t.var + " / " + std::to_string(dv) + ")", (t.ext - 1) / dv);
+            }
+          }
+        if (symbolic) d = sum.empty() ? "0" : dmax < e ? "(" + sum + ")" : "((" + sum + ") % " + std::to_string(e) + ")";
+        else d = "((" + whole + " / " + std::to_string(stride) + ") % " + std::to_string(e) + ")";
+      }
+      digits[q] = d;
+      stride *= e;
+    }
+    for (const auto& d : digits) args += ", " + d;
+    return fn_of(g.out_buf) + "(" + src + args + ")";
+  };
+  for (size_t j = chain.size(); j-- > 0;) {
+    const NestKernel& g = *chain[j];
+    os << "// the element of what kernel " << g.name << " would have written, by its loop variables\n";
+    os << "__device__ __forceinline__ float " << fn_of(g.out_buf) << "(const float* __restrict__ " << src;
+    for (const auto& l : g.loops) os << ", const idx_t " << l.var;
+    os << ") {\n";
+    ExprRenderer er;
+    if (j + 1 < chain.size()) {
+      const NestKernel* inner = chain[j + 1];
+      er.load_hook = [&, inner](const Node& ld, std::string* out) {
+        if (ld.args[0]->op != Op::Var || ld.args[0]->name != inner->out_buf) return false;
+        *out = call_of(*inner, *ld.args[1], g.loops);
+        return true;
+      };
+    }
+    os << "  return (float)(" << er.expr(*g.value) << ");\n}\n";
+  }
+  // parameters: r's own, with the window buffer replaced by the source
+  const std::string T = chain[0]->out_buf;
+  std::string sig;
+  bool src_listed = false;
+  for (const auto& p : r.params) {
+    std::string name = p.name;
+    if (name == T) name = src;
+    if (name == src) {
+      if (src_listed) continue;
+      src_listed = true;
+    }
+    sig += (sig.empty() ? "" : ", ") + std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + name;
+    ls.arg_bufs.push_back(name);
+  }
+  os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << sig << ") {\n";
+  os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
+  os << "  idx_t eh_rem = eh_o;\n";
+  for (size_t q = live.size(); q-- > 0;) {
+    os << "  const idx_t " << live[q].var << " = eh_rem % " << live[q].extent << ";\n";
+    if (q) os << "  eh_rem /= " << live[q].extent << ";\n";
+  }
+  for (const auto& l : r.loops)
+    if (l.extent == 1) os << "  const idx_t " << l.var << " = 0;\n";
+  ExprRenderer er;
+  std::vector<Loop> rvars = r.loops;
+  rvars.push_back(r.rloop);
+  er.load_hook = [&](const Node& ld, std::string* out) {
+    if (ld.args[0]->op != Op::Var || ld.args[0]->name != T) return false;
+    *out = call_of(*chain[0], *ld.args[1], rvars);
+    return true;
+  };
+  os << "  float acc = " << literal(*r.identity) << ";\n#pragma unroll\n";
+  os << "  for (idx_t " << r.rloop.var << " = 0; " << r.rloop.var << " < " << r.rloop.extent << "; ++" << r.rloop.var << ") {\n";
+  os << "    acc = " << combine_text(r.rkind, r.acc_dtype, "acc", "(float)(" + er.expr(*r.value) + ")") << ";\n  }\n";
+  NodePtr oi = rename(r.out_index, {{r.rloop.var, make_i64(0)}});
+  ExprRenderer eo;
+  os << "  " << r.out_buf << "[" << eo.expr(*oi) << "] = acc;\n}\n";
+  ls.source = os.str();
+  ls.grid[0] = static_cast<unsigned>((N + 255) / 256);
+  ls.block[0] = 256;
+  ls.schedule = "window-reduce(window=" + std::to_string(r.rloop.extent) + ",gathers=" + std::to_string(chain.size()) + ")";
+  // smallest buffers: the source as the innermost gather reads it (unguarded loads), r's other
+  // operands and its output as r indexes them
+  std::map<std::string, int64_t> need;
+  for (const auto& lr : deep) {
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a || lr.guarded) continue;
+    auto& n = need[src];
+    n = std::max(n, max_abs_index(*a, chain.back()->loops, nullptr) + 1);
+  }
+  for (const auto& lr : rloads) {
+    const std::string& b = lr.load->args[0]->name;
+    auto a = affine_of(*lr.load->args[1]);
+    if (b == T || !a || lr.guarded) continue;
+    auto& n = need[b];
+    n = std::max(n, max_abs_index(*a, r.loops, &r.rloop) + 1);
+  }
+  need[r.out_buf] = max_abs_index(*r.out_aff, r.loops, nullptr) + 1;
+  std::set<std::string> counted;
+  for (const auto& b : ls.arg_bufs) {
+    auto it = need.find(b);
+    ls.arg_min_bytes.push_back(it == need.end() ? 0 : static_cast<size_t>(it->second) * 4);
+    auto e = elems.find(b);
+    if (e != elems.end() && counted.insert(b).second) ls.algo_bytes += 4.0 * static_cast<double>(e->second);
+  }
+  return ls;
+}
 
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan) {
   SerialReduce sr(k, opt);

@@ -20,6 +20,7 @@ struct GenOptions {
   bool fuse = true;          // merge compatible kernels of a Program into one launch
   bool vectorize = true;     // 128-bit accesses where alignment allows
   bool transpose = true;     // transposing elementwise groups go through 64x64 LDS tiles
+  bool window = true;             // short reduces over gathered windows read the source directly
   int row_threads = 0;       // threads cooperating on one row; 0 = choose from the row length
   int row_elems = 8;         // target elements per thread per row when choosing row_threads
   int flat_block = 256;

@@ -86,7 +86,7 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
 /* ---- Renderer: AST -> source + dispatch sizes, no device needed
  *      (src/backend/renderer.rs:20-35; KernelSourceRenderer and extract_kernel_config,
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
- *      arch, fuse, vectorize, transpose, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
+ *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
  *      gemm_epilogue, gemm_dma, gemm_merge_batch, nontemporal. ----------------------------- */
 typedef struct eh_launch_info {

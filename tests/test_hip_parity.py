@@ -979,6 +979,49 @@ def test_vector_times_matrix_follows_the_matrix_layout(frontend, hip, shapes, fa
     assert np.all(np.abs(ref.ravel() - exact) <= 1e-5 * scale)
 
 
+POOLS = {
+    # name: (input shape, graph, exact mode, numpy statement or None)
+    "max2": ((3, 5, 12, 16), lambda nn, t: nn.max_pool2d(t, (2, 2)), True,
+             lambda x: x.reshape(3, 5, 6, 2, 8, 2).max((3, 5))),
+    "max2_as_written": ((3, 5, 12, 16), lambda nn, t: nn.max_pool2d(t, (2, 2)), False, None),
+    "max3s2p1": ((2, 4, 15, 13), lambda nn, t: nn.max_pool2d(t, (3, 3), (2, 2), (1, 1)), True, None),
+    "max3s1d2": ((2, 3, 17, 17), lambda nn, t: nn.max_pool2d(t, (3, 3), (1, 1), (0, 0), (2, 2)), True, None),
+    "avg2": ((4, 3, 10, 14), lambda nn, t: nn.avg_pool2d(t, (2, 2), exact=True), True,
+             lambda x: x.reshape(4, 3, 5, 2, 7, 2).mean((3, 5))),
+    "avg3s2p1": ((2, 3, 9, 9), lambda nn, t: nn.avg_pool2d(t, (3, 3), (2, 2), (1, 1), exact=True), True, None),
+    "avg3s2p1_as_written": ((2, 3, 9, 9), lambda nn, t: nn.avg_pool2d(t, (3, 3), (2, 2), (1, 1)), False, None),
+}
+
+
+@pytest.mark.parametrize("name", sorted(POOLS))
+def test_pooling_reads_its_windows_from_the_source(frontend, hip, name):
+    """Pooling is lowered as unfold (a gather that lays the windows out), sometimes a copy, then a
+    short reduce over the window axis (src/tensor/nn/pool.rs:146-160 in the reference).  With a
+    buffer table the reduce reads the source through the gathers' index maps, one work-item
+    per output, and the window buffers are never written; results match the oracle, which
+    runs the kernels as lowered, and numpy where the case has a closed form."""
+    from harp_amd import workloads as wl
+    import contextlib
+    shape, graph, exact, closed = POOLS[name]
+    fn = lambda t: graph(frontend.nn, t)
+    with (frontend.exact_mode() if exact else contextlib.nullcontext()):
+        plan = hip.render_program(wl.lower_with_table([shape], fn)[0])
+        scheds = [l["schedule"] for l in plan.launches]
+        assert any(s.startswith("window-reduce(") for s in scheds), scheds
+        win = [l for l in plan.launches if l["schedule"].startswith("window-reduce(")][0]
+        elided = {b["name"] for b in plan.buffers if b["elided"]}
+        assert len(elided) == len(win["kernels"]) - 1 and not elided & set(win["args"])
+        x = RNG(len(name)).uniform(-2, 2, shape).astype(np.float32)
+        ref, got = both(frontend, fn, [x], True)
+        off = realize_on(frontend, "hip", fn, [x], fuse=False)
+    if "max" in name:
+        assert bits_equal_mod_zero(ref, got) and bits_equal_mod_zero(off, got)
+    else:
+        assert np.allclose(got, ref, rtol=1e-5, atol=1e-6) and np.allclose(got, off, rtol=1e-5, atol=1e-6)
+    if closed is not None:
+        assert np.allclose(got, closed(x.astype(np.float64)).ravel(), rtol=1e-5, atol=1e-6)
+
+
 LONG_LINES = {
     # name: (shape, graph, float64 statement of the same, entry of the kernel that cuts the lines)
     "sum_4x10M": ((4, 10_000_000), lambda t: t.sum(1), lambda x: x.sum(1), "row"),

@@ -389,6 +389,30 @@ def test_few_very_long_scan_lines_are_planned_as_totals_then_scan(frontend):
     assert [l["schedule"] for l in many.launches] == ["scan-row(lines=512,length=16384)"]
 
 
+def test_pooling_plan_reads_the_source_through_the_gathers(frontend):
+    """max-pool as lowered (unfold gather, a second gather through the same view, reduce over the
+    window): one launch, both window buffers elided, the gathers as device functions whose
+    loop variables the caller passes without divisions where the indices line up.  Switched
+    off, or when something else reads the windows too, the gathers stay launches."""
+    from harp_amd import backend as hb, workloads as wl
+    fn = lambda t: frontend.nn.max_pool2d(t, (2, 2))
+    ast = wl.lower_with_table([(2, 3, 8, 8)], fn)[0]
+    plan = hb.render_program(ast)
+    assert [l["schedule"] for l in plan.launches] == ["window-reduce(window=4,gathers=2)"]
+    (l,) = plan.launches
+    assert len(l["kernels"]) == 3 and l["args"] == ["buf0", "buf6"]
+    assert sorted(b["name"] for b in plan.buffers if b["elided"]) == ["buf2", "buf4"]
+    assert "eh_win_buf4(buf0, (ridx0), (ridx1), (ridx2), (ridx3), ((ridx4 / 2)), ((ridx4) % 2))" in l["source"]
+    assert "eh_win_buf2(buf0, (ridx0), (ridx1), (ridx2), ((ridx3 / 2) + ridx4 * 2), ((ridx3) % 2), (ridx5))" in l["source"]
+    assert len(hb.compile_source(l["source"])) > 1000
+    off = hb.render_program(ast, {"window": 0})
+    assert len(off.launches) == 3 and not any(b["elided"] for b in off.buffers)
+    with frontend.exact_mode():
+        shared = wl.lower_with_table([(2, 3, 8, 8)], lambda t: (lambda w: w.max(4).sum(3) + w.sum(4).sum(3))(
+            t.unfold([2, 3], [2, 2], [2, 2], [1, 1]).contiguous().reshape([2, 3, 4, 4, 4])))[0]
+    assert not any(s["schedule"].startswith("window") for s in hb.render_program(shared).launches)
+
+
 def test_option_beam_search_on_a_synthetic_cost():
     """The schedule search without a device: suggesters propose neighbours by the schedules in
     the plan, the beam keeps the cheapest states, the search stops when nothing improves."""
