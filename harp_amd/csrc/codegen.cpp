@@ -1013,7 +1013,7 @@ std::optional<std::vector<int64_t>> dense_strides(const NestKernel& k, int64_t* 
   }
   for (const auto& kv : k.out_aff->coef) {
     bool live = false;
-    for (const auto& l : k.loops) live = live || (l.var == kv.first && l.extent > 1);
+    for (const auto& l : k.loops) live = live || l.var == kv.first;     // a loop that runs once adds nothing
     if (kv.second != 0 && !live) return std::nullopt;
   }
   *numel = stride;
@@ -1040,7 +1040,7 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   }
   for (const auto& kv : k.out_aff->coef) {
     bool live = false;
-    for (const auto& l : k.loops) live = live || (l.var == kv.first && l.extent > 1);
+    for (const auto& l : k.loops) live = live || l.var == kv.first;     // a loop that runs once adds nothing
     if (kv.second != 0 && !live) return std::nullopt;
   }
   (void)used;
@@ -1099,7 +1099,7 @@ std::optional<Affine> relayout(const NestKernel& g, const NestKernel& sk, const 
   }
   for (const auto& kv : read.coef) {
     bool live = false;
-    for (const auto& l : sk.loops) live = live || (l.var == kv.first && l.extent > 1);
+    for (const auto& l : sk.loops) live = live || l.var == kv.first;    // a loop that runs once adds nothing
     if (kv.second != 0 && !live) return std::nullopt;
   }
   std::sort(cv.begin(), cv.end(), [](const CV& a, const CV& b) { return a.read > b.read; });

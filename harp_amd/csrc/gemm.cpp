@@ -77,7 +77,7 @@ double estimate_us(const GemmShape& s, const Candidate& c, int split) {
 }
 
 // Tile and K split for a contraction.
-bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
+bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool computed_operand = false) {
   if (s.K < 8 || s.M < 2 || s.N < 2) return false;
   Choice best;
   if (opt.gemm_bm > 0) {
@@ -91,6 +91,10 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out) {
   double best_us = 0;
   bool have = false;
   for (const auto& c : kCandidates) {
+    // an operand evaluated in the tile loader (index decode, guards) slows every k-step of a
+    // workgroup down; many small workgroups hide that, a few large ones do not (measured: a
+    // 3x3 convolution over [32,128,28,28], 64x64 tiles 142 us, 128x128 295 us, 256x256 380 us)
+    if (computed_operand && c.tile.bm > 64) continue;
     const int64_t ksteps = ceil_div(s.K, c.tile.bk);
     for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
@@ -222,8 +226,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
                                       const FoldMap* folded, const EpilogueSpec* epilogue) {
   auto s = match_gemm(k);
   Choice ch;
-  if (!s || !choose(*s, opt, &ch)) return {};
-  const Tile& t = ch.tile;
+  if (!s) return {};
   const FoldedOperand* fa = nullptr;
   const FoldedOperand* fb = nullptr;
   if (folded) {
@@ -231,6 +234,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     if (ia != folded->end()) fa = &ia->second;
     if (ib != folded->end()) fb = &ib->second;
   }
+  if (!choose(*s, opt, &ch, fa || fb)) return {};
+  const Tile& t = ch.tile;
   // each thread fetches four elements along the operand's faster axis
   bool a_kc = s->a_k <= s->a_m, b_nc = s->b_n <= s->b_k;
   // a computed operand is walked along whichever of its axes is contiguous in the memory its
