@@ -1174,6 +1174,32 @@ def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
         assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
 
 
+LONG_LINE_SEEDS = [(7007, 0), (7052, 0), (7084, 0), (7092, 0), (7229, 0), (7264, 0), (7282, 0), (7284, 0), (7296, 0),
+                   (7024, 8), (7028, 8), (7087, 8), (7107, 8), (7154, 8), (7373, 8)]
+
+
+@pytest.mark.parametrize("seed,first_kind", LONG_LINE_SEEDS)
+def test_random_graphs_with_few_long_lines_match_the_oracle(frontend, hip, seed, first_kind):
+    """The same generator over one to twenty lines of 40 000 or 300 000 elements, seeds chosen
+    so that the plan cuts a reduce or a scan line over workgroups (totals, row normalisations,
+    gathers before a reduce, prefix scans after elementwise chains)."""
+    import graph_fuzz
+    from harp_amd import workloads as wl
+    dims = (1, 2, 3, 7, 20, 40000, 300000)
+    with frontend.exact_mode():
+        shapes, fn, desc = graph_fuzz.build(seed, frontend, dims=dims, max_rank=2, kinds=(first_kind, first_kind + (8 if first_kind == 0 else 4)))
+        launches = hip.render_program(wl.lower_with_table(shapes, fn)[0]).launches
+        assert any(l["entry"].endswith("_rows") or l["schedule"].startswith("scan-row-totals(") for l in launches), desc
+        rng = RNG(seed)
+        arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+        rtol = 2e-4 if "kind 8" in desc else 2e-5
+        for fuse in (True, False):
+            ref, got = both(frontend, fn, arrays, fuse)
+            assert ref.shape == got.shape, desc
+            scale = max(1.0, float(np.abs(ref).max()))
+            assert np.allclose(got, ref, rtol=rtol, atol=rtol / 10 * scale), (desc, fuse)
+
+
 @pytest.mark.parametrize("seed", range(400, 405))
 def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
     """Random conv + pool + linear classifiers (tests/graph_fuzz.py): forward with the fused
