@@ -1020,6 +1020,97 @@ std::optional<std::vector<int64_t>> dense_strides(const NestKernel& k, int64_t* 
   return strides;
 }
 
+std::string gather_fn_name(const std::string& buf) { return "eh_win_" + buf; }
+
+// The arguments of gather g's function for the element at `index` of its dense output: one
+// per loop of g, the digit (index / stride) % extent.  `index` is affine over the caller's
+// loops, so most digits come out as one of those loops (or a constant after unrolling)
+// without a division: terms whose coefficient is a multiple of stride * extent vanish,
+// terms below the stride cannot carry when together they stay below it.
+std::string gather_call(const NestKernel& g, const std::string& src, const Node& index, const std::vector<Loop>& caller,
+                        const std::string& idx_type) {
+  ExprRenderer plain;
+  const std::string whole = "((" + idx_type + ")(" + plain.expr(index) + "))";
+  auto a = affine_of(index);
+  std::string args;
+  // the index as a mixed-radix number over the caller's loops: coefficients ascending, each
+  // above everything the smaller terms can add up to
+  struct Term { int64_t c, ext; std::string var; };
+  std::vector<Term> terms;
+  bool nested = a.has_value() && a->c == 0;
+  if (nested) {
+    for (const auto& kv : a->coef) {
+      if (kv.second == 0) continue;
+      int64_t ext = 0;
+      for (const auto& l : caller)
+        if (l.var == kv.first) ext = l.extent;
+      if (kv.second < 0 || ext <= 0) { nested = false; break; }
+      if (ext > 1) terms.push_back({kv.second, ext, kv.first});
+    }
+    std::sort(terms.begin(), terms.end(), [](const Term& x, const Term& y) { return x.c < y.c; });
+    int64_t reach = 0;
+    for (const auto& t : terms) {
+      if (t.c <= reach) { nested = false; break; }
+      reach += t.c * (t.ext - 1);
+    }
+  }
+  int64_t stride = 1;
+  std::vector<std::string> digits(g.loops.size());
+  for (size_t q = g.loops.size(); q-- > 0;) {
+    const int64_t e = g.loops[q].extent;
+    std::string d;
+    if (e == 1) {
+      d = "0";
+    } else {
+      bool symbolic = nested;
+      int64_t dmax = 0;
+      std::string sum;
+      auto add = [&](const std::string& t, int64_t tmax) {
+        sum += (sum.empty() ? "" : " + ") + t;
+        dmax += tmax;
+      };
+      if (symbolic)
+        for (const auto& t : terms) {
+          if (t.c % (stride * e) == 0) continue;                       // vanishes modulo the extent
+          if (t.c >= stride) {
+            if (t.c % stride) { symbolic = false; break; }
+            const int64_t m = t.c / stride;
+            add(m == 1 ? t.var : t.var + " * " + std::to_string(m), m * (t.ext - 1));
+          } else if (t.c * (t.ext - 1) >= stride) {                      // reaches into this digit from below
+            if (stride % t.c) { symbolic = false; break; }
+            const int64_t dv = stride / t.c;
+            add("(" + t.var + " / " + std::to_string(dv) + ")", (t.ext - 1) / dv);
+          }
+        }
+      if (symbolic) d = sum.empty() ? "0" : dmax < e ? "(" + sum + ")" : "((" + sum + ") % " + std::to_string(e) + ")";
+      else d = "((" + whole + " / " + std::to_string(stride) + ") % " + std::to_string(e) + ")";
+    }
+    digits[q] = d;
+    stride *= e;
+  }
+  for (const auto& d : digits) args += ", " + d;
+  return gather_fn_name(g.out_buf) + "(" + src + args + ")";
+}
+
+// Gather g as a device function of its own loop variables; `inner`, when given, is the gather
+// whose output g reads: that load becomes a call of inner's function.
+std::string gather_fn_text(const NestKernel& g, const std::string& src, const NestKernel* inner, const std::string& idx_type) {
+  std::ostringstream os;
+  os << "// the element of what kernel " << g.name << " would have written, by its loop variables\n";
+  os << "__device__ __forceinline__ float " << gather_fn_name(g.out_buf) << "(const float* __restrict__ " << src;
+  for (const auto& l : g.loops) os << ", const " << idx_type << " " << l.var;
+  os << ") {\n";
+  ExprRenderer er;
+  if (inner)
+    er.load_hook = [&](const Node& ld, std::string* out) {
+      if (ld.args[0]->op != Op::Var || ld.args[0]->name != inner->out_buf) return false;
+      *out = gather_call(*inner, src, *ld.args[1], g.loops, idx_type);
+      return true;
+    };
+  os << "  return (float)(" << er.expr(*g.value) << ");\n}\n";
+  return os.str();
+}
+
 // An elementwise kernel as a function of the linear index of its (dense, row-major) output, for
 // contractions that evaluate it in their tile loader.  Only kernels reading one f32 buffer.
 std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems) {
@@ -1490,6 +1581,44 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (!ok) continue;
       auto f = make_fold(pk, elems);
       if (!f || folded.count(f->src)) continue;
+      // The gather's own source may be a buffer another pure gather wrote for it alone (a
+      // convolution as the reference lowers it applies the unfold view twice): that gather
+      // becomes a device function the first one calls, and its buffer goes too.
+      for (size_t q = 0; q < p && opt.window; ++q) {
+        if (!nests[q] || nests[q]->out_buf != f->src || nests[q]->rkind != ReduceKind::None) continue;
+        if (folded_kernels.count(q) || absorbed.count(q) || role_of(f->src) != "temp") break;
+        if (readers[f->src] != std::vector<size_t>{p}) break;
+        auto fi = make_fold(*nests[q], elems);
+        auto in_elems = elems.find(f->src);
+        if (!fi || folded.count(fi->src) || in_elems == elems.end()) break;
+        std::vector<LoadRef> pl;
+        collect_loads(*pk.value, pl);
+        bool ok = true;
+        for (const auto& lr : pl) {
+          auto a = affine_of(*lr.load->args[1]);
+          if (!a) { ok = false; break; }
+          if (!lr.guarded && max_abs_index(*a, pk.loops, nullptr) >= static_cast<int64_t>(in_elems->second)) ok = false;
+        }
+        if (!ok) break;
+        const NestKernel& inner = *nests[q];
+        f->small = f->small && fi->small;
+        const std::string IT = f->small ? "int" : "long long";
+        f->prelude = gather_fn_text(inner, fi->src, nullptr, IT);
+        ExprRenderer er;
+        er.load_hook = [&](const Node& ld, std::string* out) {
+          if (ld.args[0]->op != Op::Var || ld.args[0]->name != inner.out_buf) return false;
+          *out = gather_call(inner, fi->src, *ld.args[1], pk.loops, IT);
+          return true;
+        };
+        f->expr = er.expr(*pk.value);
+        f->kernel = inner.name + ", then " + pk.name;
+        f->src = fi->src;
+        f->src_bytes = fi->src_bytes;
+        f->src_stride.clear();
+        folded_kernels.insert(q);
+        plan.elided.insert(inner.out_buf);
+        break;
+      }
       folded[pk.out_buf] = *f;
       folded_kernels.insert(p);
       plan.elided.insert(pk.out_buf);
@@ -2738,92 +2867,8 @@ LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestK
   for (const auto& lr : rloads) idx64 = idx64 || big(lr.load->args[0]->name);
   std::ostringstream os;
   os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
-  auto fn_of = [](const std::string& buf) { return "eh_win_" + buf; };
-  // The arguments of gather g's function for the element at `index` of its dense output: one
-  // per loop of g, the digit (index / stride) % extent.  `index` is affine over the caller's
-  // loops, so most digits come out as one of those loops (or a constant after unrolling)
-  // without a division: terms whose coefficient is a multiple of stride * extent vanish,
-  // terms below the stride cannot carry when together they stay below it.
-  auto call_of = [&](const NestKernel& g, const Node& index, const std::vector<Loop>& caller) {
-    ExprRenderer plain;
-    const std::string whole = "((idx_t)(" + plain.expr(index) + "))";
-    auto a = affine_of(index);
-    std::string args;
-    // the index as a mixed-radix number over the caller's loops: coefficients ascending, each
-    // above everything the smaller terms can add up to
-    struct Term { int64_t c, ext; std::string var; };
-    std::vector<Term> terms;
-    bool nested = a.has_value() && a->c == 0;
-    if (nested) {
-      for (const auto& kv : a->coef) {
-        if (kv.second == 0) continue;
-        int64_t ext = 0;
-        for (const auto& l : caller)
-          if (l.var == kv.first) ext = l.extent;
-        if (kv.second < 0 || ext <= 0) { nested = false; break; }
-        if (ext > 1) terms.push_back({kv.second, ext, kv.first});
-      }
-      std::sort(terms.begin(), terms.end(), [](const Term& x, const Term& y) { return x.c < y.c; });
-      int64_t reach = 0;
-      for (const auto& t : terms) {
-        if (t.c <= reach) { nested = false; break; }
-        reach += t.c * (t.ext - 1);
-      }
-    }
-    int64_t stride = 1;
-    std::vector<std::string> digits(g.loops.size());
-    for (size_t q = g.loops.size(); q-- > 0;) {
-      const int64_t e = g.loops[q].extent;
-      std::string d;
-      if (e == 1) {
-        d = "0";
-      } else {
-        bool symbolic = nested;
-        int64_t dmax = 0;
-        std::string sum;
-        auto add = [&](const std::string& t, int64_t tmax) {
-          sum += (sum.empty() ? "" : " + ") + t;
-          dmax += tmax;
-        };
-        if (symbolic)
-          for (const auto& t : terms) {
-            if (t.c % (stride * e) == 0) continue;                       // vanishes modulo the extent
-            if (t.c >= stride) {
-              if (t.c % stride) { symbolic = false; break; }
-              const int64_t m = t.c / stride;
-              add(m == 1 ? t.var : t.var + " * " + std::to_string(m), m * (t.ext - 1));
-            } else if (t.c * (t.ext - 1) >= stride) {                      // reaches into this digit from below
-              if (stride % t.c) { symbolic = false; break; }
-              const int64_t dv = stride / t.c;
-              add("(" + t.var + " / " + std::to_string(dv) + ")", (t.ext - 1) / dv);
-            }
-          }
-        if (symbolic) d = sum.empty() ? "0" : dmax < e ? "(" + sum + ")" : "((" + sum + ") % " + std::to_string(e) + ")";
-        else d = "((" + whole + " / " + std::to_string(stride) + ") % " + std::to_string(e) + ")";
-      }
-      digits[q] = d;
-      stride *= e;
-    }
-    for (const auto& d : digits) args += ", " + d;
-    return fn_of(g.out_buf) + "(" + src + args + ")";
-  };
-  for (size_t j = chain.size(); j-- > 0;) {
-    const NestKernel& g = *chain[j];
-    os << "// the element of what kernel " << g.name << " would have written, by its loop variables\n";
-    os << "__device__ __forceinline__ float " << fn_of(g.out_buf) << "(const float* __restrict__ " << src;
-    for (const auto& l : g.loops) os << ", const idx_t " << l.var;
-    os << ") {\n";
-    ExprRenderer er;
-    if (j + 1 < chain.size()) {
-      const NestKernel* inner = chain[j + 1];
-      er.load_hook = [&, inner](const Node& ld, std::string* out) {
-        if (ld.args[0]->op != Op::Var || ld.args[0]->name != inner->out_buf) return false;
-        *out = call_of(*inner, *ld.args[1], g.loops);
-        return true;
-      };
-    }
-    os << "  return (float)(" << er.expr(*g.value) << ");\n}\n";
-  }
+  for (size_t j = chain.size(); j-- > 0;)
+    os << gather_fn_text(*chain[j], src, j + 1 < chain.size() ? chain[j + 1] : nullptr, "idx_t");
   // parameters: r's own, with the window buffer replaced by the source
   const std::string T = chain[0]->out_buf;
   std::string sig;
@@ -2852,7 +2897,7 @@ LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestK
   rvars.push_back(r.rloop);
   er.load_hook = [&](const Node& ld, std::string* out) {
     if (ld.args[0]->op != Op::Var || ld.args[0]->name != T) return false;
-    *out = call_of(*chain[0], *ld.args[1], rvars);
+    *out = gather_call(*chain[0], src, *ld.args[1], rvars, "idx_t");
     return true;
   };
   os << "  float acc = " << literal(*r.identity) << ";\n#pragma unroll\n";

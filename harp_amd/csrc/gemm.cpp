@@ -310,6 +310,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     const std::string IT = f->small ? "int" : "long long";
     os << "#define EH_" << X << "_FOLD 1\n#define EH_" << X << "_FOLD_MODE " << mode << "\n#define EH_" << X << "_FOLD_Q " << Q
        << "LL\n";
+    os << f->prelude;
     os << "// element (eh_U * " << Q << " + eh_I) of what kernel " << f->kernel << " would have written\n";
     os << "__device__ __forceinline__ float " << fn << "(const float* __restrict__ " << f->src
        << ", long long eh_U64, long long eh_I64) {\n";

@@ -32,6 +32,7 @@ struct FoldedOperand {
   std::string src;        // the one buffer the producer reads
   std::string kernel;     // the producer's name (for comments)
   std::string expr;       // C expression over the loop variables and `src`
+  std::string prelude;    // device functions `expr` calls (a gather folded into this one), or empty
   struct LoopVar {
     std::string name;
     int64_t extent, stride;   // stride in the producer's dense output

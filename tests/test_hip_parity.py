@@ -979,6 +979,39 @@ def test_vector_times_matrix_follows_the_matrix_layout(frontend, hip, shapes, fa
     assert np.all(np.abs(ref.ravel() - exact) <= 1e-5 * scale)
 
 
+CONVS_AS_WRITTEN = {
+    # name: (input shape, weight shape, graph)
+    "3x3_pad1": ((3, 5, 12, 10), (7, 5, 3, 3), lambda nn, x, w: nn.conv2d(x, w, None, (1, 1), (1, 1))),
+    "1x1": ((2, 16, 9, 9), (8, 16, 1, 1), lambda nn, x, w: nn.conv2d(x, w)),
+    "5x5_stride2": ((2, 3, 21, 19), (6, 3, 5, 5), lambda nn, x, w: nn.conv2d(x, w, None, (2, 2), (2, 2))),
+    "conv1d_k5": ((4, 6, 100), (9, 6, 5), lambda nn, x, w: nn.conv1d(x, w)),
+    "3x3_64ch": ((2, 64, 14, 14), (64, 64, 3, 3), lambda nn, x, w: nn.conv2d(x, w, None, (1, 1), (1, 1))),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CONVS_AS_WRITTEN))
+def test_convolution_as_the_reference_lowers_it_has_no_gather_launch(frontend, hip, name):
+    """As the reference lowers a convolution, the unfold view is applied twice: a gather writes
+    the windows, a second gather reads that buffer through the same view, the contraction
+    reads the second.  Both gathers are evaluated in the contraction's tile loader (the first
+    as a device function the second calls) and neither buffer exists; results equal the
+    oracle's, which runs the three kernels, and the per-kernel HIP path's."""
+    from harp_amd import workloads as wl
+    xs, ws, graph = CONVS_AS_WRITTEN[name]
+    fn = lambda x, w: graph(frontend.nn, x, w)
+    plan = hip.render_program(wl.lower_with_table([xs, ws], fn)[0])
+    assert len(plan.launches) <= 2 and "/folded" in plan.launches[0]["schedule"], [l["schedule"] for l in plan.launches]
+    assert all(l["schedule"].startswith(("mfma", "split-k-final")) for l in plan.launches)
+    assert sum(b["elided"] for b in plan.buffers) == 2 and "eh_win_" in plan.launches[0]["source"]
+    rng = RNG(len(name))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.uniform(-1, 1, ws).astype(np.float32)
+    ref, got = both(frontend, fn, [x, w], True)
+    off = realize_on(frontend, "hip", fn, [x, w], fuse=False)
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5 * scale) and np.allclose(got, off, rtol=1e-5, atol=1e-5 * scale)
+
+
 POOLS = {
     # name: (input shape, graph, exact mode, numpy statement or None)
     "max2": ((3, 5, 12, 16), lambda nn, t: nn.max_pool2d(t, (2, 2)), True,
