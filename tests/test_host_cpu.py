@@ -413,6 +413,28 @@ def test_pooling_plan_reads_the_source_through_the_gathers(frontend):
     assert not any(s["schedule"].startswith("window") for s in hb.render_program(shared).launches)
 
 
+def test_convolution_plan_folds_both_gathers(frontend):
+    """A 3x3 convolution as the reference lowers it (gather, gather through the same view,
+    contraction): one MFMA launch whose A loader calls the first gather as a device function;
+    both window buffers are elided.  In exact mode (one gather) and for a pointwise
+    convolution (window loops that run once) the single gather is folded."""
+    from harp_amd import backend as hb, workloads as wl
+    conv = lambda x, w: frontend.nn.conv2d(x, w, None, (1, 1), (1, 1))
+    shapes = [(2, 4, 10, 10), (8, 4, 3, 3)]
+    plan = hb.render_program(wl.lower_with_table(shapes, conv)[0])
+    (l,) = plan.launches
+    assert l["schedule"].startswith("mfma32x32x2(") and "A:m/folded" in l["schedule"] and len(l["args"]) == 3
+    assert sum(b["elided"] for b in plan.buffers) == 2
+    assert "__device__ __forceinline__ float eh_win_" in l["source"] and "? eh_win_" in l["source"]
+    assert len(hb.compile_source(l["source"])) > 1000
+    assert len(hb.render_program(wl.lower_with_table(shapes, conv)[0], {"gemm_fold": 0}).launches) == 3
+    with frontend.exact_mode():
+        exact = hb.render_program(wl.lower_with_table(shapes, conv)[0])
+        point = hb.render_program(wl.lower_with_table([(2, 16, 9, 9), (8, 16, 1, 1)], lambda x, w: frontend.nn.conv2d(x, w))[0])
+    for p in (exact, point):
+        assert len(p.launches) == 1 and "/folded" in p.launches[0]["schedule"] and sum(b["elided"] for b in p.buffers) == 1
+
+
 def test_option_beam_search_on_a_synthetic_cost():
     """The schedule search without a device: suggesters propose neighbours by the schedules in
     the plan, the beam keeps the cheapest states, the search stops when nothing improves."""
