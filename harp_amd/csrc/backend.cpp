@@ -436,15 +436,19 @@ HipProgram::~HipProgram() {
 }
 
 void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
-  if (n != plan_.buffers.size())
-    throw Error("program binds " + std::to_string(plan_.buffers.size()) + " buffers, " + std::to_string(n) + " given");
+  // the caller's table comes first; scratch temps the plan appended may be left out
+  const size_t total = plan_.buffers.size();
+  bool enough = n <= total;
+  for (size_t i = n; enough && i < total; ++i) enough = plan_.buffers[i].role == "temp";
+  if (!enough)
+    throw Error("program binds " + std::to_string(total) + " buffers, " + std::to_string(n) + " given");
   std::lock_guard<std::mutex> lk(mu_);
   dev_->make_current();
-  std::vector<HipBuffer*> bound(n, nullptr);
-  for (size_t i = 0; i < n; ++i) {
+  std::vector<HipBuffer*> bound(total, nullptr);
+  for (size_t i = 0; i < total; ++i) {
     const BufferInfo& bi = plan_.buffers[i];
     if (plan_.elided.count(bi.name)) continue;
-    HipBuffer* b = bufs[i];
+    HipBuffer* b = i < n ? bufs[i] : nullptr;
     if (!b) {
       if (bi.role != "temp")
         throw Error("MissingInput: buffer '" + bi.name + "' (" + bi.role + ") was not provided");

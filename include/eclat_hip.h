@@ -129,8 +129,10 @@ int eh_program_num_buffers(eh_program* prog, int* n);
 int eh_program_buffer(eh_program* prog, int i, const char** name, const char** role, size_t* bytes, int* elided);
 int eh_program_num_launches(eh_program* prog, int* n);
 int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
-/* bufs[i] binds buffer i of the table; NULL is allowed for elided buffers and for temps (the
- * program then keeps its own).  sync != 0 waits for completion (the reference's kernels are
+/* bufs[i] binds buffer i of the table eh_program_buffer reports: the caller's entries in their
+ * order, then scratch temps the plan added (names starting with "eh_").  NULL is allowed for
+ * elided buffers and for temps (the program then keeps its own), and bufs may stop anywhere
+ * after the last input or output.  sync != 0 waits for completion (the reference's kernels are
  * synchronous); sync == 0 only queues the launches on the device's stream. */
 int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,

@@ -1131,6 +1131,33 @@ def test_few_very_long_scan_lines_are_cut_over_workgroups(frontend, hip, name):
     assert np.all(np.abs(ref.ravel() - exact) <= 1e-3 * scale)
 
 
+def test_scratch_temps_of_a_plan_may_be_left_unbound(frontend, hip):
+    """A plan may append scratch temps to the caller's buffer table (the pieces of cut lines);
+    through the C ABI the caller may bind its own entries only, or all of them."""
+    import ctypes
+    from harp_amd import workloads as wl
+    from harp_amd._lib import lib, check
+    shape = (4, 300_000)
+    x = RNG(11).uniform(-1, 1, shape).astype(np.float32)
+    ast, names, out, consts, _ = wl.lower_with_table([shape], lambda t: t.max(1))
+    dev = hip.HipDevice(0)
+    prog = hip.HipProgram(dev, ast, None)
+    assert [b["name"].startswith("eh_rowpart_") for b in prog.buffers] == [False, False, True]
+    xin, res = dev.alloc(x.nbytes), dev.alloc(16)
+    xin.write_array(x)
+    by_name = {names[0]: xin, out: res}
+    for n in (2, 3):
+        arr = (ctypes.c_void_p * n)()
+        for i in range(2):
+            arr[i] = by_name[prog.buffers[i]["name"]]._h
+        check(lib.eh_program_execute(prog._h, arr, n, 1))
+        assert np.array_equal(res.read_array(np.float32), x.max(1))
+    arr = (ctypes.c_void_p * 1)()
+    arr[0] = xin._h
+    with pytest.raises(Exception, match="binds 3 buffers, 1 given"):
+        check(lib.eh_program_execute(prog._h, arr, 1, 1))
+
+
 def test_softmax_over_two_rows_of_millions(frontend, hip):
     """Row softmax whose rows are too long for one workgroup each: every reduce in it is cut."""
     shape = (2, 1 << 22)
