@@ -251,6 +251,11 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
                "algo_bytes": sum(l["algo_bytes"] for l in prog.launches),
                "lowered_kernels": len(plain.args), "launches": len(prog.launches),
                "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
+        from harp_amd import measure
+        gms, gwall = measure.time_replays(dev, prog, sets, k, min(args.warmup, 5))
+        cnn["graph_ms"], cnn["graph_wall_ms"], cnn["wall_ms"] = gms, gwall, wall_ms
+        log(f"[bench] cnn step replayed as one HIP graph: {gms:.3f} ms/step (host wall {gwall:.3f} ms; "
+            f"eager host wall {wall_ms:.3f} ms)")
         log(f"[bench] cnn step (batch {sizes[0]}): {ms:.3f} ms/step -> {sizes[0] / ms * 1e3:.0f} images/s; "
             f"{cnn['lowered_kernels']} kernels -> {cnn['launches']} launches ({cnn['gemm_launches']} MFMA)")
         if not args.no_check:
@@ -366,6 +371,8 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             "steps": cnn["steps"], "algorithmic_bytes": cnn["algo_bytes"],
             "lowered_kernels": cnn["lowered_kernels"], "launches": cnn["launches"],
             "gemm_launches": cnn["gemm_launches"], "loss": cnn.get("loss"),
+            "ms_per_step_hip_graph": round(cnn["graph_ms"], 4),
+            "host_ms_per_step": {"eager": round(cnn["wall_ms"], 4), "hip_graph": round(cnn["graph_wall_ms"], 4)},
             "workload": "CNN 1x28x28: conv3x3(32)+relu+pool, conv3x3(64)+relu+pool, fc 3136-128-10, "
                         "cross-entropy; batch 256 forward + exact backward, plus the SGD update (more than the "
                         "configuration asks for, inside the timed region), one Program"}

@@ -179,6 +179,23 @@ class HipBuffer:
         return b
 
 
+class HipGraph:
+    """The launches of one program run on fixed buffers, replayed as a whole (eh_program_record)."""
+
+    def __init__(self, program, binding):
+        self._h = c_void_p()
+        self._keep = (program, binding)
+        check(lib.eh_program_record(program._h, binding[0], len(program.buffers), byref(self._h)))
+
+    def replay(self, sync: bool = True) -> None:
+        check(lib.eh_graph_replay(self._h, 1 if sync else 0))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib.eh_graph_release(h)
+
+
 class HipProgram:
     """A Program AST compiled for a device (`eh_program_*`)."""
 
@@ -218,6 +235,10 @@ class HipProgram:
 
     def run(self, binding, sync: bool = True) -> None:
         check(lib.eh_program_execute(self._h, binding[0], len(self.buffers), 1 if sync else 0))
+
+    def record(self, binding) -> "HipGraph":
+        """One `run` on this binding captured as a HIP graph; `replay` queues it with one call."""
+        return HipGraph(self, binding)
 
     def execute(self, inputs: Dict[str, HipBuffer]) -> Dict[str, HipBuffer]:
         """Binds inputs by name, allocates the outputs, queues the launches, returns the

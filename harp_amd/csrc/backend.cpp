@@ -435,14 +435,13 @@ HipProgram::~HipProgram() {
     if (b && b->release()) delete b;
 }
 
-void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
+std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n) {
   // the caller's table comes first; scratch temps the plan appended may be left out
   const size_t total = plan_.buffers.size();
   bool enough = n <= total;
   for (size_t i = n; enough && i < total; ++i) enough = plan_.buffers[i].role == "temp";
   if (!enough)
     throw Error("program binds " + std::to_string(total) + " buffers, " + std::to_string(n) + " given");
-  std::lock_guard<std::mutex> lk(mu_);
   dev_->make_current();
   std::vector<HipBuffer*> bound(total, nullptr);
   for (size_t i = 0; i < total; ++i) {
@@ -463,6 +462,10 @@ void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
     }
     bound[i] = b;
   }
+  return bound;
+}
+
+void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
   for (size_t l = 0; l < plan_.launches.size(); ++l) {
     const LaunchSpec& ls = plan_.launches[l];
     std::vector<void*> ptrs;
@@ -478,6 +481,68 @@ void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
     }
     kernels_[l]->launch(ls.grid, ls.block, ls.lds_bytes, ptrs);
   }
+}
+
+void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
+  std::lock_guard<std::mutex> lk(mu_);
+  launch_all(bind(bufs, n));
+  if (sync) dev_->synchronize();
+}
+
+// ---------------------------------------------------------------------------------------------
+// HipGraph: the launches of one execute, captured once on fixed buffers and replayed as a whole
+// ---------------------------------------------------------------------------------------------
+
+HipGraph::HipGraph(HipProgram* prog, HipBuffer* const* bufs, size_t n) : dev_(prog->device()) {
+  std::lock_guard<std::mutex> lk(prog->mu_);
+  // binding allocates missing temps: all of it happens before the capture starts, the capture
+  // itself records kernel launches only (no memset or copy nodes)
+  std::vector<HipBuffer*> bound = prog->bind(bufs, n);
+  launches_ = prog->plan().launches.size();
+  kernels_ = prog->kernels_;
+  // the program's own temps are shared with it by reference count; the caller's buffers are kept
+  // alive by whoever owns their handles
+  for (size_t i = 0; i < bound.size(); ++i)
+    if (bound[i] && (i >= n || !bufs[i])) {
+      bound[i]->retain();
+      held_.push_back(bound[i]);
+    }
+  hipGraph_t graph = nullptr;
+  try {
+    check(hipStreamBeginCapture(dev_->stream(), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    try {
+      prog->launch_all(bound);
+    } catch (...) {
+      (void)hipStreamEndCapture(dev_->stream(), &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      throw;
+    }
+    check(hipStreamEndCapture(dev_->stream(), &graph), "hipStreamEndCapture");
+    hipError_t e = hipGraphInstantiate(&exec_, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    check(e, "hipGraphInstantiate");
+  } catch (...) {
+    drop();
+    throw;
+  }
+}
+
+void HipGraph::drop() {
+  for (HipBuffer* b : held_)
+    if (b->release()) delete b;
+  held_.clear();
+}
+
+HipGraph::~HipGraph() {
+  (void)hipSetDevice(dev_->index());
+  (void)hipStreamSynchronize(dev_->stream());
+  if (exec_) (void)hipGraphExecDestroy(exec_);
+  drop();
+}
+
+void HipGraph::replay(bool sync) {
+  dev_->make_current();
+  check(hipGraphLaunch(exec_, dev_->stream()), "hipGraphLaunch");
   if (sync) dev_->synchronize();
 }
 

@@ -140,12 +140,36 @@ class HipProgram {
   HipDevice* device() const { return dev_; }
 
  private:
+  friend class HipGraph;
+  std::vector<HipBuffer*> bind(HipBuffer* const* bufs, size_t n);   // checks sizes, allocates missing temps
+  void launch_all(const std::vector<HipBuffer*>& bound);            // queues every launch on the stream
   HipDevice* dev_;
   ProgramPlan plan_;
   std::vector<std::shared_ptr<HipKernel>> kernels_;
   std::map<std::string, size_t> index_;          // buffer name -> table index
   std::vector<HipBuffer*> temps_;                // owned, by table index (nullptr if unused)
   std::mutex mu_;
+};
+
+// One execute of a program on fixed buffers, captured from the device's stream as a HIP graph of
+// kernel nodes: a replay queues all launches with one call.  Holds a reference to the program's
+// temps and code objects, so it may outlive the program; the caller keeps its own buffers alive.
+class HipGraph {
+ public:
+  HipGraph(HipProgram* prog, HipBuffer* const* bufs, size_t n);
+  ~HipGraph();
+  HipGraph(const HipGraph&) = delete;
+  HipGraph& operator=(const HipGraph&) = delete;
+  void replay(bool sync);
+  size_t launches() const { return launches_; }
+
+ private:
+  void drop();
+  HipDevice* dev_;
+  hipGraphExec_t exec_ = nullptr;
+  std::vector<HipBuffer*> held_;                 // program temps, by reference count
+  std::vector<std::shared_ptr<HipKernel>> kernels_;
+  size_t launches_ = 0;
 };
 
 GenOptions parse_options(const char* text);       // "key=value,key=value" -> GenOptions

@@ -4,6 +4,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <memory>
 #include <string>
 
 #include "../../include/eclat_hip.h"
@@ -25,6 +26,15 @@ struct eh_program {
 };
 struct eh_plan {
   ProgramPlan plan;
+};
+struct eh_graph {
+  std::unique_ptr<HipGraph> graph;
+  std::vector<eh_buffer*> held;          // the caller's buffers, one reference each
+  ~eh_graph() {
+    graph.reset();                       // waits for queued replays before the buffers may go
+    for (eh_buffer* b : held)
+      if (b->buf.release()) delete b;
+  }
 };
 struct eh_module {
   HipDevice* dev;
@@ -319,6 +329,32 @@ int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int
     for (int i = 0; i < n_bufs; ++i) v[static_cast<size_t>(i)] = bufs[i] ? &bufs[i]->buf : nullptr;
     prog->prog.execute(v.data(), v.size(), sync != 0);
   });
+}
+
+int eh_program_record(eh_program* prog, eh_buffer* const* bufs, int n_bufs, eh_graph** out) {
+  REQUIRE(prog && out && (bufs || n_bufs == 0) && n_bufs >= 0, "program, bufs or out is NULL");
+  return guard([&] {
+    std::vector<HipBuffer*> v(static_cast<size_t>(n_bufs), nullptr);
+    for (int i = 0; i < n_bufs; ++i) v[static_cast<size_t>(i)] = bufs[i] ? &bufs[i]->buf : nullptr;
+    std::unique_ptr<eh_graph> g(new eh_graph());
+    g->graph.reset(new HipGraph(&prog->prog, v.data(), v.size()));
+    for (int i = 0; i < n_bufs; ++i)
+      if (bufs[i]) {
+        bufs[i]->buf.retain();
+        g->held.push_back(bufs[i]);
+      }
+    *out = g.release();
+  });
+}
+
+int eh_graph_replay(eh_graph* graph, int sync) {
+  REQUIRE(graph, "graph is NULL");
+  return guard([&] { graph->graph->replay(sync != 0); });
+}
+
+int eh_graph_release(eh_graph* graph) {
+  REQUIRE(graph, "graph is NULL");
+  return guard([&] { delete graph; });
 }
 
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs, eh_buffer* const* outputs,

@@ -51,3 +51,21 @@ def time_steps(dev, prog, sets, steps, warmup):
     dev.sync()
     wall = (time.perf_counter() - t0) * 1e3
     return e0.elapsed_ms(e1) / steps, wall / steps
+
+
+def time_replays(dev, prog, sets, steps, warmup):
+    """As `time_steps`, with each binding recorded once as a HIP graph and a step = one replay."""
+    graphs = [prog.record(b) for b, _ in sets]
+    for i in range(warmup):
+        graphs[i % len(graphs)].replay(sync=False)
+    dev.sync()
+    e0, e1 = hb.Event(dev), hb.Event(dev)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        graphs[i % len(graphs)].replay(sync=False)
+    e1.record()
+    e1.sync()
+    dev.sync()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_ms(e1) / steps, wall / steps

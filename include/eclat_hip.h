@@ -33,6 +33,7 @@ extern "C" {
 typedef struct eh_device eh_device;
 typedef struct eh_buffer eh_buffer;
 typedef struct eh_program eh_program;   /* one or more launches compiled from a Program AST */
+typedef struct eh_graph eh_graph;       /* one execute of a program on fixed buffers, replayable */
 typedef struct eh_plan eh_plan;         /* rendered sources + dispatch, no device involved */
 typedef struct eh_event eh_event;
 typedef struct eh_module eh_module;     /* one entry point of a loaded code object */
@@ -137,6 +138,15 @@ int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
 int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,
                                   eh_buffer* const* outputs, int n_outputs, int sync);
+/* The launches of one eh_program_execute(prog, bufs, n_bufs, .) captured as a HIP graph of kernel
+ * nodes and replayed with one call: for callers that run the same program on the same buffers
+ * many times (the training loop of examples/function_fitting/main.rs:60-120 runs one compiled
+ * step per iteration).  The reference has no counterpart; results are those of eh_program_execute.
+ * The graph holds references to the bound buffers, so they may be released while it lives; their
+ * CONTENTS are read at replay time.  Replays are ordered on the device's stream like launches. */
+int eh_program_record(eh_program* prog, eh_buffer* const* bufs, int n_bufs, eh_graph** out);
+int eh_graph_replay(eh_graph* graph, int sync);
+int eh_graph_release(eh_graph* graph);
 /* Kernel::get_binary / BackendRegistry::compile_from_binary (src/backend/traits.rs:576-586,
  * src/backend/device.rs:161-170): the gfx950 code object of one launch. */
 int eh_program_binary(eh_program* prog, int launch, const void** blob, size_t* len);
