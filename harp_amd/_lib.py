@@ -85,6 +85,7 @@ _SIGS = {
     "eh_program_num_launches": ([_P, POINTER(c_int)], c_int),
     "eh_program_launch": ([_P, c_int, POINTER(LaunchInfo)], c_int),
     "eh_program_execute": ([_P, POINTER(_P), c_int, c_int], c_int),
+    "eh_program_execute_static": ([_P, POINTER(_P), c_int, c_int], c_int),
     "eh_program_record": ([_P, POINTER(_P), c_int, POINTER(_P)], c_int),
     "eh_graph_replay": ([_P, c_int], c_int),
     "eh_graph_release": ([_P], c_int),

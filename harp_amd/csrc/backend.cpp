@@ -1,4 +1,5 @@
 #include "backend.hpp"
+#include "static_scratch.hpp"
 
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
@@ -210,6 +211,18 @@ HipDevice::HipDevice(int index) : index_(index) {
   profile_.l2_bytes = p.l2CacheSize;
   check(hipStreamCreate(&stream_), "hipStreamCreate");
   pool_limit_ = std::getenv("ECLAT_HIP_NO_POOL") ? 0 : profile_.global_memory_size / 4;
+  // resolved here, with this device current, so that the entry point which must not allocate
+  // never triggers the load of the library's code object itself
+  try {
+    static_scratch_ = static_scratch_ptr(index_);
+  } catch (const Error& e) {
+    static_scratch_error_ = e.what();
+  }
+}
+
+void* HipDevice::static_scratch() const {
+  if (!static_scratch_) throw Error("the static scratch block is not available: " + static_scratch_error_);
+  return static_scratch_;
 }
 
 HipDevice::~HipDevice() {
@@ -466,18 +479,24 @@ std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n) {
 }
 
 void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
+  std::vector<Span> spans(bound.size());
+  for (size_t i = 0; i < bound.size(); ++i)
+    if (bound[i]) spans[i] = {bound[i]->device_ptr(), bound[i]->byte_len(), true};
+  launch_spans(spans);
+}
+
+void HipProgram::launch_spans(const std::vector<Span>& bound) {
   for (size_t l = 0; l < plan_.launches.size(); ++l) {
     const LaunchSpec& ls = plan_.launches[l];
     std::vector<void*> ptrs;
     for (size_t a = 0; a < ls.arg_bufs.size(); ++a) {
-      size_t bi = index_.at(ls.arg_bufs[a]);
-      HipBuffer* b = bound[bi];
-      if (!b) throw Error("launch '" + ls.entry + "' needs buffer '" + ls.arg_bufs[a] + "', which is not bound");
-      if (a < ls.arg_min_bytes.size() && b->byte_len() < ls.arg_min_bytes[a])
+      const Span& b = bound[index_.at(ls.arg_bufs[a])];
+      if (!b.bound) throw Error("launch '" + ls.entry + "' needs buffer '" + ls.arg_bufs[a] + "', which is not bound");
+      if (a < ls.arg_min_bytes.size() && b.bytes < ls.arg_min_bytes[a])
         throw Error("Buffer size mismatch: '" + ls.arg_bufs[a] + "' needs at least " +
                     std::to_string(ls.arg_min_bytes[a]) + " bytes for '" + ls.entry + "', has " +
-                    std::to_string(b->byte_len()));
-      ptrs.push_back(b->device_ptr());
+                    std::to_string(b.bytes));
+      ptrs.push_back(b.ptr);
     }
     kernels_[l]->launch(ls.grid, ls.block, ls.lds_bytes, ptrs);
   }
@@ -486,6 +505,53 @@ void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
 void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
   std::lock_guard<std::mutex> lk(mu_);
   launch_all(bind(bufs, n));
+  if (sync) dev_->synchronize();
+}
+
+// Scratch temps the plan appended (names starting with "eh_") sit behind the caller's table.
+static bool plan_scratch(const ProgramPlan& plan, size_t i) {
+  return plan.buffers[i].role == "temp" && plan.buffers[i].name.rfind("eh_", 0) == 0 && !plan.elided.count(plan.buffers[i].name);
+}
+
+size_t HipProgram::static_scratch_needed() const {
+  size_t need = 0;
+  for (size_t i = 0; i < plan_.buffers.size(); ++i)
+    if (plan_scratch(plan_, i))
+      need += (plan_.buffers[i].bytes() + kStaticScratchAlign - 1) / kStaticScratchAlign * kStaticScratchAlign;
+  return need;
+}
+
+void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
+  std::lock_guard<std::mutex> lk(mu_);
+  const size_t total = plan_.buffers.size();
+  if (n > total) throw Error("program binds " + std::to_string(total) + " buffers, " + std::to_string(n) + " given");
+  const size_t need = static_scratch_needed();
+  if (need > kStaticScratchBytes)
+    throw Error("Buffer size mismatch: the program's scratch buffers need " + std::to_string(need) +
+                " bytes, the static scratch block holds " + std::to_string(kStaticScratchBytes) +
+                "; use eh_program_execute, which allocates them");
+  dev_->make_current();
+  char* block = need ? static_cast<char*>(dev_->static_scratch()) : nullptr;
+  std::vector<Span> bound(total);
+  size_t off = 0;
+  for (size_t i = 0; i < total; ++i) {
+    const BufferInfo& bi = plan_.buffers[i];
+    if (plan_.elided.count(bi.name)) continue;
+    if (plan_scratch(plan_, i) && !(i < n && bufs[i])) {
+      bound[i] = {block + off, bi.bytes(), true};
+      off += (bi.bytes() + kStaticScratchAlign - 1) / kStaticScratchAlign * kStaticScratchAlign;
+      continue;
+    }
+    HipBuffer* b = i < n ? bufs[i] : nullptr;
+    if (!b)
+      throw Error("MissingInput: buffer '" + bi.name + "' (" + bi.role + ") was not provided; this entry point allocates nothing");
+    if (b->device() != dev_) throw Error("buffer '" + bi.name + "' lives on another device");
+    if (bi.shape_known && b->byte_len() < bi.bytes())
+      throw Error("Buffer size mismatch: '" + bi.name + "' needs " + std::to_string(bi.bytes()) + " bytes, has " +
+                  std::to_string(b->byte_len()));
+    bound[i] = {b->device_ptr(), b->byte_len(), true};
+  }
+  launch_spans(bound);
   if (sync) dev_->synchronize();
 }
 

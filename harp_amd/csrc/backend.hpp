@@ -73,6 +73,9 @@ class HipDevice {
   void release(void* ptr, size_t bytes);
   void trim();                         // returns every kept block to the driver
   size_t pooled_bytes() const { return pooled_bytes_; }
+  // This device's static scratch block (static_scratch.hpp), resolved when the device was
+  // opened; throws when that failed.
+  void* static_scratch() const;
 
  private:
   int index_;
@@ -81,6 +84,8 @@ class HipDevice {
   std::mutex pool_mu_;
   std::multimap<size_t, void*> pool_;  // size -> free block
   size_t pooled_bytes_ = 0, pool_limit_ = 0;
+  void* static_scratch_ = nullptr;
+  std::string static_scratch_error_;
 };
 
 class HipBuffer {
@@ -136,6 +141,12 @@ class HipProgram {
   void execute(HipBuffer* const* bufs, size_t n, bool sync);
   // Positional form (Kernel::execute): immutable pointer parameters, then mutable ones.
   void execute_positional(HipBuffer* const* inputs, size_t n_in, HipBuffer* const* outputs, size_t n_out, bool sync);
+  // execute() without any device allocation: every buffer of the caller's table that reaches
+  // memory must be given, and the scratch temps the plan appended (partial sums of split
+  // reductions and contractions, chunk totals of scans) are placed in the device's static
+  // scratch block instead of buffers of their own.  Throws when they do not fit.
+  void execute_static(HipBuffer* const* bufs, size_t n, bool sync);
+  size_t static_scratch_needed() const;          // bytes of the block execute_static() would use
   const HipKernel& kernel(size_t launch) const { return *kernels_.at(launch); }
   HipDevice* device() const { return dev_; }
 
@@ -143,6 +154,12 @@ class HipProgram {
   friend class HipGraph;
   std::vector<HipBuffer*> bind(HipBuffer* const* bufs, size_t n);   // checks sizes, allocates missing temps
   void launch_all(const std::vector<HipBuffer*>& bound);            // queues every launch on the stream
+  struct Span {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    bool bound = false;
+  };
+  void launch_spans(const std::vector<Span>& bound);                // the same, over plain address ranges
   HipDevice* dev_;
   ProgramPlan plan_;
   std::vector<std::shared_ptr<HipKernel>> kernels_;

@@ -9,6 +9,7 @@
 
 #include "../../include/eclat_hip.h"
 #include "backend.hpp"
+#include "static_scratch.hpp"
 
 using namespace eh;
 
@@ -328,6 +329,15 @@ int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int
     std::vector<HipBuffer*> v(static_cast<size_t>(n_bufs), nullptr);
     for (int i = 0; i < n_bufs; ++i) v[static_cast<size_t>(i)] = bufs[i] ? &bufs[i]->buf : nullptr;
     prog->prog.execute(v.data(), v.size(), sync != 0);
+  });
+}
+
+int eh_program_execute_static(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync) {
+  REQUIRE(prog && (bufs || n_bufs == 0) && n_bufs >= 0, "program or bufs is NULL");
+  return guard([&] {
+    std::vector<HipBuffer*> v(static_cast<size_t>(n_bufs), nullptr);
+    for (int i = 0; i < n_bufs; ++i) v[static_cast<size_t>(i)] = bufs[i] ? &bufs[i]->buf : nullptr;
+    prog->prog.execute_static(v.data(), v.size(), sync != 0);
   });
 }
 

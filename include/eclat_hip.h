@@ -138,6 +138,21 @@ int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
 int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,
                                   eh_buffer* const* outputs, int n_outputs, int sync);
+/* eh_program_execute for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * It calls no hipMalloc or hipFree: the scratch temps the plan appended to the buffer table (names
+ * starting with "eh_": partial results of split reductions and split-K contractions, chunk totals
+ * of scans) are placed, each at a 256-byte boundary, in one static block of device memory of
+ * EH_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends;
+ * every other buffer that reaches memory (inputs, outputs and the caller's own temps) must be
+ * given.  A program whose scratch temps do not fit fails with EH_ERR_SIZE and launches nothing.
+ * All calls on one device share that device's block, which keeps the previous call's contents
+ * (no kernel relies on them: every scratch element is written before it is read), so calls that
+ * overlap on one device race: queue them on the device's stream one after the other, as this
+ * library does, and do not run two host threads through this entry point on one device at once
+ * with sync == 0 on different programs unless both finish in stream order. */
+#define EH_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+int eh_program_execute_static(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 /* The launches of one eh_program_execute(prog, bufs, n_bufs, .) captured as a HIP graph of kernel
  * nodes and replayed with one call: for callers that run the same program on the same buffers
  * many times (the training loop of examples/function_fitting/main.rs:60-120 runs one compiled
