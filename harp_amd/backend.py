@@ -78,6 +78,16 @@ def render_program(ast, options=None) -> Plan:
     return Plan(ast, options)
 
 
+def normalize_ast(ast) -> str:
+    """AST text of `ast` with the reference optimiser's rewrites undone (`eh_normalize_ast`)."""
+    out = c_void_p()
+    check(lib.eh_normalize_ast(_sexpr(ast), byref(out)))
+    try:
+        return ctypes.string_at(out).decode()
+    finally:
+        lib.eh_free(out)
+
+
 def compile_source(source: str, arch: str = "gfx950") -> bytes:
     """hiprtc: HIP C -> code object.  Works without a GPU."""
     blob, n = c_void_p(), c_size_t()

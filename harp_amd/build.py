@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libeclat_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
-SOURCES = ["ast.cpp", "analysis.cpp", "codegen.cpp", "gemm.cpp", "backend.cpp", "capi.cpp"]
+SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "gemm.cpp", "backend.cpp", "capi.cpp"]
 # compiled as HIP for gfx950: holds the library's one statically allocated device array
 DEVICE_SOURCES = ["static_scratch.hip"]
 TEMPLATES = ["kernels/gemm_f32_mfma.hip"]

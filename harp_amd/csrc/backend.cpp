@@ -411,6 +411,8 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_dma") o.gemm_dma = as_int() != 0;
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;
     else if (k == "nontemporal") o.nontemporal = as_int();
+    else if (k == "normalize") o.normalize = as_int() != 0;
+    else if (k == "allow_serial") o.allow_serial = as_int() != 0;
     else throw Error("unknown option '" + k + "'");
   }
   if (o.flat_block < 64 || o.flat_block > 1024 || (o.flat_block & (o.flat_block - 1)))

@@ -9,6 +9,7 @@
 
 #include "../../include/eclat_hip.h"
 #include "backend.hpp"
+#include "normalize.hpp"
 #include "static_scratch.hpp"
 
 using namespace eh;
@@ -222,6 +223,28 @@ int eh_render_program(const char* ast_text, const char* options, eh_plan** out) 
       throw;
     }
     *out = p;
+  });
+}
+
+int eh_normalize_ast(const char* ast_text, char** out_text) {
+  REQUIRE(ast_text && out_text, "ast_text or out_text is NULL");
+  return guard([&] {
+    NodePtr ast = parse_ast(ast_text);
+    std::string text;
+    if (ast->op == Op::Kernel) {
+      text = to_text(*normalize_kernel(ast));
+    } else if (ast->op == Op::Program) {
+      auto p = std::make_shared<Node>(*ast);
+      for (auto& f : p->args)
+        if (f->op == Op::Kernel) f = normalize_kernel(f);
+      text = to_text(*p);
+    } else {
+      throw Error("expected a program or kernel node");
+    }
+    char* buf = static_cast<char*>(std::malloc(text.size() + 1));
+    if (!buf) throw std::bad_alloc();
+    std::memcpy(buf, text.c_str(), text.size() + 1);
+    *out_text = buf;
   });
 }
 

@@ -7,6 +7,7 @@
 #include <sstream>
 
 #include "gemm.hpp"
+#include "normalize.hpp"
 
 namespace eh {
 
@@ -365,6 +366,20 @@ std::string render_expr_text(const Node& e) {
   return er.expr(e);
 }
 
+namespace {
+// A kernel (or one of its loop nests) that is about to run in a single work-item: fine for the
+// few statements of a short scan, hopeless for millions of iterations.  Refused rather than
+// launched, unless the caller asked for it.
+void refuse_long_serial(const std::string& kernel, const Node& body, const GenOptions& opt) {
+  const double limit = 131072;
+  const double n = serial_iterations(body);
+  if (n <= limit || opt.allow_serial) return;
+  throw Error("kernel '" + kernel + "' has a form no schedule of this backend recognises and would run its " +
+              std::to_string(static_cast<long long>(n)) +
+              " loop iterations in one work-item: not supported (compile with allow_serial=1 to run it anyway)");
+}
+}  // namespace
+
 LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
   if (k.op != Op::Kernel) throw Error("expected a kernel node");
   LaunchSpec ls;
@@ -404,6 +419,8 @@ LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
     ls.block[i] = static_cast<unsigned>(t);
     ls.grid[i] = static_cast<unsigned>(g);   // the AST's grid size counts workgroups
   }
+  if (1ull * ls.grid[0] * ls.grid[1] * ls.grid[2] * ls.block[0] * ls.block[1] * ls.block[2] == 1)
+    refuse_long_serial(k.name, *k.args[0], opt);
   return ls;
 }
 
@@ -820,6 +837,7 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + (colliding ? ",atomics)" : ")");
       any_parallel = true;
     } else {
+      refuse_long_serial(k.name, *tops[t], opt);
       os << "extern \"C\" __global__ void " << ls.entry << "(" << sig << ") {\n" << sr.stmt(*tops[t]) << "}\n";
       ls.schedule = "as-written";
     }
@@ -1372,9 +1390,21 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   }
   if (kernels.empty()) throw Error("program holds no kernel");
 
+  std::vector<NodePtr> rewritten;          // owns the kernels that replace given ones
+  // what the reference's AST optimiser did to the lowered loop nests is undone first
+  if (opt.normalize)
+    for (size_t q = 0; q < kernels.size(); ++q)
+      for (const auto& f : program.args)
+        if (f.get() == kernels[q]) {
+          NodePtr nk = normalize_kernel(f);
+          if (nk != f) {
+            rewritten.push_back(nk);
+            kernels[q] = nk.get();
+          }
+        }
+
   // buffer table: given, or synthesised from the kernels' pointer parameters
   plan.buffers = program.buffers;
-  std::vector<NodePtr> rewritten;          // owns the kernels that replace split ones
   if (!plan.buffers.empty() && opt.fuse) {
     std::vector<const Node*> out;
     for (const Node* k : kernels) {

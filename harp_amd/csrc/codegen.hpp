@@ -35,6 +35,8 @@ struct GenOptions {
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
   int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores
+  bool normalize = true;     // undo the reference optimiser's rewrites (shifts, tiling, unrolling) before planning
+  bool allow_serial = false; // let a kernel no schedule recognises run in one work-item however long its loops are
 };
 
 struct LaunchSpec {

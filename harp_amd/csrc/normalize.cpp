@@ -1,0 +1,500 @@
+#include "normalize.hpp"
+
+#include <algorithm>
+#include <set>
+
+#include "analysis.hpp"
+
+namespace eh {
+
+NodePtr substitute_vars(const NodePtr& n, const std::map<std::string, NodePtr>& m) {
+  if (n->op == Op::Var) {
+    auto it = m.find(n->name);
+    return it == m.end() ? n : it->second;
+  }
+  bool changed = false;
+  std::vector<NodePtr> args;
+  args.reserve(n->args.size());
+  for (const auto& a : n->args) {
+    NodePtr r = substitute_vars(a, m);
+    changed = changed || r != a;
+    args.push_back(std::move(r));
+  }
+  if (!changed) return n;
+  auto c = std::make_shared<Node>(*n);
+  c->args = std::move(args);
+  return c;
+}
+
+namespace {
+
+bool int_const(const Node& n, int64_t* v) {
+  if (n.op != Op::Const || n.dtype.is_float()) return false;
+  *v = n.ival;
+  return true;
+}
+
+bool int_type(const DType& d) {
+  switch (d.ty) {
+    case Ty::I8: case Ty::I16: case Ty::I32: case Ty::I64: case Ty::U8: case Ty::U16: case Ty::U32: case Ty::U64:
+    case Ty::Int:
+      return true;
+    default:
+      return false;
+  }
+}
+
+NodePtr with_args(const Node& n, std::vector<NodePtr> args) {
+  auto c = std::make_shared<Node>(n);
+  c->args = std::move(args);
+  return c;
+}
+
+NodePtr int_like(const Node& like, int64_t v) {
+  auto c = std::make_shared<Node>(Op::Const);
+  c->dtype = like.dtype;
+  c->ival = v;
+  return c;
+}
+
+bool mentions(const Node& n, const std::string& var) {
+  if ((n.op == Op::Var || n.op == Op::Assign) && n.name == var) return true;
+  for (const auto& a : n.args)
+    if (mentions(*a, var)) return true;
+  return false;
+}
+
+bool assigns(const Node& n, const std::string& var) {
+  if ((n.op == Op::Assign || n.op == Op::Range) && n.name == var) return true;
+  for (const auto& a : n.args)
+    if (assigns(*a, var)) return true;
+  return false;
+}
+
+// c + sum(coef * var), variables in name order
+NodePtr affine_to_node(const Affine& a) {
+  NodePtr sum;
+  for (const auto& kv : a.coef) {
+    if (kv.second == 0) continue;
+    NodePtr t = kv.second == 1 ? make_var(kv.first) : make(Op::Mul, {make_var(kv.first), make_i64(kv.second)});
+    sum = sum ? make(Op::Add, {sum, t}) : t;
+  }
+  if (!sum) return make_i64(a.c);
+  return a.c == 0 ? sum : make(Op::Add, {sum, make_i64(a.c)});
+}
+
+// Shifts by a constant back to multiplications (the reference only ever produces left shifts,
+// from `x * 2^n`), and integer constant subtrees folded.
+NodePtr fold_expr(const NodePtr& n) {
+  if (n->args.empty()) return n;
+  bool changed = false;
+  std::vector<NodePtr> args;
+  args.reserve(n->args.size());
+  for (const auto& a : n->args) {
+    NodePtr r = fold_expr(a);
+    changed = changed || r != a;
+    args.push_back(std::move(r));
+  }
+  NodePtr cur = changed ? with_args(*n, args) : n;
+  int64_t a = 0, b = 0;
+  if (cur->op == Op::Shl && cur->args.size() == 2 && int_const(*cur->args[1], &b) && b >= 0 && b < 62) {
+    if (int_const(*cur->args[0], &a)) return int_like(*cur->args[0], a * (int64_t{1} << b));
+    return make(Op::Mul, {cur->args[0], int_like(*cur->args[1], int64_t{1} << b)});
+  }
+  if (cur->args.size() == 2 && int_const(*cur->args[0], &a) && int_const(*cur->args[1], &b)) {
+    switch (cur->op) {
+      case Op::Add: return int_like(*cur->args[0], a + b);
+      case Op::Mul: return int_like(*cur->args[0], a * b);
+      case Op::Max: return int_like(*cur->args[0], std::max(a, b));
+      case Op::Idiv: if (b != 0) return int_like(*cur->args[0], a / b); break;
+      case Op::Rem: if (b != 0) return int_like(*cur->args[0], a % b); break;
+      default: break;
+    }
+  }
+  return cur;
+}
+
+bool is_empty_stmt(const Node& n) {
+  if (n.op == Op::Block) return n.args.empty();
+  if (n.op == Op::Range) {
+    int64_t s, e;
+    return int_const(*n.args[0], &s) && int_const(*n.args[2], &e) && s >= e;
+  }
+  return false;
+}
+
+NodePtr make_block(std::vector<NodePtr> stmts, std::vector<std::pair<std::string, DType>> decls) {
+  if (decls.empty() && stmts.size() == 1) return stmts[0];
+  auto b = std::make_shared<Node>(Op::Block);
+  b->args = std::move(stmts);
+  b->decls = std::move(decls);
+  return b;
+}
+
+NodePtr make_loop(const Node& like, const std::string& var, NodePtr start, NodePtr step, NodePtr stop, NodePtr body) {
+  auto r = std::make_shared<Node>(Op::Range);
+  r->name = var;
+  r->parallel = like.parallel;
+  r->args = {std::move(start), std::move(step), std::move(stop), std::move(body)};
+  return r;
+}
+
+struct Normalizer {
+  std::set<std::string> int_vars;     // loop variables and integer block variables of the kernel
+  int fresh = 0;
+
+  void collect_int_vars(const Node& n) {
+    if (n.op == Op::Range) int_vars.insert(n.name);
+    for (const auto& d : n.decls)
+      if (int_type(d.second)) int_vars.insert(d.first);
+    for (const auto& p : n.params)
+      if (p.kind != VarKind::Normal || int_type(p.dtype)) int_vars.insert(p.name);
+    for (const auto& a : n.args) collect_int_vars(*a);
+  }
+
+  // affine over integer variables only
+  std::optional<Affine> int_affine(const Node& e) const {
+    auto a = affine_of(e);
+    if (!a) return std::nullopt;
+    for (const auto& kv : a->coef)
+      if (!int_vars.count(kv.first)) return std::nullopt;
+    return a;
+  }
+
+  // ---- rolling a block of repeated statements back into a loop ------------------------------
+
+  // One template for `copies` (the same statement or expression in each repetition) over the new
+  // loop variable `u`, or null.  Integer positions are compared by their affine forms, so that a
+  // copy the reference's simplifier rewrote (`0 * 1024 + j` to `j`) still matches its siblings.
+  NodePtr unify(const std::vector<NodePtr>& copies, const std::string& u, bool int_pos) const {
+    const Node& f = *copies[0];
+    bool same = true;
+    const std::string text0 = to_text(f);
+    for (size_t t = 1; t < copies.size() && same; ++t) same = copies[t] == copies[0] || to_text(*copies[t]) == text0;
+    if (same) return copies[0];
+    if (int_pos) {
+      std::vector<Affine> affs;
+      for (const auto& c : copies) {
+        auto a = int_affine(*c);
+        if (!a) break;
+        affs.push_back(*a);
+      }
+      if (affs.size() == copies.size()) {
+        const int64_t d = affs[1].c - affs[0].c;
+        for (size_t t = 0; t < affs.size(); ++t)
+          if (affs[t].coef != affs[0].coef || affs[t].c != affs[0].c + d * static_cast<int64_t>(t)) return nullptr;
+        Affine r = affs[0];
+        if (d != 0) r.coef[u] += d;
+        return affine_to_node(r);
+      }
+    }
+    for (const auto& c : copies) {
+      if (c->op != f.op || c->name != f.name || !(c->dtype == f.dtype) || c->count != f.count ||
+          c->parallel != f.parallel || c->args.size() != f.args.size() || c->decls.size() != f.decls.size())
+        return nullptr;
+      for (size_t i = 0; i < f.decls.size(); ++i)
+        if (c->decls[i].first != f.decls[i].first || !(c->decls[i].second == f.decls[i].second)) return nullptr;
+    }
+    if (f.op == Op::Const) {
+      if (f.dtype.is_float()) return nullptr;            // equal floats were caught by the text comparison
+      const int64_t d = copies[1]->ival - f.ival;
+      for (size_t t = 0; t < copies.size(); ++t)
+        if (copies[t]->ival != f.ival + d * static_cast<int64_t>(t)) return nullptr;
+      return make(Op::Add, {copies[0], make(Op::Mul, {make_var(u), int_like(f, d)})});
+    }
+    if (f.args.empty()) return nullptr;
+    std::vector<NodePtr> args;
+    for (size_t i = 0; i < f.args.size(); ++i) {
+      std::vector<NodePtr> sub;
+      for (const auto& c : copies) sub.push_back(c->args[i]);
+      bool pos = int_pos;
+      switch (f.op) {
+        case Op::Load: case Op::Store: case Op::AtomicAdd: case Op::AtomicMax: case Op::SharedLoad: case Op::SharedStore:
+          pos = i == 1;
+          break;
+        case Op::Assign: pos = int_vars.count(f.name) > 0; break;
+        case Op::Range: pos = i < 3; break;
+        case Op::Block: case Op::If: case Op::Select: pos = false; break;
+        case Op::Lt: pos = true; break;                    // guards compare indices
+        default: break;
+      }
+      NodePtr r = unify(sub, u, pos);
+      if (!r) return nullptr;
+      args.push_back(std::move(r));
+    }
+    return with_args(f, std::move(args));
+  }
+
+  // A block whose statements are k >= 2 repetitions of p statements that differ only by integers
+  // in arithmetic progression (what full unrolling leaves, src/opt/ast/transforms.rs:238-361)
+  // becomes `for u in 0..k { the p statements over u }`.  Variables the block declares move into
+  // the loop body, which is sound when every repetition assigns them before it reads them.
+  NodePtr reroll(const std::vector<NodePtr>& stmts, const std::vector<std::pair<std::string, DType>>& decls) {
+    const size_t n = stmts.size();
+    for (size_t p = 1; p * 2 <= n; ++p) {
+      if (n % p) continue;
+      const size_t k = n / p;
+      bool shape = true;
+      for (size_t j = 0; j < n && shape; ++j) shape = stmts[j]->op == stmts[j % p]->op;
+      if (!shape) continue;
+      bool decls_ok = true;
+      for (const auto& d : decls) {
+        for (size_t j = 0; j < p; ++j) {
+          const Node& s = *stmts[j];
+          if (!mentions(s, d.first)) continue;
+          decls_ok = decls_ok && s.op == Op::Assign && s.name == d.first && !mentions(*s.args[0], d.first);
+          break;
+        }
+      }
+      if (!decls_ok) continue;
+      const std::string u = "eh_u" + std::to_string(fresh);
+      std::vector<NodePtr> body;
+      for (size_t j = 0; j < p; ++j) {
+        std::vector<NodePtr> copies;
+        for (size_t t = 0; t < k; ++t) copies.push_back(stmts[t * p + j]);
+        NodePtr tpl = unify(copies, u, false);
+        if (!tpl) break;
+        body.push_back(std::move(tpl));
+      }
+      if (body.size() != p) continue;
+      ++fresh;
+      int_vars.insert(u);
+      Node like(Op::Range);
+      like.parallel = "sequential";
+      return loop(make_loop(like, u, make_i64(0), make_i64(1), make_i64(static_cast<int64_t>(k)), block(body, decls)));
+    }
+    return nullptr;
+  }
+
+  // ---- loops ----------------------------------------------------------------------------------
+
+  // `decls` without `var`; false when it is not declared there
+  static bool drop_decl(std::vector<std::pair<std::string, DType>>* decls, const std::string& var) {
+    for (auto it = decls->begin(); it != decls->end(); ++it)
+      if (it->first == var) {
+        decls->erase(it);
+        return true;
+      }
+    return false;
+  }
+
+  // The loop after every rewrite that applies to it (its body is already normal).
+  NodePtr loop(NodePtr r) {
+    for (;;) {
+      int64_t s = 0, step = 0, e = 0;
+      const bool consts = int_const(*r->args[0], &s) && int_const(*r->args[1], &step) && int_const(*r->args[2], &e);
+      const NodePtr& body = r->args[3];
+      if (!consts || step < 1) return r;
+      // strip-mined pair: for o in s..e step T { for i in 0..T { v = o + i; rest } } -> for v in s..e { rest }
+      // (tile_loop, src/opt/ast/transforms.rs:393-500), or with a guard: for o in 0..G { for i in 0..T {
+      // v = o * T + i; if (v < E) { rest } } } -> for v in 0..E { rest } (tile_loop_with_guard, :520-630)
+      if (body->op == Op::Range) {
+        const Node& in = *body;
+        int64_t is = 0, istep = 0, T = 0;
+        const Node& ib = *in.args[3];
+        if (int_const(*in.args[0], &is) && int_const(*in.args[1], &istep) && int_const(*in.args[2], &T) && is == 0 &&
+            istep == 1 && T >= 1 && ib.op == Op::Block && ib.args.size() >= 2 && ib.args[0]->op == Op::Assign) {
+          const std::string& v = ib.args[0]->name;
+          auto a = int_affine(*ib.args[0]->args[0]);
+          auto decls = ib.decls;
+          bool clean = a && a->c == 0 && a->coef.size() == 2 && a->of(in.name) == 1 && drop_decl(&decls, v);
+          for (size_t q = 1; q < ib.args.size() && clean; ++q)
+            clean = !mentions(*ib.args[q], r->name) && !mentions(*ib.args[q], in.name) && !assigns(*ib.args[q], v);
+          if (clean && a->of(r->name) == 1 && step == T && (e - s) % T == 0) {
+            std::vector<NodePtr> rest(ib.args.begin() + 1, ib.args.end());
+            r = make_loop(*r, v, r->args[0], make_i64(1), r->args[2], block(rest, decls));
+            int_vars.insert(v);
+            continue;
+          }
+          if (clean && a->of(r->name) == T && step == 1 && s == 0 && T >= 2) {
+            const Node& g = *ib.args[1];
+            int64_t E = 0;
+            if (ib.args.size() == 2 && g.op == Op::If && g.args.size() == 2 && g.args[0]->op == Op::Lt &&
+                g.args[0]->args[0]->op == Op::Var && g.args[0]->args[0]->name == v &&
+                int_const(*g.args[0]->args[1], &E) && E <= e * T && E > (e - 1) * T) {
+              r = make_loop(*r, v, make_i64(0), make_i64(1), make_i64(E), block({g.args[1]}, decls));
+              int_vars.insert(v);
+              continue;
+            }
+            bool guarded = false;
+            for (size_t q = 1; q < ib.args.size(); ++q) guarded = guarded || ib.args[q]->op == Op::If;
+            if (!guarded) {
+              std::vector<NodePtr> rest(ib.args.begin() + 1, ib.args.end());
+              r = make_loop(*r, v, make_i64(0), make_i64(1), make_i64(e * T), block(rest, decls));
+              int_vars.insert(v);
+              continue;
+            }
+          }
+        }
+      }
+      // renamed loop variable: for q in s..e { v = q + d; rest } -> for v in s+d..e+d { rest }
+      // (the remainder loop of tile_loop; a rolled-back unrolled loop)
+      if (body->op == Op::Block && body->args.size() >= 2 && body->args[0]->op == Op::Assign && step == 1) {
+        const Node& b = *body;
+        const std::string& v = b.args[0]->name;
+        auto a = int_affine(*b.args[0]->args[0]);
+        auto decls = b.decls;
+        bool clean = a && a->coef.size() == 1 && a->of(r->name) == 1 && drop_decl(&decls, v);
+        for (size_t q = 1; q < b.args.size() && clean; ++q)
+          clean = !mentions(*b.args[q], r->name) && !assigns(*b.args[q], v);
+        if (clean) {
+          std::vector<NodePtr> rest(b.args.begin() + 1, b.args.end());
+          r = make_loop(*r, v, make_i64(s + a->c), make_i64(1), make_i64(e + a->c), block(rest, decls));
+          int_vars.insert(v);
+          continue;
+        }
+      }
+      return r;
+    }
+  }
+
+  // ---- blocks ---------------------------------------------------------------------------------
+
+  NodePtr block(std::vector<NodePtr> stmts, std::vector<std::pair<std::string, DType>> decls) {
+    stmts.erase(std::remove_if(stmts.begin(), stmts.end(), [](const NodePtr& s) { return is_empty_stmt(*s); }),
+                stmts.end());
+    // neighbouring loops over adjoining ranges with the same body are one loop
+    for (size_t j = 0; j + 1 < stmts.size();) {
+      const Node &x = *stmts[j], &y = *stmts[j + 1];
+      int64_t xs, xt, xe, ys, yt, ye;
+      bool join = x.op == Op::Range && y.op == Op::Range && int_const(*x.args[0], &xs) && int_const(*x.args[1], &xt) &&
+                  int_const(*x.args[2], &xe) && int_const(*y.args[0], &ys) && int_const(*y.args[1], &yt) &&
+                  int_const(*y.args[2], &ye) && xt == 1 && yt == 1 && xe == ys && x.parallel == y.parallel;
+      if (join) {
+        NodePtr yb = y.name == x.name ? y.args[3] : substitute_vars(y.args[3], {{y.name, make_var(x.name)}});
+        join = (y.name == x.name || !mentions(*y.args[3], x.name)) && to_text(*yb) == to_text(*x.args[3]);
+      }
+      if (!join) {
+        ++j;
+        continue;
+      }
+      stmts[j] = make_loop(x, x.name, x.args[0], x.args[1], y.args[2], x.args[3]);
+      stmts.erase(stmts.begin() + static_cast<long>(j) + 1);
+    }
+    if (stmts.size() >= 2)
+      if (NodePtr rolled = reroll(stmts, decls)) return rolled;
+    return make_block(std::move(stmts), std::move(decls));
+  }
+
+  NodePtr stmt(const NodePtr& n) {
+    switch (n->op) {
+      case Op::Block: {
+        std::vector<NodePtr> stmts;
+        for (const auto& a : n->args) stmts.push_back(stmt(a));
+        return block(std::move(stmts), n->decls);
+      }
+      case Op::Range:
+        return loop(make_loop(*n, n->name, fold_expr(n->args[0]), fold_expr(n->args[1]), fold_expr(n->args[2]),
+                              stmt(n->args[3])));
+      case Op::If: {
+        std::vector<NodePtr> args = {fold_expr(n->args[0])};
+        for (size_t i = 1; i < n->args.size(); ++i) args.push_back(stmt(n->args[i]));
+        return with_args(*n, std::move(args));
+      }
+      default:
+        return fold_expr(n);
+    }
+  }
+
+  // ---- second pass: what the first left behind ------------------------------------------------
+
+  // Integer block variables assigned once from an affine expression are substituted into the
+  // statements that follow (a strip-mined pair whose loops were interchanged apart keeps its
+  // `v = o + i`), and every loop with constant bounds starts at 0 and steps by 1.
+  NodePtr settle(const NodePtr& n) {
+    switch (n->op) {
+      case Op::Block: {
+        std::vector<NodePtr> stmts = n->args;
+        auto decls = n->decls;
+        for (size_t j = 0; j < stmts.size();) {
+          const Node& s = *stmts[j];
+          bool sub = s.op == Op::Assign && int_vars.count(s.name) > 0 && int_affine(*s.args[0]).has_value() &&
+                     !mentions(*s.args[0], s.name);
+          if (sub) {
+            bool declared = false;
+            for (const auto& d : decls) declared = declared || d.first == s.name;
+            sub = declared;
+            for (size_t q = 0; q < stmts.size() && sub; ++q)
+              sub = q == j || !assigns(*stmts[q], s.name);
+            for (size_t q = 0; q < j && sub; ++q) sub = !mentions(*stmts[q], s.name);
+          }
+          if (!sub) {
+            ++j;
+            continue;
+          }
+          const std::string v = s.name;
+          const NodePtr e = s.args[0];
+          for (size_t q = j + 1; q < stmts.size(); ++q) stmts[q] = substitute_vars(stmts[q], {{v, e}});
+          stmts.erase(stmts.begin() + static_cast<long>(j));
+          drop_decl(&decls, v);
+        }
+        for (auto& s : stmts) s = settle(s);
+        return make_block(std::move(stmts), std::move(decls));
+      }
+      case Op::Range: {
+        int64_t s = 0, step = 0, e = 0;
+        NodePtr body = n->args[3];
+        if (int_const(*n->args[0], &s) && int_const(*n->args[1], &step) && int_const(*n->args[2], &e) && step >= 1 &&
+            (s != 0 || step != 1) && !assigns(*body, n->name)) {
+          const int64_t count = e > s ? (e - s + step - 1) / step : 0;
+          Affine a;
+          a.c = s;
+          a.coef[n->name] = step;
+          body = substitute_vars(body, {{n->name, affine_to_node(a)}});
+          return make_loop(*n, n->name, make_i64(0), make_i64(1), make_i64(count), settle(body));
+        }
+        return make_loop(*n, n->name, n->args[0], n->args[1], n->args[2], settle(body));
+      }
+      case Op::If: {
+        std::vector<NodePtr> args = {n->args[0]};
+        for (size_t i = 1; i < n->args.size(); ++i) args.push_back(settle(n->args[i]));
+        return with_args(*n, std::move(args));
+      }
+      default:
+        return n;
+    }
+  }
+};
+
+}  // namespace
+
+NodePtr normalize_kernel(const NodePtr& kernel) {
+  if (kernel->op != Op::Kernel || kernel->args.size() != 1) return kernel;
+  Normalizer nz;
+  nz.collect_int_vars(*kernel);
+  NodePtr body = nz.stmt(kernel->args[0]);
+  body = nz.settle(body);
+  body = nz.stmt(body);                       // substitutions may have exposed foldable integers
+  if (to_text(*body) == to_text(*kernel->args[0])) return kernel;
+  return [&] {
+    auto k = std::make_shared<Node>(*kernel);
+    k->args = {body};
+    return k;
+  }();
+}
+
+double serial_iterations(const Node& n) {
+  switch (n.op) {
+    case Op::Range: {
+      int64_t s, step, e;
+      double trips = 1;
+      if (int_const(*n.args[0], &s) && int_const(*n.args[1], &step) && int_const(*n.args[2], &e) && step >= 1)
+        trips = e > s ? static_cast<double>((e - s + step - 1) / step) : 0.0;
+      return trips * std::max(1.0, serial_iterations(*n.args[3]));
+    }
+    case Op::Block: case Op::Kernel: {
+      double sum = 0;
+      for (const auto& a : n.args) sum += serial_iterations(*a);
+      return sum;
+    }
+    case Op::If: {
+      double m = 0;
+      for (size_t i = 1; i < n.args.size(); ++i) m = std::max(m, serial_iterations(*n.args[i]));
+      return m;
+    }
+    default:
+      return 0;
+  }
+}
+
+}  // namespace eh

@@ -1,7 +1,8 @@
 """`execute_graph`: lower a graph and run its kernels on the default device.
 
 Host-side mirror of the reference's `src/backend/executor.rs:149-450`:
-lower (+ graph fusion), then per kernel split the pointer parameters into
+lower (+ graph fusion), the AST optimisation stage at ECLAT_OPT_LEVEL (default 3,
+`:169-176`; `optimize.py` says what of it is mirrored), then per kernel split the pointer parameters into
 immutable inputs / mutable outputs (`:257-270`), look inputs up by buffer name,
 allocate zero-filled outputs with the lowerer's shape (`:288-315`), compile
 through the kernel cache (`:323-338`), execute (`:347`), publish outputs under
@@ -22,6 +23,7 @@ from .device import (DeviceError, compile_ast_with_cache, compile_program_with_c
                      get_default_device)
 from .graph import GraphNode, collect_inputs
 from .lowerer import lower_graph
+from .optimize import optimize_program
 
 
 class ExecutionError(Exception):
@@ -87,6 +89,8 @@ def execute_graph(roots: Sequence[GraphNode], input_buffers: Dict[int, object],
     if not roots:
         return []
     program, lowerer, opt_roots = lower_graph(roots)
+    # pipeline.optimize (executor.rs:169-176): ECLAT_OPT_LEVEL 0 leaves the program as lowered
+    program = optimize_program(program)
     kernels = [k for k in program.args if k.op == "kernel"]
 
     input_nodes = collect_inputs(roots)

@@ -13,6 +13,7 @@ import numpy as np
 from .frontend import AstNode, Tensor, lower_graph, nn
 from .frontend.executor import buffer_table
 from .frontend.graph import collect_inputs
+from .frontend.optimize import optimize_program
 
 
 def config1_inputs(n: int = 1024, seed: int = 1234) -> List[np.ndarray]:
@@ -59,6 +60,7 @@ def lower_with_table(shapes: List[Tuple[int, ...]], graph_fn: Callable):
     tensors = [Tensor.input(list(s)) for s in shapes]
     y = graph_fn(*tensors)
     prog, lw, _ = lower_graph([y.graph])
+    prog = optimize_program(prog)            # what the executor's optimisation stage hands on
     by_id = {id(n): lw.lookup_buffer_name(n) for n in collect_inputs([y.graph])}
     arg_names = [by_id[id(t.graph)] for t in tensors]
     produced = [p.name for k in prog.args for p in k.attrs["params"] if p.dtype.is_ptr() and p.mutable]
@@ -178,6 +180,7 @@ def lower_multi(tensors_in, roots):
     from .frontend.executor import _root_buffer_name
     with exact_mode():
         prog, lw, opt_roots = lower_graph([r.graph for r in roots])
+    prog = optimize_program(prog)
     all_inputs = collect_inputs([r.graph for r in roots])
     by_id = {id(n): lw.lookup_buffer_name(n) for n in all_inputs}
     arg_names = [by_id[id(t.graph)] for t in tensors_in]

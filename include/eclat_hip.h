@@ -41,7 +41,7 @@ typedef struct eh_module eh_module;     /* one entry point of a loaded code obje
 /* ---- library ---------------------------------------------------------------------------- */
 int eh_version(void);                   /* 100 * major + minor */
 const char* eh_last_error(void);        /* valid until the calling thread's next failing call */
-void eh_free(void* p);                  /* releases memory handed out by eh_compile_source */
+void eh_free(void* p);                  /* releases memory handed out by eh_compile_source and eh_normalize_ast */
 
 /* ---- BackendRegistry: kind/name/is_available/list_devices/create_device
  *      (src/backend/device.rs:83-131), Device::profile (src/backend/traits.rs:273-306) ------- */
@@ -89,7 +89,9 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
  *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
- *      gemm_epilogue, gemm_dma, gemm_merge_batch, nontemporal. ----------------------------- */
+ *      gemm_epilogue, gemm_dma, gemm_merge_batch, nontemporal, normalize, allow_serial.
+ *      A kernel that no schedule recognises, would run in a single work-item and loops more than
+ *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1. ----------------- */
 typedef struct eh_launch_info {
   const char* entry;                    /* kernel symbol */
   const char* source;                   /* HIP C translation unit */
@@ -104,6 +106,14 @@ typedef struct eh_launch_info {
 } eh_launch_info;
 
 int eh_render_program(const char* ast_text, const char* options, eh_plan** out);
+/* The program (or kernel) with the rewrites of the reference's AST optimiser undone where they are
+ * recognised -- what eh_render_program and eh_program_compile plan from.  That optimiser runs
+ * before any backend sees a kernel (pipeline.optimize, src/backend/executor.rs:169-176,
+ * src/backend/compile.rs:246-265): shifts for multiplications by powers of two
+ * (src/opt/ast/rules/bit_ops.rs:19-83), tiled loops with remainder loops or guards and unrolled
+ * loops (src/opt/ast/transforms.rs:238-361, 393-630).  The result computes what the input
+ * computes, statement for statement.  *out_text is AST text, released with eh_free. */
+int eh_normalize_ast(const char* ast_text, char** out_text);
 int eh_plan_num_launches(eh_plan* plan, int* n);
 int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out);    /* strings live as long as the plan */
 int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name);

@@ -76,7 +76,10 @@ def _add_openmp_pragmas(src: str) -> str:
 
 
 class CKernel:
-    def __init__(self, source: str, entry_point: str, n_ptr_args: int, openmp: bool = False):
+    def __init__(self, source: str, entry_point: str, n_ptr_args: int, openmp: bool = False,
+                 gcc_args: Optional[Sequence[str]] = None):
+        """`gcc_args` replaces the reference's flags; tests that compare two forms of one
+        kernel for equal evaluation order use it to compile without -ffast-math."""
         self.source = source
         self.entry_point = entry_point
         self.n_ptr_args = n_ptr_args
@@ -85,7 +88,7 @@ class CKernel:
         lib_path = os.path.join(self._tmp.name, f"lib{entry_point}.so")
         with open(src_path, "w") as f:
             f.write(source)
-        args = ["gcc"] + GCC_ARGS + (["-fopenmp"] if openmp else []) + \
+        args = ["gcc"] + list(GCC_ARGS if gcc_args is None else gcc_args) + (["-fopenmp"] if openmp else []) + \
                ["-o", lib_path, src_path, "-lm"]
         r = subprocess.run(args, capture_output=True, text=True)
         if r.returncode != 0:

@@ -1,0 +1,245 @@
+"""Kernels as the reference's AST optimiser may hand them over (ECLAT_OPT_LEVEL > 0,
+`src/backend/executor.rs:169-176`): shifts for power-of-two strides, sums re-associated, loops
+tiled with a remainder or a guard, tile and remainder loops unrolled, loops interchanged.
+
+CPU part: the backend plans them exactly as it plans the lowered kernel; the normalised AST
+computes, through the C oracle, bit for bit what the rewritten one computes (and the rewritten
+one what the lowered one computes, which pins the test's own transforms); a kernel nothing
+recognises is refused instead of run in one work-item.  GPU part: parity with the oracle on the
+rewritten ASTs.
+"""
+
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from conftest import bits_equal_mod_zero, realize_on
+
+RNG = np.random.default_rng
+
+TRANSFORMS = [
+    [], ["tile=7"], ["tile=2"], ["guard=5"], ["tile=7", "unroll"], ["guard=3", "unroll"],
+    ["tile_all=3"], ["tile_all=5", "unroll"], ["tile_outer=7"], ["interchange"],
+    ["tile_outer=3", "unroll"], ["unroll"], ["tile_outer=5", "tile=3"],
+]
+IDS = ["+".join(t) or "rules" for t in TRANSFORMS]
+
+
+@pytest.fixture
+def opt_env(monkeypatch):
+    def set_(level, transforms=()):
+        monkeypatch.setenv("ECLAT_OPT_LEVEL", str(level))
+        monkeypatch.setenv("ECLAT_OPT_TRANSFORMS", ",".join(transforms))
+    return set_
+
+
+def _headline(name):
+    from harp_amd import workloads as wl
+    shapes = {"config1_relu_sum": [(1024, 1024)] * 3, "config2_softmax": [(4096, 4096)],
+              "config3_matmul": [(4096, 4096)] * 2}[name]
+    return shapes, wl.CONFIGS[name][1]
+
+
+@pytest.mark.parametrize("transforms", TRANSFORMS, ids=IDS)
+@pytest.mark.parametrize("config", ["config1_relu_sum", "config2_softmax", "config3_matmul"])
+def test_rewritten_headline_kernels_are_planned_like_the_lowered_ones(frontend, opt_env, config, transforms):
+    """Same schedule, grid and block as the as-lowered AST, on the whole-program path and kernel
+    by kernel (what `compile_ast` receives)."""
+    from harp_amd import backend as hb
+    from harp_amd import workloads as wl
+    from harp_amd.frontend import AstNode
+    shapes, fn = _headline(config)
+    opt_env(0)
+    table0, _, _, _, plain0 = wl.lower_with_table(shapes, fn)
+    opt_env(3, transforms)
+    table1, _, _, _, plain1 = wl.lower_with_table(shapes, fn)
+    if transforms or config != "config2_softmax":
+        assert table1.to_sexpr() != table0.to_sexpr()          # the optimiser did rewrite something
+    if config != "config2_softmax":
+        assert "(shl " in table1.to_sexpr()                      # power-of-two strides became shifts
+
+    def dispatch(ast):
+        return [(l["schedule"], l["grid"], l["block"]) for l in hb.render_program(ast).launches]
+    assert dispatch(table1) == dispatch(table0)
+    for k0, k1 in zip(plain0.args, plain1.args):
+        assert dispatch(AstNode.program([k1])) == dispatch(AstNode.program([k0])), k0.attrs["name"]
+
+
+def _graphs(fe):
+    nn = fe.nn
+    return {
+        "mul_add_bcast": ([(6, 23), (23,)], lambda a, b: a * b.unsqueeze(0).expand(0, 6) + a),
+        "sum_last": ([(5, 37)], lambda a: (a * a).sum(1)),
+        "max_first": ([(9, 16)], lambda a: a.max(0)),
+        "softmax": ([(7, 19)], lambda a: nn.softmax(a, 1)),
+        "matmul": ([(10, 21), (21, 8)], lambda a, b: nn.matmul(a, b)),
+        "permute_copy": ([(4, 9, 8)], lambda a: a.permute([2, 0, 1]).contiguous() + a.permute([2, 0, 1])),
+        "pad": ([(5, 11)], lambda a: a.pad([(1, 2), (3, 0)]) * a.pad([(1, 2), (3, 0)])),
+        "cumsum": ([(4, 29)], lambda a: a.cumsum(1)),
+    }
+
+
+GRAPHS = ["mul_add_bcast", "sum_last", "max_first", "softmax", "matmul", "permute_copy", "pad", "cumsum"]
+
+
+@pytest.mark.parametrize("name", GRAPHS)
+def test_normalised_kernels_compute_what_the_rewritten_ones_compute(frontend, opt_env, name):
+    """Every kernel of the graph, in every rewritten form, through the C oracle: the rewritten
+    kernel against the lowered one (equal bits unless the rules re-associated a float sum), and
+    the backend's normalised AST against the rewritten one (equal bits always)."""
+    from harp_amd import backend as hb
+    from harp_amd.frontend import AstNode, lower_graph, optimize
+    from oracle.c_backend import CKernel
+    from oracle.c_renderer import render_program
+    shapes, fn = _graphs(frontend)[name]
+    opt_env(0)
+    ts = [frontend.Tensor.input(list(s)) for s in shapes]
+    prog, lw, _ = lower_graph([fn(*ts).graph])
+    rng = RNG(len(name))
+    for kern in prog.args:
+        params = [p for p in kern.attrs["params"] if p.dtype.is_ptr()]
+        variants = {"lowered": kern}
+        for t, tid in zip(TRANSFORMS, IDS):
+            rewritten = optimize.optimize_kernel(kern, t)
+            variants["rw_" + tid] = rewritten
+            variants["nm_" + tid] = hb.normalize_ast(rewritten)
+        # one translation unit: every variant under its own entry point
+        funcs, entries = {}, {}
+        for i, (vid, k) in enumerate(variants.items()):
+            text = k if isinstance(k, str) else k.to_sexpr()
+            entry = f"v{i}_{kern.attrs['name']}"
+            assert text.startswith(f'(kernel "{kern.attrs["name"]}"')
+            funcs[vid] = text.replace(f'(kernel "{kern.attrs["name"]}"', f'(kernel "{entry}"', 1)
+            entries[vid] = entry
+
+        def build(vids):
+            # strict IEEE arithmetic: with -ffast-math gcc re-associates a reduction differently for
+            # every loop structure, and equal evaluation order could not be seen in the bits
+            return CKernel(render_program("(program " + " ".join(funcs[v] for v in vids) + ")"),
+                           entries["lowered"], len(params), gcc_args=["-O1", "-shared", "-fPIC"])
+        live = list(variants)
+        try:
+            lib = build(live)
+        except RuntimeError:
+            # The reference renders a nested block without braces (src/backend/renderer.rs:604-624),
+            # so a rewritten form that repeats a block with a declaration (an unrolled loop around
+            # an accumulator) is not valid C for its own C backend either: such forms are left out
+            # here (the GPU test still runs them).
+            live = ["lowered"]
+            for tid in IDS:
+                try:
+                    build(["lowered", "rw_" + tid])
+                    live += ["rw_" + tid, "nm_" + tid]
+                except RuntimeError as e:
+                    assert "redeclaration" in str(e), str(e)
+            lib = build(live)
+        assert len(live) >= 1 + 2 * 8, live
+        sizes = {p.name: int(np.prod([int(e.evaluate()) for e in lw.get_buffer_info_by_name(p.name)[0]]))
+                 for p in params}
+        inputs = {p.name: rng.uniform(-2, 2, sizes[p.name]).astype(np.float32) for p in params if not p.mutable}
+
+        def run(entry):
+            outs = {p.name: np.zeros(sizes[p.name], np.float32) for p in params if p.mutable}
+            args = [inputs[p.name] if not p.mutable else outs[p.name] for p in params]
+            fn_ = getattr(lib._lib, entry)
+            fn_.restype = None
+            fn_(*[ctypes.c_void_p(a.ctypes.data) for a in args])
+            return np.concatenate([outs[p.name] for p in params if p.mutable])
+        base = run(entries["lowered"])
+        for tid in IDS:
+            if "rw_" + tid not in live:
+                continue
+            rw, nm = run(entries["rw_" + tid]), run(entries["nm_" + tid])
+            assert np.allclose(rw, base, rtol=1e-5, atol=1e-6), (kern.attrs["name"], tid)
+            assert bits_equal_mod_zero(nm, rw), (kern.attrs["name"], tid)
+
+
+def test_normalisation_restores_the_lowered_loop_nest(frontend, opt_env):
+    """For the plain forms the normalised text is the lowered text itself, shifts, tiles and
+    unrolled remainders gone."""
+    from harp_amd import backend as hb
+    from harp_amd.frontend import lower_graph, optimize
+    opt_env(0)
+    a, b = frontend.Tensor.input([64, 100]), frontend.Tensor.input([64, 100])
+    prog, _, _ = lower_graph([(a * b).graph])
+    kern = prog.args[0]
+    want = hb.normalize_ast(kern)
+    assert "(shl" not in want and "ridx" in want
+    for t in (["tile=7"], ["tile=7", "unroll"], ["guard=3"], ["tile_all=3"], ["tile_outer=5", "tile=3"]):
+        rewritten = optimize.optimize_kernel(kern, t)
+        assert rewritten.to_sexpr() != kern.to_sexpr()
+        assert hb.normalize_ast(rewritten) == want, t
+
+
+def _odd_kernel(n):
+    """out[i] = t, t = t * 0.5 + x[i]: a recurrence no schedule recognises."""
+    from harp_amd.frontend import AstNode as A
+    from harp_amd.frontend.ast import DType, F32, VarDecl
+    c = A.const_i64
+    step = A.assign("t", A.add(A.mul(A.var("t"), A.const_f32(0.5)), A.load(A.var("x"), A.var("i"), F32)))
+    body = A.block([A.assign("t", A.const_f32(0.0)),
+                    A.range("i", c(0), c(1), c(n), A.block([step, A.store(A.var("y"), A.var("i"), A.var("t"))]))],
+                   decls=[("t", F32)])
+    params = [VarDecl("x", DType.ptr(F32)), VarDecl("y", DType.ptr(F32), mutable=True)]
+    return A.program([A.kernel("odd_recurrence", params, body)])
+
+
+def test_long_serial_kernels_are_refused_not_run_in_one_work_item():
+    from harp_amd import backend as hb
+    from harp_amd._lib import EhError
+    small = hb.render_program(_odd_kernel(1000)).launches
+    assert [l["schedule"] for l in small] == ["as-written"] and small[0]["grid"] == [1, 1, 1]
+    with pytest.raises(EhError, match="would run its 300000 loop iterations in one work-item") as e:
+        hb.render_program(_odd_kernel(300_000))
+    assert e.value.code == 3                         # EH_ERR_UNSUPPORTED
+    forced = hb.render_program(_odd_kernel(300_000), "allow_serial=1").launches
+    assert [l["schedule"] for l in forced] == ["as-written"]
+
+
+# ---------------------------------------------------------------------------------------------
+# GPU
+# ---------------------------------------------------------------------------------------------
+
+GPU_TRANSFORMS = [[], ["tile=7"], ["guard=5"], ["tile=7", "unroll"], ["tile_all=3"], ["tile_outer=7"],
+                  ["interchange"], ["tile=7", "interchange"]]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transforms", GPU_TRANSFORMS, ids=["+".join(t) or "rules" for t in GPU_TRANSFORMS])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_rewritten_kernels_match_the_oracle_on_the_gpu(frontend, hip, opt_env, transforms, fuse):
+    """Configs 1 to 3 (reduced sizes), both paths, HIP and oracle on the same rewritten AST:
+    elementwise outputs bit-exact, reductions within 1e-5, matmul within 1e-3 of the row scale."""
+    from harp_amd import workloads as wl
+    opt_env(3, transforms)
+    a, b, c = [RNG(s).normal(0, 1, (300, 1000)).astype(np.float32) for s in (1, 2, 3)]
+    ref = realize_on(frontend, "c", lambda x, y, z: x * y + z, [a, b, c])
+    got = realize_on(frontend, "hip", lambda x, y, z: x * y + z, [a, b, c], fuse=fuse)
+    assert bits_equal_mod_zero(ref, got)
+    ref = realize_on(frontend, "c", wl.config1_graph, [a, b, c])
+    got = realize_on(frontend, "hip", wl.config1_graph, [a, b, c], fuse=fuse)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5)
+    x = RNG(4).normal(0, 2, (257, 4096)).astype(np.float32)
+    ref = realize_on(frontend, "c", wl.config2_graph, [x])
+    got = realize_on(frontend, "hip", wl.config2_graph, [x], fuse=fuse)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-12)
+    p, q = RNG(5).uniform(-1, 1, (192, 640)).astype(np.float32), RNG(6).uniform(-1, 1, (640, 160)).astype(np.float32)
+    ref = realize_on(frontend, "c", wl.config3_graph, [p, q])
+    got = realize_on(frontend, "hip", wl.config3_graph, [p, q], fuse=fuse)
+    scale = np.abs(p).astype(np.float64) @ np.abs(q).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref.reshape(got.shape)) <= 1e-3 * scale.reshape(got.shape))
+    assert np.allclose(got.reshape(192, 160), p.astype(np.float64) @ q.astype(np.float64), rtol=0, atol=1e-4 * scale.max())
+
+
+@pytest.mark.gpu
+def test_opt_levels_give_the_same_results_on_the_gpu(frontend, hip, opt_env):
+    """Level 0 and level 3 (rule set) differ in the AST text only."""
+    from harp_amd import workloads as wl
+    x = RNG(9).normal(0, 2, (128, 2048)).astype(np.float32)
+    outs = []
+    for level in (0, 3):
+        opt_env(level)
+        outs.append(realize_on(frontend, "hip", wl.config2_graph, [x]))
+    assert np.allclose(outs[0], outs[1], rtol=1e-6, atol=1e-12)
