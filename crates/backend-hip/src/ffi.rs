@@ -59,6 +59,11 @@ unsafe extern "C" {
     pub fn eh_program_compile(dev: *mut eh_device, ast_text: *const c_char, options: *const c_char,
                               out: *mut *mut eh_program) -> c_int;
     pub fn eh_program_release(prog: *mut eh_program) -> c_int;
+    pub fn eh_program_num_buffers(prog: *mut eh_program, n: *mut c_int) -> c_int;
+    pub fn eh_program_buffer(prog: *mut eh_program, i: c_int, name: *mut *const c_char, role: *mut *const c_char,
+                             bytes: *mut usize, elided: *mut c_int) -> c_int;
+    pub fn eh_program_num_launches(prog: *mut eh_program, n: *mut c_int) -> c_int;
+    pub fn eh_program_execute(prog: *mut eh_program, bufs: *const *mut eh_buffer, n_bufs: c_int, sync: c_int) -> c_int;
     pub fn eh_program_execute_positional(prog: *mut eh_program, inputs: *const *mut eh_buffer, n_in: c_int,
                                          outputs: *const *mut eh_buffer, n_out: c_int, sync: c_int) -> c_int;
     pub fn eh_program_binary(prog: *mut eh_program, launch: c_int, blob: *mut *const c_void,

@@ -2,6 +2,11 @@
 //! One form per variant of `eclat::ast::AstNode`; float literals travel as IEEE bit patterns.
 
 use eclat::ast::{AddressSpace, AstNode, DType, Literal, Mutability, VarDecl, VarKind};
+use eclat::backend::device::ProgramBuffer;
+
+/// A node the text form has no spelling for (`Allocate`, `Deallocate`, `CallKernel`,
+/// `WmmaMatmul`, `src/ast/mod.rs:246-290`): compiling such a program is an error, not a panic.
+pub type SerResult = Result<String, String>;
 
 pub fn first_kernel_name(program: &AstNode) -> Option<String> {
     if let AstNode::Program { functions, .. } = program {
@@ -11,6 +16,8 @@ pub fn first_kernel_name(program: &AstNode) -> Option<String> {
     }
     None
 }
+
+pub fn dtype_text(d: &DType) -> String { dtype(d) }
 
 fn dtype(d: &DType) -> String {
     match d {
@@ -51,83 +58,104 @@ fn param(p: &VarDecl) -> String {
     format!("(\"{}\" {} {} {})", p.name, dtype(&p.dtype), m, k)
 }
 
-fn list(op: &str, items: &[&AstNode]) -> String {
+fn list(op: &str, items: &[&AstNode]) -> SerResult {
     let mut s = format!("({op}");
-    for i in items { s.push(' '); s.push_str(&to_text(i)); }
+    for i in items { s.push(' '); s.push_str(&to_text(i)?); }
+    s.push(')');
+    Ok(s)
+}
+
+/// `(buffers ("name" dtype (shape ...) role) ...)`: the table that lets the library compile the
+/// program as a whole (fuse kernels, keep temporaries out of memory).
+pub fn buffer_table(table: &[ProgramBuffer]) -> String {
+    let mut s = String::from("(buffers");
+    for b in table {
+        let dims: Vec<String> = b.shape.iter().map(|d| d.to_string()).collect();
+        s.push_str(&format!(" (\"{}\" {} (shape {}) {})", b.name, dtype(&b.dtype), dims.join(" "), b.role.as_str()));
+    }
     s.push(')');
     s
 }
 
-pub fn to_text(n: &AstNode) -> String {
+/// A Program with its buffer table in front of the kernels.
+pub fn program_text(kernels: &[AstNode], table: &[ProgramBuffer]) -> SerResult {
+    let mut s = String::from("(program ");
+    s.push_str(&buffer_table(table));
+    for k in kernels { s.push(' '); s.push_str(&to_text(k)?); }
+    s.push(')');
+    Ok(s)
+}
+
+pub fn to_text(n: &AstNode) -> SerResult {
     use AstNode::*;
-    match n {
+    Ok(match n {
         Wildcard(s) => format!("(wildcard \"{s}\")"),
         Const(l) => literal(l),
         Var(s) => format!("(var \"{s}\")"),
-        Add(a, b) => list("add", &[a, b]), Mul(a, b) => list("mul", &[a, b]), Max(a, b) => list("max", &[a, b]),
-        Rem(a, b) => list("rem", &[a, b]), Idiv(a, b) => list("idiv", &[a, b]), Lt(a, b) => list("lt", &[a, b]),
-        And(a, b) => list("and", &[a, b]), BitwiseAnd(a, b) => list("bitand", &[a, b]),
-        BitwiseOr(a, b) => list("bitor", &[a, b]), BitwiseXor(a, b) => list("bitxor", &[a, b]),
-        LeftShift(a, b) => list("shl", &[a, b]), RightShift(a, b) => list("shr", &[a, b]),
-        Recip(a) => list("recip", &[a]), Sqrt(a) => list("sqrt", &[a]), Log2(a) => list("log2", &[a]),
-        Exp2(a) => list("exp2", &[a]), Sin(a) => list("sin", &[a]), Floor(a) => list("floor", &[a]),
-        Not(a) => list("not", &[a]), BitwiseNot(a) => list("bitnot", &[a]),
-        Cast(a, d) => format!("(cast {} {})", dtype(d), to_text(a)),
-        Fma { a, b, c } => list("fma", &[a, b, c]),
-        Select { cond, then_val, else_val } => list("select", &[cond, then_val, else_val]),
-        Load { ptr, offset, count, dtype: d } => format!("(load {} {} {} {})", to_text(ptr), to_text(offset), count, dtype(d)),
-        Store { ptr, offset, value } => list("store", &[ptr, offset, value]),
-        Assign { var, value } => format!("(assign \"{var}\" {})", to_text(value)),
+        Add(a, b) => list("add", &[a, b])?, Mul(a, b) => list("mul", &[a, b])?, Max(a, b) => list("max", &[a, b])?,
+        Rem(a, b) => list("rem", &[a, b])?, Idiv(a, b) => list("idiv", &[a, b])?, Lt(a, b) => list("lt", &[a, b])?,
+        And(a, b) => list("and", &[a, b])?, BitwiseAnd(a, b) => list("bitand", &[a, b])?,
+        BitwiseOr(a, b) => list("bitor", &[a, b])?, BitwiseXor(a, b) => list("bitxor", &[a, b])?,
+        LeftShift(a, b) => list("shl", &[a, b])?, RightShift(a, b) => list("shr", &[a, b])?,
+        Recip(a) => list("recip", &[a])?, Sqrt(a) => list("sqrt", &[a])?, Log2(a) => list("log2", &[a])?,
+        Exp2(a) => list("exp2", &[a])?, Sin(a) => list("sin", &[a])?, Floor(a) => list("floor", &[a])?,
+        Not(a) => list("not", &[a])?, BitwiseNot(a) => list("bitnot", &[a])?,
+        Cast(a, d) => format!("(cast {} {})", dtype(d), to_text(a)?),
+        Fma { a, b, c } => list("fma", &[a, b, c])?,
+        Select { cond, then_val, else_val } => list("select", &[cond, then_val, else_val])?,
+        Load { ptr, offset, count, dtype: d } => format!("(load {} {} {} {})", to_text(ptr)?, to_text(offset)?, count, dtype(d)),
+        Store { ptr, offset, value } => list("store", &[ptr, offset, value])?,
+        Assign { var, value } => format!("(assign \"{var}\" {})", to_text(value)?),
         AtomicAdd { ptr, offset, value, dtype: d } =>
-            format!("(atomic_add {} {} {} {})", to_text(ptr), to_text(offset), to_text(value), dtype(d)),
+            format!("(atomic_add {} {} {} {})", to_text(ptr)?, to_text(offset)?, to_text(value)?, dtype(d)),
         AtomicMax { ptr, offset, value, dtype: d } =>
-            format!("(atomic_max {} {} {} {})", to_text(ptr), to_text(offset), to_text(value), dtype(d)),
+            format!("(atomic_max {} {} {} {})", to_text(ptr)?, to_text(offset)?, to_text(value)?, dtype(d)),
         Rand => "(rand)".into(),
         Barrier => "(barrier)".into(),
         Block { statements, scope } => {
             let mut s = String::from("(block (decls");
             for v in scope.local_variables() { s.push_str(&format!(" (\"{}\" {})", v.name, dtype(&v.dtype))); }
             s.push(')');
-            for st in statements { s.push(' '); s.push_str(&to_text(st)); }
+            for st in statements { s.push(' '); s.push_str(&to_text(st)?); }
             s.push(')');
             s
         }
         Range { var, start, step, stop, body, parallel } => {
             let kind = if parallel.is_parallel { format!("{:?}", parallel.kind).to_lowercase() } else { "sequential".into() };
-            format!("(range \"{var}\" {} {} {} {} {kind})", to_text(start), to_text(step), to_text(stop), to_text(body))
+            format!("(range \"{var}\" {} {} {} {} {kind})", to_text(start)?, to_text(step)?, to_text(stop)?, to_text(body)?)
         }
         If { condition, then_body, else_body } => match else_body {
-            Some(e) => list("if", &[condition, then_body, e]),
-            None => list("if", &[condition, then_body]),
+            Some(e) => list("if", &[condition, then_body, e])?,
+            None => list("if", &[condition, then_body])?,
         },
         Call { name, args } => {
             let mut s = format!("(call \"{name}\"");
-            for a in args { s.push(' '); s.push_str(&to_text(a)); }
+            for a in args { s.push(' '); s.push_str(&to_text(a)?); }
             s.push(')');
             s
         }
-        Return { value } => list("return", &[value]),
-        SharedAlloc { name, dtype: d, size } => format!("(shared_alloc \"{name}\" {} {})", dtype(d), to_text(size)),
-        SharedLoad { ptr, offset, dtype: d } => format!("(shared_load {} {} {})", to_text(ptr), to_text(offset), dtype(d)),
-        SharedStore { ptr, offset, value } => list("shared_store", &[ptr, offset, value]),
+        Return { value } => list("return", &[value])?,
+        SharedAlloc { name, dtype: d, size } => format!("(shared_alloc \"{name}\" {} {})", dtype(d), to_text(size)?),
+        SharedLoad { ptr, offset, dtype: d } => format!("(shared_load {} {} {})", to_text(ptr)?, to_text(offset)?, dtype(d)),
+        SharedStore { ptr, offset, value } => list("shared_store", &[ptr, offset, value])?,
         Kernel { name, params, body, default_grid_size: g, default_thread_group_size: t, .. } => {
             let ps: Vec<String> = params.iter().map(param).collect();
             format!("(kernel \"{}\" (params {}) (grid {} {} {}) (tg {} {} {}) {})",
                     name.clone().unwrap_or_else(|| "kernel".into()), ps.join(" "),
-                    to_text(&g[0]), to_text(&g[1]), to_text(&g[2]),
-                    to_text(&t[0]), to_text(&t[1]), to_text(&t[2]), to_text(body))
+                    to_text(&g[0])?, to_text(&g[1])?, to_text(&g[2])?,
+                    to_text(&t[0])?, to_text(&t[1])?, to_text(&t[2])?, to_text(body)?)
         }
         Function { name, params, return_type, body } => {
             let ps: Vec<String> = params.iter().map(param).collect();
             format!("(function \"{}\" (params {}) (ret {}) {})", name.clone().unwrap_or_else(|| "anonymous".into()),
-                    ps.join(" "), dtype(return_type), to_text(body))
+                    ps.join(" "), dtype(return_type), to_text(body)?)
         }
         Program { functions, .. } => {
             let mut s = String::from("(program");
-            for f in functions { s.push(' '); s.push_str(&to_text(f)); }
+            for f in functions { s.push(' '); s.push_str(&to_text(f)?); }
             s.push(')');
             s
         }
-        other => panic!("backend-hip: AST node not serialisable: {other:?}"),
-    }
+        other => return Err(format!("backend-hip: AST node has no text form: {other:?}")),
+    })
 }

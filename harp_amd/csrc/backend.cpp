@@ -102,7 +102,9 @@ std::string HipCompiler::cache_dir() {
   if (const char* d = std::getenv("HARP_CACHE_DIR")) base = d;
   else if (const char* h = std::getenv("HOME")) base = std::string(h) + "/.cache/harp";
   else base = "/tmp/harp-cache";
-  return base + "/kernels/Hip";
+  // not kernels/<DeviceKind>: that is where the reference keeps its own disk cache, with a
+  // different side-file schema (src/backend/cache/disk.rs:63-115)
+  return base + "/code_objects/gfx950";
 }
 
 Binary HipCompiler::compile(const std::string& source, const std::string& arch, bool use_disk_cache, bool refresh) {

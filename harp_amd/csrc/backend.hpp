@@ -42,7 +42,7 @@ class HipCompiler {
   static Binary compile(const std::string& source, const std::string& arch, bool use_disk_cache = true,
                         bool refresh = false);
   static std::vector<std::string> options(const std::string& arch);
-  static std::string cache_dir();      // HARP_CACHE_DIR or ~/.cache/harp, + /kernels/Hip
+  static std::string cache_dir();      // HARP_CACHE_DIR or ~/.cache/harp, + /code_objects/gfx950
   static bool disk_cache_enabled();    // HARP_NO_DISK_CACHE unset
 };
 

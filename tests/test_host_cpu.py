@@ -41,6 +41,48 @@ def test_rust_binding_names_only_declared_symbols():
     for name, n in bound.items():
         assert name in declared, f"{name} bound in ffi.rs but not declared in eclat_hip.h"
         assert declared[name] == n, f"{name}: {n} parameters in ffi.rs, {declared[name]} in the header"
+    # the whole-program path of the binding
+    assert {"eh_program_num_buffers", "eh_program_buffer", "eh_program_execute"} <= set(bound)
+    with open(os.path.join(ROOT, "crates", "backend-hip", "src", "lib.rs")) as f:
+        lib_rs = f.read()
+    for name in re.findall(r"ffi::(eh_[a-z_0-9]+)\(", lib_rs):
+        assert name in bound, f"lib.rs calls ffi::{name}, which ffi.rs does not declare"
+    assert "fn execute_program(" in lib_rs and "panic!" not in lib_rs
+    with open(os.path.join(ROOT, "crates", "backend-hip", "src", "ser.rs")) as f:
+        assert "panic!" not in f.read()
+
+
+def test_core_edits_patch_is_well_formed():
+    """Every hunk header of crates/backend-hip/core-edits.patch counts its own lines right, new
+    line numbers follow from the old ones, and the executor hunks (skip of the optimisation
+    stage for the HIP device, whole-program hook) are there."""
+    with open(os.path.join(ROOT, "crates", "backend-hip", "core-edits.patch")) as f:
+        lines = f.read().split("\n")
+    delta, seen_files, i = 0, [], 0
+    while i < len(lines):
+        l = lines[i]
+        if l.startswith("diff "):
+            delta = 0
+            seen_files.append(l.split(" b/")[1])
+        m = re.match(r"@@ -(\d+)(?:,(\d+))? \+(\d+)(?:,(\d+))? @@", l)
+        if m:
+            old_start, old_n = int(m.group(1)), int(m.group(2) or 1)
+            new_start, new_n = int(m.group(3)), int(m.group(4) or 1)
+            body = []
+            i += 1
+            while i < len(lines) and lines[i][:1] in ("+", "-") and not lines[i].startswith(("+++", "---")):
+                body.append(lines[i])
+                i += 1
+            assert sum(b[0] == "-" for b in body) == old_n, l
+            assert sum(b[0] == "+" for b in body) == new_n, l
+            if old_start or old_n:
+                assert new_start == old_start + delta + (1 if old_n == 0 else 0), l
+            delta += new_n - old_n
+            continue
+        i += 1
+    assert {"src/backend/executor.rs", "src/backend/device.rs", "src/backend/program_exec.rs"} <= set(seen_files)
+    text = "\n".join(lines)
+    assert "if device_kind == DeviceKind::Hip" in text and "try_execute_program" in text
 
 
 def test_c_client_renders_and_compiles_without_a_gpu():
