@@ -5,9 +5,10 @@ A step is one pass of the hot path (execute the compiled Program) over one batch
 of synthetic input.  The headline workload is benchmark configuration 2 -- row softmax of
 fp32 [4096, 4096], compiled from the reference's five-kernel lowering into one
 fused launch -- reported as HBM GB/s of algorithmic traffic (one read + one
-write).  The same JSON line carries config 3 (4096^3 fp32 matmul, TFLOP/s on the
-FP32 MFMA schedule) and config 1 under "extra", a roofline object per dominant
-kernel, and the CPU baseline (the oracle's C kernels, unfused, on host cores).
+write).  The same JSON line carries configs 3, 1, 4 and 5 under "extra", each with a
+roofline object; for configs 1, 2, 4 and 5 also the per-kernel path (what the reference's
+unmodified executor would drive: one synchronous launch per lowered kernel); and the CPU
+baseline (the oracle's C kernels, unfused, on host cores).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--options key=value,...]
 """
@@ -18,46 +19,15 @@ import argparse
 import json
 import os
 import sys
-import time
 
 import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
-FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix peak
-
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
-
-
-def measured_traffic(kernel):
-    """HBM bytes per launch from the committed counter summary (rocprofv3 --pmc FETCH_SIZE /
-    WRITE_SIZE, scaled by a copy kernel of known size); None when the kernel is not in it."""
-    try:
-        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            return json.load(f)["kernels"][kernel]["traffic_bytes"]
-    except (OSError, KeyError, ValueError):
-        return None
-
-
-def build(dev, hb, wl, name, shapes, options):
-    inputs_fn, graph_fn = wl.CONFIGS[name]
-    prog_ast, arg_names, out_name, const_inputs, _ = wl.lower_with_table(shapes, graph_fn)
-    prog = hb.HipProgram(dev, prog_ast, options)
-    return prog, arg_names, out_name, const_inputs
-
-
-def make_sets(dev, hb, prog, arg_names, const_inputs, arrays, nsets):
-    from harp_amd import measure
-    return measure.make_sets(dev, prog, arg_names, const_inputs, arrays, nsets)
-
-
-def time_steps(dev, hb, prog, sets, steps, warmup):
-    from harp_amd import measure
-    return measure.time_steps(dev, prog, sets, steps, warmup)
 
 
 def main():
@@ -67,8 +37,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak (default: all but copy)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak (default: all but the last two)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-kernel", action="store_true", help="skip the per-kernel (unfused, synchronous) path")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -78,7 +49,9 @@ def main():
         sys.exit("bench.py: --steps must be >= 1 and --warmup >= 0")
 
     from harp_amd import backend as hb
+    from harp_amd import measure
     from harp_amd import workloads as wl
+    from harp_amd.measure import FP32_MFMA_PEAK_TFLOPS, HBM_PEAK_GBS      # MI355X published peaks
     if hb.device_count() == 0:
         sys.exit("bench.py: no HIP device present; the HIP backend has no CPU path")
     dev = hb.HipDevice(0)
@@ -87,93 +60,95 @@ def main():
         f"clock={props['clock_khz'] / 1e6:.2f} GHz LDS/CU={props['local_memory_size']}")
     options = args.options or None
     want = lambda n: not args.only or args.only == n
-    result_extra = {}
+    extra = {}
+
+    # ---- calibration kernels (ceilings the profiles quote; not results) ----------------------
+    if args.only == "copy":
+        gbs, launch, ms = measure.copy_rate(dev, (4096, 4096), args.steps, args.warmup, args.sets, options)
+        log(f"[bench] copy 4096^2 ({launch['entry']}, {launch['schedule']}): {ms * 1e3:.1f} us/step -> {gbs:.0f} GB/s")
+        return
+    if args.only == "mfma_peak":
+        tflops, blocks, ms = measure.mfma_issue_rate(dev)
+        log(f"[bench] MFMA f32 32x32x2 issue-rate ceiling: {tflops:.1f} TFLOP/s ({tflops / FP32_MFMA_PEAK_TFLOPS:.1%} of "
+            f"the published {FP32_MFMA_PEAK_TFLOPS}); {blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
+        return
+
+    def roofline(bound, achieved, unit, algo, launch=None):
+        """Roofline object of one kernel (`launch` given) or of a whole step: `achieved` is
+        algorithmic work over measured time."""
+        peak = HBM_PEAK_GBS if bound == "hbm" else FP32_MFMA_PEAK_TFLOPS
+        r = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+             "frac": round(achieved / peak, 4), "traffic": None,
+             "algorithmic_bytes" if bound == "hbm" else "algorithmic_flops": algo}
+        if launch is not None:
+            traffic, stale = (None, False) if args.options else measure.measured_traffic(launch["entry"], launch["source"])
+            r["traffic"] = traffic
+            if stale:
+                r["traffic_stale"] = True    # the kernel's source changed since the counters were read
+            r["traffic_source"] = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by "
+                                   "the same counters on this backend's plain copy kernel of known size (assumed free "
+                                   "of wasted traffic); counted only for the kernel source hash it was read on")
+            r["kernel"], r["schedule"] = launch["entry"], launch["schedule"]
+        return r
+
+    def unfused(prog_ast, arg_names, consts, arrays, steps, warmup, check=None):
+        """The per-kernel path: every lowered kernel compiled and launched on its own,
+        synchronously, every intermediate buffer in memory (src/backend/executor.rs:245-372)."""
+        if args.no_per_kernel:
+            return None
+        path = measure.PerKernelPath(dev, prog_ast, options)
+        inputs = measure.upload_inputs(dev, prog_ast, arg_names, consts, arrays)
+        ms = path.time(inputs, steps, warmup)
+        if check is not None and not args.no_check:
+            check(path.step(inputs))
+        dev.trim()
+        return {"ms_per_step": round(ms, 4), "steps": steps, "launches": len(path.launches),
+                "lowered_kernels": len(path.kernels),
+                "algorithmic_bytes": sum(l["algo_bytes"] for l in path.launches),
+                "timing": "host wall clock; every launch waits for completion, as Kernel::execute does"}
 
     # ---- config 2: row softmax 4096 x 4096 (headline) --------------------------------
     softmax = None
     if want("softmax"):
-        shapes = [(4096, 4096)]
         arrays = wl.config2_inputs()
-        prog, arg_names, out_name, consts = build(dev, hb, wl, "config2_softmax", shapes, options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
-        ms, wall_ms = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
+        prog_ast, arg_names, out_name, consts, _ = wl.lower_with_table([(4096, 4096)], wl.config2_graph)
+        prog = hb.HipProgram(dev, prog_ast, options)
+        sets = measure.make_sets(dev, prog, arg_names, consts, arrays, args.sets)
+        ms, wall_ms = measure.time_steps(dev, prog, sets, args.steps, args.warmup)
         algo = sum(l["algo_bytes"] for l in prog.launches)
-        softmax = {"ms": ms, "wall_ms": wall_ms, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
-                   "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
+        softmax = {"ms": ms, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo, "launch": prog.launches[0],
+                   "n_launches": len(prog.launches)}
         log(f"[bench] softmax 4096^2: {ms * 1e3:.1f} us/step -> {softmax['gbs']:.0f} GB/s "
-            f"({softmax['gbs'] / HBM_PEAK_GBS:.1%} of 8 TB/s); {softmax['launches']}")
-        if not args.no_check:
-            got = sets[0][1][out_name].read_array(np.float32, (4096, 4096))
+            f"({softmax['gbs'] / HBM_PEAK_GBS:.1%} of 8 TB/s); {[(l['entry'], l['schedule']) for l in prog.launches]}")
+
+        def check_softmax(got):
             x = arrays[0].astype(np.float64)
             e = np.exp(x[:64] - x[:64].max(1, keepdims=True))
-            assert np.allclose(got[:64], e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12), \
-                "softmax result check failed"
+            assert np.allclose(got[:64], e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12), "softmax result check failed"
             assert np.allclose(got.sum(1), 1.0, atol=1e-5), "softmax rows do not sum to 1"
+        if not args.no_check:
+            check_softmax(sets[0][1][out_name].read_array(np.float32, (4096, 4096)))
         del sets
-
-    # ---- calibration: plain copy of the same size (for counter scaling, not a result) ------
-    if args.only == "copy":
-        wl.CONFIGS["copy"] = (wl.config2_inputs, lambda x: x.contiguous())
-        arrays = wl.config2_inputs()
-        prog, arg_names, out_name, consts = build(dev, hb, wl, "copy", [(4096, 4096)], options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
-        ms, _ = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
-        log(f"[bench] copy 4096^2 ({prog.launches[0]['entry']}, {prog.launches[0]['schedule']}): "
-            f"{ms * 1e3:.1f} us/step -> {2 * 4096 * 4096 * 4 / (ms * 1e-3) / 1e9:.0f} GB/s")
-        return
-
-    # ---- calibration: MFMA issue rate with operands in registers (not a result) -------------
-    if args.only == "mfma_peak":
-        iters, waves_per_cu = 4096, 8
-        src = """
-typedef float f16v __attribute__((ext_vector_type(16)));
-extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
-  f16v acc[4];
-  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
-  float a = threadIdx.x * 1e-3f, b = blockIdx.x * 1e-3f;
-  for (int it = 0; it < %d; ++it) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
-  }
-  float s = 0.0f;
-  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += acc[i][r];
-  out[blockIdx.x * 256 + threadIdx.x] = s;
-}
-""" % iters
-        blocks = props["compute_units"] * waves_per_cu // 4
-        mod = hb.HipModule(dev, hb.compile_source(src), "eh_mfma_peak")
-        out = hb.HipBuffer(dev, [blocks * 256 * 4], None, nbytes=blocks * 256 * 4)
-        for _ in range(3):
-            mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
-        dev.sync()
-        e0, e1 = hb.Event(dev), hb.Event(dev)
-        e0.record()
-        reps = 20
-        for _ in range(reps):
-            mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
-        e1.record()
-        e1.sync()
-        ms = e0.elapsed_ms(e1) / reps
-        flops = blocks * 4 * iters * 4 * (32 * 32 * 2 * 2)
-        log(f"[bench] MFMA f32 32x32x2 issue-rate ceiling: {flops / ms / 1e9:.1f} TFLOP/s "
-            f"({flops / ms / 1e9 / FP32_MFMA_PEAK_TFLOPS:.1%} of the published {FP32_MFMA_PEAK_TFLOPS}); "
-            f"{blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
-        return
+        softmax["per_kernel"] = unfused(prog_ast, arg_names, consts, arrays, max(5, min(args.steps, 50)), 3,
+                                        lambda named: check_softmax(named[out_name].read_array(np.float32, (4096, 4096))))
+        if softmax["per_kernel"]:
+            log(f"[bench] softmax, per-kernel path: {softmax['per_kernel']['ms_per_step'] * 1e3:.1f} us/step, "
+                f"{softmax['per_kernel']['launches']} launches")
 
     # ---- config 3: 4096^3 fp32 matmul --------------------------------------------------
     matmul = None
     if want("matmul"):
-        shapes = [(4096, 4096), (4096, 4096)]
         arrays = wl.config3_inputs()
-        prog, arg_names, out_name, consts = build(dev, hb, wl, "config3_matmul", shapes, options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 2)
+        prog_ast, arg_names, out_name, consts, _ = wl.lower_with_table([(4096, 4096)] * 2, wl.config3_graph)
+        prog = hb.HipProgram(dev, prog_ast, options)
+        sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 2)
         k = max(5, min(args.steps, 50))
-        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 5))
+        ms, _ = measure.time_steps(dev, prog, sets, k, min(args.warmup, 5))
         flops = sum(l["flops"] for l in prog.launches)
-        matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k,
-                  "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
+        matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k, "flops": flops, "launch": prog.launches[0]}
         log(f"[bench] matmul 4096^3: {ms:.3f} ms/step -> {matmul['tflops']:.1f} TFLOP/s "
-            f"({matmul['tflops'] / FP32_MFMA_PEAK_TFLOPS:.1%} of FP32 MFMA peak); {matmul['launches']}")
+            f"({matmul['tflops'] / FP32_MFMA_PEAK_TFLOPS:.1%} of FP32 MFMA peak); "
+            f"{[(l['entry'], l['schedule']) for l in prog.launches]}")
         if not args.no_check:
             got = sets[0][1][out_name].read_array(np.float32, (4096, 4096))
             a, b = arrays
@@ -185,16 +160,24 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
     # ---- config 1: fused elementwise + reduce, 1024 x 1024 ------------------------------
     cfg1 = None
     if want("config1"):
-        shapes = [(1024, 1024)] * 3
         arrays = wl.config1_inputs()
-        prog, arg_names, out_name, consts = build(dev, hb, wl, "config1_relu_sum", shapes, options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, args.sets)
-        ms, _ = time_steps(dev, hb, prog, sets, args.steps, args.warmup)
+        prog_ast, arg_names, out_name, consts, _ = wl.lower_with_table([(1024, 1024)] * 3, wl.config1_graph)
+        prog = hb.HipProgram(dev, prog_ast, options)
+        sets = measure.make_sets(dev, prog, arg_names, consts, arrays, max(args.sets, 24))
+        ms, wall_ms = measure.time_steps(dev, prog, sets, args.steps, args.warmup)
         algo = sum(l["algo_bytes"] for l in prog.launches)
-        cfg1 = {"us": ms * 1e3, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
-                "launches": [(l["entry"], l["schedule"]) for l in prog.launches]}
-        log(f"[bench] config1 relu-sum 1024^2: {cfg1['us']:.1f} us/step -> {cfg1['gbs']:.0f} GB/s")
+        cfg1 = {"us": ms * 1e3, "wall_us": wall_ms * 1e3, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
+                "launch": prog.launches[0]}
+        log(f"[bench] config1 relu-sum 1024^2: {cfg1['us']:.2f} us/step -> {cfg1['gbs']:.0f} GB/s")
+
+        def check_cfg1(got):
+            a, b, c = [x.astype(np.float64) for x in arrays]
+            assert np.allclose(got.ravel(), np.maximum(a * b + c, 0).sum(1), rtol=1e-5, atol=1e-4), "config1 check failed"
+        if not args.no_check:
+            check_cfg1(sets[0][1][out_name].read_array(np.float32, (1024,)))
         del sets
+        cfg1["per_kernel"] = unfused(prog_ast, arg_names, consts, arrays, max(5, min(args.steps, 100)), 5,
+                                     lambda named: check_cfg1(named[out_name].read_array(np.float32, (1024,))))
 
     # ---- config 4: MLP 1024-4096-4096-1024, batch 8192, forward + backward + SGD ---------
     mlp = None
@@ -206,9 +189,9 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
         roots = wl.config4_graph(*ts)
         prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
         prog = hb.HipProgram(dev, prog_ast, options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 1)
+        sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 1)
         k = max(3, min(args.steps, 20))
-        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 3))
+        ms, wall_ms = measure.time_steps(dev, prog, sets, k, min(args.warmup, 3))
         flops = sum(l["flops"] for l in prog.launches)
         algo = sum(l["algo_bytes"] for l in prog.launches)
         mlp = {"ms": ms, "steps": k, "flops": flops, "algo_bytes": algo,
@@ -216,23 +199,29 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
                "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
         log(f"[bench] mlp step (batch {batch}, {dims}): {ms:.2f} ms/step -> {flops / ms / 1e9:.1f} TFLOP/s, "
             f"{batch / ms * 1e3:.0f} samples/s; {mlp['lowered_kernels']} kernels -> {mlp['launches']} launches")
-        if not args.no_check:
-            named = sets[0][1]
-            x, t, params = arrays[0], arrays[1], arrays[2:]
-            h = x
-            for i in range(len(params) // 2):
-                h = h @ params[2 * i].T + params[2 * i + 1]
-                if i + 1 < len(params) // 2:
-                    h = np.tanh(h)
-            d = h.astype(np.float64) - t
-            loss = float((d * d).mean())
+
+        mlp_want = []
+
+        def check_mlp(named):
+            # loss and every updated parameter against the float64 statement of the step
+            from harp_amd.checks import mlp_step
+            if not mlp_want:
+                mlp_want.extend(mlp_step(arrays)[:2])
+            loss, grads = mlp_want
             got_loss = float(named[outs[-1]].read_array(np.float32, (1,))[0])
-            assert abs(got_loss - loss) <= 1e-3 * abs(loss), f"mlp loss check failed: {got_loss} vs {loss}"
-            nb = params[-1].astype(np.float64) - 1e-3 * (2.0 * d / d.size).sum(0)
-            got_b = named[outs[-2]].read_array(np.float32, (dims[-1],))
-            assert np.allclose(got_b, nb, rtol=1e-4, atol=1e-7), "mlp bias update check failed"
-            mlp["loss"] = got_loss
+            assert abs(got_loss - loss) <= 1e-5 * abs(loss), f"mlp loss check failed: {got_loss} vs {loss}"
+            for name, p, g in zip(outs[:-1], arrays[2:], grads):
+                got = named[name].read_array(np.float32, p.shape)
+                assert np.allclose(got, p - 1e-3 * g, rtol=1e-5, atol=1e-7), f"mlp update of {p.shape} check failed"
+            return got_loss
+        if not args.no_check:
+            mlp["loss"] = check_mlp(sets[0][1])
         del sets
+        dev.trim()
+        mlp["per_kernel"] = unfused(prog_ast, arg_names, consts, arrays, 3, 1, check_mlp)
+        if mlp["per_kernel"]:
+            log(f"[bench] mlp step, per-kernel path: {mlp['per_kernel']['ms_per_step']:.2f} ms/step, "
+                f"{mlp['per_kernel']['launches']} launches")
 
     # ---- config 5: MNIST-shaped CNN, batch 256, forward + backward + SGD update ------------
     cnn = None
@@ -244,26 +233,41 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
         roots = wl.config5_graph(*ts, lr=1e-2)
         prog_ast, arg_names, outs, consts, plain = wl.lower_multi(ts, roots)
         prog = hb.HipProgram(dev, prog_ast, options)
-        sets = make_sets(dev, hb, prog, arg_names, consts, arrays, 1)
+        sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 1)
         k = max(3, min(args.steps, 50))
-        ms, wall_ms = time_steps(dev, hb, prog, sets, k, min(args.warmup, 5))
+        ms, wall_ms = measure.time_steps(dev, prog, sets, k, min(args.warmup, 5))
         cnn = {"ms": ms, "steps": k, "flops": sum(l["flops"] for l in prog.launches),
                "algo_bytes": sum(l["algo_bytes"] for l in prog.launches),
                "lowered_kernels": len(plain.args), "launches": len(prog.launches),
                "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
-        from harp_amd import measure
         gms, gwall = measure.time_replays(dev, prog, sets, k, min(args.warmup, 5))
         cnn["graph_ms"], cnn["graph_wall_ms"], cnn["wall_ms"] = gms, gwall, wall_ms
         log(f"[bench] cnn step replayed as one HIP graph: {gms:.3f} ms/step (host wall {gwall:.3f} ms; "
             f"eager host wall {wall_ms:.3f} ms)")
         log(f"[bench] cnn step (batch {sizes[0]}): {ms:.3f} ms/step -> {sizes[0] / ms * 1e3:.0f} images/s; "
             f"{cnn['lowered_kernels']} kernels -> {cnn['launches']} launches ({cnn['gemm_launches']} MFMA)")
-        if not args.no_check:
-            named = sets[0][1]
+
+        cnn_want = []
+
+        def check_cnn(named):
+            # loss and every updated parameter against the float64 statement of the step
+            from harp_amd.checks import cnn_step
+            if not cnn_want:
+                cnn_want.extend(cnn_step(arrays[0], arrays[1], arrays[2:]))
+            loss, grads = cnn_want
             got_loss = float(named[outs[-1]].read_array(np.float32, (1,))[0])
-            assert np.isfinite(got_loss) and abs(got_loss - np.log(10.0)) < 0.5, f"cnn loss {got_loss}"
-            cnn["loss"] = got_loss
+            assert abs(got_loss - loss) <= 1e-5 * abs(loss), f"cnn loss check failed: {got_loss} vs {loss}"
+            for name, p, g in zip(outs[:-1], arrays[2:], grads):
+                got = named[name].read_array(np.float32, p.shape)
+                assert np.allclose(got, p - 1e-2 * g, rtol=1e-4, atol=1e-6), f"cnn update of {p.shape} check failed"
+            return got_loss
+        if not args.no_check:
+            cnn["loss"] = check_cnn(sets[0][1])
         del sets
+        cnn["per_kernel"] = unfused(prog_ast, arg_names, consts, arrays, 5, 2, check_cnn)
+        if cnn["per_kernel"]:
+            log(f"[bench] cnn step, per-kernel path: {cnn['per_kernel']['ms_per_step']:.3f} ms/step, "
+                f"{cnn['per_kernel']['launches']} launches")
 
     # ---- CPU baseline: the oracle's unfused C kernels on host cores -------------------------
     cpu = None
@@ -280,19 +284,19 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
         cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
         os.environ["OMP_NUM_THREADS"] = str(cores)
         sec_o, reps_o, _ = baseline.time_graph(wl.config2_graph, arrays, min_seconds=4.0, max_reps=40, openmp=True)
-        result_extra["cpu_baseline_openmp"] = {
+        extra["cpu_baseline_openmp"] = {
             "value": softmax["algo_bytes"] / sec_o / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"full 4096x4096 softmax, the same five kernels with '#pragma omp parallel for' on the "
                       f"outer loop (gcc -O3 -ffast-math -fopenmp), median of {reps_o} passes, {sec_o * 1e3:.1f} ms/pass"}
         log(f"[bench] cpu baseline softmax, OpenMP: {sec_o * 1e3:.1f} ms/pass -> "
-            f"{result_extra['cpu_baseline_openmp']['value']:.1f} GB/s ({cores} cores)")
+            f"{extra['cpu_baseline_openmp']['value']:.1f} GB/s ({cores} cores)")
         if matmul is not None:
             a, b = wl.config3_inputs()
             sub = 8
             sec_m, reps_m, _ = baseline.time_graph(wl.config3_graph, [a[:sub].copy(), b],
                                                    min_seconds=4.0, max_reps=10)
             gflops = 2.0 * sub * 4096 * 4096 / sec_m / 1e9
-            result_extra["cpu_baseline_matmul"] = {
+            extra["cpu_baseline_matmul"] = {
                 "value": gflops / 1e3, "unit": "TFLOP/s", "cores": 1, "kind": "port",
                 "sample": f"{sub} of 4096 rows of A through the reference's ijk kernel "
                           f"(gcc -O3 -ffast-math), median of {reps_m} passes, {sec_m * 1e3:.0f} ms/pass"}
@@ -305,7 +309,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             with exact_mode():
                 sec_p, reps_p, _ = baseline.time_graph(lambda *ts: wl.config4_graph(*ts), arrays,
                                                        min_seconds=4.0, max_reps=3)
-            result_extra["cpu_baseline_mlp"] = {
+            extra["cpu_baseline_mlp"] = {
                 "value": sub / sec_p, "unit": "samples/s", "cores": 1, "kind": "port",
                 "sample": f"batch {sub} of 8192 through the same lowered kernels, unfused "
                           f"(gcc -O3 -ffast-math), median of {reps_p} passes, {sec_p * 1e3:.0f} ms/pass"}
@@ -319,7 +323,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
             with exact_mode():
                 sec_c, reps_c, _ = baseline.time_graph(lambda *ts: wl.config5_graph(*ts, lr=1e-2), arrays,
                                                        min_seconds=4.0, max_reps=10)
-            result_extra["cpu_baseline_cnn"] = {
+            extra["cpu_baseline_cnn"] = {
                 "value": sub / sec_c, "unit": "images/s", "cores": 1, "kind": "port",
                 "sample": f"batch {sub} of 256 through the same lowered kernels, unfused "
                           f"(gcc -O3 -ffast-math), median of {reps_c} passes, {sec_c * 1e3:.0f} ms/pass"}
@@ -327,7 +331,7 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
 
     head = softmax
     out = {
-        "metric": "fused-kernel HBM GB/s (softmax 4096\u00b2)" + (" + fp32 matmul TFLOP/s (4096\u00b3)" if matmul else ""),
+        "metric": "fused-kernel HBM GB/s (softmax 4096²)" + (" + fp32 matmul TFLOP/s (4096³)" if matmul else ""),
         "value": round(head["gbs"], 1) if head else None,
         "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -338,47 +342,60 @@ extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
                    "buffer_sets": args.sets, "options": args.options},
     }
     if head:
-        out["roofline"] = {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
-                           "traffic": measured_traffic(head["launches"][0][0]) if not args.options else None,
-                           "algorithmic_bytes": head["algo_bytes"],
-                           "kernel": head["launches"][0][0], "schedule": head["launches"][0][1]}
+        out["roofline"] = roofline("hbm", head["gbs"], "GB/s", head["algo_bytes"], head["launch"])
+        if head["per_kernel"]:
+            extra["per_kernel_path"] = {"config2_softmax_4096": head["per_kernel"]}
     if cpu:
         out["cpu_baseline"] = cpu
     if matmul:
-        result_extra["matmul_4096"] = {
+        extra["matmul_4096"] = {
             "value": round(matmul["tflops"], 2), "unit": "TFLOP/s", "ms_per_step": round(matmul["ms"], 4),
             "steps": matmul["steps"], "dtype": "f32",
-            "roofline": {"bound": "mfma", "achieved": round(matmul["tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(matmul["tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
-                         "traffic": measured_traffic(matmul["launches"][0][0]) if not args.options else None,
-                         "kernel": matmul["launches"][0][0],
-                         "schedule": matmul["launches"][0][1]}}
+            "roofline": roofline("mfma", matmul["tflops"], "TFLOP/s", matmul["flops"], matmul["launch"]),
+            "per_kernel_path": "the same single kernel on both paths"}
     if cfg1:
-        result_extra["config1_relu_sum_1024"] = {"us_per_step": round(cfg1["us"], 2),
-                                                 "value": round(cfg1["gbs"], 1), "unit": "GB/s",
-                                                 "schedule": cfg1["launches"][0][1]}
+        extra["config1_relu_sum_1024"] = {
+            "us_per_step": round(cfg1["us"], 2), "host_us_per_step": round(cfg1["wall_us"], 2),
+            "value": round(cfg1["gbs"], 1), "unit": "GB/s", "schedule": cfg1["launch"]["schedule"],
+            "roofline": roofline("hbm", cfg1["gbs"], "GB/s", cfg1["algo_bytes"], cfg1["launch"]),
+            "note": "12.6 MB per launch is 1.6 us at peak: the step is bound by launch and drain of one small grid"}
+        if cfg1["per_kernel"]:
+            extra.setdefault("per_kernel_path", {})["config1_relu_sum_1024"] = cfg1["per_kernel"]
     if mlp:
-        result_extra["config4_mlp_step"] = {
+        tflops = mlp["flops"] / mlp["ms"] / 1e9
+        extra["config4_mlp_step"] = {
             "value": round(8192 / mlp["ms"] * 1e3, 1), "unit": "samples/s", "ms_per_step": round(mlp["ms"], 3),
-            "steps": mlp["steps"], "tflops": round(mlp["flops"] / mlp["ms"] / 1e9, 2),
+            "steps": mlp["steps"], "tflops": round(tflops, 2),
             "algorithmic_bytes": mlp["algo_bytes"], "lowered_kernels": mlp["lowered_kernels"],
             "launches": mlp["launches"], "gemm_launches": mlp["gemm_launches"], "loss": mlp.get("loss"),
+            "roofline": roofline("mfma", tflops, "TFLOP/s", mlp["flops"]),
             "workload": "MLP 1024-4096-4096-1024, batch 8192: forward, MSE, exact backward, SGD update, one Program"}
+        if mlp["per_kernel"]:
+            extra.setdefault("per_kernel_path", {})["config4_mlp_step"] = mlp["per_kernel"]
     if cnn:
-        result_extra["config5_cnn_step"] = {
+        # the step's roofline: whichever of its algorithmic bytes at HBM peak and its flops at MFMA
+        # peak takes longer
+        t_hbm = cnn["algo_bytes"] / (HBM_PEAK_GBS * 1e9)
+        t_mfma = cnn["flops"] / (FP32_MFMA_PEAK_TFLOPS * 1e12)
+        if t_hbm >= t_mfma:
+            roof = roofline("hbm", cnn["algo_bytes"] / (cnn["ms"] * 1e-3) / 1e9, "GB/s", cnn["algo_bytes"])
+        else:
+            roof = roofline("mfma", cnn["flops"] / cnn["ms"] / 1e9, "TFLOP/s", cnn["flops"])
+        extra["config5_cnn_step"] = {
             "value": round(256 / cnn["ms"] * 1e3, 1), "unit": "images/s", "ms_per_step": round(cnn["ms"], 4),
-            "steps": cnn["steps"], "algorithmic_bytes": cnn["algo_bytes"],
+            "steps": cnn["steps"], "algorithmic_bytes": cnn["algo_bytes"], "algorithmic_flops": cnn["flops"],
             "lowered_kernels": cnn["lowered_kernels"], "launches": cnn["launches"],
-            "gemm_launches": cnn["gemm_launches"], "loss": cnn.get("loss"),
+            "gemm_launches": cnn["gemm_launches"], "loss": cnn.get("loss"), "roofline": roof,
             "ms_per_step_hip_graph": round(cnn["graph_ms"], 4),
             "host_ms_per_step": {"eager": round(cnn["wall_ms"], 4), "hip_graph": round(cnn["graph_wall_ms"], 4)},
             "workload": "CNN 1x28x28: conv3x3(32)+relu+pool, conv3x3(64)+relu+pool, fc 3136-128-10, "
                         "cross-entropy; batch 256 forward + exact backward, plus the SGD update (more than the "
                         "configuration asks for, inside the timed region), one Program"}
-    result_extra["device"] = {"name": props["name"] or "MI355X (name not reported by the runtime)", "arch": props["arch"],
-                              "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
-    out["extra"] = result_extra
+        if cnn["per_kernel"]:
+            extra.setdefault("per_kernel_path", {})["config5_cnn_step"] = cnn["per_kernel"]
+    extra["device"] = {"name": props["name"] or "MI355X (name not reported by the runtime)", "arch": props["arch"],
+                       "compute_units": props["compute_units"], "clock_khz": props["clock_khz"]}
+    out["extra"] = extra
     print(json.dumps(out), flush=True)
 
 

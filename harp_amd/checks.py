@@ -1,7 +1,11 @@
-"""float64 numpy restatement of the config-5 CNN step (conv3x3 pad 1 + relu + maxpool2, twice;
-fc + relu; fc; cross-entropy), forward and backward, for checking the graph-built step.
-Max-pool ties share the gradient (every maximal element receives it), as the graph's
-equality mask does."""
+"""float64 numpy statements of the two training steps, for checking what the backend computes
+(the benchmark's result checks and the parity tests use them; they are plain mathematics, not the
+reference's lowering).
+
+`cnn_step`: the config-5 CNN (conv3x3 pad 1 + relu + maxpool2, twice; fc + relu; fc;
+cross-entropy), forward and backward.  Max-pool ties share the gradient (every maximal element
+receives it), as the graph's equality mask does.  `mlp_step`: the config-4 MLP with tanh and
+mean-squared error."""
 
 import numpy as np
 def im2col(xp, kh, kw):
@@ -61,3 +65,26 @@ def cnn_step(x, onehot, params):
     gz1 = pool_bwd(gp1, xr1, p1) * (z1 >= 0)
     _, gw1, gb1 = conv_bwd(gz1, x, w1, cols1)
     return loss, [gw1, gb1, gw2, gb2, gw3, gb3, gw4, gb4]
+
+
+def mlp_step(arrays):
+    """(loss, gradient of every parameter, network output) of the config-4 step for
+    [x, target, w1, b1, w2, b2, ...], in float64."""
+    x, t = arrays[0].astype(np.float64), arrays[1].astype(np.float64)
+    ps = [p.astype(np.float64) for p in arrays[2:]]
+    hs, pre = [x], []
+    nl = len(ps) // 2
+    for i in range(nl):
+        z = hs[-1] @ ps[2 * i].T + ps[2 * i + 1]
+        pre.append(z)
+        hs.append(np.tanh(z) if i + 1 < nl else z)
+    d = hs[-1] - t
+    loss = (d * d).mean()
+    gz = 2 * d / d.size
+    grads = [None] * len(ps)
+    for i in range(nl - 1, -1, -1):
+        grads[2 * i] = gz.T @ hs[i]
+        grads[2 * i + 1] = gz.sum(0)
+        if i > 0:
+            gz = (gz @ ps[2 * i]) * (1 - np.tanh(pre[i - 1]) ** 2)
+    return loss, grads, hs[-1]

@@ -8,11 +8,18 @@ events on the launch stream with a device synchronisation on both sides.
 
 from __future__ import annotations
 
+import hashlib
+import json
+import os
 import time
 
 import numpy as np
 
 from . import backend as hb
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix peak
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "profiles", "traffic.json")
 
 
 def make_sets(dev, prog, arg_names, const_inputs, arrays, nsets):
@@ -69,3 +76,149 @@ def time_replays(dev, prog, sets, steps, warmup):
     dev.sync()
     wall = (time.perf_counter() - t0) * 1e3
     return e0.elapsed_ms(e1) / steps, wall / steps
+
+
+# ---------------------------------------------------------------------------
+# the per-kernel path: what the reference's unmodified executor drives
+# ---------------------------------------------------------------------------
+
+class PerKernelPath:
+    """The kernels of a lowered Program compiled one by one (`compile_ast`) and run as
+    `execute_graph` runs them (src/backend/executor.rs:245-372): per kernel, allocate the
+    outputs zero-filled, `Kernel::execute(inputs, outputs)` synchronously, publish the outputs
+    by name for the kernels that follow.  Nothing is fused across kernels and every
+    intermediate buffer exists."""
+
+    def __init__(self, dev, program_ast, options=None):
+        from .frontend import AstNode
+        self.dev = dev
+        self.table = {b["name"]: b for b in program_ast.attrs["buffers"]}
+        self.kernels = []
+        for k in program_ast.args:
+            params = [p for p in k.attrs["params"] if p.dtype.is_ptr()]
+            kern = hb.HipKernel(dev, AstNode.program([k]), options)
+            self.kernels.append((kern, [p.name for p in params if not p.mutable],
+                                 [p.name for p in params if p.mutable]))
+        self.launches = [l for kern, _, _ in self.kernels for l in kern.launches]
+
+    def _nbytes(self, name):
+        b = self.table[name]
+        n = b["dtype"].itemsize()
+        for d in b["shape"]:
+            n *= int(d)
+        return n
+
+    def step(self, inputs):
+        """One pass; `inputs` maps buffer name -> HipBuffer.  Returns all buffers by name."""
+        named = dict(inputs)
+        for kern, ins, outs in self.kernels:
+            out_bufs = [self.dev.alloc(self._nbytes(n)) for n in outs]
+            kern.execute([named[n] for n in ins], out_bufs)
+            named.update(zip(outs, out_bufs))
+        return named
+
+    def time(self, inputs, steps, warmup):
+        """Wall-clock ms per step (every launch is synchronous, so wall time is device time
+        plus what the host spends between launches, as it would be for the reference)."""
+        for _ in range(warmup):
+            self.step(inputs)
+        self.dev.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.step(inputs)
+        self.dev.sync()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def upload_inputs(dev, program_ast, arg_names, const_inputs, arrays):
+    """Device buffers for every input row of the program's table, by name."""
+    named = {}
+    for b in program_ast.attrs["buffers"]:
+        if b["role"] not in ("input", "ones", "zeros"):
+            continue
+        n = b["dtype"].itemsize()
+        for d in b["shape"]:
+            n *= int(d)
+        buf = dev.alloc(n)
+        if b["name"] in arg_names:
+            buf.write_array(np.ascontiguousarray(arrays[arg_names.index(b["name"])]))
+        else:
+            fill = {"ones": 1.0, "zeros": 0.0, "scalar": 1.0}[const_inputs.get(b["name"], b["role"])]
+            buf.write_array(np.full(n // 4, fill, dtype=np.float32))
+        named[b["name"]] = buf
+    return named
+
+
+# ---------------------------------------------------------------------------
+# counter-derived traffic, tied to the kernel source it was measured on
+# ---------------------------------------------------------------------------
+
+def source_hash(source: str) -> str:
+    return hashlib.sha1(source.encode()).hexdigest()
+
+
+def measured_traffic(entry: str, source: str):
+    """(HBM bytes per launch, stale?) for kernel `entry` from profiles/traffic.json (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size).  The figure counts only
+    while the generated source is the one it was measured on: otherwise (None, True).
+    (None, False): the kernel is not in the file."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)["kernels"][entry]
+    except (OSError, KeyError, ValueError):
+        return None, False
+    if rec.get("source_sha1") != source_hash(source):
+        return None, True
+    return rec["traffic_bytes"], False
+
+
+# ---------------------------------------------------------------------------
+# calibration kernels (ceilings the profiles quote; not results)
+# ---------------------------------------------------------------------------
+
+MFMA_PEAK_SOURCE = """
+typedef float f16v __attribute__((ext_vector_type(16)));
+extern "C" __global__ void __launch_bounds__(256) eh_mfma_peak(float* out) {
+  f16v acc[4];
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  float a = threadIdx.x * 1e-3f, b = blockIdx.x * 1e-3f;
+  for (int it = 0; it < %d; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+  }
+  float s = 0.0f;
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += acc[i][r];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+"""
+
+
+def mfma_issue_rate(dev, iters=4096, waves_per_cu=8, reps=20):
+    """TFLOP/s of v_mfma_f32_32x32x2_f32 issued back to back with operands in registers."""
+    blocks = dev.props["compute_units"] * waves_per_cu // 4
+    mod = hb.HipModule(dev, hb.compile_source(MFMA_PEAK_SOURCE % iters), "eh_mfma_peak")
+    out = hb.HipBuffer(dev, [blocks * 256 * 4], None, nbytes=blocks * 256 * 4)
+    for _ in range(3):
+        mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+    dev.sync()
+    e0, e1 = hb.Event(dev), hb.Event(dev)
+    e0.record()
+    for _ in range(reps):
+        mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+    e1.record()
+    e1.sync()
+    ms = e0.elapsed_ms(e1) / reps
+    flops = blocks * 4 * iters * 4 * (32 * 32 * 2 * 2)
+    return flops / ms / 1e9, blocks, ms
+
+
+def copy_rate(dev, shape=(4096, 4096), steps=200, warmup=20, nsets=4, options=None):
+    """GB/s of a plain fp32 copy of `shape` (read + write), rotating buffer sets: the ceiling a
+    memory-bound kernel of that size can reach, and the kernel the traffic counters are scaled by."""
+    from . import workloads as wl
+    x = np.zeros(shape, np.float32)
+    ast, arg_names, _out, consts, _ = wl.lower_with_table([shape], lambda t: t.contiguous())
+    prog = hb.HipProgram(dev, ast, options)
+    sets = make_sets(dev, prog, arg_names, consts, [x], nsets)
+    ms, _ = time_steps(dev, prog, sets, steps, warmup)
+    return 2 * x.nbytes / (ms * 1e-3) / 1e9, prog.launches[0], ms

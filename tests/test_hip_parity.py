@@ -745,7 +745,7 @@ def test_config5_cnn_training_step(frontend, hip, sizes, fuse):
     parameter gradient and the loss match the C oracle running the same exact-mode graph,
     and a float64 numpy CNN."""
     from harp_amd import workloads as wl
-    from cnn_reference import cnn_step
+    from harp_amd.checks import cnn_step
     arrays = wl.config5_inputs(*sizes, seed=77)
     ref = _cnn_step_on(frontend, "c", arrays)
     got = _cnn_step_on(frontend, "hip", arrays, fuse)
@@ -762,7 +762,7 @@ def test_config5_cnn_step_with_sgd_update(frontend, hip):
     """The form the benchmark times: the same step with p - lr * gradient for every parameter
     as the roots (the updates ride on the gradient contractions where they can)."""
     from harp_amd import workloads as wl
-    from cnn_reference import cnn_step
+    from harp_amd.checks import cnn_step
     arrays = wl.config5_inputs(8, 28, 32, 64, 128, 10, seed=78)
     ref = _cnn_step_on(frontend, "c", arrays, lr=0.05)
     got = _cnn_step_on(frontend, "hip", arrays, lr=0.05)

@@ -252,7 +252,7 @@ def test_exact_unfold_views_and_cnn_step(frontend):
     cross_entropy_loss plus exact VJPs matches a float64 numpy CNN."""
     from harp_amd import workloads as wl
     from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
-    from cnn_reference import cnn_step
+    from harp_amd.checks import cnn_step
     frontend.set_device_str("c")
     x = np.arange(2 * 2 * 4 * 4, dtype=np.float32).reshape(2, 2, 4, 4)
     win = np.empty((2, 2, 2, 2, 3, 3), np.float32)
