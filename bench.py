@@ -143,7 +143,7 @@ def main():
         prog = hb.HipProgram(dev, prog_ast, options)
         sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 2)
         k = max(5, min(args.steps, 50))
-        ms, _ = measure.time_steps(dev, prog, sets, k, min(args.warmup, 5))
+        ms, _ = measure.time_steps(dev, prog, sets, k, args.warmup)
         flops = sum(l["flops"] for l in prog.launches)
         matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k, "flops": flops, "launch": prog.launches[0]}
         log(f"[bench] matmul 4096^3: {ms:.3f} ms/step -> {matmul['tflops']:.1f} TFLOP/s "

@@ -411,6 +411,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_fold") o.gemm_fold = as_int() != 0;
     else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
     else if (k == "gemm_dma") o.gemm_dma = as_int() != 0;
+    else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;
     else if (k == "nontemporal") o.nontemporal = as_int();
     else if (k == "normalize") o.normalize = as_int() != 0;

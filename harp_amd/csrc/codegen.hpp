@@ -28,6 +28,7 @@ struct GenOptions {
   int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
   int gemm_setprio = 0;               // wave priority during the multiply loop
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
+  bool gemm_mix = true;               // LDS operand reads interleaved with the MFMAs of the block before
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
   bool gemm_merge_batch = false;      // per-batch contractions summed over the batch become one contraction
   bool gemm_epilogue = true;          // run elementwise consumers of a contraction on its accumulators

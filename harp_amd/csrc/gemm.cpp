@@ -340,6 +340,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     os << "#define EH_WAVES_PER_SIMD " << std::min(8, waves) << "\n";
   }
   os << "#define EH_SETPRIO " << std::max(0, std::min(3, opt.gemm_setprio)) << "\n";
+  os << "#define EH_MIX " << (opt.gemm_mix ? 1 : 0) << "\n";
   os << kGemmSource;
   ls.source = os.str();
   const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;

@@ -64,6 +64,26 @@
 #ifndef EH_SETPRIO
 #define EH_SETPRIO 0     // wave priority while multiplying
 #endif
+#ifndef EH_MIX
+#define EH_MIX 1         // LDS operand reads are issued one at a time between the MFMAs of the block before
+#endif
+// The operand reads of a k-block and the MFMAs of the block before it, as one scheduling region:
+// with EH_MIX the reads go out one after every MFMA instead of all at once.  Sixteen waves that
+// leave a barrier together and each issue all their reads first fill the LDS queue, and a wave
+// whose read cannot issue cannot issue the MFMAs behind it either (in-order issue): the matrix
+// cores then wait for the LDS to drain.  Spread out, a read is still more than half a block
+// (hundreds of cycles) ahead of its first use.  0x008: MFMA, 0x100: LDS read.
+#if EH_MIX
+#define EH_MIX_REGION()                                         \
+  _Pragma("unroll") for (int eh_g = 0; eh_g < 12; ++eh_g) {     \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          \
+  }
+#define EH_FETCH_FENCE()
+#else
+#define EH_MIX_REGION()
+#define EH_FETCH_FENCE() __builtin_amdgcn_sched_barrier(0)
+#endif
 
 typedef float eh_f16v __attribute__((ext_vector_type(16)));
 typedef float eh_f4v __attribute__((ext_vector_type(4)));
@@ -371,8 +391,9 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #pragma unroll
     for (int j = 0; j < NBLK - 1; ++j) {
       fetch(a_cur, b_cur, j + 1, (j + 1) & 1);
-      __builtin_amdgcn_sched_barrier(0);   // reads of the next block stay ahead of these MFMAs
+      EH_FETCH_FENCE();                    // (without EH_MIX) reads of the next block stay ahead of these MFMAs
       multiply(j & 1);
+      EH_MIX_REGION();
       __builtin_amdgcn_sched_barrier(0);
     }
 #if EH_SETPRIO
@@ -381,8 +402,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
     if (more) sstore(a_nxt, b_nxt);
     __syncthreads();
     if (more) fetch(a_nxt, b_nxt, 0, NBLK & 1);
-    __builtin_amdgcn_sched_barrier(0);
+    EH_FETCH_FENCE();
     multiply((NBLK - 1) & 1);
+    EH_MIX_REGION();
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   fetch(As0, Bs0, 0, 0);

@@ -89,7 +89,7 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
  *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
- *      gemm_epilogue, gemm_dma, gemm_merge_batch, nontemporal, normalize, allow_serial.
+ *      gemm_epilogue, gemm_dma, gemm_mix, gemm_merge_batch, nontemporal, normalize, allow_serial.
  *      A kernel that no schedule recognises, would run in a single work-item and loops more than
  *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1. ----------------- */
 typedef struct eh_launch_info {
