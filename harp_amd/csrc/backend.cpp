@@ -267,6 +267,7 @@ void HipDevice::release(void* ptr, size_t bytes) {
       return;
     }
   }
+  auto lk = stream_lock();
   (void)hipStreamSynchronize(stream_);
   (void)hipFree(ptr);
 }
@@ -279,6 +280,7 @@ void HipDevice::trim() {
     pooled_bytes_ = 0;
   }
   if (blocks.empty()) return;
+  auto lk = stream_lock();
   (void)hipStreamSynchronize(stream_);
   for (auto& kv : blocks) (void)hipFree(kv.second);
 }
@@ -286,6 +288,7 @@ void HipDevice::trim() {
 void HipDevice::make_current() const { check(hipSetDevice(index_), "hipSetDevice"); }
 
 void HipDevice::synchronize() const {
+  auto lk = stream_lock();
   make_current();
   check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
 }
@@ -295,6 +298,7 @@ std::shared_ptr<HipKernel> HipDevice::load(const Binary& bin, const std::string&
 }
 
 HipBuffer::HipBuffer(HipDevice* dev, size_t bytes) : dev_(dev), bytes_(bytes) {
+  auto lk = dev_->stream_lock();
   dev_->make_current();
   if (bytes_ == 0) return;
   ptr_ = dev_->allocate(bytes_);
@@ -316,6 +320,7 @@ void HipBuffer::write_from_host(const void* src, size_t bytes) {
   if (bytes != bytes_)
     throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(bytes));
   if (!bytes_) return;
+  auto lk = dev_->stream_lock();
   dev_->make_current();
   check(hipMemcpyAsync(ptr_, src, bytes_, hipMemcpyHostToDevice, dev_->stream()), "hipMemcpyAsync(H2D)");
   check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
@@ -325,6 +330,7 @@ void HipBuffer::read_to_host(void* dst, size_t bytes) const {
   if (bytes != bytes_)
     throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(bytes));
   if (!bytes_) return;
+  auto lk = dev_->stream_lock();
   dev_->make_current();
   check(hipMemcpyAsync(dst, ptr_, bytes_, hipMemcpyDeviceToHost, dev_->stream()), "hipMemcpyAsync(D2H)");
   check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
@@ -334,6 +340,7 @@ void HipBuffer::copy_from(const HipBuffer& src) {
   if (src.bytes_ != bytes_)
     throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(src.bytes_));
   if (!bytes_) return;
+  auto lk = dev_->stream_lock();
   dev_->make_current();
   check(hipMemcpyAsync(ptr_, src.ptr_, bytes_, hipMemcpyDeviceToDevice, dev_->stream()), "hipMemcpyAsync(D2D)");
 }
@@ -352,6 +359,7 @@ HipKernel::HipKernel(HipDevice* dev, const Binary& bin, const std::string& entry
 
 HipKernel::~HipKernel() {
   if (module_) {
+    auto lk = dev_->stream_lock();
     (void)hipSetDevice(dev_->index());
     (void)hipStreamSynchronize(dev_->stream());
     (void)hipModuleUnload(module_);
@@ -360,6 +368,7 @@ HipKernel::~HipKernel() {
 
 void HipKernel::launch(const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
                        const std::vector<void*>& device_ptrs) const {
+  auto lk = dev_->stream_lock();
   std::vector<void*> vals = device_ptrs;
   std::vector<void*> params(vals.size());
   for (size_t i = 0; i < vals.size(); ++i) params[i] = &vals[i];
@@ -491,6 +500,7 @@ void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
 }
 
 void HipProgram::launch_spans(const std::vector<Span>& bound) {
+  auto lk = dev_->stream_lock();               // the program's launches go out as one run
   for (size_t l = 0; l < plan_.launches.size(); ++l) {
     const LaunchSpec& ls = plan_.launches[l];
     std::vector<void*> ptrs;
@@ -509,6 +519,7 @@ void HipProgram::launch_spans(const std::vector<Span>& bound) {
 
 void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
   std::lock_guard<std::mutex> lk(mu_);
+  auto sl = dev_->stream_lock();               // binding may allocate (and fill) temps
   launch_all(bind(bufs, n));
   if (sync) dev_->synchronize();
 }
@@ -528,6 +539,7 @@ size_t HipProgram::static_scratch_needed() const {
 
 void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
   std::lock_guard<std::mutex> lk(mu_);
+  auto sl = dev_->stream_lock();
   const size_t total = plan_.buffers.size();
   if (n > total) throw Error("program binds " + std::to_string(total) + " buffers, " + std::to_string(n) + " given");
   const size_t need = static_scratch_needed();
@@ -566,6 +578,9 @@ void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
 
 HipGraph::HipGraph(HipProgram* prog, HipBuffer* const* bufs, size_t n) : dev_(prog->device()) {
   std::lock_guard<std::mutex> lk(prog->mu_);
+  // held across the whole capture: whatever another thread wants to put on this stream (a buffer
+  // fill, a copy, another program's launches, a synchronisation) waits until the capture ended
+  auto sl = dev_->stream_lock();
   // binding allocates missing temps: all of it happens before the capture starts, the capture
   // itself records kernel launches only (no memset or copy nodes)
   std::vector<HipBuffer*> bound = prog->bind(bufs, n);
@@ -605,6 +620,7 @@ void HipGraph::drop() {
 }
 
 HipGraph::~HipGraph() {
+  auto sl = dev_->stream_lock();
   (void)hipSetDevice(dev_->index());
   (void)hipStreamSynchronize(dev_->stream());
   if (exec_) (void)hipGraphExecDestroy(exec_);
@@ -612,6 +628,7 @@ HipGraph::~HipGraph() {
 }
 
 void HipGraph::replay(bool sync) {
+  auto sl = dev_->stream_lock();
   dev_->make_current();
   check(hipGraphLaunch(exec_, dev_->stream()), "hipGraphLaunch");
   if (sync) dev_->synchronize();

@@ -57,6 +57,12 @@ class HipDevice {
 
   int index() const { return index_; }
   hipStream_t stream() const { return stream_; }
+  // Everything that enqueues on (or waits for) the device's one stream holds this lock while it
+  // does: buffer fills and copies, launches of a program, graph replays, synchronisation -- and
+  // a graph capture holds it from begin to end, so that no other thread's work is recorded into
+  // the graph instead of running (or fails for touching a capturing stream).  Recursive: an
+  // execute that synchronises at its end takes it twice.
+  std::unique_lock<std::recursive_mutex> stream_lock() const { return std::unique_lock<std::recursive_mutex>(stream_mu_); }
   const DeviceProfile& profile() const { return profile_; }
   void make_current() const;
   void synchronize() const;
@@ -81,6 +87,7 @@ class HipDevice {
   int index_;
   hipStream_t stream_ = nullptr;
   DeviceProfile profile_;
+  mutable std::recursive_mutex stream_mu_;
   std::mutex pool_mu_;
   std::multimap<size_t, void*> pool_;  // size -> free block
   size_t pooled_bytes_ = 0, pool_limit_ = 0;

@@ -442,6 +442,7 @@ int eh_module_launch(eh_module* mod, const unsigned grid[3], const unsigned bloc
       if (args[i]->buf.device() != mod->dev) throw Error("argument " + std::to_string(i) + " lives on another device");
       ptrs.push_back(args[i]->buf.device_ptr());
     }
+    auto lk = mod->dev->stream_lock();
     mod->dev->make_current();
     mod->kernel->launch(grid, block, lds_bytes, ptrs);
     if (sync) mod->dev->synchronize();
@@ -467,6 +468,7 @@ int eh_event_create(eh_device* dev, eh_event** out) {
 int eh_event_record(eh_event* ev) {
   REQUIRE(ev, "event is NULL");
   return guard([&] {
+    auto lk = ev->dev->stream_lock();
     ev->dev->make_current();
     hipError_t r = hipEventRecord(ev->ev, ev->dev->stream());
     if (r != hipSuccess) throw Error(std::string("hipEventRecord: ") + hipGetErrorString(r) + " (hip error)");

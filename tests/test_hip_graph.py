@@ -78,3 +78,49 @@ def test_record_rejects_a_missing_input(hip):
     with pytest.raises(Exception, match="MissingInput"):
         prog.record(prog.bind(named))
     prog.run(sets[0][0], sync=True)          # the stream is still usable (no capture left open)
+
+
+def test_other_threads_may_use_the_device_while_a_graph_is_recorded(hip):
+    """Recording captures the device's one stream.  A second thread that allocates (a fill),
+    writes, reads back and runs another program on the same device meanwhile must neither fail
+    nor end up inside the graph: its work waits for the capture to end.  Every recorded graph
+    still replays to the eager result, and everything the other thread read back is right."""
+    import threading
+    hb = hip
+    dev = hb.HipDevice(0)
+    prog, sets, arg_names, outs, arrays = _cnn_sets(hb, dev, 4, seed=94)
+    prog.run(sets[0][0], sync=True)
+    want = _read_outputs(sets[0][1], outs)
+    from harp_amd import workloads as wl
+    ast, names, out, consts, _ = wl.lower_with_table([(64, 96)], lambda t: t * t + t)
+    other = hb.HipProgram(dev, ast, None)
+    stop, errors, rounds = threading.Event(), [], [0]
+
+    def churn():
+        rng = np.random.default_rng(5)
+        try:
+            while not stop.is_set():
+                x = rng.normal(0, 1, (64, 96)).astype(np.float32)
+                xin, res = dev.alloc(x.nbytes), dev.alloc(x.nbytes)        # alloc = a fill on the stream
+                assert not res.read_array(np.float32).any()
+                xin.write_array(x)
+                other.run(other.bind({names[0]: xin, out: res}), sync=True)
+                assert np.array_equal(res.read_array(np.float32, x.shape), x * x + x)
+                rounds[0] += 1
+        except Exception as e:                                             # noqa: BLE001
+            errors.append(e)
+
+    t = threading.Thread(target=churn)
+    t.start()
+    try:
+        for _ in range(12):
+            graph = prog.record(sets[1][0])
+            graph.replay(sync=True)
+            for g, w in zip(_read_outputs(sets[1][1], outs), want):
+                assert np.array_equal(g, w)
+            del graph
+    finally:
+        stop.set()
+        t.join(60)
+    assert not errors, errors
+    assert rounds[0] > 0
