@@ -110,6 +110,37 @@ def build_capi_client() -> str:
     return CLIENT
 
 
+FUZZ_SRC = os.path.join(os.path.dirname(HERE), "tests", "host_fuzz.cpp")
+FUZZ = os.path.join(os.path.dirname(HERE), "tests", "host_fuzz.bin")
+GENERATOR_SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "gemm.cpp"]   # no HIP runtime involved
+
+
+def build_host_fuzz(force: bool = False) -> str:
+    """tests/host_fuzz.cpp with the AST reader, the normaliser and the planner, built by g++ with
+    AddressSanitizer and UndefinedBehaviorSanitizer (any finding aborts): host code only."""
+    wrap_templates()
+    srcs = [os.path.join(CSRC, s) for s in GENERATOR_SOURCES] + [FUZZ_SRC]
+    deps = srcs + [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith((".hpp", ".inc"))] + \
+        [os.path.join(CSRC, t) for t in TEMPLATES]
+    if not force and os.path.exists(FUZZ) and os.path.getmtime(FUZZ) >= max(os.path.getmtime(p) for p in deps):
+        return FUZZ
+    with tempfile.TemporaryDirectory() as tmp:
+        procs, objs = [], []
+        for s in srcs:
+            o = os.path.join(tmp, os.path.basename(s) + ".o")
+            objs.append(o)
+            cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                   "-fno-omit-frame-pointer", "-Wall", "-Wextra", "-c", s, "-o", o]
+            procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+        for cmd, p in procs:
+            out, err = p.communicate()
+            if p.returncode != 0:
+                raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), out, err))
+        # the sanitizer runtimes linked statically: the binary then runs whatever else is preloaded
+        _run(["g++", "-fsanitize=address,undefined", "-static-libasan", "-static-libubsan", "-o", FUZZ] + objs)
+    return FUZZ
+
+
 if __name__ == "__main__":
     print(build(check="--check" in sys.argv))
     print(build_capi_client())

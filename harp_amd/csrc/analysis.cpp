@@ -1,5 +1,6 @@
 #include "analysis.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace eh {
@@ -32,9 +33,9 @@ std::optional<Affine> affine_of(const Node& n) {
       auto l = affine_of(*n.args[0]);
       auto r = affine_of(*n.args[1]);
       if (!l || !r) return std::nullopt;
-      l->c += r->c;
+      l->c = add_ck(l->c, r->c);
       for (auto& kv : r->coef) {
-        l->coef[kv.first] += kv.second;
+        l->coef[kv.first] = add_ck(l->coef[kv.first], kv.second);
         if (l->coef[kv.first] == 0) l->coef.erase(kv.first);
       }
       return l;
@@ -46,9 +47,9 @@ std::optional<Affine> affine_of(const Node& n) {
       if (!l->coef.empty() && !r->coef.empty()) return std::nullopt;
       const Affine& k = l->coef.empty() ? *l : *r;   // the constant side
       Affine v = l->coef.empty() ? *r : *l;
-      v.c *= k.c;
+      v.c = mul_ck(v.c, k.c);
       for (auto it = v.coef.begin(); it != v.coef.end();) {
-        it->second *= k.c;
+        it->second = mul_ck(it->second, k.c);
         it = it->second == 0 ? v.coef.erase(it) : std::next(it);
       }
       return v;
@@ -77,8 +78,8 @@ void collect_loads(const Node& e, std::vector<LoadRef>& out, bool guarded) {
 int64_t max_abs_index(const Affine& a, const std::vector<Loop>& loops, const Loop* rloop) {
   int64_t hi = a.c > 0 ? a.c : 0, lo = a.c < 0 ? a.c : 0;
   auto add = [&](const Loop& l) {
-    int64_t k = a.of(l.var) * (l.extent > 0 ? l.extent - 1 : 0);
-    if (k > 0) hi += k; else lo += k;
+    int64_t k = mul_ck(a.of(l.var), l.extent > 0 ? l.extent - 1 : 0);
+    if (k > 0) hi = add_ck(hi, k); else lo = add_ck(lo, k);
   };
   for (const auto& l : loops) add(l);
   if (rloop) add(*rloop);
@@ -259,6 +260,58 @@ std::optional<NestKernel> extract_nest(const Node& kernel) {
     for (const auto& a : n->args) stack.push_back(a.get());
   }
   return k;
+}
+
+namespace {
+
+// Sizes are caller-supplied.  Everything the planner later multiplies -- loop extents, strides,
+// footprints, largest reachable indices -- is bounded here once (with checked arithmetic), so
+// that the products it forms stay far inside 64 bits: a loop runs at most 2^33 times, a nest at
+// most 2^48, a constant is at most 2^46 in magnitude, and no index expression can reach beyond
+// 2^46 elements.  Larger programs are refused, not wrapped.
+constexpr int64_t kMaxExtent = int64_t{1} << 33, kMaxNest = int64_t{1} << 48, kMaxIndex = int64_t{1} << 46;
+
+void validate_node(const Node& n, std::vector<Loop>& loops, int64_t nest) {
+  auto too_big = [](const std::string& what) {
+    throw Error(what + " is beyond the sizes this backend plans for: not supported");
+  };
+  if (n.op == Op::Const && !n.dtype.is_float() && (n.ival > kMaxIndex || n.ival < -kMaxIndex)) too_big("an integer constant");
+  if (n.op == Op::Range && n.args.size() == 4) {
+    for (int i = 0; i < 3; ++i) validate_node(*n.args[i], loops, nest);
+    int64_t extent = 1;
+    const Node &s = *n.args[0], &st = *n.args[1], &e = *n.args[2];
+    if (s.op == Op::Const && st.op == Op::Const && e.op == Op::Const && !s.dtype.is_float() && !e.dtype.is_float() &&
+        !st.dtype.is_float() && st.ival >= 1)
+      extent = e.ival > s.ival ? (e.ival - s.ival + st.ival - 1) / st.ival : 0;
+    if (extent > kMaxExtent) too_big("the extent of loop '" + n.name + "'");
+    const int64_t inner = mul_ck(nest, std::max<int64_t>(extent, 1));
+    if (inner > kMaxNest) too_big("the iteration count of the nest around loop '" + n.name + "'");
+    loops.push_back({n.name, extent});
+    validate_node(*n.args[3], loops, inner);
+    loops.pop_back();
+    return;
+  }
+  const bool indexed = (n.op == Op::Load || n.op == Op::Store || n.op == Op::AtomicAdd || n.op == Op::AtomicMax) &&
+                       n.args.size() >= 2;
+  if (indexed)
+    if (auto a = affine_of(*n.args[1]))
+      if (max_abs_index(*a, loops, nullptr) > kMaxIndex) too_big("an index of buffer access in a kernel");
+  for (const auto& c : n.args) validate_node(*c, loops, nest);
+}
+
+}  // namespace
+
+void validate_sizes(const Node& n) {
+  for (const auto& b : n.buffers) {
+    int64_t numel = 1;
+    for (auto d : b.shape) {
+      if (d < 0) throw Error("buffer '" + b.name + "' has a negative dimension");
+      numel = mul_ck(numel, std::max<int64_t>(d, 1));
+      if (numel > kMaxIndex) throw Error("buffer '" + b.name + "' is beyond the sizes this backend plans for: not supported");
+    }
+  }
+  std::vector<Loop> loops;
+  validate_node(n, loops, 1);
 }
 
 }  // namespace eh

@@ -12,6 +12,18 @@
 
 namespace eh {
 
+// Index arithmetic on caller-supplied constants: an overflow is an error, never wrapped.
+inline int64_t mul_ck(int64_t a, int64_t b) {
+  int64_t r;
+  if (__builtin_mul_overflow(a, b, &r)) throw Error("integer overflow in index arithmetic: sizes of this magnitude are not supported");
+  return r;
+}
+inline int64_t add_ck(int64_t a, int64_t b) {
+  int64_t r;
+  if (__builtin_add_overflow(a, b, &r)) throw Error("integer overflow in index arithmetic: sizes of this magnitude are not supported");
+  return r;
+}
+
 // value = c + sum(coef[var] * var)
 struct Affine {
   int64_t c = 0;
@@ -67,6 +79,11 @@ struct LoadRef {
   bool guarded;
 };
 void collect_loads(const Node& expr, std::vector<LoadRef>& out, bool guarded = false);
+
+// Refuses (eh::Error) a program, kernel or statement whose sizes are beyond what the planner's
+// integer arithmetic is laid out for; see the bounds in analysis.cpp.  Everything that takes
+// caller-supplied ASTs calls this first.
+void validate_sizes(const Node& n);
 
 // Largest absolute element index an affine form can reach over the given loops.
 int64_t max_abs_index(const Affine& a, const std::vector<Loop>& loops, const Loop* rloop);

@@ -172,7 +172,14 @@ double to_float(const SX& s, bool bits32) {
   if (a == "inf") return INFINITY;
   if (a == "-inf") return -INFINITY;
   if (!a.empty() && a[0] == '#') {
-    uint64_t bits = std::stoull(a.substr(1), nullptr, 16);
+    uint64_t bits = 0;
+    try {
+      size_t used = 0;
+      bits = std::stoull(a.substr(1), &used, 16);
+      if (used + 1 != a.size()) fail(s, "bad float bit pattern '" + a + "'");
+    } catch (const std::logic_error&) {
+      fail(s, "bad float bit pattern '" + a + "'");
+    }
     if (bits32) {
       uint32_t b = static_cast<uint32_t>(bits);
       float f;

@@ -434,12 +434,31 @@ GenOptions parse_options(const char* text) {
   return o;
 }
 
+void dump_plan(const ProgramPlan& plan) {
+  const char* dir = std::getenv("ECLAT_HIP_DUMP");
+  if (!dir || !*dir) return;
+  mkdirs(dir);
+  for (const auto& ls : plan.launches) {
+    const std::string base = std::string(dir) + "/" + ls.entry;
+    std::ofstream(base + ".hip") << ls.source;
+    std::ofstream t(base + ".txt");
+    t << "entry: " << ls.entry << "\nschedule: " << ls.schedule << "\ngrid: " << ls.grid[0] << " " << ls.grid[1] << " "
+      << ls.grid[2] << "\nblock: " << ls.block[0] << " " << ls.block[1] << " " << ls.block[2]
+      << "\nlds_bytes: " << ls.lds_bytes << "\nalgorithmic_bytes: " << ls.algo_bytes << "\nflops: " << ls.flops << "\nbuffers:";
+    for (const auto& b : ls.arg_bufs) t << " " << b;
+    t << "\nkernels:";
+    for (const auto& k : ls.kernels) t << " " << k;
+    t << "\n";
+  }
+}
+
 HipProgram::HipProgram(HipDevice* dev, const std::string& ast_text, const GenOptions& opt) : dev_(dev) {
   NodePtr ast = parse_ast(ast_text);
   if (ast->op == Op::Kernel) ast = make(Op::Program, {ast});
   GenOptions o = opt;
   if (dev_->profile().arch.rfind("gfx", 0) == 0) o.arch = dev_->profile().arch;
   plan_ = plan_program(*ast, o);
+  dump_plan(plan_);
   for (size_t i = 0; i < plan_.buffers.size(); ++i) index_[plan_.buffers[i].name] = i;
   temps_.assign(plan_.buffers.size(), nullptr);
   for (const auto& ls : plan_.launches) {

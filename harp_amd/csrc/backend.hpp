@@ -198,6 +198,12 @@ class HipGraph {
 
 GenOptions parse_options(const char* text);       // "key=value,key=value" -> GenOptions
 
+// With ECLAT_HIP_DUMP=<dir> in the environment, writes every launch of a plan there:
+// <entry>.hip (the translation unit handed to hiprtc) and <entry>.txt (schedule, grid, block,
+// LDS bytes, bound buffers, the lowered kernels the launch covers).  The counterpart of the
+// reference's debug dumps of generated kernels (src/backend/pipeline.rs:150-153).
+void dump_plan(const ProgramPlan& plan);
+
 class HipBackendRegistry {
  public:
   static const char* kind() { return "hip"; }

@@ -218,6 +218,7 @@ int eh_render_program(const char* ast_text, const char* options, eh_plan** out) 
     auto* p = new eh_plan;
     try {
       p->plan = plan_program(*ast, o);
+      dump_plan(p->plan);
     } catch (...) {
       delete p;
       throw;
@@ -230,6 +231,7 @@ int eh_normalize_ast(const char* ast_text, char** out_text) {
   REQUIRE(ast_text && out_text, "ast_text or out_text is NULL");
   return guard([&] {
     NodePtr ast = parse_ast(ast_text);
+    validate_sizes(*ast);
     std::string text;
     if (ast->op == Op::Kernel) {
       text = to_text(*normalize_kernel(ast));

@@ -1382,6 +1382,7 @@ std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
 
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
+  validate_sizes(program);
   ProgramPlan plan;
   std::vector<const Node*> kernels;
   for (const auto& f : program.args) {
@@ -1389,7 +1390,6 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     else if (f->op == Op::Function) throw Error("helper functions in a program are not supported by this backend");
   }
   if (kernels.empty()) throw Error("program holds no kernel");
-
   std::vector<NodePtr> rewritten;          // owns the kernels that replace given ones
   // what the reference's AST optimiser did to the lowered loop nests is undone first
   if (opt.normalize)

@@ -1,6 +1,7 @@
 #include "normalize.hpp"
 
 #include <algorithm>
+#include <cstring>
 #include <set>
 
 #include "analysis.hpp"
@@ -98,16 +99,16 @@ NodePtr fold_expr(const NodePtr& n) {
   NodePtr cur = changed ? with_args(*n, args) : n;
   int64_t a = 0, b = 0;
   if (cur->op == Op::Shl && cur->args.size() == 2 && int_const(*cur->args[1], &b) && b >= 0 && b < 62) {
-    if (int_const(*cur->args[0], &a)) return int_like(*cur->args[0], a * (int64_t{1} << b));
+    if (int_const(*cur->args[0], &a)) return int_like(*cur->args[0], mul_ck(a, int64_t{1} << b));
     return make(Op::Mul, {cur->args[0], int_like(*cur->args[1], int64_t{1} << b)});
   }
   if (cur->args.size() == 2 && int_const(*cur->args[0], &a) && int_const(*cur->args[1], &b)) {
     switch (cur->op) {
-      case Op::Add: return int_like(*cur->args[0], a + b);
-      case Op::Mul: return int_like(*cur->args[0], a * b);
+      case Op::Add: return int_like(*cur->args[0], add_ck(a, b));
+      case Op::Mul: return int_like(*cur->args[0], mul_ck(a, b));
       case Op::Max: return int_like(*cur->args[0], std::max(a, b));
-      case Op::Idiv: if (b != 0) return int_like(*cur->args[0], a / b); break;
-      case Op::Rem: if (b != 0) return int_like(*cur->args[0], a % b); break;
+      case Op::Idiv: if (b != 0 && b != -1) return int_like(*cur->args[0], a / b); break;
+      case Op::Rem: if (b != 0 && b != -1) return int_like(*cur->args[0], a % b); break;
       default: break;
     }
   }
@@ -169,8 +170,7 @@ struct Normalizer {
   NodePtr unify(const std::vector<NodePtr>& copies, const std::string& u, bool int_pos) const {
     const Node& f = *copies[0];
     bool same = true;
-    const std::string text0 = to_text(f);
-    for (size_t t = 1; t < copies.size() && same; ++t) same = copies[t] == copies[0] || to_text(*copies[t]) == text0;
+    for (size_t t = 1; t < copies.size() && same; ++t) same = copies[t] == copies[0];
     if (same) return copies[0];
     if (int_pos) {
       std::vector<Affine> affs;
@@ -183,6 +183,9 @@ struct Normalizer {
         const int64_t d = affs[1].c - affs[0].c;
         for (size_t t = 0; t < affs.size(); ++t)
           if (affs[t].coef != affs[0].coef || affs[t].c != affs[0].c + d * static_cast<int64_t>(t)) return nullptr;
+        bool identical = d == 0;
+        for (size_t t = 1; t < copies.size() && identical; ++t) identical = shape_of(*copies[t]) == shape_of(f);
+        if (identical) return copies[0];               // same form as well as same value: keep the text
         Affine r = affs[0];
         if (d != 0) r.coef[u] += d;
         return affine_to_node(r);
@@ -196,14 +199,20 @@ struct Normalizer {
         if (c->decls[i].first != f.decls[i].first || !(c->decls[i].second == f.decls[i].second)) return nullptr;
     }
     if (f.op == Op::Const) {
-      if (f.dtype.is_float()) return nullptr;            // equal floats were caught by the text comparison
+      if (f.dtype.is_float()) {
+        for (const auto& c : copies)
+          if (std::memcmp(&c->fval, &f.fval, sizeof f.fval) != 0) return nullptr;
+        return copies[0];
+      }
       const int64_t d = copies[1]->ival - f.ival;
       for (size_t t = 0; t < copies.size(); ++t)
         if (copies[t]->ival != f.ival + d * static_cast<int64_t>(t)) return nullptr;
+      if (d == 0) return copies[0];
       return make(Op::Add, {copies[0], make(Op::Mul, {make_var(u), int_like(f, d)})});
     }
-    if (f.args.empty()) return nullptr;
+    if (f.args.empty()) return copies[0];                 // a variable (names compared above), a barrier
     std::vector<NodePtr> args;
+    bool changed = false;
     for (size_t i = 0; i < f.args.size(); ++i) {
       std::vector<NodePtr> sub;
       for (const auto& c : copies) sub.push_back(c->args[i]);
@@ -220,9 +229,36 @@ struct Normalizer {
       }
       NodePtr r = unify(sub, u, pos);
       if (!r) return nullptr;
+      changed = changed || r != f.args[i];
       args.push_back(std::move(r));
     }
-    return with_args(f, std::move(args));
+    return changed ? with_args(f, std::move(args)) : copies[0];
+  }
+
+  // The form of a statement with its integer literals blanked: repetitions of an unrolled loop
+  // share it.  Memoised per node (the nodes of a kernel outlive the pass).
+  mutable std::map<const Node*, uint64_t> shape_memo;
+  uint64_t shape_of(const Node& n) const {
+    auto it = shape_memo.find(&n);
+    if (it != shape_memo.end()) return it->second;
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&](uint64_t v) {
+      h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+    };
+    mix(static_cast<uint64_t>(n.op));
+    for (unsigned char c : n.name) mix(c);
+    mix(static_cast<uint64_t>(n.dtype.ty));
+    mix(static_cast<uint64_t>(n.count));
+    mix(n.args.size());
+    mix(n.decls.size());
+    if (n.op == Op::Const && n.dtype.is_float()) {
+      uint64_t bits;
+      std::memcpy(&bits, &n.fval, sizeof bits);
+      mix(bits);
+    }
+    for (const auto& a : n.args) mix(shape_of(*a));
+    shape_memo[&n] = h;
+    return h;
   }
 
   // A block whose statements are k >= 2 repetitions of p statements that differ only by integers
@@ -231,12 +267,21 @@ struct Normalizer {
   // the loop body, which is sound when every repetition assigns them before it reads them.
   NodePtr reroll(const std::vector<NodePtr>& stmts, const std::vector<std::pair<std::string, DType>>& decls) {
     const size_t n = stmts.size();
-    for (size_t p = 1; p * 2 <= n; ++p) {
+    // the smallest period of the statements' forms (failure function over their hashes); a
+    // nest of unrolled loops repeats at multiples of it
+    std::vector<uint64_t> sig(n);
+    for (size_t j = 0; j < n; ++j) sig[j] = shape_of(*stmts[j]);
+    std::vector<size_t> fail(n, 0);
+    for (size_t j = 1, k = 0; j < n; ++j) {
+      while (k > 0 && sig[j] != sig[k]) k = fail[k - 1];
+      if (sig[j] == sig[k]) ++k;
+      fail[j] = k;
+    }
+    const size_t p0 = n - fail[n - 1];
+    if (n % p0 != 0 || p0 == n) return nullptr;
+    for (size_t p = p0; p * 2 <= n; p += p0) {
       if (n % p) continue;
       const size_t k = n / p;
-      bool shape = true;
-      for (size_t j = 0; j < n && shape; ++j) shape = stmts[j]->op == stmts[j % p]->op;
-      if (!shape) continue;
       bool decls_ok = true;
       for (const auto& d : decls) {
         for (size_t j = 0; j < p; ++j) {
@@ -294,7 +339,7 @@ struct Normalizer {
         const Node& ib = *in.args[3];
         if (int_const(*in.args[0], &is) && int_const(*in.args[1], &istep) && int_const(*in.args[2], &T) && is == 0 &&
             istep == 1 && T >= 1 && ib.op == Op::Block && ib.args.size() >= 2 && ib.args[0]->op == Op::Assign) {
-          const std::string& v = ib.args[0]->name;
+          const std::string v = ib.args[0]->name;         // a copy: `r` is replaced below, and its body with it
           auto a = int_affine(*ib.args[0]->args[0]);
           auto decls = ib.decls;
           bool clean = a && a->c == 0 && a->coef.size() == 2 && a->of(in.name) == 1 && drop_decl(&decls, v);
@@ -331,7 +376,7 @@ struct Normalizer {
       // (the remainder loop of tile_loop; a rolled-back unrolled loop)
       if (body->op == Op::Block && body->args.size() >= 2 && body->args[0]->op == Op::Assign && step == 1) {
         const Node& b = *body;
-        const std::string& v = b.args[0]->name;
+        const std::string v = b.args[0]->name;
         auto a = int_affine(*b.args[0]->args[0]);
         auto decls = b.decls;
         bool clean = a && a->coef.size() == 1 && a->of(r->name) == 1 && drop_decl(&decls, v);

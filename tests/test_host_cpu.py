@@ -509,3 +509,16 @@ def test_option_beam_search_on_a_synthetic_cost():
     assert all("flat_" in k or k == "nontemporal" for sg in (tune.suggest_flat, tune.suggest_streaming)
                for st in sg({}, ["flat(V=4,block=256)"]) for k in st)
     assert tune.options_string(tune._freeze({"b": 2, "a": 1})) == "a=1,b=2"
+
+
+def test_dump_directory_receives_every_launch(frontend, tmp_path, monkeypatch):
+    """ECLAT_HIP_DUMP=<dir>: the generated HIP source and the dispatch of every launch."""
+    from harp_amd import backend as hb
+    from harp_amd import workloads as wl
+    monkeypatch.setenv("ECLAT_HIP_DUMP", str(tmp_path / "dump"))
+    plan = hb.render_program(wl.lower_with_table([(64, 256)], wl.config2_graph)[0])
+    for l in plan.launches:
+        src = (tmp_path / "dump" / (l["entry"] + ".hip")).read_text()
+        assert src == l["source"] and "__global__" in src
+        info = (tmp_path / "dump" / (l["entry"] + ".txt")).read_text()
+        assert "schedule: " + l["schedule"] in info and "grid: %d %d %d" % tuple(l["grid"]) in info
