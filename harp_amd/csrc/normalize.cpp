@@ -236,11 +236,8 @@ struct Normalizer {
   }
 
   // The form of a statement with its integer literals blanked: repetitions of an unrolled loop
-  // share it.  Memoised per node (the nodes of a kernel outlive the pass).
-  mutable std::map<const Node*, uint64_t> shape_memo;
+  // share it.
   uint64_t shape_of(const Node& n) const {
-    auto it = shape_memo.find(&n);
-    if (it != shape_memo.end()) return it->second;
     uint64_t h = 1469598103934665603ull;
     auto mix = [&](uint64_t v) {
       h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
@@ -256,8 +253,31 @@ struct Normalizer {
       std::memcpy(&bits, &n.fval, sizeof bits);
       mix(bits);
     }
-    for (const auto& a : n.args) mix(shape_of(*a));
-    shape_memo[&n] = h;
+    for (size_t i = 0; i < n.args.size(); ++i) {
+      // an integer position counts by its affine coefficients, not by its spelling: the
+      // reference's simplifier rewrites one repetition (`o + 0` to `o`) and not its siblings
+      bool pos = false;
+      switch (n.op) {
+        case Op::Load: case Op::Store: case Op::AtomicAdd: case Op::AtomicMax: case Op::SharedLoad: case Op::SharedStore:
+          pos = i == 1;
+          break;
+        case Op::Assign: pos = int_vars.count(n.name) > 0; break;
+        case Op::Range: pos = i < 3; break;
+        default: break;
+      }
+      std::optional<Affine> a;
+      if (pos) a = int_affine(*n.args[i]);
+      if (a) {
+        mix(0xaff1e);
+        for (const auto& kv : a->coef) {
+          if (kv.second == 0) continue;
+          for (unsigned char c : kv.first) mix(c);
+          mix(static_cast<uint64_t>(kv.second));
+        }
+      } else {
+        mix(shape_of(*n.args[i]));
+      }
+    }
     return h;
   }
 
