@@ -2699,10 +2699,10 @@ struct SerialReduce {
     std::map<std::string, int64_t> need;
     std::vector<LoadRef> loads;
     collect_loads(*k.value, loads);
-    bool opaque = false;
+    std::set<std::string> opaque;          // buffers some load reaches through a non-affine index
     for (const auto& lr : loads) {
       auto a = affine_of(*lr.load->args[1]);
-      if (!a) { opaque = true; continue; }
+      if (!a) { opaque.insert(lr.load->args[0]->name); continue; }
       if (lr.guarded) continue;
       auto& n = need[lr.load->args[0]->name];
       n = std::max(n, max_abs_index(*a, k.loops, &k.rloop) + 1);
@@ -2714,7 +2714,7 @@ struct SerialReduce {
       for (const auto& p : k.params)
         if (p.name == b) { item = p.dtype.elem().itemsize(); is_out = p.mut_; }
       auto it = need.find(b);
-      ls->arg_min_bytes.push_back(it == need.end() || (opaque && !is_out) ? 0 : static_cast<size_t>(it->second) * item);
+      ls->arg_min_bytes.push_back(it == need.end() || (opaque.count(b) && !is_out) ? 0 : static_cast<size_t>(it->second) * item);
     }
   }
 

@@ -79,6 +79,9 @@ double estimate_us(const GemmShape& s, const Candidate& c, int split) {
 // Tile and K split for a contraction.
 bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool computed_operand = false) {
   if (s.K < 8 || s.M < 2 || s.N < 2) return false;
+  // the batch rides on blockIdx.z (at most 65535 workgroups); the tiles of one batch on blockIdx.x.
+  // Beyond either the contraction is left to the other reduce schedules.
+  if (s.batch > 65535 || ceil_div(s.M, 64) * ceil_div(s.N, 64) >= (int64_t{1} << 31)) return false;
   Choice best;
   if (opt.gemm_bm > 0) {
     best.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};

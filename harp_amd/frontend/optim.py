@@ -7,12 +7,18 @@ builds the update as tensor graphs over the (lazy) gradients and realizes the ne
 parameters and optimizer states as the roots of one Program: forward, backward and update run
 once, on the device, and the results become the parameters' new buffers without a host copy.
 The arithmetic is the reference's, in its order: `p - lr*g`; `v = mu*v - lr*g, p + v`;
-Adam's `m, v, m/(1-b1^t), v/(1-b2^t), p - lr*m_hat/(sqrt(v_hat)+eps)`.
+Adam's `m, v, m/(1-b1^t), v/(1-b2^t), p - (lr*m_hat)/(sqrt(v_hat)+eps)` with the bias corrections
+computed in float32 by the square-and-multiply `powi` (`adam.rs:108-110`).  One difference is left:
+the AST has no division node, a quotient in a graph is `x * recip(y)` (as the reference's own
+tensor division is), so each of the three quotients of an Adam update may differ from the host
+loop's IEEE division by one unit in the last place.
 """
 
 from __future__ import annotations
 
 from typing import List, Optional, Sequence
+
+import numpy as np
 
 from .layers import Parameter
 from .tensor import Tensor, realize_many
@@ -24,7 +30,6 @@ class OptimError(Exception):
 
 def _state(shape) -> Tensor:
     t = Tensor.input(shape)
-    import numpy as np
     t.set_data(np.zeros(int(np.prod(shape)) if shape else 1, np.float32))
     return t
 
@@ -95,6 +100,19 @@ class SGD(_Optimizer):
             self.velocity[i] = _as_input(t)
 
 
+def powi_f32(base: float, exp: int) -> np.float32:
+    """`f32::powi`: square-and-multiply in float32, the exponent's bits from the lowest up."""
+    a, r, b = np.float32(base), np.float32(1.0), abs(int(exp))
+    while True:
+        if b & 1:
+            r = np.float32(r * a)
+        b >>= 1
+        if b == 0:
+            break
+        a = np.float32(a * a)
+    return np.float32(1.0) / r if exp < 0 else r
+
+
 class Adam(_Optimizer):
     def __init__(self, params: Sequence[Parameter], lr: float, betas=(0.9, 0.999), eps: float = 1e-8):
         super().__init__(params, lr)
@@ -118,17 +136,23 @@ class Adam(_Optimizer):
     def step(self, also: Sequence[Tensor] = ()) -> None:
         grads = self._grads()
         self.t += 1
-        b1, b2 = self._betas
-        c1, c2 = 1.0 - b1 ** self.t, 1.0 - b2 ** self.t
+        b1, b2 = np.float32(self._betas[0]), np.float32(self._betas[1])
+        one = np.float32(1.0)
+        c1, c2 = one - powi_f32(b1, self.t), one - powi_f32(b2, self.t)
+        lr, eps = np.float32(self.lr), np.float32(self._eps)
+
+        def over(x: Tensor, c) -> Tensor:                      # x / c, the way a graph divides
+            return x * Tensor.ones_like(x).scale_exact(float(c)).recip()
         new_p, new_m, new_v = [], [], []
         for i, (p, g) in enumerate(zip(self.params, grads)):
             if self.m[i] is None:
                 self.m[i], self.v[i] = _state(p.shape()), _state(p.shape())
-            m = self.m[i].scale_exact(b1) + g.scale_exact(1.0 - b1)
-            v = self.v[i].scale_exact(b2) + (g * g).scale_exact(1.0 - b2)
-            m_hat, v_hat = m.scale_exact(1.0 / c1), v.scale_exact(1.0 / c2)
-            denom = v_hat.sqrt() + Tensor.ones_like(v_hat).scale_exact(self._eps)
-            new_p.append(p.tensor() - (m_hat / denom).scale_exact(self.lr))
+            m = self.m[i].scale_exact(float(b1)) + g.scale_exact(float(one - b1))
+            # (1 - b2) * g * g associates to the left
+            v = self.v[i].scale_exact(float(b2)) + g.scale_exact(float(one - b2)) * g
+            m_hat, v_hat = over(m, c1), over(v, c2)
+            denom = v_hat.sqrt() + Tensor.ones_like(v_hat).scale_exact(float(eps))
+            new_p.append(p.tensor() - m_hat.scale_exact(float(lr)) * denom.recip())
             new_m.append(m)
             new_v.append(v)
         realize_many(new_p + new_m + new_v + list(also))

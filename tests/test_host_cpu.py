@@ -522,3 +522,18 @@ def test_dump_directory_receives_every_launch(frontend, tmp_path, monkeypatch):
         assert src == l["source"] and "__global__" in src
         info = (tmp_path / "dump" / (l["entry"] + ".txt")).read_text()
         assert "schedule: " + l["schedule"] in info and "grid: %d %d %d" % tuple(l["grid"]) in info
+
+
+def test_contraction_with_more_batches_than_grid_z_allows_is_not_put_on_mfma(frontend):
+    """The batch axis of a contraction rides on blockIdx.z, which holds at most 65535 workgroups: a
+    per-group contraction over 70000 groups is planned with another reduce schedule instead of a
+    launch the runtime would refuse."""
+    from harp_amd import backend as hb
+    from harp_amd import workloads as wl
+    fn = lambda g, c: (g.unsqueeze(3) * c.unsqueeze(2)).sum(1)          # [G,R,O],[G,R,K] -> [G,O,K]
+    small = hb.render_program(wl.lower_with_table([(6, 16, 8), (6, 16, 8)], fn)[0]).launches
+    assert any(l["schedule"].startswith("mfma32x32x2(") for l in small)
+    big = hb.render_program(wl.lower_with_table([(70000, 16, 8), (70000, 16, 8)], fn)[0]).launches
+    assert not any(l["schedule"].startswith("mfma") for l in big), [l["schedule"] for l in big]
+    for l in big:
+        assert l["grid"][2] <= 65535 and l["grid"][1] <= 65535 and l["grid"][0] < 2 ** 31, l["grid"]

@@ -392,6 +392,54 @@ def test_training_loop_matches_numpy(frontend, optimizer):
     assert losses[-1] < losses[0]
 
 
+def test_adam_trajectory_follows_the_reference_loop_in_float32(frontend):
+    """Three Adam steps on a parameter whose gradient is `w * p` against the reference's host loop
+    (`crates/nn/src/optim/adam.rs:104-137`) restated in float32 in its order of operations: bias
+    corrections by float32 square-and-multiply, `m / bc1`, `v / bc2`, `(lr * m_hat) / (sqrt + eps)`.
+    The graph divides by multiplying with a reciprocal (the AST has no division), so each of the
+    three quotients may be one unit in the last place off; the update is lr * O(1), so three steps
+    stay within a few ulp of the parameter."""
+    from harp_amd.frontend.layers import Parameter
+    from harp_amd.frontend.optim import Adam, powi_f32
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    f = np.float32
+    b = f(0.999)
+    assert powi_f32(b, 1) == b and powi_f32(b, 2) == f(b * b)
+    assert powi_f32(b, 3) == f(b * f(b * b))
+    assert powi_f32(b, 5) == f(b * f(f(b * b) * f(b * b)))
+    assert powi_f32(f(2.0), -2) == f(0.25) and powi_f32(b, 0) == f(1.0)
+    frontend.set_device_str("c")
+    rng = np.random.default_rng(11)
+    p0 = rng.uniform(-1, 1, 37).astype(f)
+    w = rng.uniform(0.5, 2, 37).astype(f)
+    lr, b1, b2, eps = f(0.01), f(0.9), f(0.999), f(1e-8)
+    try:
+        with frontend.exact_mode():
+            param = Parameter.from_data("p", p0, [37])
+            wt = frontend.Tensor.input([37])
+            wt.set_data(w)
+            opt = Adam([param], float(lr))
+            for _ in range(3):
+                opt.zero_grad()
+                pt = param.tensor()
+                loss = (pt * pt * wt).sum(0).scale_exact(0.5)
+                loss.backward_with_params([pt])
+                opt.step()
+            got = param.to_numpy()
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+    p, m, v = p0.copy(), np.zeros(37, f), np.zeros(37, f)
+    for t in range(1, 4):
+        g = f(w * p)
+        bc1, bc2 = f(1) - powi_f32(b1, t), f(1) - powi_f32(b2, t)
+        m = b1 * m + (f(1) - b1) * g
+        v = b2 * v + (f(1) - b2) * g * g
+        p = p - lr * (m / bc1) / (np.sqrt(v / bc2) + eps)
+    assert p.dtype == f and m.dtype == f
+    assert np.abs(got - p).max() <= 4 * np.spacing(f(1.0)), np.abs(got - p).max()
+    assert np.median(np.abs(got - p0)) > 0.029                 # three steps of about lr each were taken
+
+
 def test_parameter_and_layer_api(frontend):
     """`Parameter` (parameter.rs:31-214) and the deterministic layer initialisation
     (`linear.rs:57-68`: sin(0.1 i) * sqrt(1/in), zero bias)."""
