@@ -21,6 +21,8 @@ pub struct eh_launch_info {
     pub n_kernels: c_int,
     pub algo_bytes: f64,
     pub flops: f64,
+    pub lane: c_int,
+    pub n_waits: c_int,
 }
 
 #[repr(C)]

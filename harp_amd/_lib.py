@@ -45,7 +45,7 @@ class LaunchInfo(Structure):
     _fields_ = [("entry", c_char_p), ("source", c_char_p), ("schedule", c_char_p),
                 ("grid", c_uint * 3), ("block", c_uint * 3), ("lds_bytes", c_uint),
                 ("n_args", c_int), ("n_kernels", c_int), ("algo_bytes", c_double),
-                ("flops", c_double)]
+                ("flops", c_double), ("lane", c_int), ("n_waits", c_int)]
 
 
 _P = c_void_p
@@ -73,6 +73,8 @@ _SIGS = {
     "eh_plan_launch": ([_P, c_int, POINTER(LaunchInfo)], c_int),
     "eh_plan_launch_arg": ([_P, c_int, c_int, POINTER(c_char_p)], c_int),
     "eh_plan_launch_kernel": ([_P, c_int, c_int, POINTER(c_char_p)], c_int),
+    "eh_plan_launch_arg_written": ([_P, c_int, c_int, POINTER(c_int)], c_int),
+    "eh_plan_launch_wait": ([_P, c_int, c_int, POINTER(c_int)], c_int),
     "eh_plan_num_buffers": ([_P, POINTER(c_int)], c_int),
     "eh_plan_buffer": ([_P, c_int, POINTER(c_char_p), POINTER(c_char_p), POINTER(c_size_t),
                         POINTER(c_int)], c_int),

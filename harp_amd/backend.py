@@ -34,7 +34,8 @@ def _launch_dict(info: LaunchInfo) -> dict:
     return {"entry": info.entry.decode(), "source": info.source.decode(),
             "schedule": info.schedule.decode(), "grid": list(info.grid),
             "block": list(info.block), "lds_bytes": info.lds_bytes, "n_args": info.n_args,
-            "n_kernels": info.n_kernels, "algo_bytes": info.algo_bytes, "flops": info.flops}
+            "n_kernels": info.n_kernels, "algo_bytes": info.algo_bytes, "flops": info.flops,
+            "lane": info.lane, "n_waits": info.n_waits}
 
 
 # ---------------------------------------------------------------------------
@@ -54,11 +55,16 @@ class Plan:
             info = LaunchInfo()
             check(lib.eh_plan_launch(self._h, i, byref(info)))
             d = _launch_dict(info)
-            d["args"], d["kernels"] = [], []
-            s = c_char_p()
+            d["args"], d["kernels"], d["written"], d["waits"] = [], [], [], []
+            s, v = c_char_p(), c_int()
             for a in range(info.n_args):
                 check(lib.eh_plan_launch_arg(self._h, i, a, byref(s)))
                 d["args"].append(s.value.decode())
+                check(lib.eh_plan_launch_arg_written(self._h, i, a, byref(v)))
+                d["written"].append(bool(v.value))
+            for w in range(info.n_waits):
+                check(lib.eh_plan_launch_wait(self._h, i, w, byref(v)))
+                d["waits"].append(v.value)
             for k in range(info.n_kernels):
                 check(lib.eh_plan_launch_kernel(self._h, i, k, byref(s)))
                 d["kernels"].append(s.value.decode())

@@ -231,9 +231,25 @@ HipDevice::~HipDevice() {
   if (stream_) {
     (void)hipSetDevice(index_);
     (void)hipStreamSynchronize(stream_);
+    for (hipStream_t st : side_streams_) {
+      (void)hipStreamSynchronize(st);
+      (void)hipStreamDestroy(st);
+    }
     for (auto& kv : pool_) (void)hipFree(kv.second);
     (void)hipStreamDestroy(stream_);
   }
+}
+
+hipStream_t HipDevice::lane_stream(int lane) {
+  if (lane <= 0) return stream_;
+  auto lk = stream_lock();
+  make_current();
+  while (side_streams_.size() < static_cast<size_t>(lane)) {
+    hipStream_t st = nullptr;
+    check(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    side_streams_.push_back(st);
+  }
+  return side_streams_[static_cast<size_t>(lane) - 1];
 }
 
 void* HipDevice::allocate(size_t bytes) {
@@ -367,13 +383,13 @@ HipKernel::~HipKernel() {
 }
 
 void HipKernel::launch(const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
-                       const std::vector<void*>& device_ptrs) const {
+                       const std::vector<void*>& device_ptrs, hipStream_t stream) const {
   auto lk = dev_->stream_lock();
   std::vector<void*> vals = device_ptrs;
   std::vector<void*> params(vals.size());
   for (size_t i = 0; i < vals.size(); ++i) params[i] = &vals[i];
-  check(hipModuleLaunchKernel(fn_, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, dev_->stream(),
-                              params.data(), nullptr),
+  check(hipModuleLaunchKernel(fn_, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes,
+                              stream ? stream : dev_->stream(), params.data(), nullptr),
         ("launch of " + entry_).c_str());
 }
 
@@ -421,6 +437,8 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
     else if (k == "gemm_dma") o.gemm_dma = as_int() != 0;
     else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
+    else if (k == "lanes") o.lanes = std::max(1, as_int());
+    else if (k == "lane_us") o.lane_us = std::max(0, as_int());
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;
     else if (k == "nontemporal") o.nontemporal = as_int();
     else if (k == "normalize") o.normalize = as_int() != 0;
@@ -477,6 +495,13 @@ HipProgram::HipProgram(HipDevice* dev, const std::string& ast_text, const GenOpt
 }
 
 HipProgram::~HipProgram() {
+  // every execute joined its lanes back into the device's stream, which the temps' release waits
+  // for; an event may be destroyed while work queued behind it is still pending
+  for (hipEvent_t e : events_)
+    if (e) (void)hipEventDestroy(e);
+  for (hipEvent_t e : join_)
+    if (e) (void)hipEventDestroy(e);
+  if (fork_) (void)hipEventDestroy(fork_);
   for (HipBuffer* b : temps_)
     if (b && b->release()) delete b;
 }
@@ -520,8 +545,48 @@ void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
 
 void HipProgram::launch_spans(const std::vector<Span>& bound) {
   auto lk = dev_->stream_lock();               // the program's launches go out as one run
+  const int lanes = plan_.lanes;
+  std::vector<hipStream_t> streams(static_cast<size_t>(std::max(lanes, 1)), dev_->stream());
+  if (lanes > 1) {
+    dev_->make_current();
+    if (events_.empty()) {
+      // an event behind every launch somebody on another lane waits for
+      events_.assign(plan_.launches.size(), nullptr);
+      for (const LaunchSpec& ls : plan_.launches)
+        for (int w : ls.waits)
+          if (!events_[static_cast<size_t>(w)])
+            check(hipEventCreateWithFlags(&events_[static_cast<size_t>(w)], hipEventDisableTiming), "hipEventCreateWithFlags");
+      join_.assign(static_cast<size_t>(lanes - 1), nullptr);
+      for (auto& e : join_) check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreateWithFlags");
+      check(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "hipEventCreateWithFlags");
+    }
+    // fork: the side lanes start behind everything queued on the device's stream so far
+    check(hipEventRecord(fork_, dev_->stream()), "hipEventRecord");
+    for (int s = 1; s < lanes; ++s) {
+      streams[static_cast<size_t>(s)] = dev_->lane_stream(s);
+      check(hipStreamWaitEvent(streams[static_cast<size_t>(s)], fork_, 0), "hipStreamWaitEvent");
+    }
+  }
+  // Whatever happens, the side lanes are joined back: a launch that fails half-way must not
+  // leave work on a side stream that later work on the device's stream does not wait for.
+  struct Join {
+    HipProgram* p;
+    const std::vector<hipStream_t>& st;
+    int lanes;
+    ~Join() {
+      for (int s = 1; s < lanes; ++s) {
+        hipEvent_t e = p->join_.size() >= static_cast<size_t>(s) ? p->join_[static_cast<size_t>(s) - 1] : nullptr;
+        if (!e || st[static_cast<size_t>(s)] == p->dev_->stream()) continue;
+        (void)hipEventRecord(e, st[static_cast<size_t>(s)]);
+        (void)hipStreamWaitEvent(p->dev_->stream(), e, 0);
+      }
+    }
+  } join{this, streams, lanes};
   for (size_t l = 0; l < plan_.launches.size(); ++l) {
     const LaunchSpec& ls = plan_.launches[l];
+    hipStream_t stream = streams[static_cast<size_t>(lanes > 1 ? ls.lane : 0)];
+    if (lanes > 1)
+      for (int w : ls.waits) check(hipStreamWaitEvent(stream, events_[static_cast<size_t>(w)], 0), "hipStreamWaitEvent");
     std::vector<void*> ptrs;
     for (size_t a = 0; a < ls.arg_bufs.size(); ++a) {
       const Span& b = bound[index_.at(ls.arg_bufs[a])];
@@ -532,7 +597,8 @@ void HipProgram::launch_spans(const std::vector<Span>& bound) {
                     std::to_string(b.bytes));
       ptrs.push_back(b.ptr);
     }
-    kernels_[l]->launch(ls.grid, ls.block, ls.lds_bytes, ptrs);
+    kernels_[l]->launch(ls.grid, ls.block, ls.lds_bytes, ptrs, stream);
+    if (lanes > 1 && events_[l]) check(hipEventRecord(events_[l], stream), "hipEventRecord");
   }
 }
 

@@ -57,6 +57,10 @@ class HipDevice {
 
   int index() const { return index_; }
   hipStream_t stream() const { return stream_; }
+  // Side stream `lane` (1, 2, ...; default priority, created on first use): a program whose plan
+  // spreads independent launches over lanes forks them off the device's stream and joins them
+  // back before its execute returns, so to everybody else the device still has one stream.
+  hipStream_t lane_stream(int lane);
   // Everything that enqueues on (or waits for) the device's one stream holds this lock while it
   // does: buffer fills and copies, launches of a program, graph replays, synchronisation -- and
   // a graph capture holds it from begin to end, so that no other thread's work is recorded into
@@ -86,6 +90,7 @@ class HipDevice {
  private:
   int index_;
   hipStream_t stream_ = nullptr;
+  std::vector<hipStream_t> side_streams_;
   DeviceProfile profile_;
   mutable std::recursive_mutex stream_mu_;
   std::mutex pool_mu_;
@@ -123,8 +128,9 @@ class HipKernel {
  public:
   HipKernel(HipDevice* dev, const Binary& bin, const std::string& entry);
   ~HipKernel();
+  // Queues the kernel on `stream` (nullptr: the device's stream).
   void launch(const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
-              const std::vector<void*>& device_ptrs) const;
+              const std::vector<void*>& device_ptrs, hipStream_t stream = nullptr) const;
   const std::vector<char>& binary() const { return binary_; }   // Kernel::get_binary
   const std::string& entry() const { return entry_; }
 
@@ -172,6 +178,11 @@ class HipProgram {
   std::vector<std::shared_ptr<HipKernel>> kernels_;
   std::map<std::string, size_t> index_;          // buffer name -> table index
   std::vector<HipBuffer*> temps_;                // owned, by table index (nullptr if unused)
+  // Lanes (plan().lanes > 1): events_[l] is recorded behind launch l when a launch on another
+  // lane waits for it; fork_ is recorded on the device's stream before the first launch and
+  // join_[s-1] on side lane s behind its last one.  Created on the first execute.
+  std::vector<hipEvent_t> events_, join_;
+  hipEvent_t fork_ = nullptr;
   std::mutex mu_;
 };
 

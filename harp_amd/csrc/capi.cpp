@@ -94,6 +94,8 @@ void fill_info(const LaunchSpec& ls, eh_launch_info* out) {
   out->n_kernels = static_cast<int>(ls.kernels.size());
   out->algo_bytes = ls.algo_bytes;
   out->flops = ls.flops;
+  out->lane = ls.lane;
+  out->n_waits = static_cast<int>(ls.waits.size());
 }
 
 int buffer_entry(const ProgramPlan& p, int i, const char** name, const char** role, size_t* bytes, int* elided) {
@@ -269,6 +271,24 @@ int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_n
   const auto& a = plan->plan.launches[static_cast<size_t>(launch)].arg_bufs;
   REQUIRE(arg >= 0 && arg < static_cast<int>(a.size()), "argument index out of range");
   *buffer_name = a[static_cast<size_t>(arg)].c_str();
+  return EH_OK;
+}
+
+int eh_plan_launch_arg_written(eh_plan* plan, int launch, int arg, int* written) {
+  REQUIRE(plan && written, "plan or written is NULL");
+  REQUIRE(launch >= 0 && launch < static_cast<int>(plan->plan.launches.size()), "launch index out of range");
+  const auto& a = plan->plan.launches[static_cast<size_t>(launch)].arg_written;
+  REQUIRE(arg >= 0 && arg < static_cast<int>(a.size()), "argument index out of range");
+  *written = a[static_cast<size_t>(arg)] ? 1 : 0;
+  return EH_OK;
+}
+
+int eh_plan_launch_wait(eh_plan* plan, int launch, int i, int* waited_launch) {
+  REQUIRE(plan && waited_launch, "plan or waited_launch is NULL");
+  REQUIRE(launch >= 0 && launch < static_cast<int>(plan->plan.launches.size()), "launch index out of range");
+  const auto& w = plan->plan.launches[static_cast<size_t>(launch)].waits;
+  REQUIRE(i >= 0 && i < static_cast<int>(w.size()), "wait index out of range");
+  *waited_launch = w[static_cast<size_t>(i)];
   return EH_OK;
 }
 

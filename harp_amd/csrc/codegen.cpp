@@ -1380,6 +1380,167 @@ std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
 
 }  // namespace
 
+
+// Which buffers each launch writes, and which launches may run beside each other.
+//
+// A program's launches are planned in an order that is valid one after the other.  Many of them
+// do not depend on each other, though: in a training step the gradient of every parameter and
+// its update hang off the chain that carries the gradient back through the layers, and most of
+// them are small launches that cost their few microseconds of launch latency whatever they
+// compute.  Launches are therefore given lanes: lane 0 (the device's stream) takes the chain of
+// dependent launches with the largest estimated duration, the others go to side lanes that run
+// concurrently; a launch waits for the launches on other lanes whose buffers it reads or
+// overwrites (`waits`), and the executor joins the lanes at the end of the program.  The results
+// do not depend on the lanes: every launch still sees exactly the inputs it would have seen.
+void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, const GenOptions& opt) {
+  auto& L = plan->launches;
+  const size_t n = L.size();
+  std::map<std::string, const Node*> by_name;
+  for (const Node* k : kernels) by_name[k->name] = k;
+  // written: outputs of the lowered kernels a launch covers; a scratch buffer the plan added is
+  // written by the first launch that binds it and read by the later ones
+  std::set<std::string> scratch_seen;
+  for (auto& ls : L) {
+    std::set<std::string> outs;
+    bool known = !ls.kernels.empty();
+    for (const auto& kn : ls.kernels) {
+      auto it = by_name.find(kn);
+      if (it == by_name.end()) { known = false; continue; }
+      for (const auto& p : it->second->params)
+        if (p.dtype.is_ptr() && p.mut_) outs.insert(p.name);
+    }
+    // a launch whose kernels cannot be looked up is taken to write everything it binds
+    ls.arg_written.assign(ls.arg_bufs.size(), known ? 0 : 1);
+    for (size_t a = 0; a < ls.arg_bufs.size() && known; ++a) {
+      const std::string& b = ls.arg_bufs[a];
+      bool declared = false;
+      for (const Node* k : kernels)
+        for (const auto& p : k->params) declared = declared || p.name == b;
+      if (outs.count(b)) ls.arg_written[a] = 1;
+      else if (!declared && scratch_seen.insert(b).second) ls.arg_written[a] = 1;
+    }
+  }
+  plan->lanes = 1;
+  for (auto& ls : L) { ls.lane = 0; ls.waits.clear(); }
+  if (opt.lanes < 2 || n < 8) return;
+  // dependences: read after write, write after write, write after read
+  std::vector<std::vector<int>> deps(n);
+  for (size_t j = 0; j < n; ++j)
+    for (size_t i = 0; i < j; ++i) {
+      bool dep = false;
+      for (size_t a = 0; a < L[i].arg_bufs.size() && !dep; ++a)
+        for (size_t b = 0; b < L[j].arg_bufs.size() && !dep; ++b)
+          dep = L[i].arg_bufs[a] == L[j].arg_bufs[b] && (L[i].arg_written[a] || L[j].arg_written[b]);
+      if (dep) deps[j].push_back(static_cast<int>(i));
+    }
+  // estimated microseconds: a launch floor plus traffic at half the memory rate or the matrix
+  // cores at a third of theirs
+  std::vector<double> est(n), path(n);
+  std::vector<int> prev(n, -1);
+  for (size_t j = 0; j < n; ++j) {
+    est[j] = 4.0 + std::max(L[j].algo_bytes / 4.0e6, L[j].flops / 5.0e7);
+    path[j] = est[j];
+    for (int i : deps[j])
+      if (path[static_cast<size_t>(i)] + est[j] > path[j]) {
+        path[j] = path[static_cast<size_t>(i)] + est[j];
+        prev[j] = i;
+      }
+  }
+  size_t end = 0;
+  for (size_t j = 0; j < n; ++j)
+    if (path[j] > path[end]) end = j;
+  std::vector<char> on_main(n, 0);
+  for (int j = static_cast<int>(end); j >= 0; j = prev[static_cast<size_t>(j)]) on_main[static_cast<size_t>(j)] = 1;
+  // a launch that fills the chip for long gains nothing from company and slows down in it
+  if (opt.lane_us > 0)
+    for (size_t j = 0; j < n; ++j)
+      if (est[j] > opt.lane_us) on_main[j] = 1;
+  double side_us = 0;
+  for (size_t j = 0; j < n; ++j)
+    if (!on_main[j]) side_us += est[j];
+  if (side_us < 24.0) return;                       // not worth a fork and a join
+  const int lanes = std::min(opt.lanes, 4);
+  // bottom level: what still has to run behind a launch, the launch included
+  std::vector<double> tail(n);
+  for (size_t j = n; j-- > 0;) {
+    tail[j] = std::max(tail[j], est[j]);
+    for (int i : deps[j]) tail[static_cast<size_t>(i)] = std::max(tail[static_cast<size_t>(i)], est[static_cast<size_t>(i)] + tail[j]);
+  }
+  // List scheduling: of the launches whose producers are placed, the one that can start first
+  // goes next (the longer tail on a tie); chain launches on lane 0, the others on the side lane
+  // that is free first.  The order of placement is the order of issue: a lane runs in order, so
+  // a side lane must be handed its launches in the order in which their inputs become ready.
+  std::vector<double> lane_free(static_cast<size_t>(lanes), 0.0), finish(n, 0.0);
+  std::vector<char> placed(n, 0);
+  std::vector<int> lane_of(n, 0);
+  std::vector<size_t> order;
+  while (order.size() < n) {
+    int best = -1, best_lane = 0;
+    double best_start = 0;
+    for (size_t j = 0; j < n; ++j) {
+      if (placed[j]) continue;
+      bool ok = true;
+      double ready = 0;
+      int dep_lane = -1;
+      for (int i : deps[j]) {
+        ok = ok && placed[static_cast<size_t>(i)];
+        if (finish[static_cast<size_t>(i)] >= ready) {
+          ready = finish[static_cast<size_t>(i)];
+          dep_lane = lane_of[static_cast<size_t>(i)];
+        }
+      }
+      if (!ok) continue;
+      int lane = 0;
+      if (!on_main[j]) {
+        lane = 1;
+        for (int t = 2; t < lanes; ++t)
+          if (lane_free[static_cast<size_t>(t)] < lane_free[static_cast<size_t>(lane)]) lane = t;
+        // behind its last producer when that costs nothing: no wait across lanes then
+        if (dep_lane > 0 && lane_free[static_cast<size_t>(dep_lane)] <= std::max(ready, lane_free[static_cast<size_t>(lane)])) lane = dep_lane;
+      }
+      const double start = std::max(ready, lane_free[static_cast<size_t>(lane)]);
+      if (best < 0 || start < best_start - 1e-9 || (start < best_start + 1e-9 && tail[j] > tail[static_cast<size_t>(best)])) {
+        best = static_cast<int>(j);
+        best_lane = lane;
+        best_start = start;
+      }
+    }
+    const size_t j = static_cast<size_t>(best);
+    placed[j] = 1;
+    lane_of[j] = best_lane;
+    finish[j] = best_start + est[j];
+    lane_free[static_cast<size_t>(best_lane)] = finish[j];
+    order.push_back(j);
+  }
+  std::vector<int> position(n);
+  for (size_t q = 0; q < n; ++q) position[order[q]] = static_cast<int>(q);
+  std::vector<LaunchSpec> sorted;
+  sorted.reserve(n);
+  for (size_t q = 0; q < n; ++q) {
+    sorted.push_back(std::move(L[order[q]]));
+    sorted.back().lane = lane_of[order[q]];
+    plan->lanes = std::max(plan->lanes, sorted.back().lane + 1);
+  }
+  // a lane runs its launches in order, so waiting for one launch of a lane covers that lane's
+  // earlier launches too
+  std::vector<std::vector<int>> waited(static_cast<size_t>(lanes), std::vector<int>(static_cast<size_t>(lanes), -1));
+  for (size_t q = 0; q < n; ++q) {
+    const size_t lj = static_cast<size_t>(sorted[q].lane);
+    std::vector<int> latest(static_cast<size_t>(lanes), -1);
+    for (int i : deps[order[q]]) {
+      const int pi = position[static_cast<size_t>(i)];
+      const size_t li = static_cast<size_t>(sorted[static_cast<size_t>(pi)].lane);
+      if (li != lj) latest[li] = std::max(latest[li], pi);
+    }
+    for (size_t t = 0; t < latest.size(); ++t)
+      if (latest[t] > waited[lj][t]) {
+        sorted[q].waits.push_back(latest[t]);
+        waited[lj][t] = latest[t];
+      }
+  }
+  L = std::move(sorted);
+}
+
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
   validate_sizes(program);
@@ -2015,6 +2176,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       for (const auto& a : ls.arg_bufs) bound = bound || a == c.first;
     if (!bound) plan.elided.insert(c.first);
   }
+  assign_lanes(&plan, kernels, opt);
   return plan;
 }
 

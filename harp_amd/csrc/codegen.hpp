@@ -28,6 +28,8 @@ struct GenOptions {
   int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
   int gemm_setprio = 0;               // wave priority during the multiply loop
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
+  int lanes = 2;                      // streams a program's launches may be spread over (1 = one after the other)
+  int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
   bool gemm_mix = true;               // LDS operand reads interleaved with the MFMAs of the block before
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
   bool gemm_merge_batch = false;      // per-batch contractions summed over the batch become one contraction
@@ -52,12 +54,17 @@ struct LaunchSpec {
   std::vector<std::string> kernels;    // names of the lowered kernels this launch covers
   double algo_bytes = 0;               // bytes of each distinct external buffer touched once
   double flops = 0;
+  // Filled in by plan_program once all launches are known:
+  std::vector<char> arg_written;       // per parameter: the launch writes that buffer
+  int lane = 0;                        // 0 = the device's stream, 1.. = side streams that run beside it
+  std::vector<int> waits;              // launches on other lanes that must have finished first
 };
 
 struct ProgramPlan {
   std::vector<LaunchSpec> launches;
   std::vector<BufferInfo> buffers;     // table (possibly synthesised from kernel params)
   std::set<std::string> elided;        // temp buffers that never reach memory
+  int lanes = 1;                       // lanes in use (1: every launch on the device's stream)
 };
 
 // Plans a whole Program (one or more kernels, executed in order).  When the program carries no

@@ -89,7 +89,12 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
  *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
- *      gemm_epilogue, gemm_dma, gemm_mix, gemm_merge_batch, nontemporal, normalize, allow_serial.
+ *      gemm_epilogue, gemm_dma, gemm_mix, gemm_merge_batch, nontemporal, normalize, allow_serial,
+ *      lanes, lane_us.
+ *      lanes (default 2): launches of a program that do not depend on each other may be spread
+ *      over that many streams (lane 0 is the device's stream; a program's execute forks the side
+ *      lanes off it and joins them back, so callers still see one stream); launches estimated
+ *      above lane_us microseconds (default 100) stay on lane 0.  lanes=1: one after the other.
  *      A kernel that no schedule recognises, would run in a single work-item and loops more than
  *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1. ----------------- */
 typedef struct eh_launch_info {
@@ -103,6 +108,8 @@ typedef struct eh_launch_info {
   int n_kernels;                        /* lowered kernels covered by this launch */
   double algo_bytes;                    /* each distinct external buffer counted once */
   double flops;                         /* 2*M*N*K for contractions, else 0 */
+  int lane;                             /* 0: the device's stream; 1..: a side stream beside it */
+  int n_waits;                          /* launches on other lanes this one waits for */
 } eh_launch_info;
 
 int eh_render_program(const char* ast_text, const char* options, eh_plan** out);
@@ -118,6 +125,11 @@ int eh_plan_num_launches(eh_plan* plan, int* n);
 int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out);    /* strings live as long as the plan */
 int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name);
 int eh_plan_launch_kernel(eh_plan* plan, int launch, int k, const char** kernel_name);
+/* Whether the launch writes the buffer of parameter `arg`, and launch number `i` (of n_waits) on
+ * another lane that must have finished before this one starts.  Launches are listed in the order
+ * in which they are issued; every launch a launch depends on comes before it. */
+int eh_plan_launch_arg_written(eh_plan* plan, int launch, int arg, int* written);
+int eh_plan_launch_wait(eh_plan* plan, int launch, int i, int* waited_launch);
 int eh_plan_num_buffers(eh_plan* plan, int* n);
 int eh_plan_buffer(eh_plan* plan, int i, const char** name, const char** role, size_t* bytes, int* elided);
 int eh_plan_release(eh_plan* plan);

@@ -8,14 +8,14 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def _cnn_sets(hb, dev, batch, seed):
+def _cnn_sets(hb, dev, batch, seed, options=None):
     from harp_amd import measure, workloads as wl
     from harp_amd.frontend import Tensor
     arrays = wl.config5_inputs(batch, 28, 32, 64, 128, 10, seed=seed)
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     roots = wl.config5_graph(*ts, lr=0.05)
     prog_ast, arg_names, outs, consts, _ = wl.lower_multi(ts, roots)
-    prog = hb.HipProgram(dev, prog_ast, None)
+    prog = hb.HipProgram(dev, prog_ast, options)
     sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 2)
     return prog, sets, arg_names, outs, arrays
 
@@ -124,3 +124,32 @@ def test_other_threads_may_use_the_device_while_a_graph_is_recorded(hip):
         t.join(60)
     assert not errors, errors
     assert rounds[0] > 0
+
+
+def test_lanes_change_nothing_but_the_timing(hip):
+    """The CNN training step with its launches on one stream, on two (the default) and spread over
+    four lanes with no size limit: the same kernels see the same inputs, so every output is equal
+    bit for bit -- on back-to-back executes that reuse the program's temps (a launch of the next
+    execute must not overtake a side-lane launch of the one before), and as a recorded graph."""
+    hb = hip
+    dev = hb.HipDevice(0)
+    want = None
+    for options in ("lanes=1", None, "lanes=4,lane_us=0"):
+        prog, sets, arg_names, outs, arrays = _cnn_sets(hb, dev, 16, seed=94, options=options)
+        lanes = {l["lane"] for l in prog.launches}
+        assert (len(lanes) == 1) == (options == "lanes=1"), lanes
+        for _ in range(3):
+            prog.run(sets[0][0], sync=False)
+        dev.sync()
+        got = _read_outputs(sets[0][1], outs)
+        if want is None:
+            want = got
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), options
+        graph = prog.record(sets[1][0])
+        for _ in range(2):
+            graph.replay()
+        for g, w in zip(_read_outputs(sets[1][1], outs), want):
+            assert np.array_equal(g, w), options
+        del graph, prog, sets
+        dev.trim()

@@ -537,3 +537,58 @@ def test_contraction_with_more_batches_than_grid_z_allows_is_not_put_on_mfma(fro
     assert not any(l["schedule"].startswith("mfma") for l in big), [l["schedule"] for l in big]
     for l in big:
         assert l["grid"][2] <= 65535 and l["grid"][1] <= 65535 and l["grid"][0] < 2 ** 31, l["grid"]
+
+
+def _lane_plan_is_sound(launches):
+    """Issue order is a valid sequential order, and every dependence between launches on different
+    lanes is covered by a wait (directly, or by a later launch of the producer's lane that the
+    consumer's lane has waited for: lanes run in order)."""
+    lanes = max(l["lane"] for l in launches) + 1
+    waited = [[-1] * lanes for _ in range(lanes)]          # [consumer lane][producer lane] -> launch
+    for j, lj in enumerate(launches):
+        for w in lj["waits"]:
+            assert w < j and launches[w]["lane"] != lj["lane"]
+            waited[lj["lane"]][launches[w]["lane"]] = max(waited[lj["lane"]][launches[w]["lane"]], w)
+        for i in range(j):
+            li = launches[i]
+            hazard = any(a == b and (wa or wb) for a, wa in zip(li["args"], li["written"])
+                         for b, wb in zip(lj["args"], lj["written"]))
+            if hazard and li["lane"] != lj["lane"]:
+                assert waited[lj["lane"]][li["lane"]] >= i, (i, li["entry"], j, lj["entry"])
+    return lanes
+
+
+def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
+    """The CNN training step: independent launches (the gradients of the parameters beside the
+    chain that carries the gradient back) go to a side lane.  Producers come before consumers in
+    the issue order, every buffer has its writer marked, and every cross-lane dependence is
+    covered by a wait; with lanes=1 the plan is the same set of launches on lane 0."""
+    from harp_amd import backend as hb
+    from harp_amd import workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config5_inputs(8, *wl.cnn_sizes(False)[1:])
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    prog_ast, arg_names, outs, consts, _ = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))
+    plan = hb.render_program(prog_ast, "lanes=3,lane_us=0")
+    assert _lane_plan_is_sound(plan.launches) == 3
+    assert sum(l["lane"] > 0 for l in plan.launches) >= 8
+    roles = {b["name"]: b["role"] for b in plan.buffers}
+    written = {a for l in plan.launches for a, w in zip(l["args"], l["written"]) if w}
+    read_first = set()
+    seen = set()
+    for l in plan.launches:
+        for a, w in zip(l["args"], l["written"]):
+            if not w and a not in seen and roles.get(a) != "input" and roles.get(a) not in ("ones", "zeros"):
+                read_first.add(a)
+        seen.update(a for a, w in zip(l["args"], l["written"]) if w)
+    assert not read_first, read_first                      # nothing but inputs is read before it is written
+    assert {n for n, r in roles.items() if r == "output"} <= written
+    one = hb.render_program(prog_ast, "lanes=1")
+    assert all(l["lane"] == 0 and not l["waits"] for l in one.launches)
+    assert sorted(l["entry"] for l in one.launches) == sorted(l["entry"] for l in plan.launches)
+    default = hb.render_program(prog_ast)
+    assert _lane_plan_is_sound(default.launches) == 2
+    # a single softmax has nothing to spread
+    from harp_amd import workloads
+    sm = hb.render_program(workloads.lower_with_table([(64, 256)], workloads.config2_graph)[0])
+    assert all(l["lane"] == 0 for l in sm.launches)
