@@ -437,6 +437,8 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
     else if (k == "gemm_dma") o.gemm_dma = as_int() != 0;
     else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
+    else if (k == "reindex") o.reindex = as_int() != 0;
+    else if (k == "guard_branches") o.guard_branches = as_int() != 0;
     else if (k == "lanes") o.lanes = std::max(1, as_int());
     else if (k == "lane_us") o.lane_us = std::max(0, as_int());
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;

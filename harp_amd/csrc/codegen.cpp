@@ -193,9 +193,30 @@ const char* infix(Op op) {
 
 using LoadHook = std::function<bool(const Node& load, std::string* out)>;
 
+bool holds_load(const Node& n) {
+  if (n.op == Op::Load) return true;
+  for (const auto& a : n.args)
+    if (a && holds_load(*a)) return true;
+  return false;
+}
+
+// set by plan_program for the plan it is making (GenOptions::guard_branches)
+thread_local bool g_guard_branches = false;
+
 struct ExprRenderer {
   LoadHook load_hook;
   const std::map<std::string, Ty>* var_types = nullptr;
+  // Conditions of the selects around the expression being rendered.  A load under a select
+  // (padding, window edges: `inside ? x[i] : 0`) is not left to a branch: a load in a branch is
+  // waited for at the branch's end, so the guarded loads of a work-item would go to memory one
+  // after the other, a full latency each.  Both arms are evaluated, the load with its index
+  // clamped to element 0 where the condition does not hold (every buffer has one), and the
+  // select picks: the loads are independent and in flight together.
+  // A load that a hook renders (a value kept in a register, a call of another gather) cannot
+  // have its index clamped here: a select that holds one keeps its branch.
+  mutable std::vector<std::string> guards;
+  mutable bool hooked_under_guard = false;
+  mutable int plain_selects = 0;
 
   std::string math1(const char* f32, const char* f64, const Node& n) const {
     bool dbl = infer_ty(*n.args[0], var_types) == Ty::F64;
@@ -203,6 +224,9 @@ struct ExprRenderer {
   }
 
   std::string expr(const Node& n) const {
+    // a conjunction of pure conditions is evaluated without short-circuit branches (the compiler
+    // otherwise keeps the branches and sinks guarded loads back into them)
+    if (n.op == Op::And && !holds_load(n)) return "((bool)" + expr(*n.args[0]) + " & (bool)" + expr(*n.args[1]) + ")";
     if (const char* s = infix(n.op)) return "(" + expr(*n.args[0]) + " " + s + " " + expr(*n.args[1]) + ")";
     switch (n.op) {
       case Op::Const: return literal(n);
@@ -230,11 +254,41 @@ struct ExprRenderer {
         return std::string(dbl ? "fma(" : "fmaf(") + expr(*n.args[0]) + ", " + expr(*n.args[1]) + ", " +
                expr(*n.args[2]) + ")";
       }
-      case Op::Select:
-        return "(" + expr(*n.args[0]) + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
+      case Op::Select: {
+        if (g_guard_branches || plain_selects > 0 || (!holds_load(*n.args[1]) && !holds_load(*n.args[2])))
+          return "(" + expr(*n.args[0]) + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
+        const std::string c = expr(*n.args[0]);
+        const bool outer_hooked = hooked_under_guard;
+        hooked_under_guard = false;
+        guards.push_back("(bool)" + c);
+        const std::string a = expr(*n.args[1]);
+        guards.back() = "(!" + c + ")";
+        const std::string b = expr(*n.args[2]);
+        guards.pop_back();
+        const bool hooked = hooked_under_guard;
+        hooked_under_guard = outer_hooked || hooked;
+        if (hooked) {
+          ++plain_selects;
+          const std::vector<std::string> saved = std::move(guards);
+          guards.clear();
+          const std::string r = "(" + c + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
+          guards = saved;
+          --plain_selects;
+          return r;
+        }
+        return "({ const auto eh_sa = " + a + "; const auto eh_sb = " + b + "; " + c + " ? eh_sa : eh_sb; })";
+      }
       case Op::Load: {
         std::string s;
-        if (load_hook && load_hook(n, &s)) return s;
+        if (load_hook && load_hook(n, &s)) {
+          if (!guards.empty()) hooked_under_guard = true;
+          return s;
+        }
+        if (n.count == 1 && !guards.empty()) {
+          std::string g = guards[0];
+          for (size_t i = 1; i < guards.size(); ++i) g += " & " + guards[i];
+          return expr(*n.args[0]) + "[(" + g + ") ? " + expr(*n.args[1]) + " : 0]";
+        }
         if (n.count == 1) return expr(*n.args[0]) + "[" + expr(*n.args[1]) + "]";
         return "*reinterpret_cast<const " + ctype(n.dtype) + "*>(&" + expr(*n.args[0]) + "[" + expr(*n.args[1]) + "])";
       }
@@ -1378,6 +1432,188 @@ std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
   return rs;
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// elementwise producers read through another index space: evaluated where they are read
+// ---------------------------------------------------------------------------------------------
+
+// Kernel P computes a temp elementwise, and one other elementwise kernel C is all that reads it --
+// but through other loops: a permutation made contiguous, windows put back into an image, a
+// reshape that regroups axes.  The ordinary fusion needs both kernels to walk the same index
+// space.  Here C's loops are split where P's loop boundaries cut them, so that every loop
+// variable of P becomes a sum of C's (sub-)loop variables, and P's expression takes the place of
+// the load: P, its launch and the temp disappear, and C reads P's operands directly.  Only
+// exact digit correspondences are taken (no division or remainder is ever introduced); C must
+// compute something itself (a pure gather is left alone: contractions and window reductions
+// fold those into their loaders in their own way).
+struct Inlined {
+  NodePtr kernel;            // replaces C
+};
+
+bool pure_gather(const NestKernel& k) {
+  const Node* v = k.value.get();
+  if (v->op == Op::Select && v->args[2]->op == Op::Const) v = v->args[1].get();
+  return v->op == Op::Load;
+}
+
+NodePtr replace_loads(const NodePtr& n, const std::string& buf, const NodePtr& with) {
+  if (n->op == Op::Load && n->args[0]->op == Op::Var && n->args[0]->name == buf) return with;
+  bool changed = false;
+  std::vector<NodePtr> args;
+  args.reserve(n->args.size());
+  for (const auto& a : n->args) {
+    NodePtr r = a ? replace_loads(a, buf, with) : a;
+    changed = changed || r != a;
+    args.push_back(std::move(r));
+  }
+  if (!changed) return n;
+  auto c = std::make_shared<Node>(*n);
+  c->args = std::move(args);
+  return c;
+}
+
+std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C) {
+  if (P.rkind != ReduceKind::None || C.rkind != ReduceKind::None) return std::nullopt;
+  // a pure gather stays one: contractions and window reductions fold gathers (and chains of them)
+  // into their loaders in their own way, which a gather that computes would be lost to
+  if (pure_gather(C) || !C.out_aff) return std::nullopt;
+  int64_t numel = 0;
+  auto strides = dense_strides(P, &numel);
+  if (!strides) return std::nullopt;
+  // every load of the temp in C, all through the same affine index without offset
+  std::vector<LoadRef> loads;
+  collect_loads(*C.value, loads);
+  std::optional<Affine> idx;
+  for (const auto& lr : loads) {
+    if (lr.load->args[0]->op != Op::Var) return std::nullopt;
+    if (lr.load->args[0]->name != P.out_buf) {
+      for (const auto& pp : P.params)               // C must not write what P reads
+        if (pp.name == C.out_buf) return std::nullopt;
+      continue;
+    }
+    if (lr.load->count != 1) return std::nullopt;
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a || a->c != 0) return std::nullopt;
+    if (idx && !(*idx == *a)) return std::nullopt;
+    idx = a;
+  }
+  if (!idx) return std::nullopt;
+  {
+    // the same index space already: the ordinary fusion takes it
+    bool same = P.loops.size() == C.loops.size();
+    for (size_t i = 0; same && i < P.loops.size(); ++i)
+      same = P.loops[i].extent == C.loops[i].extent && idx->of(C.loops[i].var) == (*strides)[i] * (P.loops[i].extent > 1 ? 1 : 0);
+    if (same) return std::nullopt;
+  }
+  // C's terms of the index, ascending; each must rise above what the smaller ones reach
+  struct Term { std::string var; int64_t c, ext; };
+  std::vector<Term> terms;
+  for (const auto& l : C.loops) {
+    const int64_t c = idx->of(l.var);
+    if (c < 0) return std::nullopt;
+    if (c > 0 && l.extent > 1) terms.push_back({l.var, c, l.extent});
+  }
+  for (const auto& kv : idx->coef) {
+    bool known = kv.second == 0;
+    for (const auto& l : C.loops) known = known || l.var == kv.first;
+    if (!known) return std::nullopt;
+  }
+  std::sort(terms.begin(), terms.end(), [](const Term& a, const Term& b) { return a.c < b.c; });
+  int64_t reach = 0;
+  for (const auto& t : terms) {
+    if (t.c <= reach) return std::nullopt;
+    reach += t.c * (t.ext - 1);
+  }
+  if (reach >= numel) return std::nullopt;
+  // cut every term at P's loop boundaries that fall inside it
+  struct Sub { std::string var; int64_t c, ext; };
+  std::vector<Sub> subs;
+  std::map<std::string, NodePtr> c_map;               // C's split variables as sums of their parts
+  std::map<std::string, std::vector<Loop>> c_split;
+  for (const auto& t : terms) {
+    std::vector<int64_t> cuts;                         // factors of the extent, ascending
+    for (size_t q = 0; q < P.loops.size(); ++q) {
+      const int64_t b = (*strides)[q];
+      if (P.loops[q].extent <= 1 || b <= t.c || b >= t.c * t.ext) continue;
+      if (b % t.c || (t.c * t.ext) % b) return std::nullopt;
+      cuts.push_back(b / t.c);
+    }
+    std::sort(cuts.begin(), cuts.end());
+    cuts.erase(std::unique(cuts.begin(), cuts.end()), cuts.end());
+    for (size_t i = 0; i + 1 < cuts.size(); ++i)
+      if (cuts[i + 1] % cuts[i]) return std::nullopt;
+    if (cuts.empty()) {
+      subs.push_back({t.var, t.c, t.ext});
+      continue;
+    }
+    if (t.ext % cuts.back()) return std::nullopt;
+    NodePtr sum;
+    std::vector<Loop> parts;                           // outermost first
+    int64_t below = 1;
+    cuts.push_back(t.ext);
+    for (size_t i = 0; i < cuts.size(); ++i) {
+      const std::string name = t.var + "_p" + std::to_string(i);
+      const int64_t ext = cuts[i] / below;
+      subs.push_back({name, t.c * below, ext});
+      NodePtr part = below == 1 ? make_var(name) : make(Op::Mul, {make_var(name), make_i64(below)});
+      sum = sum ? make(Op::Add, {part, sum}) : part;
+      parts.insert(parts.begin(), Loop{name, ext});
+      below = cuts[i];
+    }
+    c_map[t.var] = sum;
+    c_split[t.var] = parts;
+  }
+  // every loop variable of P as the sum of the parts that lie inside its digit
+  std::map<std::string, NodePtr> p_map;
+  for (size_t q = 0; q < P.loops.size(); ++q) {
+    const int64_t s = (*strides)[q], e = P.loops[q].extent;
+    NodePtr sum;
+    int64_t top = 0;
+    if (e > 1)
+      for (const auto& sb : subs) {
+        if (sb.c * sb.ext <= s || sb.c >= s * e) continue;      // entirely below or above this digit
+        if (sb.c < s || sb.c % s || sb.c * sb.ext > s * e) return std::nullopt;
+        const int64_t m = sb.c / s;
+        NodePtr part = m == 1 ? make_var(sb.var) : make(Op::Mul, {make_var(sb.var), make_i64(m)});
+        sum = sum ? make(Op::Add, {sum, part}) : part;
+        top += m * (sb.ext - 1);
+      }
+    if (top > e - 1) return std::nullopt;
+    p_map[P.loops[q].var] = sum ? sum : make_i64(0);
+  }
+  // the new C: split loops, P's value (cast to the temp's element type) where the temp was read
+  NodePtr pv = rename(P.value, p_map);
+  if (!(P.out_dtype.ty == Ty::F32 && infer_ty(*P.value, nullptr) == Ty::F32)) {
+    auto cast = make(Op::Cast, {pv});
+    cast->dtype = P.out_dtype;
+    pv = cast;
+  }
+  NodePtr value = replace_loads(rename(C.value, c_map), P.out_buf, pv);
+  NodePtr body = make(Op::Store, {make_var(C.out_buf), rename(C.out_index, c_map), value});
+  for (size_t i = C.loops.size(); i-- > 0;) {
+    auto it = c_split.find(C.loops[i].var);
+    if (it == c_split.end()) {
+      body = make_range(C.loops[i].var, C.loops[i].extent, body);
+    } else {
+      for (size_t j = it->second.size(); j-- > 0;) body = make_range(it->second[j].var, it->second[j].extent, body);
+    }
+  }
+  std::vector<Param> params;
+  std::set<std::string> have;
+  for (const auto& pp : C.params)
+    if (pp.name != P.out_buf && have.insert(pp.name).second) params.push_back(pp);
+  // P's operands go in front of C's output (immutable parameters first, as kernels list them)
+  std::vector<Param> ins;
+  for (const auto& pp : P.params)
+    if (pp.dtype.is_ptr() && !pp.mut_ && have.insert(pp.name).second) ins.push_back(pp);
+  size_t first_mut = 0;
+  while (first_mut < params.size() && !params[first_mut].mut_) ++first_mut;
+  params.insert(params.begin() + static_cast<long>(first_mut), ins.begin(), ins.end());
+  Inlined r;
+  r.kernel = make_kernel(C.name, params, body);
+  return r;
+}
+
 }  // namespace
 
 
@@ -1455,6 +1691,10 @@ void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, co
   if (opt.lane_us > 0)
     for (size_t j = 0; j < n; ++j)
       if (est[j] > opt.lane_us) on_main[j] = 1;
+  // lane 0 never waits for a side lane: whatever a launch of lane 0 depends on is on lane 0 too
+  for (size_t j = n; j-- > 0;)
+    if (on_main[j])
+      for (int i : deps[j]) on_main[static_cast<size_t>(i)] = 1;
   double side_us = 0;
   for (size_t j = 0; j < n; ++j)
     if (!on_main[j]) side_us += est[j];
@@ -1543,6 +1783,7 @@ void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, co
 
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
+  g_guard_branches = opt.guard_branches;
   validate_sizes(program);
   ProgramPlan plan;
   std::vector<const Node*> kernels;
@@ -1579,6 +1820,113 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       plan.buffers.push_back(rs->scratch);
     }
     kernels = out;
+  }
+  if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
+    auto is_temp = [&](const std::string& name) {
+      for (const auto& b : plan.buffers)
+        if (b.name == name) return b.role == "temp";
+      return false;
+    };
+    auto writers_of = [&](const std::string& name) {
+      size_t n = 0;
+      for (const Node* k : kernels)
+        for (const auto& pp : k->params) n += pp.dtype.is_ptr() && pp.mut_ && pp.name == name;
+      return n;
+    };
+    auto rename_buffer = [&](const NodePtr& k, const std::string& from, const std::string& to) {
+      NodePtr body = rename(k->args[0], {{from, make_var(to)}});
+      std::vector<Param> params;
+      bool have = false;
+      for (const auto& pp : k->params) have = have || pp.name == to;
+      for (auto pp : k->params) {
+        if (pp.name == from) {
+          if (have) continue;
+          pp.name = to;
+        }
+        params.push_back(pp);
+      }
+      auto c = std::make_shared<Node>(*k);
+      c->params = std::move(params);
+      c->args = {body};
+      return c;
+    };
+    for (bool again = true; again;) {
+      again = false;
+      for (size_t p = 0; p < kernels.size() && !again; ++p) {
+        auto np = extract_nest(*kernels[p]);
+        if (!np || np->rkind != ReduceKind::None || !is_temp(np->out_buf) || writers_of(np->out_buf) != 1) continue;
+        std::vector<size_t> rd;
+        bool early = false;
+        for (size_t c = 0; c < kernels.size(); ++c)
+          for (const auto& pp : kernels[c]->params)
+            if (pp.dtype.is_ptr() && !pp.mut_ && pp.name == np->out_buf) {
+              rd.push_back(c);
+              early = early || c <= p;
+            }
+        if (rd.empty() || early) continue;
+        // a copy of a whole buffer, element for element: its readers read the original
+        if (np->value->op == Op::Load && np->value->args[0]->op == Op::Var && np->value->count == 1 && np->out_aff) {
+          const std::string& src = np->value->args[0]->name;
+          auto a = affine_of(*np->value->args[1]);
+          int64_t numel = 0;
+          bool same_type = false;
+          for (const auto& pp : np->params) same_type = same_type || (pp.name == src && pp.dtype.is_ptr() && pp.dtype.elem().ty == np->out_dtype.ty);
+          if (a && *a == *np->out_aff && dense_strides(*np, &numel) && same_type && src != np->out_buf && writers_of(src) <= 1) {
+            bool src_written_later = false;
+            for (size_t m = p + 1; m < kernels.size(); ++m)
+              for (const auto& pm : kernels[m]->params) src_written_later = src_written_later || (pm.dtype.is_ptr() && pm.mut_ && pm.name == src);
+            if (!src_written_later) {
+              for (size_t c : rd) {
+                NodePtr owner;
+                for (const auto& f : program.args)
+                  if (f.get() == kernels[c]) owner = f;
+                for (const auto& f : rewritten)
+                  if (f.get() == kernels[c]) owner = f;
+                if (!owner) throw Error("internal: kernel without owner");
+                NodePtr nk = rename_buffer(owner, np->out_buf, src);
+                rewritten.push_back(nk);
+                kernels[c] = nk.get();
+              }
+              plan.elided.insert(np->out_buf);
+              kernels.erase(kernels.begin() + static_cast<long>(p));
+              again = true;
+              continue;
+            }
+          }
+        }
+        if (rd.size() > 3) continue;
+        {
+          std::vector<LoadRef> pl;
+          collect_loads(*np->value, pl);
+          std::set<std::string> srcs;
+          for (const auto& lr : pl)
+            if (lr.load->args[0]->op == Op::Var) srcs.insert(lr.load->args[0]->name);
+          if (rd.size() > 1 && srcs.size() > 4) continue;    // evaluated once per reader: keep it cheap
+        }
+        size_t left = rd.size();
+        for (size_t reader : rd) {
+          // nothing between the two may write what P reads
+          bool clobbered = false;
+          for (size_t m = p + 1; m <= reader; ++m)
+            for (const auto& pm : kernels[m]->params)
+              if (pm.dtype.is_ptr() && pm.mut_)
+                for (const auto& pp : kernels[p]->params) clobbered = clobbered || (pp.name == pm.name && !pp.mut_);
+          if (clobbered) continue;
+          auto nc = extract_nest(*kernels[reader]);
+          if (!nc) continue;
+          auto in = inline_producer(*np, *nc);
+          if (!in) continue;
+          rewritten.push_back(in->kernel);
+          kernels[reader] = in->kernel.get();
+          --left;
+          again = true;
+        }
+        if (left == 0) {
+          plan.elided.insert(np->out_buf);
+          kernels.erase(kernels.begin() + static_cast<long>(p));
+        }
+      }
+    }
   }
   std::map<std::string, size_t> elems;
   bool have_table = !plan.buffers.empty();

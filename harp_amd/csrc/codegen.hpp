@@ -30,6 +30,8 @@ struct GenOptions {
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
   int lanes = 2;                      // streams a program's launches may be spread over (1 = one after the other)
   int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
+  bool reindex = true;                // elementwise producers evaluated in a reader that walks another index space
+  bool guard_branches = false;        // guarded loads (padding, edges) behind branches instead of clamped indices and selects
   bool gemm_mix = true;               // LDS operand reads interleaved with the MFMAs of the block before
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
   bool gemm_merge_batch = false;      // per-batch contractions summed over the batch become one contraction

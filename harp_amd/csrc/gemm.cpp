@@ -1,6 +1,7 @@
 #include "gemm.hpp"
 
 #include <algorithm>
+#include <cctype>
 #include <cmath>
 #include <cstdlib>
 #include <sstream>
@@ -32,6 +33,13 @@ const Candidate kCandidates[] = {
     {{256, 256, 16, 64, 64}, 1, 133.0, 1.0, 1.2},    // 16 waves
     {{128, 128, 16, 64, 64}, 4, 124.0, 0.4, 1.0},    // 4 waves
     {{64, 64, 16, 32, 32}, 8, 105.0, 0.25, 0.8},     // 4 waves
+    // narrow tiles for contractions with few rows or columns (a convolution's 32 channels, a
+    // 3x3 filter's nine taps, ten classes), where a 64-wide tile multiplies mostly padding
+    // (measured on the CNN step: 32x64 takes the first convolution, 32 channels by 784 pixels,
+    // from 23 to 16 us; 128x32x32 and 32x32x16 tiles were tried as well and lost to 64x64 wherever
+    // they were chosen)
+    {{64, 32, 16, 32, 32}, 12, 80.0, 0.12, 0.8},     // 2 waves
+    {{32, 64, 16, 32, 32}, 12, 80.0, 0.12, 0.8},     // 2 waves
 };
 
 bool tile_valid(const Tile& t) {
@@ -81,7 +89,7 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool compute
   if (s.K < 8 || s.M < 2 || s.N < 2) return false;
   // the batch rides on blockIdx.z (at most 65535 workgroups); the tiles of one batch on blockIdx.x.
   // Beyond either the contraction is left to the other reduce schedules.
-  if (s.batch > 65535 || ceil_div(s.M, 64) * ceil_div(s.N, 64) >= (int64_t{1} << 31)) return false;
+  if (s.batch > 65535 || ceil_div(s.M, 32) * ceil_div(s.N, 32) >= (int64_t{1} << 31)) return false;
   Choice best;
   if (opt.gemm_bm > 0) {
     best.tile = Tile{opt.gemm_bm, opt.gemm_bn, opt.gemm_bk, opt.gemm_wm, opt.gemm_wn};
@@ -97,7 +105,7 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool compute
     // an operand evaluated in the tile loader (index decode, guards) slows every k-step of a
     // workgroup down; many small workgroups hide that, a few large ones do not (measured: a
     // 3x3 convolution over [32,128,28,28], 64x64 tiles 142 us, 128x128 295 us, 256x256 380 us)
-    if (computed_operand && c.tile.bm > 64) continue;
+    if (computed_operand && c.tile.bm * c.tile.bn > 64 * 64) continue;
     const int64_t ksteps = ceil_div(s.K, c.tile.bk);
     for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
@@ -291,7 +299,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   // only moves the quotient and the k part only the remainder (mode 1), or the other way round
   // (mode 2), the part that belongs to the row is the same for every k step, and the compiler
   // hoists its decode out of the k loop; no division by Q is needed either.
-  auto emit_fold = [&](const FoldedOperand* f, const char* X, const char* fn, int64_t off, int64_t bs, int64_t sr,
+  auto emit_fold = [&](const FoldedOperand* f, const char* X, const char* /*fn*/, int64_t off, int64_t bs, int64_t sr,
                        int64_t sk, int64_t rows, int64_t kext) {
     if (!f) return;
     int64_t total = 1;
@@ -314,15 +322,33 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     os << "#define EH_" << X << "_FOLD 1\n#define EH_" << X << "_FOLD_MODE " << mode << "\n#define EH_" << X << "_FOLD_Q " << Q
        << "LL\n";
     os << f->prelude;
-    os << "// element (eh_U * " << Q << " + eh_I) of what kernel " << f->kernel << " would have written\n";
-    os << "__device__ __forceinline__ float " << fn << "(const float* __restrict__ " << f->src
-       << ", long long eh_U64, long long eh_I64) {\n";
-    os << "  const " << IT << " eh_U = (" << IT << ")eh_U64, eh_I = (" << IT << ")eh_I64;\n";
+    // The element at index eh_U * Q + eh_I of what the producer would have written: its loop
+    // variables above Q are decoded from eh_U, those below from eh_I, each by a function of its
+    // own, so that the caller decodes the half that belongs to the row once and the half that
+    // belongs to k once per k.
+    const std::string P = std::string("eh_") + static_cast<char>(std::tolower(X[0]));
+    std::ostringstream up, lo, dup, dlo, use;
     for (const auto& l : f->loops) {
-      if (l.extent == 1) os << "  const " << IT << " " << l.name << " = 0;\n";
-      else if (l.stride >= Q) os << "  const " << IT << " " << l.name << " = (eh_U / " << l.stride / Q << ") % " << l.extent << ";\n";
-      else os << "  const " << IT << " " << l.name << " = (eh_I / " << l.stride << ") % " << l.extent << ";\n";
+      if (l.extent == 1) {
+        use << "  const " << IT << " " << l.name << " = 0;\n";
+      } else if (l.stride >= Q) {
+        up << "  " << IT << " " << l.name << ";\n";
+        dup << "  r." << l.name << " = (eh_U / " << l.stride / Q << ") % " << l.extent << ";\n";
+        use << "  const " << IT << " " << l.name << " = eh_u." << l.name << ";\n";
+      } else {
+        lo << "  " << IT << " " << l.name << ";\n";
+        dlo << "  r." << l.name << " = (eh_I / " << l.stride << ") % " << l.extent << ";\n";
+        use << "  const " << IT << " " << l.name << " = eh_l." << l.name << ";\n";
+      }
     }
+    os << "// element (eh_U * " << Q << " + eh_I) of what kernel " << f->kernel << " would have written\n";
+    os << "struct " << P << "_upper {\n" << up.str() << "};\nstruct " << P << "_lower {\n" << lo.str() << "};\n";
+    os << "__device__ __forceinline__ " << P << "_upper " << P << "_dec_upper(long long eh_U64) {\n  const " << IT << " eh_U = ("
+       << IT << ")eh_U64;\n  (void)eh_U;\n  " << P << "_upper r;\n" << dup.str() << "  return r;\n}\n";
+    os << "__device__ __forceinline__ " << P << "_lower " << P << "_dec_lower(long long eh_I64) {\n  const " << IT << " eh_I = ("
+       << IT << ")eh_I64;\n  (void)eh_I;\n  " << P << "_lower r;\n" << dlo.str() << "  return r;\n}\n";
+    os << "__device__ __forceinline__ float " << P << "_val(const float* __restrict__ " << f->src << ", const " << P
+       << "_upper& eh_u, const " << P << "_lower& eh_l) {\n  (void)eh_u;\n  (void)eh_l;\n" << use.str();
     os << "  return (float)(" << f->expr << ");\n}\n";
   };
   const bool epi_here = epilogue && S == 1;     // with K split the epilogue runs in the summing launch
@@ -344,6 +370,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   }
   os << "#define EH_SETPRIO " << std::max(0, std::min(3, opt.gemm_setprio)) << "\n";
   os << "#define EH_MIX " << (opt.gemm_mix ? 1 : 0) << "\n";
+  os << "#define EH_LOAD_BRANCH " << (opt.guard_branches ? 1 : 0) << "\n";
   os << kGemmSource;
   ls.source = os.str();
   const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;

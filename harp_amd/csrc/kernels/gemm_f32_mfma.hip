@@ -64,6 +64,9 @@
 #ifndef EH_SETPRIO
 #define EH_SETPRIO 0     // wave priority while multiplying
 #endif
+#ifndef EH_LOAD_BRANCH
+#define EH_LOAD_BRANCH 0  // element-by-element tile loads: a branch around each out-of-range element (1) or a clamped index and a select (0)
+#endif
 #ifndef EH_MIX
 #define EH_MIX 1         // LDS operand reads are issued one at a time between the MFMAs of the block before
 #endif
@@ -122,64 +125,129 @@ static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B ca
 
 // How an operand's element (batch bz, row r, k) is obtained: from memory at
 // off + bz*bs + r*sr + k*sk, or (EH_A_FOLD / EH_B_FOLD) by evaluating the elementwise kernel
-// that would have produced that element, on that kernel's own source.  The generated function
-// takes the element's index split at Q into (quotient, remainder); in mode 1 the row decides
-// the quotient and k the remainder, in mode 2 the other way round, so whatever is decoded from
-// the row's part is loop-invariant along k.
+// that would have produced that element, on that kernel's own source.  Either way in three
+// steps, so that what depends on the row alone is worked out once per work-item, ahead of the
+// k loop, and what depends on k alone once per k: row(bz, r) and kk(bz, k) decode their share of
+// the element's index, val(p, row, kk) reads or evaluates the element.  For a computed operand
+// the generator splits the producer's loop variables at Q: in mode 1 the row decides the
+// variables above Q and k those below, in mode 2 the other way round; in mode 0 the index does
+// not separate and val decodes all of it.
 template <long long OFF, long long BS, long long SR, long long SK>
 struct EhFromMemory {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
-    return p[OFF + bz * BS + r * SR + k * SK];
-  }
+  typedef long long Row;
+  typedef long long Kk;
+  __device__ __forceinline__ static Row row(long long bz, long long r) { return OFF + bz * BS + r * SR; }
+  __device__ __forceinline__ static Kk kk(long long, long long k) { return k * SK; }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return p[r + k]; }
 };
 #ifdef EH_A_FOLD
 struct EhAElem {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
-    constexpr long long Q = EH_A_FOLD_Q;
+  static constexpr long long Q = EH_A_FOLD_Q;
 #if EH_A_FOLD_MODE == 1
-    return eh_a_elem(p, EH_A_OFF / Q + bz * (EH_A_BS / Q) + r * (EH_A_SM / Q), k * EH_A_SK);
+  typedef eh_a_upper Row;
+  typedef eh_a_lower Kk;
+  __device__ __forceinline__ static Row row(long long bz, long long r) { return eh_a_dec_upper(EH_A_OFF / Q + bz * (EH_A_BS / Q) + r * (EH_A_SM / Q)); }
+  __device__ __forceinline__ static Kk kk(long long, long long k) { return eh_a_dec_lower(k * EH_A_SK); }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return eh_a_val(p, r, k); }
 #elif EH_A_FOLD_MODE == 2
-    return eh_a_elem(p, EH_A_OFF / Q + bz * (EH_A_BS / Q) + k * (EH_A_SK / Q), r * EH_A_SM);
+  typedef eh_a_lower Row;
+  typedef eh_a_upper Kk;
+  __device__ __forceinline__ static Row row(long long, long long r) { return eh_a_dec_lower(r * EH_A_SM); }
+  __device__ __forceinline__ static Kk kk(long long bz, long long k) { return eh_a_dec_upper(EH_A_OFF / Q + bz * (EH_A_BS / Q) + k * (EH_A_SK / Q)); }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return eh_a_val(p, k, r); }
 #else
-    return eh_a_elem(p, 0, EH_A_OFF + bz * EH_A_BS + r * EH_A_SM + k * EH_A_SK);
-#endif
+  typedef long long Row;
+  typedef long long Kk;
+  __device__ __forceinline__ static Row row(long long bz, long long r) { return EH_A_OFF + bz * EH_A_BS + r * EH_A_SM; }
+  __device__ __forceinline__ static Kk kk(long long, long long k) { return k * EH_A_SK; }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) {
+    return eh_a_val(p, eh_a_dec_upper(0), eh_a_dec_lower(r + k));
   }
+#endif
 };
 #else
 using EhAElem = EhFromMemory<EH_A_OFF, EH_A_BS, EH_A_SM, EH_A_SK>;
 #endif
 #ifdef EH_B_FOLD
 struct EhBElem {
-  __device__ __forceinline__ static float at(const float* __restrict__ p, long long bz, long long r, long long k) {
-    constexpr long long Q = EH_B_FOLD_Q;
+  static constexpr long long Q = EH_B_FOLD_Q;
 #if EH_B_FOLD_MODE == 1
-    return eh_b_elem(p, EH_B_OFF / Q + bz * (EH_B_BS / Q) + r * (EH_B_SN / Q), k * EH_B_SK);
+  typedef eh_b_upper Row;
+  typedef eh_b_lower Kk;
+  __device__ __forceinline__ static Row row(long long bz, long long r) { return eh_b_dec_upper(EH_B_OFF / Q + bz * (EH_B_BS / Q) + r * (EH_B_SN / Q)); }
+  __device__ __forceinline__ static Kk kk(long long, long long k) { return eh_b_dec_lower(k * EH_B_SK); }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return eh_b_val(p, r, k); }
 #elif EH_B_FOLD_MODE == 2
-    return eh_b_elem(p, EH_B_OFF / Q + bz * (EH_B_BS / Q) + k * (EH_B_SK / Q), r * EH_B_SN);
+  typedef eh_b_lower Row;
+  typedef eh_b_upper Kk;
+  __device__ __forceinline__ static Row row(long long, long long r) { return eh_b_dec_lower(r * EH_B_SN); }
+  __device__ __forceinline__ static Kk kk(long long bz, long long k) { return eh_b_dec_upper(EH_B_OFF / Q + bz * (EH_B_BS / Q) + k * (EH_B_SK / Q)); }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return eh_b_val(p, k, r); }
 #else
-    return eh_b_elem(p, 0, EH_B_OFF + bz * EH_B_BS + r * EH_B_SN + k * EH_B_SK);
-#endif
+  typedef long long Row;
+  typedef long long Kk;
+  __device__ __forceinline__ static Row row(long long bz, long long r) { return EH_B_OFF + bz * EH_B_BS + r * EH_B_SN; }
+  __device__ __forceinline__ static Kk kk(long long, long long k) { return k * EH_B_SK; }
+  __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) {
+    return eh_b_val(p, eh_b_dec_upper(0), eh_b_dec_lower(r + k));
   }
+#endif
 };
 #else
 using EhBElem = EhFromMemory<EH_B_OFF, EH_B_BS, EH_B_SN, EH_B_SK>;
 #endif
 
+// The rows a work-item reads of an operand tile, decoded once: one row (the four elements run
+// along k) or four neighbouring ones (the four run along the row axis).  Rows past the end
+// decode row 0 and are marked.
+template <class ELEM, bool ALONG_K>
+struct EhRows {
+  static constexpr int NR = ALONG_K ? 1 : 4;
+  typename ELEM::Row row[NR];
+  bool ok[NR];
+  __device__ __forceinline__ void set(long long bz, long long r, long long R) {
+#pragma unroll
+    for (int e = 0; e < NR; ++e) {
+      ok[e] = r + e < R;
+      row[e] = ELEM::row(bz, ok[e] ? r + e : 0);
+    }
+  }
+};
+
 // Four elements of an operand starting at (r, k) and running along its fast axis; elements
 // outside [0,R) x [0,kend) read as zero.  ALONG_K says which axis the four run along; `base`
-// is the operand's offset plus the batch offset (used by the 128-bit path).
+// is the operand's offset plus the batch offset (used by the 128-bit path), `rows` the decoded
+// rows (used by the element-by-element path).
 template <class ELEM, bool VEC, bool ALONG_K, bool EDGE_R, long long SR, long long SK>
 __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long long base, long long bz, long long r,
-                                              long long k, long long R, long long kend) {
+                                              long long k, long long R, long long kend, const EhRows<ELEM, ALONG_K>& rows) {
   eh_f4v v = {0.0f, 0.0f, 0.0f, 0.0f};
   if (VEC) {
     const bool ok = (!EDGE_R || r < R) && (!EDGE_K || k < kend);
     if (ok) v = *reinterpret_cast<const eh_f4v*>(p + base + r * SR + k * SK);
-  } else {
+  } else if (ALONG_K) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const long long rr = ALONG_K ? r : r + e, kk = ALONG_K ? k + e : k;
-      if (rr < R && kk < kend) v[e] = ELEM::at(p, bz, rr, kk);
+      const bool ok = rows.ok[0] & (k + e < kend);
+#if EH_LOAD_BRANCH
+      if (ok) v[e] = ELEM::val(p, rows.row[0], ELEM::kk(bz, k + e));
+#else
+      const float x = ELEM::val(p, rows.row[0], ELEM::kk(bz, ok ? k + e : 0));
+      v[e] = ok ? x : 0.0f;
+#endif
+    }
+  } else {
+    const bool kok = k < kend;
+    const typename ELEM::Kk kinfo = ELEM::kk(bz, kok ? k : 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool ok = rows.ok[e] & kok;
+#if EH_LOAD_BRANCH
+      if (ok) v[e] = ELEM::val(p, rows.row[e], kinfo);
+#else
+      const float x = ELEM::val(p, rows.row[e], kinfo);
+      v[e] = ok ? x : 0.0f;
+#endif
     }
   }
   return v;
@@ -275,6 +343,23 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #endif
 
   eh_f4v ra[AV], rb[BV];
+  // the rows of each tile this work-item fetches, decoded once (they do not change with k)
+  EhRows<EhAElem, EH_A_KCONTIG != 0> a_rows[AV];
+  EhRows<EhBElem, EH_B_NCONTIG == 0> b_rows[BV];
+#if !EH_A_VEC && !EH_A_DMA
+#pragma unroll
+  for (int i = 0; i < AV; ++i) {
+    const int q = tid + i * NT;
+    a_rows[i].set(bz, EH_A_KCONTIG ? m0 + q / (BK / 4) : m0 + (q % (BM / 4)) * 4, M);
+  }
+#endif
+#if !EH_B_VEC && !EH_B_DMA
+#pragma unroll
+  for (int i = 0; i < BV; ++i) {
+    const int q = tid + i * NT;
+    b_rows[i].set(bz, EH_B_NCONTIG ? n0 + (q % (BN / 4)) * 4 : n0 + q / (BK / 4), N);
+  }
+#endif
 
   // thread q of the tile owns four elements: along k at (row q / (BK/4), k 4*(q % (BK/4))) for
   // a k-contiguous operand, along the row at (k q / (rows/4), row 4*(q % (rows/4))) otherwise
@@ -294,10 +379,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(A + a_base + (k0 + k) * EH_A_SK + (m0 + mq * 4) * EH_A_SM, a_tile, (tid & ~63) + i * NT);
 #elif EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend, a_rows[i]);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend);
+      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend, a_rows[i]);
 #endif
     }
 #pragma unroll
@@ -308,10 +393,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(B + b_base + (k0 + k) * EH_B_SK + (n0 + nq * 4) * EH_B_SN, b_tile, (tid & ~63) + i * NT);
 #elif EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend, b_rows[i]);
 #else
       const int n = q / (BK / 4), kq = q % (BK / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + n, k0 + kq * 4, N, kend);
+      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + n, k0 + kq * 4, N, kend, b_rows[i]);
 #endif
     }
   };
