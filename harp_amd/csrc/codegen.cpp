@@ -1901,7 +1901,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           std::set<std::string> srcs;
           for (const auto& lr : pl)
             if (lr.load->args[0]->op == Op::Var) srcs.insert(lr.load->args[0]->name);
-          if (rd.size() > 1 && srcs.size() > 4) continue;    // evaluated once per reader: keep it cheap
+          if (rd.size() > 1 && srcs.size() > 6) continue;    // evaluated once per reader: keep it cheap
         }
         size_t left = rd.size();
         for (size_t reader : rd) {
@@ -1915,6 +1915,8 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           auto nc = extract_nest(*kernels[reader]);
           if (!nc) continue;
           auto in = inline_producer(*np, *nc);
+          if (std::getenv("ECLAT_HIP_DEBUG_REINDEX"))
+            fprintf(stderr, "reindex: %s (%s) into %s: %s\n", np->name.c_str(), np->out_buf.c_str(), nc->name.c_str(), in ? "yes" : "no");
           if (!in) continue;
           rewritten.push_back(in->kernel);
           kernels[reader] = in->kernel.get();
