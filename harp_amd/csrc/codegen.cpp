@@ -1614,6 +1614,119 @@ std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C)
   return r;
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// a contraction's temp stored the other way round when its reader walks it column by column
+// ---------------------------------------------------------------------------------------------
+
+// A contraction writes a dense temp T[m][n] (n contiguous) and the one elementwise kernel that
+// reads it walks m with its innermost loop (the input gradient of a convolution: the columns
+// written by `dY x W`, summed window by window along the image's x): every lane then reads from
+// another row, N elements apart.  A temp's layout is nobody else's business, so both sides are
+// rewritten to T[n][m]: the contraction computes the transposed product (same work, stores still
+// along its tile's contiguous axis) and the reader's innermost loop becomes unit stride.
+NodePtr affine_expr(const Affine& a) {
+  NodePtr e;
+  for (const auto& kv : a.coef) {
+    if (kv.second == 0) continue;
+    NodePtr t = kv.second == 1 ? make_var(kv.first) : make(Op::Mul, {make_var(kv.first), make_i64(kv.second)});
+    e = e ? make(Op::Add, {e, t}) : t;
+  }
+  if (a.c != 0 || !e) e = e ? make(Op::Add, {e, make_i64(a.c)}) : make_i64(a.c);
+  return e;
+}
+
+// idx = m*N + n with 0 <= n < N for every value of the loops  ->  n*M + m; nullopt when the
+// split cannot be read off the coefficients
+std::optional<Affine> transposed_index(const Affine& a, const std::vector<Loop>& loops, const Loop* rloop, int64_t M, int64_t N) {
+  Affine r;
+  const int64_t lo_c = ((a.c % N) + N) % N;
+  int64_t lo_max = lo_c;
+  r.c = lo_c * M + (a.c - lo_c) / N;
+  for (const auto& kv : a.coef) {
+    if (kv.second == 0) continue;
+    int64_t ext = 0;
+    for (const auto& l : loops)
+      if (l.var == kv.first) ext = l.extent;
+    if (rloop && rloop->var == kv.first) ext = rloop->extent;
+    if (ext <= 0 || kv.second < 0) return std::nullopt;
+    if (kv.second % N == 0) {
+      r.coef[kv.first] = kv.second / N;
+    } else {
+      if (kv.second >= N) return std::nullopt;
+      lo_max += kv.second * (ext - 1);
+      r.coef[kv.first] = kv.second * M;
+    }
+  }
+  if (lo_max >= N) return std::nullopt;
+  return r;
+}
+
+NodePtr reindex_loads(const NodePtr& n, const std::string& buf, const std::function<NodePtr(const Node&)>& new_index) {
+  if (n->op == Op::Load && n->args[0]->op == Op::Var && n->args[0]->name == buf) {
+    auto c = std::make_shared<Node>(*n);
+    c->args[1] = new_index(*n->args[1]);
+    return c;
+  }
+  bool changed = false;
+  std::vector<NodePtr> args;
+  args.reserve(n->args.size());
+  for (const auto& a : n->args) {
+    NodePtr r = a ? reindex_loads(a, buf, new_index) : a;
+    changed = changed || r != a;
+    args.push_back(std::move(r));
+  }
+  if (!changed) return n;
+  auto c = std::make_shared<Node>(*n);
+  c->args = std::move(args);
+  return c;
+}
+
+// The contraction K with its output stored transposed; M and N are set to T's extents.
+NodePtr transpose_producer(const NestKernel& K, const GenOptions& opt, int64_t* Mo, int64_t* No) {
+  if (K.rkind != ReduceKind::Sum || !K.out_aff || !opt.gemm) return nullptr;
+  auto sh = match_gemm(K);
+  if (!sh || sh->batch != 1 || !gemm_output_dense(*sh) || sh->c_buf != K.out_buf) return nullptr;
+  const int64_t M = sh->M, N = sh->N;
+  if (M * N < (int64_t{1} << 20) || N < 8) return nullptr;
+  auto kout = transposed_index(*K.out_aff, K.loops, nullptr, M, N);
+  if (!kout) return nullptr;
+  NodePtr body = make_reduce_block(K, K.rloop.var, K.rloop.extent, K.value, K.out_buf, affine_expr(*kout));
+  for (size_t i = K.loops.size(); i-- > 0;) body = make_range(K.loops[i].var, K.loops[i].extent, body);
+  *Mo = M;
+  *No = N;
+  return make_kernel(K.name, K.params, body);
+}
+
+// Reader E of T[M][N] rewritten for T[N][M]; null when E does not walk T's rows with its
+// innermost loop in every load, or an index does not split.
+NodePtr transpose_reader(const NestKernel& E, const std::string& T, int64_t M, int64_t N) {
+  if (E.rkind != ReduceKind::None) return nullptr;
+  std::vector<LoadRef> loads;
+  collect_loads(*E.value, loads);
+  // the reader's innermost live loop must walk rows of T in every load of it
+  const Loop* inner = nullptr;
+  for (const auto& l : E.loops)
+    if (l.extent > 1) inner = &l;
+  if (!inner) return nullptr;
+  size_t sites = 0;
+  for (const auto& lr : loads) {
+    if (lr.load->args[0]->op != Op::Var || lr.load->args[0]->name != T) continue;
+    if (lr.load->count != 1) return nullptr;
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a || a->of(inner->var) != N) return nullptr;
+    if (!transposed_index(*a, E.loops, nullptr, M, N)) return nullptr;
+    ++sites;
+  }
+  if (!sites) return nullptr;
+  NodePtr value = reindex_loads(E.value, T, [&](const Node& idx) {
+    return affine_expr(*transposed_index(*affine_of(idx), E.loops, nullptr, M, N));
+  });
+  NodePtr body = make(Op::Store, {make_var(E.out_buf), E.out_index, value});
+  for (size_t i = E.loops.size(); i-- > 0;) body = make_range(E.loops[i].var, E.loops[i].extent, body);
+  return make_kernel(E.name, E.params, body);
+}
+
 }  // namespace
 
 
@@ -1927,6 +2040,61 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           plan.elided.insert(np->out_buf);
           kernels.erase(kernels.begin() + static_cast<long>(p));
         }
+      }
+    }
+  }
+  if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
+    // temps between a contraction and an elementwise reader that walks them column by column
+    for (size_t p = 0; p < kernels.size(); ++p) {
+      auto nk = extract_nest(*kernels[p]);
+      if (!nk || nk->rkind != ReduceKind::Sum) continue;
+      bool temp = false;
+      for (const auto& b : plan.buffers) temp = temp || (b.name == nk->out_buf && b.role == "temp");
+      if (!temp) continue;
+      std::vector<size_t> rd;
+      size_t nwriters = 0;
+      bool early = false;
+      for (size_t c = 0; c < kernels.size(); ++c)
+        for (const auto& pp : kernels[c]->params)
+          if (pp.dtype.is_ptr() && pp.name == nk->out_buf) {
+            if (pp.mut_) ++nwriters;
+            else { rd.push_back(c); early = early || c <= p; }
+          }
+      if (rd.empty() || nwriters != 1 || early) continue;
+      {
+        // one reader that reads every element once, unguarded, is a plain permutation: the
+        // contraction's epilogue writes that reader's result in place instead
+        size_t sites = 0;
+        bool guarded = false;
+        for (size_t c : rd) {
+          auto ne = extract_nest(*kernels[c]);
+          if (!ne) continue;
+          std::vector<LoadRef> lds;
+          collect_loads(*ne->value, lds);
+          for (const auto& lr : lds)
+            if (lr.load->args[0]->op == Op::Var && lr.load->args[0]->name == nk->out_buf) {
+              ++sites;
+              guarded = guarded || lr.guarded;
+            }
+        }
+        if (sites < 2 && !guarded) continue;
+      }
+      int64_t M = 0, N = 0;
+      NodePtr prod = transpose_producer(*nk, opt, &M, &N);
+      if (!prod) continue;
+      std::vector<NodePtr> readers_new;
+      for (size_t c : rd) {
+        auto ne = extract_nest(*kernels[c]);
+        NodePtr r = ne ? transpose_reader(*ne, nk->out_buf, M, N) : nullptr;
+        if (!r) break;
+        readers_new.push_back(r);
+      }
+      if (readers_new.size() != rd.size()) continue;
+      rewritten.push_back(prod);
+      kernels[p] = prod.get();
+      for (size_t i = 0; i < rd.size(); ++i) {
+        rewritten.push_back(readers_new[i]);
+        kernels[rd[i]] = readers_new[i].get();
       }
     }
   }
