@@ -167,7 +167,7 @@ def main():
         ms, wall_ms = measure.time_steps(dev, prog, sets, args.steps, args.warmup)
         algo = sum(l["algo_bytes"] for l in prog.launches)
         cfg1 = {"us": ms * 1e3, "wall_us": wall_ms * 1e3, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo,
-                "launch": prog.launches[0]}
+                "launch": prog.launches[0], "floor_us": measure.launch_floor_us(dev, prog.launches[0]["grid"][0])}
         log(f"[bench] config1 relu-sum 1024^2: {cfg1['us']:.2f} us/step -> {cfg1['gbs']:.0f} GB/s")
 
         def check_cfg1(got):
@@ -358,7 +358,10 @@ def main():
             "us_per_step": round(cfg1["us"], 2), "host_us_per_step": round(cfg1["wall_us"], 2),
             "value": round(cfg1["gbs"], 1), "unit": "GB/s", "schedule": cfg1["launch"]["schedule"],
             "roofline": roofline("hbm", cfg1["gbs"], "GB/s", cfg1["algo_bytes"], cfg1["launch"]),
-            "note": "12.6 MB per launch is 1.6 us at peak: the step is bound by launch and drain of one small grid"}
+            "empty_kernel_us_per_launch": round(cfg1["floor_us"], 2),
+            "us_above_empty_kernel": round(cfg1["us"] - cfg1["floor_us"], 2),
+            "note": "12.6 MB per launch is 1.6 us at peak; empty_kernel_us_per_launch is the same grid of a kernel that "
+                    "does nothing, queued back to back the same way: the part of the step that is launch and drain"}
         if cfg1["per_kernel"]:
             extra.setdefault("per_kernel_path", {})["config1_relu_sum_1024"] = cfg1["per_kernel"]
     if mlp:

@@ -63,8 +63,8 @@ template <class Op, int W, class T> __device__ __forceinline__ T eh_lanes_reduce
   return v;
 }
 
-// Reduction over the T threads that share a row.  T <= 64: lanes only.  T > 64: one row per
-// workgroup, per-wave partials staged through LDS (one slot array per reduction, one barrier).
+// Reduction over the T threads that share a row.  T <= 64: lanes only.  T > 64: per-wave partials
+// staged through LDS (`lds`: this row's T/64 slots, one slot array per reduction, one barrier).
 template <class Op, int T, class V> __device__ __forceinline__ V eh_row_reduce(V v, V* lds, int lr) {
   if (T <= 64) return eh_lanes_reduce<Op, T>(v);
   v = eh_lanes_reduce<Op, 64>(v);
@@ -3231,7 +3231,7 @@ struct GroupEmitter {
       int r = 0;
       for (const auto& st : g.stages)
         if (st.kind == StageKind::Reduce)
-          os << "  __shared__ " << ctype(st.acc_dtype) << " eh_red" << r++ << "[" << T / 64 << "];\n";
+          os << "  __shared__ " << ctype(st.acc_dtype) << " eh_red" << r++ << "[" << RPB * (T / 64) << "];\n";
     }
     const std::string iter_open = std::string(reg ? "#pragma unroll\n" : "") +
                                   "  for (int k = 0; k < NV; ++k) {\n    const idx_t c0 = (idx_t)(k * T + lr) * V;\n";
@@ -3270,7 +3270,9 @@ struct GroupEmitter {
            << combine_text(st.rk, st.acc_dtype, acc, "(" + TA + ")(" + value_text(st, ld) + ")") << "; }\n";
         os << "    }\n  }\n";
         os << "  const " << TA << " " << sname(st.out_buf) << " = eh_row_reduce<" << op_struct(st.rk) << ", T>(" << acc
-           << ", " << (T > 64 ? "eh_red" + std::to_string(red_i) : std::string("(" + TA + "*)nullptr")) << ", lr);\n";
+           << ", "
+           << (T > 64 ? "eh_red" + std::to_string(red_i) + " + (threadIdx.x / T) * (T / 64)" : std::string("(" + TA + "*)nullptr"))
+           << ", lr);\n";
         if (st.store)
           os << "  if (lr == 0 && eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "0") << "] = ("
              << T_out << ")" << sname(st.out_buf) << ";\n";

@@ -212,6 +212,31 @@ def mfma_issue_rate(dev, iters=4096, waves_per_cu=8, reps=20):
     return flops / ms / 1e9, blocks, ms
 
 
+EMPTY_SOURCE = """
+extern "C" __global__ void __launch_bounds__(256) eh_empty(float* out) {
+  if (out == nullptr) out[0] = 0.0f;
+}
+"""
+
+
+def launch_floor_us(dev, blocks=256, reps=2000):
+    """Microseconds per launch of a kernel that does nothing (`blocks` workgroups of 256), queued
+    back to back on the device's stream: what one kernel boundary costs whatever the kernel
+    computes -- the floor under any step made of one small grid."""
+    mod = hb.HipModule(dev, hb.compile_source(EMPTY_SOURCE), "eh_empty")
+    out = hb.HipBuffer(dev, [64], None, nbytes=256)
+    for _ in range(50):
+        mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+    dev.sync()
+    e0, e1 = hb.Event(dev), hb.Event(dev)
+    e0.record()
+    for _ in range(reps):
+        mod.launch([blocks, 1, 1], [256, 1, 1], [out], sync=False)
+    e1.record()
+    e1.sync()
+    return e0.elapsed_ms(e1) / reps * 1e3
+
+
 def copy_rate(dev, shape=(4096, 4096), steps=200, warmup=20, nsets=4, options=None):
     """GB/s of a plain fp32 copy of `shape` (read + write), rotating buffer sets: the ceiling a
     memory-bound kernel of that size can reach, and the kernel the traffic counters are scaled by."""
@@ -222,3 +247,72 @@ def copy_rate(dev, shape=(4096, 4096), steps=200, warmup=20, nsets=4, options=No
     sets = make_sets(dev, prog, arg_names, consts, [x], nsets)
     ms, _ = time_steps(dev, prog, sets, steps, warmup)
     return 2 * x.nbytes / (ms * 1e-3) / 1e9, prog.launches[0], ms
+
+
+# ---------------------------------------------------------------------------
+# profiles/traffic.json from rocprofv3 counter runs
+# ---------------------------------------------------------------------------
+
+def _counter_per_dispatch(directory: str, counter: str):
+    """{kernel name: (mean of `counter` per dispatch, dispatches)} from the counter_collection CSV
+    files rocprofv3 --pmc wrote under `directory` (one row per dispatch and counter dimension)."""
+    import csv
+    import glob
+    per = {}
+    for f in glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True):
+        with open(f) as fh:
+            for r in csv.DictReader(fh):
+                if r["Counter_Name"] != counter:
+                    continue
+                d = per.setdefault(r["Kernel_Name"], {})
+                d[r["Dispatch_Id"]] = d.get(r["Dispatch_Id"], 0.0) + float(r["Counter_Value"])
+    return {k: (sum(v.values()) / len(v), len(v)) for k, v in per.items()}
+
+
+def write_traffic_file(root: str, out_path: str = TRAFFIC_FILE):
+    """Builds profiles/traffic.json from `root`/<workload>_{fetch,write} (workloads: copy, softmax,
+    matmul, config1), each the output directory of
+        rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -d <dir> -o pmc --output-format csv -- \
+            python3 bench.py --only <workload> --steps 10 --warmup 2 --no-cpu-baseline --no-per-kernel --no-check
+    FETCH_SIZE / WRITE_SIZE are scaled so that the plain 64 MiB copy kernel reads and writes exactly
+    its 65536 KiB (it is assumed to waste nothing); every entry carries the SHA-1 of the generated
+    source it was measured on, which bench.py compares with the source it times."""
+    from . import workloads as wl
+    copy_ast = wl.lower_with_table([(4096, 4096)], lambda t: t.contiguous())[0]
+    copy_entry = hb.render_program(copy_ast).launches[0]["entry"]
+    cf = _counter_per_dispatch(os.path.join(root, "copy_fetch"), "FETCH_SIZE")[copy_entry][0]
+    cw = _counter_per_dispatch(os.path.join(root, "copy_write"), "WRITE_SIZE")[copy_entry][0]
+    kib = 4096 * 4096 * 4 / 1024
+    rec = {"calibration": {"kernel": f"{copy_entry} (plain copy, {kib:.0f} KiB read + {kib:.0f} KiB written, assumed free of wasted traffic)",
+                           "FETCH_SIZE_reading": round(cf, 1), "WRITE_SIZE_reading": round(cw, 1),
+                           "fetch_factor": round(kib / cf, 4), "write_factor": round(kib / cw, 4)},
+           "kernels": {}}
+    plans = {"softmax": wl.lower_with_table([(4096, 4096)], wl.config2_graph)[0],
+             "matmul": wl.lower_with_table([(4096, 4096)] * 2, wl.config3_graph)[0],
+             "config1": wl.lower_with_table([(1024, 1024)] * 3, wl.config1_graph)[0]}
+    for name, ast in plans.items():
+        fetch = _counter_per_dispatch(os.path.join(root, name + "_fetch"), "FETCH_SIZE")
+        write = _counter_per_dispatch(os.path.join(root, name + "_write"), "WRITE_SIZE")
+        for l in hb.render_program(ast).launches:
+            if l["entry"] not in fetch or l["entry"] not in write:
+                continue
+            rd = fetch[l["entry"]][0] * kib / cf * 1024
+            wr = write[l["entry"]][0] * kib / cw * 1024
+            rec["kernels"][l["entry"]] = {
+                "workload": name, "schedule": l["schedule"], "source_sha1": source_hash(l["source"]),
+                "FETCH_SIZE_reading": round(fetch[l["entry"]][0], 1), "WRITE_SIZE_reading": round(write[l["entry"]][0], 1),
+                "dispatches": [fetch[l["entry"]][1], write[l["entry"]][1]],
+                "read_bytes": int(rd), "written_bytes": int(wr), "traffic_bytes": int(rd + wr),
+                "algorithmic_bytes": int(l["algo_bytes"])}
+    with open(out_path, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    return rec
+
+
+if __name__ == "__main__":
+    import sys
+    if len(sys.argv) == 3 and sys.argv[1] == "traffic":
+        print(json.dumps(write_traffic_file(sys.argv[2]), indent=1))
+    else:
+        sys.exit("usage: python -m harp_amd.measure traffic <directory holding <workload>_fetch and <workload>_write>")

@@ -1331,3 +1331,39 @@ def test_random_graph_gradients_match_the_oracle(frontend, hip, seed):
         # gradient legitimately differs (the function is not differentiable there)
         allowed = 1 if ("(max)" in desc or "(min)" in desc) else 0
         assert int((~close).sum()) <= allowed, desc
+
+
+def test_producers_read_through_another_index_space(frontend, hip):
+    """A squared tensor, permuted, made contiguous and regrouped, feeding a kernel over the new
+    axes: planned as one launch (the producers are evaluated where they are read), as three with
+    reindex=0; both equal the oracle bit for bit (elementwise arithmetic only) and numpy."""
+    from test_host_cpu import _regrouped_chain
+    rng = RNG(77)
+    x = rng.uniform(-2, 2, (8, 6, 4)).astype(np.float32)
+    y = rng.uniform(-2, 2, (4, 12)).astype(np.float32)
+    got, scheds = _run_program(frontend, hip, _regrouped_chain, [x, y])
+    apart, scheds0 = _run_program(frontend, hip, _regrouped_chain, [x, y], "reindex=0")
+    assert len(scheds) == 1 and len(scheds0) == 3
+    ref = realize_on(frontend, "c", _regrouped_chain, [x, y])
+    a = (x * x).transpose(2, 0, 1).reshape(4, 4, 12)
+    want = (a * y[None] + a).ravel()
+    assert np.array_equal(got, apart) and np.array_equal(got, ref)
+    assert np.allclose(got, want, rtol=1e-6)
+
+
+@pytest.mark.parametrize("threads", [16, 32, 64, 128, 256, 512, 1024])
+def test_row_programs_with_every_thread_count(frontend, hip, threads):
+    """Softmax and a fused relu-sum with the threads per row forced to each power of two the
+    schedule takes: one wave or less per row (lane reductions), two waves per row with two rows in
+    a workgroup (each row needs LDS slots of its own), and whole workgroups per row."""
+    from harp_amd import workloads as wl
+    rng = RNG(threads)
+    x = rng.uniform(-4, 4, (96, 2048)).astype(np.float32)
+    got, scheds = _run_program(frontend, hip, wl.config2_graph, [x], f"row_threads={threads}")
+    assert f"row(T={min(threads, 512)}," in scheds[0], scheds
+    e = np.exp(x.astype(np.float64) - x.max(1, keepdims=True))
+    assert np.allclose(got.reshape(x.shape), e / e.sum(1, keepdims=True), rtol=1e-5, atol=1e-12)
+    a, b, c = [rng.uniform(-1, 1, (200, 1024)).astype(np.float32) for _ in range(3)]
+    got, scheds = _run_program(frontend, hip, wl.config1_graph, [a, b, c], f"row_threads={threads}")
+    want = np.maximum(a.astype(np.float64) * b + c, 0).sum(1)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-4)

@@ -592,3 +592,50 @@ def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
     from harp_amd import workloads
     sm = hb.render_program(workloads.lower_with_table([(64, 256)], workloads.config2_graph)[0])
     assert all(l["lane"] == 0 for l in sm.launches)
+
+
+def _regrouped_chain(x, y):
+    """[8,6,4] squared, permuted and made contiguous, its axes regrouped to [4,4,12], then used twice."""
+    a = (x * x).permute([2, 0, 1]).contiguous().reshape([4, 4, 12])
+    return a * y.unsqueeze(0) + a
+
+
+def test_elementwise_producers_are_evaluated_where_another_index_space_reads_them(frontend):
+    """A square, a permuting copy and a regrouping copy in front of the kernel that uses them: as
+    lowered that is three launches through three temps; planned, the consumer's loops are split at
+    the producers' loop boundaries, the producers' expressions take the place of the loads, and one
+    launch reads x directly.  reindex=0 keeps the kernels apart."""
+    from harp_amd import backend as hb, workloads as wl
+    ast = wl.lower_with_table([(8, 6, 4), (4, 12)], _regrouped_chain)[0]
+    plan = hb.render_program(ast)
+    (l,) = plan.launches
+    roles = {b["name"]: b["role"] for b in plan.buffers}
+    assert l["schedule"].startswith("flat(")
+    assert sorted(roles[a] for a in l["args"]) == ["input", "input", "output"], l["args"]
+    assert sum(b["elided"] for b in plan.buffers) == 4
+    src = l["source"]
+    apart = hb.render_program(ast, "reindex=0")
+    assert len(apart.launches) == 3 and sum(b["elided"] for b in apart.buffers) == 2
+    assert len(hb.compile_source(src)) > 1000
+
+
+def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
+    """The input gradient of a 3x3 convolution: `dY x W` writes columns [pixels, channels*9] that
+    nine shifted, guarded reads sum up along the image's rows.  Stored as written, neighbouring
+    lanes of that sum read 288 floats apart; the plan stores the temp transposed (the contraction
+    computes the transposed product), and the guarded reads carry no branch."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config5_inputs(64, *wl.cnn_sizes(True)[1:])
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
+    plan = hb.render_program(ast, "lanes=1")
+    cols = [l for l in plan.launches if l["schedule"].startswith("mfma") and "A:m,B:n/folded" in l["schedule"]]
+    assert len(cols) == 1, [l["schedule"] for l in plan.launches]
+    temp = cols[0]["args"][-1]
+    (reader,) = [l for l in plan.launches if temp in l["args"] and l is not cols[0]]
+    body = reader["source"][reader["source"].index("__global__"):]
+    assert body.count(temp + "[") == 9
+    assert "if (" not in body.replace("if (eh_", "")            # guarded loads: clamped index + select
+    plain = hb.render_program(ast, "lanes=1,reindex=0")
+    assert not any("A:m,B:n/folded" in l["schedule"] for l in plain.launches)
