@@ -369,6 +369,12 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   }
   os << "#define EH_SETPRIO " << std::max(0, std::min(3, opt.gemm_setprio)) << "\n";
   os << "#define EH_MIX " << (opt.gemm_mix ? 1 : 0) << "\n";
+  {
+    // small tiles multiply for a fraction of a load's latency: their loads leave three steps ahead
+    int pf = opt.gemm_prefetch > 0 ? opt.gemm_prefetch : (t.bm * t.bn <= 64 * 64 ? 3 : 1);
+    if (pf > 1 && pf % 2 == 0) ++pf;            // stages = prefetch + 1 must be even
+    os << "#define EH_PREFETCH " << pf << "\n";
+  }
   os << "#define EH_LOAD_BRANCH " << (opt.guard_branches ? 1 : 0) << "\n";
   os << kGemmSource;
   ls.source = os.str();

@@ -67,6 +67,9 @@
 #ifndef EH_LOAD_BRANCH
 #define EH_LOAD_BRANCH 0  // element-by-element tile loads: a branch around each out-of-range element (1) or a clamped index and a select (0)
 #endif
+#ifndef EH_PREFETCH
+#define EH_PREFETCH 1     // how many tile steps ahead of their use the global loads are issued
+#endif
 #ifndef EH_MIX
 #define EH_MIX 1         // LDS operand reads are issued one at a time between the MFMAs of the block before
 #endif
@@ -342,7 +345,12 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   constexpr long long CSM = EH_C_SM, CSN = EH_C_SN;
 #endif
 
-  eh_f4v ra[AV], rb[BV];
+  // Register stages of tiles on their way from global memory to LDS.  One stage: the tile of the
+  // next step.  With EH_PREFETCH = P > 1 there are P + 1 stages and the loads run P steps ahead: a
+  // small tile multiplies for a fraction of a load's latency, and with few workgroups on a CU
+  // nothing else would fill the wait.
+  constexpr int NSTAGE = (EH_PREFETCH > 1 && !(EH_A_DMA || EH_B_DMA)) ? EH_PREFETCH + 1 : 1;
+  eh_f4v ra[NSTAGE][AV], rb[NSTAGE][BV];
   // the rows of each tile this work-item fetches, decoded once (they do not change with k)
   EhRows<EhAElem, EH_A_KCONTIG != 0> a_rows[AV];
   EhRows<EhBElem, EH_B_NCONTIG == 0> b_rows[BV];
@@ -367,7 +375,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gp,
                                      (__attribute__((address_space(3))) void*)(tile + q_wave * 4), 16, 0, 0);
   };
-  auto gload = [&](int kt, float* a_tile, float* b_tile) {
+  auto gload = [&](int kt, float* a_tile, float* b_tile, const int stage) {
     (void)a_tile;
     (void)b_tile;
     const long long k0 = kbeg + (long long)kt * BK;
@@ -379,10 +387,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(A + a_base + (k0 + k) * EH_A_SK + (m0 + mq * 4) * EH_A_SM, a_tile, (tid & ~63) + i * NT);
 #elif EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend, a_rows[i]);
+      ra[stage][i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend, a_rows[i]);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
-      ra[i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend, a_rows[i]);
+      ra[stage][i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend, a_rows[i]);
 #endif
     }
 #pragma unroll
@@ -393,15 +401,15 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       to_lds(B + b_base + (k0 + k) * EH_B_SK + (n0 + nq * 4) * EH_B_SN, b_tile, (tid & ~63) + i * NT);
 #elif EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend, b_rows[i]);
+      rb[stage][i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend, b_rows[i]);
 #else
       const int n = q / (BK / 4), kq = q % (BK / 4);
-      rb[i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + n, k0 + kq * 4, N, kend, b_rows[i]);
+      rb[stage][i] = eh_tile_load<EhBElem, EH_B_VEC, true, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + n, k0 + kq * 4, N, kend, b_rows[i]);
 #endif
     }
   };
 
-  auto sstore = [&](float* a_tile, float* b_tile) {
+  auto sstore = [&](float* a_tile, float* b_tile, const int stage) {
     (void)a_tile;
     (void)b_tile;
 #if !EH_A_DMA
@@ -409,9 +417,9 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
     for (int i = 0; i < AV; ++i) {
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
-      ATile::put(a_tile, q / (BK / 4), (q % (BK / 4)) * 4, ra[i]);
+      ATile::put(a_tile, q / (BK / 4), (q % (BK / 4)) * 4, ra[stage][i]);
 #else
-      ATile::put(a_tile, (q % (BM / 4)) * 4, q / (BM / 4), ra[i]);
+      ATile::put(a_tile, (q % (BM / 4)) * 4, q / (BM / 4), ra[stage][i]);
 #endif
     }
 #endif
@@ -420,9 +428,9 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
     for (int i = 0; i < BV; ++i) {
       const int q = tid + i * NT;
 #if EH_B_NCONTIG
-      BTile::put(b_tile, (q % (BN / 4)) * 4, q / (BN / 4), rb[i]);
+      BTile::put(b_tile, (q % (BN / 4)) * 4, q / (BN / 4), rb[stage][i]);
 #else
-      BTile::put(b_tile, q / (BK / 4), (q % (BK / 4)) * 4, rb[i]);
+      BTile::put(b_tile, q / (BK / 4), (q % (BK / 4)) * 4, rb[stage][i]);
 #endif
     }
 #endif
@@ -439,8 +447,14 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  gload(0, As0, Bs0);
-  sstore(As0, Bs0);
+  gload(0, As0, Bs0, 0);
+  if (NSTAGE > 1) {
+    // the tiles of the first steps leave together
+#pragma unroll
+    for (int t = 1; t < NSTAGE - 1; ++t)
+      if (t < KT) gload(t, As0, Bs0, t);
+  }
+  sstore(As0, Bs0, 0);
   __syncthreads();
 
   // two register slots of operands: block j+1 is fetched while block j is multiplied
@@ -462,9 +476,12 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   };
   // one tile step: multiply the tile in (a_cur, b_cur) while the next one travels to (a_nxt, b_nxt)
   // (`more`: a next tile exists; a literal in the unrolled loop, uniform otherwise)
-  auto step = [&](int kt, float* a_cur, float* b_cur, float* a_nxt, float* b_nxt, const bool more) {
-    if (more) {
-      gload(kt + 1, a_nxt, b_nxt);
+  // (`load_kt`, `load_stage`: the tile whose loads leave in this step and where they land;
+  //  `store_stage`: where the next step's tile has landed)
+  auto step = [&](int kt, float* a_cur, float* b_cur, float* a_nxt, float* b_nxt, const bool more, const bool load,
+                  const int load_kt, const int load_stage, const int store_stage) {
+    if (load) {
+      gload(load_kt, a_nxt, b_nxt, load_stage);
       // keep the global loads up here: their latency is hidden by the whole multiply loop only
       // if they are issued before it (the compiler would otherwise sink them to their use)
       asm volatile("" ::: "memory");
@@ -484,7 +501,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #if EH_SETPRIO
     __builtin_amdgcn_s_setprio(0);
 #endif
-    if (more) sstore(a_nxt, b_nxt);
+    if (more) sstore(a_nxt, b_nxt, store_stage);
     __syncthreads();
     if (more) fetch(a_nxt, b_nxt, 0, NBLK & 1);
     EH_FETCH_FENCE();
@@ -495,23 +512,38 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 
   fetch(As0, Bs0, 0, 0);
 #if !(EH_A_DMA || EH_B_DMA)
-  // one loop body, buffers chosen by the step's parity
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    step(kt, As[buf], Bs[buf], As[buf ^ 1], Bs[buf ^ 1], kt + 1 < KT);
+  if (NSTAGE == 1) {
+    // one loop body, buffers chosen by the step's parity
+    for (int kt = 0; kt < KT; ++kt) {
+      const int buf = kt & 1;
+      step(kt, As[buf], Bs[buf], As[buf ^ 1], Bs[buf ^ 1], kt + 1 < KT, kt + 1 < KT, kt + 1, 0, 0);
+    }
+  } else {
+    // unrolled by the number of stages, so that every stage is a fixed set of registers
+    constexpr int P = NSTAGE - 1;
+    static_assert(NSTAGE == 1 || NSTAGE % 2 == 0, "an even number of stages keeps the LDS buffer's parity fixed per slot");
+    for (int kt0 = 0; kt0 < KT; kt0 += NSTAGE) {
+#pragma unroll
+      for (int u = 0; u < NSTAGE; ++u) {
+        const int kt = kt0 + u;
+        if (kt < KT)
+          step(kt, As[u & 1], Bs[u & 1], As[(u & 1) ^ 1], Bs[(u & 1) ^ 1], kt + 1 < KT, kt + P < KT, kt + P, (u + P) % NSTAGE,
+               (u + 1) % NSTAGE);
+      }
+    }
   }
 #else
   // unrolled by two so that each direct-to-LDS load names its destination array statically
   int kt = 0;
   for (; kt + 2 < KT; kt += 2) {
-    step(kt, As0, Bs0, As1, Bs1, true);
-    step(kt + 1, As1, Bs1, As0, Bs0, true);
+    step(kt, As0, Bs0, As1, Bs1, true, true, kt + 1, 0, 0);
+    step(kt + 1, As1, Bs1, As0, Bs0, true, true, kt + 2, 0, 0);
   }
   if (kt + 2 == KT) {
-    step(kt, As0, Bs0, As1, Bs1, true);
-    step(kt + 1, As1, Bs1, As0, Bs0, false);
+    step(kt, As0, Bs0, As1, Bs1, true, true, kt + 1, 0, 0);
+    step(kt + 1, As1, Bs1, As0, Bs0, false, false, 0, 0, 0);
   } else {
-    step(kt, As0, Bs0, As1, Bs1, false);
+    step(kt, As0, Bs0, As1, Bs1, false, false, 0, 0, 0);
   }
 #endif
 
