@@ -1434,6 +1434,120 @@ std::optional<RowSplit> split_long_rows(const NestKernel& nk) {
 
 
 // ---------------------------------------------------------------------------------------------
+// a value an earlier kernel already stored is read back instead of being computed again
+// ---------------------------------------------------------------------------------------------
+
+// Structural equality of `s` (over S's loop variables) and `r` (over R's) under a one-to-one
+// renaming of loop variables, which is built up in `map` as the trees are walked.
+bool same_under_renaming(const Node& s, const Node& r, const std::set<std::string>& s_vars, const std::set<std::string>& r_vars,
+                         std::map<std::string, std::string>* map) {
+  if (s.op != r.op || s.args.size() != r.args.size()) return false;
+  if (s.op == Op::Var) {
+    const bool sv = s_vars.count(s.name) != 0, rv = r_vars.count(r.name) != 0;
+    if (sv != rv) return false;
+    if (!sv) return s.name == r.name;
+    auto it = map->find(s.name);
+    if (it != map->end()) return it->second == r.name;
+    for (const auto& kv : *map)
+      if (kv.second == r.name) return false;
+    (*map)[s.name] = r.name;
+    return true;
+  }
+  if (s.op == Op::Const) return s.dtype.ty == r.dtype.ty && s.ival == r.ival && std::memcmp(&s.fval, &r.fval, sizeof s.fval) == 0;
+  if (s.name != r.name || s.count != r.count) return false;
+  if ((s.op == Op::Cast || s.op == Op::Load) && s.dtype.ty != r.dtype.ty) return false;
+  for (size_t i = 0; i < s.args.size(); ++i) {
+    if (!s.args[i] || !r.args[i]) return false;
+    if (!same_under_renaming(*s.args[i], *r.args[i], s_vars, r_vars, map)) return false;
+  }
+  return true;
+}
+
+size_t count_loads(const Node& n) {
+  size_t c = n.op == Op::Load ? 1 : 0;
+  for (const auto& a : n.args)
+    if (a) c += count_loads(*a);
+  return c;
+}
+
+// R with every subexpression that equals what S stored (same loop extents under the renaming)
+// replaced by a load of S's output; null when there is none.  Only expressions of two loads or
+// more are taken: the point is to read one buffer instead of several.
+NodePtr reuse_stored_value(const NestKernel& S, const NestKernel& R) {
+  if (S.rkind != ReduceKind::None || !S.out_aff || S.out_buf == R.out_buf) return nullptr;
+  if (count_loads(*S.value) < 2 || infer_ty(*S.value, nullptr) != S.out_dtype.ty) return nullptr;
+  std::set<std::string> s_vars, r_vars;
+  std::map<std::string, int64_t> s_ext, r_ext;
+  for (const auto& l : S.loops) { s_vars.insert(l.var); s_ext[l.var] = l.extent; }
+  for (const auto& l : R.loops) { r_vars.insert(l.var); r_ext[l.var] = l.extent; }
+  if (R.rkind != ReduceKind::None) { r_vars.insert(R.rloop.var); r_ext[R.rloop.var] = R.rloop.extent; }
+  for (const auto& pp : R.params)
+    if (pp.name == S.out_buf && pp.mut_) return nullptr;
+  bool changed = false;
+  std::function<NodePtr(const NodePtr&)> walk = [&](const NodePtr& n) -> NodePtr {
+    std::map<std::string, std::string> m;
+    if (same_under_renaming(*S.value, *n, s_vars, r_vars, &m)) {
+      bool ok = true;
+      std::map<std::string, NodePtr> ren;
+      for (const auto& l : S.loops) {
+        auto it = m.find(l.var);
+        if (it == m.end()) { ok = ok && (l.extent == 1 || S.out_aff->of(l.var) == 0); ren[l.var] = make_i64(0); continue; }
+        ok = ok && r_ext[it->second] == l.extent;
+        ren[l.var] = make_var(it->second);
+      }
+      if (ok) {
+        auto ld = make(Op::Load, {make_var(S.out_buf), rename(S.out_index, ren)});
+        ld->dtype = S.out_dtype;
+        changed = true;
+        return ld;
+      }
+    }
+    bool ch = false;
+    std::vector<NodePtr> args;
+    args.reserve(n->args.size());
+    for (const auto& a : n->args) {
+      NodePtr x = a ? walk(a) : a;
+      ch = ch || x != a;
+      args.push_back(std::move(x));
+    }
+    if (!ch) return n;
+    auto c = std::make_shared<Node>(*n);
+    c->args = std::move(args);
+    return c;
+  };
+  NodePtr value = walk(R.value);
+  if (!changed) return nullptr;
+  NodePtr body = R.rkind == ReduceKind::None ? make(Op::Store, {make_var(R.out_buf), R.out_index, value})
+                                             : make_reduce_block(R, R.rloop.var, R.rloop.extent, value, R.out_buf, R.out_index);
+  for (size_t i = R.loops.size(); i-- > 0;) body = make_range(R.loops[i].var, R.loops[i].extent, body);
+  // parameters: what the new value still reads, then S's output, then R's outputs
+  std::vector<LoadRef> lds;
+  collect_loads(*value, lds);
+  std::set<std::string> read;
+  for (const auto& lr : lds)
+    if (lr.load->args[0]->op == Op::Var) read.insert(lr.load->args[0]->name);
+  std::vector<Param> params;
+  bool have_s = false;
+  for (const auto& pp : R.params) {
+    if (pp.dtype.is_ptr() && !pp.mut_ && !read.count(pp.name)) continue;
+    if (pp.mut_ && !have_s) {
+      bool listed = false;
+      for (const auto& q : params) listed = listed || q.name == S.out_buf;
+      if (!listed) {
+        Param sp;
+        sp.name = S.out_buf;
+        sp.dtype.ty = Ty::Ptr;
+        sp.dtype.inner = std::make_shared<DType>(S.out_dtype);
+        params.push_back(sp);
+      }
+      have_s = true;
+    }
+    params.push_back(pp);
+  }
+  return make_kernel(R.name, params, body);
+}
+
+// ---------------------------------------------------------------------------------------------
 // elementwise producers read through another index space: evaluated where they are read
 // ---------------------------------------------------------------------------------------------
 
@@ -1963,6 +2077,25 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       c->args = {body};
       return c;
     };
+    // phase 0 drops whole-buffer copies; then values that an earlier kernel already stored are
+    // read back where a later kernel computes them again; phase 1 evaluates producers in readers
+    for (int phase = 0; phase < 2; ++phase) {
+    if (phase == 1 && !std::getenv("ECLAT_HIP_NO_REUSE")) {
+      for (size_t si = 0; si < kernels.size(); ++si) {
+        auto ns = extract_nest(*kernels[si]);
+        if (!ns || ns->rkind != ReduceKind::None || writers_of(ns->out_buf) != 1) continue;
+        for (size_t ri = si + 1; ri < kernels.size(); ++ri) {
+          auto nr = extract_nest(*kernels[ri]);
+          if (!nr) continue;
+          NodePtr nk = reuse_stored_value(*ns, *nr);
+          if (!nk) continue;
+          if (std::getenv("ECLAT_HIP_DEBUG_REINDEX"))
+            fprintf(stderr, "reuse: %s reads %s of %s\n", nr->name.c_str(), ns->out_buf.c_str(), ns->name.c_str());
+          rewritten.push_back(nk);
+          kernels[ri] = nk.get();
+        }
+      }
+    }
     for (bool again = true; again;) {
       again = false;
       for (size_t p = 0; p < kernels.size() && !again; ++p) {
@@ -2007,7 +2140,29 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             }
           }
         }
-        if (rd.size() > 3) continue;
+        if (phase == 0 || rd.size() > 3) continue;
+        {
+          // what reads a reduction's result element for element stays with it: it is that
+          // reduction's epilogue, and evaluated elsewhere it would keep the raw result alive for a
+          // reader far away
+          int64_t p_numel = 1;
+          for (const auto& l : np->loops) p_numel *= l.extent;
+          bool after_reduce = false;
+          for (const auto& pp : kernels[p]->params) {
+            if (!pp.dtype.is_ptr() || pp.mut_) continue;
+            for (size_t w = 0; w < p; ++w) {
+              bool writes = false;
+              for (const auto& pw : kernels[w]->params) writes = writes || (pw.dtype.is_ptr() && pw.mut_ && pw.name == pp.name);
+              if (!writes) continue;
+              auto nw = extract_nest(*kernels[w]);
+              int64_t w_numel = 1;
+              if (nw)
+                for (const auto& l : nw->loops) w_numel *= l.extent;
+              after_reduce = after_reduce || !nw || (nw->rkind != ReduceKind::None && w_numel == p_numel);
+            }
+          }
+          if (after_reduce) continue;
+        }
         {
           std::vector<LoadRef> pl;
           collect_loads(*np->value, pl);
@@ -2041,6 +2196,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           kernels.erase(kernels.begin() + static_cast<long>(p));
         }
       }
+    }
     }
   }
   if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
@@ -2463,6 +2619,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             const NestKernel& sk = *nests[j];
             int64_t numel = 0;
             auto strides = dense_strides(sk, &numel);
+            if (std::getenv("ECLAT_HIP_DEBUG_EPI"))
+              fprintf(stderr, "epi %s: stage %s strides %d numel %lld total %lld\n", k0.name.c_str(), sk.name.c_str(), strides ? 1 : 0,
+                      (long long)numel, (long long)total);
             if (!strides || numel != total || avail.count(sk.out_buf)) break;
             std::vector<LoadRef> loads;
             collect_loads(*sk.value, loads);
@@ -2502,6 +2661,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
                 for (size_t r : readers[kv.first]) sole = sole && r > i && r <= j;
               }
               auto na = sole ? relayout(k0, sk, *permuted) : std::nullopt;
+              if (std::getenv("ECLAT_HIP_DEBUG_EPI")) fprintf(stderr, "epi %s: sole %d relayout %d\n", k0.name.c_str(), sole ? 1 : 0, na ? 1 : 0);
               if (!na) break;
               k0r.out_aff = *na;
               if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; break; }

@@ -32,6 +32,7 @@ struct GenOptions {
   int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
   bool reindex = true;                // elementwise producers evaluated in a reader that walks another index space
   bool guard_branches = false;        // guarded loads (padding, edges) behind branches instead of clamped indices and selects
+  bool gemm_transpose = false;        // row-contiguous operands transposed over lane quads into the k-contiguous LDS layout (measured slower)
   int gemm_prefetch = 0;              // tile steps the global loads run ahead (0: 3 for tiles up to 64x64, else 1)
   bool gemm_mix = true;               // LDS operand reads interleaved with the MFMAs of the block before
   bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles

@@ -375,6 +375,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     if (pf > 1 && pf % 2 == 0) ++pf;            // stages = prefetch + 1 must be even
     os << "#define EH_PREFETCH " << pf << "\n";
   }
+  os << "#define EH_TRANSPOSE " << (opt.gemm_transpose ? 1 : 0) << "\n";
   os << "#define EH_LOAD_BRANCH " << (opt.guard_branches ? 1 : 0) << "\n";
   os << kGemmSource;
   ls.source = os.str();

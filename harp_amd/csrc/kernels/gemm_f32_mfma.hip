@@ -67,6 +67,15 @@
 #ifndef EH_LOAD_BRANCH
 #define EH_LOAD_BRANCH 0  // element-by-element tile loads: a branch around each out-of-range element (1) or a clamped index and a select (0)
 #endif
+// A row-contiguous operand read with 128-bit loads is kept in LDS in the k-contiguous layout too
+// ([k/4][row][4], one ds_read_b128 per four MFMAs instead of four scalar reads): the four lanes of
+// a quad load the same four rows at four consecutive k and exchange elements (a 4x4 transpose
+// over the quad, DPP quad permutes) before the store.  Off by default: the exchange costs about
+// thirty vector instructions per 128-bit load, issued through the same port as the MFMAs, which
+// outweighs the cheaper reads (4096^3: 135 against 140 TFLOP/s); EH_TRANSPOSE 0 keeps [k][row].
+#ifndef EH_TRANSPOSE
+#define EH_TRANSPOSE 0
+#endif
 #ifndef EH_PREFETCH
 #define EH_PREFETCH 1     // how many tile steps ahead of their use the global loads are issued
 #endif
@@ -108,6 +117,16 @@ constexpr int NWM = BM / WM, NWN = BN / WN, NT = NWM * NWN * 64;
 #endif
 #ifndef EH_B_DMA
 #define EH_B_DMA 0
+#endif
+#ifdef EH_A_FOLD
+#define EH_A_TR 0
+#else
+#define EH_A_TR (EH_TRANSPOSE && !EH_A_KCONTIG && EH_A_VEC && !EH_A_DMA)
+#endif
+#ifdef EH_B_FOLD
+#define EH_B_TR 0
+#else
+#define EH_B_TR (EH_TRANSPOSE && EH_B_NCONTIG && EH_B_VEC && !EH_B_DMA)
 #endif
 constexpr int AS = BM + (EH_A_DMA ? 0 : 4), BS = BN + (EH_B_DMA ? 0 : 4);   // (padded) rows per k in LDS
 constexpr int AV = BM * BK / 4 / NT, BV = BN * BK / 4 / NT;   // 4-element loads per thread per tile
@@ -273,8 +292,31 @@ struct EhTile {
     return v;
   }
 };
-using ATile = EhTile<EH_A_KCONTIG != 0, AS>;
-using BTile = EhTile<EH_B_NCONTIG == 0, BS>;
+using ATile = EhTile<EH_A_KCONTIG != 0 || EH_A_TR, AS>;
+using BTile = EhTile<EH_B_NCONTIG == 0 || EH_B_TR, BS>;
+
+// 4x4 transpose over the four lanes of a quad: lane t (= lane & 3) passes row t and gets column t.
+// Round s: lane j hands its element j^s to lane j^s, which files it as element j of its result.
+template <int CTRL> __device__ __forceinline__ float eh_quad(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float eh_pick4(const eh_f4v& v, int i) {
+  return i == 0 ? v[0] : i == 1 ? v[1] : i == 2 ? v[2] : v[3];
+}
+__device__ __forceinline__ void eh_file4(eh_f4v& v, int i, float x) {
+  v[0] = i == 0 ? x : v[0];
+  v[1] = i == 1 ? x : v[1];
+  v[2] = i == 2 ? x : v[2];
+  v[3] = i == 3 ? x : v[3];
+}
+__device__ __forceinline__ eh_f4v eh_quad_transpose(const eh_f4v& v, int t) {
+  eh_f4v out = {0.0f, 0.0f, 0.0f, 0.0f};
+  eh_file4(out, t, eh_pick4(v, t));
+  eh_file4(out, t ^ 1, eh_quad<0xB1>(eh_pick4(v, t ^ 1)));   // quad_perm [1,0,3,2]
+  eh_file4(out, t ^ 2, eh_quad<0x4E>(eh_pick4(v, t ^ 2)));   // quad_perm [2,3,0,1]
+  eh_file4(out, t ^ 3, eh_quad<0x1B>(eh_pick4(v, t ^ 3)));   // quad_perm [3,2,1,0]
+  return out;
+}
 }  // namespace
 
 // Epilogue: elementwise kernels that follow the contraction over the same dense index space
@@ -388,6 +430,10 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #elif EH_A_KCONTIG
       const int m = q / (BK / 4), kq = q % (BK / 4);
       ra[stage][i] = eh_tile_load<EhAElem, EH_A_VEC, true, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + m, k0 + kq * 4, M, kend, a_rows[i]);
+#elif EH_A_TR
+      // quad = four consecutive k of the same four rows
+      const int k = ((q >> 2) / (BM / 4)) * 4 + (q & 3), mq = (q >> 2) % (BM / 4);
+      ra[stage][i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend, a_rows[i]);
 #else
       const int k = q / (BM / 4), mq = q % (BM / 4);
       ra[stage][i] = eh_tile_load<EhAElem, EH_A_VEC, false, EDGE_M, EH_A_SM, EH_A_SK>(A, a_base, bz, m0 + mq * 4, k0 + k, M, kend, a_rows[i]);
@@ -399,6 +445,9 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #if EH_B_DMA
       const int k = q / (BN / 4), nq = q % (BN / 4);
       to_lds(B + b_base + (k0 + k) * EH_B_SK + (n0 + nq * 4) * EH_B_SN, b_tile, (tid & ~63) + i * NT);
+#elif EH_B_TR
+      const int k = ((q >> 2) / (BN / 4)) * 4 + (q & 3), nq = (q >> 2) % (BN / 4);
+      rb[stage][i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend, b_rows[i]);
 #elif EH_B_NCONTIG
       const int k = q / (BN / 4), nq = q % (BN / 4);
       rb[stage][i] = eh_tile_load<EhBElem, EH_B_VEC, false, EDGE_N, EH_B_SN, EH_B_SK>(B, b_base, bz, n0 + nq * 4, k0 + k, N, kend, b_rows[i]);
@@ -418,6 +467,8 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
       const int q = tid + i * NT;
 #if EH_A_KCONTIG
       ATile::put(a_tile, q / (BK / 4), (q % (BK / 4)) * 4, ra[stage][i]);
+#elif EH_A_TR
+      ATile::put(a_tile, ((q >> 2) % (BM / 4)) * 4 + (q & 3), ((q >> 2) / (BM / 4)) * 4, eh_quad_transpose(ra[stage][i], q & 3));
 #else
       ATile::put(a_tile, (q % (BM / 4)) * 4, q / (BM / 4), ra[stage][i]);
 #endif
@@ -427,7 +478,9 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #pragma unroll
     for (int i = 0; i < BV; ++i) {
       const int q = tid + i * NT;
-#if EH_B_NCONTIG
+#if EH_B_TR
+      BTile::put(b_tile, ((q >> 2) % (BN / 4)) * 4 + (q & 3), ((q >> 2) / (BN / 4)) * 4, eh_quad_transpose(rb[stage][i], q & 3));
+#elif EH_B_NCONTIG
       BTile::put(b_tile, (q % (BN / 4)) * 4, q / (BN / 4), rb[stage][i]);
 #else
       BTile::put(b_tile, q / (BK / 4), (q % (BK / 4)) * 4, rb[stage][i]);

@@ -817,6 +817,9 @@ CONTRACTIONS = [
     ("matmul", [(256, 64), (64, 128)], {"gemm_dma": 1}, "B>lds"),
     ("per_group", [(3, 64, 64), (3, 64, 128)], {"gemm_dma": 1}, "A>lds,B>lds"),
     ("matmul", [(192, 160), (160, 320)], {"gemm_bm": 128, "gemm_bn": 128, "gemm_bk": 16, "gemm_wm": 64, "gemm_wn": 64}, "tile=128x128x16"),
+    ("matmul", [(192, 160), (160, 320)], {"gemm_transpose": 1}, "mfma"),
+    ("per_group", [(3, 64, 64), (3, 64, 128)], {"gemm_transpose": 1, "gemm_prefetch": 1}, "mfma"),
+    ("matmul", [(256, 512), (512, 256)], {"gemm_prefetch": 3, "gemm_bm": 128, "gemm_bn": 128, "gemm_bk": 16, "gemm_wm": 64, "gemm_wn": 64}, "tile=128x128x16"),
     ("linear", [(130, 72), (50, 72)], None, "edges"),
     ("linear", [(33, 18), (7, 18)], None, "/scalar"),
     ("rows3d", [(6, 50, 36), (20, 36)], None, "mfma"),
