@@ -1370,3 +1370,26 @@ def test_row_programs_with_every_thread_count(frontend, hip, threads):
     got, scheds = _run_program(frontend, hip, wl.config1_graph, [a, b, c], f"row_threads={threads}")
     want = np.maximum(a.astype(np.float64) * b + c, 0).sum(1)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-4)
+
+
+def test_stored_value_read_back_by_a_later_reduction(frontend, hip):
+    """The elementwise root and the row sums of the same expression (tests/test_host_cpu.py): with
+    the stored value read back and with reindex=0, both against numpy."""
+    from harp_amd import measure
+    from harp_amd import workloads as wl
+    from harp_amd.frontend import Tensor
+    from test_host_cpu import _value_and_its_row_sums
+    rng = RNG(5)
+    x = rng.uniform(-1, 1, (64, 256)).astype(np.float32)
+    m = rng.uniform(-1, 1, (64, 256)).astype(np.float32)
+    dev = hip.HipDevice(0)
+    ts = [Tensor.input([64, 256]), Tensor.input([64, 256])]
+    ast, arg_names, outs, consts, _ = wl.lower_multi(ts, _value_and_its_row_sums(*ts))
+    want = [(x * m + x).ravel(), (x.astype(np.float64) * m + x).sum(1)]
+    for options in (None, "reindex=0"):
+        prog = hip.HipProgram(dev, ast, options)
+        (binding, named), = measure.make_sets(dev, prog, arg_names, consts, [x, m], 1)
+        prog.run(binding, sync=True)
+        got = [named[o].read_array(np.float32) for o in outs]
+        assert np.array_equal(got[0], want[0])
+        assert np.allclose(got[1], want[1], rtol=1e-5, atol=1e-5)

@@ -639,3 +639,24 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert "if (" not in body.replace("if (eh_", "")            # guarded loads: clamped index + select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
     assert not any("A:m,B:n/folded" in l["schedule"] for l in plain.launches)
+
+
+def _value_and_its_row_sums(x, m):
+    """x*m + x as one root and the row sums of the same expression, written out again, as another."""
+    return [x * m + x, (x * m + x).sum(1)]
+
+
+def test_a_stored_value_is_read_back_instead_of_computed_again(frontend):
+    """Two roots: an elementwise result and a reduction over the same expression built a second
+    time (as a training step's bias gradient repeats the masked gradient its weight gradient
+    reads).  The second product is not lowered into a kernel of its own: the reduction takes what
+    the first root's kernels hold.  reindex=0 plans all four lowered kernels."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    ts = [Tensor.input([64, 256]), Tensor.input([64, 256])]
+    ast = wl.lower_multi(ts, _value_and_its_row_sums(*ts))[0]
+    kernels = lambda plan: [k for l in plan.launches for k in l["kernels"]]
+    assert len(kernels(hb.render_program(ast, "reindex=0"))) == 4
+    plan = hb.render_program(ast)
+    assert len(kernels(plan)) == 3 and len(plan.launches) == 1
+    assert len(hb.compile_source(plan.launches[0]["source"])) > 1000
