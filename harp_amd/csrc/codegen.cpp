@@ -1238,9 +1238,12 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   for (size_t i = 0; i < k.loops.size(); ++i) f.loops.push_back({k.loops[i].var, k.loops[i].extent, strides[i]});
   ExprRenderer er;
   f.expr = er.expr(*k.value);
-  if (auto a = affine_of(*loads[0].load->args[1]))
+  if (auto a = affine_of(*loads[0].load->args[1])) {
     for (size_t i = 0; i < k.loops.size(); ++i)
       if (k.loops[i].extent > 1) f.src_stride[strides[i]] = a->of(k.loops[i].var);
+    f.plain = k.value->op == Op::Load && loads.size() == 1;
+    f.src_off = a->c;
+  }
   return f;
 }
 
@@ -2480,6 +2483,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
         f->src = fi->src;
         f->src_bytes = fi->src_bytes;
         f->src_stride.clear();
+        f->plain = false;
         folded_kernels.insert(q);
         plan.elided.insert(inner.out_buf);
         break;

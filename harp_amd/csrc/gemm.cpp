@@ -232,6 +232,59 @@ bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
   return s && choose(*s, opt, &c);
 }
 
+namespace {
+
+// A computed operand whose producer only copies through a view (one unguarded load at an affine
+// index) is, where the contraction's axes line up with the producer's loops, an ordinary strided
+// operand in the producer's source: offset and strides of (batch, row, k) there, so that it is
+// read with the plain (possibly 128-bit) loads instead of an element function.  Each axis must
+// cover exactly a run of the producer's loops (no carry into other digits), the runs must not
+// overlap, the offset must not reach into them, and along each axis the source address must be
+// linear (checked over the whole axis).
+struct PlainOperand {
+  int64_t off, bs, sr, sk;
+};
+std::optional<PlainOperand> plain_operand(const FoldedOperand& f, int64_t off, int64_t bs, int64_t sr, int64_t sk, int64_t batch,
+                                          int64_t rows, int64_t kext) {
+  if (!f.plain) return std::nullopt;
+  auto address = [&](int64_t i) {
+    int64_t a = f.src_off;
+    for (const auto& l : f.loops) {
+      if (l.extent <= 1) continue;
+      auto it = f.src_stride.find(l.stride);
+      a += ((i / l.stride) % l.extent) * (it == f.src_stride.end() ? 0 : it->second);
+    }
+    return a;
+  };
+  struct Axis { int64_t s, e, sigma; };
+  Axis axes[3] = {{bs, batch, 0}, {sr, rows, 0}, {sk, kext, 0}};
+  std::vector<std::pair<int64_t, int64_t>> spans;      // [s, s*e) of every moving axis
+  for (auto& ax : axes) {
+    if (ax.e <= 1) continue;
+    if (ax.s <= 0) return std::nullopt;
+    int64_t lo = 0, prod = 1;
+    for (const auto& l : f.loops) {
+      if (l.extent <= 1 || l.stride < ax.s || l.stride >= ax.s * ax.e) continue;
+      if (l.stride * l.extent > ax.s * ax.e) return std::nullopt;
+      lo = lo == 0 ? l.stride : std::min(lo, l.stride);
+      prod *= l.extent;
+    }
+    if (lo != ax.s || prod != ax.e) return std::nullopt;
+    if ((off / ax.s) % ax.e != 0) return std::nullopt;
+    for (const auto& sp : spans)
+      if (ax.s < sp.second && sp.first < ax.s * ax.e) return std::nullopt;
+    spans.push_back({ax.s, ax.s * ax.e});
+    ax.sigma = address(off + ax.s) - address(off);
+    for (int64_t j = 0; j < ax.e; ++j)
+      if (address(off + j * ax.s) - address(off) != j * ax.sigma) return std::nullopt;
+  }
+  PlainOperand p{address(off), axes[0].sigma, axes[1].sigma, axes[2].sigma};
+  if (p.off < 0 || p.sr < 0 || p.sk < 0 || p.bs < 0) return std::nullopt;
+  return p;
+}
+
+}  // namespace
+
 std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt, std::vector<BufferInfo>* buffers,
                                       const FoldMap* folded, const EpilogueSpec* epilogue) {
   auto s = match_gemm(k);
@@ -244,6 +297,19 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     if (ia != folded->end()) fa = &ia->second;
     if (ib != folded->end()) fb = &ib->second;
   }
+  std::string plain_tag;
+  if (fa)
+    if (auto p = plain_operand(*fa, s->a_off, s->a_b, s->a_m, s->a_k, s->batch, s->M, s->K)) {
+      s->a_buf = fa->src; s->a_off = p->off; s->a_b = p->bs; s->a_m = p->sr; s->a_k = p->sk;
+      fa = nullptr;
+      plain_tag += ",A:source";
+    }
+  if (fb)
+    if (auto p = plain_operand(*fb, s->b_off, s->b_b, s->b_n, s->b_k, s->batch, s->N, s->K)) {
+      s->b_buf = fb->src; s->b_off = p->off; s->b_b = p->bs; s->b_n = p->sr; s->b_k = p->sk;
+      fb = nullptr;
+      plain_tag += ",B:source";
+    }
   if (!choose(*s, opt, &ch, fa || fb)) return {};
   const Tile& t = ch.tile;
   // each thread fetches four elements along the operand's faster axis
@@ -384,7 +450,7 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
                 (fa ? "/folded" : a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") +
                 (fb ? "/folded" : b_vec ? "" : "/scalar") +
-                dma_tag + (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
+                plain_tag + dma_tag + (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
                 (epi_here ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
   ls.grid[1] = static_cast<unsigned>(S);

@@ -43,6 +43,8 @@ struct FoldedOperand {
   // loop stride in the producer's output -> that loop's stride in the source (only when the
   // source index is affine); tells which operand axis is contiguous in the memory actually read
   std::map<int64_t, int64_t> src_stride;
+  bool plain = false;           // the producer is one unguarded load at an affine index (a copy through a view)
+  int64_t src_off = 0;          // constant term of that index
 };
 using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer
 
