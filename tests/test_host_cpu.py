@@ -639,6 +639,10 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert "if (" not in body.replace("if (eh_", "")            # guarded loads: clamped index + select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
     assert not any("A:m,B:n/folded" in l["schedule"] for l in plain.launches)
+    # the weight gradients' dY operand is a copy through a view (NCHW read as [image, pixel, channel]):
+    # read from its source with strides, not through an element function
+    direct = [l for l in plan.launches if "A:source" in l["schedule"]]
+    assert len(direct) == 2 and all("A:k,B:n/folded" in l["schedule"] for l in direct), [l["schedule"] for l in plan.launches]
 
 
 def _value_and_its_row_sums(x, m):
