@@ -73,6 +73,7 @@ _SIGS = {
     "eh_plan_launch": ([_P, c_int, POINTER(LaunchInfo)], c_int),
     "eh_plan_launch_arg": ([_P, c_int, c_int, POINTER(c_char_p)], c_int),
     "eh_plan_launch_kernel": ([_P, c_int, c_int, POINTER(c_char_p)], c_int),
+    "eh_tune_key": ([c_char_p, POINTER(ctypes.c_ulonglong)], c_int),
     "eh_plan_launch_arg_written": ([_P, c_int, c_int, POINTER(c_int)], c_int),
     "eh_plan_launch_wait": ([_P, c_int, c_int, POINTER(c_int)], c_int),
     "eh_plan_num_buffers": ([_P, POINTER(c_int)], c_int),

@@ -94,6 +94,13 @@ def normalize_ast(ast) -> str:
         lib.eh_free(out)
 
 
+def tune_key(ast) -> str:
+    """The 16 hex digits under which the file named by ECLAT_HIP_TUNE holds this program's options."""
+    k = ctypes.c_ulonglong()
+    check(lib.eh_tune_key(_sexpr(ast), byref(k)))
+    return f"{k.value:016x}"
+
+
 def compile_source(source: str, arch: str = "gfx950") -> bytes:
     """hiprtc: HIP C -> code object.  Works without a GPU."""
     blob, n = c_void_p(), c_size_t()

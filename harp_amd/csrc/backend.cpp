@@ -397,6 +397,34 @@ void HipKernel::launch(const unsigned grid[3], const unsigned block[3], unsigned
 // HipProgram
 // ---------------------------------------------------------------------------------------------
 
+unsigned long long tune_key(const char* ast_text) {
+  unsigned long long h = 1469598103934665603ull;
+  for (const unsigned char* p = reinterpret_cast<const unsigned char*>(ast_text); *p; ++p) {
+    h ^= *p;
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+GenOptions options_for(const char* ast_text, const char* options) {
+  const char* path = std::getenv("ECLAT_HIP_TUNE");
+  if (!path || !*path || !ast_text) return parse_options(options);
+  char key[17];
+  std::snprintf(key, sizeof key, "%016llx", tune_key(ast_text));
+  std::ifstream f(path);
+  std::string line, tuned;
+  while (std::getline(f, line)) {
+    const size_t hash = line.find('#');
+    if (hash != std::string::npos) line.resize(hash);
+    std::istringstream ls(line);
+    std::string k, v;
+    if (ls >> k >> v && k == key) tuned = v;          // the last entry for a key counts
+  }
+  if (tuned.empty()) return parse_options(options);
+  const std::string both = options && *options ? tuned + "," + options : tuned;
+  return parse_options(both.c_str());
+}
+
 GenOptions parse_options(const char* text) {
   GenOptions o;
   if (const char* env = std::getenv("ECLAT_HIP_ARCH")) o.arch = env;

@@ -208,6 +208,12 @@ class HipGraph {
 };
 
 GenOptions parse_options(const char* text);       // "key=value,key=value" -> GenOptions
+// Key under which a program's tuned options are filed: FNV-1a (64 bit) of its AST text.
+unsigned long long tune_key(const char* ast_text);
+// Options for compiling `ast_text`: what the file named by ECLAT_HIP_TUNE holds for this program
+// (lines "<16 hex digits of the key> <key=value,...>"; '#' starts a comment), then `options` on
+// top.  Without the variable, or without an entry, just `options`.
+GenOptions options_for(const char* ast_text, const char* options);
 
 // With ECLAT_HIP_DUMP=<dir> in the environment, writes every launch of a plan there:
 // <entry>.hip (the translation unit handed to hiprtc) and <entry>.txt (schedule, grid, block,

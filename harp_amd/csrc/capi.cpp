@@ -211,10 +211,16 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr) {
   return EH_OK;
 }
 
+int eh_tune_key(const char* ast_text, unsigned long long* key) {
+  REQUIRE(ast_text && key, "ast_text or key is NULL");
+  *key = tune_key(ast_text);
+  return EH_OK;
+}
+
 int eh_render_program(const char* ast_text, const char* options, eh_plan** out) {
   REQUIRE(ast_text && out, "ast_text or out is NULL");
   return guard([&] {
-    GenOptions o = parse_options(options);
+    GenOptions o = options_for(ast_text, options);
     NodePtr ast = parse_ast(ast_text);
     if (ast->op == Op::Kernel) ast = make(Op::Program, {ast});
     auto* p = new eh_plan;
@@ -333,7 +339,7 @@ int eh_compile_source(const char* source, const char* arch, void** blob, size_t*
 int eh_program_compile(eh_device* dev, const char* ast_text, const char* options, eh_program** out) {
   REQUIRE(dev && ast_text && out, "device, ast_text or out is NULL");
   return guard([&] {
-    GenOptions o = parse_options(options);
+    GenOptions o = options_for(ast_text, options);
     *out = new eh_program(&dev->dev, ast_text, o);
   });
 }

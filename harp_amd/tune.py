@@ -12,9 +12,12 @@ threads and elements per row; block size, vectors per thread, streaming stores),
 states by running them: event-timed launches of the compiled Program on the GPU.
 
     python -m harp_amd.tune --config config3_matmul [--beam 3] [--steps 4]
-    python -m harp_amd.tune --config config5_cnn_step
+    python -m harp_amd.tune --config config5_cnn_step --save tuned.txt
 
-prints the best options as the "key=value,..." string `eh_program_compile` takes.
+prints the best options as the "key=value,..." string `eh_program_compile` takes.  With `--save`
+the result is also filed under the program's key (`backend.tune_key`) in the given file; a process
+that runs with ECLAT_HIP_TUNE=<that file> then compiles this program with these options (explicit
+options still win), as the reference's optimiser applies what its search found.
 """
 
 from __future__ import annotations
@@ -104,7 +107,32 @@ def suggest_streaming(state: Dict[str, int], schedules: Sequence[str]) -> Iterab
             yield {**state, "nontemporal": nt}
 
 
-SUGGESTERS: List[Callable] = [suggest_gemm, suggest_row, suggest_flat, suggest_streaming]
+def suggest_pipeline(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """How far ahead of their use a contraction's tiles are loaded (register stages), whether they
+    go through registers or straight into LDS, and how many streams a program's independent
+    launches are spread over: the register, LDS and queue budgets of a plan."""
+    if any(s.startswith("mfma") for s in schedules):
+        for p in (1, 3, 5):
+            if p != state.get("gemm_prefetch", 0):
+                yield {**state, "gemm_prefetch": p}
+        for d in (0, 1):
+            if d != state.get("gemm_dma", 0):
+                yield {**state, "gemm_dma": d}
+    if len(schedules) >= 8:
+        for n in (1, 2, 3):
+            if n != state.get("lanes", 2):
+                yield {**state, "lanes": n}
+
+
+SUGGESTERS: List[Callable] = [suggest_gemm, suggest_row, suggest_flat, suggest_streaming, suggest_pipeline]
+
+
+def save_tuned(path: str, key: str, options: str, note: str = "") -> None:
+    """Appends "<key> <options>  # note" to `path` (the last line for a key counts)."""
+    if not options:
+        options = "fuse=1"                    # an entry that changes nothing still records the search
+    with open(path, "a") as f:
+        f.write(f"{key} {options}" + (f"  # {note}" if note else "") + "\n")
 
 
 # -- the search --------------------------------------------------------------------------------
@@ -118,6 +146,7 @@ class MeasuredEstimator:
         self.arg_names, self.consts, self.arrays = arg_names, consts, arrays
         self.steps, self.warmup, self.nsets = steps, warmup, sets
         self.cache: Dict[Options, float] = {}
+        self.key = hb.tune_key(prog_ast)
 
     def schedules(self, opts: Options) -> List[str]:
         return [l["schedule"] for l in hb.render_program(self.ast, dict(opts) or None).launches]
@@ -173,7 +202,7 @@ def beam_search(estimator, start: Optional[Dict[str, int]] = None, beam_width: i
     return best, best_cost, history
 
 
-def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None):
+def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None, save=None):
     """Searches the options of one benchmark configuration on device 0: one of
     `workloads.CONFIGS`, or a whole training step (`config4_mlp_step`, `config5_cnn_step`),
     where one option set serves every launch of the step."""
@@ -187,7 +216,7 @@ def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log
         roots = wl.config4_graph(*ts) if mlp else wl.config5_graph(*ts, lr=1e-2)
         prog_ast, arg_names, _outs, consts, _ = wl.lower_multi(ts, roots)
         est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps, sets=1)
-        return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
+        return _search_and_file(est, name, beam_width, max_steps, log, save)
     default_shapes = {"config1_relu_sum": [(1024, 1024)] * 3, "config2_softmax": [(4096, 4096)],
                       "config3_matmul": [(4096, 4096)] * 2}
     shapes = shapes or default_shapes[name]
@@ -196,7 +225,14 @@ def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log
     arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
     prog_ast, arg_names, _out, consts, _ = wl.lower_with_table(shapes, graph_fn)
     est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps)
-    return beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
+    return _search_and_file(est, name, beam_width, max_steps, log, save)
+
+
+def _search_and_file(est, name, beam_width, max_steps, log, save):
+    best, cost, history = beam_search(est, beam_width=beam_width, max_steps=max_steps, log=log)
+    if save:
+        save_tuned(save, est.key, options_string(best), f"{name}: {cost:.4f} ms (defaults {history[0][2]:.4f} ms)")
+    return best, cost, history
 
 
 def main(argv=None) -> int:
@@ -205,11 +241,13 @@ def main(argv=None) -> int:
     ap.add_argument("--beam", type=int, default=3)
     ap.add_argument("--steps", type=int, default=4, help="search steps (beam expansions)")
     ap.add_argument("--launches", type=int, default=20, help="timed launches per state")
+    ap.add_argument("--save", default=None, help="file to append the result to (read back through ECLAT_HIP_TUNE)")
     args = ap.parse_args(argv)
     if hb.device_count() == 0:
         sys.exit("tune: no HIP device present")
     best, cost, history = tune_config(args.config, beam_width=args.beam, max_steps=args.steps,
-                                      steps=args.launches, log=lambda m: print(m, file=sys.stderr, flush=True))
+                                      steps=args.launches, log=lambda m: print(m, file=sys.stderr, flush=True),
+                                      save=args.save)
     print(json.dumps({"config": args.config, "options": options_string(best), "ms": cost,
                       "default_ms": history[0][2], "states_measured": len(history)}))
     return 0

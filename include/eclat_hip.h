@@ -113,6 +113,14 @@ typedef struct eh_launch_info {
 } eh_launch_info;
 
 int eh_render_program(const char* ast_text, const char* options, eh_plan** out);
+/* Tuned options.  When the environment variable ECLAT_HIP_TUNE names a file, eh_render_program and
+ * eh_program_compile look the program up in it and take the options filed there, with `options` on
+ * top: one line per program, "<key as 16 hex digits> <key=value,...>", '#' starts a comment, the
+ * last line for a key counts.  The key is what eh_tune_key returns for the program's AST text; the
+ * measured schedule search (python -m harp_amd.tune --save <file>) writes such lines.  It stands
+ * where the reference's optimiser picks its rewrites by a static cost
+ * (src/opt/ast/optimizer/beam_search.rs:34-66): here the choice is measured once and filed. */
+int eh_tune_key(const char* ast_text, unsigned long long* key);
 /* The program (or kernel) with the rewrites of the reference's AST optimiser undone where they are
  * recognised -- what eh_render_program and eh_program_compile plan from.  That optimiser runs
  * before any backend sees a kernel (pipeline.optimize, src/backend/executor.rs:169-176,
@@ -169,10 +177,9 @@ int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, in
  * every other buffer that reaches memory (inputs, outputs and the caller's own temps) must be
  * given.  A program whose scratch temps do not fit fails with EH_ERR_SIZE and launches nothing.
  * All calls on one device share that device's block, which keeps the previous call's contents
- * (no kernel relies on them: every scratch element is written before it is read), so calls that
- * overlap on one device race: queue them on the device's stream one after the other, as this
- * library does, and do not run two host threads through this entry point on one device at once
- * with sync == 0 on different programs unless both finish in stream order. */
+ * (no kernel relies on them: every scratch element is written before it is read).  Calls that
+ * overlap on one device would race on it; calls made through this library do not overlap, because
+ * every call's launches are ordered on the device's stream behind those of the call before. */
 #define EH_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
 int eh_program_execute_static(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 /* The launches of one eh_program_execute(prog, bufs, n_bufs, .) captured as a HIP graph of kernel

@@ -899,13 +899,22 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
         assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
 
 
-def test_measured_option_search(frontend, hip):
+def test_measured_option_search(frontend, hip, tmp_path, monkeypatch):
     """One expansion of the beam search on a 512^3 matmul: every proposed state compiles or is
-    rejected cleanly, the winner is no slower than the defaults, and it computes the same C."""
+    rejected cleanly, the winner is no slower than the defaults, and it computes the same C.  The
+    result is filed, and a compile under ECLAT_HIP_TUNE plans the program with it."""
     from harp_amd import tune
+    from harp_amd import workloads as wl
     msgs = []
+    saved = tmp_path / "tuned.txt"
     best, cost, history = tune.tune_config("config3_matmul", shapes=[(512, 512), (512, 512)],
-                                           beam_width=2, max_steps=1, steps=10, log=msgs.append)
+                                           beam_width=2, max_steps=1, steps=10, log=msgs.append, save=str(saved))
+    ast = wl.lower_with_table([(512, 512), (512, 512)], wl.config3_graph)[0]
+    assert saved.read_text().startswith(hip.tune_key(ast) + " ")
+    monkeypatch.setenv("ECLAT_HIP_TUNE", str(saved))
+    filed = [l["schedule"] for l in hip.render_program(ast).launches]
+    monkeypatch.delenv("ECLAT_HIP_TUNE")
+    assert filed == [l["schedule"] for l in hip.render_program(ast, dict(best) or None).launches]
     assert len(history) > 5 and history[0][1] == ""
     assert cost <= history[0][2] * 1.02 and np.isfinite(cost)
     rng = RNG(5)

@@ -664,3 +664,29 @@ def test_a_stored_value_is_read_back_instead_of_computed_again(frontend):
     plan = hb.render_program(ast)
     assert len(kernels(plan)) == 3 and len(plan.launches) == 1
     assert len(hb.compile_source(plan.launches[0]["source"])) > 1000
+
+
+def test_tuned_options_are_filed_and_applied(frontend, tmp_path, monkeypatch):
+    """What the measured search found is kept: a line "<key> <options>" in the file that
+    ECLAT_HIP_TUNE names makes every later compile of that program take those options; explicit
+    options still win, other programs and a missing file change nothing."""
+    from harp_amd import backend as hb, tune, workloads as wl
+    softmax = wl.lower_with_table([(64, 2048)], wl.config2_graph)[0]
+    other = wl.lower_with_table([(32, 2048)], wl.config2_graph)[0]
+    key = hb.tune_key(softmax)
+    assert len(key) == 16 and key != hb.tune_key(other) and key == hb.tune_key(softmax)
+    sched = lambda ast, o=None: hb.render_program(ast, o).launches[0]["schedule"]
+    default = sched(softmax)
+    assert "row(T=256," in default
+    path = tmp_path / "tuned.txt"
+    monkeypatch.setenv("ECLAT_HIP_TUNE", str(path))
+    assert sched(softmax) == default                                   # no file yet
+    tune.save_tuned(str(path), key, "row_threads=64", "an older result")
+    tune.save_tuned(str(path), key, "row_threads=512,nontemporal=1", "softmax 64x2048")
+    path.write_text("# tuned on MI355X\n" + path.read_text())
+    assert "row(T=512," in sched(softmax) and "nt-store" in sched(softmax)
+    assert "row(T=128," in sched(softmax, "row_threads=128") and "nt-store" in sched(softmax, "row_threads=128")
+    assert "row(T=256," in sched(other)
+    monkeypatch.delenv("ECLAT_HIP_TUNE")
+    assert sched(softmax) == default
+    assert {"gemm_prefetch", "gemm_dma", "lanes"} <= {k for st in tune.suggest_pipeline({}, ["mfma32x32x2(...)"] * 8) for k in st}
