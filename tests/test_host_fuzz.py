@@ -36,9 +36,18 @@ def _corpus(fe):
             out.append(AstNode.program([k]).to_sexpr())
             for tf in (["tile=3"], ["guard=5", "unroll"], ["tile_all=2", "unroll"], ["interchange"]):
                 out.append(optimize.optimize_kernel(k, tf).to_sexpr())
+    # whole training steps (exact mode): many kernels behind one buffer table, which is what the
+    # program-level passes work on (producers inlined through re-indexing, stored values read
+    # back, transposed temps, epilogues, lanes)
+    from harp_amd.frontend import Tensor
+    steps = []
+    for arrays, fn in ((wl.config5_inputs(2, 8, 4, 4, 8, 10), lambda *t: wl.config5_graph(*t, lr=1e-2)),
+                       (wl.config4_inputs(8, [16, 32, 32, 16]), lambda *t: wl.config4_graph(*t, lr=1e-3))):
+        ts = [Tensor.input(list(a.shape)) for a in arrays]
+        steps.append(wl.lower_multi(ts, fn(*ts))[0].to_sexpr())
     # the reference's search drops candidates above 10 000 nodes (src/opt/ast/optimizer/beam_search.rs:67):
     # texts beyond that (a convolution unrolled at every level) are left out
-    return [o for o in out if len(o) < 100_000]
+    return [o for o in out if len(o) < 100_000] + steps
 
 
 def test_reader_normaliser_and_planner_survive_mutated_asts_under_sanitizers(frontend, tmp_path):
