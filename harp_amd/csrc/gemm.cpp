@@ -241,8 +241,15 @@ namespace {
 // cover exactly a run of the producer's loops (no carry into other digits), the runs must not
 // overlap, the offset must not reach into them, and along each axis the source address must be
 // linear (checked over the whole axis).
+// offset of the last row of an axis of `rows` rows (stride sr, or two nested extents)
+int64_t row_reach(int64_t rows, int64_t sr, int64_t split, int64_t sr2) {
+  if (!split) return (rows - 1) * sr;
+  return (rows / split - 1) * sr2 + (split - 1) * sr;
+}
+
 struct PlainOperand {
   int64_t off, bs, sr, sk;
+  int64_t rsplit = 0, sr2 = 0;      // the row axis in two nested extents: rows per inner extent, outer stride
 };
 std::optional<PlainOperand> plain_operand(const FoldedOperand& f, int64_t off, int64_t bs, int64_t sr, int64_t sk, int64_t batch,
                                           int64_t rows, int64_t kext) {
@@ -258,6 +265,7 @@ std::optional<PlainOperand> plain_operand(const FoldedOperand& f, int64_t off, i
   };
   struct Axis { int64_t s, e, sigma; };
   Axis axes[3] = {{bs, batch, 0}, {sr, rows, 0}, {sk, kext, 0}};
+  int64_t rsplit = 0, sr2 = 0;
   std::vector<std::pair<int64_t, int64_t>> spans;      // [s, s*e) of every moving axis
   for (auto& ax : axes) {
     if (ax.e <= 1) continue;
@@ -275,11 +283,20 @@ std::optional<PlainOperand> plain_operand(const FoldedOperand& f, int64_t off, i
       if (ax.s < sp.second && sp.first < ax.s * ax.e) return std::nullopt;
     spans.push_back({ax.s, ax.s * ax.e});
     ax.sigma = address(off + ax.s) - address(off);
+    int64_t first_bad = 0;
+    for (int64_t j = 0; j < ax.e && !first_bad; ++j)
+      if (address(off + j * ax.s) - address(off) != j * ax.sigma) first_bad = j;
+    if (!first_bad) continue;
+    // the row axis may run over two nested extents (pixels inside images): linear inside, one
+    // more stride between them
+    if (&ax != &axes[1] || ax.e % first_bad) return std::nullopt;
+    rsplit = first_bad;
+    sr2 = address(off + rsplit * ax.s) - address(off);
     for (int64_t j = 0; j < ax.e; ++j)
-      if (address(off + j * ax.s) - address(off) != j * ax.sigma) return std::nullopt;
+      if (address(off + j * ax.s) - address(off) != (j / rsplit) * sr2 + (j % rsplit) * ax.sigma) return std::nullopt;
   }
-  PlainOperand p{address(off), axes[0].sigma, axes[1].sigma, axes[2].sigma};
-  if (p.off < 0 || p.sr < 0 || p.sk < 0 || p.bs < 0) return std::nullopt;
+  PlainOperand p{address(off), axes[0].sigma, axes[1].sigma, axes[2].sigma, rsplit, sr2};
+  if (p.off < 0 || p.sr < 0 || p.sk < 0 || p.bs < 0 || p.sr2 < 0) return std::nullopt;
   return p;
 }
 
@@ -301,12 +318,14 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   if (fa)
     if (auto p = plain_operand(*fa, s->a_off, s->a_b, s->a_m, s->a_k, s->batch, s->M, s->K)) {
       s->a_buf = fa->src; s->a_off = p->off; s->a_b = p->bs; s->a_m = p->sr; s->a_k = p->sk;
+      s->a_msplit = p->rsplit; s->a_m2 = p->sr2;
       fa = nullptr;
       plain_tag += ",A:source";
     }
   if (fb)
     if (auto p = plain_operand(*fb, s->b_off, s->b_b, s->b_n, s->b_k, s->batch, s->N, s->K)) {
       s->b_buf = fb->src; s->b_off = p->off; s->b_b = p->bs; s->b_n = p->sr; s->b_k = p->sk;
+      s->b_nsplit = p->rsplit; s->b_n2 = p->sr2;
       fb = nullptr;
       plain_tag += ",B:source";
     }
@@ -324,8 +343,11 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   };
   if (fa) a_kc = along_k(*fa, s->a_m, s->a_k);
   if (fb) b_nc = !along_k(*fb, s->b_n, s->b_k);
-  const bool a_vec = !fa && (a_kc ? vec_ok(s->K, s->a_k, s->a_m, s->a_off, s->a_b) : vec_ok(s->M, s->a_m, s->a_k, s->a_off, s->a_b));
-  const bool b_vec = !fb && (b_nc ? vec_ok(s->N, s->b_n, s->b_k, s->b_off, s->b_b) : vec_ok(s->K, s->b_k, s->b_n, s->b_off, s->b_b));
+  // (a split row axis: vectors along the rows must not straddle two inner extents)
+  const bool a_split_ok = !s->a_msplit || (s->a_m2 % 4 == 0 && (a_kc || s->a_msplit % 4 == 0));
+  const bool b_split_ok = !s->b_nsplit || (s->b_n2 % 4 == 0 && (!b_nc || s->b_nsplit % 4 == 0));
+  const bool a_vec = !fa && a_split_ok && (a_kc ? vec_ok(s->K, s->a_k, s->a_m, s->a_off, s->a_b) : vec_ok(s->M, s->a_m, s->a_k, s->a_off, s->a_b));
+  const bool b_vec = !fb && b_split_ok && (b_nc ? vec_ok(s->N, s->b_n, s->b_k, s->b_off, s->b_b) : vec_ok(s->K, s->b_k, s->b_n, s->b_off, s->b_b));
   const int S = ch.split_k;
   std::vector<LaunchSpec> out(S > 1 ? 2 : 1);
   LaunchSpec& ls = out[0];
@@ -346,8 +368,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   {
     // direct-to-LDS loads: row-contiguous operand, 128-bit loads, no guards needed on its tile
     const bool k_exact = s->K % t.bk == 0 && ((s->K / t.bk) % ch.split_k) == 0;
-    const bool a_dma = opt.gemm_dma && !a_kc && a_vec && k_exact && s->M % t.bm == 0;
-    const bool b_dma = opt.gemm_dma && b_nc && b_vec && k_exact && s->N % t.bn == 0;
+    const bool a_dma = opt.gemm_dma && !a_kc && a_vec && k_exact && s->M % t.bm == 0 && !s->a_msplit;
+    const bool b_dma = opt.gemm_dma && b_nc && b_vec && k_exact && s->N % t.bn == 0 && !s->b_nsplit;
     os << "#define EH_A_DMA " << (a_dma ? 1 : 0) << "\n#define EH_B_DMA " << (b_dma ? 1 : 0) << "\n";
     dma_tag = std::string(a_dma ? ",A>lds" : "") + (b_dma ? ",B>lds" : "");
   }
@@ -357,6 +379,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_A_OFF " << s->a_off << "LL\n#define EH_B_OFF " << s->b_off << "LL\n#define EH_C_OFF " << s->c_off
      << "LL\n";
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
+  os << "#define EH_A_MSPLIT " << s->a_msplit << "LL\n#define EH_A_SM2 " << s->a_m2 << "LL\n";
+  os << "#define EH_B_NSPLIT " << s->b_nsplit << "LL\n#define EH_B_SN2 " << s->b_n2 << "LL\n";
   os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
   // A computed operand's element (row r, k) sits at off + bz*bs + r*sr + k*sk of the producer's
@@ -462,8 +486,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   ls.arg_bufs = {fa ? fa->src : s->a_buf, fb ? fb->src : s->b_buf};
   // a folded operand binds the producer's source, whose size the buffer table already fixes
   ls.arg_min_bytes = {
-      fa ? 0 : 4 * static_cast<size_t>(s->a_off + (s->M - 1) * s->a_m + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
-      fb ? 0 : 4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + (s->N - 1) * s->b_n + (s->batch - 1) * s->b_b + 1)};
+      fa ? 0 : 4 * static_cast<size_t>(s->a_off + row_reach(s->M, s->a_m, s->a_msplit, s->a_m2) + (s->K - 1) * s->a_k + (s->batch - 1) * s->a_b + 1),
+      fb ? 0 : 4 * static_cast<size_t>(s->b_off + (s->K - 1) * s->b_k + row_reach(s->N, s->b_n, s->b_nsplit, s->b_n2) + (s->batch - 1) * s->b_b + 1)};
   if (!(epi_here && !epilogue->store_c)) {
     ls.arg_bufs.push_back(S > 1 ? scratch : s->c_buf);
     ls.arg_min_bytes.push_back(4 * (S > 1 ? part_elems : c_elems));

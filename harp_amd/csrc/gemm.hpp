@@ -20,6 +20,9 @@ struct GemmShape {
   int64_t a_m = 0, a_k = 0, a_b = 0, a_off = 0;   // element strides / offset of A
   int64_t b_k = 0, b_n = 0, b_b = 0, b_off = 0;
   int64_t c_m = 0, c_n = 0, c_b = 0, c_off = 0;
+  // a row axis that runs over two nested extents of the memory it reads: rows per inner extent
+  // (0: one stride) and the stride between inner extents
+  int64_t a_msplit = 0, a_m2 = 0, b_nsplit = 0, b_n2 = 0;
 };
 
 // An elementwise producer (im2col gather, layout copy, padding ...) whose dense output a

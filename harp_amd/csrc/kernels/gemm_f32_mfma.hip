@@ -76,6 +76,14 @@
 #ifndef EH_TRANSPOSE
 #define EH_TRANSPOSE 0
 #endif
+#ifndef EH_A_MSPLIT
+#define EH_A_MSPLIT 0     // rows of A per inner extent when its row axis is split in memory (0: one stride)
+#define EH_A_SM2 0
+#endif
+#ifndef EH_B_NSPLIT
+#define EH_B_NSPLIT 0
+#define EH_B_SN2 0
+#endif
 #ifndef EH_PREFETCH
 #define EH_PREFETCH 1     // how many tile steps ahead of their use the global loads are issued
 #endif
@@ -154,17 +162,25 @@ static_assert(!EH_B_VEC || (EH_B_NCONTIG ? EH_N % 4 == 0 : EH_K % 4 == 0), "B ca
 // the generator splits the producer's loop variables at Q: in mode 1 the row decides the
 // variables above Q and k those below, in mode 2 the other way round; in mode 0 the index does
 // not separate and val decodes all of it.
-template <long long OFF, long long BS, long long SR, long long SK>
+// RSPLIT > 0: the row axis runs over two nested extents of the memory it reads (images of RSPLIT
+// pixels each, say): row r sits at (r / RSPLIT) * SR2 + (r % RSPLIT) * SR.  Rows are decoded
+// once per work-item, so the division is off the k loop.
+template <long long OFF, long long BS, long long SR, long long SK, long long RSPLIT, long long SR2>
 struct EhFromMemory {
   typedef long long Row;
   typedef long long Kk;
-  __device__ __forceinline__ static Row row(long long bz, long long r) { return OFF + bz * BS + r * SR; }
+  __device__ __forceinline__ static Row row(long long bz, long long r) {
+    if (RSPLIT > 0) return OFF + bz * BS + (r / RSPLIT) * SR2 + (r % RSPLIT) * SR;
+    return OFF + bz * BS + r * SR;
+  }
   __device__ __forceinline__ static Kk kk(long long, long long k) { return k * SK; }
   __device__ __forceinline__ static float val(const float* __restrict__ p, const Row& r, const Kk& k) { return p[r + k]; }
+  __device__ __forceinline__ static long long mem(const Row& r) { return r; }     // a row's offset in memory (128-bit path)
 };
 #ifdef EH_A_FOLD
 struct EhAElem {
   static constexpr long long Q = EH_A_FOLD_Q;
+  template <class R> __device__ __forceinline__ static long long mem(const R&) { return 0; }   // never read as vectors
 #if EH_A_FOLD_MODE == 1
   typedef eh_a_upper Row;
   typedef eh_a_lower Kk;
@@ -188,11 +204,12 @@ struct EhAElem {
 #endif
 };
 #else
-using EhAElem = EhFromMemory<EH_A_OFF, EH_A_BS, EH_A_SM, EH_A_SK>;
+using EhAElem = EhFromMemory<EH_A_OFF, EH_A_BS, EH_A_SM, EH_A_SK, EH_A_MSPLIT, EH_A_SM2>;
 #endif
 #ifdef EH_B_FOLD
 struct EhBElem {
   static constexpr long long Q = EH_B_FOLD_Q;
+  template <class R> __device__ __forceinline__ static long long mem(const R&) { return 0; }   // never read as vectors
 #if EH_B_FOLD_MODE == 1
   typedef eh_b_upper Row;
   typedef eh_b_lower Kk;
@@ -216,7 +233,7 @@ struct EhBElem {
 #endif
 };
 #else
-using EhBElem = EhFromMemory<EH_B_OFF, EH_B_BS, EH_B_SN, EH_B_SK>;
+using EhBElem = EhFromMemory<EH_B_OFF, EH_B_BS, EH_B_SN, EH_B_SK, EH_B_NSPLIT, EH_B_SN2>;
 #endif
 
 // The rows a work-item reads of an operand tile, decoded once: one row (the four elements run
@@ -245,8 +262,9 @@ __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long
                                               long long k, long long R, long long kend, const EhRows<ELEM, ALONG_K>& rows) {
   eh_f4v v = {0.0f, 0.0f, 0.0f, 0.0f};
   if (VEC) {
+    // (the first of the work-item's rows: four rows of one vector never straddle a split)
     const bool ok = (!EDGE_R || r < R) && (!EDGE_K || k < kend);
-    if (ok) v = *reinterpret_cast<const eh_f4v*>(p + base + r * SR + k * SK);
+    if (ok) v = *reinterpret_cast<const eh_f4v*>(p + ELEM::mem(rows.row[0]) + k * SK);
   } else if (ALONG_K) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -396,18 +414,18 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   // the rows of each tile this work-item fetches, decoded once (they do not change with k)
   EhRows<EhAElem, EH_A_KCONTIG != 0> a_rows[AV];
   EhRows<EhBElem, EH_B_NCONTIG == 0> b_rows[BV];
-#if !EH_A_VEC && !EH_A_DMA
+#if !EH_A_DMA
 #pragma unroll
   for (int i = 0; i < AV; ++i) {
     const int q = tid + i * NT;
-    a_rows[i].set(bz, EH_A_KCONTIG ? m0 + q / (BK / 4) : m0 + (q % (BM / 4)) * 4, M);
+    a_rows[i].set(bz, EH_A_KCONTIG ? m0 + q / (BK / 4) : EH_A_TR ? m0 + ((q >> 2) % (BM / 4)) * 4 : m0 + (q % (BM / 4)) * 4, M);
   }
 #endif
-#if !EH_B_VEC && !EH_B_DMA
+#if !EH_B_DMA
 #pragma unroll
   for (int i = 0; i < BV; ++i) {
     const int q = tid + i * NT;
-    b_rows[i].set(bz, EH_B_NCONTIG ? n0 + (q % (BN / 4)) * 4 : n0 + q / (BK / 4), N);
+    b_rows[i].set(bz, EH_B_TR ? n0 + ((q >> 2) % (BN / 4)) * 4 : EH_B_NCONTIG ? n0 + (q % (BN / 4)) * 4 : n0 + q / (BK / 4), N);
   }
 #endif
 

@@ -630,7 +630,8 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
     plan = hb.render_program(ast, "lanes=1")
-    cols = [l for l in plan.launches if l["schedule"].startswith("mfma") and "A:m,B:n/folded" in l["schedule"]]
+    # (transposed product: W as rows; dY, a copy through a view, read from its source with strides)
+    cols = [l for l in plan.launches if l["schedule"].startswith("mfma") and "A:m,B:n,B:source" in l["schedule"]]
     assert len(cols) == 1, [l["schedule"] for l in plan.launches]
     temp = cols[0]["args"][-1]
     (reader,) = [l for l in plan.launches if temp in l["args"] and l is not cols[0]]
@@ -638,7 +639,7 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert body.count(temp + "[") == 9
     assert "if (" not in body.replace("if (eh_", "")            # guarded loads: clamped index + select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
-    assert not any("A:m,B:n/folded" in l["schedule"] for l in plain.launches)
+    assert not any("A:m,B:n,B:source" in l["schedule"] for l in plain.launches)
     # the weight gradients' dY operand is a copy through a view (NCHW read as [image, pixel, channel]):
     # read from its source with strides, not through an element function
     direct = [l for l in plan.launches if "A:source" in l["schedule"]]
