@@ -463,7 +463,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_waves") o.gemm_waves = as_int();
     else if (k == "gemm_fold") o.gemm_fold = as_int() != 0;
     else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
-    else if (k == "gemm_dma") o.gemm_dma = as_int() != 0;
+    else if (k == "gemm_dma") o.gemm_dma = std::max(0, std::min(3, as_int()));
     else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
     else if (k == "gemm_transpose") o.gemm_transpose = as_int() != 0;
     else if (k == "gemm_prefetch") o.gemm_prefetch = std::max(0, as_int());

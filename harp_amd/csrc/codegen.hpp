@@ -35,7 +35,7 @@ struct GenOptions {
   bool gemm_transpose = false;        // row-contiguous operands transposed over lane quads into the k-contiguous LDS layout (measured slower)
   int gemm_prefetch = 0;              // tile steps the global loads run ahead (0: 3 for tiles up to 64x64, else 1)
   bool gemm_mix = true;               // LDS operand reads interleaved with the MFMAs of the block before
-  bool gemm_dma = false;              // global_load_lds for row-contiguous operand tiles
+  int gemm_dma = 2;                   // global_load_lds for row-contiguous operand tiles: 0 never, 1 wherever possible, 2 B only, 3 A only
   bool gemm_merge_batch = false;      // per-batch contractions summed over the batch become one contraction
   bool gemm_epilogue = true;          // run elementwise consumers of a contraction on its accumulators
   bool gemm_fold = true;              // evaluate gather/copy producers inside the tile loader (implicit GEMM)

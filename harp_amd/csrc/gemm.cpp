@@ -368,8 +368,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   {
     // direct-to-LDS loads: row-contiguous operand, 128-bit loads, no guards needed on its tile
     const bool k_exact = s->K % t.bk == 0 && ((s->K / t.bk) % ch.split_k) == 0;
-    const bool a_dma = opt.gemm_dma && !a_kc && a_vec && k_exact && s->M % t.bm == 0 && !s->a_msplit;
-    const bool b_dma = opt.gemm_dma && b_nc && b_vec && k_exact && s->N % t.bn == 0 && !s->b_nsplit;
+    const bool a_dma = (opt.gemm_dma == 1 || opt.gemm_dma == 3) && !a_kc && a_vec && k_exact && s->M % t.bm == 0 && !s->a_msplit;
+    const bool b_dma = (opt.gemm_dma == 1 || opt.gemm_dma == 2) && b_nc && b_vec && k_exact && s->N % t.bn == 0 && !s->b_nsplit;
     os << "#define EH_A_DMA " << (a_dma ? 1 : 0) << "\n#define EH_B_DMA " << (b_dma ? 1 : 0) << "\n";
     dma_tag = std::string(a_dma ? ",A>lds" : "") + (b_dma ? ",B>lds" : "");
   }
