@@ -1844,6 +1844,214 @@ NodePtr transpose_reader(const NestKernel& E, const std::string& T, int64_t M, i
   return make_kernel(E.name, E.params, body);
 }
 
+
+// The program-level rewrites in front of planning (option `reindex`): whole-buffer copies dropped,
+// stored values read back, elementwise producers evaluated in readers that walk another index
+// space, contraction temps stored the way their readers walk them.  `kernels` is the program's
+// kernel list in execution order (entries are replaced or removed), `rewritten` owns the new
+// kernels, `plan->elided` collects the temps that disappear.
+void rewrite_for_readers(const Node& program, const GenOptions& opt, std::vector<const Node*>* kernels,
+                         std::vector<NodePtr>* rewritten, ProgramPlan* plan) {
+  auto is_temp = [&](const std::string& name) {
+    for (const auto& b : plan->buffers)
+      if (b.name == name) return b.role == "temp";
+    return false;
+  };
+  auto writers_of = [&](const std::string& name) {
+    size_t n = 0;
+    for (const Node* k : *kernels)
+      for (const auto& pp : k->params) n += pp.dtype.is_ptr() && pp.mut_ && pp.name == name;
+    return n;
+  };
+  auto rename_buffer = [&](const NodePtr& k, const std::string& from, const std::string& to) {
+    NodePtr body = rename(k->args[0], {{from, make_var(to)}});
+    std::vector<Param> params;
+    bool have = false;
+    for (const auto& pp : k->params) have = have || pp.name == to;
+    for (auto pp : k->params) {
+      if (pp.name == from) {
+        if (have) continue;
+        pp.name = to;
+      }
+      params.push_back(pp);
+    }
+    auto c = std::make_shared<Node>(*k);
+    c->params = std::move(params);
+    c->args = {body};
+    return c;
+  };
+  // phase 0 drops whole-buffer copies; then values that an earlier kernel already stored are
+  // read back where a later kernel computes them again; phase 1 evaluates producers in readers
+  for (int phase = 0; phase < 2; ++phase) {
+    if (phase == 1) {
+      for (size_t si = 0; si < kernels->size(); ++si) {
+        auto ns = extract_nest(*(*kernels)[si]);
+        if (!ns || ns->rkind != ReduceKind::None || writers_of(ns->out_buf) != 1) continue;
+        for (size_t ri = si + 1; ri < kernels->size(); ++ri) {
+          auto nr = extract_nest(*(*kernels)[ri]);
+          if (!nr) continue;
+          NodePtr nk = reuse_stored_value(*ns, *nr);
+          if (!nk) continue;
+          rewritten->push_back(nk);
+          (*kernels)[ri] = nk.get();
+        }
+      }
+    }
+    for (bool again = true; again;) {
+      again = false;
+      for (size_t p = 0; p < kernels->size() && !again; ++p) {
+        auto np = extract_nest(*(*kernels)[p]);
+        if (!np || np->rkind != ReduceKind::None || !is_temp(np->out_buf) || writers_of(np->out_buf) != 1) continue;
+        std::vector<size_t> rd;
+        bool early = false;
+        for (size_t c = 0; c < kernels->size(); ++c)
+          for (const auto& pp : (*kernels)[c]->params)
+            if (pp.dtype.is_ptr() && !pp.mut_ && pp.name == np->out_buf) {
+              rd.push_back(c);
+              early = early || c <= p;
+            }
+        if (rd.empty() || early) continue;
+        // a copy of a whole buffer, element for element: its readers read the original
+        if (np->value->op == Op::Load && np->value->args[0]->op == Op::Var && np->value->count == 1 && np->out_aff) {
+          const std::string& src = np->value->args[0]->name;
+          auto a = affine_of(*np->value->args[1]);
+          int64_t numel = 0;
+          bool same_type = false;
+          for (const auto& pp : np->params) same_type = same_type || (pp.name == src && pp.dtype.is_ptr() && pp.dtype.elem().ty == np->out_dtype.ty);
+          if (a && *a == *np->out_aff && dense_strides(*np, &numel) && same_type && src != np->out_buf && writers_of(src) <= 1) {
+            bool src_written_later = false;
+            for (size_t m = p + 1; m < kernels->size(); ++m)
+              for (const auto& pm : (*kernels)[m]->params) src_written_later = src_written_later || (pm.dtype.is_ptr() && pm.mut_ && pm.name == src);
+            if (!src_written_later) {
+              for (size_t c : rd) {
+                NodePtr owner;
+                for (const auto& f : program.args)
+                  if (f.get() == (*kernels)[c]) owner = f;
+                for (const auto& f : *rewritten)
+                  if (f.get() == (*kernels)[c]) owner = f;
+                if (!owner) throw Error("internal: kernel without owner");
+                NodePtr nk = rename_buffer(owner, np->out_buf, src);
+                rewritten->push_back(nk);
+                (*kernels)[c] = nk.get();
+              }
+              plan->elided.insert(np->out_buf);
+              kernels->erase(kernels->begin() + static_cast<long>(p));
+              again = true;
+              continue;
+            }
+          }
+        }
+        if (phase == 0 || rd.size() > 3) continue;
+        {
+          // what reads a reduction's result element for element stays with it: it is that
+          // reduction's epilogue, and evaluated elsewhere it would keep the raw result alive for a
+          // reader far away
+          int64_t p_numel = 1;
+          for (const auto& l : np->loops) p_numel *= l.extent;
+          bool after_reduce = false;
+          for (const auto& pp : (*kernels)[p]->params) {
+            if (!pp.dtype.is_ptr() || pp.mut_) continue;
+            for (size_t w = 0; w < p; ++w) {
+              bool writes = false;
+              for (const auto& pw : (*kernels)[w]->params) writes = writes || (pw.dtype.is_ptr() && pw.mut_ && pw.name == pp.name);
+              if (!writes) continue;
+              auto nw = extract_nest(*(*kernels)[w]);
+              int64_t w_numel = 1;
+              if (nw)
+                for (const auto& l : nw->loops) w_numel *= l.extent;
+              after_reduce = after_reduce || !nw || (nw->rkind != ReduceKind::None && w_numel == p_numel);
+            }
+          }
+          if (after_reduce) continue;
+        }
+        {
+          std::vector<LoadRef> pl;
+          collect_loads(*np->value, pl);
+          std::set<std::string> srcs;
+          for (const auto& lr : pl)
+            if (lr.load->args[0]->op == Op::Var) srcs.insert(lr.load->args[0]->name);
+          if (rd.size() > 1 && srcs.size() > 6) continue;    // evaluated once per reader: keep it cheap
+        }
+        size_t left = rd.size();
+        for (size_t reader : rd) {
+          // nothing between the two may write what P reads
+          bool clobbered = false;
+          for (size_t m = p + 1; m <= reader; ++m)
+            for (const auto& pm : (*kernels)[m]->params)
+              if (pm.dtype.is_ptr() && pm.mut_)
+                for (const auto& pp : (*kernels)[p]->params) clobbered = clobbered || (pp.name == pm.name && !pp.mut_);
+          if (clobbered) continue;
+          auto nc = extract_nest(*(*kernels)[reader]);
+          if (!nc) continue;
+          auto in = inline_producer(*np, *nc);
+          if (!in) continue;
+          rewritten->push_back(in->kernel);
+          (*kernels)[reader] = in->kernel.get();
+          --left;
+          again = true;
+        }
+        if (left == 0) {
+          plan->elided.insert(np->out_buf);
+          kernels->erase(kernels->begin() + static_cast<long>(p));
+        }
+      }
+    }
+  }
+  // temps between a contraction and an elementwise reader that walks them column by column
+  for (size_t p = 0; p < kernels->size(); ++p) {
+    auto nk = extract_nest(*(*kernels)[p]);
+    if (!nk || nk->rkind != ReduceKind::Sum) continue;
+    bool temp = false;
+    for (const auto& b : plan->buffers) temp = temp || (b.name == nk->out_buf && b.role == "temp");
+    if (!temp) continue;
+    std::vector<size_t> rd;
+    size_t nwriters = 0;
+    bool early = false;
+    for (size_t c = 0; c < kernels->size(); ++c)
+      for (const auto& pp : (*kernels)[c]->params)
+        if (pp.dtype.is_ptr() && pp.name == nk->out_buf) {
+          if (pp.mut_) ++nwriters;
+          else { rd.push_back(c); early = early || c <= p; }
+        }
+    if (rd.empty() || nwriters != 1 || early) continue;
+    {
+      // one reader that reads every element once, unguarded, is a plain permutation: the
+      // contraction's epilogue writes that reader's result in place instead
+      size_t sites = 0;
+      bool guarded = false;
+      for (size_t c : rd) {
+        auto ne = extract_nest(*(*kernels)[c]);
+        if (!ne) continue;
+        std::vector<LoadRef> lds;
+        collect_loads(*ne->value, lds);
+        for (const auto& lr : lds)
+          if (lr.load->args[0]->op == Op::Var && lr.load->args[0]->name == nk->out_buf) {
+            ++sites;
+            guarded = guarded || lr.guarded;
+          }
+      }
+      if (sites < 2 && !guarded) continue;
+    }
+    int64_t M = 0, N = 0;
+    NodePtr prod = transpose_producer(*nk, opt, &M, &N);
+    if (!prod) continue;
+    std::vector<NodePtr> readers_new;
+    for (size_t c : rd) {
+      auto ne = extract_nest(*(*kernels)[c]);
+      NodePtr r = ne ? transpose_reader(*ne, nk->out_buf, M, N) : nullptr;
+      if (!r) break;
+      readers_new.push_back(r);
+    }
+    if (readers_new.size() != rd.size()) continue;
+    rewritten->push_back(prod);
+    (*kernels)[p] = prod.get();
+    for (size_t i = 0; i < rd.size(); ++i) {
+      rewritten->push_back(readers_new[i]);
+      (*kernels)[rd[i]] = readers_new[i].get();
+    }
+  }
+}
+
 }  // namespace
 
 
@@ -2051,212 +2259,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
     kernels = out;
   }
-  if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
-    auto is_temp = [&](const std::string& name) {
-      for (const auto& b : plan.buffers)
-        if (b.name == name) return b.role == "temp";
-      return false;
-    };
-    auto writers_of = [&](const std::string& name) {
-      size_t n = 0;
-      for (const Node* k : kernels)
-        for (const auto& pp : k->params) n += pp.dtype.is_ptr() && pp.mut_ && pp.name == name;
-      return n;
-    };
-    auto rename_buffer = [&](const NodePtr& k, const std::string& from, const std::string& to) {
-      NodePtr body = rename(k->args[0], {{from, make_var(to)}});
-      std::vector<Param> params;
-      bool have = false;
-      for (const auto& pp : k->params) have = have || pp.name == to;
-      for (auto pp : k->params) {
-        if (pp.name == from) {
-          if (have) continue;
-          pp.name = to;
-        }
-        params.push_back(pp);
-      }
-      auto c = std::make_shared<Node>(*k);
-      c->params = std::move(params);
-      c->args = {body};
-      return c;
-    };
-    // phase 0 drops whole-buffer copies; then values that an earlier kernel already stored are
-    // read back where a later kernel computes them again; phase 1 evaluates producers in readers
-    for (int phase = 0; phase < 2; ++phase) {
-    if (phase == 1 && !std::getenv("ECLAT_HIP_NO_REUSE")) {
-      for (size_t si = 0; si < kernels.size(); ++si) {
-        auto ns = extract_nest(*kernels[si]);
-        if (!ns || ns->rkind != ReduceKind::None || writers_of(ns->out_buf) != 1) continue;
-        for (size_t ri = si + 1; ri < kernels.size(); ++ri) {
-          auto nr = extract_nest(*kernels[ri]);
-          if (!nr) continue;
-          NodePtr nk = reuse_stored_value(*ns, *nr);
-          if (!nk) continue;
-          if (std::getenv("ECLAT_HIP_DEBUG_REINDEX"))
-            fprintf(stderr, "reuse: %s reads %s of %s\n", nr->name.c_str(), ns->out_buf.c_str(), ns->name.c_str());
-          rewritten.push_back(nk);
-          kernels[ri] = nk.get();
-        }
-      }
-    }
-    for (bool again = true; again;) {
-      again = false;
-      for (size_t p = 0; p < kernels.size() && !again; ++p) {
-        auto np = extract_nest(*kernels[p]);
-        if (!np || np->rkind != ReduceKind::None || !is_temp(np->out_buf) || writers_of(np->out_buf) != 1) continue;
-        std::vector<size_t> rd;
-        bool early = false;
-        for (size_t c = 0; c < kernels.size(); ++c)
-          for (const auto& pp : kernels[c]->params)
-            if (pp.dtype.is_ptr() && !pp.mut_ && pp.name == np->out_buf) {
-              rd.push_back(c);
-              early = early || c <= p;
-            }
-        if (rd.empty() || early) continue;
-        // a copy of a whole buffer, element for element: its readers read the original
-        if (np->value->op == Op::Load && np->value->args[0]->op == Op::Var && np->value->count == 1 && np->out_aff) {
-          const std::string& src = np->value->args[0]->name;
-          auto a = affine_of(*np->value->args[1]);
-          int64_t numel = 0;
-          bool same_type = false;
-          for (const auto& pp : np->params) same_type = same_type || (pp.name == src && pp.dtype.is_ptr() && pp.dtype.elem().ty == np->out_dtype.ty);
-          if (a && *a == *np->out_aff && dense_strides(*np, &numel) && same_type && src != np->out_buf && writers_of(src) <= 1) {
-            bool src_written_later = false;
-            for (size_t m = p + 1; m < kernels.size(); ++m)
-              for (const auto& pm : kernels[m]->params) src_written_later = src_written_later || (pm.dtype.is_ptr() && pm.mut_ && pm.name == src);
-            if (!src_written_later) {
-              for (size_t c : rd) {
-                NodePtr owner;
-                for (const auto& f : program.args)
-                  if (f.get() == kernels[c]) owner = f;
-                for (const auto& f : rewritten)
-                  if (f.get() == kernels[c]) owner = f;
-                if (!owner) throw Error("internal: kernel without owner");
-                NodePtr nk = rename_buffer(owner, np->out_buf, src);
-                rewritten.push_back(nk);
-                kernels[c] = nk.get();
-              }
-              plan.elided.insert(np->out_buf);
-              kernels.erase(kernels.begin() + static_cast<long>(p));
-              again = true;
-              continue;
-            }
-          }
-        }
-        if (phase == 0 || rd.size() > 3) continue;
-        {
-          // what reads a reduction's result element for element stays with it: it is that
-          // reduction's epilogue, and evaluated elsewhere it would keep the raw result alive for a
-          // reader far away
-          int64_t p_numel = 1;
-          for (const auto& l : np->loops) p_numel *= l.extent;
-          bool after_reduce = false;
-          for (const auto& pp : kernels[p]->params) {
-            if (!pp.dtype.is_ptr() || pp.mut_) continue;
-            for (size_t w = 0; w < p; ++w) {
-              bool writes = false;
-              for (const auto& pw : kernels[w]->params) writes = writes || (pw.dtype.is_ptr() && pw.mut_ && pw.name == pp.name);
-              if (!writes) continue;
-              auto nw = extract_nest(*kernels[w]);
-              int64_t w_numel = 1;
-              if (nw)
-                for (const auto& l : nw->loops) w_numel *= l.extent;
-              after_reduce = after_reduce || !nw || (nw->rkind != ReduceKind::None && w_numel == p_numel);
-            }
-          }
-          if (after_reduce) continue;
-        }
-        {
-          std::vector<LoadRef> pl;
-          collect_loads(*np->value, pl);
-          std::set<std::string> srcs;
-          for (const auto& lr : pl)
-            if (lr.load->args[0]->op == Op::Var) srcs.insert(lr.load->args[0]->name);
-          if (rd.size() > 1 && srcs.size() > 6) continue;    // evaluated once per reader: keep it cheap
-        }
-        size_t left = rd.size();
-        for (size_t reader : rd) {
-          // nothing between the two may write what P reads
-          bool clobbered = false;
-          for (size_t m = p + 1; m <= reader; ++m)
-            for (const auto& pm : kernels[m]->params)
-              if (pm.dtype.is_ptr() && pm.mut_)
-                for (const auto& pp : kernels[p]->params) clobbered = clobbered || (pp.name == pm.name && !pp.mut_);
-          if (clobbered) continue;
-          auto nc = extract_nest(*kernels[reader]);
-          if (!nc) continue;
-          auto in = inline_producer(*np, *nc);
-          if (std::getenv("ECLAT_HIP_DEBUG_REINDEX"))
-            fprintf(stderr, "reindex: %s (%s) into %s: %s\n", np->name.c_str(), np->out_buf.c_str(), nc->name.c_str(), in ? "yes" : "no");
-          if (!in) continue;
-          rewritten.push_back(in->kernel);
-          kernels[reader] = in->kernel.get();
-          --left;
-          again = true;
-        }
-        if (left == 0) {
-          plan.elided.insert(np->out_buf);
-          kernels.erase(kernels.begin() + static_cast<long>(p));
-        }
-      }
-    }
-    }
-  }
-  if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
-    // temps between a contraction and an elementwise reader that walks them column by column
-    for (size_t p = 0; p < kernels.size(); ++p) {
-      auto nk = extract_nest(*kernels[p]);
-      if (!nk || nk->rkind != ReduceKind::Sum) continue;
-      bool temp = false;
-      for (const auto& b : plan.buffers) temp = temp || (b.name == nk->out_buf && b.role == "temp");
-      if (!temp) continue;
-      std::vector<size_t> rd;
-      size_t nwriters = 0;
-      bool early = false;
-      for (size_t c = 0; c < kernels.size(); ++c)
-        for (const auto& pp : kernels[c]->params)
-          if (pp.dtype.is_ptr() && pp.name == nk->out_buf) {
-            if (pp.mut_) ++nwriters;
-            else { rd.push_back(c); early = early || c <= p; }
-          }
-      if (rd.empty() || nwriters != 1 || early) continue;
-      {
-        // one reader that reads every element once, unguarded, is a plain permutation: the
-        // contraction's epilogue writes that reader's result in place instead
-        size_t sites = 0;
-        bool guarded = false;
-        for (size_t c : rd) {
-          auto ne = extract_nest(*kernels[c]);
-          if (!ne) continue;
-          std::vector<LoadRef> lds;
-          collect_loads(*ne->value, lds);
-          for (const auto& lr : lds)
-            if (lr.load->args[0]->op == Op::Var && lr.load->args[0]->name == nk->out_buf) {
-              ++sites;
-              guarded = guarded || lr.guarded;
-            }
-        }
-        if (sites < 2 && !guarded) continue;
-      }
-      int64_t M = 0, N = 0;
-      NodePtr prod = transpose_producer(*nk, opt, &M, &N);
-      if (!prod) continue;
-      std::vector<NodePtr> readers_new;
-      for (size_t c : rd) {
-        auto ne = extract_nest(*kernels[c]);
-        NodePtr r = ne ? transpose_reader(*ne, nk->out_buf, M, N) : nullptr;
-        if (!r) break;
-        readers_new.push_back(r);
-      }
-      if (readers_new.size() != rd.size()) continue;
-      rewritten.push_back(prod);
-      kernels[p] = prod.get();
-      for (size_t i = 0; i < rd.size(); ++i) {
-        rewritten.push_back(readers_new[i]);
-        kernels[rd[i]] = readers_new[i].get();
-      }
-    }
-  }
+  if (!plan.buffers.empty() && opt.fuse && opt.reindex) rewrite_for_readers(program, opt, &kernels, &rewritten, &plan);
   std::map<std::string, size_t> elems;
   bool have_table = !plan.buffers.empty();
   if (have_table) {
@@ -2623,9 +2626,6 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             const NestKernel& sk = *nests[j];
             int64_t numel = 0;
             auto strides = dense_strides(sk, &numel);
-            if (std::getenv("ECLAT_HIP_DEBUG_EPI"))
-              fprintf(stderr, "epi %s: stage %s strides %d numel %lld total %lld\n", k0.name.c_str(), sk.name.c_str(), strides ? 1 : 0,
-                      (long long)numel, (long long)total);
             if (!strides || numel != total || avail.count(sk.out_buf)) break;
             std::vector<LoadRef> loads;
             collect_loads(*sk.value, loads);
@@ -2665,7 +2665,6 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
                 for (size_t r : readers[kv.first]) sole = sole && r > i && r <= j;
               }
               auto na = sole ? relayout(k0, sk, *permuted) : std::nullopt;
-              if (std::getenv("ECLAT_HIP_DEBUG_EPI")) fprintf(stderr, "epi %s: sole %d relayout %d\n", k0.name.c_str(), sole ? 1 : 0, na ? 1 : 0);
               if (!na) break;
               k0r.out_aff = *na;
               if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; break; }
