@@ -172,7 +172,7 @@ impl Kernel for HipKernel {
             .expect("buffer is not a HipBuffer").raw).collect();
         match self.loaded {
             Loaded::Program(p) => check(unsafe {
-                ffi::eh_program_execute_positional(p, ins.as_ptr(), ins.len() as i32, outs.as_ptr(), outs.len() as i32, 1)
+                ffi::eh_program_execute_positional(p, ins.as_ptr(), ins.len() as i32, outs.as_ptr(), outs.len() as i32, wait_per_launch())
             }),
             Loaded::Module(_) => {
                 let g = self.config.global_work_size;
@@ -389,9 +389,18 @@ fn run_program(device: &dyn Any, kernels: &[AstNode], table: &[ProgramBuffer],
             .ok_or_else(|| err(format!("buffer '{name}' is not a HipBuffer")))?;
         raws.push(b.raw);
     }
-    // synchronous, as every Kernel::execute of the reference is
-    if unsafe { ffi::eh_program_execute(prog.raw, raws.as_ptr(), n, 1) } != 0 { return Err(err(ffi::last_error())); }
+    if unsafe { ffi::eh_program_execute(prog.raw, raws.as_ptr(), n, wait_per_launch()) } != 0 { return Err(err(ffi::last_error())); }
     Ok(())
+}
+
+/// Launches are queued on the device's stream and not waited for: every read of a buffer
+/// (`Buffer::read_to_host` waits for the stream), every copy and every reuse of released memory is
+/// ordered behind them there, so a caller cannot see the difference except in time -- and in where
+/// a device fault is reported (at the next read instead of at `execute`).  ECLAT_HIP_SYNC=1 makes
+/// every `execute` wait, as the reference's own backends do.
+fn wait_per_launch() -> i32 {
+    static WAIT: OnceLock<i32> = OnceLock::new();
+    *WAIT.get_or_init(|| if std::env::var("ECLAT_HIP_SYNC").map(|v| v == "1").unwrap_or(false) { 1 } else { 0 })
 }
 
 /// Registers the backend (called at program start when the crate is linked).

@@ -285,16 +285,19 @@ class HipProgram:
 
 
 class HipKernel:
-    """One compiled kernel: `Kernel::execute(inputs, outputs)`, synchronous."""
+    """One compiled kernel: `Kernel::execute(inputs, outputs)`.  The reference's kernels return when
+    the work is done; `sync=False` only queues the launch on the device's stream, which every read
+    of a buffer and every reuse of its memory is ordered behind (what the Rust binding does unless
+    ECLAT_HIP_SYNC=1)."""
 
     def __init__(self, device: HipDevice, program_ast, options=None):
         self._prog = HipProgram(device, program_ast, options)
 
-    def execute(self, inputs: Sequence[HipBuffer], outputs: Sequence[HipBuffer]) -> None:
+    def execute(self, inputs: Sequence[HipBuffer], outputs: Sequence[HipBuffer], sync: bool = True) -> None:
         ins = (c_void_p * max(len(inputs), 1))(*[b._h for b in inputs])
         outs = (c_void_p * max(len(outputs), 1))(*[b._h for b in outputs])
         check(lib.eh_program_execute_positional(self._prog._h, ins, len(inputs), outs,
-                                                len(outputs), 1))
+                                                len(outputs), 1 if sync else 0))
 
     def get_binary(self) -> bytes:
         return self._prog.binary(0)

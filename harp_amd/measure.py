@@ -108,24 +108,26 @@ class PerKernelPath:
             n *= int(d)
         return n
 
-    def step(self, inputs):
-        """One pass; `inputs` maps buffer name -> HipBuffer.  Returns all buffers by name."""
+    def step(self, inputs, sync=True):
+        """One pass; `inputs` maps buffer name -> HipBuffer.  Returns all buffers by name.
+        `sync=False`: launches are only queued (the Rust binding's default)."""
         named = dict(inputs)
         for kern, ins, outs in self.kernels:
             out_bufs = [self.dev.alloc(self._nbytes(n)) for n in outs]
-            kern.execute([named[n] for n in ins], out_bufs)
+            kern.execute([named[n] for n in ins], out_bufs, sync)
             named.update(zip(outs, out_bufs))
         return named
 
-    def time(self, inputs, steps, warmup):
-        """Wall-clock ms per step (every launch is synchronous, so wall time is device time
-        plus what the host spends between launches, as it would be for the reference)."""
+    def time(self, inputs, steps, warmup, sync=True):
+        """Wall-clock ms per step.  With `sync` every launch waits for completion, so wall time is
+        device time plus what the host spends between launches, as it would be for the reference's
+        own backends; without, launches are queued and the device is waited for once at the end."""
         for _ in range(warmup):
-            self.step(inputs)
+            self.step(inputs, sync)
         self.dev.sync()
         t0 = time.perf_counter()
         for _ in range(steps):
-            self.step(inputs)
+            self.step(inputs, sync)
         self.dev.sync()
         return (time.perf_counter() - t0) * 1e3 / steps
 
