@@ -39,6 +39,9 @@ const Candidate kCandidates[] = {
     // from 23 to 16 us; 64x32, 128x32x32 and 32x32x16 tiles were tried as well and lost to 64x64 wherever
     // they were chosen)
     {{32, 64, 16, 32, 32}, 12, 80.0, 0.12, 0.8},     // 2 waves
+    // one wave: only for results that fit one MFMA tile (the first convolution's weight gradient,
+    // 32 channels by 9 taps per image: 19.5 -> 14.9 us, the second wave multiplied only padding)
+    {{32, 32, 16, 32, 32}, 16, 50.0, 0.06, 0.8},
 };
 
 bool tile_valid(const Tile& t) {
@@ -105,6 +108,7 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool compute
     // workgroup down; many small workgroups hide that, a few large ones do not (measured: a
     // 3x3 convolution over [32,128,28,28], 64x64 tiles 142 us, 128x128 295 us, 256x256 380 us)
     if (computed_operand && c.tile.bm * c.tile.bn > 64 * 64) continue;
+    if (c.tile.bm * c.tile.bn == 32 * 32 && (s.M > 32 || s.N > 32)) continue;
     const int64_t ksteps = ceil_div(s.K, c.tile.bk);
     for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
@@ -187,9 +191,26 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
   collapse(&mv, {&*aa, &ac});
   collapse(&nv, {&*ab, &ac});
   collapse(&bv, {&*aa, &*ab, &ac});
-  // a leftover outer row (column) axis can ride on the batch axis: the other operand simply
-  // does not move with it
-  if (bv.empty() && mv.size() == 2) {
+  GemmShape s;
+  // Two row (column) axes left: where the operand walks them as one axis and the inner extent
+  // would leave every image's last tile ragged (196 pixels an image), they are one axis and only
+  // C's address keeps the two extents (tiles run across images, none is padded per image) ...
+  auto merge_for = [&](std::vector<VarUse>* v, Affine* op, int64_t* split, int64_t* outer_stride) {
+    if (!bv.empty() || v->size() != 2) return false;
+    const VarUse o = (*v)[0], in = (*v)[1];
+    if (in.extent % 64 == 0 || op->of(o.var) != in.extent * op->of(in.var)) return false;
+    *split = in.extent;
+    *outer_stride = ac.of(o.var);
+    op->coef.erase(o.var);
+    (*v)[1].extent *= o.extent;
+    v->erase(v->begin());
+    return true;
+  };
+  if (merge_for(&mv, &*aa, &s.c_msplit, &s.c_m2) || merge_for(&nv, &*ab, &s.c_nsplit, &s.c_n2)) {
+    // one axis now
+  } else if (bv.empty() && mv.size() == 2) {
+    // ... otherwise the outer one rides on the batch axis: the other operand simply does not
+    // move with it
     bv.push_back(mv[0]);
     mv.erase(mv.begin());
   } else if (bv.empty() && nv.size() == 2) {
@@ -198,7 +219,6 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
   }
   if (mv.size() != 1 || nv.size() != 1 || bv.size() > 1) return std::nullopt;
   const std::string &mvar = mv[0].var, &nvar = nv[0].var;
-  GemmShape s;
   s.M = mv[0].extent; s.N = nv[0].extent; s.K = k.rloop.extent;
   s.a_buf = la->args[0]->name; s.b_buf = lb->args[0]->name; s.c_buf = k.out_buf;
   s.a_m = aa->of(mvar); s.a_k = aa->of(kv); s.a_off = aa->c;
@@ -217,13 +237,14 @@ std::optional<GemmShape> match_gemm(const NestKernel& k) {
     t.a_m = s.b_n; t.a_k = s.b_k; t.a_off = s.b_off; t.a_b = s.b_b;
     t.b_n = s.a_m; t.b_k = s.a_k; t.b_off = s.a_off; t.b_b = s.a_b;
     t.c_m = s.c_n; t.c_n = s.c_m;
+    t.c_msplit = s.c_nsplit; t.c_m2 = s.c_n2; t.c_nsplit = s.c_msplit; t.c_n2 = s.c_m2;
     return t;
   }
   return s;
 }
 
 bool gemm_output_dense(const GemmShape& s) {
-  return s.c_off == 0 && s.c_n == 1 && s.c_m == s.N && (s.batch == 1 || s.c_b == s.M * s.N);
+  return s.c_off == 0 && s.c_n == 1 && s.c_m == s.N && (s.batch == 1 || s.c_b == s.M * s.N) && !s.c_msplit && !s.c_nsplit;
 }
 
 bool gemm_shaped(const NestKernel& k, const GenOptions& opt) {
@@ -381,6 +402,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_A_BS " << s->a_b << "LL\n#define EH_B_BS " << s->b_b << "LL\n#define EH_C_BS " << s->c_b << "LL\n";
   os << "#define EH_A_MSPLIT " << s->a_msplit << "LL\n#define EH_A_SM2 " << s->a_m2 << "LL\n";
   os << "#define EH_B_NSPLIT " << s->b_nsplit << "LL\n#define EH_B_SN2 " << s->b_n2 << "LL\n";
+  os << "#define EH_C_MSPLIT " << s->c_msplit << "LL\n#define EH_C_SM2 " << s->c_m2 << "LL\n";
+  os << "#define EH_C_NSPLIT " << s->c_nsplit << "LL\n#define EH_C_SN2 " << s->c_n2 << "LL\n";
   os << "#define EH_SPLITK " << S << "\n";
   os << "#define EH_GROUP_M 8\n";
   // A computed operand's element (row r, k) sits at off + bz*bs + r*sr + k*sk of the producer's
@@ -474,14 +497,15 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +
                 (fa ? "/folded" : a_vec ? "" : "/scalar") + (b_nc ? ",B:n" : ",B:k") +
                 (fb ? "/folded" : b_vec ? "" : "/scalar") +
-                plain_tag + dma_tag + (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
+                plain_tag + dma_tag + (s->c_msplit || s->c_nsplit ? ",C:split" : "") + (ragged ? ",edges" : "") + (S > 1 ? ",split-k=" + std::to_string(S) : "") +
                 (epi_here ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(ceil_div(s->M, t.bm) * ceil_div(s->N, t.bn));
   ls.grid[1] = static_cast<unsigned>(S);
   ls.grid[2] = static_cast<unsigned>(s->batch);
   ls.block[0] = static_cast<unsigned>(nt);
   const size_t c_elems =
-      static_cast<size_t>(s->c_off + (s->M - 1) * s->c_m + (s->N - 1) * s->c_n + (s->batch - 1) * s->c_b + 1);
+      static_cast<size_t>(s->c_off + row_reach(s->M, s->c_m, s->c_msplit, s->c_m2) + row_reach(s->N, s->c_n, s->c_nsplit, s->c_n2) +
+                          (s->batch - 1) * s->c_b + 1);
   const size_t part_elems = static_cast<size_t>(S) * static_cast<size_t>(s->batch * s->M * s->N);
   ls.arg_bufs = {fa ? fa->src : s->a_buf, fb ? fb->src : s->b_buf};
   // a folded operand binds the producer's source, whose size the buffer table already fixes
@@ -550,12 +574,19 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     fs << "  float acc = 0.0f;\n  for (int s = 0; s < " << S << "; ++s) acc += P[(long long)s * " << total << "LL + o];\n";
     fs << "  const long long n = o % " << s->N << "LL, m = (o / " << s->N << "LL) % " << s->M << "LL, b = o / "
        << (s->M * s->N) << "LL;\n";
+    auto axis = [](const char* v, int64_t stride, int64_t split, int64_t outer) {
+      std::ostringstream a;
+      if (split) a << "(" << v << " / " << split << "LL) * " << outer << "LL + (" << v << " % " << split << "LL) * " << stride << "LL";
+      else a << v << " * " << stride << "LL";
+      return a.str();
+    };
+    fs << "  const long long e = " << s->c_off << "LL + b * " << s->c_b << "LL + " << axis("m", s->c_m, s->c_msplit, s->c_m2) << " + "
+       << axis("n", s->c_n, s->c_nsplit, s->c_n2) << ";\n";
     if (epilogue) {
       // the epilogue takes the address of the element in C's layout
-      fs << "  eh_epilogue(" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n
-         << "LL, acc" << (epilogue->store_c ? ", C" : "") << epilogue->args << ");\n}\n";
+      fs << "  eh_epilogue(e, acc" << (epilogue->store_c ? ", C" : "") << epilogue->args << ");\n}\n";
     } else {
-      fs << "  C[" << s->c_off << "LL + b * " << s->c_b << "LL + m * " << s->c_m << "LL + n * " << s->c_n << "LL] = acc;\n}\n";
+      fs << "  C[e] = acc;\n}\n";
     }
     fin.source = fs.str();
   }

@@ -23,6 +23,9 @@ struct GemmShape {
   // a row axis that runs over two nested extents of the memory it reads: rows per inner extent
   // (0: one stride) and the stride between inner extents
   int64_t a_msplit = 0, a_m2 = 0, b_nsplit = 0, b_n2 = 0;
+  // the same for C: rows (columns) the operand walks as one axis while the output keeps them in
+  // two nested extents (images x pixels written as NCHW)
+  int64_t c_msplit = 0, c_m2 = 0, c_nsplit = 0, c_n2 = 0;
 };
 
 // An elementwise producer (im2col gather, layout copy, padding ...) whose dense output a

@@ -84,6 +84,12 @@
 #define EH_B_NSPLIT 0
 #define EH_B_SN2 0
 #endif
+#ifndef EH_C_MSPLIT
+#define EH_C_MSPLIT 0     // rows of C per inner extent when its row axis is split in memory; likewise its columns
+#define EH_C_SM2 0
+#define EH_C_NSPLIT 0
+#define EH_C_SN2 0
+#endif
 #ifndef EH_PREFETCH
 #define EH_PREFETCH 1     // how many tile steps ahead of their use the global loads are issued
 #endif
@@ -352,6 +358,13 @@ __device__ __forceinline__ eh_f4v eh_quad_transpose(const eh_f4v& v, int t) {
 #define EH_C_ARG , C
 #endif
 
+// offset of position v along an axis of stride S, or of SPLIT positions of stride S inside extents S2 apart
+template <long long SPLIT, long long S, long long S2>
+__device__ __forceinline__ long long eh_axis_offset(long long v) {
+  constexpr long long D = SPLIT > 0 ? SPLIT : 1;
+  return SPLIT > 0 ? (v / D) * S2 + (v % D) * S : v * S;
+}
+
 #ifndef EH_WAVES_PER_SIMD
 #define EH_WAVES_PER_SIMD 4   // register budget: 512 / this many VGPRs+AGPRs per lane
 #endif
@@ -402,7 +415,6 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
 #else
   const long long kbeg = 0, kend = K;
   float* Cb = C + EH_C_OFF + bz * EH_C_BS;
-  constexpr long long CSM = EH_C_SM, CSN = EH_C_SN;
 #endif
 
   // Register stages of tiles on their way from global memory to LDS.  One stage: the tile of the
@@ -628,10 +640,17 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
         const long long row = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * kh + (r % 4);
         const long long col = n0 + wn * WN + j * 32 + l32;
         if ((!EDGE_M || row < M) && (!EDGE_N || col < N)) {
-#if defined(EH_EPILOGUE) && EH_SPLITK == 1
-          eh_epilogue(EH_C_OFF + bz * EH_C_BS + row * EH_C_SM + col * EH_C_SN, acc[i][j][r] EH_C_ARG EH_EPI_ARGS);
-#else
+#if EH_SPLITK > 1
           Cb[row * CSM + col * CSN] = acc[i][j][r];
+#else
+          // an axis of C may run over two nested extents (pixels inside images)
+          const long long crow = eh_axis_offset<EH_C_MSPLIT, EH_C_SM, EH_C_SM2>(row);
+          const long long ccol = eh_axis_offset<EH_C_NSPLIT, EH_C_SN, EH_C_SN2>(col);
+#if defined(EH_EPILOGUE)
+          eh_epilogue(EH_C_OFF + bz * EH_C_BS + crow + ccol, acc[i][j][r] EH_C_ARG EH_EPI_ARGS);
+#else
+          Cb[crow + ccol] = acc[i][j][r];
+#endif
 #endif
         }
       }

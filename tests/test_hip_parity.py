@@ -855,6 +855,36 @@ def test_contraction_variants_on_mfma(frontend, hip, kind, shapes, options, expe
     assert np.all(np.abs(got - exact.ravel()) <= 1e-5 * scale.ravel() + 1e-30)
 
 
+@pytest.mark.parametrize("shapes,options,expect", [
+    ([(5, 50, 36), (20, 36), (20,)], None, "C:split"),
+    ([(3, 50, 2048), (24, 2048), (24,)], None, "split-k="),
+    ([(3, 50, 2048), (24, 2048), (24,)], {"gemm_split_k": 4}, "split-k=4"),
+    ([(4, 196, 72), (64, 72), (64,)], None, "C:split"),
+])
+def test_contraction_rows_across_groups_into_a_permuted_result(frontend, hip, shapes, options, expect):
+    """x [G,R,K] . w [O,K] written as [G,O,R] with a bias per O (a convolution's NCHW output): R
+    is no multiple of the tile, so (G,R) is one row axis of the contraction and only the
+    result's address keeps the two extents; with K split the summing launch computes that
+    address.  Against the C oracle and float64 numpy."""
+    rng = RNG(sum(sum(s) for s in shapes))
+    arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
+
+    def fn(x, w, b):
+        y = (x.unsqueeze(2) * w.unsqueeze(0).unsqueeze(0)).sum(3)
+        return y.permute([0, 2, 1]).contiguous() + b.unsqueeze(0).unsqueeze(2)
+
+    got, scheds = _run_program(frontend, hip, fn, arrays, options)
+    assert any(s.startswith("mfma32x32x2(") and "C:split" in s and expect in s for s in scheds), scheds
+    assert len(scheds) == (2 if "split-k" in expect else 1), scheds
+    ref = realize_on(frontend, "c", fn, arrays)
+    a64 = [a.astype(np.float64) for a in arrays]
+    exact = np.einsum("grk,ok->gor", a64[0], a64[1]) + a64[2][None, :, None]
+    scale = np.einsum("grk,ok->gor", np.abs(a64[0]), np.abs(a64[1])) + np.abs(a64[2])[None, :, None]
+    assert got.shape == ref.shape == (exact.size,)
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale.ravel() + 1e-30)
+    assert np.all(np.abs(got - exact.ravel()) <= 1e-5 * scale.ravel() + 1e-30)
+
+
 def test_config5_with_implicit_gemm_loader(frontend, hip):
     """im2col gathers and layout copies that only contractions read are evaluated inside the
     contractions' tile loaders (no launch, no buffer); option gemm_fold=0 materialises them.

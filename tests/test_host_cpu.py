@@ -646,6 +646,26 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert len(direct) == 2 and all("A:k,B:n/folded" in l["schedule"] for l in direct), [l["schedule"] for l in plan.launches]
 
 
+def test_convolution_rows_run_across_images(frontend):
+    """196 pixels an image are no multiple of a 64-wide tile: the second convolution's forward
+    contraction takes (image, pixel) as one axis (784 tiles for 256 images, none padded per
+    image, where one image at a time would need 1024) and only the result's NCHW address keeps
+    the two extents.  The first convolution's weight gradient, 32 channels by 9 taps per image,
+    takes the one-wave tile."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config5_inputs(*wl.cnn_sizes(True))
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
+    plan = hb.render_program(ast, "lanes=1")
+    (fwd,) = [l for l in plan.launches if l["entry"] == "ehk_R_256_196_64_1_9"]
+    assert "C:split" in fwd["schedule"] and "edges" not in fwd["schedule"], fwd["schedule"]
+    assert fwd["grid"] == [256 * 196 // 64, 1, 1]
+    assert "#define EH_C_NSPLIT 196LL" in fwd["source"] and "#define EH_C_SN2 12544LL" in fwd["source"]
+    small = [l for l in plan.launches if "tile=32x32x16" in l["schedule"]]
+    assert [l["entry"] for l in small] == ["ehk_R_256_1_32_9_79_part"], [l["schedule"] for l in plan.launches]
+
+
 def _value_and_its_row_sums(x, m):
     """x*m + x as one root and the row sums of the same expression, written out again, as another."""
     return [x * m + x, (x * m + x).sum(1)]
