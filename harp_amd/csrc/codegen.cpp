@@ -2695,6 +2695,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             epi.store_c = needed(k0.out_buf);
             if (!epi.store_c) plan.elided.insert(k0.out_buf);
             const std::string IT = small ? "int" : "long long";
+            const std::string UT = small ? "unsigned" : "unsigned long long";
             body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
             body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
             if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
@@ -2704,7 +2705,8 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
               for (size_t li = 0; li < sk.loops.size(); ++li) {
                 const Loop& l = sk.loops[li];
                 if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
-                else body << "    const " << IT << " " << l.var << " = (" << from << " / " << strides[li] << ") % " << l.extent << ";\n";
+                else body << "    const " << IT << " " << l.var << " = (" << IT << ")(((" << UT << ")" << from << " / " << strides[li] << "u) % "
+                          << l.extent << "u);\n";    // (never negative: the unsigned division is the cheaper one)
               }
             };
             if (c_relaid && relaid_pos > 0) {

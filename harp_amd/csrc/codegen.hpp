@@ -28,7 +28,7 @@ struct GenOptions {
   int gemm_bm = 0, gemm_bn = 0, gemm_bk = 0, gemm_wm = 0, gemm_wn = 0;  // 0 = defaults
   int gemm_setprio = 0;               // wave priority during the multiply loop
   int gemm_waves = 0;                 // waves per SIMD the register allocation aims at (0 = from the tile)
-  int lanes = 2;                      // streams a program's launches may be spread over (1 = one after the other)
+  int lanes = 1;                      // streams a program's launches may be spread over (1 = one after the other)
   int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
   bool reindex = true;                // elementwise producers evaluated in a reader that walks another index space
   bool guard_branches = false;        // guarded loads (padding, edges) behind branches instead of clamped indices and selects

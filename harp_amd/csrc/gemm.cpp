@@ -445,20 +445,24 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
         use << "  const " << IT << " " << l.name << " = 0;\n";
       } else if (l.stride >= Q) {
         up << "  " << IT << " " << l.name << ";\n";
-        dup << "  r." << l.name << " = (eh_U / " << l.stride / Q << ") % " << l.extent << ";\n";
+        dup << "  r." << l.name << " = (" << IT << ")((eh_U / " << l.stride / Q << "u) % " << l.extent << "u);\n";
         use << "  const " << IT << " " << l.name << " = eh_u." << l.name << ";\n";
       } else {
         lo << "  " << IT << " " << l.name << ";\n";
-        dlo << "  r." << l.name << " = (eh_I / " << l.stride << ") % " << l.extent << ";\n";
+        dlo << "  r." << l.name << " = (" << IT << ")((eh_I / " << l.stride << "u) % " << l.extent << "u);\n";
         use << "  const " << IT << " " << l.name << " = eh_l." << l.name << ";\n";
       }
+      // the guards of a padded gather repeat what the loops' extents already say: let the compiler drop those
+      if (l.extent > 1) use << "  __builtin_assume(" << l.name << " >= 0 && " << l.name << " < " << l.extent << ");\n";
     }
     os << "// element (eh_U * " << Q << " + eh_I) of what kernel " << f->kernel << " would have written\n";
     os << "struct " << P << "_upper {\n" << up.str() << "};\nstruct " << P << "_lower {\n" << lo.str() << "};\n";
-    os << "__device__ __forceinline__ " << P << "_upper " << P << "_dec_upper(long long eh_U64) {\n  const " << IT << " eh_U = ("
-       << IT << ")eh_U64;\n  (void)eh_U;\n  " << P << "_upper r;\n" << dup.str() << "  return r;\n}\n";
-    os << "__device__ __forceinline__ " << P << "_lower " << P << "_dec_lower(long long eh_I64) {\n  const " << IT << " eh_I = ("
-       << IT << ")eh_I64;\n  (void)eh_I;\n  " << P << "_lower r;\n" << dlo.str() << "  return r;\n}\n";
+    // (indices are never negative: unsigned division by a constant is the cheaper one)
+    const std::string UT = f->small ? "unsigned" : "unsigned long long";
+    os << "__device__ __forceinline__ " << P << "_upper " << P << "_dec_upper(long long eh_U64) {\n  const " << UT << " eh_U = ("
+       << UT << ")eh_U64;\n  (void)eh_U;\n  " << P << "_upper r;\n" << dup.str() << "  return r;\n}\n";
+    os << "__device__ __forceinline__ " << P << "_lower " << P << "_dec_lower(long long eh_I64) {\n  const " << UT << " eh_I = ("
+       << UT << ")eh_I64;\n  (void)eh_I;\n  " << P << "_lower r;\n" << dlo.str() << "  return r;\n}\n";
     os << "__device__ __forceinline__ float " << P << "_val(const float* __restrict__ " << f->src << ", const " << P
        << "_upper& eh_u, const " << P << "_lower& eh_l) {\n  (void)eh_u;\n  (void)eh_l;\n" << use.str();
     os << "  return (float)(" << f->expr << ");\n}\n";

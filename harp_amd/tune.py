@@ -116,11 +116,11 @@ def suggest_pipeline(state: Dict[str, int], schedules: Sequence[str]) -> Iterabl
             if p != state.get("gemm_prefetch", 0):
                 yield {**state, "gemm_prefetch": p}
         for d in (0, 1):
-            if d != state.get("gemm_dma", 0):
+            if d != state.get("gemm_dma", 2):
                 yield {**state, "gemm_dma": d}
     if len(schedules) >= 8:
         for n in (1, 2, 3):
-            if n != state.get("lanes", 2):
+            if n != state.get("lanes", 1):
                 yield {**state, "lanes": n}
 
 

@@ -91,10 +91,10 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold,
  *      gemm_epilogue, gemm_dma, gemm_mix, gemm_prefetch, gemm_transpose, gemm_merge_batch, nontemporal,
  *      normalize, allow_serial, reindex, guard_branches, lanes, lane_us.
- *      lanes (default 2): launches of a program that do not depend on each other may be spread
+ *      lanes (default 1; 2 or more): launches of a program that do not depend on each other are spread
  *      over that many streams (lane 0 is the device's stream; a program's execute forks the side
  *      lanes off it and joins them back, so callers still see one stream); launches estimated
- *      above lane_us microseconds (default 100) stay on lane 0.  lanes=1: one after the other.
+ *      above lane_us microseconds (default 100) stay on lane 0.
  *      A kernel that no schedule recognises, would run in a single work-item and loops more than
  *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1. ----------------- */
 typedef struct eh_launch_info {

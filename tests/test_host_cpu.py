@@ -562,7 +562,7 @@ def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
     """The CNN training step: independent launches (the gradients of the parameters beside the
     chain that carries the gradient back) go to a side lane.  Producers come before consumers in
     the issue order, every buffer has its writer marked, and every cross-lane dependence is
-    covered by a wait; with lanes=1 the plan is the same set of launches on lane 0."""
+    covered by a wait; with lanes=1 (the default) the plan is the same set of launches on lane 0."""
     from harp_amd import backend as hb
     from harp_amd import workloads as wl
     from harp_amd.frontend import Tensor
@@ -586,8 +586,10 @@ def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
     one = hb.render_program(prog_ast, "lanes=1")
     assert all(l["lane"] == 0 and not l["waits"] for l in one.launches)
     assert sorted(l["entry"] for l in one.launches) == sorted(l["entry"] for l in plan.launches)
-    default = hb.render_program(prog_ast)
-    assert _lane_plan_is_sound(default.launches) == 2
+    two = hb.render_program(prog_ast, "lanes=2")
+    assert _lane_plan_is_sound(two.launches) == 2
+    default = hb.render_program(prog_ast)                  # one lane unless asked (or tuned) otherwise
+    assert [l["entry"] for l in default.launches] == [l["entry"] for l in one.launches]
     # a single softmax has nothing to spread
     from harp_amd import workloads
     sm = hb.render_program(workloads.lower_with_table([(64, 256)], workloads.config2_graph)[0])
