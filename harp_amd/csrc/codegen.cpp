@@ -2984,24 +2984,29 @@ struct GroupEmitter {
   }
   static const std::vector<Loop>& loads_loops(const std::vector<Loop>& l) { return l; }
 
-  // 128-bit accesses need every vectorised access to start on a 4-element boundary.
-  bool aligned4(const Affine& a) const {
-    if (a.c % 4) return false;
+  // every vectorised access of `width` elements starts on a multiple of the width
+  bool aligned(const Affine& a, int width) const {
+    if (a.c % width) return false;
     for (const auto& kv : a.coef)
-      if (kv.first != "c" && kv.second % 4) return false;
+      if (kv.first != "c" && kv.second % width) return false;
+    return true;
+  }
+  bool vector_ok(int width) const {
+    if (!opt.vectorize || g.C % width) return false;
+    for (const auto& e : ext)
+      if (!aligned(e.aff, width) || e.dtype.itemsize() != 4) return false;
+    for (const auto& st : g.stages)
+      if (st.kind == StageKind::Wide && st.store &&
+          (st.out_aff.of("c") != 1 || !aligned(st.out_aff, width) || st.out_dtype.itemsize() != 4))
+        return false;
     return true;
   }
 
-  void choose_vector() {
-    V = 1;
-    if (!opt.vectorize || g.C % 4) return;
-    for (const auto& e : ext)
-      if (!aligned4(e.aff) || e.dtype.itemsize() != 4) return;
-    for (const auto& st : g.stages)
-      if (st.kind == StageKind::Wide && st.store &&
-          (st.out_aff.of("c") != 1 || !aligned4(st.out_aff) || st.out_dtype.itemsize() != 4))
-        return;
-    V = 4;
+  void choose_vector() { V = vector_ok(4) ? 4 : 1; }
+  // the flat schedule also takes pairs (a pooling window two wide: 64-bit accesses, one index
+  // decode and one read of everything that does not move along the pair per two elements)
+  void choose_vector_flat() {
+    if (V == 1 && vector_ok(2)) V = 2;
   }
 
   std::string affine_text(const Affine& a, const std::string& cvar) const {
@@ -3138,6 +3143,14 @@ struct GroupEmitter {
     ls.block[0] = static_cast<unsigned>(block);
     std::ostringstream os;
     os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    if (V == 2)
+      os << "template <typename T> using EhV2 = T __attribute__((ext_vector_type(2)));\n"
+            "template <bool NT, typename T> __device__ __forceinline__ EhV2<T> eh_load2(const T* p) {\n"
+            "  if (NT) return __builtin_nontemporal_load(reinterpret_cast<const EhV2<T>*>(p));\n"
+            "  return *reinterpret_cast<const EhV2<T>*>(p);\n}\n"
+            "template <bool NT, typename T> __device__ __forceinline__ void eh_store2(T* p, EhV2<T> v) {\n"
+            "  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<EhV2<T>*>(p));\n"
+            "  else *reinterpret_cast<EhV2<T>*>(p) = v;\n}\n";
     os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "("
        << params_text(&ls.arg_bufs) << ") {\n";
     os << "  const idx_t eh_nvec = " << NVEC << ";\n";
@@ -3152,19 +3165,23 @@ struct GroupEmitter {
     }
     // vector loads
     auto ld = [&](int id) -> std::string {
-      return V == 4 ? "ld" + std::to_string(id) + "[v]" : std::string();
+      return V > 1 ? "ld" + std::to_string(id) + "[v]" : std::string();
     };
     if (V == 4)
       for (const auto& e : ext)
         os << "  const EhV4<" << ctype(e.dtype) << "> ld" << e.id << " = eh_load4<" << nt << ">(" << e.buf << " + "
            << affine_text(e.aff, "c0") << ");\n";
+    if (V == 2)
+      for (const auto& e : ext)
+        os << "  const EhV2<" << ctype(e.dtype) << "> ld" << e.id << " = eh_load2<" << nt << ">(" << e.buf << " + "
+           << affine_text(e.aff, "c0") << ");\n";
     for (const auto& st : g.stages) {
       if (!st.store) continue;
       std::string T = ctype(st.out_dtype);
-      if (V == 4) {
-        os << "  { EhV4<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o[v] = ("
+      if (V > 1) {
+        os << "  { EhV" << V << "<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < " << V << "; ++v) { const idx_t c = c0 + v; o[v] = ("
            << T << ")(" << value_text(st, ld) << "); }\n";
-        os << "  eh_store4<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ", o); }\n";
+        os << "  eh_store" << V << "<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ", o); }\n";
       } else {
         os << "  { const idx_t c = c0; " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << T << ")("
            << value_text(st, ld) << "); }\n";
@@ -3483,7 +3500,9 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
     std::vector<GroupEmitter::TransposedLoad> tl;
     GroupEmitter::TransposePlan tp;
     if (opt.transpose) tp = ge.transposed_axes(&tl);
-    return tp.row_run.empty() ? ge.emit_flat(elems) : ge.emit_transposed(elems, tp, tl);
+    if (!tp.row_run.empty()) return ge.emit_transposed(elems, tp, tl);
+    ge.choose_vector_flat();
+    return ge.emit_flat(elems);
   }
   return ge.emit_rows(elems);
 }
