@@ -55,13 +55,14 @@ class Plan:
             info = LaunchInfo()
             check(lib.eh_plan_launch(self._h, i, byref(info)))
             d = _launch_dict(info)
-            d["args"], d["kernels"], d["written"], d["waits"] = [], [], [], []
+            d["args"], d["kernels"], d["written"], d["overwrites"], d["waits"] = [], [], [], [], []
             s, v = c_char_p(), c_int()
             for a in range(info.n_args):
                 check(lib.eh_plan_launch_arg(self._h, i, a, byref(s)))
                 d["args"].append(s.value.decode())
                 check(lib.eh_plan_launch_arg_written(self._h, i, a, byref(v)))
                 d["written"].append(bool(v.value))
+                d["overwrites"].append(v.value == 2)      # every element of an exactly-sized buffer
             for w in range(info.n_waits):
                 check(lib.eh_plan_launch_wait(self._h, i, w, byref(v)))
                 d["waits"].append(v.value)

@@ -5,6 +5,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -318,11 +319,15 @@ HipBuffer::HipBuffer(HipDevice* dev, size_t bytes) : dev_(dev), bytes_(bytes) {
   dev_->make_current();
   if (bytes_ == 0) return;
   ptr_ = dev_->allocate(bytes_);
-  hipError_t e = hipMemsetAsync(ptr_, 0, bytes_, dev_->stream());
-  if (e != hipSuccess) {
-    dev_->release(ptr_, bytes_);
-    check(e, "hipMemsetAsync");
-  }
+  zero_pending_ = true;
+}
+
+void HipBuffer::settle() {
+  auto lk = dev_->stream_lock();
+  if (!zero_pending_) return;
+  dev_->make_current();
+  check(hipMemsetAsync(ptr_, 0, bytes_, dev_->stream()), "hipMemsetAsync");
+  zero_pending_ = false;
 }
 
 HipBuffer::~HipBuffer() {
@@ -340,6 +345,7 @@ void HipBuffer::write_from_host(const void* src, size_t bytes) {
   dev_->make_current();
   check(hipMemcpyAsync(ptr_, src, bytes_, hipMemcpyHostToDevice, dev_->stream()), "hipMemcpyAsync(H2D)");
   check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
+  zero_pending_ = false;
 }
 
 void HipBuffer::read_to_host(void* dst, size_t bytes) const {
@@ -347,6 +353,10 @@ void HipBuffer::read_to_host(void* dst, size_t bytes) const {
     throw Error("Buffer size mismatch: expected " + std::to_string(bytes_) + ", got " + std::to_string(bytes));
   if (!bytes_) return;
   auto lk = dev_->stream_lock();
+  if (zero_pending_) {                         // never written: zeros, without touching the device
+    std::memset(dst, 0, bytes_);
+    return;
+  }
   dev_->make_current();
   check(hipMemcpyAsync(dst, ptr_, bytes_, hipMemcpyDeviceToHost, dev_->stream()), "hipMemcpyAsync(D2H)");
   check(hipStreamSynchronize(dev_->stream()), "hipStreamSynchronize");
@@ -358,7 +368,12 @@ void HipBuffer::copy_from(const HipBuffer& src) {
   if (!bytes_) return;
   auto lk = dev_->stream_lock();
   dev_->make_current();
-  check(hipMemcpyAsync(ptr_, src.ptr_, bytes_, hipMemcpyDeviceToDevice, dev_->stream()), "hipMemcpyAsync(D2D)");
+  if (src.zero_pending_) {                     // a copy of zeros
+    check(hipMemsetAsync(ptr_, 0, bytes_, dev_->stream()), "hipMemsetAsync");
+  } else {
+    check(hipMemcpyAsync(ptr_, src.ptr_, bytes_, hipMemcpyDeviceToDevice, dev_->stream()), "hipMemcpyAsync(D2D)");
+  }
+  zero_pending_ = false;
 }
 
 HipKernel::HipKernel(HipDevice* dev, const Binary& bin, const std::string& entry)
@@ -511,9 +526,19 @@ HipProgram::HipProgram(HipDevice* dev, const std::string& ast_text, const GenOpt
   dump_plan(plan_);
   for (size_t i = 0; i < plan_.buffers.size(); ++i) index_[plan_.buffers[i].name] = i;
   temps_.assign(plan_.buffers.size(), nullptr);
+  first_full_.assign(plan_.buffers.size(), 0);
+  std::vector<char> touched(plan_.buffers.size(), 0);
   for (const auto& ls : plan_.launches) {
     for (const auto& a : ls.arg_bufs)
       if (!index_.count(a)) throw Error("launch '" + ls.entry + "' binds unknown buffer '" + a + "'");
+    // (a buffer bound to two parameters of its first launch may be read there: no shortcut)
+    for (size_t a = 0; a < ls.arg_bufs.size(); ++a) {
+      const size_t i = index_.at(ls.arg_bufs[a]);
+      const bool whole = a < ls.arg_written.size() && ls.arg_written[a] && a < ls.arg_full_bytes.size() &&
+                         std::count(ls.arg_bufs.begin(), ls.arg_bufs.end(), ls.arg_bufs[a]) == 1;
+      if (!touched[i] && whole) first_full_[i] = ls.arg_full_bytes[a];
+    }
+    for (const auto& a : ls.arg_bufs) touched[index_.at(a)] = 1;
     Binary bin = HipCompiler::compile(ls.source, o.arch);
     try {
       kernels_.push_back(dev_->load(bin, ls.entry));
@@ -538,7 +563,7 @@ HipProgram::~HipProgram() {
     if (b && b->release()) delete b;
 }
 
-std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n) {
+std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n, std::vector<HipBuffer*>* cancelled) {
   // the caller's table comes first; scratch temps the plan appended may be left out
   const size_t total = plan_.buffers.size();
   bool enough = n <= total;
@@ -564,6 +589,19 @@ std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n) {
                     std::to_string(b->byte_len()));
     }
     bound[i] = b;
+  }
+  // zero fills still owed: cancelled where the program overwrites the whole buffer before it
+  // reads it (and the caller can take the debt back), queued now otherwise
+  for (size_t i = 0; i < total; ++i) {
+    HipBuffer* b = bound[i];
+    if (!b || !b->zero_pending()) continue;
+    if (cancelled && first_full_[i] != 0 && first_full_[i] == b->byte_len() &&
+        std::count(bound.begin(), bound.end(), b) == 1) {
+      b->set_zero_pending(false);
+      cancelled->push_back(b);
+    } else {
+      b->settle();
+    }
   }
   return bound;
 }
@@ -637,7 +675,14 @@ void HipProgram::launch_spans(const std::vector<Span>& bound) {
 void HipProgram::execute(HipBuffer* const* bufs, size_t n, bool sync) {
   std::lock_guard<std::mutex> lk(mu_);
   auto sl = dev_->stream_lock();               // binding may allocate (and fill) temps
-  launch_all(bind(bufs, n));
+  std::vector<HipBuffer*> cancelled;
+  try {
+    launch_all(bind(bufs, n, &cancelled));
+  } catch (...) {
+    // some launch was not queued: what it would have overwritten is owed its zeros again
+    for (HipBuffer* b : cancelled) b->set_zero_pending(true);
+    throw;
+  }
   if (sync) dev_->synchronize();
 }
 
@@ -683,6 +728,7 @@ void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
     if (bi.shape_known && b->byte_len() < bi.bytes())
       throw Error("Buffer size mismatch: '" + bi.name + "' needs " + std::to_string(bi.bytes()) + " bytes, has " +
                   std::to_string(b->byte_len()));
+    b->settle();                                 // (queues a fill at most; allocates nothing)
     bound[i] = {b->device_ptr(), b->byte_len(), true};
   }
   launch_spans(bound);
@@ -700,7 +746,7 @@ HipGraph::HipGraph(HipProgram* prog, HipBuffer* const* bufs, size_t n) : dev_(pr
   auto sl = dev_->stream_lock();
   // binding allocates missing temps: all of it happens before the capture starts, the capture
   // itself records kernel launches only (no memset or copy nodes)
-  std::vector<HipBuffer*> bound = prog->bind(bufs, n);
+  std::vector<HipBuffer*> bound = prog->bind(bufs, n, nullptr);
   launches_ = prog->plan().launches.size();
   kernels_ = prog->kernels_;
   // the program's own temps are shared with it by reference count; the caller's buffers are kept

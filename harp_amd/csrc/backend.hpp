@@ -102,13 +102,20 @@ class HipDevice {
 
 class HipBuffer {
  public:
-  HipBuffer(HipDevice* dev, size_t bytes);   // zero-filled, as the reference's buffers are
+  // Reads as zeros until something is written, as the reference's buffers do.  The fill itself
+  // is put off until something needs the memory's contents: a kernel that overwrites the whole
+  // buffer (the usual fate of an output the executor has just allocated) or a full write from
+  // the host cancels it.
+  HipBuffer(HipDevice* dev, size_t bytes);
   ~HipBuffer();
   HipBuffer(const HipBuffer&) = delete;
   HipBuffer& operator=(const HipBuffer&) = delete;
 
   size_t byte_len() const { return bytes_; }
-  void* device_ptr() const { return ptr_; }
+  void* device_ptr() const { return ptr_; }       // the memory as it is: settle() first unless it is about to be overwritten
+  bool zero_pending() const { return zero_pending_; }
+  void settle();                                   // queues the fill if it is still owed
+  void set_zero_pending(bool owed) { zero_pending_ = owed && ptr_; }   // (under the device's stream lock)
   HipDevice* device() const { return dev_; }
   void write_from_host(const void* src, size_t bytes);   // size must match exactly
   void read_to_host(void* dst, size_t bytes) const;
@@ -120,6 +127,7 @@ class HipBuffer {
   HipDevice* dev_;
   void* ptr_ = nullptr;
   size_t bytes_;
+  bool zero_pending_ = false;                      // guarded by the device's stream lock
   std::atomic<int> refs_{1};
 };
 
@@ -165,7 +173,10 @@ class HipProgram {
 
  private:
   friend class HipGraph;
-  std::vector<HipBuffer*> bind(HipBuffer* const* bufs, size_t n);   // checks sizes, allocates missing temps
+  // checks sizes, allocates missing temps; a buffer still owed its zero fill gets it now, unless
+  // the first launch that touches it overwrites all of it (`cancelled` then lists it, so that a
+  // failed execute can put the debt back)
+  std::vector<HipBuffer*> bind(HipBuffer* const* bufs, size_t n, std::vector<HipBuffer*>* cancelled);
   void launch_all(const std::vector<HipBuffer*>& bound);            // queues every launch on the stream
   struct Span {
     void* ptr = nullptr;
@@ -177,6 +188,7 @@ class HipProgram {
   ProgramPlan plan_;
   std::vector<std::shared_ptr<HipKernel>> kernels_;
   std::map<std::string, size_t> index_;          // buffer name -> table index
+  std::vector<size_t> first_full_;               // by table index: size of the buffer the first launch that binds it overwrites whole (0: none)
   std::vector<HipBuffer*> temps_;                // owned, by table index (nullptr if unused)
   // Lanes (plan().lanes > 1): events_[l] is recorded behind launch l when a launch on another
   // lane waits for it; fork_ is recorded on the device's stream before the first launch and

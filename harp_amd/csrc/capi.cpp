@@ -207,8 +207,10 @@ int eh_buffer_copy(eh_buffer* dst, eh_buffer* src) {
 
 int eh_buffer_device_ptr(eh_buffer* buf, void** ptr) {
   REQUIRE(buf && ptr, "buffer or ptr is NULL");
-  *ptr = buf->buf.device_ptr();
-  return EH_OK;
+  return guard([&] {
+    buf->buf.settle();               // the caller may read through the pointer
+    *ptr = buf->buf.device_ptr();
+  });
 }
 
 int eh_tune_key(const char* ast_text, unsigned long long* key) {
@@ -285,7 +287,9 @@ int eh_plan_launch_arg_written(eh_plan* plan, int launch, int arg, int* written)
   REQUIRE(launch >= 0 && launch < static_cast<int>(plan->plan.launches.size()), "launch index out of range");
   const auto& a = plan->plan.launches[static_cast<size_t>(launch)].arg_written;
   REQUIRE(arg >= 0 && arg < static_cast<int>(a.size()), "argument index out of range");
-  *written = a[static_cast<size_t>(arg)] ? 1 : 0;
+  const auto& f = plan->plan.launches[static_cast<size_t>(launch)].arg_full_bytes;
+  const bool whole = static_cast<size_t>(arg) < f.size() && f[static_cast<size_t>(arg)] != 0;
+  *written = a[static_cast<size_t>(arg)] ? (whole ? 2 : 1) : 0;
   return EH_OK;
 }
 
@@ -468,9 +472,12 @@ int eh_module_launch(eh_module* mod, const unsigned grid[3], const unsigned bloc
     for (int i = 0; i < n_args; ++i) {
       if (!args[i]) throw Error("argument " + std::to_string(i) + " is NULL");
       if (args[i]->buf.device() != mod->dev) throw Error("argument " + std::to_string(i) + " lives on another device");
-      ptrs.push_back(args[i]->buf.device_ptr());
     }
     auto lk = mod->dev->stream_lock();
+    for (int i = 0; i < n_args; ++i) {
+      args[i]->buf.settle();         // nothing is known about what the code object reads
+      ptrs.push_back(args[i]->buf.device_ptr());
+    }
     mod->dev->make_current();
     mod->kernel->launch(grid, block, lds_bytes, ptrs);
     if (sync) mod->dev->synchronize();

@@ -2859,6 +2859,26 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       for (const auto& a : ls.arg_bufs) bound = bound || a == c.first;
     if (!bound) plan.elided.insert(c.first);
   }
+  // A lowered kernel whose output index is the dense index of its loops writes every element of
+  // its output; the launch that stores it overwrites a buffer of exactly that size, whatever it
+  // held (the executor need not have zero-filled it first).
+  {
+    std::map<std::string, std::pair<std::string, size_t>> dense_out;     // kernel -> (buffer, bytes)
+    for (const auto& nk : nests) {
+      int64_t numel = 0;
+      if (nk && dense_strides(*nk, &numel))
+        dense_out[nk->name] = {nk->out_buf, static_cast<size_t>(numel) * nk->out_dtype.itemsize()};
+    }
+    for (auto& ls : plan.launches) {
+      ls.arg_full_bytes.assign(ls.arg_bufs.size(), 0);
+      for (const auto& kn : ls.kernels) {
+        auto it = dense_out.find(kn);
+        if (it == dense_out.end()) continue;
+        for (size_t a = 0; a < ls.arg_bufs.size(); ++a)
+          if (ls.arg_bufs[a] == it->second.first) ls.arg_full_bytes[a] = it->second.second;
+      }
+    }
+  }
   assign_lanes(&plan, kernels, opt);
   return plan;
 }

@@ -60,6 +60,7 @@ struct LaunchSpec {
   double flops = 0;
   // Filled in by plan_program once all launches are known:
   std::vector<char> arg_written;       // per parameter: the launch writes that buffer
+  std::vector<size_t> arg_full_bytes;  // per parameter: the launch writes every byte of a buffer of exactly this size (0: not known to)
   int lane = 0;                        // 0 = the device's stream, 1.. = side streams that run beside it
   std::vector<int> waits;              // launches on other lanes that must have finished first
 };

@@ -69,7 +69,11 @@ int eh_device_sync(eh_device* dev);     /* waits for everything queued on the de
  *      read_to_host, clone_buffer (src/backend/traits.rs:455-482;
  *      crates/backend-c/src/buffer.rs:84-131); BackendRegistry::allocate_buffer
  *      (src/backend/device.rs:132-134) -------------------------------------------------------- */
-/* Released buffers' memory is kept by the device (up to a quarter of its memory) and reused by
+/* A new buffer reads as zeros.  The fill is put off until the contents are needed (a kernel that
+ * reads the buffer or writes part of it, a copy out of it, eh_buffer_device_ptr) and dropped
+ * when a full write from the host or a launch that writes every element comes first: an output
+ * the executor allocates per kernel costs no fill.
+ * Released buffers' memory is kept by the device (up to a quarter of its memory) and reused by
  * later allocations of the same size, so the executor's allocate-per-kernel pattern
  * (src/backend/executor.rs:313-332) costs no hipMalloc/hipFree after the first pass.
  * eh_device_trim gives the kept blocks back to the driver; *kept_bytes (may be NULL) receives
@@ -133,8 +137,10 @@ int eh_plan_num_launches(eh_plan* plan, int* n);
 int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out);    /* strings live as long as the plan */
 int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name);
 int eh_plan_launch_kernel(eh_plan* plan, int launch, int k, const char** kernel_name);
-/* Whether the launch writes the buffer of parameter `arg`, and launch number `i` (of n_waits) on
- * another lane that must have finished before this one starts.  Launches are listed in the order
+/* Whether the launch writes the buffer of parameter `arg` (0 no, 1 yes, 2: every element of it,
+ * given a buffer of exactly the kernel's output size: such a buffer need not hold anything
+ * before), and launch number `i` (of n_waits) on another lane that must have finished before
+ * this one starts.  Launches are listed in the order
  * in which they are issued; every launch a launch depends on comes before it. */
 int eh_plan_launch_arg_written(eh_plan* plan, int launch, int arg, int* written);
 int eh_plan_launch_wait(eh_plan* plan, int launch, int i, int* waited_launch);

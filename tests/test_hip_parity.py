@@ -91,6 +91,23 @@ def test_elementwise_bit_exact(frontend, hip, shape, name, fuse):
     assert bits_equal_mod_zero(ref, got)
 
 
+@pytest.mark.parametrize("shapes", [[(33, 7, 2), (33, 7)], [(129, 5, 6), (129, 5)], [(1, 1, 2), (1, 1)], [(64, 14, 2, 14, 2), (64, 14, 2, 14)]])
+@pytest.mark.parametrize("fuse", [False, True])
+def test_elementwise_in_pairs_bit_exact(frontend, hip, shapes, fuse):
+    """A contiguous extent two (or six) wide next to an operand that does not move along it (a
+    pooling window put back over its image): the flat schedule works in pairs, 64-bit accesses
+    for what moves and one read for what does not.  Bit-exact against the oracle."""
+    rng = RNG(sum(sum(s) for s in shapes))
+    arrs = [rng.normal(0, 1, s).astype(np.float32) for s in shapes]
+    fn = lambda x, y: x * y.unsqueeze(len(shapes[0]) - 1) + x
+    if fuse:
+        from harp_amd import workloads as wl
+        plan = hip.render_program(wl.lower_with_table(shapes, fn)[0])
+        assert [l["schedule"] for l in plan.launches] == ["flat(V=2,block=256)"]
+    ref, got = both(frontend, fn, arrs, fuse)
+    assert bits_equal_mod_zero(ref, got)
+
+
 @pytest.mark.parametrize("op", ["sqrt", "recip", "exp", "ln", "sin", "cos", "exp2", "log2"])
 @pytest.mark.parametrize("fuse", [False, True])
 def test_transcendental_elementwise(frontend, hip, op, fuse):
@@ -567,6 +584,57 @@ def test_released_memory_is_reused_and_zero_filled(hip):
     assert c.device_ptr() != ptr
     del b, c
     assert dev.trim() == 2 * n and dev.trim() == 0
+
+
+def test_a_new_buffer_reads_as_zeros_whenever_its_fill_happens(frontend, hip):
+    """The zero fill of a new buffer is put off until its contents are needed.  On recycled
+    memory full of 0xAB: a kernel that writes every element cancels the fill (and is right), a
+    kernel that reads the buffer or writes only part of it gets zeros first, a read or a copy
+    before any write gives zeros, and an execute that fails before its launch leaves a buffer
+    that still reads as zeros."""
+    dev = hip.HipDevice(0)
+    F32 = frontend.F32
+    n = 64 * 64
+
+    def dirty(count=4):
+        bufs = [dev.alloc(4 * n) for _ in range(count)]
+        for b in bufs:
+            b.write_array(np.full(4 * n, 0xAB, np.uint8))
+        del bufs                                            # back to the pool, contents kept
+
+    a = frontend.Tensor.input([64, 64])
+    prog, _, _ = frontend.lower_graph([(a + a).graph])
+    k = hip.HipKernel(dev, prog)
+    assert [l["overwrites"] for l in hip.render_program(prog).launches] == [[False, True]]
+    x = hip.HipBuffer(dev, [64, 64], F32)
+    data = RNG(7).normal(0, 1, (64, 64)).astype(np.float32)
+    x.write_array(data)
+    dirty()
+    out = hip.HipBuffer(dev, [64, 64], F32)
+    k.execute([x], [out])                                   # overwrites all of `out`: no fill
+    assert np.array_equal(out.read_array(np.float32), (data + data).ravel())
+    dirty()
+    fresh = hip.HipBuffer(dev, [64, 64], F32)
+    out2 = hip.HipBuffer(dev, [64, 64], F32)
+    k.execute([fresh], [out2])                              # reads a buffer nothing wrote: zeros
+    assert not out2.read_array(np.float32).any() and not fresh.read_array(np.float32).any()
+    dirty()
+    never = hip.HipBuffer(dev, [64, 64], F32)
+    assert not never.read_array(np.float32).any()           # read before any write
+    assert not never.clone_buffer().read_array(np.float32).any()
+    dirty()
+    big = hip.HipBuffer(dev, [2 * n], F32)                  # larger than the kernel's output: only half is written
+    k.execute([x], [big])
+    got = big.read_array(np.float32)
+    assert np.array_equal(got[:n], (data + data).ravel()) and not got[n:].any()
+    dirty()
+    out3 = hip.HipBuffer(dev, [64, 64], F32)
+    with pytest.raises(hip.EhError):
+        k.execute([hip.HipBuffer(dev, [16], F32)], [out3])  # refused before the launch
+    assert not out3.read_array(np.float32).any()
+    dirty()
+    handed_out = hip.HipBuffer(dev, [64, 64], F32)          # asking for the address queues the fill
+    assert handed_out.device_ptr() and not handed_out.read_array(np.float32).any()
 
 
 def test_undersized_buffer_is_rejected_before_launch(frontend, hip):
