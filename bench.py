@@ -37,7 +37,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak (default: all but the last two)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak | mfma_valu (default: all but the last three)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-kernel", action="store_true", help="skip the per-kernel (unfused, synchronous) path")
     ap.add_argument("--no-check", action="store_true")
@@ -71,6 +71,13 @@ def main():
         tflops, blocks, ms = measure.mfma_issue_rate(dev)
         log(f"[bench] MFMA f32 32x32x2 issue-rate ceiling: {tflops:.1f} TFLOP/s ({tflops / FP32_MFMA_PEAK_TFLOPS:.1%} of "
             f"the published {FP32_MFMA_PEAK_TFLOPS}); {blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
+        return
+
+    if args.only == "mfma_valu":
+        r = measure.mfma_valu_overlap(dev)
+        log("[bench] one SIMD, MFMAs and as many cycles of ordinary vector instructions: "
+            f"MFMAs alone {r['mfma_only']:.0f} us, vector instructions alone {r['valu_only']:.0f} us, both in every wave "
+            f"{r['both_in_each_wave']:.0f} us, one wave of each {r['one_wave_of_each_per_simd']:.0f} us")
         return
 
     def roofline(bound, achieved, unit, algo, launch=None):

@@ -214,6 +214,60 @@ def mfma_issue_rate(dev, iters=4096, waves_per_cu=8, reps=20):
     return flops / ms / 1e9, blocks, ms
 
 
+MFMA_VALU_SOURCE = """
+typedef float f16v __attribute__((ext_vector_type(16)));
+// MODE 0: every wave multiplies; 1: every wave runs ordinary vector instructions; 2: every wave
+// does both in turn; 3: waves 0-3 multiply, waves 4-7 run vector instructions (one of each per SIMD)
+extern "C" __global__ void __launch_bounds__(512) eh_mfma_valu(float* out) {
+  const int wave = threadIdx.x >> 6;
+  f16v acc[4];
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+  float a = threadIdx.x * 1e-3f, b = blockIdx.x * 1e-3f;
+  float v[8];
+  for (int i = 0; i < 8; ++i) v[i] = a + i;
+  const bool mfma = %(mode)d == 0 || %(mode)d == 2 || (%(mode)d == 3 && wave < 4);
+  const bool valu = %(mode)d == 1 || %(mode)d == 2 || (%(mode)d == 3 && wave >= 4);
+  for (int it = 0; it < %(iters)d; ++it) {
+    if (mfma) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+    }
+    if (valu) {                          // 64 fused multiply-adds: as many cycles as the four MFMAs
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(v[i], 1.0001f, 0.5f);
+    }
+  }
+  float s = 0.0f;
+  for (int i = 0; i < 8; ++i) s += v[i];
+  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += acc[i][r];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+"""
+
+
+def mfma_valu_overlap(dev, iters=20000):
+    """Whether a SIMD runs one wave's MFMAs beside ordinary vector instructions (its own or another
+    wave's).  Returns microseconds for: MFMAs only and vector instructions only (one wave per
+    SIMD each), both in every wave, and one wave of each kind per SIMD.  If the last two equal the
+    sum of the first two, nothing overlaps."""
+    cus = dev.props["compute_units"]
+    out = hb.HipBuffer(dev, [cus * 512 * 4], None, nbytes=cus * 512 * 4)
+
+    def run(mode, waves):
+        mod = hb.HipModule(dev, hb.compile_source(MFMA_VALU_SOURCE % {"mode": mode, "iters": iters}), "eh_mfma_valu")
+        mod.launch([cus, 1, 1], [waves * 64, 1, 1], [out], sync=True)
+        e0, e1 = hb.Event(dev), hb.Event(dev)
+        e0.record()
+        mod.launch([cus, 1, 1], [waves * 64, 1, 1], [out], sync=False)
+        e1.record()
+        e1.sync()
+        return e0.elapsed_ms(e1) * 1e3
+
+    return {"mfma_only": run(0, 4), "valu_only": run(1, 4), "both_in_each_wave": run(2, 4), "one_wave_of_each_per_simd": run(3, 8)}
+
+
 EMPTY_SOURCE = """
 extern "C" __global__ void __launch_bounds__(256) eh_empty(float* out) {
   if (out == nullptr) out[0] = 0.0f;
