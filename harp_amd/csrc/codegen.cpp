@@ -202,6 +202,7 @@ bool holds_load(const Node& n) {
 
 // set by plan_program for the plan it is making (GenOptions::guard_branches)
 thread_local bool g_guard_branches = false;
+thread_local bool g_ranged_loads = true;
 
 struct ExprRenderer {
   LoadHook load_hook;
@@ -217,6 +218,16 @@ struct ExprRenderer {
   mutable std::vector<std::string> guards;
   mutable bool hooked_under_guard = false;
   mutable int plain_selects = 0;
+  // Buffers (name -> bytes, below 2^31) read through a buffer resource `eh_rs_<name>` instead
+  // of a pointer: the hardware checks the byte offset against the resource's size and an
+  // out-of-range load returns zero.  A guarded fp32 load is then one load whose offset is out
+  // of range where the guard fails, and `guard ? load : 0` needs no select; the address is a
+  // 32-bit offset, not a 64-bit pointer sum.
+  const std::map<std::string, size_t>* ranged = nullptr;
+  bool is_ranged(const Node& n) const {
+    return ranged && n.op == Op::Load && n.count == 1 && n.dtype.ty == Ty::F32 && n.args[0]->op == Op::Var &&
+           ranged->count(n.args[0]->name) && !load_hook;
+  }
 
   std::string math1(const char* f32, const char* f64, const Node& n) const {
     bool dbl = infer_ty(*n.args[0], var_types) == Ty::F64;
@@ -258,6 +269,14 @@ struct ExprRenderer {
         if (g_guard_branches || plain_selects > 0 || (!holds_load(*n.args[1]) && !holds_load(*n.args[2])))
           return "(" + expr(*n.args[0]) + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
         const std::string c = expr(*n.args[0]);
+        // `inside ? x[i] : 0` through a buffer resource: the load alone
+        if (is_ranged(*n.args[1]) && n.args[2]->op == Op::Const && n.args[2]->dtype.ty == Ty::F32 && n.args[2]->fval == 0.0 &&
+            !std::signbit(n.args[2]->fval)) {
+          guards.push_back("(bool)" + c);
+          const std::string a = expr(*n.args[1]);
+          guards.pop_back();
+          return a;
+        }
         const bool outer_hooked = hooked_under_guard;
         hooked_under_guard = false;
         guards.push_back("(bool)" + c);
@@ -283,6 +302,13 @@ struct ExprRenderer {
         if (load_hook && load_hook(n, &s)) {
           if (!guards.empty()) hooked_under_guard = true;
           return s;
+        }
+        if (is_ranged(n)) {
+          const std::string off = "((unsigned)(" + expr(*n.args[1]) + ") << 2)";
+          if (guards.empty()) return "eh_ranged_load(eh_rs_" + n.args[0]->name + ", " + off + ")";
+          std::string g = guards[0];
+          for (size_t i = 1; i < guards.size(); ++i) g += " & " + guards[i];
+          return "eh_ranged_load(eh_rs_" + n.args[0]->name + ", (" + g + ") ? " + off + " : 0x80000000u)";
         }
         if (n.count == 1 && !guards.empty()) {
           std::string g = guards[0];
@@ -1237,6 +1263,12 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   f.src_bytes = it == elems.end() ? 0.0 : 4.0 * static_cast<double>(it->second);
   for (size_t i = 0; i < k.loops.size(); ++i) f.loops.push_back({k.loops[i].var, k.loops[i].extent, strides[i]});
   ExprRenderer er;
+  std::map<std::string, size_t> ranged;
+  if (g_ranged_loads && !g_guard_branches && small && it->second * 4 < (size_t{1} << 31)) {
+    f.ranged_bytes = it->second * 4;
+    ranged[src] = f.ranged_bytes;
+    er.ranged = &ranged;
+  }
   f.expr = er.expr(*k.value);
   if (auto a = affine_of(*loads[0].load->args[1])) {
     for (size_t i = 0; i < k.loops.size(); ++i)
@@ -2222,6 +2254,7 @@ void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, co
 ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   if (program.op != Op::Program) throw Error("expected a program node");
   g_guard_branches = opt.guard_branches;
+  g_ranged_loads = opt.ranged_loads;
   validate_sizes(program);
   ProgramPlan plan;
   std::vector<const Node*> kernels;
@@ -2487,6 +2520,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
         f->src_bytes = fi->src_bytes;
         f->src_stride.clear();
         f->plain = false;
+        f->ranged_bytes = 0;              // (the expression now calls the inner gather's function)
         folded_kernels.insert(q);
         plan.elided.insert(inner.out_buf);
         break;

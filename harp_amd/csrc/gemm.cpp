@@ -433,6 +433,10 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
     const std::string IT = f->small ? "int" : "long long";
     os << "#define EH_" << X << "_FOLD 1\n#define EH_" << X << "_FOLD_MODE " << mode << "\n#define EH_" << X << "_FOLD_Q " << Q
        << "LL\n";
+    if (f->ranged_bytes)
+      os << "#ifndef EH_RANGED_LOAD\n#define EH_RANGED_LOAD 1\n// one fp32 at a byte offset into a buffer resource; zero beyond the resource's size\n"
+            "__device__ __forceinline__ float eh_ranged_load(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {\n"
+            "  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));\n}\n#endif\n";
     os << f->prelude;
     // The element at index eh_U * Q + eh_I of what the producer would have written: its loop
     // variables above Q are decoded from eh_U, those below from eh_I, each by a function of its
@@ -465,6 +469,9 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
        << UT << ")eh_I64;\n  (void)eh_I;\n  " << P << "_lower r;\n" << dlo.str() << "  return r;\n}\n";
     os << "__device__ __forceinline__ float " << P << "_val(const float* __restrict__ " << f->src << ", const " << P
        << "_upper& eh_u, const " << P << "_lower& eh_l) {\n  (void)eh_u;\n  (void)eh_l;\n" << use.str();
+    if (f->ranged_bytes)
+      os << "  const __amdgpu_buffer_rsrc_t eh_rs_" << f->src << " = __builtin_amdgcn_make_buffer_rsrc((void*)" << f->src << ", 0, "
+         << f->ranged_bytes << ", 0x00020000);\n";
     os << "  return (float)(" << f->expr << ");\n}\n";
   };
   const bool epi_here = epilogue && S == 1;     // with K split the epilogue runs in the summing launch

@@ -51,6 +51,9 @@ struct FoldedOperand {
   std::map<int64_t, int64_t> src_stride;
   bool plain = false;           // the producer is one unguarded load at an affine index (a copy through a view)
   int64_t src_off = 0;          // constant term of that index
+  // nonzero: `expr` reads `src` through the buffer resource `eh_rs_<src>` over that many bytes
+  // (the element function declares it); a byte offset beyond them reads as zero
+  size_t ranged_bytes = 0;
 };
 using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer
 
