@@ -223,10 +223,14 @@ struct ExprRenderer {
   // out-of-range load returns zero.  A guarded fp32 load is then one load whose offset is out
   // of range where the guard fails, and `guard ? load : 0` needs no select; the address is a
   // 32-bit offset, not a 64-bit pointer sum.
+  // With a load hook installed (a schedule that renders plain loads itself) only guarded loads
+  // take this form, and only under guards that test indices: an offset that waits for another
+  // load's value (a mask read from memory) would put the two loads one after the other.
   const std::map<std::string, size_t>* ranged = nullptr;
-  bool is_ranged(const Node& n) const {
+  mutable int value_guards = 0;         // selects around the current node whose condition holds a load
+  bool is_ranged(const Node& n, bool guarded) const {
     return ranged && n.op == Op::Load && n.count == 1 && n.dtype.ty == Ty::F32 && n.args[0]->op == Op::Var &&
-           ranged->count(n.args[0]->name) && !load_hook;
+           ranged->count(n.args[0]->name) && (!load_hook || (guarded && value_guards == 0));
   }
 
   std::string math1(const char* f32, const char* f64, const Node& n) const {
@@ -269,8 +273,14 @@ struct ExprRenderer {
         if (g_guard_branches || plain_selects > 0 || (!holds_load(*n.args[1]) && !holds_load(*n.args[2])))
           return "(" + expr(*n.args[0]) + " ? " + expr(*n.args[1]) + " : " + expr(*n.args[2]) + ")";
         const std::string c = expr(*n.args[0]);
+        struct ValueGuard {
+          int& n;
+          bool on;
+          ValueGuard(int& c, bool o) : n(c), on(o) { n += on; }
+          ~ValueGuard() { n -= on; }
+        } value_guard(value_guards, holds_load(*n.args[0]));
         // `inside ? x[i] : 0` through a buffer resource: the load alone
-        if (is_ranged(*n.args[1]) && n.args[2]->op == Op::Const && n.args[2]->dtype.ty == Ty::F32 && n.args[2]->fval == 0.0 &&
+        if (is_ranged(*n.args[1], true) && n.args[2]->op == Op::Const && n.args[2]->dtype.ty == Ty::F32 && n.args[2]->fval == 0.0 &&
             !std::signbit(n.args[2]->fval)) {
           guards.push_back("(bool)" + c);
           const std::string a = expr(*n.args[1]);
@@ -299,11 +309,11 @@ struct ExprRenderer {
       }
       case Op::Load: {
         std::string s;
-        if (load_hook && load_hook(n, &s)) {
+        if (!is_ranged(n, !guards.empty()) && load_hook && load_hook(n, &s)) {
           if (!guards.empty()) hooked_under_guard = true;
           return s;
         }
-        if (is_ranged(n)) {
+        if (is_ranged(n, !guards.empty())) {
           const std::string off = "((unsigned)(" + expr(*n.args[1]) + ") << 2)";
           if (guards.empty()) return "eh_ranged_load(eh_rs_" + n.args[0]->name + ", " + off + ")";
           std::string g = guards[0];
@@ -2978,6 +2988,8 @@ struct GroupEmitter {
   std::map<std::string, int64_t> need;   // elements each bound buffer must hold (max index + 1)
   // lets a schedule serve some external loads from somewhere else (an LDS tile)
   std::function<bool(const std::string& buf, const Affine& index, std::string* text)> load_override;
+  // fp32 inputs whose guarded loads go through a buffer resource (name -> bytes); see ExprRenderer::ranged
+  std::map<std::string, size_t> ranged;
 
   GroupEmitter(const Group& grp, const GenOptions& o) : g(grp), opt(o) {}
 
@@ -3079,6 +3091,7 @@ struct GroupEmitter {
   // `ld` maps a cached/vectorised external load id to the text that yields its value.
   std::string value_text(const Stage& st, const std::function<std::string(int)>& ld) const {
     ExprRenderer er;
+    if (!ranged.empty()) er.ranged = &ranged;
     er.load_hook = [&](const Node& load, std::string* out) {
       const std::string& b = load.args[0]->name;
       const Stage* p = nullptr;
@@ -3205,8 +3218,23 @@ struct GroupEmitter {
             "template <bool NT, typename T> __device__ __forceinline__ void eh_store2(T* p, EhV2<T> v) {\n"
             "  if (NT) __builtin_nontemporal_store(v, reinterpret_cast<EhV2<T>*>(p));\n"
             "  else *reinterpret_cast<EhV2<T>*>(p) = v;\n}\n";
+    // guarded reads of an input whose size the buffer table fixes: one load each, out of range
+    // (and so zero) where the guard fails
+    bool any_guarded = false;
+    for_each_external_load([&](const LoadRef& lr) { any_guarded = any_guarded || lr.guarded; });
+    if (any_guarded && g_ranged_loads && !g_guard_branches && !idx64)
+      for (const auto& b : in_bufs) {
+        auto it = elems.find(b);
+        if (it != elems.end() && in_dtype.at(b).ty == Ty::F32 && it->second * 4 < (size_t{1} << 31)) ranged[b] = it->second * 4;
+      }
+    if (!ranged.empty())
+      os << "__device__ __forceinline__ float eh_ranged_load(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {\n"
+            "  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_offset, 0, 0));\n}\n";
     os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "("
        << params_text(&ls.arg_bufs) << ") {\n";
+    for (const auto& rb : ranged)
+      os << "  const __amdgpu_buffer_rsrc_t eh_rs_" << rb.first << " = __builtin_amdgcn_make_buffer_rsrc((void*)" << rb.first
+         << ", 0, " << rb.second << ", 0x00020000);\n";
     os << "  const idx_t eh_nvec = " << NVEC << ";\n";
     os << "  const idx_t eh_stride = (idx_t)gridDim.x * " << block << ";\n";
     os << "  for (idx_t eh_g = (idx_t)blockIdx.x * " << block << " + threadIdx.x; eh_g < eh_nvec; eh_g += eh_stride) {\n";

@@ -979,6 +979,17 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
     got = _cnn_step_on(frontend, "hip", arrays, True)
     for g, p in zip(got, got_plain):
         assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
+    # guarded reads (padding) through a buffer resource, out of range where the guard fails
+    # (default), or at a clamped index with a select behind them (ranged_loads=0): same bits
+    assert any("eh_ranged_load(eh_rs_" in l["source"] for l in folded.launches)
+    assert not any("eh_ranged_load" in l["source"] for l in hip.render_program(prog_ast, {"ranged_loads": 0}).launches)
+    reg.options = {"ranged_loads": 0}
+    try:
+        got_clamped = _cnn_step_on(frontend, "hip", arrays, True)
+    finally:
+        reg.options = old
+    for g, c in zip(got, got_clamped):
+        assert np.array_equal(g, c)
     # option gemm_merge_batch=1: per-image weight-gradient contractions and the sum over images
     # that follows become one contraction with the batch folded into k
     merged = hip.render_program(prog_ast, {"gemm_merge_batch": 1})

@@ -638,8 +638,11 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     temp = cols[0]["args"][-1]
     (reader,) = [l for l in plan.launches if temp in l["args"] and l is not cols[0]]
     body = reader["source"][reader["source"].index("__global__"):]
-    assert body.count(temp + "[") == 9
-    assert "if (" not in body.replace("if (eh_", "")            # guarded loads: clamped index + select
+    assert body.count("eh_ranged_load(eh_rs_" + temp + ",") == 9   # guarded loads: out of range where the guard fails
+    assert "if (" not in body.replace("if (eh_", "") and temp + "[" not in body
+    clamped = hb.render_program(ast, "lanes=1,ranged_loads=0")
+    (reader0,) = [l for l in clamped.launches if l["entry"] == reader["entry"]]
+    assert reader0["source"].count(temp + "[") == 9             # ... or a clamped index and a select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
     assert not any("A:m,B:n,B:source" in l["schedule"] for l in plain.launches)
     # the weight gradients' dY operand is a copy through a view (NCHW read as [image, pixel, channel]):
