@@ -326,6 +326,12 @@ void HipBuffer::settle() {
   auto lk = dev_->stream_lock();
   if (!zero_pending_) return;
   dev_->make_current();
+  // a fill recorded into somebody's graph would run again on every replay, over whatever the
+  // buffer holds by then
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(dev_->stream(), &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+    throw Error("a buffer that nothing has written yet is read under stream capture: write it, read it or take its "
+                "address once before the capture starts");
   check(hipMemsetAsync(ptr_, 0, bytes_, dev_->stream()), "hipMemsetAsync");
   zero_pending_ = false;
 }
@@ -591,9 +597,14 @@ std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n, std::
     }
     bound[i] = b;
   }
-  // zero fills still owed: cancelled where the program overwrites the whole buffer before it
-  // reads it (and the caller can take the debt back), queued now otherwise
-  for (size_t i = 0; i < total; ++i) {
+  resolve_fills(bound, cancelled);
+  return bound;
+}
+
+// Zero fills still owed to the buffers of a table: cancelled where the program overwrites the
+// whole buffer before it reads it (the caller can take the debt back), queued now otherwise.
+void HipProgram::resolve_fills(const std::vector<HipBuffer*>& bound, std::vector<HipBuffer*>* cancelled) {
+  for (size_t i = 0; i < bound.size(); ++i) {
     HipBuffer* b = bound[i];
     if (!b || !b->zero_pending()) continue;
     if (cancelled && first_full_[i] != 0 && first_full_[i] == b->byte_len() &&
@@ -604,7 +615,6 @@ std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n, std::
       b->settle();
     }
   }
-  return bound;
 }
 
 void HipProgram::launch_all(const std::vector<HipBuffer*>& bound) {
@@ -713,6 +723,7 @@ void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
   dev_->make_current();
   char* block = need ? static_cast<char*>(dev_->static_scratch()) : nullptr;
   std::vector<Span> bound(total);
+  std::vector<HipBuffer*> given(total, nullptr);
   size_t off = 0;
   for (size_t i = 0; i < total; ++i) {
     const BufferInfo& bi = plan_.buffers[i];
@@ -729,10 +740,17 @@ void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
     if (bi.shape_known && b->byte_len() < bi.bytes())
       throw Error("Buffer size mismatch: '" + bi.name + "' needs " + std::to_string(bi.bytes()) + " bytes, has " +
                   std::to_string(b->byte_len()));
-    b->settle();                                 // (queues a fill at most; allocates nothing)
+    given[i] = b;
     bound[i] = {b->device_ptr(), b->byte_len(), true};
   }
-  launch_spans(bound);
+  std::vector<HipBuffer*> cancelled;
+  resolve_fills(given, &cancelled);              // (queues fills at most; allocates nothing)
+  try {
+    launch_spans(bound);
+  } catch (...) {
+    for (HipBuffer* b : cancelled) b->set_zero_pending(true);
+    throw;
+  }
   if (sync) dev_->synchronize();
 }
 

@@ -177,6 +177,7 @@ class HipProgram {
   // the first launch that touches it overwrites all of it (`cancelled` then lists it, so that a
   // failed execute can put the debt back)
   std::vector<HipBuffer*> bind(HipBuffer* const* bufs, size_t n, std::vector<HipBuffer*>* cancelled);
+  void resolve_fills(const std::vector<HipBuffer*>& bound, std::vector<HipBuffer*>* cancelled);
   void launch_all(const std::vector<HipBuffer*>& bound);            // queues every launch on the stream
   struct Span {
     void* ptr = nullptr;

@@ -185,7 +185,10 @@ int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, in
  * All calls on one device share that device's block, which keeps the previous call's contents
  * (no kernel relies on them: every scratch element is written before it is read).  Calls that
  * overlap on one device would race on it; calls made through this library do not overlap, because
- * every call's launches are ordered on the device's stream behind those of the call before. */
+ * every call's launches are ordered on the device's stream behind those of the call before.
+ * A given buffer that nothing has written yet and that the program does not overwrite whole gets
+ * its zero fill queued first (no allocation); under stream capture that is an error instead,
+ * since a recorded fill would run again on every replay: write or read such a buffer once before. */
 #define EH_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
 int eh_program_execute_static(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 /* The launches of one eh_program_execute(prog, bufs, n_bufs, .) captured as a HIP graph of kernel
