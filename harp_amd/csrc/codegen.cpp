@@ -1101,7 +1101,7 @@ Canon canon_as(const NestKernel& k, StageKind kind) {
 // The emitters live below; declared here so plan_program reads top-down.
 namespace {
 LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& buf_elems);
-void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan);
+void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan, const EpilogueSpec* epi = nullptr);
 LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestKernel*>& chain, const GenOptions& opt,
                               const std::map<std::string, size_t>& elems);
 }  // namespace
@@ -2621,6 +2621,194 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // Elementwise kernels that follow kernel i (a reduce with a dense output of `total` elements)
+  // over the same dense index space and feed on its result: the function that applies them to
+  // one element while it is still in a register.  `k0r`: k0 with its output laid out as a
+  // consumer that reads it through a permutation wants it, when that applies and is allowed.
+  auto build_epilogue = [&](size_t i, const NestKernel& k0, int64_t total, bool allow_relayout, NestKernel& k0r,
+                            EpilogueSpec& epi, size_t& after) -> bool {
+    bool have_epi = false;
+    const bool small = total < (int64_t{1} << 30);
+    std::map<std::string, DType> avail;          // values held in registers: C and stage outputs
+    avail[k0.out_buf] = k0.out_dtype;
+    bool c_relaid = false;
+    size_t relaid_pos = 0;                       // position in `taken` of the stage that reads through a permutation
+    Affine relaid_read;                          // ... and the index it reads at, over its own loops
+    std::set<std::string> old_space;             // values produced before that stage
+    std::set<size_t> independent;                // taken stages that read no value of the chain
+    std::vector<size_t> taken;
+    size_t j = i + 1;
+    for (; j < kernels.size(); ++j) {
+      if (absorbed.count(j)) continue;
+      if (!nests[j] || folded_kernels.count(j) || nests[j]->rkind != ReduceKind::None) break;
+      const NestKernel& sk = *nests[j];
+      int64_t numel = 0;
+      auto strides = dense_strides(sk, &numel);
+      if (!strides || numel != total || avail.count(sk.out_buf)) break;
+      std::vector<LoadRef> loads;
+      collect_loads(*sk.value, loads);
+      bool feeds = false, ok = true;
+      std::optional<Affine> permuted;            // the one index all values of the chain are read at, if not the aligned one
+      for (const auto& lr : loads) {
+        if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
+        const std::string& b = lr.load->args[0]->name;
+        if (!avail.count(b)) continue;
+        auto a = affine_of(*lr.load->args[1]);
+        if (!a) { ok = false; break; }
+        const bool aligned = *a == *sk.out_aff;
+        if (c_relaid && (old_space.count(b) || !aligned)) { ok = false; break; }
+        if (!aligned) {
+          if (feeds && !permuted) { ok = false; break; }          // the stage reads the chain both ways
+          if (permuted && !(*permuted == *a)) { ok = false; break; }
+          permuted = *a;
+        } else if (permuted) {
+          ok = false;
+          break;
+        }
+        feeds = true;
+      }
+      if (!ok) break;
+      // a stage over the same index space that reads nothing of the chain (the square of a
+      // saved activation, say) rides along when a later stage combines it with the chain
+      if (!feeds) independent.insert(j);
+      if (permuted) {
+        // A consumer may read the chain's values through a permutation (a transposed weight
+        // gradient and its update, NHWC -> NCHW after a convolution).  If nothing computed so
+        // far is needed outside the chain, the contraction can put each element where this
+        // consumer wants it: C takes the consumer's index space, the stages before it are
+        // evaluated at the element's original position, and the read becomes the aligned one.
+        bool sole = true;
+        for (const auto& kv : avail) {
+          sole = sole && role_of(kv.first) == "temp";
+          for (size_t r : readers[kv.first]) sole = sole && r > i && r <= j;
+        }
+        auto na = sole && allow_relayout ? relayout(k0, sk, *permuted) : std::nullopt;
+        if (!na) break;
+        k0r.out_aff = *na;
+        if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; break; }
+        c_relaid = true;
+        relaid_pos = taken.size();
+        relaid_read = *permuted;
+        for (const auto& kv : avail) old_space.insert(kv.first);
+      }
+      avail[sk.out_buf] = sk.out_dtype;
+      taken.push_back(j);
+    }
+    while (!taken.empty() && independent.count(taken.back())) {
+      avail.erase(nests[taken.back()]->out_buf);      // nothing after it uses the chain: leave it out
+      independent.erase(taken.back());
+      taken.pop_back();
+    }
+    if (!taken.empty()) {
+      after = taken.back() + 1;
+      auto needed = [&](const std::string& buf) {
+        if (role_of(buf) != "temp") return true;
+        for (size_t r : readers[buf])
+          if (r <= i || r >= after) return true;
+        return false;
+      };
+      std::ostringstream fn, body;
+      std::vector<std::string> ext_order;
+      std::map<std::string, std::pair<std::string, size_t>> ext;   // name -> (declaration, min bytes)
+      epi.store_c = needed(k0.out_buf);
+      if (!epi.store_c) plan.elided.insert(k0.out_buf);
+      const std::string IT = small ? "int" : "long long";
+      const std::string UT = small ? "unsigned" : "unsigned long long";
+      body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
+      body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
+      if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
+      auto decode = [&](const NestKernel& sk, const std::string& from) {
+        int64_t numel = 0;
+        auto strides = *dense_strides(sk, &numel);
+        for (size_t li = 0; li < sk.loops.size(); ++li) {
+          const Loop& l = sk.loops[li];
+          if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
+          else body << "    const " << IT << " " << l.var << " = (" << IT << ")(((" << UT << ")" << from << " / " << strides[li] << "u) % "
+                    << l.extent << "u);\n";    // (never negative: the unsigned division is the cheaper one)
+        }
+      };
+      if (c_relaid && relaid_pos > 0) {
+        // where this element sat before C took the later consumer's layout: the stages
+        // ahead of that consumer index their other operands with it
+        if (epi.store_c) throw Error("internal: relaid contraction '" + k0.name + "' must not store C");
+        body << "  " << IT << " eh_lo;\n  {\n";
+        decode(*nests[taken[relaid_pos]], "eh_l");
+        body << "    eh_lo = ";
+        bool first_term = true;
+        for (const auto& kv : relaid_read.coef) {
+          if (kv.second == 0) continue;
+          body << (first_term ? "" : " + ") << kv.first << " * " << kv.second;
+          first_term = false;
+        }
+        if (first_term) body << "0";
+        body << ";\n  }\n";
+      }
+      for (size_t ti = 0; ti < taken.size(); ++ti) {
+        const size_t j2 = taken[ti];
+        const NestKernel& sk = *nests[j2];
+        epi.kernels.push_back(sk.name);
+        body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
+        decode(sk, (c_relaid && ti < relaid_pos) ? "eh_lo" : "eh_l");
+        ExprRenderer er;
+        er.load_hook = [&](const Node& ld, std::string* out) {
+          const std::string& b = ld.args[0]->name;
+          if (!avail.count(b)) return false;
+          *out = "eh_v_" + b;
+          return true;
+        };
+        std::vector<LoadRef> loads;
+        collect_loads(*sk.value, loads);
+        for (const auto& lr : loads) {
+          const std::string& b = lr.load->args[0]->name;
+          if (avail.count(b) || ext.count(b)) {
+            if (ext.count(b) && !lr.guarded) {
+              if (auto a = affine_of(*lr.load->args[1]))
+                ext[b].second = std::max(ext[b].second, static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) *
+                                                             lr.load->dtype.itemsize());
+            }
+            continue;
+          }
+          size_t mb = 0;
+          if (!lr.guarded)
+            if (auto a = affine_of(*lr.load->args[1]))
+              mb = static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) * lr.load->dtype.itemsize();
+          DType et = lr.load->dtype;
+          for (const auto& pp : sk.params)
+            if (pp.name == b) et = pp.dtype.elem();
+          ext[b] = {"const " + ctype(et) + "* __restrict__ " + b, mb};
+          ext_order.push_back(b);
+          epi.bytes += static_cast<double>(elems.count(b) ? elems.at(b) : 0) * et.itemsize();
+        }
+        body << "    eh_v_" << sk.out_buf << " = (" << ctype(sk.out_dtype) << ")(" << er.expr(*sk.value) << ");\n";
+        if (needed(sk.out_buf)) {
+          body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
+          ext[sk.out_buf] = {ctype(sk.out_dtype) + "* __restrict__ " + sk.out_buf,
+                             static_cast<size_t>(total) * sk.out_dtype.itemsize()};
+          ext_order.push_back(sk.out_buf);
+          epi.bytes += static_cast<double>(total) * sk.out_dtype.itemsize();
+        } else {
+          plan.elided.insert(sk.out_buf);
+        }
+        body << "  }\n";
+      }
+      for (const auto& b : ext_order) {
+        epi.params += ", " + ext[b].first;
+        epi.args += ", " + b;
+        epi.bufs.push_back(b);
+        epi.min_bytes.push_back(ext[b].second);
+      }
+      fn << "// what kernels";
+      for (const auto& n : epi.kernels) fn << " " << n;
+      fn << " do to element eh_e of " << k0.out_buf << "\n";
+      fn << "__device__ __forceinline__ void eh_epilogue(long long eh_e, float eh_acc"
+         << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params
+         << ") {\n" << body.str() << "}\n";
+      epi.function = fn.str();
+      have_epi = true;
+    }
+    return have_epi;
+  };
+
   size_t i = 0;
   while (i < kernels.size()) {
     if (folded_kernels.count(i) || absorbed.count(i)) {
@@ -2653,185 +2841,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (opt.gemm_epilogue && opt.fuse && have_table && gemm_shaped(k0, opt)) {
         auto gs = match_gemm(k0);
         if (gs && gemm_output_dense(*gs)) {
-          const int64_t total = gs->batch * gs->M * gs->N;
-          const bool small = total < (int64_t{1} << 30);
-          std::map<std::string, DType> avail;          // values held in registers: C and stage outputs
-          avail[k0.out_buf] = k0.out_dtype;
-          bool c_relaid = false;
-          size_t relaid_pos = 0;                       // position in `taken` of the stage that reads through a permutation
-          Affine relaid_read;                          // ... and the index it reads at, over its own loops
-          std::set<std::string> old_space;             // values produced before that stage
-          std::set<size_t> independent;                // taken stages that read no value of the chain
-          std::vector<size_t> taken;
-          size_t j = i + 1;
-          for (; j < kernels.size(); ++j) {
-            if (absorbed.count(j)) continue;
-            if (!nests[j] || folded_kernels.count(j) || nests[j]->rkind != ReduceKind::None) break;
-            const NestKernel& sk = *nests[j];
-            int64_t numel = 0;
-            auto strides = dense_strides(sk, &numel);
-            if (!strides || numel != total || avail.count(sk.out_buf)) break;
-            std::vector<LoadRef> loads;
-            collect_loads(*sk.value, loads);
-            bool feeds = false, ok = true;
-            std::optional<Affine> permuted;            // the one index all values of the chain are read at, if not the aligned one
-            for (const auto& lr : loads) {
-              if (lr.load->args[0]->op != Op::Var || lr.load->count != 1) { ok = false; break; }
-              const std::string& b = lr.load->args[0]->name;
-              if (!avail.count(b)) continue;
-              auto a = affine_of(*lr.load->args[1]);
-              if (!a) { ok = false; break; }
-              const bool aligned = *a == *sk.out_aff;
-              if (c_relaid && (old_space.count(b) || !aligned)) { ok = false; break; }
-              if (!aligned) {
-                if (feeds && !permuted) { ok = false; break; }          // the stage reads the chain both ways
-                if (permuted && !(*permuted == *a)) { ok = false; break; }
-                permuted = *a;
-              } else if (permuted) {
-                ok = false;
-                break;
-              }
-              feeds = true;
-            }
-            if (!ok) break;
-            // a stage over the same index space that reads nothing of the chain (the square of a
-            // saved activation, say) rides along when a later stage combines it with the chain
-            if (!feeds) independent.insert(j);
-            if (permuted) {
-              // A consumer may read the chain's values through a permutation (a transposed weight
-              // gradient and its update, NHWC -> NCHW after a convolution).  If nothing computed so
-              // far is needed outside the chain, the contraction can put each element where this
-              // consumer wants it: C takes the consumer's index space, the stages before it are
-              // evaluated at the element's original position, and the read becomes the aligned one.
-              bool sole = true;
-              for (const auto& kv : avail) {
-                sole = sole && role_of(kv.first) == "temp";
-                for (size_t r : readers[kv.first]) sole = sole && r > i && r <= j;
-              }
-              auto na = sole ? relayout(k0, sk, *permuted) : std::nullopt;
-              if (!na) break;
-              k0r.out_aff = *na;
-              if (!gemm_shaped(k0r, opt)) { k0r.out_aff = k0.out_aff; break; }
-              c_relaid = true;
-              relaid_pos = taken.size();
-              relaid_read = *permuted;
-              for (const auto& kv : avail) old_space.insert(kv.first);
-            }
-            avail[sk.out_buf] = sk.out_dtype;
-            taken.push_back(j);
-          }
-          while (!taken.empty() && independent.count(taken.back())) {
-            avail.erase(nests[taken.back()]->out_buf);      // nothing after it uses the chain: leave it out
-            independent.erase(taken.back());
-            taken.pop_back();
-          }
-          if (!taken.empty()) {
-            after = taken.back() + 1;
-            auto needed = [&](const std::string& buf) {
-              if (role_of(buf) != "temp") return true;
-              for (size_t r : readers[buf])
-                if (r <= i || r >= after) return true;
-              return false;
-            };
-            std::ostringstream fn, body;
-            std::vector<std::string> ext_order;
-            std::map<std::string, std::pair<std::string, size_t>> ext;   // name -> (declaration, min bytes)
-            epi.store_c = needed(k0.out_buf);
-            if (!epi.store_c) plan.elided.insert(k0.out_buf);
-            const std::string IT = small ? "int" : "long long";
-            const std::string UT = small ? "unsigned" : "unsigned long long";
-            body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
-            body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
-            if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
-            auto decode = [&](const NestKernel& sk, const std::string& from) {
-              int64_t numel = 0;
-              auto strides = *dense_strides(sk, &numel);
-              for (size_t li = 0; li < sk.loops.size(); ++li) {
-                const Loop& l = sk.loops[li];
-                if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
-                else body << "    const " << IT << " " << l.var << " = (" << IT << ")(((" << UT << ")" << from << " / " << strides[li] << "u) % "
-                          << l.extent << "u);\n";    // (never negative: the unsigned division is the cheaper one)
-              }
-            };
-            if (c_relaid && relaid_pos > 0) {
-              // where this element sat before C took the later consumer's layout: the stages
-              // ahead of that consumer index their other operands with it
-              if (epi.store_c) throw Error("internal: relaid contraction '" + k0.name + "' must not store C");
-              body << "  " << IT << " eh_lo;\n  {\n";
-              decode(*nests[taken[relaid_pos]], "eh_l");
-              body << "    eh_lo = ";
-              bool first_term = true;
-              for (const auto& kv : relaid_read.coef) {
-                if (kv.second == 0) continue;
-                body << (first_term ? "" : " + ") << kv.first << " * " << kv.second;
-                first_term = false;
-              }
-              if (first_term) body << "0";
-              body << ";\n  }\n";
-            }
-            for (size_t ti = 0; ti < taken.size(); ++ti) {
-              const size_t j2 = taken[ti];
-              const NestKernel& sk = *nests[j2];
-              epi.kernels.push_back(sk.name);
-              body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
-              decode(sk, (c_relaid && ti < relaid_pos) ? "eh_lo" : "eh_l");
-              ExprRenderer er;
-              er.load_hook = [&](const Node& ld, std::string* out) {
-                const std::string& b = ld.args[0]->name;
-                if (!avail.count(b)) return false;
-                *out = "eh_v_" + b;
-                return true;
-              };
-              std::vector<LoadRef> loads;
-              collect_loads(*sk.value, loads);
-              for (const auto& lr : loads) {
-                const std::string& b = lr.load->args[0]->name;
-                if (avail.count(b) || ext.count(b)) {
-                  if (ext.count(b) && !lr.guarded) {
-                    if (auto a = affine_of(*lr.load->args[1]))
-                      ext[b].second = std::max(ext[b].second, static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) *
-                                                                   lr.load->dtype.itemsize());
-                  }
-                  continue;
-                }
-                size_t mb = 0;
-                if (!lr.guarded)
-                  if (auto a = affine_of(*lr.load->args[1]))
-                    mb = static_cast<size_t>(max_abs_index(*a, sk.loops, nullptr) + 1) * lr.load->dtype.itemsize();
-                DType et = lr.load->dtype;
-                for (const auto& pp : sk.params)
-                  if (pp.name == b) et = pp.dtype.elem();
-                ext[b] = {"const " + ctype(et) + "* __restrict__ " + b, mb};
-                ext_order.push_back(b);
-                epi.bytes += static_cast<double>(elems.count(b) ? elems.at(b) : 0) * et.itemsize();
-              }
-              body << "    eh_v_" << sk.out_buf << " = (" << ctype(sk.out_dtype) << ")(" << er.expr(*sk.value) << ");\n";
-              if (needed(sk.out_buf)) {
-                body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
-                ext[sk.out_buf] = {ctype(sk.out_dtype) + "* __restrict__ " + sk.out_buf,
-                                   static_cast<size_t>(total) * sk.out_dtype.itemsize()};
-                ext_order.push_back(sk.out_buf);
-                epi.bytes += static_cast<double>(total) * sk.out_dtype.itemsize();
-              } else {
-                plan.elided.insert(sk.out_buf);
-              }
-              body << "  }\n";
-            }
-            for (const auto& b : ext_order) {
-              epi.params += ", " + ext[b].first;
-              epi.args += ", " + b;
-              epi.bufs.push_back(b);
-              epi.min_bytes.push_back(ext[b].second);
-            }
-            fn << "// what kernels";
-            for (const auto& n : epi.kernels) fn << " " << n;
-            fn << " do to element eh_e of " << k0.out_buf << "\n";
-            fn << "__device__ __forceinline__ void eh_epilogue(long long eh_e, float eh_acc"
-               << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params
-               << ") {\n" << body.str() << "}\n";
-            epi.function = fn.str();
-            have_epi = true;
-          }
+          have_epi = build_epilogue(i, k0, gs->batch * gs->M * gs->N, true, k0r, epi, after);
         }
       }
       auto gl = try_emit_gemm(have_epi ? k0r : k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
@@ -2844,8 +2854,18 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (have_epi) throw Error("internal: contraction '" + k0.name + "' matched but could not be emitted");
     }
     if (k0.rkind != ReduceKind::None && !reduce_is_rowwise(k0)) {
-      emit_serial_reduce(k0, opt, &plan);
-      ++i;
+      // elementwise kernels over the reduce's (dense) output that feed on it ride along: a
+      // parameter's update in the launch that finishes its gradient's sum
+      EpilogueSpec epi;
+      size_t after = i + 1;
+      NestKernel k0r = k0;
+      int64_t numel = 0;
+      bool have_epi = false;
+      if (opt.gemm_epilogue && opt.fuse && have_table && k0.acc_dtype.ty == Ty::F32 && k0.out_dtype.ty == Ty::F32 &&
+          dense_strides(k0, &numel))
+        have_epi = build_epilogue(i, k0, numel, false, k0r, epi, after);
+      emit_serial_reduce(k0, opt, &plan, have_epi ? &epi : nullptr);
+      i = have_epi ? after : i + 1;
       continue;
     }
     // start a group with kernel i and extend it while the next kernels fit
@@ -3602,8 +3622,11 @@ struct SerialReduce {
   std::map<std::string, NodePtr> zero;
   int64_t N = 1;
   bool idx64 = false;
+  // elementwise kernels applied to each result before it is stored (the update that follows a
+  // gradient's sum), or null
+  const EpilogueSpec* epi = nullptr;
 
-  SerialReduce(const NestKernel& kk, const GenOptions& o) : k(kk), opt(o) {
+  SerialReduce(const NestKernel& kk, const GenOptions& o, const EpilogueSpec* e = nullptr) : k(kk), opt(o), epi(e) {
     for (const auto& l : k.loops) {
       if (l.extent == 0) throw Error("kernel '" + k.name + "' has an empty loop");
       if (l.extent == 1) zero[l.var] = make_i64(0);
@@ -3625,13 +3648,35 @@ struct SerialReduce {
   std::string params(LaunchSpec* ls, bool with_out, const std::string& extra) const {
     std::string t;
     for (const auto& p : k.params) {
-      if (p.mut_ && !with_out) continue;
+      if (p.mut_ && (!with_out || (epi && !epi->store_c))) continue;
       t += (t.empty() ? "" : ", ") + std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + p.name;
       ls->arg_bufs.push_back(p.name);
     }
     if (!extra.empty()) t += (t.empty() ? "" : ", ") + extra;
+    if (with_out && epi) t += epi->params;        // (bound by finish_epilogue, after the reduce's own buffers)
     return t;
   }
+
+  // the statement that puts result `value` of the current output where it belongs
+  std::string store(const std::string& value, const std::string& indent) const {
+    NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
+    ExprRenderer er;
+    if (!epi) return indent + k.out_buf + "[" + er.expr(*oi) + "] = (" + ctype(k.out_dtype) + ")" + value + ";\n";
+    return indent + "eh_epilogue((long long)(" + er.expr(*oi) + "), (float)" + value + (epi->store_c ? ", " + k.out_buf : std::string()) +
+           epi->args + ");\n";
+  }
+  // the launch that stores the results also binds what the epilogue reads and writes
+  void finish_epilogue(LaunchSpec* ls) const {
+    if (!epi) return;
+    for (size_t i = 0; i < epi->bufs.size(); ++i) {
+      ls->arg_bufs.push_back(epi->bufs[i]);
+      ls->arg_min_bytes.push_back(epi->min_bytes[i]);
+    }
+    for (const auto& n : epi->kernels) ls->kernels.push_back(n);
+    ls->schedule.insert(ls->schedule.size() - 1, ",epilogue=" + std::to_string(epi->kernels.size()));
+    ls->algo_bytes += epi->bytes;
+  }
+  std::string epilogue_function() const { return epi ? epi->function : std::string(); }
 
   std::string decode(const std::string& ovar) const {
     std::string t = "  idx_t eh_rem = " + ovar + ";\n";
@@ -3677,7 +3722,7 @@ struct SerialReduce {
     ls.grid[0] = static_cast<unsigned>(blocks);
     ls.block[0] = block;
     std::ostringstream os;
-    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n" << epilogue_function();
     os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << params(&ls, true, "") << ") {\n";
     os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
     os << decode("eh_o");
@@ -3686,10 +3731,10 @@ struct SerialReduce {
     os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
     os << "  for (idx_t " << k.rloop.var << " = 0; " << k.rloop.var << " < " << k.rloop.extent << "; ++" << k.rloop.var << ") {\n";
     os << "    acc = " << combine_text(k.rkind, k.acc_dtype, "acc", "(" + TA + ")(" + er.expr(*k.value) + ")") << ";\n  }\n";
-    NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
-    os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
+    os << store("acc", "  ") << "}\n";
     ls.source = os.str();
     min_bytes(&ls);
+    finish_epilogue(&ls);
     return ls;
   }
 
@@ -3713,7 +3758,7 @@ struct SerialReduce {
     const std::string TA = ctype(k.acc_dtype);
     ExprRenderer er;
     std::ostringstream os;
-    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n" << epilogue_function();
     os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << ls.entry << "(" << params(&ls, true, "")
        << ") {\n";
     os << "  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;\n";
@@ -3728,10 +3773,10 @@ struct SerialReduce {
     os << "  __shared__ " << TA << " eh_sm[" << RG << "][64];\n  eh_sm[ty][tx] = acc;\n  __syncthreads();\n";
     os << "  if (ty == 0 && eh_ok) {\n    " << TA << " r = eh_sm[0][tx];\n";
     os << "    for (int q = 1; q < " << RG << "; ++q) r = " << combine_text(k.rkind, k.acc_dtype, "r", "eh_sm[q][tx]") << ";\n";
-    NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
-    os << "    " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")r;\n  }\n}\n";
+    os << store("r", "    ") << "  }\n}\n";
     ls.source = os.str();
     min_bytes(&ls);
+    finish_epilogue(&ls);
     return ls;
   }
 
@@ -3792,20 +3837,24 @@ struct SerialReduce {
       ls.grid[0] = static_cast<unsigned>((N + 255) / 256);
       ls.block[0] = 256;
       std::ostringstream os;
-      os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+      os << hdr(opt) << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n" << epilogue_function();
+      const bool with_out = !(epi && !epi->store_c);
       os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(const " << TA << "* __restrict__ "
-         << scratch << ", " << ctype(k.out_dtype) << "* __restrict__ " << k.out_buf << ") {\n";
-      ls.arg_bufs = {scratch, k.out_buf};
+         << scratch << (with_out ? ", " + ctype(k.out_dtype) + "* __restrict__ " + k.out_buf : std::string())
+         << (epi ? epi->params : std::string()) << ") {\n";
+      ls.arg_bufs = {scratch};
+      if (with_out) ls.arg_bufs.push_back(k.out_buf);
       os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
       os << decode("eh_o");
       os << "  " << TA << " acc = " << literal(*k.identity) << ";\n";
       os << "  for (idx_t s = 0; s < " << S << "; ++s) acc = "
          << combine_text(k.rkind, k.acc_dtype, "acc", scratch + "[s * " + std::to_string(N) + " + eh_o]") << ";\n";
-      NodePtr oi = rename(k.out_index, {{k.rloop.var, make_i64(0)}});
-      os << "  " << k.out_buf << "[" << er.expr(*oi) << "] = (" << ctype(k.out_dtype) << ")acc;\n}\n";
+      os << store("acc", "  ") << "}\n";
       ls.source = os.str();
-      ls.arg_min_bytes = {static_cast<size_t>(S * N) * k.acc_dtype.itemsize(),
-                          static_cast<size_t>(max_abs_index(*k.out_aff, k.loops, nullptr) + 1) * k.out_dtype.itemsize()};
+      ls.arg_min_bytes = {static_cast<size_t>(S * N) * k.acc_dtype.itemsize()};
+      if (with_out)
+        ls.arg_min_bytes.push_back(static_cast<size_t>(max_abs_index(*k.out_aff, k.loops, nullptr) + 1) * k.out_dtype.itemsize());
+      finish_epilogue(&ls);
     }
     return out;
   }
@@ -3915,8 +3964,8 @@ LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestK
   return ls;
 }
 
-void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan) {
-  SerialReduce sr(k, opt);
+void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan, const EpilogueSpec* epi) {
+  SerialReduce sr(k, opt, epi);
   if (sr.wants_split()) {
     for (auto& ls : sr.split(&plan->buffers)) plan->launches.push_back(std::move(ls));
   } else if (sr.wants_columns()) {
