@@ -2475,6 +2475,82 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // A sum over one axis whose result the next kernel only sums over a neighbouring axis (a bias
+  // gradient as the reference lowers it: over the image's columns, then its rows, then the
+  // batch) is one sum over both when every operand walks the two axes as one: the second kernel
+  // and the buffer between them disappear, and what was two short strided passes is one pass
+  // along memory.  (The order of the additions changes, as it does in every parallel reduce.)
+  if (opt.fuse && opt.reindex && have_table) {
+    for (size_t i = 0; i + 1 < kernels.size(); ++i) {
+      if (!nests[i] || !nests[i + 1] || absorbed.count(i) || absorbed.count(i + 1)) continue;
+      const NestKernel& r1 = *nests[i];
+      const NestKernel& r2 = *nests[i + 1];
+      if (r1.rkind != ReduceKind::Sum || r2.rkind != ReduceKind::Sum || !r1.out_aff || !r2.out_aff) continue;
+      if (r1.acc_dtype.ty != Ty::F32 || r1.out_dtype.ty != Ty::F32 || r2.acc_dtype.ty != Ty::F32 || r2.out_dtype.ty != Ty::F32) continue;
+      if (!r1.identity || r1.identity->fval != 0.0 || !r2.identity || r2.identity->fval != 0.0) continue;
+      if (opt.gemm && (gemm_shaped(r1, opt) || gemm_shaped(r2, opt))) continue;
+      if (role_of(r1.out_buf) != "temp" || readers[r1.out_buf] != std::vector<size_t>{i + 1}) continue;
+      if (r1.out_buf.rfind("eh_", 0) == 0) continue;       // pieces of lines the planner itself cut: they stay two reduces
+      const Node& v2 = *r2.value;
+      if (v2.op != Op::Load || v2.count != 1 || v2.args[0]->op != Op::Var || v2.args[0]->name != r1.out_buf) continue;
+      auto ra = affine_of(*v2.args[1]);
+      if (!ra || ra->c != r1.out_aff->c) continue;
+      // r2's loops (and its reduce loop) against r1's output loops, matched by their stride in the buffer between
+      std::map<std::string, NodePtr> to_r1;       // r2's loop variables in terms of r1's
+      const Loop* outer = nullptr;                // the loop of r1 that r2 sums over
+      bool ok = true;
+      size_t matched = 0;
+      auto match = [&](const Loop& l2) -> const Loop* {
+        const Loop* hit = nullptr;
+        for (const auto& l1 : r1.loops)
+          if (l1.extent > 1 && l1.extent == l2.extent && r1.out_aff->of(l1.var) == ra->of(l2.var)) hit = &l1;
+        return hit;
+      };
+      for (const auto& l2 : r2.loops) {
+        if (l2.extent <= 1) { to_r1[l2.var] = make_i64(0); continue; }
+        const Loop* hit = match(l2);
+        if (!hit) { ok = false; break; }
+        to_r1[l2.var] = make_var(hit->var);
+        ++matched;
+      }
+      if (!ok || r2.rloop.extent < 2) continue;
+      outer = match(r2.rloop);
+      size_t live1 = 0;
+      for (const auto& l1 : r1.loops) live1 += l1.extent > 1;
+      if (!outer || matched + 1 != live1) continue;
+      // every load of r1 must walk (outer, r1's reduce loop) as one axis, unguarded
+      std::vector<LoadRef> loads;
+      collect_loads(*r1.value, loads);
+      for (const auto& lr : loads) {
+        auto a = affine_of(*lr.load->args[1]);
+        ok = ok && a && !lr.guarded && a->of(outer->var) == r1.rloop.extent * a->of(r1.rloop.var);
+      }
+      // (not into few long lines: one workgroup per line needs many lines to fill the chip)
+      int64_t lines = 1;
+      for (const auto& l2 : r2.loops) lines *= l2.extent;
+      if (!ok || loads.empty() || r1.rloop.extent * outer->extent > 8192 || lines < 1024) continue;
+      NestKernel m = r1;
+      m.value = rename(r1.value, {{outer->var, make_i64(0)}});
+      m.rloop.extent = r1.rloop.extent * outer->extent;
+      for (auto& l : m.loops)
+        if (l.var == outer->var) l.extent = 1;
+      m.out_buf = r2.out_buf;
+      m.out_dtype = r2.out_dtype;
+      m.out_index = rename(rename(r2.out_index, {{r2.rloop.var, make_i64(0)}}), to_r1);
+      m.out_aff = affine_of(*m.out_index);
+      for (const auto& p : r2.params)
+        if (p.mut_) {
+          for (auto& q : m.params)
+            if (q.mut_) q = p;
+        }
+      if (!m.out_aff) continue;
+      plan.elided.insert(r1.out_buf);
+      absorbed_name[i] = r2.name;
+      absorbed.insert(i + 1);
+      nests[i] = m;
+    }
+  }
+
   // gather / copy kernels read only by contractions are evaluated inside those contractions'
   // tile loaders (implicit GEMM): no launch, no buffer
   FoldMap folded;
@@ -2922,6 +2998,15 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     for (const auto& ls : plan.launches)
       for (const auto& a : ls.arg_bufs) bound = bound || a == c.first;
     if (!bound) plan.elided.insert(c.first);
+  }
+  // a launch that covers a kernel which took another one in covers that one too
+  for (auto& ls : plan.launches) {
+    const std::vector<std::string> covered = ls.kernels;
+    for (const auto& kn : covered)
+      for (const auto& an : absorbed_name)
+        if (nests[an.first] && nests[an.first]->name == kn &&
+            std::find(ls.kernels.begin(), ls.kernels.end(), an.second) == ls.kernels.end())
+          ls.kernels.push_back(an.second);
   }
   // A lowered kernel whose output index is the dense index of its loops writes every element of
   // its output; the launch that stores it overwrites a buffer of exactly that size, whatever it

@@ -953,6 +953,23 @@ def test_contraction_rows_across_groups_into_a_permuted_result(frontend, hip, sh
     assert np.all(np.abs(got - exact.ravel()) <= 1e-5 * scale.ravel() + 1e-30)
 
 
+@pytest.mark.parametrize("shape", [(64, 32, 14, 14), (40, 32, 7, 5), (33, 64, 28, 28)])
+def test_bias_gradient_chain_matches_the_oracle(frontend, hip, shape):
+    """b - lr * sum over (columns, rows, batch) of x: the sums over columns and rows run as one sum
+    along memory and the update in the launch that finishes the sum over the batch; against the
+    oracle's kernel-by-kernel result (reduction tolerance) and float64 numpy."""
+    from test_host_cpu import _bias_gradient_step
+    rng = RNG(sum(shape))
+    arrays = [rng.normal(0, 1, shape).astype(np.float32), rng.normal(0, 1, shape[1]).astype(np.float32),
+              np.full(shape[1], 0.01, np.float32)]
+    got, scheds = _run_program(frontend, hip, _bias_gradient_step, arrays)
+    assert len(scheds) == 2 and "epilogue=2" in scheds[1], scheds
+    ref = realize_on(frontend, "c", _bias_gradient_step, arrays)
+    exact = arrays[1].astype(np.float64) - arrays[0].astype(np.float64).sum((0, 2, 3)) * 0.01
+    scale = np.abs(arrays[0]).astype(np.float64).sum((0, 2, 3)) * 0.01 + np.abs(arrays[1])
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale) and np.all(np.abs(got - exact) <= 1e-5 * scale)
+
+
 def test_config5_with_implicit_gemm_loader(frontend, hip):
     """im2col gathers and layout copies that only contractions read are evaluated inside the
     contractions' tile loaders (no launch, no buffer); option gemm_fold=0 materialises them.

@@ -671,6 +671,31 @@ def test_convolution_rows_run_across_images(frontend):
     assert [l["entry"] for l in small] == ["ehk_R_256_1_32_9_79_part"], [l["schedule"] for l in plan.launches]
 
 
+def _bias_gradient_step(x, b, lr):
+    """A bias's gradient as the reference lowers it (sums over columns, rows, then the batch) and its update."""
+    return b - x.sum(3).sum(2).sum(0) * lr
+
+
+def test_bias_gradient_chain_is_two_launches(frontend):
+    """Sums over an image's columns and then its rows are one sum along memory (the second
+    kernel is taken into the first), and the update rides in the launch that finishes the sum
+    over the batch: four launches become two.  A total over everything is not merged into one
+    long line, and reindex=0 / gemm_epilogue=0 plan the kernels as lowered."""
+    from harp_amd import backend as hb, workloads as wl
+    shapes = [(64, 32, 14, 14), (32,), (32,)]
+    ast = wl.lower_with_table(shapes, _bias_gradient_step)[0]
+    plan = hb.render_program(ast)
+    assert [l["kernels"] for l in plan.launches] == [["R_64_32_14_1_0", "R_64_32_1_1"], ["R_1_32_2", "E_32_3", "E_32_4"]]
+    assert plan.launches[0]["schedule"].startswith("row(T=32,V=4") and "epilogue=2" in plan.launches[1]["schedule"]
+    assert "eh_epilogue(" in plan.launches[1]["source"]
+    elided = {b["name"] for b in plan.buffers if b["elided"]}
+    assert len(elided) == 3                                # the two partial sums' buffers and the gradient itself
+    plain = hb.render_program(ast, "reindex=0,gemm_epilogue=0")
+    assert len(plain.launches) == 4
+    total = hb.render_program(wl.lower_with_table([(8192, 1024)], lambda t: t.sum(1).sum(0))[0])
+    assert [l["kernels"] for l in total.launches] == [["R_8192_1_0"], ["R_1_1"]]
+
+
 def _value_and_its_row_sums(x, m):
     """x*m + x as one root and the row sums of the same expression, written out again, as another."""
     return [x * m + x, (x * m + x).sum(1)]
