@@ -2529,6 +2529,15 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       int64_t lines = 1;
       for (const auto& l2 : r2.loops) lines *= l2.extent;
       if (!ok || loads.empty() || r1.rloop.extent * outer->extent > 8192 || lines < 1024) continue;
+      // the two loop variables may appear in load indices only (not as values: an iota, a mask by position)
+      std::function<bool(const Node&)> as_value = [&](const Node& n) {
+        if (n.op == Op::Load) return false;
+        if ((n.op == Op::Var || n.op == Op::Wildcard) && (n.name == outer->var || n.name == r1.rloop.var)) return true;
+        for (const auto& a : n.args)
+          if (a && as_value(*a)) return true;
+        return false;
+      };
+      if (as_value(*r1.value)) continue;
       NestKernel m = r1;
       m.value = rename(r1.value, {{outer->var, make_i64(0)}});
       m.rloop.extent = r1.rloop.extent * outer->extent;

@@ -69,7 +69,11 @@ double estimate_us(const GemmShape& s, const Candidate& c, int split) {
   const int64_t ksteps = ceil_div(ceil_div(s.K, c.tile.bk), split);
   const double wg_flops = 2.0 * c.tile.bm * c.tile.bn * static_cast<double>(ksteps) * c.tile.bk;
   const double slots = cus * c.wgs_per_cu;
-  const double round_us = slots * wg_flops / (c.rate * 1e6);
+  // with at most four k-steps a workgroup is all fill and drain: the small tiles then run at
+  // the same rate, and the one that pads less wins (the second convolution's input gradient,
+  // 288 rows and K = 64: 27.1 us with 64x64 tiles, 24.8 us with 32x64)
+  const double rate = (ksteps <= 4 && c.tile.bm * c.tile.bn <= 64 * 64) ? 105.0 : c.rate;
+  const double round_us = slots * wg_flops / (rate * 1e6);
   const int64_t full = wgs / static_cast<int64_t>(slots);
   const int64_t rest = wgs - full * static_cast<int64_t>(slots);
   double us = static_cast<double>(full) * round_us;
