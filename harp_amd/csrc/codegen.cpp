@@ -1631,7 +1631,7 @@ NodePtr replace_loads(const NodePtr& n, const std::string& buf, const NodePtr& w
   return c;
 }
 
-std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C) {
+std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C, bool same_space = false) {
   if (P.rkind != ReduceKind::None || C.rkind != ReduceKind::None) return std::nullopt;
   // a pure gather stays one: contractions and window reductions fold gathers (and chains of them)
   // into their loaders in their own way, which a gather that computes would be lost to
@@ -1657,12 +1657,53 @@ std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C)
     idx = a;
   }
   if (!idx) return std::nullopt;
+  // the new C: (split) loops, P's value (cast to the temp's element type) where the temp was read
+  auto build = [&](const std::map<std::string, NodePtr>& p_map, const std::map<std::string, NodePtr>& c_map,
+                   const std::map<std::string, std::vector<Loop>>& c_split) {
+    NodePtr pv = rename(P.value, p_map);
+    if (!(P.out_dtype.ty == Ty::F32 && infer_ty(*P.value, nullptr) == Ty::F32)) {
+      auto cast = make(Op::Cast, {pv});
+      cast->dtype = P.out_dtype;
+      pv = cast;
+    }
+    NodePtr value = replace_loads(rename(C.value, c_map), P.out_buf, pv);
+    NodePtr body = make(Op::Store, {make_var(C.out_buf), rename(C.out_index, c_map), value});
+    for (size_t i = C.loops.size(); i-- > 0;) {
+      auto it = c_split.find(C.loops[i].var);
+      if (it == c_split.end()) {
+        body = make_range(C.loops[i].var, C.loops[i].extent, body);
+      } else {
+        for (size_t j = it->second.size(); j-- > 0;) body = make_range(it->second[j].var, it->second[j].extent, body);
+      }
+    }
+    std::vector<Param> params;
+    std::set<std::string> have;
+    for (const auto& pp : C.params)
+      if (pp.name != P.out_buf && have.insert(pp.name).second) params.push_back(pp);
+    // P's operands go in front of C's output (immutable parameters first, as kernels list them)
+    std::vector<Param> ins;
+    for (const auto& pp : P.params)
+      if (pp.dtype.is_ptr() && !pp.mut_ && have.insert(pp.name).second) ins.push_back(pp);
+    size_t first_mut = 0;
+    while (first_mut < params.size() && !params[first_mut].mut_) ++first_mut;
+    params.insert(params.begin() + static_cast<long>(first_mut), ins.begin(), ins.end());
+    Inlined r;
+    r.kernel = make_kernel(C.name, params, body);
+    return r;
+  };
   {
-    // the same index space already: the ordinary fusion takes it
+    // the same index space already: the ordinary fusion takes neighbours; a reader far away
+    // (`same_space`) evaluates P at its own loop variables
     bool same = P.loops.size() == C.loops.size();
     for (size_t i = 0; same && i < P.loops.size(); ++i)
       same = P.loops[i].extent == C.loops[i].extent && idx->of(C.loops[i].var) == (*strides)[i] * (P.loops[i].extent > 1 ? 1 : 0);
-    if (same) return std::nullopt;
+    if (same) {
+      if (!same_space) return std::nullopt;
+      std::map<std::string, NodePtr> p_map;
+      for (size_t i = 0; i < P.loops.size(); ++i) p_map[P.loops[i].var] = make_var(C.loops[i].var);
+      return build(p_map, {}, {});
+    }
+    if (same_space) return std::nullopt;
   }
   // C's terms of the index, ascending; each must rise above what the smaller ones reach
   struct Term { std::string var; int64_t c, ext; };
@@ -1740,37 +1781,7 @@ std::optional<Inlined> inline_producer(const NestKernel& P, const NestKernel& C)
     if (top > e - 1) return std::nullopt;
     p_map[P.loops[q].var] = sum ? sum : make_i64(0);
   }
-  // the new C: split loops, P's value (cast to the temp's element type) where the temp was read
-  NodePtr pv = rename(P.value, p_map);
-  if (!(P.out_dtype.ty == Ty::F32 && infer_ty(*P.value, nullptr) == Ty::F32)) {
-    auto cast = make(Op::Cast, {pv});
-    cast->dtype = P.out_dtype;
-    pv = cast;
-  }
-  NodePtr value = replace_loads(rename(C.value, c_map), P.out_buf, pv);
-  NodePtr body = make(Op::Store, {make_var(C.out_buf), rename(C.out_index, c_map), value});
-  for (size_t i = C.loops.size(); i-- > 0;) {
-    auto it = c_split.find(C.loops[i].var);
-    if (it == c_split.end()) {
-      body = make_range(C.loops[i].var, C.loops[i].extent, body);
-    } else {
-      for (size_t j = it->second.size(); j-- > 0;) body = make_range(it->second[j].var, it->second[j].extent, body);
-    }
-  }
-  std::vector<Param> params;
-  std::set<std::string> have;
-  for (const auto& pp : C.params)
-    if (pp.name != P.out_buf && have.insert(pp.name).second) params.push_back(pp);
-  // P's operands go in front of C's output (immutable parameters first, as kernels list them)
-  std::vector<Param> ins;
-  for (const auto& pp : P.params)
-    if (pp.dtype.is_ptr() && !pp.mut_ && have.insert(pp.name).second) ins.push_back(pp);
-  size_t first_mut = 0;
-  while (first_mut < params.size() && !params[first_mut].mut_) ++first_mut;
-  params.insert(params.begin() + static_cast<long>(first_mut), ins.begin(), ins.end());
-  Inlined r;
-  r.kernel = make_kernel(C.name, params, body);
-  return r;
+  return build(p_map, c_map, c_split);
 }
 
 
@@ -2026,6 +2037,38 @@ void rewrite_for_readers(const Node& program, const GenOptions& opt, std::vector
           auto nc = extract_nest(*(*kernels)[reader]);
           if (!nc) continue;
           auto in = inline_producer(*np, *nc);
+          // A reader over the same index space that the ordinary fusion cannot reach (a reduce
+          // or a contraction lies between the two: the backward pass reading what the forward
+          // pass saved) evaluates a cheap producer again instead of reading its stored result,
+          // when what the producer reads is kept in memory for later readers anyway: one store
+          // and one load of the whole tensor less, the same operations on the same values.
+          if (!in && opt.rematerialize && reader > p + 1) {
+            bool barrier = false;
+            for (size_t m = p + 1; m < reader && !barrier; ++m) {
+              auto nm = extract_nest(*(*kernels)[m]);
+              barrier = !nm || nm->rkind != ReduceKind::None;
+            }
+            std::function<size_t(const Node&)> size_of = [&](const Node& n) {
+              size_t c = 1;
+              for (const auto& a : n.args)
+                if (a && n.op != Op::Load) c += size_of(*a);
+              return c;
+            };
+            std::vector<LoadRef> pl;
+            collect_loads(*np->value, pl);
+            bool kept = barrier && pl.size() <= 2 && size_of(*np->value) <= 8;
+            for (const auto& lr : pl) {
+              if (!kept) break;
+              if (lr.load->args[0]->op != Op::Var) { kept = false; break; }
+              const std::string& b = lr.load->args[0]->name;
+              if (!is_temp(b)) continue;
+              bool later = false;          // read by this reader already, or by a kernel after it
+              for (size_t q = reader; q < kernels->size() && !later; ++q)
+                for (const auto& pq : (*kernels)[q]->params) later = later || (pq.dtype.is_ptr() && !pq.mut_ && pq.name == b);
+              kept = later;
+            }
+            if (kept) in = inline_producer(*np, *nc, true);
+          }
           if (!in) continue;
           rewritten->push_back(in->kernel);
           (*kernels)[reader] = in->kernel.get();

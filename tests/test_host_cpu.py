@@ -696,6 +696,27 @@ def test_bias_gradient_chain_is_two_launches(frontend):
     assert [l["kernels"] for l in total.launches] == [["R_8192_1_0"], ["R_1_1"]]
 
 
+def test_backward_pass_recomputes_cheap_saved_values(frontend):
+    """The MLP training step: the exact tanh saves exp(-2x), 1 + exp(-2x) and the activation for the
+    backward pass.  The second is one addition away from the first, which stays in memory
+    anyway: its backward reader evaluates it again instead of loading it, and the forward
+    contraction's epilogue no longer stores it (one tensor less per tanh layer);
+    rematerialize=0 keeps every saved value."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config4_inputs(*wl.mlp_sizes(False))
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config4_graph(*ts, lr=1e-3))[0]
+    stored = lambda plan: sorted(b["name"] for b in plan.buffers if b["role"] == "temp" and not b["elided"])
+    with_remat, without = hb.render_program(ast), hb.render_program(ast, "rematerialize=0")
+    assert len(with_remat.launches) == len(without.launches)
+    gone = set(stored(without)) - set(stored(with_remat))
+    assert len(gone) == 2 and set(stored(with_remat)) <= set(stored(without)), gone
+    fwd = [l for l in with_remat.launches if "epilogue=8" in l["schedule"]]
+    fwd0 = [l for l in without.launches if "epilogue=8" in l["schedule"]]
+    assert len(fwd) == len(fwd0) == 2 and all(len(a["args"]) + 1 == len(b["args"]) for a, b in zip(fwd, fwd0))
+
+
 def _value_and_its_row_sums(x, m):
     """x*m + x as one root and the row sums of the same expression, written out again, as another."""
     return [x * m + x, (x * m + x).sum(1)]
