@@ -274,7 +274,7 @@ __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long
   } else if (ALONG_K) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const bool ok = rows.ok[0] & (k + e < kend);
+      const bool ok = (!EDGE_R || rows.ok[0]) & (!EDGE_K || k + e < kend);     // (no test where the tiles have no edge)
 #if EH_LOAD_BRANCH
       if (ok) v[e] = ELEM::val(p, rows.row[0], ELEM::kk(bz, k + e));
 #else
@@ -283,11 +283,11 @@ __device__ __forceinline__ eh_f4v eh_tile_load(const float* __restrict__ p, long
 #endif
     }
   } else {
-    const bool kok = k < kend;
+    const bool kok = !EDGE_K || k < kend;
     const typename ELEM::Kk kinfo = ELEM::kk(bz, kok ? k : 0);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const bool ok = rows.ok[e] & kok;
+      const bool ok = (!EDGE_R || rows.ok[e]) & kok;
 #if EH_LOAD_BRANCH
       if (ok) v[e] = ELEM::val(p, rows.row[e], kinfo);
 #else
