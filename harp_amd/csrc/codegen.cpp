@@ -3302,7 +3302,8 @@ struct GroupEmitter {
     std::string s;
     if (g.rows.empty()) return s;
     if (g.rows.size() == 1) return "  const idx_t r0 = " + rowvar + ";\n";
-    s += "  idx_t eh_rem = " + rowvar + ";\n";
+    // (never negative: lets the compiler take the cheaper unsigned forms of the divisions)
+    s += "  idx_t eh_rem = " + rowvar + ";\n  __builtin_assume(eh_rem >= 0);\n";
     for (size_t i = g.rows.size(); i-- > 0;) {
       if (i == 0) s += "  const idx_t r0 = eh_rem;\n";
       else {
@@ -3397,7 +3398,7 @@ struct GroupEmitter {
     os << "  for (idx_t eh_g = (idx_t)blockIdx.x * " << block << " + threadIdx.x; eh_g < eh_nvec; eh_g += eh_stride) {\n";
     os << "  const idx_t eh_p = eh_g * " << V << ";\n";
     if (!g.rows.empty()) {
-      os << "  const idx_t eh_row = eh_p / " << g.C << ";\n  const idx_t c0 = eh_p % " << g.C << ";\n";
+      os << "  __builtin_assume(eh_p >= 0);\n  const idx_t eh_row = eh_p / " << g.C << ";\n  const idx_t c0 = eh_p % " << g.C << ";\n";
       os << row_decode("eh_row");
     } else {
       os << "  const idx_t c0 = eh_p;\n";
@@ -3816,7 +3817,7 @@ struct SerialReduce {
   std::string epilogue_function() const { return epi ? epi->function : std::string(); }
 
   std::string decode(const std::string& ovar) const {
-    std::string t = "  idx_t eh_rem = " + ovar + ";\n";
+    std::string t = "  idx_t eh_rem = " + ovar + ";\n  __builtin_assume(eh_rem >= 0);\n";
     for (size_t i = live.size(); i-- > 0;) {
       t += "  const idx_t " + live[i].var + " = eh_rem % " + std::to_string(live[i].extent) + ";\n";
       if (i) t += "  eh_rem /= " + std::to_string(live[i].extent) + ";\n";
@@ -4049,7 +4050,7 @@ LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestK
   }
   os << "extern \"C\" __global__ void __launch_bounds__(256) " << ls.entry << "(" << sig << ") {\n";
   os << "  const idx_t eh_o = (idx_t)blockIdx.x * 256 + threadIdx.x;\n  if (eh_o >= " << N << ") return;\n";
-  os << "  idx_t eh_rem = eh_o;\n";
+  os << "  idx_t eh_rem = eh_o;\n  __builtin_assume(eh_rem >= 0);\n";
   for (size_t q = live.size(); q-- > 0;) {
     os << "  const idx_t " << live[q].var << " = eh_rem % " << live[q].extent << ";\n";
     if (q) os << "  eh_rem /= " << live[q].extent << ";\n";
