@@ -2975,6 +2975,45 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       auto gl = try_emit_gemm(have_epi ? k0r : k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
       if (!gl.empty()) {
         if (absorbed_name.count(i)) gl.back().kernels.push_back(absorbed_name[i]);
+        // K was split and the next kernel only sums the (dense) result over the batch axis: it
+        // sums the partial tiles of all chunks and all batch elements in one go (chunks lie
+        // above the batch in the scratch buffer, so the two walk as one axis), and the launch
+        // that would add the chunks up goes
+        if (gl.size() == 2 && !have_epi && !absorbed_name.count(i) && opt.fuse && opt.reindex && have_table) {
+          size_t j = i + 1;
+          while (j < kernels.size() && (absorbed.count(j) || folded_kernels.count(j))) ++j;
+          auto gs = match_gemm(k0);
+          const std::string& scratch = gl[0].arg_bufs.back();
+          if (j < kernels.size() && nests[j] && gs && gs->batch > 1 && gemm_output_dense(*gs) &&
+              gl[0].grid[1] > 1 && scratch.rfind("eh_part_", 0) == 0) {
+            NestKernel& r2 = *nests[j];
+            const Node& v2 = *r2.value;
+            auto ra = v2.op == Op::Load && v2.count == 1 && v2.args[0]->op == Op::Var && v2.args[0]->name == k0.out_buf
+                          ? affine_of(*v2.args[1]) : std::nullopt;
+            const int64_t tile = gs->M * gs->N;
+            bool ok = r2.rkind == ReduceKind::Sum && ra && ra->c == 0 && r2.acc_dtype.ty == Ty::F32 &&
+                      r2.rloop.extent == gs->batch && ra->of(r2.rloop.var) == tile && role_of(k0.out_buf) == "temp" &&
+                      readers[k0.out_buf] == std::vector<size_t>{j} && !(opt.gemm && gemm_shaped(r2, opt));
+            // the other loops of r2 stay inside one tile
+            int64_t reach = 0;
+            if (ok)
+              for (const auto& l : r2.loops) {
+                if (l.extent <= 1) continue;
+                ok = ok && ra->of(l.var) > 0;
+                reach += ra->of(l.var) * (l.extent - 1);
+              }
+            if (ok && reach < tile) {
+              const int64_t S = gl[0].grid[1];
+              std::map<std::string, NodePtr> to_scratch{{k0.out_buf, make_var(scratch)}};
+              r2.value = rename(r2.value, to_scratch);
+              r2.rloop.extent *= S;
+              for (auto& pp : r2.params)
+                if (pp.name == k0.out_buf) pp.name = scratch;
+              plan.elided.insert(k0.out_buf);
+              gl.pop_back();
+            }
+          }
+        }
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
         i = have_epi ? after : i + 1;
         continue;
@@ -3876,7 +3915,8 @@ struct SerialReduce {
     return ls;
   }
 
-  bool wants_split() const { return k.rloop.extent >= 512 && N <= (1 << 18); }
+  // (two launches pay only where there is enough to read: a megabyte goes through one)
+  bool wants_split() const { return k.rloop.extent >= 512 && N <= (1 << 18) && N * k.rloop.extent >= (int64_t{1} << 21); }
   bool wants_columns() const { return k.rloop.extent >= 32 && N <= (1 << 16); }
 
   // One launch; a workgroup owns 64 outputs and RG threads share each output's reduction
