@@ -492,6 +492,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "guard_branches") o.guard_branches = as_int() != 0;
     else if (k == "ranged_loads") o.ranged_loads = as_int() != 0;
     else if (k == "rematerialize") o.rematerialize = as_int() != 0;
+    else if (k == "merge_launches") o.merge_launches = as_int() != 0;
     else if (k == "lanes") o.lanes = std::max(1, as_int());
     else if (k == "lane_us") o.lane_us = std::max(0, as_int());
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;

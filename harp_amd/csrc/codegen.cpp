@@ -1102,6 +1102,8 @@ Canon canon_as(const NestKernel& k, StageKind kind) {
 namespace {
 LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std::string, size_t>& buf_elems);
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan, const EpilogueSpec* epi = nullptr);
+bool serial_reduce_is_one_launch(const NestKernel& k, const GenOptions& opt);
+LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions& opt);
 LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestKernel*>& chain, const GenOptions& opt,
                               const std::map<std::string, size_t>& elems);
 }  // namespace
@@ -2937,6 +2939,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     return have_epi;
   };
 
+  std::vector<LaunchSpec> held_back;       // independent final reductions, issued together at the end
   size_t i = 0;
   while (i < kernels.size()) {
     if (folded_kernels.count(i) || absorbed.count(i)) {
@@ -3032,6 +3035,27 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           dense_strides(k0, &numel))
         have_epi = build_epilogue(i, k0, numel, false, k0r, epi, after);
       emit_serial_reduce(k0, opt, &plan, have_epi ? &epi : nullptr);
+      // A one-launch reduce at the end of its chain (nothing later reads what it writes or
+      // writes what it reads: a parameter's update) can run whenever its inputs are ready:
+      // it is held back and issued together with the others of its kind as one launch.
+      if (opt.fuse && opt.reindex && opt.merge_launches && have_table && serial_reduce_is_one_launch(k0, opt)) {
+        const size_t next = have_epi ? after : i + 1;
+        std::set<std::string> written{k0.out_buf};
+        for (size_t q = i + 1; q < next; ++q)
+          if (nests[q]) written.insert(nests[q]->out_buf);
+        bool sink = true;
+        for (const auto& b : written)
+          for (size_t r : readers[b]) sink = sink && r < next;
+        const LaunchSpec& ls = plan.launches.back();
+        for (size_t m = next; m < kernels.size() && sink; ++m)
+          for (const auto& pm : kernels[m]->params)
+            if (pm.dtype.is_ptr() && pm.mut_)
+              sink = sink && std::find(ls.arg_bufs.begin(), ls.arg_bufs.end(), pm.name) == ls.arg_bufs.end();
+        if (sink) {
+          held_back.push_back(plan.launches.back());
+          plan.launches.pop_back();
+        }
+      }
       i = have_epi ? after : i + 1;
       continue;
     }
@@ -3083,6 +3107,8 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
     plan.launches.push_back(emit_group(g, opt, elems));
   }
+  if (held_back.size() >= 2) plan.launches.push_back(merge_launches(held_back, opt));
+  else for (auto& ls : held_back) plan.launches.push_back(std::move(ls));
   // constant inputs no launch binds any more need not exist
   for (const auto& c : consts) {
     bool bound = false;
@@ -4151,6 +4177,71 @@ void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan*
   } else {
     plan->launches.push_back(sr.single());
   }
+}
+
+bool serial_reduce_is_one_launch(const NestKernel& k, const GenOptions& opt) { return !SerialReduce(k, opt).wants_split(); }
+
+// Several launches of the serial-reduce family that do not depend on each other, as one launch:
+// each becomes a device function in a namespace of its own (its index type, its epilogue), and
+// the merged kernel hands every workgroup to the part whose range of workgroup numbers it falls
+// into.  Every dependent launch costs about four microseconds whatever it computes, so the
+// updates of a training step's parameters, each a few workgroups, are worth taking together.
+LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions& opt) {
+  LaunchSpec out;
+  const std::string head = hdr(opt);
+  unsigned block = 0;
+  for (const auto& p : parts) block = std::max(block, p.block[0]);
+  out.entry = parts.front().entry + "_and_" + std::to_string(parts.size() - 1);
+  std::ostringstream os, sig, body;
+  os << head;
+  unsigned first = 0;
+  for (size_t i = 0; i < parts.size(); ++i) {
+    const LaunchSpec& p = parts[i];
+    if (p.source.rfind(head, 0) != 0 || p.grid[1] != 1 || p.grid[2] != 1 || p.block[1] != 1 || p.block[2] != 1 || p.block[0] % 64 || p.lds_bytes)
+      throw Error("internal: launch '" + p.entry + "' cannot be merged");
+    std::string text = p.source.substr(head.size());
+    const std::string open = "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(p.block[0]) + ") " + p.entry + "(";
+    const size_t at = text.find(open);
+    const size_t close = at == std::string::npos ? at : text.find(") {\n", at);
+    if (close == std::string::npos) throw Error("internal: launch '" + p.entry + "' has no entry point to merge");
+    const std::string params = text.substr(at + open.size(), close - at - open.size());
+    text.replace(at, open.size(), "__device__ __forceinline__ void eh_run(const unsigned eh_bx, ");
+    for (size_t q = text.find("blockIdx.x"); q != std::string::npos; q = text.find("blockIdx.x", q)) text.replace(q, 10, "eh_bx");
+    const std::string ns = "eh_part" + std::to_string(i);
+    os << "namespace " << ns << " {\n" << text << "}  // namespace " << ns << "\n";
+    // the part's parameters, renamed, in the merged signature; the same names in the call
+    std::string call;
+    size_t from = 0, n = 0;
+    while (from < params.size()) {
+      size_t comma = params.find(", ", from);
+      if (comma == std::string::npos) comma = params.size();
+      const std::string one = params.substr(from, comma - from);
+      const size_t sp = one.rfind(' ');
+      const std::string name = "p" + std::to_string(i) + "_" + one.substr(sp + 1);
+      sig << (sig.tellp() > 0 ? ", " : "") << one.substr(0, sp + 1) << name;
+      call += ", " + name;
+      from = comma + 2;
+      ++n;
+    }
+    if (n != p.arg_bufs.size()) throw Error("internal: launch '" + p.entry + "' lists " + std::to_string(p.arg_bufs.size()) + " buffers for " + std::to_string(n) + " parameters");
+    body << "  if (blockIdx.x < " << first + p.grid[0] << "u) {\n    if (threadIdx.x < " << p.block[0] << "u) " << ns << "::eh_run(blockIdx.x - "
+         << first << "u" << call << ");\n    return;\n  }\n";
+    first += p.grid[0];
+    for (size_t a = 0; a < p.arg_bufs.size(); ++a) {
+      out.arg_bufs.push_back(p.arg_bufs[a]);
+      out.arg_min_bytes.push_back(a < p.arg_min_bytes.size() ? p.arg_min_bytes[a] : 0);
+    }
+    for (const auto& kn : p.kernels) out.kernels.push_back(kn);
+    out.algo_bytes += p.algo_bytes;
+    out.flops += p.flops;
+    out.schedule += (i ? " + " : "together(") + p.schedule;
+  }
+  out.schedule += ")";
+  os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << out.entry << "(" << sig.str() << ") {\n" << body.str() << "}\n";
+  out.source = os.str();
+  out.grid[0] = first;
+  out.block[0] = block;
+  return out;
 }
 
 }  // namespace

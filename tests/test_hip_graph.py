@@ -134,10 +134,10 @@ def test_lanes_change_nothing_but_the_timing(hip):
     hb = hip
     dev = hb.HipDevice(0)
     want = None
-    for options in (None, "lanes=2", "lanes=4,lane_us=0"):
+    for options in (None, "lanes=2,merge_launches=0", "lanes=4,lane_us=0,merge_launches=0", "lanes=4,lane_us=0"):
         prog, sets, arg_names, outs, arrays = _cnn_sets(hb, dev, 16, seed=94, options=options)
         lanes = {l["lane"] for l in prog.launches}
-        assert (len(lanes) == 1) == (options is None), lanes
+        assert (len(lanes) == 1) == (options is None) or "merge_launches" not in options, lanes
         for _ in range(3):
             prog.run(sets[0][0], sync=False)
         dev.sync()

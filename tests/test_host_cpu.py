@@ -359,7 +359,11 @@ def test_config4_training_step_plan(frontend):
     assert len(plan.launches) < len(plain.args) // 2
     scheds = [l["schedule"] for l in plan.launches]
     assert sum(s.startswith("mfma32x32x2(") for s in scheds) == 8      # 3 forward, 3 dW, 2 dX
-    assert sum("-reduce(" in s for s in scheds) == 3                   # bias gradients (column sums)
+    assert sum(s.count("-reduce(") for s in scheds) == 3               # bias gradients (column sums) ...
+    together = [l for l in plan.launches if l["schedule"].startswith("together(")]
+    assert len(together) == 1 and len(together[0]["kernels"]) == 9      # ... and their updates, issued as one launch
+    apart = hb.render_program(prog_ast, {"merge_launches": 0})
+    assert len(apart.launches) == len(plan.launches) + 2 and not any("together(" in l["schedule"] for l in apart.launches)
     # bias add and activation chains ride on the forward contractions' accumulators
     epi = [l for l in plan.launches if "epilogue=" in l["schedule"]]
     assert len(epi) >= 3 and all("eh_epilogue(" in l["source"] for l in epi)
@@ -569,7 +573,7 @@ def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
     arrays = wl.config5_inputs(8, *wl.cnn_sizes(False)[1:])
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     prog_ast, arg_names, outs, consts, _ = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))
-    plan = hb.render_program(prog_ast, "lanes=3,lane_us=0")
+    plan = hb.render_program(prog_ast, "lanes=3,lane_us=0,merge_launches=0")
     assert _lane_plan_is_sound(plan.launches) == 3
     assert sum(l["lane"] > 0 for l in plan.launches) >= 8
     roles = {b["name"]: b["role"] for b in plan.buffers}
@@ -583,13 +587,15 @@ def test_training_step_launches_are_spread_over_lanes_soundly(frontend):
         seen.update(a for a, w in zip(l["args"], l["written"]) if w)
     assert not read_first, read_first                      # nothing but inputs is read before it is written
     assert {n for n, r in roles.items() if r == "output"} <= written
-    one = hb.render_program(prog_ast, "lanes=1")
+    one = hb.render_program(prog_ast, "lanes=1,merge_launches=0")
     assert all(l["lane"] == 0 and not l["waits"] for l in one.launches)
     assert sorted(l["entry"] for l in one.launches) == sorted(l["entry"] for l in plan.launches)
-    two = hb.render_program(prog_ast, "lanes=2")
+    two = hb.render_program(prog_ast, "lanes=2,merge_launches=0")
     assert _lane_plan_is_sound(two.launches) == 2
-    default = hb.render_program(prog_ast)                  # one lane unless asked (or tuned) otherwise
+    default = hb.render_program(prog_ast, "merge_launches=0")   # one lane unless asked (or tuned) otherwise
     assert [l["entry"] for l in default.launches] == [l["entry"] for l in one.launches]
+    merged = hb.render_program(prog_ast, "lanes=2")        # with the updates issued together: still sound
+    assert _lane_plan_is_sound(merged.launches) in (1, 2) and len(merged.launches) < len(two.launches)
     # a single softmax has nothing to spread
     from harp_amd import workloads
     sm = hb.render_program(workloads.lower_with_table([(64, 256)], workloads.config2_graph)[0])
