@@ -80,6 +80,10 @@ template <class Op, int T, class V> __device__ __forceinline__ V eh_row_reduce(V
   return s;
 }
 
+std::string kernel_header() {
+  return "// generated for gfx950 by eclat backend-hip\n#ifndef __HIPCC_RTC__\n#include <hip/hip_runtime.h>\n#endif\n" + preamble();
+}
+
 // ---------------------------------------------------------------------------------------------
 // types and literals
 // ---------------------------------------------------------------------------------------------
@@ -350,10 +354,7 @@ struct ExprRenderer {
   }
 };
 
-std::string hdr(const GenOptions&) {
-  return "// generated for gfx950 by eclat backend-hip\n#ifndef __HIPCC_RTC__\n#include <hip/hip_runtime.h>\n#endif\n" +
-         preamble();
-}
+std::string hdr(const GenOptions&) { return kernel_header(); }
 
 // ---------------------------------------------------------------------------------------------
 // statement-by-statement rendering (kernels no schedule recognises)
@@ -2940,6 +2941,28 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
   };
 
   std::vector<LaunchSpec> held_back;       // independent final reductions, issued together at the end
+  // The launch just planned for kernels [i, next) (the last of them, when there are two) can run
+  // whenever its inputs are ready if nothing later reads what it writes or writes what it reads
+  // (a parameter's update at the end of its gradient's chain): it is taken out of the sequence.
+  auto hold_back_if_sink = [&](size_t i, size_t next) {
+    if (!(opt.fuse && opt.reindex && opt.merge_launches && have_table) || plan.launches.empty()) return;
+    const LaunchSpec& ls = plan.launches.back();
+    if (ls.grid[1] != 1 || ls.grid[2] != 1 || ls.lds_bytes || ls.block[0] % 64 || ls.source.rfind(kernel_header(), 0) != 0) return;
+    std::set<std::string> written;
+    for (size_t q = i; q < next; ++q)
+      if (nests[q]) written.insert(nests[q]->out_buf);
+      else return;
+    bool sink = true;
+    for (const auto& b : written)
+      for (size_t r : readers[b]) sink = sink && r < next;
+    for (size_t m = next; m < kernels.size() && sink; ++m)
+      for (const auto& pm : kernels[m]->params)
+        if (pm.dtype.is_ptr() && pm.mut_)
+          sink = sink && std::find(ls.arg_bufs.begin(), ls.arg_bufs.end(), pm.name) == ls.arg_bufs.end();
+    if (!sink) return;
+    held_back.push_back(plan.launches.back());
+    plan.launches.pop_back();
+  };
   size_t i = 0;
   while (i < kernels.size()) {
     if (folded_kernels.count(i) || absorbed.count(i)) {
@@ -3017,7 +3040,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             }
           }
         }
+        const bool two = gl.size() == 2;
         for (auto& ls : gl) plan.launches.push_back(std::move(ls));
+        if (two && !absorbed_name.count(i)) hold_back_if_sink(i, have_epi ? after : i + 1);   // the launch that sums the chunks (and updates the weight)
         i = have_epi ? after : i + 1;
         continue;
       }
@@ -3038,24 +3063,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       // A one-launch reduce at the end of its chain (nothing later reads what it writes or
       // writes what it reads: a parameter's update) can run whenever its inputs are ready:
       // it is held back and issued together with the others of its kind as one launch.
-      if (opt.fuse && opt.reindex && opt.merge_launches && have_table && serial_reduce_is_one_launch(k0, opt)) {
-        const size_t next = have_epi ? after : i + 1;
-        std::set<std::string> written{k0.out_buf};
-        for (size_t q = i + 1; q < next; ++q)
-          if (nests[q]) written.insert(nests[q]->out_buf);
-        bool sink = true;
-        for (const auto& b : written)
-          for (size_t r : readers[b]) sink = sink && r < next;
-        const LaunchSpec& ls = plan.launches.back();
-        for (size_t m = next; m < kernels.size() && sink; ++m)
-          for (const auto& pm : kernels[m]->params)
-            if (pm.dtype.is_ptr() && pm.mut_)
-              sink = sink && std::find(ls.arg_bufs.begin(), ls.arg_bufs.end(), pm.name) == ls.arg_bufs.end();
-        if (sink) {
-          held_back.push_back(plan.launches.back());
-          plan.launches.pop_back();
-        }
-      }
+      hold_back_if_sink(i, have_epi ? after : i + 1);
       i = have_epi ? after : i + 1;
       continue;
     }
@@ -3107,8 +3115,15 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
     plan.launches.push_back(emit_group(g, opt, elems));
   }
-  if (held_back.size() >= 2) plan.launches.push_back(merge_launches(held_back, opt));
-  else for (auto& ls : held_back) plan.launches.push_back(std::move(ls));
+  {
+    // by workgroup size: a part's surplus work-items leave at once, but they are launched all the same
+    std::map<unsigned, std::vector<LaunchSpec>> by_block;
+    for (auto& ls : held_back) by_block[ls.block[0]].push_back(std::move(ls));
+    for (auto& kv : by_block) {
+      if (kv.second.size() >= 2) plan.launches.push_back(merge_launches(kv.second, opt));
+      else plan.launches.push_back(std::move(kv.second.front()));
+    }
+  }
   // constant inputs no launch binds any more need not exist
   for (const auto& c : consts) {
     bool bound = false;

@@ -95,5 +95,7 @@ std::string render_expr_text(const Node& e);
 
 // Shared preamble (vector type, cross-lane reductions).
 const std::string& preamble();
+// What every generated translation unit of the elementwise / reduce schedules starts with.
+std::string kernel_header();
 
 }  // namespace eh

@@ -573,9 +573,9 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
       fin.arg_min_bytes.push_back(4 * c_elems);
     }
     std::ostringstream fs;
-    fs << "// generated for gfx950 by eclat backend-hip: sum of split-K partial tiles\n";
+    fs << kernel_header() << "// sum of split-K partial tiles\n";
     if (epilogue) {
-      fs << "#ifndef __HIPCC_RTC__\n#include <hip/hip_runtime.h>\n#endif\n" << epilogue->function;
+      fs << epilogue->function;
       for (size_t i = 0; i < epilogue->bufs.size(); ++i) {
         fin.arg_bufs.push_back(epilogue->bufs[i]);
         fin.arg_min_bytes.push_back(epilogue->min_bytes[i]);
