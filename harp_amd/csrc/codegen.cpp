@@ -2154,9 +2154,10 @@ void rewrite_for_readers(const Node& program, const GenOptions& opt, std::vector
 // concurrently; a launch waits for the launches on other lanes whose buffers it reads or
 // overwrites (`waits`), and the executor joins the lanes at the end of the program.  The results
 // do not depend on the lanes: every launch still sees exactly the inputs it would have seen.
-void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, const GenOptions& opt) {
+// Which of its buffers each launch writes: the outputs of the lowered kernels it covers; a scratch
+// buffer the plan added is written by the first launch that binds it and read by the later ones.
+void mark_written(ProgramPlan* plan, const std::vector<const Node*>& kernels) {
   auto& L = plan->launches;
-  const size_t n = L.size();
   std::map<std::string, const Node*> by_name;
   for (const Node* k : kernels) by_name[k->name] = k;
   // written: outputs of the lowered kernels a launch covers; a scratch buffer the plan added is
@@ -2182,6 +2183,56 @@ void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, co
       else if (!declared && scratch_seen.insert(b).second) ls.arg_written[a] = 1;
     }
   }
+}
+
+// Launches of the elementwise / reduce schedules that do not depend on each other are issued as one
+// launch (merge_launches).  A launch that could be merged is held until a launch that depends on it
+// (reads what it writes, writes what it reads or writes) comes up; launches that depend on nothing
+// held pass it by, which only changes the order among independent launches.  What is held at
+// that point goes out together, grouped by workgroup size.
+void issue_independent_launches_together(ProgramPlan* plan, const std::vector<const Node*>& kernels, const GenOptions& opt) {
+  if (!(opt.fuse && opt.reindex && opt.merge_launches) || plan->launches.size() < 3) return;
+  mark_written(plan, kernels);
+  const std::string head = kernel_header();
+  auto mergeable = [&](const LaunchSpec& ls) {
+    if (ls.grid[1] != 1 || ls.grid[2] != 1 || ls.block[1] != 1 || ls.block[2] != 1 || ls.block[0] % 64 || ls.lds_bytes) return false;
+    if (ls.source.rfind(head, 0) != 0 || ls.schedule.rfind("together(", 0) == 0 || ls.kernels.empty()) return false;
+    const std::string open = "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(ls.block[0]) + ") " + ls.entry + "(";
+    const size_t at = ls.source.find(open);
+    return at != std::string::npos && ls.source.find("__global__", at + open.size()) == std::string::npos &&
+           ls.source.find("blockIdx.y") == std::string::npos && ls.source.find("blockDim") == std::string::npos;
+  };
+  auto conflict = [](const LaunchSpec& a, const LaunchSpec& b) {
+    for (size_t i = 0; i < a.arg_bufs.size(); ++i)
+      for (size_t j = 0; j < b.arg_bufs.size(); ++j)
+        if (a.arg_bufs[i] == b.arg_bufs[j] && (a.arg_written[i] || b.arg_written[j])) return true;
+    return false;
+  };
+  std::vector<LaunchSpec> in = std::move(plan->launches), out, held;
+  auto flush = [&] {
+    std::map<unsigned, std::vector<LaunchSpec>> by_block;
+    for (auto& ls : held) by_block[ls.block[0]].push_back(std::move(ls));
+    held.clear();
+    for (auto& kv : by_block) {
+      if (kv.second.size() >= 2) out.push_back(merge_launches(kv.second, opt));
+      else out.push_back(std::move(kv.second.front()));
+    }
+  };
+  for (auto& ls : in) {
+    bool dep = false;
+    for (const auto& h : held) dep = dep || conflict(ls, h);
+    if (dep) flush();
+    if (mergeable(ls)) held.push_back(std::move(ls));
+    else out.push_back(std::move(ls));
+  }
+  flush();
+  plan->launches = std::move(out);
+}
+
+void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, const GenOptions& opt) {
+  auto& L = plan->launches;
+  const size_t n = L.size();
+  mark_written(plan, kernels);
   plan->lanes = 1;
   for (auto& ls : L) { ls.lane = 0; ls.waits.clear(); }
   if (opt.lanes < 2 || n < 8) return;
@@ -3132,6 +3183,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     if (!bound) plan.elided.insert(c.first);
   }
   // a launch that covers a kernel which took another one in covers that one too
+  // (before launches are merged: the covered kernels decide which buffers a launch writes)
   for (auto& ls : plan.launches) {
     const std::vector<std::string> covered = ls.kernels;
     for (const auto& kn : covered)
@@ -3140,6 +3192,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
             std::find(ls.kernels.begin(), ls.kernels.end(), an.second) == ls.kernels.end())
           ls.kernels.push_back(an.second);
   }
+  issue_independent_launches_together(&plan, kernels, opt);
   // A lowered kernel whose output index is the dense index of its loops writes every element of
   // its output; the launch that stores it overwrites a buffer of exactly that size, whatever it
   // held (the executor need not have zero-filled it first).
@@ -4222,6 +4275,8 @@ LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions
     const std::string params = text.substr(at + open.size(), close - at - open.size());
     text.replace(at, open.size(), "__device__ __forceinline__ void eh_run(const unsigned eh_bx, ");
     for (size_t q = text.find("blockIdx.x"); q != std::string::npos; q = text.find("blockIdx.x", q)) text.replace(q, 10, "eh_bx");
+    const std::string own_grid = std::to_string(p.grid[0]) + "u";
+    for (size_t q = text.find("gridDim.x"); q != std::string::npos; q = text.find("gridDim.x", q)) text.replace(q, 9, own_grid);
     const std::string ns = "eh_part" + std::to_string(i);
     os << "namespace " << ns << " {\n" << text << "}  // namespace " << ns << "\n";
     // the part's parameters, renamed, in the merged signature; the same names in the call
