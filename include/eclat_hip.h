@@ -170,7 +170,10 @@ int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
  * order, then scratch temps the plan added (names starting with "eh_").  NULL is allowed for
  * elided buffers and for temps (the program then keeps its own), and bufs may stop anywhere
  * after the last input or output.  sync != 0 waits for completion (the reference's kernels are
- * synchronous); sync == 0 only queues the launches on the device's stream. */
+ * synchronous); sync == 0 only queues the launches on the device's stream.
+ * Different entries of the table must be different buffers (an output must not alias an input):
+ * launches that do not depend on each other by buffer name may run in another order than the
+ * kernels were written, or together. */
 int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,
                                   eh_buffer* const* outputs, int n_outputs, int sync);
