@@ -970,6 +970,63 @@ def test_bias_gradient_chain_matches_the_oracle(frontend, hip, shape):
     assert np.all(np.abs(got - ref) <= 1e-5 * scale) and np.all(np.abs(got - exact) <= 1e-5 * scale)
 
 
+def _independent_roots(a, b, c, d, e):
+    """Three results over different index spaces that have nothing to do with each other, and a
+    column sum that needs the first."""
+    x = a * b + a
+    y = (c - d).maximum(d)
+    z = e.sum(1)
+    return [x, y, z, x.sum(0)]
+
+
+def test_independent_launches_issued_together_match_the_oracle(frontend, hip):
+    """Roots that do not depend on each other become one launch (each part with its own range of
+    workgroups and its own grid-stride loop, several iterations per work-item at this size); the
+    root that needs one of them follows.  Bit-exact against the oracle for the elementwise
+    roots, reduction tolerance for the sums; merge_launches=0 plans them one by one."""
+    import os
+    from harp_amd import workloads as wl
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    shapes = [(1500, 1024), (1500, 1024), (1100, 2048), (1100, 2048), (700, 512)]
+    rng = RNG(77)
+    arrays = [rng.normal(0, 1, s).astype(np.float32) for s in shapes]
+    ts = [frontend.Tensor.input(list(s)) for s in shapes]
+    ast = wl.lower_multi(ts, _independent_roots(*ts))[0]
+    plan = hip.render_program(ast)
+    apart = hip.render_program(ast, {"merge_launches": 0})
+    together = [l for l in plan.launches if l["schedule"].startswith("together(")]
+    assert len(together) == 1 and together[0]["schedule"].count("flat(") == 2 and len(plan.launches) < len(apart.launches), \
+        [l["schedule"] for l in plan.launches]
+    assert together[0]["grid"][0] > 500                      # real grid-stride loops, not one workgroup each
+
+    def run(kind):
+        frontend.set_device_str(kind)
+        old = os.environ.get("ECLAT_HIP_FUSE")
+        os.environ["ECLAT_HIP_FUSE"] = "1"
+        try:
+            tensors = []
+            for a in arrays:
+                t = frontend.Tensor.input(list(a.shape))
+                t.set_data(a)
+                tensors.append(t)
+            roots = _independent_roots(*tensors)
+            frontend.realize_many(roots)
+            return [r.to_numpy() for r in roots]
+        finally:
+            _INPUT_BUFFER_CACHE.clear()
+            if old is None:
+                os.environ.pop("ECLAT_HIP_FUSE", None)
+            else:
+                os.environ["ECLAT_HIP_FUSE"] = old
+
+    ref, got = run("c"), run("hip")
+    for i in (0, 1):
+        assert bits_equal_mod_zero(ref[i], got[i]), i
+    assert np.all(np.abs(got[2].astype(np.float64) - ref[2]) <= 1e-5 * np.abs(arrays[4]).astype(np.float64).sum(1))
+    x = np.abs(arrays[0] * arrays[1] + arrays[0]).astype(np.float64)
+    assert np.all(np.abs(got[3].astype(np.float64) - ref[3]) <= 1e-5 * x.sum(0))
+
+
 def test_config5_with_implicit_gemm_loader(frontend, hip):
     """im2col gathers and layout copies that only contractions read are evaluated inside the
     contractions' tile loaders (no launch, no buffer); option gemm_fold=0 materialises them.
