@@ -2400,6 +2400,54 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     kernels = out;
   }
   if (!plan.buffers.empty() && opt.fuse && opt.reindex) rewrite_for_readers(program, opt, &kernels, &rewritten, &plan);
+  if (!plan.buffers.empty() && opt.fuse && opt.reindex) {
+    // An elementwise kernel separated from the kernel that produces what it reads by small
+    // kernels it has nothing to do with (the roots of a step are lowered one after another, so
+    // the loss's bookkeeping of a few thousand elements can land inside another root's chain)
+    // moves up behind its producer, where the producer's fused launch can take it.  Past a large
+    // kernel it stays: computed early, its result would have to be kept in memory instead.
+    auto outs_of = [](const Node* k) {
+      std::set<std::string> o;
+      for (const auto& p : k->params)
+        if (p.dtype.is_ptr() && p.mut_) o.insert(p.name);
+      return o;
+    };
+    auto small = [&](const Node* k) {
+      for (const auto& p : k->params) {
+        if (!p.dtype.is_ptr() || !p.mut_) continue;
+        bool known = false;
+        for (const auto& b : plan.buffers)
+          if (b.name == p.name) { known = true; if (b.numel() > (size_t{1} << 16)) return false; }
+        if (!known) return false;
+      }
+      return true;
+    };
+    for (size_t c = 2; c < kernels.size(); ++c) {
+      const Node* kc = kernels[c];
+      if (kc->name.rfind("E_", 0) != 0) continue;
+      std::set<std::string> c_in, c_all;
+      for (const auto& p : kc->params)
+        if (p.dtype.is_ptr()) { c_all.insert(p.name); if (!p.mut_) c_in.insert(p.name); }
+      const auto co = outs_of(kc);
+      size_t pos = c;
+      bool found = false;
+      while (pos > 0) {
+        const Node* kb = kernels[pos - 1];
+        bool produces = false, clash = false;
+        for (const auto& p : kb->params) {
+          if (!p.dtype.is_ptr()) continue;
+          produces = produces || (p.mut_ && c_in.count(p.name));
+          clash = clash || co.count(p.name) || (p.mut_ && c_all.count(p.name) && !c_in.count(p.name));
+        }
+        if (produces) { found = true; break; }
+        if (clash || !small(kb)) break;
+        --pos;
+      }
+      if (!found || pos == c) continue;
+      kernels.erase(kernels.begin() + static_cast<long>(c));
+      kernels.insert(kernels.begin() + static_cast<long>(pos), kc);
+    }
+  }
   std::map<std::string, size_t> elems;
   bool have_table = !plan.buffers.empty();
   if (have_table) {

@@ -675,6 +675,11 @@ def test_convolution_rows_run_across_images(frontend):
     assert "#define EH_C_NSPLIT 196LL" in fwd["source"] and "#define EH_C_SN2 12544LL" in fwd["source"]
     small = [l for l in plan.launches if "tile=32x32x16" in l["schedule"]]
     assert [l["entry"] for l in small] == ["ehk_R_256_1_32_9_79_part"], [l["schedule"] for l in plan.launches]
+    # the kernel that prepares the second fully connected layer's operand is lowered behind two
+    # small kernels of the loss (another root); it moves up behind its producer and rides on the
+    # first layer's contraction like the rest of that chain
+    fc1 = [l for l in plan.launches if "R_256_1_128_16" in l["kernels"] and "E_256_128_23" in l["kernels"]]
+    assert len(fc1) == 1 and "epilogue=4" in fc1[0]["schedule"], [l["kernels"] for l in plan.launches]
 
 
 def _bias_gradient_step(x, b, lr):
@@ -710,7 +715,7 @@ def test_backward_pass_recomputes_cheap_saved_values(frontend):
     rematerialize=0 keeps every saved value."""
     from harp_amd import backend as hb, workloads as wl
     from harp_amd.frontend import Tensor
-    arrays = wl.config4_inputs(*wl.mlp_sizes(False))
+    arrays = wl.config4_inputs(512, [64, 256, 256, 64])       # (activations beyond what counts as a small kernel)
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     ast = wl.lower_multi(ts, wl.config4_graph(*ts, lr=1e-3))[0]
     stored = lambda plan: sorted(b["name"] for b in plan.buffers if b["role"] == "temp" and not b["elided"])
