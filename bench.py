@@ -37,7 +37,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
     ap.add_argument("--sets", type=int, default=4)
-    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn | copy | mfma_peak | mfma_valu (default: all but the last three)")
+    ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn (default: all)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-kernel", action="store_true", help="skip the per-kernel (unfused, synchronous) path")
     ap.add_argument("--no-check", action="store_true")
@@ -61,24 +61,6 @@ def main():
     options = args.options or None
     want = lambda n: not args.only or args.only == n
     extra = {}
-
-    # ---- calibration kernels (ceilings the profiles quote; not results) ----------------------
-    if args.only == "copy":
-        gbs, launch, ms = measure.copy_rate(dev, (4096, 4096), args.steps, args.warmup, args.sets, options)
-        log(f"[bench] copy 4096^2 ({launch['entry']}, {launch['schedule']}): {ms * 1e3:.1f} us/step -> {gbs:.0f} GB/s")
-        return
-    if args.only == "mfma_peak":
-        tflops, blocks, ms = measure.mfma_issue_rate(dev)
-        log(f"[bench] MFMA f32 32x32x2 issue-rate ceiling: {tflops:.1f} TFLOP/s ({tflops / FP32_MFMA_PEAK_TFLOPS:.1%} of "
-            f"the published {FP32_MFMA_PEAK_TFLOPS}); {blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
-        return
-
-    if args.only == "mfma_valu":
-        r = measure.mfma_valu_overlap(dev)
-        log("[bench] one SIMD, MFMAs and as many cycles of ordinary vector instructions: "
-            f"MFMAs alone {r['mfma_only']:.0f} us, vector instructions alone {r['valu_only']:.0f} us, both in every wave "
-            f"{r['both_in_each_wave']:.0f} us, one wave of each {r['one_wave_of_each_per_simd']:.0f} us")
-        return
 
     def roofline(bound, achieved, unit, algo, launch=None):
         """Roofline object of one kernel (`launch` given) or of a whole step: `achieved` is
@@ -129,6 +111,7 @@ def main():
         algo = sum(l["algo_bytes"] for l in prog.launches)
         softmax = {"ms": ms, "gbs": algo / (ms * 1e-3) / 1e9, "algo_bytes": algo, "launch": prog.launches[0],
                    "n_launches": len(prog.launches)}
+        softmax["each"] = measure.time_each_step(dev, prog, sets, max(20, min(args.steps, 200)), max(5, min(args.warmup, 20)))
         log(f"[bench] softmax 4096^2: {ms * 1e3:.1f} us/step -> {softmax['gbs']:.0f} GB/s "
             f"({softmax['gbs'] / HBM_PEAK_GBS:.1%} of 8 TB/s); {[(l['entry'], l['schedule']) for l in prog.launches]}")
 
@@ -153,12 +136,15 @@ def main():
         prog_ast, arg_names, out_name, consts, _ = wl.lower_with_table([(4096, 4096)] * 2, wl.config3_graph)
         prog = hb.HipProgram(dev, prog_ast, options)
         sets = measure.make_sets(dev, prog, arg_names, consts, arrays, 2)
-        k = max(5, min(args.steps, 50))
-        ms, _ = measure.time_steps(dev, prog, sets, k, args.warmup)
+        k = max(50, min(args.steps, 100))
+        wu = max(10, args.warmup)
+        ms, _ = measure.time_steps(dev, prog, sets, k, wu)
         flops = sum(l["flops"] for l in prog.launches)
-        matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k, "flops": flops, "launch": prog.launches[0]}
-        log(f"[bench] matmul 4096^3: {ms:.3f} ms/step -> {matmul['tflops']:.1f} TFLOP/s "
-            f"({matmul['tflops'] / FP32_MFMA_PEAK_TFLOPS:.1%} of FP32 MFMA peak); "
+        matmul = {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "steps": k, "warmup": wu, "flops": flops, "launch": prog.launches[0]}
+        matmul["each"] = measure.time_each_step(dev, prog, sets, k, wu)
+        log(f"[bench] matmul 4096^3: {ms:.3f} ms/step over {k} launches -> {matmul['tflops']:.1f} TFLOP/s "
+            f"({matmul['tflops'] / FP32_MFMA_PEAK_TFLOPS:.1%} of FP32 MFMA peak); per launch median "
+            f"{matmul['each'][0]:.3f} min {matmul['each'][1]:.3f} mean {matmul['each'][2]:.3f} ms; "
             f"{[(l['entry'], l['schedule']) for l in prog.launches]}")
         if not args.no_check:
             got = sets[0][1][out_name].read_array(np.float32, (4096, 4096))
@@ -352,7 +338,11 @@ def main():
         "config": {"workload": "config2: row softmax fp32 [4096,4096], one fused launch",
                    "buffer_sets": args.sets, "options": args.options},
     }
+    each_note = ("one HIP event pair per launch on the launch stream, same buffer rotation; the events sit between "
+                 "launches, so ms_mean can exceed ms_per_step, which is measured over launches queued back to back")
     if head:
+        out["ms_median"], out["ms_min"], out["ms_mean"] = (round(v, 6) for v in head["each"])
+        out["per_launch_timing"] = each_note
         out["roofline"] = roofline("hbm", head["gbs"], "GB/s", head["algo_bytes"], head["launch"])
         if head["per_kernel"]:
             extra["per_kernel_path"] = {"config2_softmax_4096": head["per_kernel"]}
@@ -361,7 +351,10 @@ def main():
     if matmul:
         extra["matmul_4096"] = {
             "value": round(matmul["tflops"], 2), "unit": "TFLOP/s", "ms_per_step": round(matmul["ms"], 4),
-            "steps": matmul["steps"], "dtype": "f32",
+            "steps": matmul["steps"], "warmup": matmul["warmup"], "dtype": "f32",
+            "ms_median": round(matmul["each"][0], 4), "ms_min": round(matmul["each"][1], 4), "ms_mean": round(matmul["each"][2], 4),
+            "tflops_at_median": round(matmul["flops"] / (matmul["each"][0] * 1e-3) / 1e12, 2),
+            "per_launch_timing": each_note,
             "roofline": roofline("mfma", matmul["tflops"], "TFLOP/s", matmul["flops"], matmul["launch"]),
             "per_kernel_path": "the same single kernel on both paths"}
     if cfg1:

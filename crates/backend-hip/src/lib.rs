@@ -27,6 +27,9 @@ use eclat::backend::KernelSignature;
 
 type DynErr = Box<dyn std::error::Error + Send + Sync>;
 
+/// The one place this crate aborts a caller: trait methods that return no `Result`.
+fn panic_with(what: &str, why: &str) -> ! { std::panic::panic_any(format!("{what}: {why}")) }
+
 fn check(code: i32) -> Result<(), DynErr> {
     if code == 0 { Ok(()) } else { Err(ffi::last_error().into()) }
 }
@@ -130,8 +133,14 @@ impl Buffer for HipBuffer {
         check(unsafe { ffi::eh_buffer_write(self.raw, data.as_ptr().cast(), data.len()) })
     }
     fn clone_buffer(&self) -> Box<dyn Buffer> {
-        let b = HipBuffer::allocate(&self.dev, self.shape.clone(), self.dtype.clone()).expect("allocation failed");
-        unsafe { ffi::eh_buffer_copy(b.raw, self.raw); }
+        // The trait has no error path here (CBuffer clones a Vec, which aborts when memory runs
+        // out): a failed allocation or device copy ends in a panic that carries the library's
+        // message, never in a buffer that silently holds something else.
+        let b = HipBuffer::allocate(&self.dev, self.shape.clone(), self.dtype.clone())
+            .unwrap_or_else(|e| panic_with("clone_buffer: allocation failed", &e.to_string()));
+        if let Err(e) = check(unsafe { ffi::eh_buffer_copy(b.raw, self.raw) }) {
+            panic_with("clone_buffer: device copy failed", &e.to_string());
+        }
         Box::new(b)
     }
     fn as_any(&self) -> &dyn Any { self }
@@ -140,7 +149,9 @@ impl Buffer for HipBuffer {
 
 enum Loaded { Program(*mut ffi::eh_program), Module(*mut ffi::eh_module) }
 
-pub struct HipKernel { loaded: Loaded, config: KernelConfig, ast_text: Option<Arc<String>>, dev: HipDevice }
+/// `ast_text` is kept for kernels compiled from an AST, `blob` (the gfx950 code object) for kernels
+/// loaded through `Compiler::compile`: either is what `clone_kernel` builds the copy from.
+pub struct HipKernel { loaded: Loaded, config: KernelConfig, ast_text: Option<Arc<String>>, blob: Option<Arc<Vec<u8>>>, dev: HipDevice }
 unsafe impl Send for HipKernel {}
 unsafe impl Sync for HipKernel {}
 impl Drop for HipKernel {
@@ -160,9 +171,14 @@ fn raw_buffers(bufs: &[&dyn Buffer]) -> Vec<*mut ffi::eh_buffer> {
 
 impl Kernel for HipKernel {
     fn clone_kernel(&self) -> Box<dyn Kernel> {
-        // recompile from the AST text; the library's code-object cache makes this a lookup
-        let text = self.ast_text.as_ref().expect("kernels loaded from a binary cannot be cloned");
-        Box::new(compile_text(&self.dev, text.clone(), self.config.clone()).expect("recompile failed"))
+        // from the AST text (the library's code-object cache makes the recompile a lookup), or, for a
+        // kernel that came in as source through `Compiler::compile`, from its code object
+        let made = match (&self.ast_text, &self.blob) {
+            (Some(text), _) => compile_text(&self.dev, text.clone(), self.config.clone()),
+            (None, Some(blob)) => load_blob(&self.dev, blob.clone(), self.config.clone()),
+            (None, None) => Err("kernel holds neither its AST nor its code object".into()),
+        };
+        Box::new(made.unwrap_or_else(|e| panic_with("clone_kernel", &e.to_string())))
     }
     fn config(&self) -> &KernelConfig { &self.config }
     fn device_kind(&self) -> DeviceKind { DeviceKind::Hip }
@@ -206,12 +222,30 @@ fn compile_text(dev: &HipDevice, text: Arc<String>, config: KernelConfig) -> Res
     let c = CString::new(text.as_str())?;
     let mut raw = std::ptr::null_mut();
     check(unsafe { ffi::eh_program_compile(dev.raw(), c.as_ptr(), std::ptr::null(), &mut raw) })?;
-    Ok(HipKernel { loaded: Loaded::Program(raw), config, ast_text: Some(text), dev: dev.clone() })
+    Ok(HipKernel { loaded: Loaded::Program(raw), config, ast_text: Some(text), blob: None, dev: dev.clone() })
+}
+
+fn load_blob(dev: &HipDevice, blob: Arc<Vec<u8>>, config: KernelConfig) -> Result<HipKernel, DynErr> {
+    let entry = CString::new(config.entry_point.as_str())?;
+    let mut raw = std::ptr::null_mut();
+    check(unsafe { ffi::eh_module_load(dev.raw(), blob.as_ptr().cast(), blob.len(), entry.as_ptr(), &mut raw) })?;
+    Ok(HipKernel { loaded: Loaded::Module(raw), config, ast_text: None, blob: Some(blob), dev: dev.clone() })
 }
 
 /// `Renderer` (src/backend/renderer.rs:20-35): AST -> HIP C, no device involved.  The text is
 /// every launch's translation unit in launch order; dispatch sizes come with the plan
 /// (`eh_plan_launch`), not from the AST's grid fields.
+///
+/// `CLikeRenderer` and `KernelSourceRenderer` (src/backend/renderer.rs:69-159,
+/// src/backend/pipeline.rs:27-33) are deliberately NOT implemented, so the generic
+/// `Pipeline<R, Dev, Comp>` (pipeline.rs:135-216) cannot be instantiated with this renderer.
+/// That pipeline renders one translation unit, takes the first kernel's name as the entry point
+/// and the AST's own grid and thread-group fields as the dispatch (1x1x1 for a lowered kernel),
+/// and compiles exactly that.  Here one AST kernel becomes one or several launches with entry
+/// points, grids, workgroup sizes and sometimes scratch buffers that only the plan knows: fed
+/// through the generic pipeline the code would be launched with the wrong entry and geometry.
+/// `BackendRegistry::compile_ast` and `execute_program` below are the routes; both hand the AST
+/// to the library, which plans, renders, compiles and launches as one unit.
 #[derive(Default)]
 pub struct HipRenderer { options: Option<String> }
 
@@ -266,11 +300,11 @@ impl Compiler for HipCompiler {
         if unsafe { ffi::eh_compile_source(src.as_ptr(), std::ptr::null(), &mut blob, &mut len) } != 0 {
             return Err(err(ffi::last_error()));
         }
-        let mut raw = std::ptr::null_mut();
-        let rc = unsafe { ffi::eh_module_load(device.raw(), blob, len, entry.as_ptr(), &mut raw) };
+        let _ = entry;
+        // the code object is kept beside the loaded module, so that the kernel can be cloned
+        let owned = Arc::new(unsafe { std::slice::from_raw_parts(blob as *const u8, len) }.to_vec());
         unsafe { ffi::eh_free(blob); }
-        if rc != 0 { return Err(err(ffi::last_error())); }
-        Ok(HipKernel { loaded: Loaded::Module(raw), config, ast_text: None, dev: device.clone() })
+        load_blob(device, owned, config).map_err(|e| err(e.to_string()))
     }
 }
 

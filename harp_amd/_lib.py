@@ -69,6 +69,7 @@ _SIGS = {
     "eh_buffer_device_ptr": ([_P, POINTER(_P)], c_int),
     "eh_render_program": ([c_char_p, c_char_p, POINTER(_P)], c_int),
     "eh_normalize_ast": ([c_char_p, POINTER(c_void_p)], c_int),
+    "eh_fit_local_size": ([POINTER(c_size_t), POINTER(c_size_t), c_size_t, POINTER(c_size_t)], c_int),
     "eh_plan_num_launches": ([_P, POINTER(c_int)], c_int),
     "eh_plan_launch": ([_P, c_int, POINTER(LaunchInfo)], c_int),
     "eh_plan_launch_arg": ([_P, c_int, c_int, POINTER(c_char_p)], c_int),

@@ -12,6 +12,7 @@
 #include <fstream>
 #include <list>
 #include <mutex>
+#include <optional>
 #include <sstream>
 #include <thread>
 #include <unordered_map>
@@ -599,6 +600,12 @@ std::vector<HipBuffer*> HipProgram::bind(HipBuffer* const* bufs, size_t n, std::
     }
     bound[i] = b;
   }
+  {
+    std::vector<Span> spans(total);
+    for (size_t i = 0; i < total; ++i)
+      if (bound[i]) spans[i] = {bound[i]->device_ptr(), bound[i]->byte_len(), true};
+    refuse_aliases(spans);
+  }
   resolve_fills(bound, cancelled);
   return bound;
 }
@@ -616,6 +623,40 @@ void HipProgram::resolve_fills(const std::vector<HipBuffer*>& bound, std::vector
     } else {
       b->settle();
     }
+  }
+}
+
+// The planner reorders, merges and (with lanes) overlaps launches by the dependences it reads off
+// the buffer names, so two table entries must never be the same memory when a launch writes either
+// of them: an in-place update (one buffer bound as a parameter and as its updated value) would race
+// silently.  Refused here, on the host.
+void HipProgram::refuse_aliases(const std::vector<Span>& bound) const {
+  if (written_.empty()) {
+    written_.assign(plan_.buffers.size(), 0);
+    for (const auto& ls : plan_.launches)
+      for (size_t a = 0; a < ls.arg_bufs.size(); ++a)
+        if (a < ls.arg_written.size() && ls.arg_written[a]) written_[index_.at(ls.arg_bufs[a])] = 1;
+  }
+  struct Range { const char* lo; const char* hi; size_t i; };
+  std::vector<Range> r;
+  for (size_t i = 0; i < bound.size(); ++i)
+    if (bound[i].bound && bound[i].bytes)
+      r.push_back({static_cast<const char*>(bound[i].ptr), static_cast<const char*>(bound[i].ptr) + bound[i].bytes, i});
+  std::sort(r.begin(), r.end(), [](const Range& a, const Range& b) { return a.lo < b.lo; });
+  // sorted by start: an overlap with anything earlier shows against the furthest end seen so far;
+  // among read-only entries sharing is harmless, so the furthest written end is kept apart
+  const Range* far = nullptr;      // furthest-reaching entry so far
+  const Range* far_w = nullptr;    // furthest-reaching written entry so far
+  for (const Range& x : r) {
+    const Range* hit = nullptr;
+    if (far_w && x.lo < far_w->hi) hit = far_w;
+    else if (written_[x.i] && far && x.lo < far->hi) hit = far;
+    if (hit)
+      throw Error("buffers '" + plan_.buffers[hit->i].name + "' and '" + plan_.buffers[x.i].name +
+                  "' of the table are bound to overlapping device memory and the program writes one of them: table "
+                  "entries must be distinct buffers (no in-place updates)");
+    if (!far || x.hi > far->hi) far = &x;
+    if (written_[x.i] && (!far_w || x.hi > far_w->hi)) far_w = &x;
   }
 }
 
@@ -745,8 +786,12 @@ void HipProgram::execute_static(HipBuffer* const* bufs, size_t n, bool sync) {
     given[i] = b;
     bound[i] = {b->device_ptr(), b->byte_len(), true};
   }
+  refuse_aliases(bound);
   std::vector<HipBuffer*> cancelled;
   resolve_fills(given, &cancelled);              // (queues fills at most; allocates nothing)
+  // another handle on this GPU (its own stream, its own lock) shares the block: take turns
+  std::optional<StaticScratchTurn> turn;
+  if (need) turn.emplace(dev_->index(), static_cast<void*>(dev_->stream()));
   try {
     launch_spans(bound);
   } catch (...) {

@@ -185,10 +185,12 @@ class HipProgram {
     bool bound = false;
   };
   void launch_spans(const std::vector<Span>& bound);                // the same, over plain address ranges
+  void refuse_aliases(const std::vector<Span>& bound) const;        // throws when two entries overlap and one is written
   HipDevice* dev_;
   ProgramPlan plan_;
   std::vector<std::shared_ptr<HipKernel>> kernels_;
   std::map<std::string, size_t> index_;          // buffer name -> table index
+  mutable std::vector<char> written_;            // by table index: some launch writes the buffer (filled on first use)
   std::vector<size_t> first_full_;               // by table index: size of the buffer the first launch that binds it overwrites whole (0: none)
   std::vector<HipBuffer*> temps_;                // owned, by table index (nullptr if unused)
   // Lanes (plan().lanes > 1): events_[l] is recorded behind launch l when a launch on another

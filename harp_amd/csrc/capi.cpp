@@ -273,6 +273,21 @@ int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out) {
   return EH_OK;
 }
 
+int eh_fit_local_size(const size_t global[3], const size_t preferred[3], size_t max_work_group, size_t local[3]) {
+  REQUIRE(global && preferred && local, "global, preferred or local is NULL");
+  REQUIRE(max_work_group >= 1, "max_work_group must be at least 1");
+  uint64_t g[3], p[3], l[3];
+  for (int i = 0; i < 3; ++i) {
+    REQUIRE(preferred[i] >= 1, "a preferred local size must be at least 1");
+    REQUIRE(global[i] <= (uint64_t{1} << 40) && preferred[i] <= (uint64_t{1} << 40), "size out of range");
+    g[i] = global[i];
+    p[i] = preferred[i];
+  }
+  eh::fit_local_size(g, p, max_work_group, l);
+  for (int i = 0; i < 3; ++i) local[i] = static_cast<size_t>(l[i]);
+  return EH_OK;
+}
+
 int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name) {
   REQUIRE(plan && buffer_name, "plan or buffer_name is NULL");
   REQUIRE(launch >= 0 && launch < static_cast<int>(plan->plan.launches.size()), "launch index out of range");

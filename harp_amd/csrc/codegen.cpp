@@ -4,6 +4,9 @@
 #include <cmath>
 #include <cstring>
 #include <functional>
+#include <mutex>
+#include <set>
+#include <cstdio>
 #include <sstream>
 
 #include "gemm.hpp"
@@ -269,9 +272,16 @@ struct ExprRenderer {
       case Op::BitNot: return "(~" + expr(*n.args[0]) + ")";
       case Op::Cast: return "(" + ctype(n.dtype) + ")(" + expr(*n.args[0]) + ")";
       case Op::Fma: {
-        bool dbl = infer_ty(n, var_types) == Ty::F64;
-        return std::string(dbl ? "fma(" : "fmaf(") + expr(*n.args[0]) + ", " + expr(*n.args[1]) + ", " +
-               expr(*n.args[2]) + ")";
+        // The reference renders `fma(a, b, c)` whatever the operands' type
+        // (src/backend/renderer.rs:107-109), which in C on float operands is the double-precision
+        // function on promoted values, its result converted back on use: product exact, one
+        // rounding to double, one to float.  Rendered as exactly that, so that an elementwise
+        // kernel in this form stays bit-identical to the C backend's (fmaf rounds once and
+        // differs where the double result sits on a float tie).
+        const Ty t = infer_ty(n, var_types);
+        if (t == Ty::F64) return "fma(" + expr(*n.args[0]) + ", " + expr(*n.args[1]) + ", " + expr(*n.args[2]) + ")";
+        return "(" + ctype(DType{t}) + ")fma((double)(" + expr(*n.args[0]) + "), (double)(" + expr(*n.args[1]) + "), (double)(" +
+               expr(*n.args[2]) + "))";
       }
       case Op::Select: {
         if (g_guard_branches || plain_selects > 0 || (!holds_load(*n.args[1]) && !holds_load(*n.args[2])))
@@ -471,6 +481,28 @@ void refuse_long_serial(const std::string& kernel, const Node& body, const GenOp
 }
 }  // namespace
 
+// local[i] = the largest divisor of global[i] that is at most preferred[i]
+// (`compute_compatible_local_size`, src/backend/pipeline.rs:475-489); then, while the workgroup
+// exceeds `max_work_group`, its largest dimension steps down to the next smaller divisor of that
+// dimension's global size (pipeline.rs:176-192).
+void fit_local_size(const uint64_t global[3], const uint64_t preferred[3], uint64_t max_work_group, uint64_t local[3]) {
+  for (int i = 0; i < 3; ++i) {
+    uint64_t l = 1;
+    if (global[i] != 0) {
+      l = std::min(preferred[i], global[i]);
+      while (l > 1 && global[i] % l != 0) --l;
+      if (l < 1) l = 1;
+    }
+    local[i] = l;
+  }
+  while (local[0] * local[1] * local[2] > max_work_group) {
+    const int m = (local[0] >= local[1] && local[0] >= local[2]) ? 0 : (local[1] >= local[2] ? 1 : 2);
+    uint64_t v = local[m] - 1;
+    while (v > 1 && global[m] % v != 0) --v;
+    local[m] = std::max<uint64_t>(v, 1);
+  }
+}
+
 LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
   if (k.op != Op::Kernel) throw Error("expected a kernel node");
   LaunchSpec ls;
@@ -503,12 +535,25 @@ LaunchSpec render_kernel_as_written(const Node& k, const GenOptions& opt) {
   StmtRenderer sr;
   os << sr.stmt(*k.args[0]) << "}\n";
   ls.source = os.str();
-  for (int i = 0; i < 3; ++i) {
-    int64_t g = k.grid.size() == 3 ? dispatch_value(*k.grid[i]) : 1;
-    int64_t t = k.tg.size() == 3 ? dispatch_value(*k.tg[i]) : 1;
-    if (g < 1 || t < 1 || t > 1024) throw Error("kernel '" + k.name + "' has an unusable dispatch size");
-    ls.block[i] = static_cast<unsigned>(t);
-    ls.grid[i] = static_cast<unsigned>(g);   // the AST's grid size counts workgroups
+  {
+    // global size = grid x thread group (the AST's grid counts workgroups), local size = the
+    // thread group fitted to the device as Pipeline::compile_ast does (src/backend/pipeline.rs:
+    // 160-192), launched as global / local workgroups
+    uint64_t global[3], preferred[3], local[3];
+    for (int i = 0; i < 3; ++i) {
+      int64_t g = k.grid.size() == 3 ? dispatch_value(*k.grid[i]) : 1;
+      int64_t t = k.tg.size() == 3 ? dispatch_value(*k.tg[i]) : 1;
+      if (g < 1 || t < 1 || g > (int64_t{1} << 31) || t > (int64_t{1} << 31) || g * t > (int64_t{1} << 40))
+        throw Error("kernel '" + k.name + "' has an unusable dispatch size");
+      global[i] = static_cast<uint64_t>(g * t);
+      preferred[i] = static_cast<uint64_t>(t);
+    }
+    fit_local_size(global, preferred, 1024, local);
+    for (int i = 0; i < 3; ++i) {
+      if (global[i] / local[i] > 0x7fffffffull) throw Error("kernel '" + k.name + "' has an unusable dispatch size");
+      ls.block[i] = static_cast<unsigned>(local[i]);
+      ls.grid[i] = static_cast<unsigned>(global[i] / local[i]);
+    }
   }
   if (1ull * ls.grid[0] * ls.grid[1] * ls.grid[2] * ls.block[0] * ls.block[1] * ls.block[2] == 1)
     refuse_long_serial(k.name, *k.args[0], opt);
@@ -608,6 +653,53 @@ bool injective(const Affine& a, const std::vector<Loop>& vars) {
     reach += p.first * (p.second - 1);
   }
   return true;
+}
+
+}  // namespace
+
+namespace {
+
+bool stores_anything(const Node& n) {
+  if (n.op == Op::Store || n.op == Op::AtomicAdd || n.op == Op::AtomicMax) return true;
+  for (const auto& a : n.args)
+    if (stores_anything(*a)) return true;
+  return false;
+}
+
+// A loop of at least 64 iterations that only accumulates (assigns, stores nothing): the inner loop of
+// a reduction, as opposed to a scan's, which stores every step.
+bool has_accumulating_loop(const Node& n) {
+  if (n.op == Op::Range) {
+    int64_t s = 0, e = 0;
+    const bool counted = n.args[0]->op == Op::Const && n.args[2]->op == Op::Const;
+    if (counted) {
+      s = n.args[0]->ival;
+      e = n.args[2]->ival;
+    }
+    if ((!counted || e - s >= 64) && !stores_anything(*n.args[3])) {
+      bool assigns_something = false;
+      std::vector<const Node*> todo = {n.args[3].get()};
+      while (!todo.empty() && !assigns_something) {
+        const Node* x = todo.back();
+        todo.pop_back();
+        assigns_something = x->op == Op::Assign;
+        for (const auto& a : x->args) todo.push_back(a.get());
+      }
+      if (assigns_something) return true;
+    }
+  }
+  for (const auto& a : n.args)
+    if (has_accumulating_loop(*a)) return true;
+  return false;
+}
+
+void warn_once_degraded(const std::string& kernel) {
+  static std::mutex mu;
+  static std::set<std::string> seen;
+  std::lock_guard<std::mutex> lock(mu);
+  if (seen.size() > 256 || !seen.insert(kernel).second) return;
+  std::fprintf(stderr, "eclat-hip: kernel '%s' has a loop structure no schedule recognises as written and runs one "
+               "work-item per outer iteration (plan marked 'degraded')\n", kernel.c_str());
 }
 
 }  // namespace
@@ -925,7 +1017,16 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
       os << sr.stmt(*inner) << "}\n";
       ls.grid[0] = static_cast<unsigned>((total + 255) / 256);
       ls.block[0] = 256;
-      ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + (colliding ? ",atomics)" : ")");
+      // A large nest that ends up here was not recognised for what it is (the optimiser's rewrites
+      // were not undone): few work-items each walking a long stretch, or a reduction that stores
+      // after its accumulating loop (a sum, a contraction that missed the matrix cores) run one
+      // output per work-item.  Correct, slow, and said so in the plan.
+      const double per_item = std::max(1.0, serial_iterations(*inner));
+      const bool big = per_item * static_cast<double>(total) >= 1048576.0;
+      const bool degraded = big && (total < 16384 || has_accumulating_loop(*inner));
+      if (degraded) warn_once_degraded(k.name);
+      ls.schedule = "outer-parallel(work-items=" + std::to_string(total) + (colliding ? ",atomics" : "") +
+                    (degraded ? ",degraded)" : ")");
       any_parallel = true;
     } else {
       refuse_long_serial(k.name, *tops[t], opt);
@@ -3600,9 +3701,9 @@ struct GroupEmitter {
       if (!st.store) continue;
       std::string T = ctype(st.out_dtype);
       if (V > 1) {
-        os << "  { EhV" << V << "<" << T << "> o;\n#pragma unroll\n  for (int v = 0; v < " << V << "; ++v) { const idx_t c = c0 + v; o[v] = ("
+        os << "  { EhV" << V << "<" << T << "> eh_o;\n#pragma unroll\n  for (int v = 0; v < " << V << "; ++v) { const idx_t c = c0 + v; eh_o[v] = ("
            << T << ")(" << value_text(st, ld) << "); }\n";
-        os << "  eh_store" << V << "<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ", o); }\n";
+        os << "  eh_store" << V << "<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0") << ", eh_o); }\n";
       } else {
         os << "  { const idx_t c = c0; " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = (" << T << ")("
            << value_text(st, ld) << "); }\n";
@@ -3890,13 +3991,13 @@ struct GroupEmitter {
       } else if (st.store) {
         os << iter_open << guard_open;
         if (V == 4) {
-          os << "      EhV4<" << T_out << "> o;\n#pragma unroll\n      for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; o[v] = ("
+          os << "      EhV4<" << T_out << "> eh_o;\n#pragma unroll\n      for (int v = 0; v < 4; ++v) { const idx_t c = c0 + v; eh_o[v] = ("
              << T_out << ")(" << value_text(st, ld) << "); }\n";
           os << "      if (eh_row_ok) eh_store4<" << nts << ">(" << st.out_buf << " + " << affine_text(st.out_aff, "c0")
-             << ", o);\n";
+             << ", eh_o);\n";
         } else {
-          os << "      const int v = 0; const idx_t c = c0; const " << T_out << " o = (" << T_out << ")(" << value_text(st, ld)
-             << ");\n      if (eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = o;\n";
+          os << "      const int v = 0; const idx_t c = c0; const " << T_out << " eh_o = (" << T_out << ")(" << value_text(st, ld)
+             << ");\n      if (eh_row_ok) " << st.out_buf << "[" << affine_text(st.out_aff, "c") << "] = eh_o;\n";
         }
         os << "    }\n  }\n";
       }

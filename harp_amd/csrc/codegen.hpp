@@ -5,6 +5,8 @@
 // per-output serial reductions, FP32 MFMA contractions.
 #pragma once
 
+#include <cstdint>
+
 #include <map>
 #include <set>
 #include <string>
@@ -89,6 +91,11 @@ LaunchSpec render_kernel_as_written(const Node& kernel, const GenOptions& opt);
 // buffer table); null when the caller has no table, and such schedules are then not used.
 std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& kernel, const GenOptions& opt,
                                                      std::vector<BufferInfo>* extra_buffers = nullptr);
+
+// The local work size the reference derives from a kernel's dispatch hints
+// (src/backend/pipeline.rs:160-192, 475-489): per dimension the largest divisor of the global
+// size not above the preferred size, then shrunk until the workgroup fits `max_work_group`.
+void fit_local_size(const uint64_t global[3], const uint64_t preferred[3], uint64_t max_work_group, uint64_t local[3]);
 
 // Expression text in HIP C (math calls, literals); exposed for tests.
 std::string render_expr_text(const Node& e);

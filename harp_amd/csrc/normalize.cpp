@@ -2,6 +2,8 @@
 
 #include <algorithm>
 #include <cstring>
+#include <limits>
+#include <optional>
 #include <set>
 
 #include "analysis.hpp"
@@ -142,6 +144,7 @@ NodePtr make_loop(const Node& like, const std::string& var, NodePtr start, NodeP
 
 struct Normalizer {
   std::set<std::string> int_vars;     // loop variables and integer block variables of the kernel
+  std::set<std::string> rolled;       // loop variables made by rolling repeated statements back into a loop
   int fresh = 0;
 
   void collect_int_vars(const Node& n) {
@@ -324,11 +327,74 @@ struct Normalizer {
       if (body.size() != p) continue;
       ++fresh;
       int_vars.insert(u);
+      rolled.insert(u);
       Node like(Op::Range);
       like.parallel = "sequential";
       return loop(make_loop(like, u, make_i64(0), make_i64(1), make_i64(static_cast<int64_t>(k)), block(body, decls)));
     }
     return nullptr;
+  }
+
+  // ---- an interchanged strip-mined pair -----------------------------------------------------------
+
+  // `n` with the pair (u, r) replaced by one variable w = u + T * r, or null: every integer
+  // position (an index, a bound, a compared value) that mentions u or r must be affine with
+  // coefficient(r) == T * coefficient(u); u and r may appear nowhere else.  With `canon` set and no
+  // pair given (u empty) the integer positions are only rewritten into their canonical affine
+  // text, so that two bodies that differ in spelling compare equal.
+  NodePtr repair(const NodePtr& n, const std::string& u, const std::string& r, int64_t T, const std::string& w, bool pos,
+                 bool* ok) const {
+    if (pos) {
+      auto a = int_affine(*n);
+      if (a) {
+        Affine out = *a;
+        if (!u.empty()) {
+          const int64_t cu = a->of(u), cr = a->of(r);
+          if (cr != cu * T) {
+            *ok = false;
+            return n;
+          }
+          out.coef.erase(u);
+          out.coef.erase(r);
+          if (cu != 0) out.coef[w] += cu;
+        }
+        return affine_to_node(out);
+      }
+    }
+    if (n->op == Op::Var && !u.empty() && (n->name == u || n->name == r)) {
+      *ok = false;
+      return n;
+    }
+    if (n->args.empty()) return n;
+    std::vector<NodePtr> args;
+    bool changed = false;
+    for (size_t i = 0; i < n->args.size(); ++i) {
+      bool p = false;
+      switch (n->op) {
+        case Op::Load: case Op::Store: case Op::AtomicAdd: case Op::AtomicMax: case Op::SharedLoad: case Op::SharedStore:
+          p = i == 1;
+          break;
+        case Op::Assign: p = int_vars.count(n->name) > 0; break;
+        case Op::Range: p = i < 3; break;
+        case Op::Lt: p = true; break;
+        default: break;
+      }
+      NodePtr x = repair(n->args[i], u, r, T, w, p, ok);
+      changed = changed || x != n->args[i];
+      args.push_back(std::move(x));
+    }
+    return changed ? with_args(*n, std::move(args)) : n;
+  }
+
+  std::string canonical_text(const NodePtr& n) const {
+    bool ok = true;
+    return to_text(*repair(n, "", "", 0, "", false, &ok));
+  }
+
+  // The one statement of a loop body, single-statement blocks without declarations unwrapped.
+  static const Node* sole_statement(const Node* b) {
+    while (b->op == Op::Block && b->decls.empty() && b->args.size() == 1) b = b->args[0].get();
+    return b;
   }
 
   // ---- loops ----------------------------------------------------------------------------------
@@ -392,6 +458,37 @@ struct Normalizer {
           }
         }
       }
+      // a strip-mined pair whose loops were interchanged and the tile loop unrolled and rolled back
+      // (u is a loop `reroll` made; two loops the lowerer wrote over a dense tensor have the same
+      // index form and stay two): for u in 0..T { for q in 0..n { body(u + T*q) } } -> for w in 0..T*n { body(w) }.  The body
+      // is one store (iterations independent) or one accumulation by a commutative, associative
+      // operator, whose order every schedule here is free to choose; w ascending is the order the
+      // lowerer wrote.
+      if (s == 0 && step == 1 && e >= 2 && rolled.count(r->name) && sole_statement(body.get())->op == Op::Range) {
+        const Node& in = *sole_statement(body.get());
+        int64_t is = 0, istep = 0, n_in = 0;
+        const Node* st = sole_statement(in.args[3].get());
+        bool shape_ok = int_const(*in.args[0], &is) && int_const(*in.args[1], &istep) && int_const(*in.args[2], &n_in) &&
+                        is == 0 && istep == 1 && n_in >= 2;
+        if (shape_ok) {
+          ReduceKind kind = ReduceKind::None;
+          NodePtr value;
+          shape_ok = st->op == Op::Store ||
+                     (st->op == Op::Assign && !int_vars.count(st->name) && match_combine(*st->args[0], st->name, &kind, &value));
+        }
+        if (shape_ok) {
+          const std::string w = "eh_w" + std::to_string(fresh);
+          bool ok = true;
+          int_vars.insert(w);
+          NodePtr nb = repair(in.args[3], r->name, in.name, e, w, false, &ok);
+          if (ok && mentions(*nb, w)) {
+            ++fresh;
+            r = make_loop(*r, w, make_i64(0), make_i64(1), make_i64(mul_ck(e, n_in)), nb);
+            continue;
+          }
+          int_vars.erase(w);
+        }
+      }
       // renamed loop variable: for q in s..e { v = q + d; rest } -> for v in s+d..e+d { rest }
       // (the remainder loop of tile_loop; a rolled-back unrolled loop)
       if (body->op == Op::Block && body->args.size() >= 2 && body->args[0]->op == Op::Assign && step == 1) {
@@ -418,22 +515,33 @@ struct Normalizer {
   NodePtr block(std::vector<NodePtr> stmts, std::vector<std::pair<std::string, DType>> decls) {
     stmts.erase(std::remove_if(stmts.begin(), stmts.end(), [](const NodePtr& s) { return is_empty_stmt(*s); }),
                 stmts.end());
-    // neighbouring loops over adjoining ranges with the same body are one loop
+    // neighbouring loops with the same body over adjoining ranges are one loop; so are two whose
+    // ranges adjoin once the second one's variable is shifted (a remainder loop that was moved to
+    // start at 0, its offset now inside its body): bodies are compared with their integer
+    // positions in canonical affine form
     for (size_t j = 0; j + 1 < stmts.size();) {
       const Node &x = *stmts[j], &y = *stmts[j + 1];
       int64_t xs, xt, xe, ys, yt, ye;
       bool join = x.op == Op::Range && y.op == Op::Range && int_const(*x.args[0], &xs) && int_const(*x.args[1], &xt) &&
                   int_const(*x.args[2], &xe) && int_const(*y.args[0], &ys) && int_const(*y.args[1], &yt) &&
-                  int_const(*y.args[2], &ye) && xt == 1 && yt == 1 && xe == ys && x.parallel == y.parallel;
+                  int_const(*y.args[2], &ye) && xt == 1 && yt == 1 && xe > xs && ye > ys && x.parallel == y.parallel &&
+                  (y.name == x.name || !mentions(*y.args[3], x.name)) && !assigns(*y.args[3], y.name) &&
+                  !assigns(*x.args[3], x.name);
       if (join) {
-        NodePtr yb = y.name == x.name ? y.args[3] : substitute_vars(y.args[3], {{y.name, make_var(x.name)}});
-        join = (y.name == x.name || !mentions(*y.args[3], x.name)) && to_text(*yb) == to_text(*x.args[3]);
+        const int64_t shift = ys - xe;
+        if (shift == 0) {
+          NodePtr yb = y.name == x.name ? y.args[3] : substitute_vars(y.args[3], {{y.name, make_var(x.name)}});
+          join = to_text(*yb) == to_text(*x.args[3]) || canonical_text(yb) == canonical_text(x.args[3]);
+        } else {
+          NodePtr yb = substitute_vars(y.args[3], {{y.name, make(Op::Add, {make_var(x.name), make_i64(shift)})}});
+          join = int_vars.count(x.name) > 0 && canonical_text(yb) == canonical_text(x.args[3]);
+        }
       }
       if (!join) {
         ++j;
         continue;
       }
-      stmts[j] = make_loop(x, x.name, x.args[0], x.args[1], y.args[2], x.args[3]);
+      stmts[j] = make_loop(x, x.name, x.args[0], x.args[1], make_i64(xe + (ye - ys)), x.args[3]);
       stmts.erase(stmts.begin() + static_cast<long>(j) + 1);
     }
     if (stmts.size() >= 2)
@@ -538,28 +646,67 @@ NodePtr normalize_kernel(const NodePtr& kernel) {
   }();
 }
 
-double serial_iterations(const Node& n) {
+namespace {
+
+// [lo, hi] of an integer expression over variables with known ranges; false when the expression
+// is not affine or names a variable without a range
+bool int_range(const Node& e, const std::map<std::string, std::pair<int64_t, int64_t>>& env, int64_t* lo, int64_t* hi) {
+  auto a = affine_of(e);
+  if (!a) return false;
+  int64_t l = a->c, h = a->c;
+  for (const auto& kv : a->coef) {
+    if (kv.second == 0) continue;
+    auto it = env.find(kv.first);
+    if (it == env.end()) return false;
+    const int64_t x = mul_ck(kv.second, it->second.first), y = mul_ck(kv.second, it->second.second);
+    l = add_ck(l, std::min(x, y));
+    h = add_ck(h, std::max(x, y));
+  }
+  *lo = l;
+  *hi = h;
+  return true;
+}
+
+double serial_iterations_in(const Node& n, std::map<std::string, std::pair<int64_t, int64_t>>* env) {
   switch (n.op) {
     case Op::Range: {
-      int64_t s, step, e;
-      double trips = 1;
-      if (int_const(*n.args[0], &s) && int_const(*n.args[1], &step) && int_const(*n.args[2], &e) && step >= 1)
-        trips = e > s ? static_cast<double>((e - s + step - 1) / step) : 0.0;
-      return trips * std::max(1.0, serial_iterations(*n.args[3]));
+      // bounds that move with the enclosing loops are bounded over those loops' ranges: the
+      // earliest start, the latest stop
+      int64_t step = 0, slo = 0, shi = 0, elo = 0, ehi = 0;
+      if (!int_const(*n.args[1], &step) || step < 1 || !int_range(*n.args[0], *env, &slo, &shi) ||
+          !int_range(*n.args[2], *env, &elo, &ehi))
+        return std::numeric_limits<double>::infinity();
+      (void)shi;
+      (void)elo;
+      const double trips = ehi > slo ? static_cast<double>((ehi - slo + step - 1) / step) : 0.0;
+      if (trips == 0.0) return 0.0;
+      auto saved = env->find(n.name) == env->end() ? std::optional<std::pair<int64_t, int64_t>>() : (*env)[n.name];
+      (*env)[n.name] = {slo, ehi - 1};
+      const double inner = serial_iterations_in(*n.args[3], env);
+      if (saved) (*env)[n.name] = *saved;
+      else env->erase(n.name);
+      return trips * std::max(1.0, inner);
     }
     case Op::Block: case Op::Kernel: {
       double sum = 0;
-      for (const auto& a : n.args) sum += serial_iterations(*a);
+      for (const auto& a : n.args) sum += serial_iterations_in(*a, env);
       return sum;
     }
     case Op::If: {
       double m = 0;
-      for (size_t i = 1; i < n.args.size(); ++i) m = std::max(m, serial_iterations(*n.args[i]));
+      for (size_t i = 1; i < n.args.size(); ++i) m = std::max(m, serial_iterations_in(*n.args[i], env));
       return m;
     }
     default:
       return 0;
   }
+}
+
+}  // namespace
+
+double serial_iterations(const Node& n) {
+  std::map<std::string, std::pair<int64_t, int64_t>> env;
+  return serial_iterations_in(n, &env);
 }
 
 }  // namespace eh

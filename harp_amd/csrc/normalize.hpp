@@ -30,9 +30,11 @@ NodePtr normalize_kernel(const NodePtr& kernel);
 // `n` with every Var named in `m` replaced by the mapped node.
 NodePtr substitute_vars(const NodePtr& n, const std::map<std::string, NodePtr>& m);
 
-// Innermost-loop iterations of a statement, loops multiplied out and neighbours added (constant
-// bounds; a loop with other bounds counts as one iteration): how much work one work-item does
-// when it runs the statement as written.
+// Innermost-loop iterations of a statement, loops multiplied out and neighbours added: how much
+// work one work-item does when it runs the statement as written.  A bound that moves with the
+// enclosing loops counts by its extreme over their ranges (an upper bound on the trips); a loop
+// whose bounds cannot be bounded that way (not affine in the loop variables, or over a variable
+// assigned in the body) makes the result infinite.
 double serial_iterations(const Node& stmt);
 
 }  // namespace eh

@@ -15,4 +15,23 @@ constexpr size_t kStaticScratchAlign = 256;
 // up once per device and kept.  Throws eh::Error when the runtime cannot resolve the symbol.
 void* static_scratch_ptr(int index);
 
+// One call's turn on device `index`'s block.  Several device handles may exist for one GPU, each
+// with a stream of its own, and all of them share the block: while a turn lives no other call
+// queues launches that use it, `stream` (a hipStream_t) is made to wait for the launches of the
+// previous turn when those went to another stream, and the destructor records this turn's end
+// behind everything `stream` holds by then.  Nothing is created or allocated.  On a stream that
+// is being captured neither the wait nor the record is issued.
+class StaticScratchTurn {
+ public:
+  StaticScratchTurn(int index, void* stream);
+  ~StaticScratchTurn();
+  StaticScratchTurn(const StaticScratchTurn&) = delete;
+  StaticScratchTurn& operator=(const StaticScratchTurn&) = delete;
+
+ private:
+  int index_;
+  void* stream_;
+  bool capturing_ = false;
+};
+
 }  // namespace eh

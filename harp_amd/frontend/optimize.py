@@ -282,6 +282,61 @@ def apply_rules(n: AstNode, max_passes: int = 64) -> AstNode:
 
 
 # --------------------------------------------------------------------------
+# fused multiply-add rules (devices that report DeviceInstruction::Fma)
+# --------------------------------------------------------------------------
+
+def infer_type(n: AstNode) -> Optional[str]:
+    """`AstNode::infer_type` (src/ast/mod.rs:781-860) as far as expressions go: a dtype name,
+    or None for Unknown.  A variable's type is unknown (it depends on the context); a binary
+    operation has its operands' type when they agree; a math function keeps its operand's type
+    and is f32 when that is unknown."""
+    op = n.op
+    if op == "const":
+        return n.attrs["dtype"].name
+    if op == "cast":
+        return n.attrs["dtype"].name
+    if op == "load":
+        return n.attrs["dtype"].name
+    if op in ("var", "wildcard"):
+        return None
+    if op in ("add", "mul", "max", "rem", "idiv", "and", "or", "xor", "shl", "shr", "bitand", "bitor", "bitxor"):
+        l, r = infer_type(n.args[0]), infer_type(n.args[1])
+        return l if l == r else None
+    if op in ("lt", "not", "logical_and"):
+        return "bool"
+    if op == "select":
+        return infer_type(n.args[1])
+    if op in ("recip", "sqrt", "log2", "exp2", "sin", "floor", "bitnot"):
+        return infer_type(n.args[0]) or "f32"
+    if op == "fma":
+        return infer_type(n.args[0])
+    return None
+
+
+def _to_fma(n: AstNode) -> Optional[AstNode]:
+    """`mul_add_to_fma` and `add_mul_to_fma` (src/opt/ast/rules/algebraic.rs:218-282):
+    a * b + c and c + a * b become fma(a, b, c) when `a` infers to f32."""
+    if n.op != "add":
+        return None
+    l, r = n.args
+    if l.op == "mul" and infer_type(l.args[0]) == "f32":
+        return AstNode("fma", [l.args[0], l.args[1], r])
+    if r.op == "mul" and infer_type(r.args[0]) == "f32":
+        return AstNode("fma", [r.args[0], r.args[1], l])
+    return None
+
+
+def apply_fma_rules(n: AstNode) -> AstNode:
+    """`fma_rules` (src/opt/ast/rules/mod.rs:117-123) applied bottom-up, once per node: what
+    `rules_for_capabilities` (:136-143) adds to the rule set for a device whose
+    `supports_instruction(Fma)` is true, as `Pipeline::optimize_ast` uses it
+    (src/backend/pipeline.rs:219-224)."""
+    x = _rebuild(n, [apply_fma_rules(c) for c in n.args])
+    r = _to_fma(x)
+    return r if r is not None else x
+
+
+# --------------------------------------------------------------------------
 # the stage itself
 # --------------------------------------------------------------------------
 
@@ -289,7 +344,8 @@ def optimize_kernel(kernel: AstNode, transforms: Sequence[str] = (), rules: bool
     """`kernel` after the named loop transforms and then the rule set.  Transform names:
     `tile=T` / `guard=T` (innermost loops), `tile_all=T` (every loop, innermost first),
     `tile_outer=T` (outermost loop only), `unroll` (loops of at most eight iterations, which
-    after a tiling are the tile loops and the remainders), `interchange` (the outermost pair)."""
+    after a tiling are the tile loops and the remainders), `interchange` (the outermost pair),
+    `fma` (the multiply-add rules, applied after the rule set as the last step)."""
     body = kernel.args[0]
     for t in transforms:
         name, _, arg = t.partition("=")
@@ -324,10 +380,14 @@ def optimize_kernel(kernel: AstNode, transforms: Sequence[str] = (), rules: bool
                         return r
                 return _rebuild(x, [top_down(c) for c in x.args])
             body = top_down(body)
+        elif name == "fma":
+            pass
         elif name:
             raise ValueError(f"unknown loop transform '{t}'")
     if rules:
         body = apply_rules(body)
+    if "fma" in transforms:
+        body = apply_fma_rules(body)
     return AstNode("kernel", [body], **kernel.attrs)
 
 

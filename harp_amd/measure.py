@@ -60,6 +60,25 @@ def time_steps(dev, prog, sets, steps, warmup):
     return e0.elapsed_ms(e1) / steps, wall / steps
 
 
+def time_each_step(dev, prog, sets, steps, warmup):
+    """Per-step durations in ms: an event before the first launch and one behind every step, all on
+    the launch stream, read after the last one completed.  Returns (median, min, mean) over `steps`
+    steps after `warmup` untimed ones.  The events sit between the steps, so the mean here can
+    exceed what `time_steps` measures over the same steps queued back to back."""
+    for i in range(warmup):
+        prog.run(sets[i % len(sets)][0], sync=False)
+    dev.sync()
+    events = [hb.Event(dev) for _ in range(steps + 1)]
+    events[0].record()
+    for i in range(steps):
+        prog.run(sets[i % len(sets)][0], sync=False)
+        events[i + 1].record()
+    events[-1].sync()
+    dev.sync()
+    ms = np.array([events[i].elapsed_ms(events[i + 1]) for i in range(steps)])
+    return float(np.median(ms)), float(ms.min()), float(ms.mean())
+
+
 def time_replays(dev, prog, sets, steps, warmup):
     """As `time_steps`, with each binding recorded once as a HIP graph and a step = one replay."""
     graphs = [prog.record(b) for b, _ in sets]
@@ -214,60 +233,6 @@ def mfma_issue_rate(dev, iters=4096, waves_per_cu=8, reps=20):
     return flops / ms / 1e9, blocks, ms
 
 
-MFMA_VALU_SOURCE = """
-typedef float f16v __attribute__((ext_vector_type(16)));
-// MODE 0: every wave multiplies; 1: every wave runs ordinary vector instructions; 2: every wave
-// does both in turn; 3: waves 0-3 multiply, waves 4-7 run vector instructions (one of each per SIMD)
-extern "C" __global__ void __launch_bounds__(512) eh_mfma_valu(float* out) {
-  const int wave = threadIdx.x >> 6;
-  f16v acc[4];
-  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
-  float a = threadIdx.x * 1e-3f, b = blockIdx.x * 1e-3f;
-  float v[8];
-  for (int i = 0; i < 8; ++i) v[i] = a + i;
-  const bool mfma = %(mode)d == 0 || %(mode)d == 2 || (%(mode)d == 3 && wave < 4);
-  const bool valu = %(mode)d == 1 || %(mode)d == 2 || (%(mode)d == 3 && wave >= 4);
-  for (int it = 0; it < %(iters)d; ++it) {
-    if (mfma) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
-    }
-    if (valu) {                          // 64 fused multiply-adds: as many cycles as the four MFMAs
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf(v[i], 1.0001f, 0.5f);
-    }
-  }
-  float s = 0.0f;
-  for (int i = 0; i < 8; ++i) s += v[i];
-  for (int i = 0; i < 4; ++i) for (int r = 0; r < 16; ++r) s += acc[i][r];
-  out[blockIdx.x * 512 + threadIdx.x] = s;
-}
-"""
-
-
-def mfma_valu_overlap(dev, iters=20000):
-    """Whether a SIMD runs one wave's MFMAs beside ordinary vector instructions (its own or another
-    wave's).  Returns microseconds for: MFMAs only and vector instructions only (one wave per
-    SIMD each), both in every wave, and one wave of each kind per SIMD.  If the last two equal the
-    sum of the first two, nothing overlaps."""
-    cus = dev.props["compute_units"]
-    out = hb.HipBuffer(dev, [cus * 512 * 4], None, nbytes=cus * 512 * 4)
-
-    def run(mode, waves):
-        mod = hb.HipModule(dev, hb.compile_source(MFMA_VALU_SOURCE % {"mode": mode, "iters": iters}), "eh_mfma_valu")
-        mod.launch([cus, 1, 1], [waves * 64, 1, 1], [out], sync=True)
-        e0, e1 = hb.Event(dev), hb.Event(dev)
-        e0.record()
-        mod.launch([cus, 1, 1], [waves * 64, 1, 1], [out], sync=False)
-        e1.record()
-        e1.sync()
-        return e0.elapsed_ms(e1) * 1e3
-
-    return {"mfma_only": run(0, 4), "valu_only": run(1, 4), "both_in_each_wave": run(2, 4), "one_wave_of_each_per_simd": run(3, 8)}
-
-
 EMPTY_SOURCE = """
 extern "C" __global__ void __launch_bounds__(256) eh_empty(float* out) {
   if (out == nullptr) out[0] = 0.0f;
@@ -330,6 +295,7 @@ def write_traffic_file(root: str, out_path: str = TRAFFIC_FILE):
     matmul, config1), each the output directory of
         rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -d <dir> -o pmc --output-format csv -- \
             python3 bench.py --only <workload> --steps 10 --warmup 2 --no-cpu-baseline --no-per-kernel --no-check
+    (for the copy kernel: -- python3 -m harp_amd.measure copy)
     FETCH_SIZE / WRITE_SIZE are scaled so that the plain 64 MiB copy kernel reads and writes exactly
     its 65536 KiB (it is assumed to waste nothing); every entry carries the SHA-1 of the generated
     source it was measured on, which bench.py compares with the source it times."""
@@ -368,7 +334,21 @@ def write_traffic_file(root: str, out_path: str = TRAFFIC_FILE):
 
 if __name__ == "__main__":
     import sys
+    usage = ("usage: python -m harp_amd.measure traffic <directory holding <workload>_fetch and <workload>_write>\n"
+             "       python -m harp_amd.measure copy        (HBM rate of this backend's plain 64 MiB copy kernel)\n"
+             "       python -m harp_amd.measure mfma_peak   (issue rate of v_mfma_f32_32x32x2_f32 from registers)")
     if len(sys.argv) == 3 and sys.argv[1] == "traffic":
         print(json.dumps(write_traffic_file(sys.argv[2]), indent=1))
+    elif len(sys.argv) >= 2 and sys.argv[1] in ("copy", "mfma_peak"):
+        if hb.device_count() == 0:
+            sys.exit("harp_amd.measure: no HIP device present")
+        _dev = hb.HipDevice(0)
+        if sys.argv[1] == "copy":
+            gbs, launch, ms = copy_rate(_dev)
+            print(f"copy 4096^2 ({launch['entry']}, {launch['schedule']}): {ms * 1e3:.1f} us/step -> {gbs:.0f} GB/s")
+        else:
+            tflops, blocks, ms = mfma_issue_rate(_dev)
+            print(f"MFMA f32 32x32x2 issue-rate ceiling: {tflops:.1f} TFLOP/s ({tflops / FP32_MFMA_PEAK_TFLOPS:.1%} of the "
+                  f"published {FP32_MFMA_PEAK_TFLOPS}); {blocks} workgroups x 4 waves, {ms * 1e3:.0f} us/launch")
     else:
-        sys.exit("usage: python -m harp_amd.measure traffic <directory holding <workload>_fetch and <workload>_write>")
+        sys.exit(usage)

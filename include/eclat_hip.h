@@ -100,7 +100,10 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      lanes off it and joins them back, so callers still see one stream); launches estimated
  *      above lane_us microseconds (default 100) stay on lane 0.
  *      A kernel that no schedule recognises, would run in a single work-item and loops more than
- *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1. ----------------- */
+ *      2^17 times is refused with EH_ERR_UNSUPPORTED unless allow_serial=1 (loops whose bounds move
+ *      with enclosing loops count by their extreme; bounds that cannot be bounded count as too many).
+ *      A large kernel that is planned one work-item per outer iteration because its loop structure
+ *      was not recognised carries ",degraded" in its schedule string and is logged once. ------- */
 typedef struct eh_launch_info {
   const char* entry;                    /* kernel symbol */
   const char* source;                   /* HIP C translation unit */
@@ -133,6 +136,14 @@ int eh_tune_key(const char* ast_text, unsigned long long* key);
  * loops (src/opt/ast/transforms.rs:238-361, 393-630).  The result computes what the input
  * computes, statement for statement.  *out_text is AST text, released with eh_free. */
 int eh_normalize_ast(const char* ast_text, char** out_text);
+/* The local work size Pipeline::compile_ast derives from a kernel's dispatch hints
+ * (src/backend/pipeline.rs:160-192 with compute_compatible_local_size, :475-489): per dimension the
+ * largest divisor of global[i] that is at most preferred[i], then, while the three multiply to more
+ * than max_work_group, the largest dimension steps down to the next smaller divisor of its global
+ * size.  Kernels that carry their own dispatch (grid x thread group in the AST) are launched with
+ * it: global = grid * thread group, workgroups = global / local.  Kernel::execute_with_sizes
+ * (src/backend/traits.rs:556-566), whose sizes are global, divides by this too. */
+int eh_fit_local_size(const size_t global[3], const size_t preferred[3], size_t max_work_group, size_t local[3]);
 int eh_plan_num_launches(eh_plan* plan, int* n);
 int eh_plan_launch(eh_plan* plan, int launch, eh_launch_info* out);    /* strings live as long as the plan */
 int eh_plan_launch_arg(eh_plan* plan, int launch, int arg, const char** buffer_name);
@@ -171,9 +182,12 @@ int eh_program_launch(eh_program* prog, int launch, eh_launch_info* out);
  * elided buffers and for temps (the program then keeps its own), and bufs may stop anywhere
  * after the last input or output.  sync != 0 waits for completion (the reference's kernels are
  * synchronous); sync == 0 only queues the launches on the device's stream.
- * Different entries of the table must be different buffers (an output must not alias an input):
- * launches that do not depend on each other by buffer name may run in another order than the
- * kernels were written, or together. */
+ * Different entries of the table must be different buffers (an output must not alias an input,
+ * no in-place update): launches that do not depend on each other by buffer name may run in another
+ * order than the kernels were written, or together.  This is checked: two entries bound to
+ * overlapping device memory, at least one of which some launch writes, fail with EH_ERR_INVALID
+ * before anything is queued (eh_program_execute, _static and _record alike); entries the program
+ * only reads may share memory. */
 int eh_program_execute(eh_program* prog, eh_buffer* const* bufs, int n_bufs, int sync);
 int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, int n_inputs,
                                   eh_buffer* const* outputs, int n_outputs, int sync);
@@ -185,10 +199,15 @@ int eh_program_execute_positional(eh_program* prog, eh_buffer* const* inputs, in
  * EH_STATIC_SCRATCH_BYTES that every device the library runs on holds until the process ends;
  * every other buffer that reaches memory (inputs, outputs and the caller's own temps) must be
  * given.  A program whose scratch temps do not fit fails with EH_ERR_SIZE and launches nothing.
- * All calls on one device share that device's block, which keeps the previous call's contents
- * (no kernel relies on them: every scratch element is written before it is read).  Calls that
- * overlap on one device would race on it; calls made through this library do not overlap, because
- * every call's launches are ordered on the device's stream behind those of the call before.
+ * All calls on one GPU share that GPU's block, whichever eh_device handle they come through, and
+ * the block keeps the previous call's contents (no kernel relies on them: every scratch element is
+ * written before it is read).  Calls that overlap on one GPU would race on it.  Calls through one
+ * handle are ordered on that handle's stream; a call through another handle of the same GPU (its
+ * own stream) is made to wait on the device for the launches of the call that used the block
+ * before it, so calls made through this library do not overlap on the block, with sync == 0 too.
+ * What the library cannot order is a launch sequence captured into a caller's graph: when a replay
+ * runs, and beside what, is the caller's business (no wait is recorded under capture), so replays
+ * of such graphs and other users of the block on that GPU must be serialised by the caller.
  * A given buffer that nothing has written yet and that the program does not overwrite whole gets
  * its zero fill queued first (no allocation); under stream capture that is an error instead,
  * since a recorded fill would run again on every replay: write or read such a buffer once before. */

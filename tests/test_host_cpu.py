@@ -41,6 +41,66 @@ def test_rust_binding_names_only_declared_symbols():
     for name, n in bound.items():
         assert name in declared, f"{name} bound in ffi.rs but not declared in eclat_hip.h"
         assert declared[name] == n, f"{name}: {n} parameters in ffi.rs, {declared[name]} in the header"
+
+    # parameter and return types, each side brought to one spelling: base type, then one
+    # "*const" or "*mut" per level of indirection, outermost last
+    def c_type(decl, is_param=True):
+        decl = decl.strip()
+        array = is_param and decl.endswith("]")
+        decl = re.sub(r"\[[0-9]*\]$", "", decl).strip()
+        if is_param:
+            decl = re.sub(r"\b[A-Za-z_][A-Za-z_0-9]*$", "", decl).strip() if not decl.endswith("*") else decl
+        toks = re.findall(r"\*|[A-Za-z_][A-Za-z_0-9]*", decl)
+        # a `const` ahead of the first `*` qualifies the base type; one behind a `*` qualifies that pointer
+        base, levels, base_const = [], [], False
+        for t in toks:
+            if t == "const":
+                if levels:
+                    levels[-1] = "ptrconst"
+                else:
+                    base_const = True
+            elif t == "*":
+                levels.append("*")
+            else:
+                base.append(t)
+        base = " ".join(base)
+        base = {"unsigned": "c_uint", "int": "c_int", "char": "c_char", "void": "c_void", "size_t": "usize",
+                "unsigned long long": "u64", "float": "f32", "double": "f64"}.get(base, base)
+        out, pointee_const = base, base_const
+        for lv in levels:
+            out += " *const" if pointee_const else " *mut"
+            pointee_const = lv == "ptrconst"      # constness of this pointer matters for the next level out
+        if array:
+            out += " *const" if base_const else " *mut"
+        return out
+
+    def rust_type(t):
+        t = t.strip()
+        levels = []
+        while t.startswith("*"):
+            m = re.match(r"\*(const|mut)\s+", t)
+            levels.append("*" + m.group(1))
+            t = t[m.end():]
+        t = {"c_ulonglong": "u64", "i32": "c_int", "u32": "c_uint"}.get(t, t)
+        return " ".join([t] + list(reversed(levels)))
+
+    def c_signature(name):
+        m = re.search(r"([A-Za-z_][A-Za-z_0-9 ]*?[ \*]+)\b" + name + r"\s*\(([^)]*)\)", header)
+        ret, params = m.group(1), m.group(2).strip()
+        ps = [] if params in ("", "void") else [c_type(p) for p in params.split(",")]
+        return c_type(ret.replace("extern", ""), is_param=False), ps
+
+    def rust_signature(name):
+        m = re.search(r"pub fn " + name + r"\(([^)]*)\)\s*(->\s*([^;]+))?;", ffi)
+        params = m.group(1).strip()
+        ps = [rust_type(p.split(":", 1)[1]) for p in params.split(",")] if params else []
+        return rust_type(m.group(3)) if m.group(3) else "c_void", ps
+
+    assert c_type("const char* ast_text") == "c_char *const" and c_type("eh_buffer* const* bufs") == "eh_buffer *mut *const"
+    assert c_type("const unsigned grid[3]") == "c_uint *const" and c_type("const void** blob") == "c_void *const *mut"
+    assert rust_type("*const *mut eh_buffer") == "eh_buffer *mut *const" and rust_type("*mut *const c_void") == "c_void *const *mut"
+    for name in bound:
+        assert rust_signature(name) == c_signature(name), (name, rust_signature(name), c_signature(name))
     # the whole-program path of the binding
     assert {"eh_program_num_buffers", "eh_program_buffer", "eh_program_execute"} <= set(bound)
     with open(os.path.join(ROOT, "crates", "backend-hip", "src", "lib.rs")) as f:
@@ -233,6 +293,51 @@ def test_dispatch_size_expressions(expr, value):
     assert l["schedule"] == "as-written" and l["grid"] == [value, 1, 1]
     with pytest.raises(hb.EhError, match="cannot be evaluated"):
         hb.render_program(text.replace(expr, '(var "n")'))
+
+
+def _fit(global_, preferred, max_wg=1024):
+    import ctypes
+    from harp_amd._lib import check, lib
+    g = (ctypes.c_size_t * 3)(*global_)
+    p = (ctypes.c_size_t * 3)(*preferred)
+    out = (ctypes.c_size_t * 3)()
+    check(lib.eh_fit_local_size(g, p, max_wg, out))
+    return list(out)
+
+
+def test_local_size_is_fitted_as_the_reference_pipeline_does():
+    """`compute_compatible_local_size` (src/backend/pipeline.rs:475-489): the largest divisor of
+    the global size not above the preferred size; then the workgroup is shrunk, largest
+    dimension first, to the next smaller divisor until it fits the device (:176-192)."""
+    assert _fit([1000, 1, 1], [48, 1, 1]) == [40, 1, 1]           # 48 does not divide 1000; 40 does
+    assert _fit([1000, 1, 1], [1000, 1, 1]) == [1000, 1, 1]
+    assert _fit([1000, 1, 1], [2000, 1, 1]) == [1000, 1, 1]       # never above the global size
+    assert _fit([997, 1, 1], [256, 1, 1]) == [1, 1, 1]            # a prime has no other divisor
+    assert _fit([0, 1, 1], [64, 1, 1]) == [1, 1, 1]               # global 0 -> 1 (:476-478)
+    assert _fit([2048, 2048, 1], [64, 64, 1]) == [32, 32, 1]      # 64x64 > 1024: 32x64, then 32x32
+    assert _fit([4096, 6, 1], [2048, 3, 1]) == [256, 3, 1]        # only the largest dimension steps down
+    assert _fit([96, 96, 96], [16, 16, 16], 256) == [6, 6, 6]     # 16^3 -> 12,16,16 -> ... by turns
+    from harp_amd._lib import EhError
+    with pytest.raises(EhError):
+        _fit([8, 8, 8], [0, 1, 1])
+
+
+def test_kernels_with_their_own_dispatch_get_the_fitted_local_size():
+    """global = grid x thread group; a thread group beyond the device's 1024 work-items is shrunk
+    to a divisor of the global size and the workgroup count grows to match."""
+    from harp_amd import backend as hb
+
+    def text(grid, tg):
+        c = lambda v: f"(const i64 {v})"
+        return ('(program (kernel "k" (params ("g" i64 imm (group_id 0)) ("o" (ptr f32 global) mut normal)) '
+                f'(grid {c(grid[0])} {c(grid[1])} {c(grid[2])}) (tg {c(tg[0])} {c(tg[1])} {c(tg[2])}) '
+                '(block (decls) (store (var "o") (var "g") (const f32 1.0)))))')
+    l, = hb.render_program(text([25, 1, 1], [40, 1, 1])).launches
+    assert (l["grid"], l["block"]) == ([25, 1, 1], [40, 1, 1])             # fits: launched as given
+    l, = hb.render_program(text([4, 4, 1], [64, 64, 1])).launches          # 4096 work-items a group
+    assert (l["grid"], l["block"]) == ([8, 8, 1], [32, 32, 1])
+    l, = hb.render_program(text([3, 1, 1], [2048, 1, 1])).launches         # global 6144
+    assert (l["grid"], l["block"]) == ([6, 1, 1], [1024, 1, 1])
 
 
 def test_no_device_is_an_error_not_a_fallback():

@@ -22,9 +22,13 @@ RNG = np.random.default_rng
 TRANSFORMS = [
     [], ["tile=7"], ["tile=2"], ["guard=5"], ["tile=7", "unroll"], ["guard=3", "unroll"],
     ["tile_all=3"], ["tile_all=5", "unroll"], ["tile_outer=7"], ["interchange"],
-    ["tile_outer=3", "unroll"], ["unroll"], ["tile_outer=5", "tile=3"],
+    ["tile_outer=3", "unroll"], ["unroll"], ["tile_outer=5", "tile=3"], ["tile=5", "interchange", "unroll"],
+    ["fma"], ["tile=7", "fma"],
 ]
 IDS = ["+".join(t) or "rules" for t in TRANSFORMS]
+# forms whose normalisation gives a sum back the order the lowerer wrote (an interchanged tile
+# loop): the normalised kernel equals the rewritten one up to the order of the additions
+REORDERING = {"tile=5+interchange+unroll"}
 
 
 @pytest.fixture
@@ -152,8 +156,16 @@ def test_normalised_kernels_compute_what_the_rewritten_ones_compute(frontend, op
             if "rw_" + tid not in live:
                 continue
             rw, nm = run(entries["rw_" + tid]), run(entries["nm_" + tid])
-            assert np.allclose(rw, base, rtol=1e-5, atol=1e-6), (kern.attrs["name"], tid)
-            assert bits_equal_mod_zero(nm, rw), (kern.attrs["name"], tid)
+            # (interchanging the two loops of a tiled scan reorders a recurrence: the reference's
+            # suggester does not check dependences, loop_transforms.rs:710-793, and the form no longer
+            # computes the scan; the normalised kernel must still compute what that form computes)
+            if not (tid in REORDERING and kern.attrs["name"].startswith("P_")):
+                assert np.allclose(rw, base, rtol=1e-5, atol=1e-6), (kern.attrs["name"], tid)
+            if tid in REORDERING and kern.attrs["name"].startswith("R_"):
+                assert np.allclose(nm, rw, rtol=1e-5, atol=1e-6), (kern.attrs["name"], tid)
+                assert bits_equal_mod_zero(nm, base) or name == "softmax", (kern.attrs["name"], tid)   # the lowered order is back
+            else:
+                assert bits_equal_mod_zero(nm, rw), (kern.attrs["name"], tid)
 
 
 def test_normalisation_restores_the_lowered_loop_nest(frontend, opt_env):
@@ -198,12 +210,59 @@ def test_long_serial_kernels_are_refused_not_run_in_one_work_item():
     assert [l["schedule"] for l in forced] == ["as-written"]
 
 
+def _plain_kernels(config, transforms, opt_env):
+    from harp_amd import workloads as wl
+    from harp_amd.frontend import optimize
+    shapes, fn = _headline(config)
+    opt_env(0)
+    plain = wl.lower_with_table(shapes, fn)[4]
+    return [(k, optimize.optimize_kernel(k, transforms)) for k in plain.args]
+
+
+@pytest.mark.parametrize("config", ["config1_relu_sum", "config2_softmax"])
+def test_nested_tiling_with_moving_bounds_is_refused(frontend, opt_env, config):
+    """The inner loops of a tiling tiled again (src/opt/ast/suggesters/loop_transforms.rs:86-110
+    proposes tiling for every step-1 loop, nested ones included): re-tiling a remainder loop that
+    does not start at 0 (`tile_loop`, src/opt/ast/transforms.rs:450-461) leaves a nest whose inner
+    bound moves with an outer variable.  Counted over the outer loop's range it is millions of
+    iterations for one work-item: refused, never launched at 1x1x1."""
+    from harp_amd import backend as hb
+    from harp_amd._lib import EhError
+    from harp_amd.frontend import AstNode
+    for k, rw in _plain_kernels(config, ["tile=2", "tile=3"], opt_env):
+        assert "eh_u0" in hb.normalize_ast(rw)                    # the moving bound survived normalisation
+        with pytest.raises(EhError, match="loop iterations in one work-item") as e:
+            hb.render_program(AstNode.program([rw]))
+        assert e.value.code == 3, k.attrs["name"]                 # EH_ERR_UNSUPPORTED
+
+
+def test_forms_no_schedule_recovers_are_marked_degraded(frontend, opt_env, capfd):
+    """`tile_all=7` then `tile=2` re-tiles the remainder loop [4095, 4096) of a 4096-long axis with the
+    reference's wrong main-loop bound: the rewritten kernel itself reads one element past the axis.
+    Nothing is recovered from that; the plan says so (`degraded`) and the library logs it once, for
+    the elementwise and row kernels as for the contraction that misses the matrix cores.  Where the
+    same composition is clean (1024 = 7 * 146 + 2) the lowered schedules come back."""
+    from harp_amd import backend as hb
+    from harp_amd.frontend import AstNode
+    for k, rw in _plain_kernels("config3_matmul", ["tile_all=7", "tile=2"], opt_env):
+        sched = [l["schedule"] for l in hb.render_program(AstNode.program([rw])).launches]
+        assert sched == ["outer-parallel(work-items=16777216,degraded)"]
+        hb.render_program(AstNode.program([rw]))
+    assert capfd.readouterr().err.count("plan marked 'degraded'") <= 1        # logged once per kernel
+    for k, rw in _plain_kernels("config2_softmax", ["tile_all=7", "tile=2"], opt_env):
+        sched = [l["schedule"] for l in hb.render_program(AstNode.program([rw])).launches]
+        assert sched == ["outer-parallel(work-items=4096,degraded)"], k.attrs["name"]
+    for k, rw in _plain_kernels("config1_relu_sum", ["tile_all=7", "tile=2"], opt_env):
+        want = [l["schedule"] for l in hb.render_program(AstNode.program([k])).launches]
+        assert [l["schedule"] for l in hb.render_program(AstNode.program([rw])).launches] == want
+
+
 # ---------------------------------------------------------------------------------------------
 # GPU
 # ---------------------------------------------------------------------------------------------
 
 GPU_TRANSFORMS = [[], ["tile=7"], ["guard=5"], ["tile=7", "unroll"], ["tile_all=3"], ["tile_outer=7"],
-                  ["interchange"], ["tile=7", "interchange"]]
+                  ["interchange"], ["tile=7", "interchange"], ["tile=5", "interchange", "unroll"], ["fma"]]
 
 
 @pytest.mark.gpu
@@ -243,3 +302,64 @@ def test_opt_levels_give_the_same_results_on_the_gpu(frontend, hip, opt_env):
         opt_env(level)
         outs.append(realize_on(frontend, "hip", wl.config2_graph, [x]))
     assert np.allclose(outs[0], outs[1], rtol=1e-6, atol=1e-12)
+
+
+@pytest.mark.gpu
+def test_fused_multiply_add_forms_match_the_oracle_on_the_gpu(frontend, hip, opt_env):
+    """What the multiply-add rules produce for a device that reports `DeviceInstruction::Fma`
+    (src/opt/ast/rules/mod.rs:117-143; algebraic.rs:218-282), as `Pipeline::optimize_ast` would
+    hand it over.  Elementwise `fma(a, b, c)` is bit-identical to the C backend's `fma(a, b, c)`
+    (double-precision fma on promoted floats, converted back), also where float arithmetic in
+    two steps or a single-precision fused multiply-add would give another value; a reduce whose
+    step is `acc = fma(a, b, acc)` is planned as the sum of products it is (row, column and MFMA
+    schedules) and stays within the reduction tolerances."""
+    from harp_amd.frontend import AstNode as A
+    from harp_amd.frontend.ast import DType, F32, VarDecl
+    from oracle.c_backend import CBuffer, compile_program_text
+    dev = hip.HipDevice(0)
+    n = 1 << 16
+    idx = A.var("ridx0")
+    body = A.range("ridx0", A.const_i64(0), A.const_i64(1), A.const_i64(n),
+                   A.store(A.var("buf6"), idx, A("fma", [A.load(A.var("buf0"), idx, F32), A.load(A.var("buf2"), idx, F32),
+                                                         A.load(A.var("buf4"), idx, F32)])))
+    params = [VarDecl(v, DType.ptr(F32)) for v in ("buf0", "buf2", "buf4")] + [VarDecl("buf6", DType.ptr(F32), mutable=True)]
+    prog = A.program([A.kernel("E_fma", params, body)])
+    rng = RNG(11)
+    x, y = (rng.uniform(1, 2, n).astype(np.float32) for _ in range(2))
+    z = (-(x.astype(np.float64) * y.astype(np.float64))).astype(np.float32)        # cancels all but the product's low bits
+    x[:4] = [1 + 2.0 ** -12, 1 + 2.0 ** -23, 3.0, 1.5]
+    y[:4] = [1 + 2.0 ** -12, 1 - 2.0 ** -23, 7.0, -2.0]
+    z[:4] = [-1.0, -1.0, 0.25, 3.0]
+    k = hip.HipKernel(dev, prog)
+    assert k.launches[0]["schedule"].startswith("flat(") and "fma((double)" in k.launches[0]["source"]
+    bufs = [dev.alloc(4 * n) for _ in range(4)]
+    for b, a in zip(bufs, (x, y, z)):
+        b.write_array(a)
+    k.execute(bufs[:3], bufs[3:])
+    got = bufs[3].read_array(np.float32)
+    ck = compile_program_text(prog.to_sexpr())
+    cb = [CBuffer([n], "f32") for _ in range(4)]
+    for b, a in zip(cb, (x, y, z)):
+        b.write_from_host(a.tobytes())
+    ck.execute(cb[:3], cb[3:])
+    ref = np.frombuffer(cb[3].read_to_host(), np.float32)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    want = (x.astype(np.float64) * y.astype(np.float64) + z.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(got, want)
+    assert np.count_nonzero(got != (x * y + z)) > n // 4            # two float roundings lose the residue
+
+    # reductions in fma form: a row dot product, a column one, a contraction
+    opt_env(3, ["fma"])
+    a = RNG(12).normal(0, 1, (300, 1000)).astype(np.float32)
+    b = RNG(13).normal(0, 1, (300, 1000)).astype(np.float32)
+    for axis in (1, 0):
+        fn = lambda p, q: (p * q).sum(axis)                                          # noqa: E731
+        ref = realize_on(frontend, "c", fn, [a, b])
+        for fuse in (False, True):
+            got = realize_on(frontend, "hip", fn, [a, b], fuse=fuse)
+            scale = (np.abs(a.astype(np.float64)) * np.abs(b)).sum(axis)
+            assert np.all(np.abs(got.astype(np.float64).ravel() - ref.ravel()) <= 1e-5 * scale.ravel())
+    from harp_amd import workloads as wl
+    table = wl.lower_with_table([(192, 640), (640, 160)], wl.config3_graph)[0]
+    assert "(fma " in table.to_sexpr()
+    assert hip.render_program(table).launches[0]["schedule"].startswith("mfma32x32x2(")

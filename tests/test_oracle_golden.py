@@ -55,6 +55,40 @@ def test_rendered_expression_text(frontend):
     assert render_expr(A.recip(A.var("x")).to_sexpr()) == "(1.0f / x)"
 
 
+def test_fused_multiply_add_text_and_value(frontend):
+    """`render_fma` (src/backend/renderer.rs:107-109) writes `fma(a, b, c)` whatever the operand
+    type, and the C renderer does not override it (crates/backend-c/src/renderer.rs:117-224 has no
+    render_fma): on float operands that is C's double-precision fma on promoted values.  The
+    oracle renders that text, and compiled with the reference's flags it computes
+    float(double(a*b + c)) with the product exact -- checked where a*b + c rounded twice in float
+    gives another value."""
+    import ctypes
+    from oracle.c_backend import CKernel
+    from oracle.c_renderer import render_expr, render_program
+    A = frontend.AstNode
+    f = frontend.AstNode("fma", [A.var("a"), A.var("b"), A.var("c")])
+    assert render_expr(f.to_sexpr()) == "fma(a, b, c)"
+    from harp_amd.frontend.ast import DType, F32, VarDecl
+    idx = A.var("i")
+    body = A.range("i", A.const_i64(0), A.const_i64(1), A.const_i64(4),
+                   A.store(A.var("o"), idx, frontend.AstNode("fma", [A.load(A.var("x"), idx, F32), A.load(A.var("y"), idx, F32),
+                                                               A.load(A.var("z"), idx, F32)])))
+    params = [VarDecl(n, DType.ptr(F32)) for n in "xyz"] + [VarDecl("o", DType.ptr(F32), mutable=True)]
+    text = A.program([A.kernel("k_fma", params, body)]).to_sexpr()
+    src = render_program(text)
+    assert "o[i] = fma(x[i], y[i], z[i]);" in src
+    k = CKernel(src, "k_fma", 4)
+    x = np.array([1 + 2.0 ** -12, 3.0, 1.5, 1 + 2.0 ** -23], np.float32)
+    y = np.array([1 + 2.0 ** -12, 7.0, -2.0, 1 - 2.0 ** -23], np.float32)
+    z = np.array([-1.0, 0.25, 3.0, -1.0], np.float32)
+    o = np.zeros(4, np.float32)
+    k.call_raw(*[ctypes.c_void_p(a.ctypes.data) for a in (x, y, z, o)])
+    want = (x.astype(np.float64) * y.astype(np.float64) + z.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(o, want)
+    twice = (x * y + z).astype(np.float32)                  # product rounded to float first
+    assert o[0] != twice[0] and o[3] != twice[3]            # the fused form keeps 2^-24 and -2^-46
+
+
 def test_header_and_types(frontend):
     # crates/backend-c/src/renderer.rs:236-258
     from oracle.c_renderer import HEADER, render_dtype
