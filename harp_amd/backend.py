@@ -331,6 +331,7 @@ class HipModule:
 
 class Event:
     def __init__(self, device: HipDevice):
+        self.device = device           # an event must not outlive its device
         self._h = c_void_p()
         check(lib.eh_event_create(device._h, byref(self._h)))
 

@@ -1384,6 +1384,7 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
     er.ranged = &ranged;
   }
   f.expr = er.expr(*k.value);
+  f.value = k.value;
   if (auto a = affine_of(*loads[0].load->args[1])) {
     for (size_t i = 0; i < k.loops.size(); ++i)
       if (k.loops[i].extent > 1) f.src_stride[strides[i]] = a->of(k.loops[i].var);
@@ -2862,6 +2863,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
         f->src_stride.clear();
         f->plain = false;
         f->ranged_bytes = 0;              // (the expression now calls the inner gather's function)
+        f->value = nullptr;
         folded_kernels.insert(q);
         plan.elided.insert(inner.out_buf);
         break;

@@ -1,4 +1,5 @@
 #include "gemm.hpp"
+#include "window.hpp"
 
 #include <algorithm>
 #include <cctype>
@@ -354,6 +355,10 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
       fb = nullptr;
       plain_tag += ",B:source";
     }
+  if (opt.gemm_window && (fa != nullptr) != (fb != nullptr) && opt.gemm_bm == 0 && opt.gemm_split_k <= 1) {
+    auto w = try_emit_window_gemm(k, *s, fa, fb, opt, epilogue);
+    if (!w.empty()) return w;
+  }
   if (!choose(*s, opt, &ch, fa || fb)) return {};
   const Tile& t = ch.tile;
   // each thread fetches four elements along the operand's faster axis

@@ -54,6 +54,10 @@ struct FoldedOperand {
   // nonzero: `expr` reads `src` through the buffer resource `eh_rs_<src>` over that many bytes
   // (the element function declares it); a byte offset beyond them reads as zero
   size_t ranged_bytes = 0;
+  // the producer's element expression itself (a load, possibly under an index guard with a zero
+  // default), for schedules that take the gather apart instead of calling it; null when the
+  // expression calls another gather's function
+  NodePtr value;
 };
 using FoldMap = std::map<std::string, FoldedOperand>;   // by the producer's output buffer
 

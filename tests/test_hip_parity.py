@@ -1040,7 +1040,9 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
     plain = hip.render_program(prog_ast, {"gemm_fold": 0})
     folded = hip.render_program(prog_ast)
     assert len(folded.launches) < len(plain.launches)
-    assert sum("/folded" in l["schedule"] for l in folded.launches) >= 3
+    assert sum("/folded" in l["schedule"] or "(window," in l["schedule"] for l in folded.launches) >= 3
+    assert sum("(window," in l["schedule"] for l in folded.launches) >= 2
+    assert not any("(window," in l["schedule"] for l in hip.render_program(prog_ast, {"gemm_window": 0}).launches)
     assert sum(b["elided"] for b in folded.buffers) > sum(b["elided"] for b in plain.buffers)
     ref = _cnn_step_on(frontend, "c", arrays)
     reg = _BACKENDS["hip"]
@@ -1052,6 +1054,14 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
         reg.options = old
     got = _cnn_step_on(frontend, "hip", arrays, True)
     for g, p in zip(got, got_plain):
+        assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
+    # the gathers evaluated per element in the tile loader instead of staged in LDS: same sums in another order
+    reg.options = {"gemm_window": 0}
+    try:
+        got_loader = _cnn_step_on(frontend, "hip", arrays, True)
+    finally:
+        reg.options = old
+    for g, p in zip(got, got_loader):
         assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
     # guarded reads (padding) through a buffer resource, out of range where the guard fails
     # (default), or at a clamped index with a select behind them (ranged_loads=0): same bits

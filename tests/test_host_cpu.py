@@ -583,7 +583,14 @@ def test_convolution_plan_folds_both_gathers(frontend):
         exact = hb.render_program(wl.lower_with_table(shapes, conv)[0])
         point = hb.render_program(wl.lower_with_table([(2, 16, 9, 9), (8, 16, 1, 1)], lambda x, w: frontend.nn.conv2d(x, w))[0])
     for p in (exact, point):
-        assert len(p.launches) == 1 and "/folded" in p.launches[0]["schedule"] and sum(b["elided"] for b in p.buffers) == 1
+        assert len(p.launches) == 1 and sum(b["elided"] for b in p.buffers) == 1
+    # the single padded 3x3 gather is taken apart and staged in LDS (one image's channels with their
+    # zero border per workgroup); a 1x1 window has nothing to stage and stays in the tile loader
+    assert exact.launches[0]["schedule"].startswith("mfma16x16x4(window,group=100,M=8,K=36,") and exact.launches[0]["grid"] == [2, 1, 1]
+    assert "/folded" in point.launches[0]["schedule"]
+    with frontend.exact_mode():
+        loader = hb.render_program(wl.lower_with_table(shapes, conv)[0], {"gemm_window": 0})
+    assert len(loader.launches) == 1 and "/folded" in loader.launches[0]["schedule"]
 
 
 def test_option_beam_search_on_a_synthetic_cost():
@@ -742,7 +749,7 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     arrays = wl.config5_inputs(64, *wl.cnn_sizes(True)[1:])
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
-    plan = hb.render_program(ast, "lanes=1")
+    plan = hb.render_program(ast, "lanes=1,gemm_window=0")
     # (transposed product: W as rows; dY, a copy through a view, read from its source with strides)
     cols = [l for l in plan.launches if l["schedule"].startswith("mfma") and "A:m,B:n,B:source" in l["schedule"]]
     assert len(cols) == 1, [l["schedule"] for l in plan.launches]
@@ -762,6 +769,53 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert len(direct) == 2 and all("A:k,B:n/folded" in l["schedule"] for l in direct), [l["schedule"] for l in plan.launches]
 
 
+def test_convolution_windows_are_staged_in_lds(frontend):
+    """The padded 3x3 gathers of the CNN step's convolutions are taken apart (row digit + window
+    digit = source coordinate, guards = where that coordinate leaves the image) and what one
+    image's rows read is staged in LDS once per workgroup: the forward contractions of both
+    convolutions (rows = the image's pixels, the four k of a step along the channels, or along
+    the taps where there is one channel) and the second convolution's weight gradient (rows =
+    channel x tap, k = the image's pixels, two offset patterns where a step of four pixels runs
+    over the end of a row of fourteen).  The multiply loop holds no vector instruction but the
+    MFMAs.  A's rows are staged too, so the first convolution's weight gradient (K = 784 pixels, 196 steps)
+    fits as well."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config5_inputs(*wl.cnn_sizes(True))
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
+    plan = hb.render_program(ast)
+    win = {l["entry"]: l for l in plan.launches if l["schedule"].startswith("mfma16x16x4(window,")}
+    assert sorted(win) == ["ehk_R_256_196_64_1_9", "ehk_R_256_1_32_9_79", "ehk_R_256_1_64_288_88", "ehk_R_256_784_32_1_1"]
+    fwd2, wg2, fwd1 = win["ehk_R_256_196_64_1_9"], win["ehk_R_256_1_64_288_88"], win["ehk_R_256_784_32_1_1"]
+    assert fwd2["schedule"].startswith("mfma16x16x4(window,group=196,M=64,K=288,waves=4x1,blocks=1x13,steps=72,patterns=1,")
+    assert fwd2["grid"] == [256, 1, 1] and fwd2["block"] == [256, 1, 1] and "epilogue=2" in fwd2["schedule"]
+    assert wg2["schedule"].startswith("mfma16x16x4(window,group=288,M=64,K=196,waves=4x1,blocks=1x18,steps=49,patterns=2,")
+    assert wg2["grid"] == [1, 1, 256]
+    assert fwd1["schedule"].startswith("mfma16x16x4(window,group=784,M=32,K=9,waves=2x2,blocks=1x25,steps=3,patterns=3,")
+    for l in win.values():
+        assert len(hb.compile_source(l["source"])) > 1000
+    # one image: 32 channels of 16 x 16 (14 x 14 and its border), the channel stride padded off the banks
+    import re
+    m = re.search(r"axes \[32 x stride 196, valid 0\.\.32, lds (\d+)\] \[16 x stride 14, valid 1\.\.15, lds 16\] "
+                  r"\[16 x stride 1, valid 1\.\.15, lds 1\]", fwd2["source"])
+    assert m and 256 < int(m.group(1)) < 320
+    # (the four pixels of a step: consecutive, or two at the end of a row and two at the start of the next, 16 apart)
+    assert "if (p == 0) return 0 + b0 * 1 + b1 * 2 + (b0 & b1) * 0;" in wg2["source"]
+    assert "if (p == 1) return 0 + b0 * 1 + b1 * 4 + (b0 & b1) * 0;" in wg2["source"]
+    wg1 = win["ehk_R_256_1_32_9_79"]
+    assert wg1["schedule"].startswith("mfma16x16x4(window,group=9,M=32,K=784,waves=2x1,blocks=1x1,steps=196,patterns=1,")
+    assert wg1["grid"] == [1, 1, 256] and wg1["block"] == [128, 1, 1]
+    assert not any("/folded" in l["schedule"] for l in plan.launches)
+    # the same buffers elided either way (the tile loader splits K for the first convolution's weight
+    # gradient and needs a scratch buffer and a summing launch for it; the staged form does not)
+    loader = hb.render_program(ast, "gemm_window=0")
+    assert not any("(window," in l["schedule"] for l in loader.launches) and len(loader.launches) >= len(plan.launches)
+    gone = lambda p: {b["name"] for b in p.buffers if b["elided"]}          # noqa: E731
+    # (with K split, the per-image results of that weight gradient are summed from the partial tiles and never exist)
+    assert gone(plan) <= gone(loader) and len(gone(loader) - gone(plan)) <= 1
+
+
 def test_convolution_rows_run_across_images(frontend):
     """196 pixels an image are no multiple of a 64-wide tile: the second convolution's forward
     contraction takes (image, pixel) as one axis (784 tiles for 256 images, none padded per
@@ -773,7 +827,7 @@ def test_convolution_rows_run_across_images(frontend):
     arrays = wl.config5_inputs(*wl.cnn_sizes(True))
     ts = [Tensor.input(list(a.shape)) for a in arrays]
     ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
-    plan = hb.render_program(ast, "lanes=1")
+    plan = hb.render_program(ast, "lanes=1,gemm_window=0")           # the tile-loader schedule
     (fwd,) = [l for l in plan.launches if l["entry"] == "ehk_R_256_196_64_1_9"]
     assert "C:split" in fwd["schedule"] and "edges" not in fwd["schedule"], fwd["schedule"]
     assert fwd["grid"] == [256 * 196 // 64, 1, 1]
