@@ -3041,6 +3041,12 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
         return false;
       };
       std::ostringstream fn, body;
+      // the same function in two parts, for schedules that finish many elements per work-item in a
+      // row: everything read from memory first (eh_epilogue_load), the arithmetic and the stores
+      // after (eh_epilogue_apply); only when no read sits under a guard
+      std::ostringstream load_body, apply_body;
+      std::vector<std::string> slot_types;
+      bool split_ok = true;
       std::vector<std::string> ext_order;
       std::map<std::string, std::pair<std::string, size_t>> ext;   // name -> (declaration, min bytes)
       epi.store_c = needed(k0.out_buf);
@@ -3048,22 +3054,26 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       const std::string IT = small ? "int" : "long long";
       const std::string UT = small ? "unsigned" : "unsigned long long";
       body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n";
+      load_body << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n  (void)eh_l;\n";
       body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
       if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
-      auto decode = [&](const NestKernel& sk, const std::string& from) {
+      apply_body << body.str();
+      auto decode_to = [&](std::ostringstream& to, const NestKernel& sk, const std::string& from) {
         int64_t numel = 0;
         auto strides = *dense_strides(sk, &numel);
         for (size_t li = 0; li < sk.loops.size(); ++li) {
           const Loop& l = sk.loops[li];
-          if (l.extent == 1) body << "    const " << IT << " " << l.var << " = 0;\n";
-          else body << "    const " << IT << " " << l.var << " = (" << IT << ")(((" << UT << ")" << from << " / " << strides[li] << "u) % "
-                    << l.extent << "u);\n";    // (never negative: the unsigned division is the cheaper one)
+          if (l.extent == 1) to << "    const " << IT << " " << l.var << " = 0;\n";
+          else to << "    const " << IT << " " << l.var << " = (" << IT << ")(((" << UT << ")" << from << " / " << strides[li] << "u) % "
+                  << l.extent << "u);\n";    // (never negative: the unsigned division is the cheaper one)
         }
       };
+      auto decode = [&](const NestKernel& sk, const std::string& from) { decode_to(body, sk, from); };
       if (c_relaid && relaid_pos > 0) {
         // where this element sat before C took the later consumer's layout: the stages
         // ahead of that consumer index their other operands with it
         if (epi.store_c) throw Error("internal: relaid contraction '" + k0.name + "' must not store C");
+        split_ok = false;
         body << "  " << IT << " eh_lo;\n  {\n";
         decode(*nests[taken[relaid_pos]], "eh_l");
         body << "    eh_lo = ";
@@ -3113,6 +3123,35 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           epi.bytes += static_cast<double>(elems.count(b) ? elems.at(b) : 0) * et.itemsize();
         }
         body << "    eh_v_" << sk.out_buf << " = (" << ctype(sk.out_dtype) << ")(" << er.expr(*sk.value) << ");\n";
+        {
+          // the two-part form of this stage
+          std::set<const Node*> guarded;
+          for (const auto& lr : loads)
+            if (lr.guarded) guarded.insert(lr.load);
+          apply_body << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << ";\n  {\n";
+          decode_to(apply_body, sk, "eh_l");
+          load_body << "  {\n";
+          decode_to(load_body, sk, "eh_l");
+          ExprRenderer er2;
+          er2.load_hook = [&](const Node& ld, std::string* out) {
+            const std::string& lb = ld.args[0]->name;
+            if (avail.count(lb)) {
+              *out = "eh_v_" + lb;
+              return true;
+            }
+            if (guarded.count(&ld)) split_ok = false;
+            ExprRenderer plain;
+            const std::string slot = "eh_p.v" + std::to_string(slot_types.size());
+            load_body << "    " << slot << " = " << plain.expr(ld) << ";\n";
+            slot_types.push_back(ctype(ld.dtype));
+            *out = slot;
+            return true;
+          };
+          apply_body << "    eh_v_" << sk.out_buf << " = (" << ctype(sk.out_dtype) << ")(" << er2.expr(*sk.value) << ");\n";
+          load_body << "  }\n";
+          if (needed(sk.out_buf)) apply_body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
+          apply_body << "  }\n";
+        }
         if (needed(sk.out_buf)) {
           body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
           ext[sk.out_buf] = {ctype(sk.out_dtype) + "* __restrict__ " + sk.out_buf,
@@ -3137,6 +3176,18 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
          << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params
          << ") {\n" << body.str() << "}\n";
       epi.function = fn.str();
+      if (split_ok && !slot_types.empty() && slot_types.size() <= 8) {
+        std::ostringstream sp;
+        sp << "// the same in two parts: what it reads from memory, then the rest\nstruct EhEpiLoads {\n";
+        for (size_t q = 0; q < slot_types.size(); ++q) sp << "  " << slot_types[q] << " v" << q << ";\n";
+        sp << "};\n__device__ __forceinline__ void eh_epilogue_load(long long eh_e, EhEpiLoads& eh_p" << epi.params << ") {\n"
+           << load_body.str() << "}\n";
+        sp << "__device__ __forceinline__ void eh_epilogue_apply(long long eh_e, float eh_acc, const EhEpiLoads& eh_p"
+           << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params << ") {\n"
+           << apply_body.str() << "}\n";
+        epi.split_functions = sp.str();
+        epi.n_loads = static_cast<int>(slot_types.size());
+      }
       have_epi = true;
     }
     return have_epi;

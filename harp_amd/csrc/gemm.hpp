@@ -75,6 +75,12 @@ struct EpilogueSpec {
   std::vector<std::string> kernels;    // names of the kernels taken in
   bool store_c = true;
   double bytes = 0;                    // algorithmic bytes of the extra parameters
+  // The same function in two parts, when nothing it reads sits under a guard (else empty):
+  //   struct EhEpiLoads; void eh_epilogue_load(long long eh_e, EhEpiLoads&, <params>);
+  //   void eh_epilogue_apply(long long eh_e, float eh_acc, const EhEpiLoads&, [C,] <params>);
+  // for schedules that finish many elements per work-item: all reads first, then the stores.
+  std::string split_functions;
+  int n_loads = 0;                     // values eh_epilogue_load fetches per element
 };
 
 // True when element (b, m, n) of C sits at (b*M + m)*N + n, the index an epilogue is written for.

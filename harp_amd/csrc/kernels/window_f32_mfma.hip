@@ -11,7 +11,7 @@
 // nothing but ds_read_b32 at a per-lane base plus a compile-time offset, and MFMAs: no guards, no
 // address arithmetic, each source element fetched from memory once per workgroup.
 //
-// One workgroup = one group of EW_NG rows of F (the rows that share a patch) x EW_MW rows of A x
+// One workgroup = one group of EW_NG rows of F (the rows that share a patch) x all rows of A x
 // all of K.  A wave owns EW_MB x EW_NB accumulators of v_mfma_f32_16x16x4_f32 (16 rows of A by 16
 // rows of F by 4 k).  A's rows are staged in LDS too, with coalesced loads (a lane needs
 // A[i][k0(s) + j * delta] at step s: read straight from memory that is one cache line per lane
@@ -33,7 +33,6 @@
 #ifndef EW_ENTRY
 #define EW_ENTRY ehk_window_default
 #define EW_M 64            // rows of A
-#define EW_MW 64           // rows of A per workgroup (EW_M split over blockIdx.y)
 #define EW_NG 196          // rows of F per group
 #define EW_GROUPS 256      // groups per batch element
 #define EW_K 288
@@ -43,27 +42,15 @@
 #define EW_NB 13
 #define EW_KSTEPS 72
 #define EW_NPAT 1
+#define EW_KDELTA 9         // k of sub-step j of step s: ew_k0[s] + j * EW_KDELTA
 #define EW_PATCH_FLOATS 8688
 #define EW_PATCH_ELEMS 8192
-#define EW_A_OFF 0LL
-#define EW_A_BS 0LL
-#define EW_A_SM 288LL
-#define EW_A_SK 1LL
-#define EW_A_MSPLIT 0LL
-#define EW_A_SM2 0LL
 #define EW_A_VEC 1         // A is read with 128-bit loads along k
+#define EW_A_ELEMS 4608    // elements (vectors of four with EW_A_VEC) of A to fetch
+#define EW_A_ZERO 0        // A's tile has padding rows or columns, which must read as zero
 #define EW_KPAD 288        // K rounded up to a multiple of four
 #define EW_A_LDS 292       // floats between rows of A in LDS
-#define EH_C_OFF 0LL
-#define EH_C_BS 0LL
-#define EH_C_SM 196LL
-#define EH_C_SN 1LL
-#define EH_C_MSPLIT 0LL
-#define EH_C_SM2 0LL
-#define EH_C_NSPLIT 196LL
-#define EH_C_SN2 12544LL
 #define EW_SRC_BYTES 6422528u
-#define EW_KDELTA 9         // k of sub-step j of step s: ew_k0[s] + j * EW_KDELTA
 namespace {
 struct EwTables {
   int k0[EW_KSTEPS], koff[EW_KSTEPS], kpat[EW_KSTEPS];
@@ -96,6 +83,17 @@ __device__ __forceinline__ void ew_patch_elem(int e, long long g, long long bz, 
   const bool ok = (y >= 1) & (y < 15) & (x >= 1) & (x < 15);
   *src_byte = ok ? (unsigned)((g * 6272 + c * 196 + (y - 1) * 14 + (x - 1)) << 2) : 0x80000000u;
 }
+// element e of A in the order of its memory (here: vector e of four along k): offset in memory, offset in the tile
+__device__ __forceinline__ void ew_a_elem(int e, long long bz, int* lds, long long* off) {
+  (void)bz;
+  const int m = e / 72, k = (e % 72) * 4;
+  *lds = m * EW_A_LDS + k;
+  *off = (long long)m * 288 + k;
+}
+// offsets in C of row m, of row n of F (counted over all groups), of batch element bz
+__device__ __forceinline__ long long ew_c_m(int m) { return (long long)m * 196; }
+__device__ __forceinline__ long long ew_c_n(long long n) { return (n / 196) * 12544 + n % 196; }
+__device__ __forceinline__ long long ew_c_b(long long bz) { (void)bz; return 0; }
 #endif
 
 #ifndef EH_EPILOGUE
@@ -116,14 +114,9 @@ __device__ __forceinline__ void ew_patch_elem(int e, long long g, long long bz, 
 typedef float ew_f4v __attribute__((ext_vector_type(4)));
 
 namespace {
-constexpr int EW_NT = EW_WAVES_M * EW_WAVES_N * 64;
-
-// offset of position v along an axis of stride S, or of SPLIT positions of stride S inside extents S2 apart
-template <long long SPLIT, long long S, long long S2>
-__device__ __forceinline__ long long ew_axis_offset(long long v) {
-  constexpr long long D = SPLIT > 0 ? SPLIT : 1;
-  return SPLIT > 0 ? (v / D) * S2 + (v % D) * S : v * S;
-}
+// Four waves whatever the layout: waves beyond EW_WAVES_M * EW_WAVES_N only help to fetch.
+constexpr int EW_NT = 256;
+static_assert(EW_WAVES_M * EW_WAVES_N <= 4, "at most four multiplying waves");
 }  // namespace
 
 extern "C" __global__ void __launch_bounds__(EW_NT)
@@ -136,60 +129,47 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
   const int wm = wid % EW_WAVES_M, wn = wid / EW_WAVES_M;
   const int l16 = lane & 15, j4 = lane >> 4;
   const long long g = blockIdx.x, bz = blockIdx.z;
-  const int m_wg = blockIdx.y * EW_MW;
 
-  // A's rows of this workgroup into LDS, read along whichever of its axes is contiguous in memory
-  // (128-bit loads where rows allow); k beyond K and rows beyond M are zero.  Every load of a chunk is
-  // issued before the first value is stored: a workgroup is alone on its CU for most of its life, so
-  // nothing else would hide one load's latency behind another's.
+  // A into LDS, fetched in the order of its memory (128-bit loads where rows allow); rows beyond M
+  // and k beyond K of the tile are zero.  Every load of a chunk is issued before the first value is
+  // stored: a workgroup is alone on its CU for most of its life, so nothing else would hide one
+  // load's latency behind another's.
   {
-    const float* a0 = A + EW_A_OFF + bz * EW_A_BS;
-#if EW_A_VEC
-    constexpr int KQ = EW_KPAD / 4;
-    constexpr int PER = (MROWS * KQ + EW_NT - 1) / EW_NT;
+#if EW_A_ZERO
+    for (int e = tid; e < MROWS * EW_A_LDS; e += EW_NT) As[e] = 0.0f;
+    __syncthreads();
+#endif
+    constexpr int PER = (EW_A_ELEMS + EW_NT - 1) / EW_NT;
     constexpr int CH = PER < 24 ? PER : 24;
     for (int c0 = 0; c0 < PER; c0 += CH) {
+#if EW_A_VEC
       ew_f4v v[CH];
-#pragma unroll
-      for (int u = 0; u < CH; ++u) {
-        const int e = (c0 + u) * EW_NT + tid;
-        const int m = e / KQ, kq = e % KQ;
-        const bool ok = e < MROWS * KQ && m_wg + m < EW_M && m < EW_MW && kq * 4 < EW_K;
-        const long long mo = ew_axis_offset<EW_A_MSPLIT, EW_A_SM, EW_A_SM2>(ok ? m_wg + m : 0);
-        const ew_f4v x = *reinterpret_cast<const ew_f4v*>(a0 + mo + (ok ? kq * 4 : 0));
-        v[u] = ok ? x : ew_f4v{0.0f, 0.0f, 0.0f, 0.0f};
-      }
-#pragma unroll
-      for (int u = 0; u < CH; ++u) {
-        const int e = (c0 + u) * EW_NT + tid;
-        if (e < MROWS * KQ) *reinterpret_cast<ew_f4v*>(&As[(e / KQ) * EW_A_LDS + (e % KQ) * 4]) = v[u];
-      }
-    }
 #else
-    constexpr int PER = (MROWS * EW_KPAD + EW_NT - 1) / EW_NT;
-    constexpr int CH = PER < 32 ? PER : 32;
-    for (int c0 = 0; c0 < PER; c0 += CH) {
       float v[CH];
+#endif
+      int at[CH];
 #pragma unroll
       for (int u = 0; u < CH; ++u) {
         const int e = (c0 + u) * EW_NT + tid;
-        // consecutive work-items along the axis with the smaller stride
-        const int m = EW_A_SK <= EW_A_SM ? e / EW_KPAD : e % MROWS;
-        const int k = EW_A_SK <= EW_A_SM ? e % EW_KPAD : e / MROWS;
-        const bool ok = e < MROWS * EW_KPAD && m_wg + m < EW_M && m < EW_MW && k < EW_K;
-        const long long mo = ew_axis_offset<EW_A_MSPLIT, EW_A_SM, EW_A_SM2>(ok ? m_wg + m : 0);
-        const float x = a0[mo + (ok ? (long long)k * EW_A_SK : 0LL)];
-        v[u] = ok ? x : 0.0f;
+        long long off = 0;
+        ew_a_elem(e < EW_A_ELEMS ? e : 0, bz, &at[u], &off);
+#if EW_A_VEC
+        v[u] = *reinterpret_cast<const ew_f4v*>(A + off);
+#else
+        v[u] = A[off];
+#endif
       }
 #pragma unroll
       for (int u = 0; u < CH; ++u) {
-        const int e = (c0 + u) * EW_NT + tid;
-        const int m = EW_A_SK <= EW_A_SM ? e / EW_KPAD : e % MROWS;
-        const int k = EW_A_SK <= EW_A_SM ? e % EW_KPAD : e / MROWS;
-        if (e < MROWS * EW_KPAD) As[m * EW_A_LDS + k] = v[u];
+        if ((c0 + u) * EW_NT + tid < EW_A_ELEMS) {
+#if EW_A_VEC
+          *reinterpret_cast<ew_f4v*>(&As[at[u]]) = v[u];
+#else
+          As[at[u]] = v[u];
+#endif
+        }
       }
     }
-#endif
   }
 
   // the patch: every element of the source region this group's rows read, once; zeros where the
@@ -215,6 +195,7 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
     }
   }
   __syncthreads();
+  if (wid >= EW_WAVES_M * EW_WAVES_N) return;      // (no barrier follows)
 
   // per-lane LDS bases: the lane's row of A in each M-block plus its sub-k; the lane's row of F in
   // each N-block plus its sub-k offset under each pattern.  N-blocks are dealt to the waves in
@@ -279,20 +260,49 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
   // run of straight-line code: whatever the epilogue loads (a bias, a saved activation) is then
   // requested for all of them before the first store goes out, where a branch around every element
   // would make each element's load wait for the stores of the one before (one queue for both).
-  constexpr bool M_EDGE = EW_M % 16 != 0 || EW_MW % 16 != 0 || MROWS != EW_MW;
+  constexpr bool M_EDGE = MROWS != EW_M;
+  const long long c_base = ew_c_b(bz);
   auto finish = [&](const int mb, const int nb, const int v, const bool test) {
-    const int m = m_wg + (wm * EW_MB + mb) * 16 + 4 * j4 + v;
+    const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
     const int n = (nb * EW_WAVES_N + wn) * 16 + l16;
-    if (test && !(m < EW_M && m < m_wg + EW_MW && n < EW_NG)) return;
-    const long long crow = ew_axis_offset<EH_C_MSPLIT, EH_C_SM, EH_C_SM2>(m);
-    const long long ccol = ew_axis_offset<EH_C_NSPLIT, EH_C_SN, EH_C_SN2>(g * EW_NG + n);
-    const long long e = EH_C_OFF + bz * EH_C_BS + crow + ccol;
+    if (test && !(m < EW_M && n < EW_NG)) return;
+    const long long e = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
 #if defined(EH_EPILOGUE)
     eh_epilogue(e, acc[mb][nb][v] EH_C_ARG EH_EPI_ARGS);
 #else
     C[e] = acc[mb][nb][v];
 #endif
   };
+#if defined(EH_EPILOGUE_SPLIT)
+  // in runs of blocks: everything the epilogue reads for a run is requested before the run's first store
+  constexpr int RUN = EH_EPILOGUE_SPLIT <= 1 ? 12 : EH_EPILOGUE_SPLIT <= 2 ? 6 : EH_EPILOGUE_SPLIT <= 4 ? 3 : 1;
+#pragma unroll
+  for (int mb = 0; mb < EW_MB; ++mb)
+#pragma unroll
+    for (int nb0 = 0; nb0 < EW_NB; nb0 += RUN) {
+      EhEpiLoads got[RUN][4];
+      long long at[RUN][4];
+#pragma unroll
+      for (int nb = nb0; nb < nb0 + RUN && nb < EW_NB; ++nb)
+        if (!M_EDGE && (nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
+            const int n = (nb * EW_WAVES_N + wn) * 16 + l16;
+            at[nb - nb0][v] = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
+            eh_epilogue_load(at[nb - nb0][v], got[nb - nb0][v] EH_EPI_ARGS);
+          }
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int nb = nb0; nb < nb0 + RUN && nb < EW_NB; ++nb)
+        if (!M_EDGE && (nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) eh_epilogue_apply(at[nb - nb0][v], acc[mb][nb][v], got[nb - nb0][v] EH_C_ARG EH_EPI_ARGS);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#else
 #pragma unroll
   for (int mb = 0; mb < EW_MB; ++mb)
 #pragma unroll
@@ -301,6 +311,7 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
 #pragma unroll
         for (int v = 0; v < 4; ++v) finish(mb, nb, v, false);
       }
+#endif
 #pragma unroll
   for (int mb = 0; mb < EW_MB; ++mb)
 #pragma unroll

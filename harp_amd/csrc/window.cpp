@@ -1,7 +1,9 @@
 #include "window.hpp"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
+#include <functional>
 #include <map>
 #include <set>
 #include <sstream>
@@ -18,165 +20,119 @@ const char* kWindowSource =
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-enum Side { kBatch = 0, kRow = 1, kK = 2 };
+// why a problem was turned down, for whoever sets EH_WINDOW_DEBUG
+#define BAIL(n)                                                                                   \
+  do {                                                                                            \
+    if (std::getenv("EH_WINDOW_DEBUG")) std::fprintf(stderr, "window schedule: %s declined at check %d\n", p.entry.c_str(), n); \
+    return {};                                                                                    \
+  } while (0)
 
-// One loop of the folded gather: which axis of the contraction it belongs to, its unit there
-// (the index along that axis moves by `unit` per step of the loop), its stride in the source.
-struct WLoop {
-  std::string name;
-  int64_t extent = 1, ostride = 0, sstride = 0, unit = 0;
-  Side side = kRow;
-  int axis = -1;          // patch axis (loops inside the workgroup), or -1
+// A loop with what the emitter derives for it.
+struct L {
+  WLoop w;
+  int64_t unit = 1;       // weight in its side's flat index
+  int axis = -1;          // patch axis (loops inside the workgroup that move F's source), or -1
   bool in_wg = false;
 };
 
-// One coordinate of the patch: a source axis walked by one loop, or by the sum of a row loop and
-// a window loop (same stride in the source).
+// One coordinate of the patch: a source axis walked by one loop, or by a row loop and a window
+// loop together (same stride in the source, either sign: the coordinate is the sum of the digits
+// of the loops with a positive stride and of extent - 1 - digit of those with a negative one).
 struct PAxis {
-  int64_t sstride = 0, extent = 1, lds = 0;
+  int64_t sstride = 0, extent = 1, lds = 0, shift = 0;
   int64_t lo = 0, hi = 0;     // coordinates in [lo, hi) exist in the source; the rest is padding
 };
-
-// e >= bound (ge) or e < bound, e an affine form over the gather's loops without constant term
-struct Atom {
-  Affine e;
-  bool ge = false;
-  int64_t bound = 0;
-};
-
-bool collect_atoms(const Node& c, std::vector<Atom>* out) {
-  if (c.op == Op::And || c.op == Op::BitAnd) return collect_atoms(*c.args[0], out) && collect_atoms(*c.args[1], out);
-  const Node* lt = &c;
-  bool neg = false;
-  if (c.op == Op::Not && c.args[0]->op == Op::Lt) {
-    lt = c.args[0].get();
-    neg = true;
-  }
-  if (lt->op != Op::Lt) return false;
-  auto l = affine_of(*lt->args[0]);
-  auto r = affine_of(*lt->args[1]);
-  if (!l || !r) return false;
-  // l < r  <=>  (l - r without constants) < r.c - l.c
-  Atom a;
-  a.e = *l;
-  for (const auto& kv : r->coef) a.e.coef[kv.first] -= kv.second;
-  a.bound = r->c - l->c;
-  a.e.c = 0;
-  a.ge = neg;
-  for (auto it = a.e.coef.begin(); it != a.e.coef.end();)
-    it = it->second == 0 ? a.e.coef.erase(it) : std::next(it);
-  out->push_back(a);
-  return true;
-}
 
 struct Layout {
   int waves_m = 1, waves_n = 1, mb = 1, nb = 1;
 };
 
+// worst number of distinct addresses falling into one LDS bank, minus one, summed over the two
+// halves of a wave for 32 banks and over the wave for 64
+int64_t bank_cost(const int64_t (&addr)[64]) {
+  int64_t cost = 0;
+  for (int banks : {32, 64})
+    for (int g0 = 0; g0 < 64; g0 += banks) {
+      std::map<int64_t, std::set<int64_t>> per_bank;
+      for (int lane = g0; lane < g0 + banks; ++lane) per_bank[((addr[lane] % banks) + banks) % banks].insert(addr[lane]);
+      size_t worst = 1;
+      for (const auto& kv : per_bank) worst = std::max(worst, kv.second.size());
+      cost += static_cast<int64_t>(worst) - 1;
+    }
+  return cost;
+}
+
+// text: sum over `ls` of ((<var> / unit) % extent) * stride(l), as long long
+std::string digits_sum(const std::vector<const L*>& ls, const std::string& var, const std::function<int64_t(const L&)>& stride) {
+  std::ostringstream os;
+  os << "0LL";
+  for (const L* l : ls) {
+    if (stride(*l) == 0) continue;
+    os << " + (long long)((" << var << " / " << l->unit << "u) % " << l->w.extent << "u) * " << stride(*l) << "LL";
+  }
+  return os.str();
+}
+
 }  // namespace
 
-std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShape& s_in, const FoldedOperand* fa,
-                                             const FoldedOperand* fb, const GenOptions& opt, const EpilogueSpec* epilogue) {
-  if ((fa != nullptr) == (fb != nullptr)) return {};
-  // the folded operand takes the column side: C^T = F^T A^T when it came as A
-  GemmShape s = s_in;
-  const FoldedOperand* f = fb;
-  if (fa) {
-    f = fa;
-    s.M = s_in.N; s.N = s_in.M;
-    s.a_buf = s_in.b_buf; s.b_buf = s_in.a_buf;
-    s.a_m = s_in.b_n; s.a_k = s_in.b_k; s.a_off = s_in.b_off; s.a_b = s_in.b_b;
-    s.a_msplit = s_in.b_nsplit; s.a_m2 = s_in.b_n2;
-    s.b_n = s_in.a_m; s.b_k = s_in.a_k; s.b_off = s_in.a_off; s.b_b = s_in.a_b;
-    s.b_nsplit = s_in.a_msplit; s.b_n2 = s_in.a_m2;
-    s.c_m = s_in.c_n; s.c_n = s_in.c_m;
-    s.c_msplit = s_in.c_nsplit; s.c_m2 = s_in.c_n2; s.c_nsplit = s_in.c_msplit; s.c_n2 = s_in.c_m2;
+std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& opt, const EpilogueSpec* epilogue) {
+  // ---- loops by side, units ---------------------------------------------------------------------
+  std::vector<L> loops;
+  for (const auto& w : p.loops) {
+    if (w.extent < 1) BAIL(1);
+    if (w.extent == 1) continue;
+    L l;
+    l.w = w;
+    loops.push_back(l);
   }
-  if (!f->value || f->ranged_bytes == 0 || !f->small || !f->prelude.empty()) return {};
-  if (s.b_off != 0 || s.b_nsplit != 0 || s.K < 4 || s.M < 2 || s.N < 2 || s.batch > 65535) return {};
-  if (s.a_off < 0 || s.a_k <= 0 || s.a_m < 0) return {};
-
-  // ---- the gather: load index and guard ----------------------------------------------------
-  const Node* v = f->value.get();
-  std::vector<Atom> atoms;
-  if (v->op == Op::Select) {
-    if (v->args[2]->op != Op::Const || v->args[2]->fval != 0.0 || !collect_atoms(*v->args[0], &atoms)) return {};
-    v = v->args[1].get();
-  }
-  if (v->op != Op::Load || v->args[0]->op != Op::Var || v->args[0]->name != f->src) return {};
-  auto idx = affine_of(*v->args[1]);
-  if (!idx) return {};
-
-  // ---- loops by contraction axis -------------------------------------------------------------
-  std::vector<WLoop> loops;
-  struct AxisRange { int64_t s, e; Side side; };
-  const AxisRange ranges[3] = {{s.b_b, s.batch, kBatch}, {s.b_n, s.N, kRow}, {s.b_k, s.K, kK}};
-  int64_t covered[3] = {1, 1, 1}, lowest[3] = {0, 0, 0};
-  for (const auto& l : f->loops) {
-    if (l.extent <= 1) {
-      if (idx->of(l.name) != 0 && l.extent < 1) return {};
-      continue;
+  auto side_loops = [&](WSide s) {
+    std::vector<size_t> v;
+    for (size_t i = 0; i < loops.size(); ++i)
+      if (loops[i].w.side == s) v.push_back(i);
+    return v;
+  };
+  const std::vector<size_t> row_loops = side_loops(WSide::Row), k_loops = side_loops(WSide::K), m_loops = side_loops(WSide::M),
+                            batch_loops = side_loops(WSide::Batch);
+  auto set_units = [&](const std::vector<size_t>& v) {
+    int64_t u = 1;
+    for (size_t q = v.size(); q-- > 0;) {
+      loops[v[q]].unit = u;
+      u *= loops[v[q]].w.extent;
     }
-    WLoop w;
-    w.name = l.name;
-    w.extent = l.extent;
-    w.ostride = l.stride;
-    w.sstride = idx->of(l.name);
-    if (w.sstride <= 0) return {};
-    bool placed = false;
-    for (const auto& r : ranges) {
-      if (r.e <= 1 || r.s <= 0) continue;
-      if (l.stride < r.s || l.stride >= r.s * r.e) continue;
-      if (l.stride * l.extent > r.s * r.e || l.stride % r.s != 0) return {};
-      w.side = r.side;
-      w.unit = l.stride / r.s;
-      covered[r.side] *= l.extent;
-      lowest[r.side] = lowest[r.side] == 0 ? l.stride : std::min(lowest[r.side], l.stride);
-      placed = true;
-      break;
-    }
-    if (!placed) return {};
-    loops.push_back(w);
+    return u;
+  };
+  const int64_t N = set_units(row_loops), K = set_units(k_loops), M = set_units(m_loops), batch = set_units(batch_loops);
+  if (K < 4 || M < 2 || N < 2 || batch > 65535 || M > (1 << 20) || K > (1 << 20)) BAIL(2);
+  for (const auto& l : loops) {
+    if ((l.w.side == WSide::Row || l.w.side == WSide::K) && l.w.f == 0) BAIL(3);
+    if (l.w.side == WSide::M && l.w.f != 0) BAIL(4);
+    if (l.w.side == WSide::Row && l.w.a != 0) BAIL(5);
+    if (l.w.side == WSide::K && l.w.c != 0) BAIL(6);
+    if (l.w.a < 0 || l.w.c < 0) BAIL(7);
+    if (l.w.side == WSide::Batch && l.w.f < 0) BAIL(8);
   }
-  for (const auto& r : ranges) {
-    if (r.e <= 1) continue;
-    if (covered[r.side] != r.e || lowest[r.side] != r.s) return {};
-  }
-  // every variable of the index is one of these loops
-  for (const auto& kv : idx->coef) {
-    if (kv.second == 0) continue;
-    bool known = false;
-    for (const auto& l : f->loops) known = known || l.name == kv.first;
-    if (!known) return {};
-  }
-  auto find_loop = [&](const std::string& name) -> WLoop* {
-    for (auto& w : loops)
-      if (w.name == name) return &w;
+  if (p.f_bytes == 0 || p.f_bytes >= (size_t{1} << 31)) BAIL(9);
+  auto find_loop = [&](const std::string& name) -> L* {
+    for (auto& l : loops)
+      if (l.w.name == name) return &l;
     return nullptr;
   };
 
-  // ---- patch axes: loops grouped by their stride in the source ----------------------------------
-  // outermost first within each side
-  std::sort(loops.begin(), loops.end(), [](const WLoop& a, const WLoop& b) {
-    return a.side != b.side ? a.side < b.side : a.ostride > b.ostride;
-  });
+  // ---- patch axes: row and k loops grouped by the magnitude of their stride in the source ---------
   std::map<int64_t, std::vector<size_t>> by_stride;
-  for (size_t i = 0; i < loops.size(); ++i) by_stride[loops[i].sstride].push_back(i);
+  for (size_t i = 0; i < loops.size(); ++i)
+    if (loops[i].w.side == WSide::Row || loops[i].w.side == WSide::K) by_stride[std::llabs(loops[i].w.f)].push_back(i);
   std::set<size_t> paired_rows;
   for (const auto& kv : by_stride) {
     const auto& g = kv.second;
     if (g.size() == 1) continue;
-    if (g.size() != 2) return {};
-    const WLoop &x = loops[g[0]], &y = loops[g[1]];
-    if (!((x.side == kRow && y.side == kK) || (x.side == kK && y.side == kRow))) return {};
-    paired_rows.insert(x.side == kRow ? g[0] : g[1]);
+    if (g.size() != 2) BAIL(10);
+    const L &x = loops[g[0]], &y = loops[g[1]];
+    if (x.w.side == y.w.side) BAIL(11);
+    paired_rows.insert(x.w.side == WSide::Row ? g[0] : g[1]);
   }
-  if (paired_rows.empty()) return {};      // no window: a plain strided operand, handled elsewhere
-
+  if (paired_rows.empty()) BAIL(12);      // no window: a plain strided operand, handled elsewhere
   // rows inside a workgroup: from some row loop inward, at least from the outermost window row loop
-  std::vector<size_t> row_loops, k_loops, batch_loops;
-  for (size_t i = 0; i < loops.size(); ++i)
-    (loops[i].side == kRow ? row_loops : loops[i].side == kK ? k_loops : batch_loops).push_back(i);
   size_t first_needed = row_loops.size();
   for (size_t q = 0; q < row_loops.size(); ++q)
     if (paired_rows.count(row_loops[q])) {
@@ -188,22 +144,22 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
   // the four k of a step run along a k loop whose extent is a multiple of four when there is one
   int sub = -1;
   for (size_t q = 0; q < k_loops.size(); ++q)
-    if (loops[k_loops[q]].extent % 4 == 0 && (sub < 0 || loops[k_loops[q]].sstride > loops[k_loops[static_cast<size_t>(sub)]].sstride))
+    if (loops[k_loops[q]].w.extent % 4 == 0 &&
+        (sub < 0 || std::llabs(loops[k_loops[q]].w.f) > std::llabs(loops[k_loops[static_cast<size_t>(sub)]].w.f)))
       sub = static_cast<int>(q);
   const int64_t kdelta = sub >= 0 ? loops[k_loops[static_cast<size_t>(sub)]].unit : 1;
-  const int64_t ksteps = sub >= 0 ? s.K / 4 : ceil_div(s.K, 4);
-  if (ksteps > 512) return {};
+  const int64_t ksteps = sub >= 0 ? K / 4 : ceil_div(K, 4);
+  if (ksteps > 512) BAIL(13);
   std::vector<int64_t> k0(static_cast<size_t>(ksteps));
   if (sub >= 0) {
     // every combination of the other k digits, times the blocks of four of the sub digit
     std::vector<int64_t> digit(k_loops.size(), 0);
     for (int64_t st = 0; st < ksteps; ++st) {
       int64_t kk = 0;
-      for (size_t q = 0; q < k_loops.size(); ++q)
-        kk += digit[q] * loops[k_loops[q]].unit * (static_cast<int>(q) == sub ? 4 : 1);
+      for (size_t q = 0; q < k_loops.size(); ++q) kk += digit[q] * loops[k_loops[q]].unit * (static_cast<int>(q) == sub ? 4 : 1);
       k0[static_cast<size_t>(st)] = kk;
       for (size_t q = k_loops.size(); q-- > 0;) {
-        const int64_t lim = static_cast<int>(q) == sub ? loops[k_loops[q]].extent / 4 : loops[k_loops[q]].extent;
+        const int64_t lim = static_cast<int>(q) == sub ? loops[k_loops[q]].w.extent / 4 : loops[k_loops[q]].w.extent;
         if (++digit[q] < lim) break;
         digit[q] = 0;
       }
@@ -211,55 +167,58 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
   } else {
     for (int64_t st = 0; st < ksteps; ++st) k0[static_cast<size_t>(st)] = 4 * st;
   }
+  const int64_t kpad = ceil_div(K, 4) * 4;
 
   // ---- choose how many row loops a workgroup takes, and the wave layout -----------------------------
-  const int64_t mblk_all = ceil_div(s.M, 16);
+  const int64_t mblk_all = ceil_div(M, 16);
   Layout lay;
   size_t first_in = row_loops.size();
-  std::vector<PAxis> axes;
-  int64_t NG = 0, patch_elems = 0;
-  // Candidates from the largest group (fewest workgroups) to the smallest: the first that still
-  // gives the chip a workgroup per CU is taken, else the one with the most workgroups.
-  bool enough = false;
-  for (size_t start = 0; start <= first_needed && !enough; ++start) {
-    for (auto& w : loops) {
-      w.in_wg = w.side == kK;
-      w.axis = -1;
+  int64_t NG = 0;
+  auto mark = [&](size_t start, std::vector<PAxis>* ax_out) {
+    for (auto& l : loops) {
+      l.in_wg = l.w.side == WSide::K;
+      l.axis = -1;
     }
-    int64_t ng = 1;
-    for (size_t q = start; q < row_loops.size(); ++q) {
-      loops[row_loops[q]].in_wg = true;
-      ng *= loops[row_loops[q]].extent;
-    }
-    if (ng > 4096) continue;
+    for (size_t q = start; q < row_loops.size(); ++q) loops[row_loops[q]].in_wg = true;
     // axes by source stride, largest first
     std::vector<PAxis> ax;
-    bool ok = true;
-    for (auto it = by_stride.rbegin(); it != by_stride.rend() && ok; ++it) {
+    for (auto it = by_stride.rbegin(); it != by_stride.rend(); ++it) {
       PAxis a;
       a.sstride = it->first;
-      int64_t ext = 1;
+      int64_t ext = 1, shift = 0;
       bool any = false;
       for (size_t i : it->second) {
         if (!loops[i].in_wg) {
-          if (it->second.size() == 2) ok = false;     // a window pair split between workgroups
+          if (it->second.size() == 2) return false;     // a window pair split between workgroups
           continue;
         }
-        ext += loops[i].extent - 1;
+        ext += loops[i].w.extent - 1;
+        if (loops[i].w.f < 0) shift += loops[i].w.extent - 1;
         any = true;
       }
       if (!any) continue;
       a.extent = ext;
+      a.shift = shift;
       a.lo = 0;
       a.hi = ext;
       for (size_t i : it->second)
         if (loops[i].in_wg) loops[i].axis = static_cast<int>(ax.size());
       ax.push_back(a);
     }
-    if (!ok || ax.empty()) continue;
+    *ax_out = ax;
+    return !ax.empty();
+  };
+  // Candidates from the largest group (fewest workgroups) to the smallest: the first that still
+  // gives the chip a workgroup per CU is taken, else the one with the most workgroups.
+  bool enough = false;
+  for (size_t start = 0; start <= first_needed && !enough; ++start) {
+    int64_t ng = 1;
+    for (size_t q = start; q < row_loops.size(); ++q) ng *= loops[row_loops[q]].w.extent;
+    if (ng > 4096) continue;
+    std::vector<PAxis> ax;
+    if (!mark(start, &ax)) continue;
     int64_t elems = 1;
     for (const auto& a : ax) elems *= a.extent;
-    if (elems > 24576) continue;                       // 96 KiB of LDS at most
     // wave layout: M-blocks over the waves first, the N-blocks of the group over what is left
     Layout l;
     l.waves_m = mblk_all >= 4 ? 4 : mblk_all >= 2 ? 2 : 1;
@@ -272,74 +231,74 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
     const int64_t regs = 4LL * l.mb * l.nb + 2LL * (l.mb + l.nb) + 4LL * l.nb;
     if (regs > 400 || l.nb > 64) continue;
     // LDS: the patch and A's rows (K floats and a pad each)
-    if ((elems + 64 + static_cast<int64_t>(l.waves_m) * l.mb * 16 * (ceil_div(s.K, 4) * 4 + 64)) * 4 > 150 * 1024) continue;
+    if ((elems + 64 + static_cast<int64_t>(l.waves_m) * l.mb * 16 * (kpad + 4)) * 4 > 160 * 1024) continue;
     first_in = start;
     lay = l;
-    axes = ax;
     NG = ng;
-    patch_elems = elems;
-    enough = (s.N / ng) * s.batch >= 256;
+    enough = (N / ng) * batch >= 256;
   }
-  if (first_in == row_loops.size() || NG < 4) return {};
-  // restore the choice (the loop above leaves the last candidate's marks when it broke out early)
-  for (auto& w : loops) {
-    w.in_wg = w.side == kK;
-    w.axis = -1;
-  }
-  for (size_t q = first_in; q < row_loops.size(); ++q) loops[row_loops[q]].in_wg = true;
-  {
-    size_t ai = 0;
-    for (auto it = by_stride.rbegin(); it != by_stride.rend(); ++it) {
-      bool any = false;
-      for (size_t i : it->second) any = any || loops[i].in_wg;
-      if (!any) continue;
-      for (size_t i : it->second)
-        if (loops[i].in_wg) loops[i].axis = static_cast<int>(ai);
-      ++ai;
-    }
-  }
+  if (first_in == row_loops.size() || NG < 4) BAIL(14);
+  std::vector<PAxis> axes;
+  if (!mark(first_in, &axes)) BAIL(15);
+  int64_t patch_elems = 1;
+  for (const auto& a : axes) patch_elems *= a.extent;
+  const int64_t groups = N / NG;
+  if (groups > 0x7fffffffLL) BAIL(16);
 
-  // ---- guards: each atom bounds one patch coordinate (or repeats a loop's own extent) ------------
-  for (const auto& a : atoms) {
-    std::vector<WLoop*> vars;
-    for (const auto& kv : a.e.coef) {
-      WLoop* w = find_loop(kv.first);
-      if (!w) {
-        // a loop that runs once: contributes nothing
-        bool once = false;
-        for (const auto& l : f->loops) once = once || (l.name == kv.first && l.extent <= 1);
-        if (!once) return {};
+  // ---- guards: each bounds one patch coordinate (or repeats a loop's own extent) -------------------
+  for (const auto& g : p.guards) {
+    std::vector<std::pair<L*, int64_t>> vars;
+    for (const auto& t : g.terms) {
+      if (t.second == 0) continue;
+      L* l = find_loop(t.first);
+      if (!l) {
+        bool once = false;      // a loop that runs once contributes nothing
+        for (const auto& w : p.loops) once = once || (w.name == t.first && w.extent == 1);
+        if (!once) BAIL(17);
         continue;
       }
-      if (kv.second != 1) return {};
-      vars.push_back(w);
+      vars.push_back({l, t.second});
     }
     if (vars.empty()) {
-      // a constant condition: must hold
-      if (a.ge ? !(0 >= a.bound) : !(0 < a.bound)) return {};
+      if (g.ge ? !(0 >= g.bound) : !(0 < g.bound)) BAIL(18);     // a constant condition must hold
       continue;
     }
-    if (vars.size() == 1 && !vars[0]->in_wg) {
-      // a loop outside the workgroup: only the trivial bound on its own extent is accepted
-      if (a.ge ? a.bound > 0 : a.bound < vars[0]->extent) return {};
-      continue;
-    }
-    if (vars.size() > 2) return {};
-    if (vars.size() == 2 && (vars[0]->axis < 0 || vars[0]->axis != vars[1]->axis)) return {};
-    if (vars[0]->axis < 0) return {};
-    PAxis& ax = axes[static_cast<size_t>(vars[0]->axis)];
-    // a bound on one loop of a pair axis alone cannot be expressed on the pair's coordinate
+    auto trivial = [&]() {
+      // one loop with coefficient +-1: true for every value of the loop?
+      if (vars.size() != 1 || std::llabs(vars[0].second) != 1) return false;
+      const int64_t e = vars[0].first->w.extent;
+      if (vars[0].second == 1) return g.ge ? g.bound <= 0 : g.bound >= e;
+      return g.ge ? g.bound <= -(e - 1) : g.bound >= 1;
+    };
+    const int ax_id = vars[0].first->axis;
+    bool same_axis = ax_id >= 0;
+    for (const auto& v : vars) same_axis = same_axis && v.first->axis == ax_id;
     int members = 0;
-    for (const auto& w : loops) members += w.axis == vars[0]->axis ? 1 : 0;
-    if (static_cast<int>(vars.size()) != members) {
-      if (a.ge ? a.bound > 0 : a.bound < vars[0]->extent) return {};
+    for (const auto& l : loops) members += (ax_id >= 0 && l.axis == ax_id) ? 1 : 0;
+    if (!same_axis || static_cast<int>(vars.size()) != members) {
+      if (!trivial()) BAIL(19);
       continue;
     }
-    if (a.ge) ax.lo = std::max(ax.lo, a.bound);
-    else ax.hi = std::min(ax.hi, a.bound);
+    // coefficients: the signs of the loops' strides, all of them or all negated
+    int sigma = 0;
+    for (const auto& v : vars) {
+      if (std::llabs(v.second) != 1) BAIL(20);
+      const int sg = static_cast<int>(v.second) * (v.first->w.f > 0 ? 1 : -1);
+      if (sigma != 0 && sg != sigma) BAIL(21);
+      sigma = sg;
+    }
+    PAxis& ax = axes[static_cast<size_t>(ax_id)];
+    // sum(sign * digit) = coordinate - shift
+    if (sigma > 0) {
+      if (g.ge) ax.lo = std::max(ax.lo, g.bound + ax.shift);
+      else ax.hi = std::min(ax.hi, g.bound + ax.shift);
+    } else {
+      if (g.ge) ax.hi = std::min(ax.hi, ax.shift - g.bound + 1);      // -(x) >= b  <=>  x <= -b
+      else ax.lo = std::max(ax.lo, ax.shift - g.bound + 1);           // -(x) < b   <=>  x > -b
+    }
   }
   for (const auto& a : axes)
-    if (a.lo >= a.hi) return {};
+    if (a.lo >= a.hi) BAIL(22);
 
   // ---- LDS layout of the patch: dense, outermost axis padded against bank conflicts ----------------
   auto set_strides = [&](int64_t pad) {
@@ -349,55 +308,39 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
       st = axes[i].lds * axes[i].extent;
     }
   };
+  // a loop's share of the patch offset for digit d
+  auto lds_of = [&](const L& l, int64_t d) {
+    const int64_t st = axes[static_cast<size_t>(l.axis)].lds;
+    return (l.w.f > 0 ? d : l.w.extent - 1 - d) * st;
+  };
   auto k_lds = [&](int64_t kk) {
     int64_t o = 0;
-    for (size_t q : k_loops) {
-      const WLoop& w = loops[q];
-      o += ((kk / w.unit) % w.extent) * axes[static_cast<size_t>(w.axis)].lds;
-    }
+    for (size_t q : k_loops) o += lds_of(loops[q], (kk / loops[q].unit) % loops[q].w.extent);
     return o;
   };
   auto row_lds = [&](int64_t n) {
     int64_t o = 0;
-    for (size_t q = first_in; q < row_loops.size(); ++q) {
-      const WLoop& w = loops[row_loops[q]];
-      const int64_t unit_in = w.unit / loops[row_loops.back()].unit;    // unit relative to the group's first row
-      o += ((n / unit_in) % w.extent) * axes[static_cast<size_t>(w.axis)].lds;
-    }
+    for (size_t q = first_in; q < row_loops.size(); ++q)
+      o += lds_of(loops[row_loops[q]], (n / loops[row_loops[q]].unit) % loops[row_loops[q]].w.extent);
     return o;
-  };
-  // the rows of a group are NG consecutive rows of the contraction: the innermost row loop has unit 1
-  if (loops[row_loops.back()].unit != 1) return {};
-  auto conflict_cost = [&]() {
-    int64_t cost = 0;
-    const int64_t steps = std::min<int64_t>(ksteps, 12);
-    const int64_t blocks = std::min<int64_t>(ceil_div(NG, 16), 8);
-    for (int64_t st = 0; st < steps; ++st)
-      for (int64_t nb = 0; nb < blocks; ++nb) {
-        int64_t addr[64];
-        for (int lane = 0; lane < 64; ++lane) {
-          const int64_t n = std::min<int64_t>(nb * 16 + lane % 16, NG - 1);
-          const int64_t kk = std::min<int64_t>(k0[static_cast<size_t>(st)] + (lane / 16) * kdelta, s.K - 1);
-          addr[lane] = row_lds(n) + k_lds(kk);
-        }
-        for (int banks : {32, 64}) {
-          const int group = banks;                          // lanes served together
-          for (int g0 = 0; g0 < 64; g0 += group) {
-            std::map<int64_t, std::set<int64_t>> per_bank;
-            for (int lane = g0; lane < g0 + group; ++lane) per_bank[addr[lane] % banks].insert(addr[lane]);
-            size_t worst = 1;
-            for (const auto& kv : per_bank) worst = std::max(worst, kv.second.size());
-            cost += static_cast<int64_t>(worst) - 1;
-          }
-        }
-      }
-    return cost;
   };
   {
     int64_t best_pad = 0, best_cost = -1;
     for (int64_t pad = 0; pad < 64; ++pad) {
       set_strides(pad);
-      const int64_t c = conflict_cost();
+      int64_t c = 0;
+      const int64_t steps = std::min<int64_t>(ksteps, 12);
+      const int64_t blocks = std::min<int64_t>(ceil_div(NG, 16), 8);
+      for (int64_t st = 0; st < steps; ++st)
+        for (int64_t nb = 0; nb < blocks; ++nb) {
+          int64_t addr[64];
+          for (int lane = 0; lane < 64; ++lane) {
+            const int64_t n = std::min<int64_t>(nb * 16 + lane % 16, NG - 1);
+            const int64_t kk = std::min<int64_t>(k0[static_cast<size_t>(st)] + (lane / 16) * kdelta, K - 1);
+            addr[lane] = row_lds(n) + k_lds(kk);
+          }
+          c += bank_cost(addr);
+        }
       if (best_cost < 0 || c < best_cost) {
         best_cost = c;
         best_pad = pad;
@@ -408,86 +351,87 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
   }
   int64_t patch_floats = 1;
   for (const auto& a : axes) patch_floats += (a.extent - 1) * a.lds;
-  if (patch_floats * 4 > 120 * 1024) return {};
 
   // ---- step tables ---------------------------------------------------------------------------------
   std::vector<std::vector<int64_t>> patterns;
   std::vector<int64_t> koff(static_cast<size_t>(ksteps)), kpat(static_cast<size_t>(ksteps));
+  int64_t min_rel = 0;
   for (int64_t st = 0; st < ksteps; ++st) {
-    const int64_t base = k_lds(std::min<int64_t>(k0[static_cast<size_t>(st)], s.K - 1));
-    std::vector<int64_t> p(4);
-    for (int j = 0; j < 4; ++j) p[static_cast<size_t>(j)] = k_lds(std::min<int64_t>(k0[static_cast<size_t>(st)] + j * kdelta, s.K - 1)) - base;
+    const int64_t base = k_lds(std::min<int64_t>(k0[static_cast<size_t>(st)], K - 1));
+    std::vector<int64_t> pt(4);
+    for (int j = 0; j < 4; ++j) {
+      pt[static_cast<size_t>(j)] = k_lds(std::min<int64_t>(k0[static_cast<size_t>(st)] + j * kdelta, K - 1)) - base;
+      min_rel = std::min(min_rel, pt[static_cast<size_t>(j)]);
+    }
     size_t id = 0;
-    while (id < patterns.size() && patterns[id] != p) ++id;
-    if (id == patterns.size()) patterns.push_back(p);
+    while (id < patterns.size() && patterns[id] != pt) ++id;
+    if (id == patterns.size()) patterns.push_back(pt);
     koff[static_cast<size_t>(st)] = base;
     kpat[static_cast<size_t>(st)] = static_cast<int64_t>(id);
   }
-  if (patterns.size() > 16 || static_cast<int64_t>(patterns.size()) * lay.nb > 160) return {};
+  if (patterns.size() > 16 || static_cast<int64_t>(patterns.size()) * lay.nb > 160) BAIL(23);
+  // (a step's offset is an immediate of the read and must not be negative: what a pattern reaches
+  // back is moved from the steps' offsets into the lanes' bases)
+  if (min_rel < 0) {
+    for (auto& pt : patterns)
+      for (auto& o : pt) o -= min_rel;
+    for (auto& o : koff) o += min_rel;
+    for (const auto& o : koff)
+      if (o < 0) BAIL(24);
+  }
 
-  // ---- A's rows in LDS: row stride padded so that the sixteen rows and four sub-k of a read spread over the banks
-  const int64_t kpad = ceil_div(s.K, 4) * 4;
-  const bool a_vec = s.a_k == 1 && s.K % 4 == 0 && s.a_m % 4 == 0 && s.a_off % 4 == 0 && s.a_b % 4 == 0 &&
-                     (!s.a_msplit || s.a_m2 % 4 == 0);
+  // ---- A's rows in LDS: [m][k], row stride padded so that the sixteen rows and four sub-k of a read spread over the banks
+  // A is fetched in the order of its memory: the loops that index it sorted by their stride there
+  std::vector<const L*> a_order;
+  for (size_t q : m_loops) a_order.push_back(&loops[q]);
+  for (size_t q : k_loops) a_order.push_back(&loops[q]);
+  for (const L* l : a_order)
+    if (l->w.a <= 0) BAIL(25);
+  std::stable_sort(a_order.begin(), a_order.end(), [](const L* x, const L* y) { return x->w.a > y->w.a; });
+  const L* a_fast = a_order.back();
+  bool a_vec = a_fast->w.side == WSide::K && a_fast->w.a == 1 && a_fast->unit == 1 && a_fast->w.extent % 4 == 0 && p.a_c0 % 4 == 0;
+  for (const auto& l : loops)
+    if (&l != a_fast && l.w.a % 4 != 0) a_vec = false;
   int64_t a_lds = kpad;
   {
     int64_t best = -1;
     for (int64_t pad = 0; pad < 64; pad += a_vec ? 4 : 1) {
-      const int64_t ks = kpad + pad;
-      int64_t cost = 0;
-      for (int banks : {32, 64})
-        for (int g0 = 0; g0 < 64; g0 += banks) {
-          std::map<int64_t, std::set<int64_t>> per_bank;
-          for (int lane = g0; lane < g0 + banks; ++lane) {
-            const int64_t addr = (lane % 16) * ks + (lane / 16) * kdelta;
-            per_bank[addr % banks].insert(addr);
-          }
-          size_t worst = 1;
-          for (const auto& kv : per_bank) worst = std::max(worst, kv.second.size());
-          cost += static_cast<int64_t>(worst) - 1;
-        }
+      int64_t addr[64];
+      for (int lane = 0; lane < 64; ++lane) addr[lane] = (lane % 16) * (kpad + pad) + (lane / 16) * kdelta;
+      const int64_t cost = bank_cost(addr);
       if (best < 0 || cost < best) {
         best = cost;
-        a_lds = ks;
+        a_lds = kpad + pad;
       }
       if (cost == 0) break;
     }
   }
   const int64_t mrows = static_cast<int64_t>(lay.waves_m) * lay.mb * 16;
-  if ((patch_floats + mrows * a_lds) * 4 > 158 * 1024) return {};
-  // the per-lane base (row + pattern offset) plus a step's offset stays inside the patch by construction
-
-  // ---- groups: the row loops outside the workgroup, and the batch loops -----------------------------
-  int64_t groups = 1;
-  for (size_t q = 0; q < first_in; ++q) groups *= loops[row_loops[q]].extent;
-  if (groups * NG != s.N || groups > 0x7fffffffLL) return {};
+  if ((patch_floats + mrows * a_lds) * 4 > 160 * 1024) BAIL(26);
+  const bool a_zero = mrows != M || kpad != K;            // padding rows / columns of A's tile must read as zero
+  const int64_t a_elems = a_vec ? M * K / 4 : M * K;
 
   // ---- source ---------------------------------------------------------------------------------------
   std::ostringstream os;
   LaunchSpec ls;
-  ls.entry = "ehk_" + k.name;
-  ls.kernels = {k.name};
+  ls.entry = p.entry;
+  ls.kernels = p.kernels;
   os << "// generated for gfx950 by eclat backend-hip: MFMA contraction with a window operand staged in LDS\n";
   os << "#define EW_ENTRY " << ls.entry << "\n";
-  os << "#define EW_M " << s.M << "\n#define EW_MW " << s.M << "\n#define EW_NG " << NG << "\n#define EW_GROUPS " << groups
-     << "\n#define EW_K " << s.K << "\n";
+  os << "#define EW_M " << M << "\n#define EW_NG " << NG << "\n#define EW_GROUPS " << groups << "\n#define EW_K " << K << "\n";
   os << "#define EW_WAVES_M " << lay.waves_m << "\n#define EW_WAVES_N " << lay.waves_n << "\n#define EW_MB " << lay.mb
      << "\n#define EW_NB " << lay.nb << "\n";
   os << "#define EW_KSTEPS " << ksteps << "\n#define EW_NPAT " << patterns.size() << "\n#define EW_KDELTA " << kdelta << "\n";
   os << "#define EW_PATCH_FLOATS " << patch_floats << "\n#define EW_PATCH_ELEMS " << patch_elems << "\n";
-  os << "#define EW_A_OFF " << s.a_off << "LL\n#define EW_A_BS " << s.a_b << "LL\n#define EW_A_SM " << s.a_m
-     << "LL\n#define EW_A_SK " << s.a_k << "LL\n#define EW_A_MSPLIT " << s.a_msplit << "LL\n#define EW_A_SM2 " << s.a_m2 << "LL\n";
-  os << "#define EH_C_OFF " << s.c_off << "LL\n#define EH_C_BS " << s.c_b << "LL\n#define EH_C_SM " << s.c_m
-     << "LL\n#define EH_C_SN " << s.c_n << "LL\n";
-  os << "#define EH_C_MSPLIT " << s.c_msplit << "LL\n#define EH_C_SM2 " << s.c_m2 << "LL\n#define EH_C_NSPLIT " << s.c_nsplit
-     << "LL\n#define EH_C_SN2 " << s.c_n2 << "LL\n";
-  os << "#define EW_A_VEC " << (a_vec ? 1 : 0) << "\n#define EW_KPAD " << kpad << "\n#define EW_A_LDS " << a_lds << "\n";
-  os << "#define EW_SRC_BYTES " << f->ranged_bytes << "u\n";
+  os << "#define EW_A_VEC " << (a_vec ? 1 : 0) << "\n#define EW_A_ELEMS " << a_elems << "\n#define EW_A_ZERO " << (a_zero ? 1 : 0)
+     << "\n#define EW_KPAD " << kpad << "\n#define EW_A_LDS " << a_lds << "\n";
+  os << "#define EW_SRC_BYTES " << p.f_bytes << "u\n";
   os << "#define EW_MIX " << (opt.gemm_mix ? 1 : 0) << "\n";
   if (epilogue) {
     os << "#define EH_EPILOGUE 1\n#define EH_EPI_PARAMS " << epilogue->params << "\n#define EH_EPI_ARGS " << epilogue->args << "\n";
     if (!epilogue->store_c) os << "#define EH_NO_C 1\n";
     os << epilogue->function;
+    if (!epilogue->split_functions.empty()) os << "#define EH_EPILOGUE_SPLIT " << epilogue->n_loads << "\n" << epilogue->split_functions;
   }
   auto table = [&](const char* name, const std::vector<int64_t>& vals) {
     os << "constexpr int " << name << "[" << vals.size() << "] = {";
@@ -495,7 +439,7 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
     os << "};\n";
   };
   os << "// step s multiplies k = ew_k0[s] + j * EW_KDELTA (j = 0..3); in the patch those sit at\n"
-        "// ew_koff[s] + ew_pat[ew_kpat[s]][j] beyond the row's base\n";
+        "// ew_koff[s] + ew_pat_lane(ew_kpat[s], j) beyond the row's base\n";
   os << "namespace {\n";
   table("ew_k0", k0);
   table("ew_koff", koff);
@@ -503,19 +447,21 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
   os << "}\n";
   // sub-step j of a step with pattern p: offset by arithmetic on the bits of j over literals
   os << "__device__ __forceinline__ int ew_pat_lane(int p, int j) {\n  const int b0 = j & 1, b1 = j >> 1;\n  (void)b0; (void)b1;\n";
-  for (size_t p = 0; p < patterns.size(); ++p) {
-    const auto& o = patterns[p];
-    os << "  if (p == " << p << ") return " << o[0] << " + b0 * " << (o[1] - o[0]) << " + b1 * " << (o[2] - o[0]) << " + (b0 & b1) * "
+  for (size_t q = 0; q < patterns.size(); ++q) {
+    const auto& o = patterns[q];
+    os << "  if (p == " << q << ") return " << o[0] << " + b0 * " << (o[1] - o[0]) << " + b1 * " << (o[2] - o[0]) << " + (b0 & b1) * "
        << (o[3] - o[2] - o[1] + o[0]) << ";\n";
   }
   os << "  return 0;\n}\n";
   // row n of the group -> LDS offset
-  os << "// what the rows of kernel " << f->kernel << " read of " << f->src << ", as a patch in LDS: axes";
+  os << "// " << p.what << ": what a group of " << NG << " rows reads of " << p.f_buf << ", as a patch in LDS: axes";
   for (const auto& a : axes) os << " [" << a.extent << " x stride " << a.sstride << ", valid " << a.lo << ".." << a.hi << ", lds " << a.lds << "]";
   os << "\n__device__ __forceinline__ int ew_row_lds(int n) {\n  const unsigned u = (unsigned)n;\n  (void)u;\n  return 0";
   for (size_t q = first_in; q < row_loops.size(); ++q) {
-    const WLoop& w = loops[row_loops[q]];
-    os << " + (int)((u / " << w.unit << "u) % " << w.extent << "u) * " << axes[static_cast<size_t>(w.axis)].lds;
+    const L& l = loops[row_loops[q]];
+    const int64_t st = axes[static_cast<size_t>(l.axis)].lds;
+    if (l.w.f > 0) os << " + (int)((u / " << l.unit << "u) % " << l.w.extent << "u) * " << st;
+    else os << " + (" << (l.w.extent - 1) << " - (int)((u / " << l.unit << "u) % " << l.w.extent << "u)) * " << st;
   }
   os << ";\n}\n";
   // patch element e of group g, batch bz -> LDS offset, byte offset in the source (out of range where padding)
@@ -539,44 +485,76 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
     if (axes[i].lo > 0) os << " & (p" << i << " >= " << axes[i].lo << ")";
     if (axes[i].hi < axes[i].extent) os << " & (p" << i << " < " << axes[i].hi << ")";
   }
-  os << ";\n  long long src = " << idx->c << "LL";
-  for (size_t i = 0; i < axes.size(); ++i) os << " + (long long)p" << i << " * " << axes[i].sstride << "LL";
+  os << ";\n  long long src = " << p.f_c0 << "LL";
+  for (size_t i = 0; i < axes.size(); ++i) os << " + (long long)(p" << i << " - " << axes[i].shift << ") * " << axes[i].sstride << "LL";
   {
     // digits of the group over the row loops outside the workgroup, of the batch over the batch loops
     int64_t radix = 1;
     for (size_t q = first_in; q-- > 0;) {
-      const WLoop& w = loops[row_loops[q]];
-      os << " + (long long)((ug / " << radix << "u) % " << w.extent << "u) * " << w.sstride << "LL";
-      radix *= w.extent;
+      const L& l = loops[row_loops[q]];
+      if (l.w.f < 0) BAIL(27);
+      os << " + (long long)((ug / " << radix << "u) % " << l.w.extent << "u) * " << l.w.f << "LL";
+      radix *= l.w.extent;
     }
-    for (size_t q : batch_loops) {
-      const WLoop& w = loops[q];
-      os << " + (long long)((ub / " << w.unit << "u) % " << w.extent << "u) * " << w.sstride << "LL";
-    }
+    for (size_t q : batch_loops)
+      os << " + (long long)((ub / " << loops[q].unit << "u) % " << loops[q].w.extent << "u) * " << loops[q].w.f << "LL";
   }
   os << ";\n  *src_byte = ok ? (unsigned)(src << 2) : 0x80000000u;\n}\n";
+  // A: element e (in the order of A's memory; four along k at once where they can be read as one vector)
+  {
+    os << "// element (m, k) of A for e = 0.." << a_elems << ", walked in the order of A's memory: its offset there and in the tile\n";
+    os << "__device__ __forceinline__ void ew_a_elem(int e, long long bz, int* lds, long long* off) {\n";
+    os << "  const unsigned u = (unsigned)e, ub = (unsigned)bz;\n  (void)u; (void)ub;\n  long long o = " << p.a_c0 << "LL;\n  int m = 0, k = 0;\n";
+    int64_t radix = 1;
+    for (size_t i = a_order.size(); i-- > 0;) {
+      const L* l = a_order[i];
+      const bool quad = a_vec && l == a_fast;
+      const int64_t ext = quad ? l->w.extent / 4 : l->w.extent;
+      os << "  {\n    const int d = (int)((u / " << radix << "u) % " << ext << "u)" << (quad ? " * 4" : "") << ";\n";
+      os << "    o += (long long)d * " << l->w.a << "LL;\n";
+      os << "    " << (l->w.side == WSide::M ? "m" : "k") << " += d * " << l->unit << ";\n  }\n";
+      radix *= ext;
+    }
+    for (size_t q : batch_loops)
+      if (loops[q].w.a) os << "  o += (long long)((ub / " << loops[q].unit << "u) % " << loops[q].w.extent << "u) * " << loops[q].w.a << "LL;\n";
+    os << "  *lds = m * " << a_lds << " + k;\n  *off = o;\n}\n";
+  }
+  // C: offsets of row m, of row n of F (over all groups), of batch bz
+  {
+    std::vector<const L*> ms, ns, bs;
+    for (size_t q : m_loops) ms.push_back(&loops[q]);
+    for (size_t q : row_loops) ns.push_back(&loops[q]);
+    for (size_t q : batch_loops) bs.push_back(&loops[q]);
+    auto cs = [](const L& l) { return l.w.c; };
+    os << "__device__ __forceinline__ long long ew_c_m(int m) {\n  const unsigned u = (unsigned)m;\n  (void)u;\n  return "
+       << digits_sum(ms, "u", cs) << ";\n}\n";
+    os << "__device__ __forceinline__ long long ew_c_n(long long n) {\n  const unsigned u = (unsigned)n;\n  (void)u;\n  return "
+       << digits_sum(ns, "u", cs) << ";\n}\n";
+    os << "__device__ __forceinline__ long long ew_c_b(long long bz) {\n  const unsigned u = (unsigned)bz;\n  (void)u;\n  return " << p.c_c0
+       << "LL + " << digits_sum(bs, "u", cs) << ";\n}\n";
+  }
   os << kWindowSource;
   ls.source = os.str();
-  ls.schedule = "mfma16x16x4(window,group=" + std::to_string(NG) + ",M=" + std::to_string(s.M) + ",K=" + std::to_string(s.K) +
+  ls.schedule = "mfma16x16x4(window,group=" + std::to_string(NG) + ",M=" + std::to_string(M) + ",K=" + std::to_string(K) +
                 ",waves=" + std::to_string(lay.waves_m) + "x" + std::to_string(lay.waves_n) + ",blocks=" + std::to_string(lay.mb) +
                 "x" + std::to_string(lay.nb) + ",steps=" + std::to_string(ksteps) + ",patterns=" + std::to_string(patterns.size()) +
-                ",lds=" + std::to_string((patch_floats + mrows * a_lds) * 4) + "B" + (fa ? ",C^T" : "") +
+                ",lds=" + std::to_string((patch_floats + mrows * a_lds) * 4) + "B" + p.tag +
                 (epilogue ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(groups);
   ls.grid[1] = 1;
-  ls.grid[2] = static_cast<unsigned>(s.batch);
-  ls.block[0] = static_cast<unsigned>(lay.waves_m * lay.waves_n * 64);
-  auto reach = [](int64_t rows, int64_t sr, int64_t split, int64_t sr2) {
-    if (!split) return (rows - 1) * sr;
-    return (rows / split - 1) * sr2 + (split - 1) * sr;
+  ls.grid[2] = static_cast<unsigned>(batch);
+  ls.block[0] = 256;
+  // smallest buffers: the furthest element each address can reach
+  auto reach = [&](int64_t c0, int64_t WLoop::*stride) {
+    int64_t r = c0;
+    for (const auto& l : loops) r += (l.w.extent - 1) * std::max<int64_t>(0, l.w.*stride);
+    return static_cast<size_t>(r + 1);
   };
-  const size_t c_elems = static_cast<size_t>(s.c_off + reach(s.M, s.c_m, s.c_msplit, s.c_m2) + reach(s.N, s.c_n, s.c_nsplit, s.c_n2) +
-                                             (s.batch - 1) * s.c_b + 1);
-  ls.arg_bufs = {s.a_buf, f->src};
-  ls.arg_min_bytes = {4 * static_cast<size_t>(s.a_off + reach(s.M, s.a_m, s.a_msplit, s.a_m2) + (s.K - 1) * s.a_k + (s.batch - 1) * s.a_b + 1), 0};
+  ls.arg_bufs = {p.a_buf, p.f_buf};
+  ls.arg_min_bytes = {4 * reach(p.a_c0, &WLoop::a), 0};
   if (!(epilogue && !epilogue->store_c)) {
-    ls.arg_bufs.push_back(s.c_buf);
-    ls.arg_min_bytes.push_back(4 * c_elems);
+    ls.arg_bufs.push_back(p.c_buf);
+    ls.arg_min_bytes.push_back(4 * reach(p.c_c0, &WLoop::c));
   }
   if (epilogue) {
     for (size_t i = 0; i < epilogue->bufs.size(); ++i) {
@@ -585,15 +563,293 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
     }
     for (const auto& n : epilogue->kernels) ls.kernels.push_back(n);
   }
-  ls.flops = 2.0 * static_cast<double>(s.M) * static_cast<double>(s.N) * static_cast<double>(s.K) * static_cast<double>(s.batch);
+  ls.flops = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) * static_cast<double>(batch);
   {
-    const double nb = static_cast<double>(s.batch);
-    const double a_bytes = 4.0 * static_cast<double>(s.M) * s.K * (s.a_b == 0 ? 1.0 : nb);
-    const double f_bytes = f->src_bytes > 0 ? f->src_bytes : 4.0 * static_cast<double>(s.K) * s.N * nb;
-    const double c_bytes = 4.0 * nb * static_cast<double>(s.M) * s.N;
+    bool a_moves = false;
+    for (size_t q : batch_loops) a_moves = a_moves || loops[q].w.a != 0;
+    const double nb = static_cast<double>(batch);
+    const double a_bytes = 4.0 * static_cast<double>(M) * K * (a_moves ? nb : 1.0);
+    const double f_bytes = p.f_algo_bytes > 0 ? p.f_algo_bytes : 4.0 * static_cast<double>(K) * N * nb;
+    const double c_bytes = 4.0 * nb * static_cast<double>(M) * N;
     ls.algo_bytes = a_bytes + f_bytes + (epilogue && !epilogue->store_c ? 0.0 : c_bytes) + (epilogue ? epilogue->bytes : 0.0);
   }
   return {ls};
+}
+
+// ---------------------------------------------------------------------------------------------------
+// from a matched contraction and its folded operand
+// ---------------------------------------------------------------------------------------------------
+
+namespace {
+
+// e >= bound or e < bound over loop names, from one comparison of the gather's guard
+bool collect_guards(const Node& c, std::vector<WGuard>* out) {
+  if (c.op == Op::And || c.op == Op::BitAnd) return collect_guards(*c.args[0], out) && collect_guards(*c.args[1], out);
+  const Node* lt = &c;
+  bool neg = false;
+  if (c.op == Op::Not && c.args[0]->op == Op::Lt) {
+    lt = c.args[0].get();
+    neg = true;
+  }
+  if (lt->op != Op::Lt) return false;
+  auto l = affine_of(*lt->args[0]);
+  auto r = affine_of(*lt->args[1]);
+  if (!l || !r) return false;
+  // l < r  <=>  (l - r without constants) < r.c - l.c
+  Affine e = *l;
+  for (const auto& kv : r->coef) e.coef[kv.first] -= kv.second;
+  WGuard g;
+  g.bound = r->c - l->c;
+  g.ge = neg;
+  for (const auto& kv : e.coef)
+    if (kv.second != 0) g.terms.push_back({kv.first, kv.second});
+  out->push_back(g);
+  return true;
+}
+
+// stride of a loop (weight `unit` in an axis' flat index v) when v sits at
+// split ? (v / split) * s2 + (v % split) * s1 : v * s1; false when the loop straddles the split
+bool axis_stride(int64_t unit, int64_t extent, int64_t s1, int64_t split, int64_t s2, int64_t* out) {
+  if (!split) {
+    *out = unit * s1;
+    return true;
+  }
+  if (unit >= split) {
+    if (unit % split) return false;
+    *out = (unit / split) * s2;
+    return true;
+  }
+  if (unit * extent > split) return false;
+  *out = unit * s1;
+  return true;
+}
+
+}  // namespace
+
+std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShape& s_in, const FoldedOperand* fa,
+                                             const FoldedOperand* fb, const GenOptions& opt, const EpilogueSpec* epilogue) {
+  if ((fa != nullptr) == (fb != nullptr)) return {};
+  // the folded operand takes the column side: C^T = F^T A^T when it came as A
+  GemmShape s = s_in;
+  const FoldedOperand* f = fb;
+  if (fa) {
+    f = fa;
+    s.M = s_in.N; s.N = s_in.M;
+    s.a_buf = s_in.b_buf; s.b_buf = s_in.a_buf;
+    s.a_m = s_in.b_n; s.a_k = s_in.b_k; s.a_off = s_in.b_off; s.a_b = s_in.b_b;
+    s.a_msplit = s_in.b_nsplit; s.a_m2 = s_in.b_n2;
+    s.b_n = s_in.a_m; s.b_k = s_in.a_k; s.b_off = s_in.a_off; s.b_b = s_in.a_b;
+    s.b_nsplit = s_in.a_msplit; s.b_n2 = s_in.a_m2;
+    s.c_m = s_in.c_n; s.c_n = s_in.c_m;
+    s.c_msplit = s_in.c_nsplit; s.c_m2 = s_in.c_n2; s.c_nsplit = s_in.c_msplit; s.c_n2 = s_in.c_m2;
+  }
+  if (!f->value || f->ranged_bytes == 0 || !f->small || !f->prelude.empty()) return {};
+  if (s.b_off != 0 || s.b_nsplit != 0 || s.a_off < 0 || s.a_k <= 0 || s.a_m <= 0 || s.c_off < 0) return {};
+
+  WindowProblem p;
+  p.entry = "ehk_" + k.name;
+  p.kernels = {k.name};
+  p.what = "rows of kernel " + f->kernel;
+  p.a_buf = s.a_buf;
+  p.f_buf = f->src;
+  p.c_buf = s.c_buf;
+  p.f_bytes = f->ranged_bytes;
+  p.f_algo_bytes = f->src_bytes;
+  p.a_c0 = s.a_off;
+  p.c_c0 = s.c_off;
+  p.tag = fa ? ",C^T" : "";
+
+  // the gather: load index and guard
+  const Node* v = f->value.get();
+  if (v->op == Op::Select) {
+    if (v->args[2]->op != Op::Const || v->args[2]->fval != 0.0 || !collect_guards(*v->args[0], &p.guards)) return {};
+    v = v->args[1].get();
+  }
+  if (v->op != Op::Load || v->args[0]->op != Op::Var || v->args[0]->name != f->src) return {};
+  auto idx = affine_of(*v->args[1]);
+  if (!idx) return {};
+  p.f_c0 = idx->c;
+  for (const auto& kv : idx->coef) {
+    if (kv.second == 0) continue;
+    bool known = false;
+    for (const auto& l : f->loops) known = known || l.name == kv.first;
+    if (!known) return {};
+  }
+
+  // the gather's loops by the axis of the contraction their stride in its output falls into
+  struct AxisRange { int64_t s, e; WSide side; };
+  const AxisRange ranges[3] = {{s.b_b, s.batch, WSide::Batch}, {s.b_n, s.N, WSide::Row}, {s.b_k, s.K, WSide::K}};
+  std::map<WSide, int64_t> covered, lowest;
+  std::vector<std::pair<int64_t, WLoop>> placed;      // by stride in the gather's output, for ordering
+  for (const auto& l : f->loops) {
+    if (l.extent <= 1) {
+      WLoop once;               // a loop that runs once: known by name (guards may mention it), otherwise ignored
+      once.name = l.name;
+      once.extent = 1;
+      p.loops.push_back(once);
+      continue;
+    }
+    WLoop w;
+    w.name = l.name;
+    w.extent = l.extent;
+    w.f = idx->of(l.name);
+    bool ok = false;
+    for (const auto& r : ranges) {
+      if (r.e <= 1 || r.s <= 0) continue;
+      if (l.stride < r.s || l.stride >= r.s * r.e) continue;
+      if (l.stride * l.extent > r.s * r.e || l.stride % r.s != 0) return {};
+      w.side = r.side;
+      const int64_t unit = l.stride / r.s;
+      if (r.side == WSide::K) w.a = unit * s.a_k;
+      if (r.side == WSide::Batch) {
+        w.a = unit * s.a_b;
+        w.c = unit * s.c_b;
+      }
+      if (r.side == WSide::Row && !axis_stride(unit, l.extent, s.c_n, s.c_nsplit, s.c_n2, &w.c)) return {};
+      covered[r.side] = (covered.count(r.side) ? covered[r.side] : 1) * l.extent;
+      lowest[r.side] = lowest.count(r.side) ? std::min(lowest[r.side], l.stride) : l.stride;
+      ok = true;
+      break;
+    }
+    if (!ok) return {};
+    placed.push_back({l.stride, w});
+  }
+  for (const auto& r : ranges) {
+    if (r.e <= 1) continue;
+    if (covered[r.side] != r.e || lowest[r.side] != r.s) return {};
+  }
+  std::stable_sort(placed.begin(), placed.end(), [](const auto& x, const auto& y) { return x.first > y.first; });
+  for (const auto& pl : placed) p.loops.push_back(pl.second);
+  // A's and C's rows
+  if (s.a_msplit) {
+    if (s.M % s.a_msplit || (s.c_msplit && s.c_msplit != s.a_msplit)) return {};
+    WLoop o, in;
+    o.name = "eh_m_outer"; o.side = WSide::M; o.extent = s.M / s.a_msplit; o.a = s.a_m2;
+    in.name = "eh_m_inner"; in.side = WSide::M; in.extent = s.a_msplit; in.a = s.a_m;
+    if (!axis_stride(s.a_msplit, o.extent, s.c_m, s.c_msplit, s.c_m2, &o.c) || !axis_stride(1, in.extent, s.c_m, s.c_msplit, s.c_m2, &in.c))
+      return {};
+    p.loops.push_back(o);
+    p.loops.push_back(in);
+  } else if (s.c_msplit) {
+    if (s.M % s.c_msplit) return {};
+    WLoop o, in;
+    o.name = "eh_m_outer"; o.side = WSide::M; o.extent = s.M / s.c_msplit; o.a = s.a_m * s.c_msplit; o.c = s.c_m2;
+    in.name = "eh_m_inner"; in.side = WSide::M; in.extent = s.c_msplit; in.a = s.a_m; in.c = s.c_m;
+    p.loops.push_back(o);
+    p.loops.push_back(in);
+  } else {
+    WLoop m;
+    m.name = "eh_m"; m.side = WSide::M; m.extent = s.M; m.a = s.a_m; m.c = s.c_m;
+    p.loops.push_back(m);
+  }
+  return emit_window(p, opt, epilogue);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// from a kernel written as a window contraction
+// ---------------------------------------------------------------------------------------------------
+
+std::optional<WindowProblem> match_window_kernel(const Node& kernel, const std::map<std::string, size_t>& buffer_elems) {
+  if (kernel.op != Op::Kernel || kernel.args.size() != 1) return std::nullopt;
+  for (const auto& pr : kernel.params)
+    if (pr.kind != VarKind::Normal || !pr.dtype.is_ptr()) return std::nullopt;
+  struct Lp { std::string var; int64_t extent; };
+  auto range_of = [](const Node& n, Lp* out) {
+    if (n.op != Op::Range || n.args[0]->op != Op::Const || n.args[0]->ival != 0 || n.args[1]->op != Op::Const ||
+        n.args[1]->ival != 1 || n.args[2]->op != Op::Const || n.args[2]->ival < 1)
+      return false;
+    *out = {n.name, n.args[2]->ival};
+    return true;
+  };
+  auto unwrap = [](const Node* b) {
+    while (b->op == Op::Block && b->decls.empty() && b->args.size() == 1) b = b->args[0].get();
+    return b;
+  };
+  std::vector<Lp> outer, red;
+  const Node* cur = unwrap(kernel.args[0].get());
+  Lp lp;
+  while (range_of(*cur, &lp)) {
+    outer.push_back(lp);
+    cur = unwrap(cur->args[3].get());
+  }
+  // block (decls acc): acc = 0; <reduce loops>; store
+  if (cur->op != Op::Block || cur->decls.size() != 1 || cur->args.size() != 3) return std::nullopt;
+  const std::string acc = cur->decls[0].first;
+  if (cur->decls[0].second.ty != Ty::F32) return std::nullopt;
+  const Node &init = *cur->args[0], &store = *cur->args[2];
+  if (init.op != Op::Assign || init.name != acc || init.args[0]->op != Op::Const || init.args[0]->fval != 0.0) return std::nullopt;
+  if (store.op != Op::Store || store.args[0]->op != Op::Var || store.args[2]->op != Op::Var || store.args[2]->name != acc)
+    return std::nullopt;
+  const Node* r = unwrap(cur->args[1].get());
+  while (range_of(*r, &lp)) {
+    red.push_back(lp);
+    r = unwrap(r->args[3].get());
+  }
+  if (red.size() < 2 || r->op != Op::Assign || r->name != acc) return std::nullopt;      // (a single reduce loop is a NestKernel)
+  ReduceKind kind = ReduceKind::None;
+  NodePtr value;
+  if (!match_combine(*r->args[0], acc, &kind, &value) || kind != ReduceKind::Sum || value->op != Op::Mul) return std::nullopt;
+  WindowProblem p;
+  const Node *fx = value->args[0].get(), *ax = value->args[1].get();
+  auto gathered = [&](const Node* x, std::vector<WGuard>* gs) -> const Node* {
+    if (x->op == Op::Select) {
+      if (x->args[2]->op != Op::Const || x->args[2]->fval != 0.0 || !collect_guards(*x->args[0], gs)) return nullptr;
+      x = x->args[1].get();
+    }
+    return x->op == Op::Load && x->args[0]->op == Op::Var && x->dtype.ty == Ty::F32 && x->count == 1 ? x : nullptr;
+  };
+  if (fx->op != Op::Select && ax->op == Op::Select) std::swap(fx, ax);
+  const Node* fl = gathered(fx, &p.guards);
+  std::vector<WGuard> none;
+  const Node* al = gathered(ax, &none);
+  if (!fl || !al || !none.empty() || ax->op == Op::Select) return std::nullopt;
+  auto fi = affine_of(*fl->args[1]), ai = affine_of(*al->args[1]), ci = affine_of(*store.args[1]);
+  if (!fi || !ai || !ci) return std::nullopt;
+  p.f_buf = fl->args[0]->name;
+  p.a_buf = al->args[0]->name;
+  p.c_buf = store.args[0]->name;
+  if (p.f_buf == p.c_buf || p.a_buf == p.c_buf) return std::nullopt;
+  p.f_c0 = fi->c;
+  p.a_c0 = ai->c;
+  p.c_c0 = ci->c;
+  if (p.a_c0 < 0 || p.c_c0 < 0) return std::nullopt;
+  std::set<std::string> names;
+  for (const auto& l : outer) {
+    WLoop w;
+    w.name = l.var;
+    w.extent = l.extent;
+    w.f = fi->of(l.var);
+    w.a = ai->of(l.var);
+    w.c = ci->of(l.var);
+    if (w.extent > 1 && w.c <= 0) return std::nullopt;
+    w.side = w.f != 0 && w.a != 0 ? WSide::Batch : w.f != 0 ? WSide::Row : WSide::M;
+    if (w.extent > 1 && w.f == 0 && w.a == 0) return std::nullopt;
+    p.loops.push_back(w);
+    names.insert(l.var);
+  }
+  for (const auto& l : red) {
+    WLoop w;
+    w.name = l.var;
+    w.extent = l.extent;
+    w.f = fi->of(l.var);
+    w.a = ai->of(l.var);
+    w.side = WSide::K;
+    if (ci->of(l.var) != 0) return std::nullopt;
+    if (w.extent > 1 && (w.f == 0 || w.a <= 0)) return std::nullopt;
+    p.loops.push_back(w);
+    names.insert(l.var);
+  }
+  for (const Affine* a : {&*fi, &*ai, &*ci})
+    for (const auto& kv : a->coef)
+      if (kv.second != 0 && !names.count(kv.first)) return std::nullopt;
+  auto it = buffer_elems.find(p.f_buf);
+  if (it == buffer_elems.end() || it->second * 4 >= (size_t{1} << 31)) return std::nullopt;
+  p.f_bytes = it->second * 4;
+  p.f_algo_bytes = static_cast<double>(p.f_bytes);
+  p.entry = "ehk_" + kernel.name;
+  p.kernels = {kernel.name};
+  p.what = "the guarded operand of kernel " + kernel.name;
+  return p;
 }
 
 }  // namespace eh
