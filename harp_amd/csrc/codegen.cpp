@@ -10,6 +10,7 @@
 #include <sstream>
 
 #include "gemm.hpp"
+#include "window.hpp"
 #include "normalize.hpp"
 
 namespace eh {
@@ -2954,6 +2955,44 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
   }
 
+  // A contraction whose result only a run of kernels adding up shifted reads of it sees (the
+  // input gradient of a convolution) is one window contraction with those kernels.
+  std::map<size_t, ScatteredWindow> scattered;
+  std::set<std::string> partly_written;      // kernels whose output is written only where it is read
+  if (opt.gemm && opt.gemm_window && opt.fuse && opt.reindex && have_table && opt.gemm_bm == 0 && opt.gemm_split_k <= 1) {
+    ProgramView pv;
+    pv.nests = &nests;
+    pv.readers = &readers;
+    pv.elems = &elems;
+    pv.role_of = role_of;
+    pv.folded_gather = [&](const std::string& buf) -> const NestKernel* {
+      for (size_t q : folded_kernels)
+        if (nests[q] && nests[q]->out_buf == buf) return &*nests[q];
+      return nullptr;
+    };
+    pv.taken = [&](size_t q) {
+      if (folded_kernels.count(q) || absorbed.count(q) || windows.count(q)) return true;
+      for (const auto& w : windows)
+        if (std::find(w.second.begin(), w.second.end(), q) != w.second.end()) return true;
+      return false;
+    };
+    for (size_t q = 0; q + 1 < kernels.size(); ++q) {
+      if (!nests[q] || absorbed_name.count(q) || !gemm_shaped(*nests[q], opt)) continue;
+      const Node& v = *nests[q]->value;
+      bool plain = v.op == Op::Mul;
+      for (size_t o = 0; plain && o < 2; ++o)
+        plain = v.args[o]->op == Op::Load && v.args[o]->args[0]->op == Op::Var &&
+                (!folded.count(v.args[o]->args[0]->name) || folded.at(v.args[o]->args[0]->name).prelude.empty());
+      if (!plain) continue;
+      auto sw = try_emit_scattered_window(q, pv, opt);
+      if (!sw) continue;
+      for (size_t c = q + 1; c < sw->next; ++c) absorbed.insert(c);
+      for (const auto& b : sw->elided) plan.elided.insert(b);
+      if (sw->partial) partly_written.insert(nests[sw->next - 1]->name);
+      scattered[q] = std::move(*sw);
+    }
+  }
+
   // Elementwise kernels that follow kernel i (a reduce with a dense output of `total` elements)
   // over the same dense index space and feed on its result: the function that applies them to
   // one element while it is still in a register.  `k0r`: k0 with its output laid out as a
@@ -3222,6 +3261,11 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       ++i;
       continue;
     }
+    if (auto sw = scattered.find(i); sw != scattered.end()) {
+      for (auto& ls : sw->second.launches) plan.launches.push_back(std::move(ls));
+      i = sw->second.next;
+      continue;
+    }
     if (auto w = windows.find(i); w != windows.end()) {
       std::vector<const NestKernel*> chain;
       for (size_t q : w->second) chain.push_back(&*nests[q]);
@@ -3402,7 +3446,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     std::map<std::string, std::pair<std::string, size_t>> dense_out;     // kernel -> (buffer, bytes)
     for (const auto& nk : nests) {
       int64_t numel = 0;
-      if (nk && dense_strides(*nk, &numel))
+      if (nk && !partly_written.count(nk->name) && dense_strides(*nk, &numel))
         dense_out[nk->name] = {nk->out_buf, static_cast<size_t>(numel) * nk->out_dtype.itemsize()};
     }
     for (auto& ls : plan.launches) {

@@ -244,6 +244,8 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   for (const auto& a : axes) patch_elems *= a.extent;
   const int64_t groups = N / NG;
   if (groups > 0x7fffffffLL) BAIL(16);
+  // (a handful of workgroups for a large product leaves most of the chip idle: the tiled schedule then)
+  if (groups * batch < 16 && static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) * static_cast<double>(batch) > 3.0e7) BAIL(28);
 
   // ---- guards: each bounds one patch coordinate (or repeats a loop's own extent) -------------------
   for (const auto& g : p.guards) {
@@ -300,13 +302,46 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   for (const auto& a : axes)
     if (a.lo >= a.hi) BAIL(22);
 
-  // ---- LDS layout of the patch: dense, outermost axis padded against bank conflicts ----------------
-  auto set_strides = [&](int64_t pad) {
+  // ---- A's rows in LDS: [m][k], row stride padded so that the sixteen rows and four sub-k of a read spread over the banks
+  // A is fetched in the order of its memory: the loops that index it sorted by their stride there
+  std::vector<const L*> a_order;
+  for (size_t q : m_loops) a_order.push_back(&loops[q]);
+  for (size_t q : k_loops) a_order.push_back(&loops[q]);
+  for (const L* l : a_order)
+    if (l->w.a <= 0) BAIL(25);
+  std::stable_sort(a_order.begin(), a_order.end(), [](const L* x, const L* y) { return x->w.a > y->w.a; });
+  const L* a_fast = a_order.back();
+  bool a_vec = a_fast->w.side == WSide::K && a_fast->w.a == 1 && a_fast->unit == 1 && a_fast->w.extent % 4 == 0 && p.a_c0 % 4 == 0;
+  for (const auto& l : loops)
+    if (&l != a_fast && l.w.a % 4 != 0) a_vec = false;
+  int64_t a_lds = kpad;
+  {
+    int64_t best = -1;
+    for (int64_t pad = 0; pad < 64; pad += a_vec ? 4 : 1) {
+      int64_t addr[64];
+      for (int lane = 0; lane < 64; ++lane) addr[lane] = (lane % 16) * (kpad + pad) + (lane / 16) * kdelta;
+      const int64_t cost = bank_cost(addr);
+      if (best < 0 || cost < best) {
+        best = cost;
+        a_lds = kpad + pad;
+      }
+      if (cost == 0) break;
+    }
+  }
+  const int64_t mrows = static_cast<int64_t>(lay.waves_m) * lay.mb * 16;
+
+  // ---- LDS layout of the patch: dense, one axis' stride padded against bank conflicts ------------------
+  auto set_strides = [&](size_t pad_axis, int64_t pad) {
     int64_t st = 1;
     for (size_t i = axes.size(); i-- > 0;) {
-      axes[i].lds = st + (i == 0 && axes.size() > 1 ? pad : 0);
+      axes[i].lds = st + (i == pad_axis && i + 1 < axes.size() ? pad : 0);
       st = axes[i].lds * axes[i].extent;
     }
+  };
+  auto floats_now = [&]() {
+    int64_t f = 1;
+    for (const auto& a : axes) f += (a.extent - 1) * a.lds;
+    return f;
   };
   // a loop's share of the patch offset for digit d
   auto lds_of = [&](const L& l, int64_t d) {
@@ -325,29 +360,36 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
     return o;
   };
   {
-    int64_t best_pad = 0, best_cost = -1;
-    for (int64_t pad = 0; pad < 64; ++pad) {
-      set_strides(pad);
-      int64_t c = 0;
-      const int64_t steps = std::min<int64_t>(ksteps, 12);
-      const int64_t blocks = std::min<int64_t>(ceil_div(NG, 16), 8);
-      for (int64_t st = 0; st < steps; ++st)
-        for (int64_t nb = 0; nb < blocks; ++nb) {
-          int64_t addr[64];
-          for (int lane = 0; lane < 64; ++lane) {
-            const int64_t n = std::min<int64_t>(nb * 16 + lane % 16, NG - 1);
-            const int64_t kk = std::min<int64_t>(k0[static_cast<size_t>(st)] + (lane / 16) * kdelta, K - 1);
-            addr[lane] = row_lds(n) + k_lds(kk);
+    int64_t best_pad = 0, best_cost = -1, best_floats = 0;
+    size_t best_axis = 0;
+    for (size_t pa = 0; pa + 1 < std::max<size_t>(axes.size(), 2); ++pa)
+      for (int64_t pad = 0; pad < 64; ++pad) {
+        set_strides(pa, pad);
+        const int64_t fl = floats_now();
+        if ((fl + mrows * a_lds) * 4 > 160 * 1024) break;
+        int64_t c = 0;
+        const int64_t steps = std::min<int64_t>(ksteps, 12);
+        const int64_t blocks = std::min<int64_t>(ceil_div(NG, 16), 8);
+        for (int64_t st = 0; st < steps; ++st)
+          for (int64_t nb = 0; nb < blocks; ++nb) {
+            int64_t addr[64];
+            for (int lane = 0; lane < 64; ++lane) {
+              const int64_t n = std::min<int64_t>(nb * 16 + lane % 16, NG - 1);
+              const int64_t kk = std::min<int64_t>(k0[static_cast<size_t>(st)] + (lane / 16) * kdelta, K - 1);
+              addr[lane] = row_lds(n) + k_lds(kk);
+            }
+            c += bank_cost(addr);
           }
-          c += bank_cost(addr);
+        if (best_cost < 0 || c < best_cost || (c == best_cost && fl < best_floats)) {
+          best_cost = c;
+          best_pad = pad;
+          best_axis = pa;
+          best_floats = fl;
         }
-      if (best_cost < 0 || c < best_cost) {
-        best_cost = c;
-        best_pad = pad;
+        if (c == 0) break;
       }
-      if (c == 0) break;
-    }
-    set_strides(best_pad);
+    if (best_cost < 0) BAIL(26);
+    set_strides(best_axis, best_pad);
   }
   int64_t patch_floats = 1;
   for (const auto& a : axes) patch_floats += (a.extent - 1) * a.lds;
@@ -380,34 +422,6 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
       if (o < 0) BAIL(24);
   }
 
-  // ---- A's rows in LDS: [m][k], row stride padded so that the sixteen rows and four sub-k of a read spread over the banks
-  // A is fetched in the order of its memory: the loops that index it sorted by their stride there
-  std::vector<const L*> a_order;
-  for (size_t q : m_loops) a_order.push_back(&loops[q]);
-  for (size_t q : k_loops) a_order.push_back(&loops[q]);
-  for (const L* l : a_order)
-    if (l->w.a <= 0) BAIL(25);
-  std::stable_sort(a_order.begin(), a_order.end(), [](const L* x, const L* y) { return x->w.a > y->w.a; });
-  const L* a_fast = a_order.back();
-  bool a_vec = a_fast->w.side == WSide::K && a_fast->w.a == 1 && a_fast->unit == 1 && a_fast->w.extent % 4 == 0 && p.a_c0 % 4 == 0;
-  for (const auto& l : loops)
-    if (&l != a_fast && l.w.a % 4 != 0) a_vec = false;
-  int64_t a_lds = kpad;
-  {
-    int64_t best = -1;
-    for (int64_t pad = 0; pad < 64; pad += a_vec ? 4 : 1) {
-      int64_t addr[64];
-      for (int lane = 0; lane < 64; ++lane) addr[lane] = (lane % 16) * (kpad + pad) + (lane / 16) * kdelta;
-      const int64_t cost = bank_cost(addr);
-      if (best < 0 || cost < best) {
-        best = cost;
-        a_lds = kpad + pad;
-      }
-      if (cost == 0) break;
-    }
-  }
-  const int64_t mrows = static_cast<int64_t>(lay.waves_m) * lay.mb * 16;
-  if ((patch_floats + mrows * a_lds) * 4 > 160 * 1024) BAIL(26);
   const bool a_zero = mrows != M || kpad != K;            // padding rows / columns of A's tile must read as zero
   const int64_t a_elems = a_vec ? M * K / 4 : M * K;
 
@@ -850,6 +864,481 @@ std::optional<WindowProblem> match_window_kernel(const Node& kernel, const std::
   p.kernels = {kernel.name};
   p.what = "the guarded operand of kernel " + kernel.name;
   return p;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// from a contraction and the kernels that add up shifted reads of its result
+// ---------------------------------------------------------------------------------------------------
+
+namespace {
+
+void add_terms(const NodePtr& e, std::vector<NodePtr>* out) {
+  if (e->op == Op::Add) {
+    add_terms(e->args[0], out);
+    add_terms(e->args[1], out);
+  } else {
+    out->push_back(e);
+  }
+}
+
+int64_t pos_mod(int64_t a, int64_t m) { return ((a % m) + m) % m; }
+
+struct Tap {                      // one shifted read of the contraction's result
+  Affine index;                   // where, over the adding kernels' loops
+  std::vector<WGuard> guards;     // when
+  Affine op[2];                   // the addresses of the contraction's two operands this stands for
+};
+
+// a loop that runs once is at zero: its terms go
+void drop_single(Affine* a, const std::vector<Loop>& loops) {
+  for (const auto& l : loops)
+    if (l.extent <= 1) a->coef.erase(l.var);
+}
+
+// loops of extent > 1 by their stride in `a`, largest first; false unless the strides are positive
+// and no loop reaches into the next one's stride (a digit per loop)
+bool digit_loops(const std::vector<Loop>& loops, const Affine& a, std::vector<std::pair<int64_t, Loop>>* out) {
+  out->clear();
+  for (const auto& l : loops) {
+    if (l.extent <= 1) continue;
+    if (a.of(l.var) <= 0) return false;
+    out->push_back({a.of(l.var), l});
+  }
+  std::stable_sort(out->begin(), out->end(), [](const auto& x, const auto& y) { return x.first > y.first; });
+  for (size_t j = 0; j + 1 < out->size(); ++j)
+    if ((*out)[j].first < (*out)[j + 1].first * (*out)[j + 1].second.extent) return false;
+  return true;
+}
+
+// `idx` (over `loops`, wherever `guards` hold) as one affine value per loop of the producer:
+// producer.out_aff evaluated at those values is idx, and every value stays inside its loop.
+bool producer_digits(const Affine& idx, const std::vector<WGuard>& guards, const std::vector<Loop>& loops, const NestKernel& prod,
+                     std::map<std::string, Affine>* digits) {
+  // what the guards leave of each loop's range
+  std::map<std::string, std::pair<int64_t, int64_t>> range;
+  for (const auto& l : loops) range[l.var] = {0, l.extent - 1};
+  for (const auto& g : guards) {
+    if (g.terms.size() != 1 || std::llabs(g.terms[0].second) != 1 || !range.count(g.terms[0].first)) continue;
+    auto& r = range[g.terms[0].first];
+    if (g.terms[0].second == 1) {
+      if (g.ge) r.first = std::max(r.first, g.bound);
+      else r.second = std::min(r.second, g.bound - 1);
+    } else {
+      if (g.ge) r.second = std::min(r.second, -g.bound);
+      else r.first = std::max(r.first, -g.bound + 1);
+    }
+  }
+  for (const auto& kv : range)
+    if (kv.second.first > kv.second.second) return false;
+  std::vector<std::pair<int64_t, Loop>> pl;
+  if (!digit_loops(prod.loops, *prod.out_aff, &pl) || pl.empty()) return false;
+  std::vector<Affine> e(pl.size());
+  for (const auto& kv : idx.coef) {
+    if (kv.second == 0) continue;
+    if (!range.count(kv.first)) return false;
+    size_t j = 0;
+    while (j < pl.size() && pl[j].first > std::llabs(kv.second)) ++j;
+    if (j == pl.size() || kv.second % pl[j].first) return false;
+    e[j].coef[kv.first] = kv.second / pl[j].first;
+  }
+  int64_t rest = idx.c - prod.out_aff->c;
+  for (size_t j = pl.size(); j-- > 0;) {
+    int64_t vlo = 0, vhi = 0;
+    for (const auto& kv : e[j].coef) {
+      const auto& r = range[kv.first];
+      vlo += kv.second > 0 ? kv.second * r.first : kv.second * r.second;
+      vhi += kv.second > 0 ? kv.second * r.second : kv.second * r.first;
+    }
+    const int64_t s = pl[j].first, ext = pl[j].second.extent;
+    if (rest % s) return false;
+    int64_t d = rest / s;
+    if (j > 0) {
+      if (pl[j - 1].first % s) return false;
+      const int64_t ratio = pl[j - 1].first / s;
+      // d is fixed modulo the ratio to the next stride; the one value that keeps the digit in its loop
+      d = -vlo + pos_mod(d + vlo, ratio);      // the smallest such value that keeps the digit from going negative
+    }
+    if (vlo + d < 0 || vhi + d > ext - 1) return false;
+    e[j].c = d;
+    rest -= d * s;
+  }
+  if (rest != 0) return false;
+  digits->clear();
+  for (size_t j = 0; j < pl.size(); ++j) (*digits)[pl[j].second.var] = e[j];
+  for (const auto& l : prod.loops)
+    if (l.extent <= 1) (*digits)[l.var] = Affine{};
+  return true;
+}
+
+// `op` (over the producer's loops and its reduce loop) with the producer's loops replaced by `digits`
+// (its reduce loop, `kvar`, is called `kname` in the result: the names of the two nests may clash)
+bool substitute(const Affine& op, const std::map<std::string, Affine>& digits, const std::string& kvar, const std::string& kname,
+                Affine* out) {
+  Affine r;
+  r.c = op.c;
+  for (const auto& kv : op.coef) {
+    if (kv.second == 0) continue;
+    if (kv.first == kvar) {
+      r.coef[kname] += kv.second;
+      continue;
+    }
+    auto d = digits.find(kv.first);
+    if (d == digits.end()) return false;
+    r.c += kv.second * d->second.c;
+    for (const auto& dv : d->second.coef) r.coef[dv.first] += kv.second * dv.second;
+  }
+  for (auto it = r.coef.begin(); it != r.coef.end();) it = it->second == 0 ? r.coef.erase(it) : std::next(it);
+  *out = r;
+  return true;
+}
+
+// the part of each loop's range that the loads of `buf` in `reader` reach (digits of the loops'
+// strides in `out`); false when that cannot be told
+bool read_box(const NestKernel& reader, const std::string& buf, const std::vector<std::pair<int64_t, Loop>>& dl, int64_t out_c,
+              std::map<std::string, std::pair<int64_t, int64_t>>* box) {
+  std::vector<LoadRef> loads;
+  collect_loads(*reader.value, loads);
+  std::map<std::string, int64_t> extent;
+  for (const auto& l : reader.loops) extent[l.var] = l.extent;
+  if (reader.rkind != ReduceKind::None) extent[reader.rloop.var] = reader.rloop.extent;
+  for (const auto& lr : loads) {
+    if (lr.load->args[0]->op != Op::Var) return false;
+    if (lr.load->args[0]->name != buf) continue;
+    if (lr.load->count != 1) return false;
+    auto a = affine_of(*lr.load->args[1]);
+    if (!a) return false;
+    std::vector<int64_t> lo(dl.size(), 0), span(dl.size(), 0);
+    int64_t rest = a->c - out_c;
+    if (rest < 0) return false;
+    for (size_t j = 0; j < dl.size(); ++j) {
+      lo[j] = rest / dl[j].first;
+      rest -= lo[j] * dl[j].first;
+    }
+    if (rest != 0) return false;
+    for (const auto& kv : a->coef) {
+      if (kv.second == 0) continue;
+      auto ex = extent.find(kv.first);
+      if (ex == extent.end() || kv.second < 0) return false;
+      size_t j = 0;
+      while (j < dl.size() && dl[j].first > kv.second) ++j;
+      if (j == dl.size() || kv.second % dl[j].first) return false;
+      span[j] += (kv.second / dl[j].first) * (ex->second - 1);
+    }
+    for (size_t j = 0; j < dl.size(); ++j) {
+      if (lo[j] + span[j] > dl[j].second.extent - 1) return false;
+      auto it = box->find(dl[j].second.var);
+      if (it == box->end()) (*box)[dl[j].second.var] = {lo[j], lo[j] + span[j]};
+      else it->second = {std::min(it->second.first, lo[j]), std::max(it->second.second, lo[j] + span[j])};
+    }
+  }
+  return true;
+}
+
+}  // namespace
+
+// why a candidate was turned down, for whoever sets EH_WINDOW_DEBUG
+#define SW_DECLINE(n)                                                                             \
+  do {                                                                                            \
+    if (std::getenv("EH_WINDOW_DEBUG")) std::fprintf(stderr, "shifted-sum window: %s declined at check %d\n", nests[i]->name.c_str(), n); \
+    return std::nullopt;                                                                          \
+  } while (0)
+
+std::optional<ScatteredWindow> try_emit_scattered_window(size_t i, const ProgramView& pv, const GenOptions& opt) {
+  const auto& nests = *pv.nests;
+  if (i >= nests.size() || !nests[i] || pv.taken(i)) return std::nullopt;
+  const NestKernel& P = *nests[i];
+  if (P.rkind != ReduceKind::Sum || !P.identity || P.identity->fval != 0.0 || P.acc_dtype.ty != Ty::F32 || P.out_dtype.ty != Ty::F32 ||
+      !P.out_aff || P.rloop.extent < 4 || pv.role_of(P.out_buf) != "temp")
+    SW_DECLINE(2);
+  const Node& pvl = *P.value;
+  if (pvl.op != Op::Mul) SW_DECLINE(3);
+  Affine pop[2];
+  std::string pbuf[2];
+  for (int o = 0; o < 2; ++o) {
+    const Node& ld = *pvl.args[static_cast<size_t>(o)];
+    if (ld.op != Op::Load || ld.args[0]->op != Op::Var || ld.count != 1 || ld.dtype.ty != Ty::F32) SW_DECLINE(4);
+    auto a = affine_of(*ld.args[1]);
+    if (!a) SW_DECLINE(5);
+    pop[o] = *a;
+    drop_single(&pop[o], P.loops);
+    pbuf[o] = ld.args[0]->name;
+  }
+  auto rd = pv.readers->find(P.out_buf);
+  if (rd == pv.readers->end() || rd->second.empty()) SW_DECLINE(6);
+  const size_t n = rd->second.size();
+  for (size_t q = 0; q < n; ++q)
+    if (rd->second[q] != i + 1 + q) SW_DECLINE(7);
+  // an operand that is itself a gather evaluated in place (a permuting copy folded into the
+  // contraction) is read at its source
+  const NestKernel* gat[2] = {nullptr, nullptr};
+  Affine gsrc[2];
+  for (int o = 0; o < 2; ++o) {
+    gat[o] = pv.folded_gather(pbuf[o]);
+    if (!gat[o]) continue;
+    const Node& gv = *gat[o]->value;
+    if (gat[o]->rkind != ReduceKind::None || !gat[o]->out_aff || gv.op != Op::Load || gv.args[0]->op != Op::Var || gv.count != 1 ||
+        gv.dtype.ty != Ty::F32)
+      SW_DECLINE(100);
+    auto gi = affine_of(*gv.args[1]);
+    if (!gi) SW_DECLINE(101);
+    gsrc[o] = *gi;
+    drop_single(&gsrc[o], gat[o]->loops);
+    pbuf[o] = gv.args[0]->name;
+  }
+  if (i + n >= nests.size()) SW_DECLINE(8);
+
+  // ---- the adding kernels and their shifted reads --------------------------------------------------
+  std::vector<Tap> taps;
+  const NestKernel* first = nullptr;
+  ScatteredWindow out;
+  out.elided.push_back(P.out_buf);
+  for (size_t q = 0; q < n; ++q) {
+    const size_t ci = i + 1 + q;
+    if (!nests[ci] || pv.taken(ci)) SW_DECLINE(9);
+    const NestKernel& C = *nests[ci];
+    if (C.rkind != ReduceKind::None || !C.out_aff || C.out_dtype.ty != Ty::F32 || C.out_buf == pbuf[0] || C.out_buf == pbuf[1]) SW_DECLINE(10);
+    if (!first) {
+      first = &C;
+    } else {
+      if (C.loops.size() != first->loops.size() || !(*C.out_aff == *first->out_aff)) SW_DECLINE(11);
+      for (size_t l = 0; l < C.loops.size(); ++l)
+        if (C.loops[l].var != first->loops[l].var || C.loops[l].extent != first->loops[l].extent) SW_DECLINE(12);
+    }
+    if (q + 1 < n) {
+      auto r = pv.readers->find(C.out_buf);
+      if (pv.role_of(C.out_buf) != "temp" || r == pv.readers->end() || r->second != std::vector<size_t>{ci + 1}) SW_DECLINE(13);
+      out.elided.push_back(C.out_buf);
+    }
+    std::vector<NodePtr> terms;
+    add_terms(C.value, &terms);
+    int running = 0;
+    for (const auto& t : terms) {
+      const Node* x = t.get();
+      Tap tap;
+      if (x->op == Op::Select) {
+        if (x->args[2]->op != Op::Const || x->args[2]->fval != 0.0 || !collect_guards(*x->args[0], &tap.guards)) SW_DECLINE(14);
+        x = x->args[1].get();
+      }
+      if (x->op != Op::Load || x->args[0]->op != Op::Var || x->count != 1 || x->dtype.ty != Ty::F32) SW_DECLINE(15);
+      auto a = affine_of(*x->args[1]);
+      if (!a) SW_DECLINE(16);
+      if (q > 0 && x->args[0]->name == nests[ci - 1]->out_buf) {
+        if (t->op == Op::Select || !(*a == *C.out_aff)) SW_DECLINE(17);
+        ++running;
+        continue;
+      }
+      if (x->args[0]->name != P.out_buf) SW_DECLINE(18);
+      tap.index = *a;
+      drop_single(&tap.index, C.loops);
+      taps.push_back(tap);
+    }
+    if (running != (q > 0 ? 1 : 0)) SW_DECLINE(19);
+  }
+  const NestKernel& last = *nests[i + n];
+  if (taps.size() < 2 || taps.size() > 64) SW_DECLINE(20);
+  std::vector<std::pair<int64_t, Loop>> out_digits;
+  if (!digit_loops(first->loops, *first->out_aff, &out_digits)) SW_DECLINE(21);
+
+  // ---- each read as addresses of the contraction's operands ----------------------------------------
+  const std::string kname = "eh_k";
+  for (auto& t : taps) {
+    std::map<std::string, Affine> digits;
+    if (!producer_digits(t.index, t.guards, first->loops, P, &digits)) SW_DECLINE(22);
+    std::vector<Loop> around = first->loops;
+    around.push_back(Loop{kname, P.rloop.extent});
+    for (int o = 0; o < 2; ++o) {
+      if (gat[o]) {
+        Affine at;
+        std::map<std::string, Affine> gd;
+        if (!substitute(pop[o], digits, P.rloop.var, kname, &at) || !producer_digits(at, t.guards, around, *gat[o], &gd) ||
+            !substitute(gsrc[o], gd, "", "", &t.op[o]))
+          SW_DECLINE(102);
+        continue;
+      }
+      if (!substitute(pop[o], digits, P.rloop.var, kname, &t.op[o])) SW_DECLINE(23);
+    }
+  }
+  for (const auto& t : taps)
+    for (int o = 0; o < 2; ++o)
+      if (t.op[o].coef != taps[0].op[o].coef) {
+        if (std::getenv("EH_WINDOW_DEBUG")) {
+          for (const auto& kv : t.op[o].coef) std::fprintf(stderr, " %s:%lld", kv.first.c_str(), (long long)kv.second);
+          std::fprintf(stderr, " vs");
+          for (const auto& kv : taps[0].op[o].coef) std::fprintf(stderr, " %s:%lld", kv.first.c_str(), (long long)kv.second);
+          std::fprintf(stderr, "\n");
+        }
+        SW_DECLINE(24);
+      }
+  // the window operand is the one the guarded loops move
+  std::map<std::string, int64_t> extent_of;
+  for (const auto& l : first->loops) extent_of[l.var] = l.extent;
+  auto always = [&](const WGuard& g) {
+    if (g.terms.empty()) return g.ge ? 0 >= g.bound : 0 < g.bound;
+    if (g.terms.size() != 1 || std::llabs(g.terms[0].second) != 1 || !extent_of.count(g.terms[0].first)) return false;
+    const int64_t e = extent_of[g.terms[0].first];
+    if (g.terms[0].second == 1) return g.ge ? g.bound <= 0 : g.bound >= e;
+    return g.ge ? g.bound <= -(e - 1) : g.bound >= 1;
+  };
+  std::set<std::string> guard_vars;
+  for (const auto& t : taps)
+    for (const auto& g : t.guards)
+      if (!always(g))
+        for (const auto& tm : g.terms) guard_vars.insert(tm.first);
+  if (guard_vars.empty()) SW_DECLINE(25);
+  int fo = -1;
+  for (int o = 0; o < 2; ++o) {
+    bool all = true, none = true;
+    for (const auto& v : guard_vars) {
+      all = all && taps[0].op[o].of(v) != 0;
+      none = none && taps[0].op[o].of(v) == 0;
+    }
+    if (all && fo < 0) fo = o;
+    else if (!none) SW_DECLINE(26);
+  }
+  if (fo < 0) SW_DECLINE(27);
+  const int ao = 1 - fo;
+  for (const auto& v : guard_vars)
+    if (taps[0].op[ao].of(v) != 0) SW_DECLINE(28);
+
+  // ---- the shifts as one or two more reduce loops ----------------------------------------------------
+  std::stable_sort(taps.begin(), taps.end(), [&](const Tap& x, const Tap& y) {
+    return x.op[ao].c != y.op[ao].c ? x.op[ao].c < y.op[ao].c : x.op[fo].c < y.op[fo].c;
+  });
+  const int64_t nt = static_cast<int64_t>(taps.size());
+  auto vec = [&](int64_t t) { return std::pair<int64_t, int64_t>{taps[static_cast<size_t>(t)].op[fo].c, taps[static_cast<size_t>(t)].op[ao].c}; };
+  const auto v0 = vec(0);
+  const std::pair<int64_t, int64_t> d2{vec(1).first - v0.first, vec(1).second - v0.second};
+  int64_t n2 = 2;
+  while (n2 < nt && vec(n2) == std::pair<int64_t, int64_t>{v0.first + n2 * d2.first, v0.second + n2 * d2.second}) ++n2;
+  if (nt % n2) SW_DECLINE(29);
+  const int64_t n1 = nt / n2;
+  const std::pair<int64_t, int64_t> d1 = n1 > 1 ? std::pair<int64_t, int64_t>{vec(n2).first - v0.first, vec(n2).second - v0.second}
+                                                 : std::pair<int64_t, int64_t>{0, 0};
+  for (int64_t t = 0; t < nt; ++t)
+    if (vec(t) != std::pair<int64_t, int64_t>{v0.first + (t / n2) * d1.first + (t % n2) * d2.first,
+                                              v0.second + (t / n2) * d1.second + (t % n2) * d2.second})
+      SW_DECLINE(30);
+  if (d2.second <= 0 || d2.first == 0 || (n1 > 1 && (d1.second <= 0 || d1.first == 0))) SW_DECLINE(31);
+
+  WindowProblem p;
+  const char* tap_names[2] = {"eh_shift0", "eh_shift1"};
+  // guards: one family per (terms, sense); a family's bounds move with the shift digits
+  {
+    std::map<std::pair<std::vector<std::pair<std::string, int64_t>>, bool>, std::vector<std::vector<int64_t>>> fam;
+    for (int64_t t = 0; t < nt; ++t)
+      for (const auto& g : taps[static_cast<size_t>(t)].guards) {
+        auto terms = g.terms;
+        std::sort(terms.begin(), terms.end());
+        auto& f = fam[{terms, g.ge}];
+        f.resize(static_cast<size_t>(nt));
+        f[static_cast<size_t>(t)].push_back(g.bound);
+      }
+    for (const auto& kv : fam) {
+      std::vector<int64_t> b(static_cast<size_t>(nt));
+      bool everywhere = true;
+      for (int64_t t = 0; t < nt; ++t) {
+        const auto& v = kv.second[static_cast<size_t>(t)];
+        if (v.empty()) { everywhere = false; break; }
+        // several of one kind: the tightest
+        b[static_cast<size_t>(t)] = kv.first.second ? *std::max_element(v.begin(), v.end()) : *std::min_element(v.begin(), v.end());
+      }
+      if (!everywhere) {
+        // a condition some shifts lack must be one that always holds where it is stated
+        WGuard g;
+        g.terms = kv.first.first;
+        g.ge = kv.first.second;
+        for (int64_t t = 0; t < nt; ++t)
+          for (int64_t bb : kv.second[static_cast<size_t>(t)]) {
+            g.bound = bb;
+            if (!always(g)) SW_DECLINE(32);
+          }
+        continue;
+      }
+      const int64_t b0 = b[0], s2 = b[1] - b[0], s1 = n1 > 1 ? b[static_cast<size_t>(n2)] - b[0] : 0;
+      for (int64_t t = 0; t < nt; ++t)
+        if (b[static_cast<size_t>(t)] != b0 + (t / n2) * s1 + (t % n2) * s2) SW_DECLINE(33);
+      WGuard g;
+      g.terms = kv.first.first;
+      g.ge = kv.first.second;
+      g.bound = b0;
+      if (n1 > 1 && s1) g.terms.push_back({tap_names[0], -s1});
+      if (s2) g.terms.push_back({tap_names[1], -s2});
+      p.guards.push_back(g);
+    }
+  }
+
+  // ---- the contraction over (k, shifts) ---------------------------------------------------------------
+  const Affine &F = taps[0].op[fo], &A = taps[0].op[ao];
+  for (const auto& l : first->loops) {
+    WLoop w;
+    w.name = l.var;
+    w.extent = l.extent;
+    w.f = F.of(l.var);
+    w.a = A.of(l.var);
+    w.c = first->out_aff->of(l.var);
+    w.side = w.f != 0 && w.a != 0 ? WSide::Batch : w.f != 0 ? WSide::Row : WSide::M;
+    if (w.extent > 1 && w.f == 0 && w.a == 0) SW_DECLINE(34);
+    p.loops.push_back(w);
+  }
+  {
+    WLoop k;
+    k.name = kname;
+    k.extent = P.rloop.extent;
+    k.side = WSide::K;
+    k.f = F.of(kname);
+    k.a = A.of(kname);
+    if (k.f == 0 || k.a <= 0) SW_DECLINE(35);
+    p.loops.push_back(k);
+    WLoop s1, s2;
+    s1.name = tap_names[0]; s1.extent = n1; s1.side = WSide::K; s1.f = d1.first; s1.a = d1.second;
+    s2.name = tap_names[1]; s2.extent = n2; s2.side = WSide::K; s2.f = d2.first; s2.a = d2.second;
+    if (n1 > 1) p.loops.push_back(s1);
+    p.loops.push_back(s2);
+  }
+  p.f_c0 = F.c;
+  p.a_c0 = A.c;
+  p.c_c0 = first->out_aff->c;
+  p.f_buf = pbuf[fo];
+  p.a_buf = pbuf[ao];
+  p.c_buf = last.out_buf;
+  if (p.a_c0 < 0 || p.c_c0 < 0 || p.f_buf == p.c_buf || p.a_buf == p.c_buf) SW_DECLINE(36);
+
+  // ---- only what is read of the result ---------------------------------------------------------------
+  if (pv.role_of(last.out_buf) == "temp") {
+    auto r = pv.readers->find(last.out_buf);
+    std::map<std::string, std::pair<int64_t, int64_t>> box;
+    bool known = r != pv.readers->end() && !r->second.empty();
+    if (known)
+      for (size_t q : r->second) known = known && q > i + n && nests[q] && read_box(*nests[q], last.out_buf, out_digits, first->out_aff->c, &box);
+    if (known)
+      for (auto& w : p.loops) {
+        auto b = box.find(w.name);
+        if (b == box.end() || w.side == WSide::K) continue;
+        const int64_t lo = b->second.first, cnt = b->second.second - b->second.first + 1;
+        if (cnt == w.extent) continue;
+        out.partial = true;
+        w.extent = cnt;
+        p.f_c0 += lo * w.f;
+        p.a_c0 += lo * w.a;
+        p.c_c0 += lo * w.c;
+        for (auto& g : p.guards)
+          for (const auto& tm : g.terms)
+            if (tm.first == w.name) g.bound -= tm.second * lo;
+      }
+  }
+  auto fe = pv.elems->find(p.f_buf);
+  if (fe == pv.elems->end() || fe->second * 4 >= (size_t{1} << 31)) SW_DECLINE(37);
+  p.f_bytes = fe->second * 4;
+  p.f_algo_bytes = static_cast<double>(p.f_bytes);
+  p.entry = "ehk_" + P.name;
+  p.kernels = {P.name};
+  for (size_t q = 0; q < n; ++q) p.kernels.push_back(nests[i + 1 + q]->name);
+  p.what = "shifted reads of the product of kernel " + P.name + ", summed by " + std::to_string(n) + " kernels";
+  p.tag = ",shifts=" + std::to_string(nt);
+  out.launches = emit_window(p, opt, nullptr);
+  if (out.launches.empty()) SW_DECLINE(38);
+  out.next = i + 1 + n;
+  return out;
 }
 
 }  // namespace eh

@@ -7,6 +7,8 @@
 // (kernels/window_f32_mfma.hip).
 #pragma once
 
+#include <functional>
+#include <map>
 #include <optional>
 #include <string>
 #include <utility>
@@ -63,5 +65,29 @@ std::vector<LaunchSpec> try_emit_window_gemm(const NestKernel& k, const GemmShap
 //   acc = 0; for k loops ...: acc = acc + select(guard, F[..], 0) * A[..]; out[..] = acc
 // (either factor order, the guard optional), every index affine.  `f_bytes`: size of F's buffer.
 std::optional<WindowProblem> match_window_kernel(const Node& kernel, const std::map<std::string, size_t>& buffer_elems);
+
+// A contraction whose result is read only by a run of elementwise kernels that add shifted,
+// guarded reads of it to a running sum (a transposed convolution as the reference lowers it --
+// the input gradient of conv2d, crates/nn/src/functional/conv.rs:113-187 differentiated: a
+// product with the weights, then fold as a sum of padded slices): the sum over the shifts joins
+// the sum of the contraction,
+//   S[rows] = sum over (k, shift) of [guard(rows, shift)] F[rows - shift, k] * A[k, shift, m],
+// and the product's result and the partial sums never reach memory.  Elements of S no later kernel
+// reads (a border that the next kernel slices away) are not computed.
+struct ProgramView {
+  const std::vector<std::optional<NestKernel>>* nests = nullptr;
+  const std::map<std::string, std::vector<size_t>>* readers = nullptr;      // kernels (by index) reading a buffer
+  const std::map<std::string, size_t>* elems = nullptr;                     // elements per buffer
+  std::function<std::string(const std::string&)> role_of;
+  std::function<const NestKernel*(const std::string&)> folded_gather;       // the gather evaluated in place of reading this buffer, or null
+  std::function<bool(size_t)> taken;                                        // kernel already folded into another
+};
+struct ScatteredWindow {
+  std::vector<LaunchSpec> launches;
+  size_t next = 0;                      // first kernel after the run
+  std::vector<std::string> elided;      // buffers that no longer exist
+  bool partial = false;                 // the output is not written everywhere (only where it is read)
+};
+std::optional<ScatteredWindow> try_emit_scattered_window(size_t i, const ProgramView& pv, const GenOptions& opt);
 
 }  // namespace eh

@@ -1065,14 +1065,16 @@ def test_config5_with_implicit_gemm_loader(frontend, hip):
         assert np.allclose(g, p, rtol=1e-4, atol=1e-7)
     # guarded reads (padding) through a buffer resource, out of range where the guard fails
     # (default), or at a clamped index with a select behind them (ranged_loads=0): same bits
-    assert any("eh_ranged_load(eh_rs_" in l["source"] for l in folded.launches)
-    assert not any("eh_ranged_load" in l["source"] for l in hip.render_program(prog_ast, {"ranged_loads": 0}).launches)
-    reg.options = {"ranged_loads": 0}
+    # (in the plan without the LDS-staged schedules: there the shifted sums of the input gradient are a kernel of their own)
+    assert any("eh_ranged_load(eh_rs_" in l["source"] for l in hip.render_program(prog_ast, {"gemm_window": 0}).launches)
+    assert not any("eh_ranged_load" in l["source"]
+                   for l in hip.render_program(prog_ast, {"ranged_loads": 0, "gemm_window": 0}).launches)
+    reg.options = {"ranged_loads": 0, "gemm_window": 0}
     try:
         got_clamped = _cnn_step_on(frontend, "hip", arrays, True)
     finally:
         reg.options = old
-    for g, c in zip(got, got_clamped):
+    for g, c in zip(got_loader, got_clamped):
         assert np.array_equal(g, c)
     # option gemm_merge_batch=1: per-image weight-gradient contractions and the sum over images
     # that follows become one contraction with the batch folded into k
@@ -1487,6 +1489,54 @@ def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
         close = np.isclose(g, r, rtol=1e-4, atol=1e-5 * scale)
         # a relu or max-pool tie that falls differently moves one window's gradient
         assert int((~close).sum()) <= (2 if "pool True" in desc else 0), desc
+
+
+CONV_DX_CASES = [((3, 8, 10, 12), (16, 8, 3, 3), (1, 1), (1, 1), 9),
+                 ((2, 4, 9, 7), (8, 4, 5, 5), (2, 2), (1, 1), 25),
+                 ((2, 6, 8, 8), (12, 6, 2, 2), (0, 0), (1, 1), 4),
+                 ((2, 4, 6, 20), (8, 4, 1, 3), (0, 1), (1, 1), 3),
+                 ((2, 32, 14, 14), (64, 32, 3, 3), (1, 1), (1, 1), 9),
+                 ((5, 3, 10, 10), (8, 3, 3, 3), (0, 0), (1, 1), 9),
+                 ((2, 4, 12, 12), (8, 4, 3, 3), (2, 2), (2, 2), 0),
+                 ((1, 16, 30, 30), (8, 16, 3, 3), (1, 1), (1, 1), 9),
+                 ((1, 64, 20, 20), (64, 64, 3, 3), (1, 1), (1, 1), 0)]
+
+
+@pytest.mark.parametrize("xs,ws,pad,dil,shifts", CONV_DX_CASES)
+def test_convolution_input_gradients_as_one_window_contraction(frontend, hip, xs, ws, pad, dil, shifts):
+    """d/dx of sum(conv2d(x, w) * g): the product dY x W and the kernels that add up its shifted
+    reads run as one window contraction (3x3, 5x5, 2x2 and 1x3 kernels, with and without
+    padding; a dilated window and a weight tile too large for one workgroup's LDS keep the
+    separate launches).  All three gradients and the loss against the oracle."""
+    from harp_amd import workloads as wl
+    fe = frontend
+
+    def fn(x, w, g):
+        return fe.nn.conv2d(x, w, None, padding=pad, dilation=dil) * g
+
+    ho = xs[2] + 2 * pad[0] - dil[0] * (ws[2] - 1)
+    wo = xs[3] + 2 * pad[1] - dil[1] * (ws[3] - 1)
+    shapes = [xs, ws, (xs[0], ws[0], ho, wo)]
+    with fe.exact_mode():
+        ts = [fe.Tensor.input(list(sh)) for sh in shapes]
+        loss = fn(*ts)
+        while loss.ndim() > 0:
+            loss = loss.sum(loss.ndim() - 1)
+        loss.backward_with_params(ts)
+        plan = hip.render_program(wl.lower_multi(ts[1:], [ts[0].grad().contiguous()])[0])
+    fused = [l for l in plan.launches if "shifts=" in l["schedule"]]
+    assert len(fused) == (1 if shifts else 0), [l["schedule"] for l in plan.launches]
+    if shifts:
+        assert fused[0]["schedule"].endswith(",shifts=%d)" % shifts)
+    rng = RNG(sum(xs) + sum(ws))
+    arrays = [rng.uniform(-1, 1, sh).astype(np.float32) for sh in shapes]
+    ref = _grads_on(fe, "c", shapes, fn, arrays)
+    got = _grads_on(fe, "hip", shapes, fn, arrays)
+    assert ref is not None and len(ref) == len(got) == 4
+    for r, g in zip(ref, got):
+        assert r.shape == g.shape
+        scale = max(1.0, float(np.abs(r).max()))
+        assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
 
 
 def _grads_on(fe, kind, shapes, fn, arrays):

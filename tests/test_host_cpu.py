@@ -758,7 +758,7 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     body = reader["source"][reader["source"].index("__global__"):]
     assert body.count("eh_ranged_load(eh_rs_" + temp + ",") == 9   # guarded loads: out of range where the guard fails
     assert "if (" not in body.replace("if (eh_", "") and temp + "[" not in body
-    clamped = hb.render_program(ast, "lanes=1,ranged_loads=0")
+    clamped = hb.render_program(ast, "lanes=1,ranged_loads=0,gemm_window=0")
     (reader0,) = [l for l in clamped.launches if l["entry"] == reader["entry"]]
     assert reader0["source"].count(temp + "[") == 9             # ... or a clamped index and a select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
@@ -786,7 +786,8 @@ def test_convolution_windows_are_staged_in_lds(frontend):
     ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
     plan = hb.render_program(ast)
     win = {l["entry"]: l for l in plan.launches if l["schedule"].startswith("mfma16x16x4(window,")}
-    assert sorted(win) == ["ehk_R_256_196_64_1_9", "ehk_R_256_1_32_9_79", "ehk_R_256_1_64_288_88", "ehk_R_256_784_32_1_1"]
+    assert sorted(win) == ["ehk_R_256_196_1_288_59", "ehk_R_256_196_64_1_9", "ehk_R_256_1_32_9_79", "ehk_R_256_1_64_288_88",
+                           "ehk_R_256_784_32_1_1"]
     fwd2, wg2, fwd1 = win["ehk_R_256_196_64_1_9"], win["ehk_R_256_1_64_288_88"], win["ehk_R_256_784_32_1_1"]
     assert fwd2["schedule"].startswith("mfma16x16x4(window,group=196,M=64,K=288,waves=4x1,blocks=1x13,steps=72,patterns=1,")
     assert fwd2["grid"] == [256, 1, 1] and fwd2["block"] == [256, 1, 1] and "epilogue=2" in fwd2["schedule"]
@@ -800,9 +801,9 @@ def test_convolution_windows_are_staged_in_lds(frontend):
     m = re.search(r"axes \[32 x stride 196, valid 0\.\.32, lds (\d+)\] \[16 x stride 14, valid 1\.\.15, lds 16\] "
                   r"\[16 x stride 1, valid 1\.\.15, lds 1\]", fwd2["source"])
     assert m and 256 < int(m.group(1)) < 320
-    # (the four pixels of a step: consecutive, or two at the end of a row and two at the start of the next, 16 apart)
+    # (the four pixels of a step: consecutive, or two at the end of a row and two at the start of the next, a padded row stride apart)
     assert "if (p == 0) return 0 + b0 * 1 + b1 * 2 + (b0 & b1) * 0;" in wg2["source"]
-    assert "if (p == 1) return 0 + b0 * 1 + b1 * 4 + (b0 & b1) * 0;" in wg2["source"]
+    assert re.search(r"if \(p == 1\) return 0 \+ b0 \* 1 \+ b1 \* (\d+) \+ \(b0 & b1\) \* 0;", wg2["source"])
     wg1 = win["ehk_R_256_1_32_9_79"]
     assert wg1["schedule"].startswith("mfma16x16x4(window,group=9,M=32,K=784,waves=2x1,blocks=1x1,steps=196,patterns=1,")
     assert wg1["grid"] == [1, 1, 256] and wg1["block"] == [256, 1, 1]      # two waves multiply, all four fetch
@@ -813,7 +814,44 @@ def test_convolution_windows_are_staged_in_lds(frontend):
     assert not any("(window," in l["schedule"] for l in loader.launches) and len(loader.launches) >= len(plan.launches)
     gone = lambda p: {b["name"] for b in p.buffers if b["elided"]}          # noqa: E731
     # (with K split, the per-image results of that weight gradient are summed from the partial tiles and never exist)
-    assert gone(plan) <= gone(loader) and len(gone(loader) - gone(plan)) <= 1
+    # (and the columns of the second convolution's input gradient exist only in the tile-loader plan)
+    assert len(gone(loader) - gone(plan)) <= 1 and len(gone(plan) - gone(loader)) == 1
+
+
+def test_convolution_input_gradient_is_one_window_contraction(frontend):
+    """The input gradient of the second convolution as the reference lowers it: dY x W into
+    columns [pixel, channel x tap], then eight kernels that add up nine shifted, guarded reads of
+    the columns into the padded image.  The nine reads join the contraction's sum (K = 64
+    channels x 3 x 3 shifts, the shifts walking dY against the pixel), dY is read at its NCHW
+    source rather than through the permuting copy folded into the product, and the one-pixel
+    border that the next kernel slices away is not computed: one launch for nine kernels, and
+    neither the columns (58 MB) nor the partial sums reach memory."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    import re
+    arrays = wl.config5_inputs(*wl.cnn_sizes(True))
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
+    plan = hb.render_program(ast)
+    (dx,) = [l for l in plan.launches if "shifts=" in l["schedule"]]
+    assert dx["schedule"].startswith("mfma16x16x4(window,group=196,M=32,K=576,waves=2x2,blocks=1x7,steps=144,patterns=1,")
+    assert dx["schedule"].endswith(",shifts=9)") and dx["grid"] == [256, 1, 1]
+    assert dx["kernels"] == ["R_256_196_1_288_59"] + ["E_256_32_16_16_%d" % q for q in range(60, 68)]
+    assert len(dx["args"]) == 3 and dx["written"] == [False, False, True]
+    # dY's channels, and its 14 x 14 pixels inside a border of one: source coordinate = pixel - shift
+    assert re.search(r"axes \[64 x stride 196, valid 0\.\.64, lds \d+\] \[16 x stride 14, valid 1\.\.15, lds 16\] "
+                     r"\[16 x stride 1, valid 1\.\.15, lds 1\]", dx["source"])
+    # the result's interior only (offset 17 = one row and one column into the 16 x 16 image)
+    assert "return 17LL + 0LL;" in dx["source"] and "(u / 14u) % 14u) * 16LL" in dx["source"]
+    out = dx["args"][2]
+    assert dx["overwrites"] == [False, False, False]           # ... so the output is not overwritten as a whole
+    gone = {b["name"] for b in plan.buffers if b["elided"]}
+    assert len(gone & {"buf%d" % q for q in range(145, 161, 2)}) == 8 and out not in gone
+    assert len(hb.compile_source(dx["source"])) > 1000
+    assert len(plan.launches) == 22
+    # a result that is a program output is computed everywhere
+    off = hb.render_program(ast, "gemm_window=0")
+    assert not any("shifts=" in l["schedule"] for l in off.launches) and len(off.launches) == 23
 
 
 def test_convolution_rows_run_across_images(frontend):
