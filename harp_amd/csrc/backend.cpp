@@ -485,6 +485,7 @@ GenOptions parse_options(const char* text) {
     else if (k == "gemm_waves") o.gemm_waves = as_int();
     else if (k == "gemm_fold") o.gemm_fold = as_int() != 0;
     else if (k == "gemm_window") o.gemm_window = as_int() != 0;
+    else if (k == "window_passes") o.window_passes = std::max(0, std::min(4, as_int()));
     else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
     else if (k == "gemm_dma") o.gemm_dma = std::max(0, std::min(3, as_int()));
     else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;

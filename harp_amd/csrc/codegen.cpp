@@ -3086,6 +3086,12 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       std::ostringstream load_body, apply_body;
       std::vector<std::string> slot_types;
       bool split_ok = true;
+      // ... and for four elements in a row (eh_e a multiple of four): what does not move inside the
+      // four is read once, what is read at the element itself as one vector, stores as vectors
+      std::ostringstream quad_load, quad_apply;
+      std::vector<std::string> quad_slots;         // declarations of EhEpiLoads4's members
+      int quad_regs = 0;
+      bool quad_ok = !(c_relaid && relaid_pos > 0);
       std::vector<std::string> ext_order;
       std::map<std::string, std::pair<std::string, size_t>> ext;   // name -> (declaration, min bytes)
       epi.store_c = needed(k0.out_buf);
@@ -3097,6 +3103,11 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       body << "  const " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf << " = eh_acc;\n";
       if (epi.store_c) body << "  " << k0.out_buf << "[eh_e] = eh_acc;\n";
       apply_body << body.str();
+      quad_load << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n  (void)eh_l;\n";
+      quad_apply << "  const " << IT << " eh_l = (" << IT << ")eh_e;\n  (void)eh_l;\n  " << ctype(k0.out_dtype) << " eh_v_" << k0.out_buf
+                 << "[4] = {eh_acc[0], eh_acc[1], eh_acc[2], eh_acc[3]};\n";
+      if (epi.store_c)
+        quad_apply << "  *reinterpret_cast<EhQ<float>*>(" << k0.out_buf << " + eh_e) = EhQ<float>{eh_acc[0], eh_acc[1], eh_acc[2], eh_acc[3]};\n";
       auto decode_to = [&](std::ostringstream& to, const NestKernel& sk, const std::string& from) {
         int64_t numel = 0;
         auto strides = *dense_strides(sk, &numel);
@@ -3191,6 +3202,75 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           if (needed(sk.out_buf)) apply_body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
           apply_body << "  }\n";
         }
+        if (quad_ok) {
+          int64_t numel4 = 0;
+          const auto strides4 = *dense_strides(sk, &numel4);
+          std::set<std::string> still, vars;      // loops that keep their value over four aligned elements; all loops
+          for (size_t li = 0; li < sk.loops.size(); ++li) {
+            vars.insert(sk.loops[li].var);
+            if (sk.loops[li].extent == 1 || strides4[li] % 4 == 0) still.insert(sk.loops[li].var);
+          }
+          std::function<bool(const Node&)> as_value = [&](const Node& n) {
+            if (n.op == Op::Load) return false;
+            if ((n.op == Op::Var || n.op == Op::Wildcard) && vars.count(n.name)) return true;
+            for (const auto& a : n.args)
+              if (a && as_value(*a)) return true;
+            return false;
+          };
+          if (as_value(*sk.value) || (needed(sk.out_buf) && sk.out_dtype.itemsize() != 4)) quad_ok = false;
+          quad_load << "  {\n";
+          decode_to(quad_load, sk, "eh_l");
+          quad_apply << "  " << ctype(sk.out_dtype) << " eh_v_" << sk.out_buf << "[4];\n  {\n";
+          std::map<const Node*, std::string> slot_of;
+          for (int c = 0; c < 4 && quad_ok; ++c) {
+            ExprRenderer er4;
+            er4.load_hook = [&](const Node& ld, std::string* out) {
+              const std::string& lb = ld.args[0]->name;
+              const std::string comp = "[" + std::to_string(c) + "]";
+              if (avail.count(lb)) {
+                *out = "eh_v_" + lb + comp;
+                return true;
+              }
+              auto known = slot_of.find(&ld);
+              if (known == slot_of.end()) {
+                auto a = affine_of(*ld.args[1]);
+                bool uniform = a.has_value();
+                if (a)
+                  for (const auto& kv : a->coef) uniform = uniform && (kv.second == 0 || still.count(kv.first));
+                const bool at_element = a && sk.out_aff && *a == *sk.out_aff && ld.dtype.itemsize() == 4;
+                for (const auto& lr : loads)
+                  if (lr.load == &ld && lr.guarded) uniform = false;
+                const std::string name = "eh_p.s" + std::to_string(quad_slots.size());
+                if (uniform) {
+                  ExprRenderer plain;
+                  quad_load << "    " << name << " = " << plain.expr(ld) << ";\n";
+                  quad_slots.push_back(ctype(ld.dtype) + " s" + std::to_string(quad_slots.size()));
+                  quad_regs += 1;
+                  known = slot_of.emplace(&ld, name).first;
+                } else if (at_element) {
+                  quad_load << "    " << name << " = *reinterpret_cast<const EhQ<" << ctype(ld.dtype) << ">*>(" << lb << " + eh_e);\n";
+                  quad_slots.push_back("EhQ<" + ctype(ld.dtype) + "> s" + std::to_string(quad_slots.size()));
+                  quad_regs += 4;
+                  known = slot_of.emplace(&ld, name + "[]").first;
+                } else {
+                  quad_ok = false;
+                  *out = "0";
+                  return true;
+                }
+              }
+              const std::string& sl = known->second;
+              *out = sl.size() > 2 && sl.compare(sl.size() - 2, 2, "[]") == 0 ? sl.substr(0, sl.size() - 2) + comp : sl;
+              return true;
+            };
+            quad_apply << "    eh_v_" << sk.out_buf << "[" << c << "] = (" << ctype(sk.out_dtype) << ")(" << er4.expr(*sk.value) << ");\n";
+          }
+          quad_load << "  }\n";
+          if (needed(sk.out_buf))
+            quad_apply << "    *reinterpret_cast<EhQ<" << ctype(sk.out_dtype) << ">*>(" << sk.out_buf << " + eh_e) = EhQ<" << ctype(sk.out_dtype)
+                       << ">{eh_v_" << sk.out_buf << "[0], eh_v_" << sk.out_buf << "[1], eh_v_" << sk.out_buf << "[2], eh_v_" << sk.out_buf
+                       << "[3]};\n";
+          quad_apply << "  }\n";
+        }
         if (needed(sk.out_buf)) {
           body << "    " << sk.out_buf << "[eh_e] = eh_v_" << sk.out_buf << ";\n";
           ext[sk.out_buf] = {ctype(sk.out_dtype) + "* __restrict__ " + sk.out_buf,
@@ -3226,6 +3306,19 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
            << apply_body.str() << "}\n";
         epi.split_functions = sp.str();
         epi.n_loads = static_cast<int>(slot_types.size());
+      }
+      if (quad_ok && total % 4 == 0 && quad_regs <= 24) {
+        std::ostringstream qd;
+        qd << "// the same for four elements in a row (eh_e a multiple of four), reads first\n"
+              "template <typename T> using EhQ = T __attribute__((ext_vector_type(4)));\nstruct EhEpiLoads4 {\n";
+        for (const auto& d : quad_slots) qd << "  " << d << ";\n";
+        qd << "};\n__device__ __forceinline__ void eh_epilogue_load4(long long eh_e, EhEpiLoads4& eh_p" << epi.params << ") {\n"
+           << quad_load.str() << "}\n";
+        qd << "__device__ __forceinline__ void eh_epilogue_apply4(long long eh_e, const float (&eh_acc)[4], const EhEpiLoads4& eh_p"
+           << (epi.store_c ? ", " + ctype(k0.out_dtype) + "* __restrict__ " + k0.out_buf : std::string()) << epi.params << ") {\n"
+           << quad_apply.str() << "}\n";
+        epi.quad_functions = qd.str();
+        epi.quad_regs = quad_regs;
       }
       have_epi = true;
     }
@@ -3379,12 +3472,12 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       g.stages.push_back(c.stage);
     }
     ++i;
-    while (opt.fuse && i < kernels.size() && nests[i] && !folded_kernels.count(i)) {
-      const NestKernel& k = *nests[i];
-      if (k.rkind == ReduceKind::Sum && opt.gemm && gemm_shaped(k, opt)) break;
+    // kernel k as the group's next stage, if it fits
+    auto stage_for = [&](const NestKernel& k) {
       Canon pick;
+      if (k.rkind == ReduceKind::Sum && opt.gemm && gemm_shaped(k, opt)) return pick;
       if (k.rkind != ReduceKind::None) {
-        if (!reduce_is_rowwise(k)) break;
+        if (!reduce_is_rowwise(k)) return pick;
         Canon c = canon_as(k, StageKind::Reduce);
         if (c.ok && c.rows == g.rows && c.C == g.C) pick = c;
       } else {
@@ -3395,11 +3488,53 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           if (s.ok && s.rows == g.rows && g.has_reduce()) pick = s;
         }
       }
-      if (!pick.ok || !aligned_with_group(g, pick.stage)) break;
       // a buffer may be written once per group
-      if (g.producer(pick.stage.out_buf)) break;
+      if (pick.ok && (!aligned_with_group(g, pick.stage) || g.producer(pick.stage.out_buf))) pick.ok = false;
+      return pick;
+    };
+    while (opt.fuse && i < kernels.size() && nests[i] && !folded_kernels.count(i)) {
+      if (absorbed.count(i)) {
+        ++i;
+        continue;
+      }
+      Canon pick = stage_for(*nests[i]);
+      if (!pick.ok) break;
       g.stages.push_back(pick.stage);
       ++i;
+    }
+    // Kernels further down that carry on with this group's rows on a few thousand elements (the
+    // bookkeeping of a loss, lowered behind the kernels of another root) join it when nothing in
+    // between has a hand in what they read or write: one launch less on the way, and no large
+    // value has to be kept for them.
+    if (opt.fuse && opt.reindex && opt.merge_launches && have_table && g.has_reduce()) {
+      auto tiny = [&](const Node* k) {
+        for (const auto& p : k->params) {
+          if (!p.dtype.is_ptr()) continue;
+          auto e = elems.find(p.name);
+          if (e == elems.end() || e->second > (size_t{1} << 12)) return false;
+        }
+        return true;
+      };
+      for (size_t j = i; j < kernels.size() && j < i + 200; ++j) {
+        if (absorbed.count(j) || folded_kernels.count(j) || windows.count(j) || scattered.count(j) || absorbed_name.count(j)) continue;
+        if (!nests[j] || !tiny(kernels[j])) continue;
+        bool feeds = false;
+        for (const auto& p : kernels[j]->params)
+          feeds = feeds || (p.dtype.is_ptr() && !p.mut_ && g.producer(p.name));
+        if (!feeds) continue;
+        bool free_to_move = true;
+        for (size_t m = i; m < j && free_to_move; ++m) {
+          if (absorbed.count(m)) continue;              // (already part of an earlier launch, this group's included)
+          for (const auto& pm : kernels[m]->params)
+            for (const auto& pj : kernels[j]->params)
+              if (pm.dtype.is_ptr() && pj.dtype.is_ptr() && pm.name == pj.name && (pm.mut_ || pj.mut_)) free_to_move = false;
+        }
+        if (!free_to_move) continue;
+        Canon pick = stage_for(*nests[j]);
+        if (!pick.ok) continue;
+        g.stages.push_back(pick.stage);
+        absorbed.insert(j);
+      }
     }
     // which stage outputs must reach memory
     for (size_t s = 0; s < g.stages.size(); ++s) {

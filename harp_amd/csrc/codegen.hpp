@@ -45,6 +45,7 @@ struct GenOptions {
   bool gemm_epilogue = true;          // run elementwise consumers of a contraction on its accumulators
   bool gemm_fold = true;              // evaluate gather/copy producers inside the tile loader (implicit GEMM)
   bool gemm_window = true;            // a folded sliding-window gather is staged in LDS once per group of rows instead of evaluated per element
+  int window_passes = 0;              // of that schedule: passes over k, each for a share of a wave's blocks, stored while the next multiplies (0: chosen by the number of blocks)
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
   int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores

@@ -81,6 +81,12 @@ struct EpilogueSpec {
   // for schedules that finish many elements per work-item: all reads first, then the stores.
   std::string split_functions;
   int n_loads = 0;                     // values eh_epilogue_load fetches per element
+  // ... and for four elements in a row, eh_e a multiple of four (else empty): reads that do not move
+  // inside the four once, reads at the element itself and the stores as 128-bit vectors:
+  //   struct EhEpiLoads4; void eh_epilogue_load4(long long eh_e, EhEpiLoads4&, <params>);
+  //   void eh_epilogue_apply4(long long eh_e, const float (&eh_acc)[4], const EhEpiLoads4&, [C,] <params>);
+  std::string quad_functions;
+  int quad_regs = 0;                   // registers EhEpiLoads4 takes
 };
 
 // True when element (b, m, n) of C sits at (b*M + m)*N + n, the index an epilogue is written for.

@@ -110,6 +110,12 @@ __device__ __forceinline__ long long ew_c_b(long long bz) { (void)bz; return 0; 
 #ifndef EW_MIX
 #define EW_MIX 1           // LDS reads of step s+1 issued one by one between the MFMAs of step s
 #endif
+#ifndef EW_PASSES
+#define EW_PASSES 1        // passes over k, each for a share of a wave's N-blocks
+#endif
+#ifndef EW_C_VEC
+#define EW_C_VEC 1         // 4: four rows of F in a row are neighbours in C (16-byte aligned): blocks computed transposed, 128-bit stores
+#endif
 
 typedef float ew_f4v __attribute__((ext_vector_type(4)));
 
@@ -117,6 +123,8 @@ namespace {
 // Four waves whatever the layout: waves beyond EW_WAVES_M * EW_WAVES_N only help to fetch.
 constexpr int EW_NT = 256;
 static_assert(EW_WAVES_M * EW_WAVES_N <= 4, "at most four multiplying waves");
+static_assert(EW_PASSES >= 1 && EW_PASSES <= 4 && (EW_NB + EW_PASSES - 1) / EW_PASSES * (EW_PASSES - 1) < EW_NB, "every pass has blocks");
+template <int V> struct EwInt { static constexpr int value = V; };
 }  // namespace
 
 extern "C" __global__ void __launch_bounds__(EW_NT)
@@ -214,110 +222,179 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
       base[nb][p] = r + ew_pat_lane(p, j4);
   }
 
-  ew_f4v acc[EW_MB][EW_NB];
-#pragma unroll
-  for (int mb = 0; mb < EW_MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < EW_NB; ++nb) acc[mb][nb] = ew_f4v{0.0f, 0.0f, 0.0f, 0.0f};
-
-  // step s multiplies with the operands fetched during step s - 1
-  float a[2][EW_MB], b[2][EW_NB];
-#pragma unroll
-  for (int mb = 0; mb < EW_MB; ++mb) a[0][mb] = As[abase[mb] + ew_k0[0]];
-#pragma unroll
-  for (int nb = 0; nb < EW_NB; ++nb) b[0][nb] = patch[base[nb][ew_kpat[0]] + ew_koff[0]];
-#pragma unroll
-  for (int s = 0; s < EW_KSTEPS; ++s) {
-    if (s + 1 < EW_KSTEPS) {
-#pragma unroll
-      for (int mb = 0; mb < EW_MB; ++mb) a[(s + 1) & 1][mb] = As[abase[mb] + ew_k0[s + 1]];
-#pragma unroll
-      for (int nb = 0; nb < EW_NB; ++nb) b[(s + 1) & 1][nb] = patch[base[nb][ew_kpat[s + 1]] + ew_koff[s + 1]];
-    }
-#pragma unroll
-    for (int nb = 0; nb < EW_NB; ++nb)
-#pragma unroll
-      for (int mb = 0; mb < EW_MB; ++mb)
-        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s & 1][mb], b[s & 1][nb], acc[mb][nb], 0, 0, 0);
-#if EW_MIX
-    // (one LDS read after every MFMA; the reads of A's values ride with the first ones)
-#pragma unroll
-    for (int q = 0; q < EW_MB; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-#pragma unroll
-    for (int q = EW_MB; q < EW_NB * EW_MB; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-#endif
-    __builtin_amdgcn_sched_barrier(0);
-  }
-
-  // Accumulator register v of lane l holds row 4 * (l / 16) + v of the M-block, column l % 16 of the
-  // N-block.  Blocks that lie inside the group whole are finished without a test per element, in one
-  // run of straight-line code: whatever the epilogue loads (a bias, a saved activation) is then
-  // requested for all of them before the first store goes out, where a branch around every element
-  // would make each element's load wait for the stores of the one before (one queue for both).
+  // The N-blocks of a wave are multiplied in EW_PASSES passes over k, each finished (epilogue,
+  // stores) before the next starts: a store only has to be issued, so the memory traffic of one
+  // pass's results drains while the matrix pipe works on the next pass, and only the last pass's
+  // stores are waited for at the end of the kernel.
   constexpr bool M_EDGE = MROWS != EW_M;
   const long long c_base = ew_c_b(bz);
-  auto finish = [&](const int mb, const int nb, const int v, const bool test) {
-    const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
-    const int n = (nb * EW_WAVES_N + wn) * 16 + l16;
-    if (test && !(m < EW_M && n < EW_NG)) return;
-    const long long e = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
-#if defined(EH_EPILOGUE)
-    eh_epilogue(e, acc[mb][nb][v] EH_C_ARG EH_EPI_ARGS);
+  constexpr int NBP = (EW_NB + EW_PASSES - 1) / EW_PASSES;
+  auto pass = [&](auto tag) __attribute__((always_inline)) {
+    constexpr int NB0 = decltype(tag)::value * NBP;
+    constexpr int CNT = EW_NB - NB0 < NBP ? EW_NB - NB0 : NBP;
+    static_assert(CNT >= 1, "a pass without blocks");
+    ew_f4v acc[EW_MB][CNT];
+#pragma unroll
+    for (int mb = 0; mb < EW_MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < CNT; ++nb) acc[mb][nb] = ew_f4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // step s multiplies with the operands fetched during step s - 1
+    float a[2][EW_MB], b[2][CNT];
+#pragma unroll
+    for (int mb = 0; mb < EW_MB; ++mb) a[0][mb] = As[abase[mb] + ew_k0[0]];
+#pragma unroll
+    for (int nb = 0; nb < CNT; ++nb) b[0][nb] = patch[base[NB0 + nb][ew_kpat[0]] + ew_koff[0]];
+#pragma unroll
+    for (int s = 0; s < EW_KSTEPS; ++s) {
+      if (s + 1 < EW_KSTEPS) {
+#pragma unroll
+        for (int mb = 0; mb < EW_MB; ++mb) a[(s + 1) & 1][mb] = As[abase[mb] + ew_k0[s + 1]];
+#pragma unroll
+        for (int nb = 0; nb < CNT; ++nb) b[(s + 1) & 1][nb] = patch[base[NB0 + nb][ew_kpat[s + 1]] + ew_koff[s + 1]];
+      }
+#pragma unroll
+      for (int nb = 0; nb < CNT; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < EW_MB; ++mb)
+#if EW_C_VEC == 4
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[s & 1][nb], a[s & 1][mb], acc[mb][nb], 0, 0, 0);     // C^T block
 #else
-    C[e] = acc[mb][nb][v];
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s & 1][mb], b[s & 1][nb], acc[mb][nb], 0, 0, 0);
 #endif
-  };
-#if defined(EH_EPILOGUE_SPLIT)
-  // in runs of blocks: everything the epilogue reads for a run is requested before the run's first store
-  constexpr int RUN = EH_EPILOGUE_SPLIT <= 1 ? 12 : EH_EPILOGUE_SPLIT <= 2 ? 6 : EH_EPILOGUE_SPLIT <= 4 ? 3 : 1;
+#if EW_MIX
+      // (one LDS read after every MFMA; the reads of A's values ride with the first ones)
 #pragma unroll
-  for (int mb = 0; mb < EW_MB; ++mb)
+      for (int q = 0; q < EW_MB; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
 #pragma unroll
-    for (int nb0 = 0; nb0 < EW_NB; nb0 += RUN) {
-      EhEpiLoads got[RUN][4];
-      long long at[RUN][4];
-#pragma unroll
-      for (int nb = nb0; nb < nb0 + RUN && nb < EW_NB; ++nb)
-        if (!M_EDGE && (nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
-            const int n = (nb * EW_WAVES_N + wn) * 16 + l16;
-            at[nb - nb0][v] = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
-            eh_epilogue_load(at[nb - nb0][v], got[nb - nb0][v] EH_EPI_ARGS);
-          }
-        }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int nb = nb0; nb < nb0 + RUN && nb < EW_NB; ++nb)
-        if (!M_EDGE && (nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
-#pragma unroll
-          for (int v = 0; v < 4; ++v) eh_epilogue_apply(at[nb - nb0][v], acc[mb][nb][v], got[nb - nb0][v] EH_C_ARG EH_EPI_ARGS);
-        }
+      for (int q = EW_MB; q < CNT * EW_MB; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+#endif
       __builtin_amdgcn_sched_barrier(0);
     }
+
+#if EW_C_VEC == 4
+    // The blocks were computed transposed: accumulator register v of lane l holds row l % 16 of the
+    // M-block, column 4 * (l / 16) + v of the N-block -- four rows of F in a row, next to each other
+    // in C and on a 16-byte boundary (the generator checked).  A lane finishes them together: what
+    // the epilogue reads is requested for a run of blocks before the run's first store goes out
+    // (loads and stores leave through one queue, in order: a load behind a store waits for it).
+#if defined(EH_EPILOGUE)
+    constexpr int RUN = 48 / EH_EPILOGUE_QUAD < 1 ? 1 : 48 / EH_EPILOGUE_QUAD;
 #else
-#pragma unroll
-  for (int mb = 0; mb < EW_MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < EW_NB; ++nb)
-      if (!M_EDGE && (nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) finish(mb, nb, v, false);
-      }
+    constexpr int RUN = 16;
 #endif
 #pragma unroll
-  for (int mb = 0; mb < EW_MB; ++mb)
+    for (int mb = 0; mb < EW_MB; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < EW_NB; ++nb)
-      if (M_EDGE || (nb + 1) * EW_WAVES_N * 16 > EW_NG) {
+      for (int nb0 = 0; nb0 < CNT; nb0 += RUN) {
+        long long at[RUN];
+        bool in[RUN];
+#if defined(EH_EPILOGUE)
+        EhEpiLoads4 got[RUN];
+#endif
 #pragma unroll
-        for (int v = 0; v < 4; ++v) finish(mb, nb, v, true);
+        for (int nb = nb0; nb < nb0 + RUN && nb < CNT; ++nb) {
+          const int m = (wm * EW_MB + mb) * 16 + l16;
+          const int n0 = ((NB0 + nb) * EW_WAVES_N + wn) * 16 + 4 * j4;
+          in[nb - nb0] = (!M_EDGE || m < EW_M) && ((NB0 + nb + 1) * EW_WAVES_N * 16 <= EW_NG || n0 < EW_NG);
+          at[nb - nb0] = c_base + ew_c_m(m < EW_M ? m : 0) + ew_c_n(g * EW_NG + (n0 < EW_NG ? n0 : 0));
+#if defined(EH_EPILOGUE)
+          if (in[nb - nb0]) eh_epilogue_load4(at[nb - nb0], got[nb - nb0] EH_EPI_ARGS);
+#endif
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = nb0; nb < nb0 + RUN && nb < CNT; ++nb)
+          if (in[nb - nb0]) {
+#if defined(EH_EPILOGUE)
+            const float four[4] = {acc[mb][nb][0], acc[mb][nb][1], acc[mb][nb][2], acc[mb][nb][3]};
+            eh_epilogue_apply4(at[nb - nb0], four, got[nb - nb0] EH_C_ARG EH_EPI_ARGS);
+#else
+            *reinterpret_cast<ew_f4v*>(C + at[nb - nb0]) = acc[mb][nb];
+#endif
+          }
+        __builtin_amdgcn_sched_barrier(0);
       }
+#else
+    // Accumulator register v of lane l holds row 4 * (l / 16) + v of the M-block, column l % 16 of the
+    // N-block.  Blocks that lie inside the group whole are finished without a test per element, in one
+    // run of straight-line code: whatever the epilogue loads (a bias, a saved activation) is then
+    // requested for all of them before the first store goes out, where a branch around every element
+    // would make each element's load wait for the stores of the one before (one queue for both).
+    auto finish = [&](const int mb, const int nb, const int v, const bool test) {
+      const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
+      const int n = ((NB0 + nb) * EW_WAVES_N + wn) * 16 + l16;
+      if (test && !(m < EW_M && n < EW_NG)) return;
+      const long long e = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
+#if defined(EH_EPILOGUE)
+      eh_epilogue(e, acc[mb][nb][v] EH_C_ARG EH_EPI_ARGS);
+#else
+      C[e] = acc[mb][nb][v];
+#endif
+    };
+#if defined(EH_EPILOGUE_SPLIT)
+    // in runs of blocks: everything the epilogue reads for a run is requested before the run's first store
+    constexpr int RUN = EH_EPILOGUE_SPLIT <= 1 ? 12 : EH_EPILOGUE_SPLIT <= 2 ? 6 : EH_EPILOGUE_SPLIT <= 4 ? 3 : 1;
+#pragma unroll
+    for (int mb = 0; mb < EW_MB; ++mb)
+#pragma unroll
+      for (int nb0 = 0; nb0 < CNT; nb0 += RUN) {
+        EhEpiLoads got[RUN][4];
+        long long at[RUN][4];
+#pragma unroll
+        for (int nb = nb0; nb < nb0 + RUN && nb < CNT; ++nb)
+          if (!M_EDGE && (NB0 + nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const int m = (wm * EW_MB + mb) * 16 + 4 * j4 + v;
+              const int n = ((NB0 + nb) * EW_WAVES_N + wn) * 16 + l16;
+              at[nb - nb0][v] = c_base + ew_c_m(m) + ew_c_n(g * EW_NG + n);
+              eh_epilogue_load(at[nb - nb0][v], got[nb - nb0][v] EH_EPI_ARGS);
+            }
+          }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = nb0; nb < nb0 + RUN && nb < CNT; ++nb)
+          if (!M_EDGE && (NB0 + nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) eh_epilogue_apply(at[nb - nb0][v], acc[mb][nb][v], got[nb - nb0][v] EH_C_ARG EH_EPI_ARGS);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#else
+#pragma unroll
+    for (int mb = 0; mb < EW_MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < CNT; ++nb)
+        if (!M_EDGE && (NB0 + nb + 1) * EW_WAVES_N * 16 <= EW_NG) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) finish(mb, nb, v, false);
+        }
+#endif
+#pragma unroll
+    for (int mb = 0; mb < EW_MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < CNT; ++nb)
+        if (M_EDGE || (NB0 + nb + 1) * EW_WAVES_N * 16 > EW_NG) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) finish(mb, nb, v, true);
+        }
+#endif
+  };
+  pass(EwInt<0>{});
+#if EW_PASSES > 1
+  pass(EwInt<1>{});
+#endif
+#if EW_PASSES > 2
+  pass(EwInt<2>{});
+#endif
+#if EW_PASSES > 3
+  pass(EwInt<3>{});
+#endif
 }

@@ -314,6 +314,19 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   bool a_vec = a_fast->w.side == WSide::K && a_fast->w.a == 1 && a_fast->unit == 1 && a_fast->w.extent % 4 == 0 && p.a_c0 % 4 == 0;
   for (const auto& l : loops)
     if (&l != a_fast && l.w.a % 4 != 0) a_vec = false;
+  // ... or all of k as one run (every k loop's stride in A is its weight in k): four k at once whatever the loops' extents
+  bool a_flat = !a_vec && K % 4 == 0 && p.a_c0 % 4 == 0;
+  for (const auto& l : loops) {
+    if (l.w.side == WSide::K) a_flat = a_flat && l.w.a == l.unit;
+    else a_flat = a_flat && l.w.a % 4 == 0;
+  }
+  if (a_flat) {
+    a_vec = true;
+    std::vector<const L*> ms;
+    for (const L* l : a_order)
+      if (l->w.side == WSide::M) ms.push_back(l);
+    a_order = ms;
+  }
   int64_t a_lds = kpad;
   {
     int64_t best = -1;
@@ -425,6 +438,28 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   const bool a_zero = mrows != M || kpad != K;            // padding rows / columns of A's tile must read as zero
   const int64_t a_elems = a_vec ? M * K / 4 : M * K;
 
+  // ---- four rows in a row of the group next to each other in C, on a 16-byte boundary? ------------------
+  // (then the product is computed transposed: a lane ends up with four consecutive rows of F for
+  // one row of A, and stores them as one vector)
+  bool c_quad = NG % 4 == 0 && p.c_c0 % 4 == 0 && !(epilogue && epilogue->quad_functions.empty());
+  {
+    auto c_of_n = [&](int64_t n) {
+      int64_t o = 0;
+      for (size_t q = first_in; q < row_loops.size(); ++q) o += ((n / loops[row_loops[q]].unit) % loops[row_loops[q]].w.extent) * loops[row_loops[q]].w.c;
+      return o;
+    };
+    for (int64_t n = 0; n + 3 < NG && c_quad; n += 4)
+      for (int64_t q = 0; q < 4; ++q) c_quad = c_quad && c_of_n(n) % 4 == 0 && c_of_n(n + q) == c_of_n(n) + q;
+    for (size_t q = 0; q < first_in; ++q) c_quad = c_quad && loops[row_loops[q]].w.c % 4 == 0;
+    for (size_t q : m_loops) c_quad = c_quad && loops[q].w.c % 4 == 0;
+    for (size_t q : batch_loops) c_quad = c_quad && loops[q].w.c % 4 == 0;
+  }
+
+  // ---- passes over k: at least six blocks each, so that a step's reads still hide behind its MFMAs -------
+  int passes = opt.window_passes > 0 ? opt.window_passes : static_cast<int>(std::min<int64_t>(4, std::max<int64_t>(1, int64_t{lay.nb} * lay.mb / 6)));
+  passes = std::max(1, std::min(passes, lay.nb));
+  while (passes > 1 && (lay.nb + passes - 1) / passes * (passes - 1) >= lay.nb) --passes;
+
   // ---- source ---------------------------------------------------------------------------------------
   std::ostringstream os;
   LaunchSpec ls;
@@ -440,12 +475,13 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   os << "#define EW_A_VEC " << (a_vec ? 1 : 0) << "\n#define EW_A_ELEMS " << a_elems << "\n#define EW_A_ZERO " << (a_zero ? 1 : 0)
      << "\n#define EW_KPAD " << kpad << "\n#define EW_A_LDS " << a_lds << "\n";
   os << "#define EW_SRC_BYTES " << p.f_bytes << "u\n";
-  os << "#define EW_MIX " << (opt.gemm_mix ? 1 : 0) << "\n";
+  os << "#define EW_MIX " << (opt.gemm_mix ? 1 : 0) << "\n#define EW_C_VEC " << (c_quad ? 4 : 1) << "\n#define EW_PASSES " << passes << "\n";
   if (epilogue) {
     os << "#define EH_EPILOGUE 1\n#define EH_EPI_PARAMS " << epilogue->params << "\n#define EH_EPI_ARGS " << epilogue->args << "\n";
     if (!epilogue->store_c) os << "#define EH_NO_C 1\n";
     os << epilogue->function;
     if (!epilogue->split_functions.empty()) os << "#define EH_EPILOGUE_SPLIT " << epilogue->n_loads << "\n" << epilogue->split_functions;
+    if (c_quad) os << "#define EH_EPILOGUE_QUAD " << std::max(1, epilogue->quad_regs) << "\n" << epilogue->quad_functions;
   }
   auto table = [&](const char* name, const std::vector<int64_t>& vals) {
     os << "constexpr int " << name << "[" << vals.size() << "] = {";
@@ -520,9 +556,13 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
     os << "__device__ __forceinline__ void ew_a_elem(int e, long long bz, int* lds, long long* off) {\n";
     os << "  const unsigned u = (unsigned)e, ub = (unsigned)bz;\n  (void)u; (void)ub;\n  long long o = " << p.a_c0 << "LL;\n  int m = 0, k = 0;\n";
     int64_t radix = 1;
+    if (a_flat) {
+      os << "  {\n    const int d = (int)(u % " << K / 4 << "u) * 4;\n    o += d;\n    k += d;\n  }\n";
+      radix = K / 4;
+    }
     for (size_t i = a_order.size(); i-- > 0;) {
       const L* l = a_order[i];
-      const bool quad = a_vec && l == a_fast;
+      const bool quad = a_vec && !a_flat && l == a_fast;
       const int64_t ext = quad ? l->w.extent / 4 : l->w.extent;
       os << "  {\n    const int d = (int)((u / " << radix << "u) % " << ext << "u)" << (quad ? " * 4" : "") << ";\n";
       os << "    o += (long long)d * " << l->w.a << "LL;\n";
@@ -552,7 +592,7 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   ls.schedule = "mfma16x16x4(window,group=" + std::to_string(NG) + ",M=" + std::to_string(M) + ",K=" + std::to_string(K) +
                 ",waves=" + std::to_string(lay.waves_m) + "x" + std::to_string(lay.waves_n) + ",blocks=" + std::to_string(lay.mb) +
                 "x" + std::to_string(lay.nb) + ",steps=" + std::to_string(ksteps) + ",patterns=" + std::to_string(patterns.size()) +
-                ",lds=" + std::to_string((patch_floats + mrows * a_lds) * 4) + "B" + p.tag +
+                ",lds=" + std::to_string((patch_floats + mrows * a_lds) * 4) + "B" + (c_quad ? ",C:x4" : "") + (passes > 1 ? ",passes=" + std::to_string(passes) : std::string()) + p.tag +
                 (epilogue ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
   ls.grid[0] = static_cast<unsigned>(groups);
   ls.grid[1] = 1;

@@ -92,7 +92,7 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      (src/backend/renderer.rs:20-35; KernelSourceRenderer and extract_kernel_config,
  *      src/backend/pipeline.rs:27-33, 344-410).  `options` is NULL or "key=value,..." with keys
  *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
- *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold, gemm_window,
+ *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold, gemm_window, window_passes,
  *      gemm_epilogue, gemm_dma, gemm_mix, gemm_prefetch, gemm_transpose, gemm_merge_batch, nontemporal,
  *      normalize, allow_serial, reindex, rematerialize, merge_launches, guard_branches, ranged_loads, lanes, lane_us.
  *      lanes (default 1; 2 or more): launches of a program that do not depend on each other are spread

@@ -848,10 +848,33 @@ def test_convolution_input_gradient_is_one_window_contraction(frontend):
     gone = {b["name"] for b in plan.buffers if b["elided"]}
     assert len(gone & {"buf%d" % q for q in range(145, 161, 2)}) == 8 and out not in gone
     assert len(hb.compile_source(dx["source"])) > 1000
-    assert len(plan.launches) == 22
-    # a result that is a program output is computed everywhere
+    # without the LDS-staged schedules the product and the shifted sums are two launches
     off = hb.render_program(ast, "gemm_window=0")
-    assert not any("shifts=" in l["schedule"] for l in off.launches) and len(off.launches) == 23
+    assert not any("shifts=" in l["schedule"] for l in off.launches) and len(off.launches) == len(plan.launches) + 1
+
+
+def test_loss_bookkeeping_joins_the_launch_it_continues(frontend):
+    """The roots of a training step are lowered one after another, so what is left of the loss's
+    value (a few kernels on [batch] and [batch, classes]) comes behind a hundred kernels of the
+    gradients.  Those kernels carry on with the rows of the log-softmax launch and nothing in
+    between touches their buffers: they join that launch (their own launch goes), and the last
+    of them, the sum over the batch, depends on nothing later and is issued with the other final
+    launches."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+    arrays = wl.config5_inputs(*wl.cnn_sizes(True))
+    ts = [Tensor.input(list(a.shape)) for a in arrays]
+    ast = wl.lower_multi(ts, wl.config5_graph(*ts, lr=1e-2))[0]
+    plan = hb.render_program(ast)
+    (rows,) = [l for l in plan.launches if l["entry"] == "ehk_R_256_1_28"]
+    assert {"E_256_109", "E_256_10_110", "R_256_1_111"} <= set(rows["kernels"]), rows["kernels"]
+    assert rows["kernels"].index("E_256_109") > rows["kernels"].index("E_256_10_43")
+    assert sum("R_256_1_111" in l["kernels"] for l in plan.launches) == 1
+    (total,) = [l for l in plan.launches if "R_1_112" in l["kernels"]]
+    assert total["schedule"].startswith("together(") and plan.launches.index(total) > plan.launches.index(rows)
+    assert len(plan.launches) == 20
+    apart = hb.render_program(ast, "merge_launches=0")
+    assert not any("E_256_109" in l["kernels"] and "R_256_1_28" in l["kernels"] for l in apart.launches)
 
 
 def test_convolution_rows_run_across_images(frontend):
