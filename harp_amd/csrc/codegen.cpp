@@ -2312,23 +2312,49 @@ void issue_independent_launches_together(ProgramPlan* plan, const std::vector<co
     return false;
   };
   std::vector<LaunchSpec> in = std::move(plan->launches), out, held;
-  auto flush = [&] {
+  std::vector<char> taken(in.size(), 0);       // pulled forward into an earlier launch
+  // The held launches of every workgroup size that has one in the way of `trigger` (all of them
+  // at the end) go out as one launch per size.  Each takes along what further down the list could
+  // run here just as well: launches of its size that depend on nothing between here and there
+  // (the final launches of a training step, which nothing reads, were put at the end of the list).
+  auto flush = [&](size_t next, const LaunchSpec* trigger) {
     std::map<unsigned, std::vector<LaunchSpec>> by_block;
-    for (auto& ls : held) by_block[ls.block[0]].push_back(std::move(ls));
-    held.clear();
+    std::vector<LaunchSpec> stay;
+    std::set<unsigned> go;
+    for (const auto& h : held)
+      if (!trigger || conflict(*trigger, h)) go.insert(h.block[0]);
+    for (auto& h : held) {
+      if (go.count(h.block[0])) by_block[h.block[0]].push_back(std::move(h));
+      else stay.push_back(std::move(h));
+    }
+    held = std::move(stay);
     for (auto& kv : by_block) {
+      for (size_t q = next; q < in.size(); ++q) {
+        if (taken[q] || in[q].block[0] != kv.first || !mergeable(in[q])) continue;
+        bool free_to_move = true;
+        for (size_t p = next; p < q && free_to_move; ++p) free_to_move = taken[p] || !conflict(in[q], in[p]);
+        for (const auto& h : held) free_to_move = free_to_move && !conflict(in[q], h);
+        for (const auto& g : by_block)
+          for (const auto& m : g.second) free_to_move = free_to_move && !conflict(in[q], m);
+        if (!free_to_move) continue;
+        kv.second.push_back(std::move(in[q]));
+        taken[q] = 1;
+      }
       if (kv.second.size() >= 2) out.push_back(merge_launches(kv.second, opt));
       else out.push_back(std::move(kv.second.front()));
     }
   };
-  for (auto& ls : in) {
+  for (size_t q = 0; q < in.size(); ++q) {
+    if (taken[q]) continue;
+    LaunchSpec& ls = in[q];
     bool dep = false;
     for (const auto& h : held) dep = dep || conflict(ls, h);
-    if (dep) flush();
+    if (dep) flush(q, &ls);
     if (mergeable(ls)) held.push_back(std::move(ls));
     else out.push_back(std::move(ls));
+    taken[q] = 1;
   }
-  flush();
+  flush(in.size(), nullptr);
   plan->launches = std::move(out);
 }
 
@@ -3547,15 +3573,10 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     }
     plan.launches.push_back(emit_group(g, opt, elems));
   }
-  {
-    // by workgroup size: a part's surplus work-items leave at once, but they are launched all the same
-    std::map<unsigned, std::vector<LaunchSpec>> by_block;
-    for (auto& ls : held_back) by_block[ls.block[0]].push_back(std::move(ls));
-    for (auto& kv : by_block) {
-      if (kv.second.size() >= 2) plan.launches.push_back(merge_launches(kv.second, opt));
-      else plan.launches.push_back(std::move(kv.second.front()));
-    }
-  }
+  // what was held back goes to the end one by one: the pass that issues independent launches together
+  // (below) merges it with whatever else is still waiting there, by workgroup size (a part's surplus
+  // work-items leave at once, but they are launched all the same)
+  for (auto& ls : held_back) plan.launches.push_back(std::move(ls));
   // constant inputs no launch binds any more need not exist
   for (const auto& c : consts) {
     bool bound = false;

@@ -755,11 +755,14 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert len(cols) == 1, [l["schedule"] for l in plan.launches]
     temp = cols[0]["args"][-1]
     (reader,) = [l for l in plan.launches if temp in l["args"] and l is not cols[0]]
-    body = reader["source"][reader["source"].index("__global__"):]
+    # (the reader may have gone out together with an independent launch: its part of the source then)
+    src = reader["source"]
+    body = src[src.rindex("\n", 0, src.index("eh_rs_" + temp)):]
+    body = body[:body.index("}  // namespace")] if "}  // namespace" in body else body
     assert body.count("eh_ranged_load(eh_rs_" + temp + ",") == 9   # guarded loads: out of range where the guard fails
     assert "if (" not in body.replace("if (eh_", "") and temp + "[" not in body
     clamped = hb.render_program(ast, "lanes=1,ranged_loads=0,gemm_window=0")
-    (reader0,) = [l for l in clamped.launches if l["entry"] == reader["entry"]]
+    (reader0,) = [l for l in clamped.launches if temp in l["args"] and not l["schedule"].startswith("mfma")]
     assert reader0["source"].count(temp + "[") == 9             # ... or a clamped index and a select
     plain = hb.render_program(ast, "lanes=1,reindex=0")
     assert not any("A:m,B:n,B:source" in l["schedule"] for l in plain.launches)
@@ -872,7 +875,7 @@ def test_loss_bookkeeping_joins_the_launch_it_continues(frontend):
     assert sum("R_256_1_111" in l["kernels"] for l in plan.launches) == 1
     (total,) = [l for l in plan.launches if "R_1_112" in l["kernels"]]
     assert total["schedule"].startswith("together(") and plan.launches.index(total) > plan.launches.index(rows)
-    assert len(plan.launches) == 20
+    assert len(plan.launches) == 19
     apart = hb.render_program(ast, "merge_launches=0")
     assert not any("E_256_109" in l["kernels"] and "R_256_1_28" in l["kernels"] for l in apart.launches)
 
