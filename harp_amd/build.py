@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libeclat_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
-SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "gemm.cpp", "window.cpp", "backend.cpp", "capi.cpp"]
+SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "stages.cpp", "rewrites.cpp", "plan.cpp", "emitters.cpp", "launches.cpp", "gemm.cpp", "window.cpp", "backend.cpp", "capi.cpp"]
 # compiled as HIP for gfx950: holds the library's one statically allocated device array
 DEVICE_SOURCES = ["static_scratch.hip"]
 TEMPLATES = ["kernels/gemm_f32_mfma.hip", "kernels/window_f32_mfma.hip"]
@@ -112,7 +112,7 @@ def build_capi_client() -> str:
 
 FUZZ_SRC = os.path.join(os.path.dirname(HERE), "tests", "host_fuzz.cpp")
 FUZZ = os.path.join(os.path.dirname(HERE), "tests", "host_fuzz.bin")
-GENERATOR_SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "gemm.cpp", "window.cpp"]   # no HIP runtime involved
+GENERATOR_SOURCES = ["ast.cpp", "analysis.cpp", "normalize.cpp", "codegen.cpp", "stages.cpp", "rewrites.cpp", "plan.cpp", "emitters.cpp", "launches.cpp", "gemm.cpp", "window.cpp"]   # no HIP runtime involved
 
 
 def build_host_fuzz(force: bool = False) -> str:

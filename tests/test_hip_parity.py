@@ -1468,7 +1468,7 @@ def test_random_graphs_with_few_long_lines_match_the_oracle(frontend, hip, seed,
             assert np.allclose(got, ref, rtol=rtol, atol=rtol / 10 * scale), (desc, fuse)
 
 
-@pytest.mark.parametrize("seed", range(400, 405))
+@pytest.mark.parametrize("seed", range(400, 420))
 def test_random_small_cnns_match_the_oracle(frontend, hip, seed):
     """Random conv + pool + linear classifiers (tests/graph_fuzz.py): forward with the fused
     and the per-kernel path, then every gradient of the summed output in exact mode."""
@@ -1539,9 +1539,28 @@ def test_convolution_input_gradients_as_one_window_contraction(frontend, hip, xs
         assert np.allclose(g, r, rtol=1e-4, atol=1e-5 * scale)
 
 
-def _grads_on(fe, kind, shapes, fn, arrays):
+@pytest.mark.parametrize("seed", range(430, 438))
+def test_random_small_cnn_training_steps_match_the_oracle(frontend, hip, seed):
+    """The same random classifiers as one SGD step: every input after `x - 0.05 * dloss/dx` and
+    the loss, realized together (as many roots as inputs plus one)."""
+    import graph_fuzz
+    shapes, fn, desc = graph_fuzz.build_cnn(seed, frontend)
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1, 1, s).astype(np.float32) for s in shapes]
+    ref = _grads_on(frontend, "c", shapes, fn, arrays, lr=0.05)
+    got = _grads_on(frontend, "hip", shapes, fn, arrays, lr=0.05)
+    assert ref is not None and len(ref) == len(got) == len(shapes) + 1, desc
+    for r, g in zip(ref, got):
+        assert r.shape == g.shape, desc
+        scale = max(1.0, float(np.abs(r).max()))
+        close = np.isclose(g, r, rtol=1e-4, atol=1e-5 * scale)
+        assert int((~close).sum()) <= (2 if "pool True" in desc else 0), desc
+
+
+def _grads_on(fe, kind, shapes, fn, arrays, lr=None):
     """Exact-mode gradients of sum(fn(inputs)) with respect to every input, plus the sum,
-    realized together.  Returns None when the graph uses an op without an exact VJP."""
+    realized together (with `lr`: the inputs after a gradient step instead of the gradients).
+    Returns None when the graph uses an op without an exact VJP."""
     from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
     fe.set_device_str(kind)
     try:
@@ -1558,7 +1577,10 @@ def _grads_on(fe, kind, shapes, fn, arrays):
                 loss.backward_with_params(ts)
             except NotImplementedError:
                 return None
-            roots = [t.grad().contiguous() for t in ts if t.grad() is not None] + [loss]
+            if lr is None:
+                roots = [t.grad().contiguous() for t in ts if t.grad() is not None] + [loss]
+            else:
+                roots = [(t - t.grad().scale_exact(lr)).contiguous() for t in ts if t.grad() is not None] + [loss]
             fe.realize_many(roots)
             return [r.to_numpy() for r in roots]
     finally:
