@@ -21,7 +21,8 @@ from typing import Dict, List, Optional, Sequence
 
 from .ast import AstNode
 from .expr import Expr
-from .graph import GraphNode, ones, topological_sort, zeros
+from .graph import GraphNode, GraphOp, ones, topological_sort, zeros
+from .view import View
 
 
 class GradContext:
@@ -320,8 +321,18 @@ def _matmul_vjp(node, g, transpose) -> List[Optional[GraphNode]]:
 # exact VJPs (not in the reference)
 # ---------------------------------------------------------------------------
 
+def _dense_unary(g: GraphNode, f) -> GraphNode:
+    """f(g) stored contiguously.  `unary_op` hands its operand's view to the result, and
+    the lowerer stores through the result's view: over a slice that writes past a buffer
+    sized by the shape, over a broadcast it writes one element many times."""
+    if g.view.is_contiguous():
+        return g.unary_op(f)
+    return GraphNode([g], View.contiguous(g.shape()),
+                     GraphOp("map_reduce", map=f(AstNode.wildcard("0")), reduce=None), g.dtype)
+
+
 def _scaled(g: GraphNode, c: float) -> GraphNode:
-    return g.unary_op(lambda x: AstNode.mul(x, AstNode.const_f32(c)))
+    return _dense_unary(g, lambda x: AstNode.mul(x, AstNode.const_f32(c)))
 
 
 def _dense(n: GraphNode) -> GraphNode:

@@ -152,9 +152,13 @@ class Tensor:
 
     def scale_exact(self, factor: float) -> "Tensor":
         """x * factor as a literal in the map (not in the reference, whose `scale`
-        ignores the factor)."""
+        ignores the factor).  The result is dense: a unary op keeps its operand's view
+        (ops.rs:255-274) and the lowerer stores through that view, which for a slice of a
+        larger buffer (the gradient of a padded input) indexes past a result sized by its
+        shape -- neither the reference's backend-c nor the oracle checks that."""
         from .ast import AstNode
-        return Tensor(self.graph.unary_op(lambda x: AstNode.mul(x, AstNode.const_f32(factor))))
+        from .grad import _dense_unary
+        return Tensor(_dense_unary(self.graph, lambda x: AstNode.mul(x, AstNode.const_f32(factor))))
 
     # -- reductions (the reduced axis is squeezed away) ------------------------------
     def _check_axis(self, axis):

@@ -108,7 +108,7 @@ class CKernel:
         self._fn(*ptrs)
 
 
-def compile_program_text(ast_text: str, openmp: bool = False) -> CKernel:
+def compile_program_text(ast_text: str, openmp: bool = False, gcc_args: Optional[Sequence[str]] = None) -> CKernel:
     """One Program holding one kernel -> a callable (lib.rs:50-112)."""
     tree = parse(ast_text)
     kernels = [x for x in tree[1:] if isinstance(x, list) and x[0] == "kernel"]
@@ -119,15 +119,22 @@ def compile_program_text(ast_text: str, openmp: bool = False) -> CKernel:
     src = render_program(ast_text)
     if openmp:
         src = _add_openmp_pragmas(src)
-    return CKernel(src, str(k[1]), nptr, openmp=openmp)
+    return CKernel(src, str(k[1]), nptr, openmp=openmp, gcc_args=gcc_args)
 
 
 class CBackend:
     """Plugs into `harp_amd.frontend.device.register_backend` from tests."""
 
-    def __init__(self, openmp: bool = False):
-        self.kind = "openmp" if openmp else "c"
+    def __init__(self, openmp: bool = False, exact_division: bool = False):
+        """`exact_division`: the reference's flags (-O3 -ffast-math, compiler.rs:153-165) plus
+        -mno-recip, device kind "c-exactdiv".  Under -ffast-math gcc divides floats in a vectorised
+        loop with rcpps and one Newton-Raphson step, in a scalar loop with divss: the same
+        `1.0f / x` then differs in its last bit between two kernels of one program, and a test for
+        equality between a value and its recomputation (the gradient of max / min goes to the
+        elements equal to it) fails where it should hold.  Tests of such gradients use this kind."""
+        self.kind = "c-exactdiv" if exact_division else "openmp" if openmp else "c"
         self.openmp = openmp
+        self.gcc_args = list(GCC_ARGS) + ["-mno-recip"] if exact_division else None
         self._devices = {}
 
     def name(self) -> str:
@@ -146,4 +153,4 @@ class CBackend:
         return CBuffer(shape, dtype)
 
     def compile_ast(self, device, program, signature=None) -> CKernel:
-        return compile_program_text(program.to_sexpr(), openmp=self.openmp)
+        return compile_program_text(program.to_sexpr(), openmp=self.openmp, gcc_args=self.gcc_args)

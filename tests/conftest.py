@@ -20,6 +20,7 @@ def frontend():
     from oracle.c_backend import CBackend
     fe.register_backend(CBackend())
     fe.register_backend(CBackend(openmp=True))
+    fe.register_backend(CBackend(exact_division=True))
     return fe
 
 

@@ -1427,19 +1427,28 @@ def test_out_of_bounds_reader_of_a_materialised_unfold_is_refused(frontend, hip)
         realize_on(frontend, "hip", lambda t: t.unfold([1], [2], [2], [1]).contiguous().max(2), [x])
 
 
-@pytest.mark.parametrize("seed", range(5000, 5012))
+@pytest.mark.parametrize("seed", range(5000, 5020))
 def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
     """The same generator with one or two axes of up to 2048 elements: vectorised accesses,
-    rows held in registers or LDS, multi-block reductions, MFMA contractions with edges."""
-    import graph_fuzz
+    rows held in registers or LDS, multi-block reductions, MFMA contractions with edges.
+    The tolerance is per element and follows the arithmetic (tests/np_frontend.py: a float64
+    evaluation of the same graph with a running bound on what float32 rounding can do to it,
+    sums counted with their condition): two float32 evaluations may differ by twice the bound.
+    A sum of 2048 values that nearly cancel (seed 5012: -0.30470 from terms of size 1) is judged
+    by sum|x|, everything well conditioned more tightly than a fixed relative tolerance would."""
+    import graph_fuzz, np_frontend
     shapes, fn, desc = graph_fuzz.build(seed, frontend, dims=graph_fuzz.LARGE_DIMS, max_rank=2)
+    _, fn64, _ = graph_fuzz.build(seed, np_frontend.Frontend, dims=graph_fuzz.LARGE_DIMS, max_rank=2)
     rng = RNG(seed)
     arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    exact, bound = np_frontend.evaluate(fn64, arrays)
     for fuse in (True, False):
         ref, got = both(frontend, fn, arrays, fuse)
-        assert ref.shape == got.shape, desc
-        scale = max(1.0, float(np.abs(ref).max()))
-        assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), (desc, fuse)
+        assert ref.shape == got.shape and ref.size == exact.size, desc
+        exact, bound = exact.reshape(ref.shape), bound.reshape(ref.shape)
+        tol = 2.0 * bound + 4 * np_frontend.U * np.abs(exact)
+        assert np.all(np.abs(got.astype(np.float64) - ref) <= tol), (desc, fuse, float(np.max(np.abs(got.astype(np.float64) - ref) / tol)))
+        assert np.all(np.abs(got.astype(np.float64) - exact) <= 0.5 * tol + 2 * np_frontend.U * np.abs(exact)), (desc, fuse)
 
 
 LONG_LINE_SEEDS = [(7007, 0), (7052, 0), (7084, 0), (7092, 0), (7229, 0), (7264, 0), (7282, 0), (7284, 0), (7296, 0),
@@ -1587,15 +1596,19 @@ def _grads_on(fe, kind, shapes, fn, arrays, lr=None):
         _INPUT_BUFFER_CACHE.clear()
 
 
-@pytest.mark.parametrize("seed", range(200, 232))
+@pytest.mark.parametrize("seed", list(range(200, 232)) + [392])
 def test_random_graph_gradients_match_the_oracle(frontend, hip, seed):
     """The same random graphs, differentiated: loss = sum of the output, exact-mode VJPs,
-    all gradients and the loss as roots of one Program.  HIP against the C oracle."""
+    all gradients and the loss as roots of one Program.  HIP against the C oracle -- compiled
+    with the reference's flags and -mno-recip (kind "c-exactdiv"): the gradient of a max / min
+    tests a value for equality with its recomputation in another kernel, and gcc's vectorised
+    reciprocal under -ffast-math breaks that equality inside the oracle itself (seed 392: eleven
+    of 24 rows lose their gradient; tests/test_oracle_golden.py shows it without a GPU)."""
     import graph_fuzz
     shapes, fn, desc = graph_fuzz.build(seed, frontend)
     rng = RNG(seed)
     arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
-    ref = _grads_on(frontend, "c", shapes, fn, arrays)
+    ref = _grads_on(frontend, "c-exactdiv", shapes, fn, arrays)
     if ref is None:
         pytest.skip("graph uses an op without an exact VJP: " + desc)
     got = _grads_on(frontend, "hip", shapes, fn, arrays)

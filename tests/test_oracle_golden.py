@@ -494,3 +494,94 @@ def test_parameter_and_layer_api(frontend):
         Parameter.from_data("q", [1, 2, 3], [2, 2])
     with pytest.raises(frontend.optim.OptimError):
         frontend.optim.SGD([p], 0.1).step()              # no gradient yet
+
+
+def test_float64_mirror_bounds_the_oracle(frontend):
+    """tests/np_frontend.py evaluates the random graphs of tests/graph_fuzz.py in float64 and
+    carries a bound on what float32 rounding can do to every value.  The oracle's float32
+    results lie within that bound (small graphs, and large ones with sums of up to 2048 terms,
+    among them seed 5012 whose sum nearly cancels: float64 -0.304704, the oracle -0.304749, a
+    relative difference of 1.5e-4 that a fixed tolerance of 2e-5 called a failure), and for well
+    conditioned graphs the bound is tight: below 1e-5 of the value for most elements."""
+    import graph_fuzz, np_frontend
+    fe = frontend
+    fe.set_device_str("c")
+    tight, total = 0, 0
+    cases = [(s, {}) for s in range(0, 24)] + [(s, dict(dims=graph_fuzz.LARGE_DIMS, max_rank=2)) for s in range(5000, 5020)]
+    for seed, kw in cases:
+        shapes, fn, desc = graph_fuzz.build(seed, fe, **kw)
+        _, fn64, _ = graph_fuzz.build(seed, np_frontend.Frontend, **kw)
+        rng = np.random.default_rng(seed)
+        arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+        exact, bound = np_frontend.evaluate(fn64, arrays)
+        ts = []
+        for a in arrays:
+            t = fe.Tensor.input(list(a.shape))
+            t.set_data(a)
+            ts.append(t)
+        out = fn(*ts).contiguous()
+        fe.realize_many([out])
+        got = out.to_numpy().astype(np.float64)
+        assert got.size == exact.size, desc
+        got = got.reshape(exact.shape)
+        assert np.all(np.abs(got - exact) <= bound + 2 * np_frontend.U * np.abs(exact)), (desc, float(np.max(np.abs(got - exact) / np.maximum(bound, 1e-300))))
+        rel = bound / np.maximum(np.abs(exact), 1e-30)
+        tight += int((rel < 1e-5).sum())
+        total += rel.size
+        if seed == 5012:
+            assert abs(float(exact) + 0.3047036) < 1e-6 and abs(float(got) - float(exact)) > 2e-5 * abs(float(exact))
+    assert tight > 0.9 * total, (tight, total)
+
+
+def test_fast_math_reciprocal_differs_between_kernels_of_the_oracle(frontend):
+    """With the reference's flags (-O3 -ffast-math, compiler.rs:153-165) gcc computes `1.0f / x`
+    with rcpps and a Newton-Raphson step where it vectorises the loop and with divss where it
+    does not: in the gradient of sum(min(sigmoid(max(x, y) * y), axis)) (tests/graph_fuzz.py,
+    seed 392) the kernel that takes the minimum and the kernel that recomputes the values
+    disagree in the last bit, the VJP's test for equality fails, and whole rows get no gradient.
+    With -mno-recip on top (kind "c-exactdiv") every row has exactly one element with a gradient,
+    the one float64 numpy finds as the minimum."""
+    import graph_fuzz
+    from test_hip_parity import _grads_on
+    shapes, fn, desc = graph_fuzz.build(392, frontend)
+    rng = np.random.default_rng(392)
+    x, y = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    dx, dy, loss = _grads_on(frontend, "c-exactdiv", shapes, fn, [x, y])
+    s64 = 1.0 / (1.0 + np.exp(-(np.maximum(x, y).astype(np.float64) * y)))
+    where = s64.reshape(24, 5).argmin(1)
+    rows = dy.reshape(24, 5)
+    assert [list(np.nonzero(r)[0]) for r in rows] == [[int(k)] for k in where]
+    assert abs(float(loss[0]) - s64.min(2).sum()) < 1e-5
+    fast = _grads_on(frontend, "c", shapes, fn, [x, y])
+    if not np.array_equal(fast[1], dy):         # (a compiler that does not vectorise the loop shows nothing)
+        assert sum(1 for r in fast[1].reshape(24, 5) if not r.any()) >= 1
+        for r_fast, r_exact in zip(fast[1].reshape(24, 5), rows):
+            assert (not r_fast.any()) or np.allclose(r_fast, r_exact, rtol=1e-6)
+
+
+def test_scaling_the_gradient_of_a_padded_input_stores_densely(frontend):
+    """A unary op keeps its operand's view (ops.rs:255-274) and the lowerer stores through the
+    result's view.  The gradient of a padded input is a slice of the padded gradient: scaled
+    as-is it would be stored at the slice's strides, past a result that is sized by its shape
+    (backend-c and the oracle check nothing).  `scale_exact` and the exact VJPs' scale store
+    densely instead; every store of the lowered step stays inside its buffer and the step has
+    the values calculus gives."""
+    from harp_amd.frontend.tensor import _INPUT_BUFFER_CACHE
+    frontend.set_device_str("c")
+    rng = np.random.default_rng(5)
+    x0 = rng.uniform(-1, 1, (3, 5)).astype(np.float32)
+    w0 = rng.uniform(-1, 1, (5, 9)).astype(np.float32)
+    try:
+        with frontend.exact_mode():
+            x, w = frontend.Tensor.input([3, 5]), frontend.Tensor.input([5, 9])
+            x.set_data(x0), w.set_data(w0)
+            loss = (x.pad([(1, 1), (2, 2)]) * w).sum(1).sum(0)
+            loss.backward_with_params([x, w])
+            assert not x.grad().graph.view.is_contiguous()          # the slice of the padded gradient
+            step = x - x.grad().scale_exact(0.25)
+            assert x.grad().scale_exact(0.25).graph.view.is_contiguous()
+            frontend.realize_many([step])
+            got = step.to_numpy().reshape(3, 5)
+    finally:
+        _INPUT_BUFFER_CACHE.clear()
+    assert np.array_equal(got, x0 - np.float32(0.25) * w0[1:4, 2:7])
