@@ -36,6 +36,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--options", default="")
+    ap.add_argument("--no-tuned", action="store_true", help="do not load harp_amd/tuned_gfx950.txt")
     ap.add_argument("--sets", type=int, default=4)
     ap.add_argument("--only", default="", help="softmax | matmul | config1 | mlp | cnn (default: all)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -59,6 +60,12 @@ def main():
     log(f"[bench] device: {props['name']} {props['arch']} CUs={props['compute_units']} "
         f"clock={props['clock_khz'] / 1e6:.2f} GHz LDS/CU={props['local_memory_size']}")
     options = args.options or None
+    # what the measured schedule search filed for gfx950 (programs and single launches, by key) applies
+    # unless the caller names another file; explicit --options still go on top
+    tuned_file = os.environ.get("ECLAT_HIP_TUNE", "")
+    shipped = os.path.join(os.path.dirname(os.path.abspath(hb.__file__)), "tuned_gfx950.txt")
+    if not tuned_file and os.path.exists(shipped) and not args.no_tuned:
+        os.environ["ECLAT_HIP_TUNE"] = tuned_file = shipped
     want = lambda n: not args.only or args.only == n
     extra = {}
 
@@ -336,7 +343,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic (seeded N(0, std 2) fp32 [4096,4096])",
         "config": {"workload": "config2: row softmax fp32 [4096,4096], one fused launch",
-                   "buffer_sets": args.sets, "options": args.options},
+                   "buffer_sets": args.sets, "options": args.options,
+                   "tuned_options_file": os.path.relpath(tuned_file, os.path.dirname(os.path.abspath(__file__))) if tuned_file else None},
     }
     each_note = ("one HIP event pair per launch on the launch stream, same buffer rotation; the events sit between "
                  "launches, so ms_mean can exceed ms_per_step, which is measured over launches queued back to back")

@@ -23,6 +23,7 @@ pub struct eh_launch_info {
     pub flops: f64,
     pub lane: c_int,
     pub n_waits: c_int,
+    pub tune_key: std::os::raw::c_ulonglong,
 }
 
 #[repr(C)]

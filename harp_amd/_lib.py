@@ -45,7 +45,7 @@ class LaunchInfo(Structure):
     _fields_ = [("entry", c_char_p), ("source", c_char_p), ("schedule", c_char_p),
                 ("grid", c_uint * 3), ("block", c_uint * 3), ("lds_bytes", c_uint),
                 ("n_args", c_int), ("n_kernels", c_int), ("algo_bytes", c_double),
-                ("flops", c_double), ("lane", c_int), ("n_waits", c_int)]
+                ("flops", c_double), ("lane", c_int), ("n_waits", c_int), ("tune_key", ctypes.c_ulonglong)]
 
 
 _P = c_void_p
@@ -58,6 +58,7 @@ _SIGS = {
     "eh_device_close": ([_P], c_int),
     "eh_device_get_props": ([_P, POINTER(DeviceProps)], c_int),
     "eh_device_sync": ([_P], c_int),
+    "eh_device_stream": ([_P, POINTER(c_void_p)], c_int),
     "eh_device_trim": ([_P, POINTER(c_size_t)], c_int),
     "eh_buffer_alloc": ([_P, c_size_t, POINTER(_P)], c_int),
     "eh_buffer_retain": ([_P], c_int),

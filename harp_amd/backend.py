@@ -35,7 +35,7 @@ def _launch_dict(info: LaunchInfo) -> dict:
             "schedule": info.schedule.decode(), "grid": list(info.grid),
             "block": list(info.block), "lds_bytes": info.lds_bytes, "n_args": info.n_args,
             "n_kernels": info.n_kernels, "algo_bytes": info.algo_bytes, "flops": info.flops,
-            "lane": info.lane, "n_waits": info.n_waits}
+            "lane": info.lane, "n_waits": info.n_waits, "tune_key": "%016x" % info.tune_key}
 
 
 # ---------------------------------------------------------------------------

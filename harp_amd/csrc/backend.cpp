@@ -420,95 +420,47 @@ void HipKernel::launch(const unsigned grid[3], const unsigned block[3], unsigned
 // ---------------------------------------------------------------------------------------------
 
 unsigned long long tune_key(const char* ast_text) {
-  unsigned long long h = 1469598103934665603ull;
-  for (const unsigned char* p = reinterpret_cast<const unsigned char*>(ast_text); *p; ++p) {
-    h ^= *p;
-    h *= 1099511628211ull;
+  // of the canonical text, so that spacing and the like do not matter; text that does not parse is hashed as it is
+  std::string text = ast_text ? ast_text : "";
+  try {
+    text = to_text(*parse_ast(text));
+  } catch (const Error&) {
   }
-  return h;
+  return fnv1a(text);
 }
 
 GenOptions options_for(const char* ast_text, const char* options) {
   const char* path = std::getenv("ECLAT_HIP_TUNE");
   if (!path || !*path || !ast_text) return parse_options(options);
+  std::ifstream f(path);
+  if (!f) {
+    static std::once_flag warned;
+    std::call_once(warned, [&] { std::fprintf(stderr, "eclat backend-hip: cannot read the tuned-options file '%s' (ECLAT_HIP_TUNE); defaults are used\n", path); });
+    return parse_options(options);
+  }
   char key[17];
   std::snprintf(key, sizeof key, "%016llx", tune_key(ast_text));
-  std::ifstream f(path);
   std::string line, tuned;
+  std::map<std::string, std::string> others;        // lines under other keys: a launch's, if this program has such a launch
   while (std::getline(f, line)) {
     const size_t hash = line.find('#');
     if (hash != std::string::npos) line.resize(hash);
     std::istringstream ls(line);
     std::string k, v;
-    if (ls >> k >> v && k == key) tuned = v;          // the last entry for a key counts
+    if (!(ls >> k >> v)) continue;
+    if (k == key) tuned = v;                          // the last entry for a key counts
+    else if (k.size() == 16) others[k] = v;
   }
-  if (tuned.empty()) return parse_options(options);
-  const std::string both = options && *options ? tuned + "," + options : tuned;
-  return parse_options(both.c_str());
-}
-
-GenOptions parse_options(const char* text) {
-  GenOptions o;
-  if (const char* env = std::getenv("ECLAT_HIP_ARCH")) o.arch = env;
-  if (!text) return o;
-  std::stringstream ss(text);
-  std::string item;
-  while (std::getline(ss, item, ',')) {
-    if (item.empty()) continue;
-    size_t eq = item.find('=');
-    if (eq == std::string::npos) throw Error("option '" + item + "' is not key=value");
-    std::string k = item.substr(0, eq), v = item.substr(eq + 1);
-    auto as_int = [&]() {
-      try {
-        return std::stoi(v);
-      } catch (const std::logic_error&) {
-        throw Error("option '" + k + "' needs an integer, got '" + v + "'");
-      }
-    };
-    if (k == "arch") o.arch = v;
-    else if (k == "fuse") o.fuse = as_int() != 0;
-    else if (k == "vectorize") o.vectorize = as_int() != 0;
-    else if (k == "transpose") o.transpose = as_int() != 0;
-    else if (k == "window") o.window = as_int() != 0;
-    else if (k == "row_threads") o.row_threads = as_int();
-    else if (k == "row_elems") o.row_elems = std::max(1, as_int());
-    else if (k == "flat_block") o.flat_block = as_int();
-    else if (k == "flat_iters") o.flat_iters = std::max(1, as_int());
-    else if (k == "gemm") o.gemm = as_int() != 0;
-    else if (k == "gemm_bm") o.gemm_bm = as_int();
-    else if (k == "gemm_bn") o.gemm_bn = as_int();
-    else if (k == "gemm_bk") o.gemm_bk = as_int();
-    else if (k == "gemm_wm") o.gemm_wm = as_int();
-    else if (k == "gemm_wn") o.gemm_wn = as_int();
-    else if (k == "gemm_split_k") o.gemm_split_k = as_int();
-    else if (k == "gemm_setprio") o.gemm_setprio = as_int();
-    else if (k == "gemm_waves") o.gemm_waves = as_int();
-    else if (k == "gemm_fold") o.gemm_fold = as_int() != 0;
-    else if (k == "gemm_window") o.gemm_window = as_int() != 0;
-    else if (k == "window_passes") o.window_passes = std::max(0, std::min(4, as_int()));
-    else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
-    else if (k == "gemm_dma") o.gemm_dma = std::max(0, std::min(3, as_int()));
-    else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
-    else if (k == "gemm_transpose") o.gemm_transpose = as_int() != 0;
-    else if (k == "gemm_prefetch") o.gemm_prefetch = std::max(0, as_int());
-    else if (k == "reindex") o.reindex = as_int() != 0;
-    else if (k == "guard_branches") o.guard_branches = as_int() != 0;
-    else if (k == "ranged_loads") o.ranged_loads = as_int() != 0;
-    else if (k == "rematerialize") o.rematerialize = as_int() != 0;
-    else if (k == "merge_launches") o.merge_launches = as_int() != 0;
-    else if (k == "lanes") o.lanes = std::max(1, as_int());
-    else if (k == "lane_us") o.lane_us = std::max(0, as_int());
-    else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;
-    else if (k == "nontemporal") o.nontemporal = as_int();
-    else if (k == "normalize") o.normalize = as_int() != 0;
-    else if (k == "allow_serial") o.allow_serial = as_int() != 0;
-    else throw Error("unknown option '" + k + "'");
+  // a launch's options as "@<key>:<name>=<value>" items, the program's own in front, the caller's last
+  std::string all = tuned;
+  for (const auto& kv : others) {
+    std::stringstream ss(kv.second);
+    std::string item;
+    while (std::getline(ss, item, ','))
+      if (!item.empty()) all += (all.empty() ? "" : ",") + ("@" + kv.first + ":" + item);
   }
-  if (o.flat_block < 64 || o.flat_block > 1024 || (o.flat_block & (o.flat_block - 1)))
-    throw Error("flat_block must be a power of two in [64, 1024]");
-  if (o.row_threads < 0 || o.row_threads > 1024 || (o.row_threads & (o.row_threads - 1)))
-    throw Error("row_threads must be 0 or a power of two up to 1024");
-  return o;
+  if (options && *options) all += (all.empty() ? "" : ",") + std::string(options);
+  return parse_options(all.c_str());
 }
 
 void dump_plan(const ProgramPlan& plan) {

@@ -222,7 +222,6 @@ class HipGraph {
   size_t launches_ = 0;
 };
 
-GenOptions parse_options(const char* text);       // "key=value,key=value" -> GenOptions
 // Key under which a program's tuned options are filed: FNV-1a (64 bit) of its AST text.
 unsigned long long tune_key(const char* ast_text);
 // Options for compiling `ast_text`: what the file named by ECLAT_HIP_TUNE holds for this program

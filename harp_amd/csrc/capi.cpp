@@ -96,6 +96,7 @@ void fill_info(const LaunchSpec& ls, eh_launch_info* out) {
   out->flops = ls.flops;
   out->lane = ls.lane;
   out->n_waits = static_cast<int>(ls.waits.size());
+  out->tune_key = ls.tune_key;
 }
 
 int buffer_entry(const ProgramPlan& p, int i, const char** name, const char** role, size_t* bytes, int* elided) {
@@ -156,6 +157,11 @@ int eh_device_get_props(eh_device* dev, eh_device_props* out) {
 int eh_device_sync(eh_device* dev) {
   REQUIRE(dev, "device is NULL");
   return guard([&] { dev->dev.synchronize(); });
+}
+
+int eh_device_stream(eh_device* dev, void** stream) {
+  REQUIRE(dev && stream, "device or stream is NULL");
+  return guard([&] { *stream = reinterpret_cast<void*>(dev->dev.stream()); });
 }
 
 int eh_device_trim(eh_device* dev, size_t* kept_bytes) {

@@ -886,4 +886,126 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& k, const GenOpt
   return out;
 }
 
+// ---------------------------------------------------------------------------------------------
+// options
+// ---------------------------------------------------------------------------------------------
+
+unsigned long long fnv1a(const std::string& text) {
+  unsigned long long h = 1469598103934665603ull;
+  for (unsigned char c : text) {
+    h ^= c;
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+// (the kernel's own name and the names of its buffers count for nothing: the same lowered kernel
+// gets other names in another program)
+unsigned long long launch_tune_key(const Node& kernel) {
+  std::string text = to_text(kernel);
+  auto rename_all = [&](const std::string& from, const std::string& to) {
+    const std::string q = "\"" + from + "\"";
+    for (size_t at = text.find(q); at != std::string::npos; at = text.find(q, at + to.size() + 2)) text.replace(at, q.size(), "\"" + to + "\"");
+  };
+  if (!kernel.name.empty()) rename_all(kernel.name, "k");
+  size_t n = 0;
+  for (const auto& p : kernel.params)
+    if (p.dtype.is_ptr()) rename_all(p.name, "b" + std::to_string(n++));
+  return fnv1a(text);
+}
+
+void apply_options(GenOptions* out, const std::string& text) {
+  GenOptions& o = *out;
+  std::stringstream ss(text);
+  std::string item;
+  while (std::getline(ss, item, ',')) {
+    if (item.empty()) continue;
+    if (item[0] == '@') {
+      // "@<16 hex digits>:<name>=<value>": for the launch with that key only
+      const size_t colon = item.find(':');
+      if (colon != 17 || item.find('=', colon) == std::string::npos) throw Error("option '" + item + "' is not @<key>:name=value");
+      unsigned long long key = 0;
+      try {
+        key = std::stoull(item.substr(1, 16), nullptr, 16);
+      } catch (const std::logic_error&) {
+        throw Error("option '" + item + "': the key is not 16 hex digits");
+      }
+      GenOptions probe;                                  // (checked now, applied when the launch is planned)
+      apply_options(&probe, item.substr(colon + 1));
+      std::string& s = o.launch_options[key];
+      s += (s.empty() ? "" : ",") + item.substr(colon + 1);
+      continue;
+    }
+    size_t eq = item.find('=');
+    if (eq == std::string::npos) throw Error("option '" + item + "' is not key=value");
+    std::string k = item.substr(0, eq), v = item.substr(eq + 1);
+    auto as_int = [&]() {
+      try {
+        return std::stoi(v);
+      } catch (const std::logic_error&) {
+        throw Error("option '" + k + "' needs an integer, got '" + v + "'");
+      }
+    };
+    if (k == "arch") o.arch = v;
+    else if (k == "fuse") o.fuse = as_int() != 0;
+    else if (k == "vectorize") o.vectorize = as_int() != 0;
+    else if (k == "transpose") o.transpose = as_int() != 0;
+    else if (k == "window") o.window = as_int() != 0;
+    else if (k == "row_threads") o.row_threads = as_int();
+    else if (k == "row_elems") o.row_elems = std::max(1, as_int());
+    else if (k == "flat_block") o.flat_block = as_int();
+    else if (k == "flat_iters") o.flat_iters = std::max(1, as_int());
+    else if (k == "gemm") o.gemm = as_int() != 0;
+    else if (k == "gemm_bm") o.gemm_bm = as_int();
+    else if (k == "gemm_bn") o.gemm_bn = as_int();
+    else if (k == "gemm_bk") o.gemm_bk = as_int();
+    else if (k == "gemm_wm") o.gemm_wm = as_int();
+    else if (k == "gemm_wn") o.gemm_wn = as_int();
+    else if (k == "gemm_split_k") o.gemm_split_k = as_int();
+    else if (k == "gemm_setprio") o.gemm_setprio = as_int();
+    else if (k == "gemm_waves") o.gemm_waves = as_int();
+    else if (k == "gemm_fold") o.gemm_fold = as_int() != 0;
+    else if (k == "gemm_window") o.gemm_window = as_int() != 0;
+    else if (k == "window_passes") o.window_passes = std::max(0, std::min(4, as_int()));
+    else if (k == "gemm_merge_batch") o.gemm_merge_batch = as_int() != 0;
+    else if (k == "gemm_dma") o.gemm_dma = std::max(0, std::min(3, as_int()));
+    else if (k == "gemm_mix") o.gemm_mix = as_int() != 0;
+    else if (k == "gemm_transpose") o.gemm_transpose = as_int() != 0;
+    else if (k == "gemm_prefetch") o.gemm_prefetch = std::max(0, as_int());
+    else if (k == "reindex") o.reindex = as_int() != 0;
+    else if (k == "guard_branches") o.guard_branches = as_int() != 0;
+    else if (k == "ranged_loads") o.ranged_loads = as_int() != 0;
+    else if (k == "rematerialize") o.rematerialize = as_int() != 0;
+    else if (k == "merge_launches") o.merge_launches = as_int() != 0;
+    else if (k == "lanes") o.lanes = std::max(1, as_int());
+    else if (k == "lane_us") o.lane_us = std::max(0, as_int());
+    else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;
+    else if (k == "nontemporal") o.nontemporal = as_int();
+    else if (k == "normalize") o.normalize = as_int() != 0;
+    else if (k == "allow_serial") o.allow_serial = as_int() != 0;
+    else throw Error("unknown option '" + k + "'");
+  }
+  if (o.flat_block < 64 || o.flat_block > 1024 || (o.flat_block & (o.flat_block - 1)))
+    throw Error("flat_block must be a power of two in [64, 1024]");
+  if (o.row_threads < 0 || o.row_threads > 1024 || (o.row_threads & (o.row_threads - 1)))
+    throw Error("row_threads must be 0 or a power of two up to 1024");
+}
+
+GenOptions parse_options(const char* text) {
+  GenOptions o;
+  if (const char* env = std::getenv("ECLAT_HIP_ARCH")) o.arch = env;
+  if (text) apply_options(&o, text);
+  return o;
+}
+
+GenOptions options_for_launch(const GenOptions& opt, const Node& anchor) {
+  if (opt.launch_options.empty()) return opt;
+  auto it = opt.launch_options.find(launch_tune_key(anchor));
+  if (it == opt.launch_options.end()) return opt;
+  GenOptions o = opt;
+  apply_options(&o, it->second);
+  return o;
+}
+
+
 }  // namespace eh

@@ -46,6 +46,9 @@ struct GenOptions {
   bool gemm_fold = true;              // evaluate gather/copy producers inside the tile loader (implicit GEMM)
   bool gemm_window = true;            // a folded sliding-window gather is staged in LDS once per group of rows instead of evaluated per element
   int window_passes = 0;              // of that schedule: passes over k, each for a share of a wave's blocks, stored while the next multiplies (0: chosen by the number of blocks)
+  // options for single launches, "name=value,..." by the launch's key (launch_tune_key of the first kernel it covers):
+  // applied on top of the above while that launch is planned (option items "@<key>:name=value", lines of the tuned-options file)
+  std::map<unsigned long long, std::string> launch_options;
   int gemm_split_k = -1;              // -1 = decide from the shape, 0/1 = never, n = n chunks
   bool gemm = true;          // use the MFMA contraction schedule when the shape allows
   int nontemporal = -1;      // streaming hint: -1 stores of large outputs, 0 none, 1 stores, 2 loads and stores
@@ -68,6 +71,7 @@ struct LaunchSpec {
   // Filled in by plan_program once all launches are known:
   std::vector<char> arg_written;       // per parameter: the launch writes that buffer
   std::vector<size_t> arg_full_bytes;  // per parameter: the launch writes every byte of a buffer of exactly this size (0: not known to)
+  unsigned long long tune_key = 0;     // launch_tune_key of the first kernel covered: what per-launch options are filed under
   int lane = 0;                        // 0 = the device's stream, 1.. = side streams that run beside it
   std::vector<int> waits;              // launches on other lanes that must have finished first
 };
@@ -98,6 +102,16 @@ std::vector<LaunchSpec> render_kernel_outer_parallel(const Node& kernel, const G
 // (src/backend/pipeline.rs:160-192, 475-489): per dimension the largest divisor of the global
 // size not above the preferred size, then shrunk until the workgroup fits `max_work_group`.
 void fit_local_size(const uint64_t global[3], const uint64_t preferred[3], uint64_t max_work_group, uint64_t local[3]);
+
+// "key=value,key=value" on top of *o (items "@<16 hex digits>:key=value" are filed for that launch).
+void apply_options(GenOptions* o, const std::string& text);
+GenOptions parse_options(const char* text);       // ... on top of the defaults (and ECLAT_HIP_ARCH)
+// FNV-1a (64 bit); a launch's key: of the canonical text of the first lowered kernel it covers,
+// the kernel's name and its buffers' names replaced by their positions.
+unsigned long long fnv1a(const std::string& text);
+unsigned long long launch_tune_key(const Node& kernel);
+// `opt` with what is filed for the launch that starts at kernel `anchor`, if anything is.
+GenOptions options_for_launch(const GenOptions& opt, const Node& anchor);
 
 // Expression text in HIP C (math calls, literals); exposed for tests.
 std::string render_expr_text(const Node& e);

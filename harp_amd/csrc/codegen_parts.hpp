@@ -53,14 +53,15 @@ struct ExprRenderer {
   // out-of-range load returns zero.  A guarded fp32 load is then one load whose offset is out
   // of range where the guard fails, and `guard ? load : 0` needs no select; the address is a
   // 32-bit offset, not a 64-bit pointer sum.
-  // With a load hook installed (a schedule that renders plain loads itself) only guarded loads
-  // take this form, and only under guards that test indices: an offset that waits for another
-  // load's value (a mask read from memory) would put the two loads one after the other.
+  // Only guarded loads take this form (an unguarded load keeps its pointer, so that an index that
+  // runs out of its buffer is not quietly turned into a zero), and only under guards that test
+  // indices: an offset that waits for another load's value (a mask read from memory) would put the
+  // two loads one after the other.
   const std::map<std::string, size_t>* ranged = nullptr;
   mutable int value_guards = 0;         // selects around the current node whose condition holds a load
   bool is_ranged(const Node& n, bool guarded) const {
     return ranged && n.op == Op::Load && n.count == 1 && n.dtype.ty == Ty::F32 && n.args[0]->op == Op::Var &&
-           ranged->count(n.args[0]->name) && (!load_hook || (guarded && value_guards == 0));
+           ranged->count(n.args[0]->name) && guarded && value_guards == 0;
   }
 
   std::string math1(const char* f32, const char* f64, const Node& n) const {

@@ -308,12 +308,17 @@ struct GroupEmitter {
             "  else *reinterpret_cast<EhV2<T>*>(p) = v;\n}\n";
     // guarded reads of an input whose size the buffer table fixes: one load each, out of range
     // (and so zero) where the guard fails
-    bool any_guarded = false;
-    for_each_external_load([&](const LoadRef& lr) { any_guarded = any_guarded || lr.guarded; });
-    if (any_guarded && g_ranged_loads && !g_guard_branches && !idx64)
+    // (only those reads: an unguarded read keeps its pointer, so that an index that runs out of
+    // its buffer is not quietly turned into a zero)
+    std::set<std::string> guarded_bufs;
+    for_each_external_load([&](const LoadRef& lr) {
+      if (lr.guarded && lr.load->args[0]->op == Op::Var) guarded_bufs.insert(lr.load->args[0]->name);
+    });
+    if (!guarded_bufs.empty() && g_ranged_loads && !g_guard_branches && !idx64)
       for (const auto& b : in_bufs) {
         auto it = elems.find(b);
-        if (it != elems.end() && in_dtype.at(b).ty == Ty::F32 && it->second * 4 < (size_t{1} << 31)) ranged[b] = it->second * 4;
+        if (guarded_bufs.count(b) && it != elems.end() && in_dtype.at(b).ty == Ty::F32 && it->second * 4 < (size_t{1} << 31))
+          ranged[b] = it->second * 4;
       }
     if (!ranged.empty())
       os << "__device__ __forceinline__ float eh_ranged_load(__amdgpu_buffer_rsrc_t r, unsigned byte_offset) {\n"

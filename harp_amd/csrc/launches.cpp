@@ -260,6 +260,7 @@ LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions
   unsigned block = 0;
   for (const auto& p : parts) block = std::max(block, p.block[0]);
   out.entry = parts.front().entry + "_and_" + std::to_string(parts.size() - 1);
+  out.tune_key = parts.front().tune_key;
   std::ostringstream os, sig, body;
   os << head;
   unsigned first = 0;

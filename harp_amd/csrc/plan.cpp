@@ -526,12 +526,27 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     held_back.push_back(plan.launches.back());
     plan.launches.pop_back();
   };
+  // every launch carries the key of the kernel its planning started from; options filed under that
+  // key (GenOptions::launch_options) apply while it is planned
+  size_t stamped = 0, stamped_held = 0, anchor = 0;
+  auto stamp = [&] {
+    const unsigned long long key = anchor < kernels.size() ? launch_tune_key(*kernels[anchor]) : 0;
+    for (size_t q = std::min(stamped, plan.launches.size()); q < plan.launches.size(); ++q)
+      if (!plan.launches[q].tune_key) plan.launches[q].tune_key = key;
+    for (size_t q = std::min(stamped_held, held_back.size()); q < held_back.size(); ++q)
+      if (!held_back[q].tune_key) held_back[q].tune_key = key;
+    stamped = plan.launches.size();
+    stamped_held = held_back.size();
+  };
   size_t i = 0;
   while (i < kernels.size()) {
+    stamp();
+    anchor = i;
     if (folded_kernels.count(i) || absorbed.count(i)) {
       ++i;
       continue;
     }
+    const GenOptions lopt = options_for_launch(opt, *kernels[i]);
     if (auto sw = scattered.find(i); sw != scattered.end()) {
       for (auto& ls : sw->second.launches) plan.launches.push_back(std::move(ls));
       i = sw->second.next;
@@ -540,13 +555,13 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     if (auto w = windows.find(i); w != windows.end()) {
       std::vector<const NestKernel*> chain;
       for (size_t q : w->second) chain.push_back(&*nests[q]);
-      plan.launches.push_back(emit_window_reduce(*nests[i], chain, opt, elems));
+      plan.launches.push_back(emit_window_reduce(*nests[i], chain, lopt, elems));
       ++i;
       continue;
     }
     if (!nests[i]) {
-      auto spread = render_kernel_outer_parallel(*kernels[i], opt, have_table && opt.fuse ? &plan.buffers : nullptr);
-      if (spread.empty()) plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+      auto spread = render_kernel_outer_parallel(*kernels[i], lopt, have_table && opt.fuse ? &plan.buffers : nullptr);
+      if (spread.empty()) plan.launches.push_back(render_kernel_as_written(*kernels[i], lopt));
       else for (auto& ls : spread) plan.launches.push_back(std::move(ls));
       ++i;
       continue;
@@ -566,7 +581,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           have_epi = build_epilogue(i, k0, gs->batch * gs->M * gs->N, true, k0r, epi, after);
         }
       }
-      auto gl = try_emit_gemm(have_epi ? k0r : k0, opt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
+      auto gl = try_emit_gemm(have_epi ? k0r : k0, lopt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
       if (!gl.empty()) {
         if (absorbed_name.count(i)) gl.back().kernels.push_back(absorbed_name[i]);
         // K was split and the next kernel only sums the (dense) result over the batch axis: it
@@ -627,7 +642,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (opt.gemm_epilogue && opt.fuse && have_table && k0.acc_dtype.ty == Ty::F32 && k0.out_dtype.ty == Ty::F32 &&
           dense_strides(k0, &numel))
         have_epi = build_epilogue(i, k0, numel, false, k0r, epi, after);
-      emit_serial_reduce(k0, opt, &plan, have_epi ? &epi : nullptr);
+      emit_serial_reduce(k0, lopt, &plan, have_epi ? &epi : nullptr);
       // A one-launch reduce at the end of its chain (nothing later reads what it writes or
       // writes what it reads: a parameter's update) can run whenever its inputs are ready:
       // it is held back and issued together with the others of its kind as one launch.
@@ -641,7 +656,7 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
     {
       Canon c = canon_as(k0, k0.rkind == ReduceKind::None ? StageKind::Wide : StageKind::Reduce);
       if (!c.ok) {
-        plan.launches.push_back(render_kernel_as_written(*kernels[i], opt));
+        plan.launches.push_back(render_kernel_as_written(*kernels[i], lopt));
         ++i;
         continue;
       }
@@ -723,8 +738,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       st.store = needed;
       if (!needed) plan.elided.insert(st.out_buf);
     }
-    plan.launches.push_back(emit_group(g, opt, elems));
+    plan.launches.push_back(emit_group(g, lopt, elems));
   }
+  stamp();
   // what was held back goes to the end one by one: the pass that issues independent launches together
   // (below) merges it with whatever else is still waiting there, by workgroup size (a part's surplus
   // work-items leave at once, but they are launched all the same)

@@ -1269,7 +1269,7 @@ void join_shifted_sums_with_their_contraction(Planning& st) {
         plain = v.args[o]->op == Op::Load && v.args[o]->args[0]->op == Op::Var &&
                 (!folded.count(v.args[o]->args[0]->name) || folded.at(v.args[o]->args[0]->name).prelude.empty());
       if (!plain) continue;
-      auto sw = try_emit_scattered_window(q, pv, opt);
+      auto sw = try_emit_scattered_window(q, pv, options_for_launch(opt, *kernels[q]));
       if (!sw) continue;
       for (size_t c = q + 1; c < sw->next; ++c) absorbed.insert(c);
       for (const auto& b : sw->elided) plan.elided.insert(b);

@@ -13,6 +13,7 @@ states by running them: event-timed launches of the compiled Program on the GPU.
 
     python -m harp_amd.tune --config config3_matmul [--beam 3] [--steps 4]
     python -m harp_amd.tune --config config5_cnn_step --save tuned.txt
+    python -m harp_amd.tune --config config5_cnn_step --per-launch --save tuned.txt
 
 prints the best options as the "key=value,..." string `eh_program_compile` takes.  With `--save`
 the result is also filed under the program's key (`backend.tune_key`) in the given file; a process
@@ -124,7 +125,23 @@ def suggest_pipeline(state: Dict[str, int], schedules: Sequence[str]) -> Iterabl
                 yield {**state, "lanes": n}
 
 
+def suggest_window(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
+    """Passes over k of the LDS-staged window contractions (stores of one pass drain behind the
+    next), their interleaving of LDS reads with MFMAs, or the tile-loader schedule instead."""
+    if not any(s.startswith("mfma16x16x4(window,") for s in schedules) and not state.get("gemm_window", 1) == 0:
+        return
+    for p in (1, 2, 3, 4):
+        if p != state.get("window_passes", 0):
+            yield {**state, "window_passes": p}
+    for m in (0, 1):
+        if m != state.get("gemm_mix", 1):
+            yield {**state, "gemm_mix": m}
+    if state.get("gemm_window", 1):
+        yield {"gemm_window": 0}
+
+
 SUGGESTERS: List[Callable] = [suggest_gemm, suggest_row, suggest_flat, suggest_streaming, suggest_pipeline]
+LAUNCH_SUGGESTERS: List[Callable] = [suggest_gemm, suggest_window, suggest_row, suggest_flat, suggest_streaming]
 
 
 def save_tuned(path: str, key: str, options: str, note: str = "") -> None:
@@ -202,7 +219,52 @@ def beam_search(estimator, start: Optional[Dict[str, int]] = None, beam_width: i
     return best, best_cost, history
 
 
-def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None, save=None):
+def per_launch_search(estimator, base: Optional[Dict[str, int]] = None, max_launches: int = 12, log=None):
+    """One sweep over the launches of the plan, in the order of their share of the step's work: each
+    launch's own options (suggesters applied to that launch's schedule alone) are tried with
+    everything else as it stands, and kept when the whole step gains 0.5 %.  Options for a launch
+    are filed under its key (`launch["tune_key"]`), so they follow the launch's lowered kernel into
+    any program.  Returns ({key: options}, cost, history)."""
+    base = dict(base or {})
+    plan = hb.render_program(estimator.ast, base or None)
+    launches = {}
+    for l in plan.launches:            # (the two launches of a split contraction share a key)
+        k = l["tune_key"]
+        w = launches.setdefault(k, {"schedule": l["schedule"], "weight": 0.0, "entry": l["entry"]})
+        w["weight"] += 4.0 + max(l["algo_bytes"] / 4.0e6, l["flops"] / 5.0e7)
+    order = sorted(launches, key=lambda k: -launches[k]["weight"])[:max_launches]
+    chosen: Dict[str, Dict[str, int]] = {}
+
+    def state_of(extra_key=None, extra=None):
+        st = dict(base)
+        for k, o in list(chosen.items()) + ([(extra_key, extra)] if extra_key else []):
+            for name, v in o.items():
+                st[f"@{k}:{name}"] = v
+        return _freeze(st)
+
+    best_cost = estimator.cost(state_of())
+    history = [(0, "", best_cost)]
+    for k in order:
+        sched = [launches[k]["schedule"].replace("together(", "")]
+        mine = dict(chosen.get(k, {}))
+        tried = {_freeze(mine)}
+        for sg in LAUNCH_SUGGESTERS:
+            for nxt in sg(dict(mine), sched):
+                f = _freeze(nxt)
+                if f in tried:
+                    continue
+                tried.add(f)
+                c = estimator.cost(state_of(k, nxt))
+                history.append((k, options_string(f), c))
+                if log:
+                    log(f"[tune] {launches[k]['entry']} ({k}): {options_string(f)} -> {c:.4f} ms (best {best_cost:.4f})")
+                if c < best_cost * 0.995:
+                    best_cost, mine = c, dict(nxt)
+                    chosen[k] = mine
+    return {k: options_string(_freeze(o)) for k, o in chosen.items() if o}, best_cost, history
+
+
+def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log=None, save=None, per_launch=False):
     """Searches the options of one benchmark configuration on device 0: one of
     `workloads.CONFIGS`, or a whole training step (`config4_mlp_step`, `config5_cnn_step`),
     where one option set serves every launch of the step."""
@@ -216,6 +278,12 @@ def tune_config(name: str, shapes=None, beam_width=3, max_steps=4, steps=20, log
         roots = wl.config4_graph(*ts) if mlp else wl.config5_graph(*ts, lr=1e-2)
         prog_ast, arg_names, _outs, consts, _ = wl.lower_multi(ts, roots)
         est = MeasuredEstimator(dev, prog_ast, arg_names, consts, arrays, steps=steps, sets=1)
+        if per_launch:
+            chosen, cost, history = per_launch_search(est, log=log)
+            if save:
+                for k, o in chosen.items():
+                    save_tuned(save, k, o, f"{name}, one launch: step {cost:.4f} ms (defaults {history[0][2]:.4f} ms)")
+            return _freeze({f"@{k}:{n}": int(v) for k, o in chosen.items() for n, v in (i.split("=") for i in o.split(","))}), cost, history
         return _search_and_file(est, name, beam_width, max_steps, log, save)
     default_shapes = {"config1_relu_sum": [(1024, 1024)] * 3, "config2_softmax": [(4096, 4096)],
                       "config3_matmul": [(4096, 4096)] * 2}
@@ -242,12 +310,14 @@ def main(argv=None) -> int:
     ap.add_argument("--steps", type=int, default=4, help="search steps (beam expansions)")
     ap.add_argument("--launches", type=int, default=20, help="timed launches per state")
     ap.add_argument("--save", default=None, help="file to append the result to (read back through ECLAT_HIP_TUNE)")
+    ap.add_argument("--per-launch", action="store_true",
+                    help="training steps: search each launch's own options, filed under the launch's key")
     args = ap.parse_args(argv)
     if hb.device_count() == 0:
         sys.exit("tune: no HIP device present")
     best, cost, history = tune_config(args.config, beam_width=args.beam, max_steps=args.steps,
                                       steps=args.launches, log=lambda m: print(m, file=sys.stderr, flush=True),
-                                      save=args.save)
+                                      save=args.save, per_launch=args.per_launch)
     print(json.dumps({"config": args.config, "options": options_string(best), "ms": cost,
                       "default_ms": history[0][2], "states_measured": len(history)}))
     return 0

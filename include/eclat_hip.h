@@ -64,6 +64,11 @@ int eh_device_open(int index, eh_device** out);
 int eh_device_close(eh_device* dev);    /* buffers and programs of the device must be gone */
 int eh_device_get_props(eh_device* dev, eh_device_props* out);
 int eh_device_sync(eh_device* dev);     /* waits for everything queued on the device's stream */
+/* The device's stream (a hipStream_t), for callers that order their own work against the library's
+ * or capture its launches into a graph of their own (eh_program_execute_static with sync == 0
+ * between hipStreamBeginCapture and hipStreamEndCapture on this stream).  No counterpart in the
+ * reference, whose devices own their queues (src/backend/traits.rs:273-306). */
+int eh_device_stream(eh_device* dev, void** stream);
 
 /* ---- Buffer: allocate (zero-filled), byte_len, write_from_host (size must match exactly),
  *      read_to_host, clone_buffer (src/backend/traits.rs:455-482;
@@ -117,13 +122,18 @@ typedef struct eh_launch_info {
   double flops;                         /* 2*M*N*K for contractions, else 0 */
   int lane;                             /* 0: the device's stream; 1..: a side stream beside it */
   int n_waits;                          /* launches on other lanes this one waits for */
+  unsigned long long tune_key;          /* what options for this launch alone are filed under (see ECLAT_HIP_TUNE below) */
 } eh_launch_info;
 
 int eh_render_program(const char* ast_text, const char* options, eh_plan** out);
 /* Tuned options.  When the environment variable ECLAT_HIP_TUNE names a file, eh_render_program and
  * eh_program_compile look the program up in it and take the options filed there, with `options` on
  * top: one line per program, "<key as 16 hex digits> <key=value,...>", '#' starts a comment, the
- * last line for a key counts.  The key is what eh_tune_key returns for the program's AST text; the
+ * last line for a key counts.  The key is what eh_tune_key returns for the program's AST text (the
+ * FNV-1a hash of its canonical text), or a launch's key (eh_launch_info.tune_key: the same hash of the
+ * first lowered kernel the launch covers): options under a launch's key apply to that launch alone,
+ * in whatever program it turns up; in an options string the same is written "@<key>:name=value".
+ * A file that cannot be read is reported on stderr once and ignored.  The
  * measured schedule search (python -m harp_amd.tune --save <file>) writes such lines.  It stands
  * where the reference's optimiser picks its rewrites by a static cost
  * (src/opt/ast/optimizer/beam_search.rs:34-66): here the choice is measured once and filed. */

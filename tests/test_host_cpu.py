@@ -772,6 +772,33 @@ def test_convolution_input_gradient_temp_is_stored_for_its_reader(frontend):
     assert len(direct) == 2 and all("A:k,B:n/folded" in l["schedule"] for l in direct), [l["schedule"] for l in plan.launches]
 
 
+def test_only_guarded_reads_go_through_a_buffer_resource(frontend):
+    """A padded operand (guarded reads) beside an operand read as it is: the guarded reads are
+    buffer-resource loads that come back zero beyond the buffer, the unguarded ones keep their
+    pointer -- also reads of the padded buffer itself that sit under no guard -- so an index that
+    runs out of its buffer is not turned into a quiet zero."""
+    from harp_amd import backend as hb, workloads as wl
+    from harp_amd.frontend import Tensor
+
+    def graph(x, w):
+        return [(x.pad([(1, 1), (2, 2)]).contiguous() * w).contiguous(), (x * x).contiguous()]
+
+    ts = [Tensor.input([30, 60]), Tensor.input([32, 64])]
+    ast = wl.lower_multi(ts, graph(*ts))[0]
+    plan = hb.render_program(ast, "merge_launches=0")
+    names = wl.lower_multi(ts, graph(*ts))[1]
+    x_buf, w_buf = names[0], names[1]
+    padded = [l for l in plan.launches if "eh_ranged_load(" in l["source"]]
+    assert len(padded) == 1
+    src = padded[0]["source"]
+    body = src[src.index("__global__"):]
+    assert body.count("eh_ranged_load(eh_rs_" + x_buf + ",") >= 1 and "eh_rs_" + w_buf not in src
+    assert w_buf + " + " in body or w_buf + "[" in body                     # w through its pointer
+    squares = [l for l in plan.launches if l is not padded[0]]
+    assert squares and all("eh_ranged_load" not in l["source"] for l in squares)
+    assert all(len(hb.compile_source(l["source"])) > 1000 for l in plan.launches)
+
+
 def test_convolution_windows_are_staged_in_lds(frontend):
     """The padded 3x3 gathers of the CNN step's convolutions are taken apart (row digit + window
     digit = source coordinate, guards = where that coordinate leaves the image) and what one
@@ -996,3 +1023,52 @@ def test_tuned_options_are_filed_and_applied(frontend, tmp_path, monkeypatch):
     monkeypatch.delenv("ECLAT_HIP_TUNE")
     assert sched(softmax) == default
     assert {"gemm_prefetch", "gemm_dma", "lanes"} <= {k for st in tune.suggest_pipeline({}, ["mfma32x32x2(...)"] * 8) for k in st}
+    # the key is of the canonical text: spacing does not matter
+    assert hb.tune_key(softmax.to_sexpr().replace(" (", "  (")) == key
+
+
+def test_options_filed_for_one_launch(frontend, tmp_path, monkeypatch):
+    """Options can be filed for a single launch: under the key the plan reports for it (the hash
+    of the canonical text of the first lowered kernel the launch covers), in the tuned-options
+    file beside program keys or as "@<key>:name=value" in an options string.  They apply to that
+    launch alone, in whatever program the kernel turns up, on top of the program's options."""
+    import subprocess, sys, os
+    from harp_amd import backend as hb, tune, workloads as wl
+
+    def two(x, w):
+        return [x.softmax(1) if hasattr(x, "softmax") else frontend.nn.softmax(x, 1), frontend.nn.softmax(w, 1)]
+
+    from harp_amd.frontend import Tensor
+    ts = [Tensor.input([64, 2048]), Tensor.input([32, 1024])]
+    ast = wl.lower_multi(ts, two(*ts))[0]
+    plan = hb.render_program(ast, "merge_launches=0")
+    rows = [l for l in plan.launches if l["schedule"].startswith("row(")]
+    assert len(rows) == 2 and rows[0]["tune_key"] != rows[1]["tune_key"] and all(len(l["tune_key"]) == 16 for l in rows)
+    k0 = rows[0]["tune_key"]
+    tuned = hb.render_program(ast, f"merge_launches=0,@{k0}:row_threads=64")
+    by_key = {l["tune_key"]: l["schedule"] for l in tuned.launches if l["schedule"].startswith("row(")}
+    assert "row(T=64," in by_key[k0] and by_key[rows[1]["tune_key"]] == rows[1]["schedule"]
+    # the same kernel in another program has the same key
+    alone = wl.lower_multi(ts[:1], [frontend.nn.softmax(ts[0], 1)])[0]
+    assert k0 in [l["tune_key"] for l in hb.render_program(alone).launches]
+    with pytest.raises(hb.EhError):
+        hb.render_program(ast, f"@{k0}:no_such_option=1")
+    with pytest.raises(hb.EhError):
+        hb.render_program(ast, "@123:row_threads=64")
+    # in the file: a program's line and a launch's line side by side
+    path = tmp_path / "tuned.txt"
+    tune.save_tuned(str(path), hb.tune_key(ast), "merge_launches=0", "the program")
+    tune.save_tuned(str(path), k0, "row_threads=128", "one launch")
+    monkeypatch.setenv("ECLAT_HIP_TUNE", str(path))
+    filed = hb.render_program(ast)
+    assert len(filed.launches) == len(plan.launches)
+    assert ["row(T=128," in l["schedule"] for l in filed.launches if l["tune_key"] == k0] == [True]
+    assert "row(T=128," in [l for l in hb.render_program(alone).launches if l["tune_key"] == k0][0]["schedule"]
+    # a file that cannot be read is reported once and ignored
+    env = dict(os.environ, ECLAT_HIP_TUNE=str(tmp_path / "missing" / "tuned.txt"), PYTHONPATH=os.path.dirname(os.path.dirname(__file__)))
+    code = ("from harp_amd import backend as hb, workloads as wl\n"
+            "ast = wl.lower_with_table([(64, 2048)], wl.config2_graph)[0]\n"
+            "print(hb.render_program(ast).launches[0]['schedule']); print(hb.render_program(ast).launches[0]['schedule'])\n")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.count("row(T=256,") == 2
+    assert out.stderr.count("cannot read the tuned-options file") == 1
