@@ -133,3 +133,133 @@ def test_static_scratch_execute_needs_every_buffer_of_the_caller(frontend, hip):
         arr[i] = x._h if b["name"] == names[0] else None
     with pytest.raises(EhError, match="allocates nothing"):
         check(lib.eh_program_execute_static(prog._h, arr, 2, 1))
+
+
+def _hip_runtime():
+    rt = ctypes.CDLL("libamdhip64.so")
+    rt.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    rt.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    rt.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+    rt.hipGraphInstantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    rt.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    rt.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+    rt.hipGraphExecDestroy.argtypes = [ctypes.c_void_p]
+    rt.hipGraphDestroy.argtypes = [ctypes.c_void_p]
+    return rt
+
+
+def _free_bytes(rt):
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def _bound(hip, dev, prog, names, out, arrays):
+    """Every buffer of the caller's table allocated and filled; (pointer array, count, output buffer)."""
+    bufs = {}
+    for n, a in zip(names, arrays):
+        bufs[n] = dev.alloc(a.nbytes)
+        bufs[n].write_array(a)
+    own = [b for b in prog.buffers if not b["name"].startswith("eh_")]
+    for b in own:
+        if b["name"] not in bufs and not b["elided"]:
+            bufs[b["name"]] = dev.alloc(b["bytes"])
+    arr = (ctypes.c_void_p * len(own))()
+    for i, b in enumerate(own):
+        arr[i] = bufs[b["name"]]._h if b["name"] in bufs else None
+    return arr, len(own), bufs[out], bufs
+
+
+def test_static_scratch_execute_allocates_no_device_memory(frontend, hip):
+    """What the entry point is for: after a first call (which settles the output's deferred zero
+    fill), further calls leave the driver's free memory and the device's pool of released blocks
+    exactly as they were -- for a cut reduce line and for a split contraction."""
+    from harp_amd._lib import lib, check
+    rt = _hip_runtime()
+    dev = hip.HipDevice(0)
+    for ci in (0, 4):
+        name, shapes, _fn, _exact, options = CASES[ci]
+        arrays = [RNG(17 + k).uniform(-1.0, 1.5, s).astype(np.float32) for k, s in enumerate(shapes)]
+        prog, names, out = _program(hip, dev, shapes, _graph(CASES[ci]), options)
+        arr, n, res, _bufs = _bound(hip, dev, prog, names, out, arrays)
+        check(lib.eh_program_execute_static(prog._h, arr, n, 1))
+        want = res.read_array(np.float32).copy()
+        kept = ctypes.c_size_t()
+        free_before = _free_bytes(rt)
+        for _ in range(3):
+            check(lib.eh_program_execute_static(prog._h, arr, n, 1))
+        assert _free_bytes(rt) == free_before, name
+        assert np.array_equal(res.read_array(np.float32).view(np.uint32), want.view(np.uint32)), name
+
+
+def test_static_scratch_execute_under_stream_capture(frontend, hip):
+    """The advertised use: the launches of eh_program_execute_static(sync = 0) captured into a
+    caller's graph on the device's stream (eh_device_stream), replayed twice with the output
+    overwritten in between; every replay equals eh_program_execute bit for bit.  Also with the
+    program's launches spread over two lanes (the fork and join of the side stream are recorded
+    into the same graph).  Free device memory is not compared here: instantiating a graph takes
+    a few MiB for the runtime's own argument pool; the test above measures the entry point."""
+    from harp_amd._lib import lib, check
+    from harp_amd import workloads as wl
+    from harp_amd.frontend import Tensor
+    rt = _hip_runtime()
+    dev = hip.HipDevice(0)
+    stream = ctypes.c_void_p()
+    check(lib.eh_device_stream(dev._h, ctypes.byref(stream)))
+    assert stream.value
+
+    def cnn_step(options):
+        arrays = wl.config5_inputs(16, 28, 32, 64, 128, 10, seed=93)
+        ts = [Tensor.input(list(a.shape)) for a in arrays]
+        ast, names, outs, consts, _ = wl.lower_multi(ts, wl.config5_graph(*ts, lr=0.05))
+        prog = hip.HipProgram(dev, ast, options)
+        bufs = {}
+        for nme, a in zip(names, arrays):
+            bufs[nme] = dev.alloc(a.nbytes)
+            bufs[nme].write_array(a)
+        for nme, val in consts.items():
+            b = next(x for x in prog.buffers if x["name"] == nme)
+            if not b["elided"]:
+                bufs[nme] = dev.alloc(b["bytes"])
+                bufs[nme].write_array(np.full(b["bytes"] // 4, val, np.float32))
+        own = [b for b in prog.buffers if not b["name"].startswith("eh_")]
+        for b in own:
+            if b["name"] not in bufs and not b["elided"]:
+                bufs[b["name"]] = dev.alloc(b["bytes"])
+        arr = (ctypes.c_void_p * len(own))()
+        for i, b in enumerate(own):
+            arr[i] = bufs[b["name"]]._h if b["name"] in bufs else None
+        return prog, arr, len(own), [bufs[o] for o in outs], bufs      # (bufs: the handles in arr stay alive)
+
+    name, shapes, _fn, _exact, options = CASES[4]
+    arrays = [RNG(27 + k).uniform(-1.0, 1.5, s).astype(np.float32) for k, s in enumerate(shapes)]
+    prog, names, out = _program(hip, dev, shapes, _graph(CASES[4]), options)
+    arr, n, res, _bufs = _bound(hip, dev, prog, names, out, arrays)
+    cases = [("split contraction", prog, arr, n, [res])]
+    alive = [_bufs]
+    for opts in ("lanes=1", "lanes=2,lane_us=0,merge_launches=0"):
+        p2, a2, n2, outs2, keep = cnn_step(opts)
+        alive.append(keep)
+        assert any(b["name"].startswith("eh_") and not b["elided"] for b in p2.buffers)
+        if "lanes=2" in opts:
+            assert len({l["lane"] for l in p2.launches}) == 2
+        cases.append(("cnn step " + opts, p2, a2, n2, outs2))
+    for what, prg, ar, cnt, outs in cases:
+        check(lib.eh_program_execute(prg._h, ar, cnt, 1))
+        want = [o.read_array(np.float32).copy() for o in outs]
+        check(lib.eh_program_execute_static(prg._h, ar, cnt, 1))           # settles fills, creates the lanes' streams and events
+        check(lib.eh_device_sync(dev._h))
+        graph, exe = ctypes.c_void_p(), ctypes.c_void_p()
+        assert rt.hipStreamBeginCapture(stream, 2) == 0                     # hipStreamCaptureModeRelaxed
+        rc = lib.eh_program_execute_static(prg._h, ar, cnt, 0)
+        assert rt.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+        check(rc)
+        assert rt.hipGraphInstantiate(ctypes.byref(exe), graph, None, None, 0) == 0
+        for replay in range(2):
+            for o in outs:
+                o.write_array(np.full(o.byte_len() // 4, np.nan, np.float32))
+            assert rt.hipGraphLaunch(exe, stream) == 0
+            assert rt.hipStreamSynchronize(stream) == 0
+            for o, w in zip(outs, want):
+                assert np.array_equal(o.read_array(np.float32).view(np.uint32), w.view(np.uint32)), (what, replay)
+        assert rt.hipGraphExecDestroy(exe) == 0 and rt.hipGraphDestroy(graph) == 0
