@@ -200,7 +200,7 @@ def main():
         algo = sum(l["algo_bytes"] for l in prog.launches)
         mlp = {"ms": ms, "steps": k, "flops": flops, "algo_bytes": algo,
                "lowered_kernels": len(plain.args), "launches": len(prog.launches),
-               "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
+               "gemm_launches": sum(l["schedule"].count("mfma") for l in prog.launches)}
         log(f"[bench] mlp step (batch {batch}, {dims}): {ms:.2f} ms/step -> {flops / ms / 1e9:.1f} TFLOP/s, "
             f"{batch / ms * 1e3:.0f} samples/s; {mlp['lowered_kernels']} kernels -> {mlp['launches']} launches")
 
@@ -243,13 +243,13 @@ def main():
         cnn = {"ms": ms, "steps": k, "flops": sum(l["flops"] for l in prog.launches),
                "algo_bytes": sum(l["algo_bytes"] for l in prog.launches),
                "lowered_kernels": len(plain.args), "launches": len(prog.launches),
-               "gemm_launches": sum(1 for l in prog.launches if l["schedule"].startswith("mfma"))}
+               "gemm_launches": sum(l["schedule"].count("mfma") for l in prog.launches)}
         gms, gwall = measure.time_replays(dev, prog, sets, k, min(args.warmup, 5))
         cnn["graph_ms"], cnn["graph_wall_ms"], cnn["wall_ms"] = gms, gwall, wall_ms
         log(f"[bench] cnn step replayed as one HIP graph: {gms:.3f} ms/step (host wall {gwall:.3f} ms; "
             f"eager host wall {wall_ms:.3f} ms)")
         log(f"[bench] cnn step (batch {sizes[0]}): {ms:.3f} ms/step -> {sizes[0] / ms * 1e3:.0f} images/s; "
-            f"{cnn['lowered_kernels']} kernels -> {cnn['launches']} launches ({cnn['gemm_launches']} MFMA)")
+            f"{cnn['lowered_kernels']} kernels -> {cnn['launches']} launches, {cnn['gemm_launches']} MFMA contractions")
 
         cnn_want = []
 

@@ -34,6 +34,7 @@ struct GenOptions {
   int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
   bool reindex = true;                // elementwise producers evaluated in a reader that walks another index space
   bool merge_launches = true;         // independent final reductions of a program (parameter updates) are issued as one launch
+  bool merge_templates = true;        // ... and independent small MFMA contractions (template kernels) as one launch among themselves
   bool rematerialize = true;          // a cheap elementwise temp is evaluated again by a far reader of the same index space instead of being stored for it
   bool ranged_loads = true;           // a folded gather reads its source through a buffer resource: a guarded load is one load at an out-of-range offset where the guard fails
   bool guard_branches = false;        // guarded loads (padding, edges) behind branches instead of clamped indices and selects
@@ -68,6 +69,9 @@ struct LaunchSpec {
   std::vector<std::string> kernels;    // names of the lowered kernels this launch covers
   double algo_bytes = 0;               // bytes of each distinct external buffer touched once
   double flops = 0;
+  // A launch built from a kernel template that can also be compiled as a part of a larger launch
+  // (the template's EH_PART mode): the parameter list of its entry point as written there.
+  std::string part_params;
   // Filled in by plan_program once all launches are known:
   std::vector<char> arg_written;       // per parameter: the launch writes that buffer
   std::vector<size_t> arg_full_bytes;  // per parameter: the launch writes every byte of a buffer of exactly this size (0: not known to)

@@ -512,6 +512,8 @@ std::vector<LaunchSpec> try_emit_gemm(const NestKernel& k, const GenOptions& opt
   os << "#define EH_LOAD_BRANCH " << (opt.guard_branches ? 1 : 0) << "\n";
   os << kGemmSource;
   ls.source = os.str();
+  ls.part_params = std::string("const float* __restrict__ A, const float* __restrict__ B") +
+                   (epi_here && !epilogue->store_c ? "" : ", float* __restrict__ C") + (epi_here ? epilogue->params : "");
   const bool ragged = s->M % t.bm || s->N % t.bn || s->K % t.bk;
   ls.schedule = "mfma32x32x2(tile=" + std::to_string(t.bm) + "x" + std::to_string(t.bn) + "x" + std::to_string(t.bk) +
                 ",wave=" + std::to_string(t.wm) + "x" + std::to_string(t.wn) + (a_kc ? ",A:k" : ",A:m") +

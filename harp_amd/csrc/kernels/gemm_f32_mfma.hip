@@ -369,6 +369,29 @@ __device__ __forceinline__ long long eh_axis_offset(long long v) {
 #define EH_WAVES_PER_SIMD 4   // register budget: 512 / this many VGPRs+AGPRs per lane
 #endif
 
+// EH_PART: this kernel is one of several issued as one launch.  It is then a function of its
+// share of the launch's linear workgroup ids (its own grid is EH_PART_GX x EH_PART_GY x batch) and
+// of the launch's one block of LDS, which the parts use in turn; eh_lds_floats says how much it needs.
+#ifdef EH_PART
+#define EH_BLOCK_X (eh_bx % EH_PART_GX)
+#define EH_BLOCK_Y (eh_bx / EH_PART_GX % EH_PART_GY)
+#define EH_BLOCK_Z (eh_bx / (EH_PART_GX * EH_PART_GY))
+constexpr int eh_lds_floats = 2 * BK * (AS + BS);
+__device__ __forceinline__ void eh_run(const unsigned eh_bx, float* const eh_lds, const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_EPI_PARAMS) {
+  float* const As0 = eh_lds;
+  float* const As1 = eh_lds + BK * AS;
+  float* const Bs0 = eh_lds + 2 * BK * AS;
+  float* const Bs1 = Bs0 + BK * BS;
+#if !(EH_A_DMA || EH_B_DMA)
+  float (*const As)[BK * AS] = reinterpret_cast<float (*)[BK * AS]>(As0);
+  float (*const Bs)[BK * BS] = reinterpret_cast<float (*)[BK * BS]>(Bs0);
+  (void)As1;
+  (void)Bs1;
+#endif
+#else
+#define EH_BLOCK_X blockIdx.x
+#define EH_BLOCK_Y blockIdx.y
+#define EH_BLOCK_Z blockIdx.z
 extern "C" __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(EH_WAVES_PER_SIMD, EH_WAVES_PER_SIMD)))
 EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_EPI_PARAMS) {
   // two tiles per operand, as separate arrays: the compiler then knows that a direct-to-LDS
@@ -384,6 +407,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   float* const As0 = As[0];
   float* const Bs0 = Bs[0];
 #endif
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wid = tid >> 6;
@@ -391,7 +415,7 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   const int l32 = lane & 31, kh = lane >> 5;
 
   // workgroup -> tile: compact per XCD, then grouped along M so neighbours share B panels
-  int tile = blockIdx.x;
+  int tile = EH_BLOCK_X;
   if (NTILES % 8 == 0) tile = (tile % 8) * (NTILES / 8) + tile / 8;
   constexpr int GM = EH_GROUP_M < TM ? EH_GROUP_M : TM;
   const int group = tile / (GM * TN);
@@ -402,13 +426,13 @@ EH_ENTRY(const float* __restrict__ A, const float* __restrict__ B EH_C_PARAM EH_
   const int tn = in_g / gsz;
   const long long m0 = (long long)tm * BM, n0 = (long long)tn * BN;
 
-  const long long bz = blockIdx.z;
+  const long long bz = EH_BLOCK_Z;
   const long long a_base = EH_A_OFF + bz * EH_A_BS, b_base = EH_B_OFF + bz * EH_B_BS;
 #if EH_SPLITK > 1
   // partial sums go to a dense [split][batch][M][N] scratch; a second launch adds them up
-  const long long kbeg = (long long)blockIdx.y * KT * BK;
+  const long long kbeg = (long long)EH_BLOCK_Y * KT * BK;
   const long long kend = (kbeg + (long long)KT * BK) < K ? (kbeg + (long long)KT * BK) : K;
-  float* Cb = C + ((long long)blockIdx.y * EH_BATCH + bz) * (M * N);
+  float* Cb = C + ((long long)EH_BLOCK_Y * EH_BATCH + bz) * (M * N);
   constexpr long long CSM = N, CSN = 1;
 #elif defined(EH_EPILOGUE)
   const long long kbeg = 0, kend = K;

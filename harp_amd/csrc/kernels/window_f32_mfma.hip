@@ -127,16 +127,28 @@ static_assert(EW_PASSES >= 1 && EW_PASSES <= 4 && (EW_NB + EW_PASSES - 1) / EW_P
 template <int V> struct EwInt { static constexpr int value = V; };
 }  // namespace
 
+// EH_PART: this kernel is one of several issued as one launch.  It is then a function of its
+// share of the launch's linear workgroup ids (its own grid is EH_PART_GX groups x batch) and of the
+// launch's one block of LDS, which the parts use in turn; eh_lds_floats says how much it needs.
+#ifdef EH_PART
+constexpr int eh_lds_floats = ((EW_PATCH_FLOATS + 3) & ~3) + EW_WAVES_M * EW_MB * 16 * EW_A_LDS;
+__device__ __forceinline__ void eh_run(const unsigned eh_bx, float* const eh_lds, const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS) {
+  constexpr int MROWS = EW_WAVES_M * EW_MB * 16;
+  float* const patch = eh_lds;
+  float* const As = eh_lds + ((EW_PATCH_FLOATS + 3) & ~3);
+  const long long g = eh_bx % EH_PART_GX, bz = eh_bx / EH_PART_GX;
+#else
 extern "C" __global__ void __launch_bounds__(EW_NT)
 EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS) {
   constexpr int MROWS = EW_WAVES_M * EW_MB * 16;        // rows of A a workgroup multiplies (padding rows are zero)
   __shared__ __attribute__((aligned(16))) float patch[EW_PATCH_FLOATS];
   __shared__ __attribute__((aligned(16))) float As[MROWS * EW_A_LDS];
+  const long long g = blockIdx.x, bz = blockIdx.z;
+#endif
   const int tid = threadIdx.x;
   const int lane = tid & 63, wid = tid >> 6;
   const int wm = wid % EW_WAVES_M, wn = wid / EW_WAVES_M;
   const int l16 = lane & 15, j4 = lane >> 4;
-  const long long g = blockIdx.x, bz = blockIdx.z;
 
   // A into LDS, fetched in the order of its memory (128-bit loads where rows allow); rows beyond M
   // and k beyond K of the tile are zero.  Every load of a chunk is issued before the first value is

@@ -1,4 +1,5 @@
 // Passes over the planned launches: what each writes, which go out together, lanes.
+#include <cctype>
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -63,7 +64,17 @@ void issue_independent_launches_together(ProgramPlan* plan, const std::vector<co
   if (!(opt.fuse && opt.reindex && opt.merge_launches) || plan->launches.size() < 3) return;
   mark_written(plan, kernels);
   const std::string head = kernel_header();
+  // A contraction built from a kernel template can be compiled as a part of a larger launch.
+  // Only the small ones are: four waves a workgroup, at most 4 GFLOP -- the weight gradients of a
+  // small network, each a few microseconds above the cost of a launch.  A part's LDS is the
+  // launch's, so these go out among themselves, never with kernels that want many workgroups a CU.
+  auto template_part = [&](const LaunchSpec& ls) {
+    return !ls.part_params.empty() && ls.block[0] == 256 && ls.block[1] == 1 && ls.block[2] == 1 && !ls.lds_bytes &&
+           ls.flops <= 4e9 && !ls.kernels.empty() && opt.merge_templates;
+  };
+  auto size_class = [&](const LaunchSpec& ls) { return ls.block[0] * 2 + (template_part(ls) ? 1u : 0u); };
   auto mergeable = [&](const LaunchSpec& ls) {
+    if (template_part(ls)) return true;
     if (ls.grid[1] != 1 || ls.grid[2] != 1 || ls.block[1] != 1 || ls.block[2] != 1 || ls.block[0] % 64 || ls.lds_bytes) return false;
     if (ls.source.rfind(head, 0) != 0 || ls.schedule.rfind("together(", 0) == 0 || ls.kernels.empty()) return false;
     const std::string open = "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(ls.block[0]) + ") " + ls.entry + "(";
@@ -88,15 +99,15 @@ void issue_independent_launches_together(ProgramPlan* plan, const std::vector<co
     std::vector<LaunchSpec> stay;
     std::set<unsigned> go;
     for (const auto& h : held)
-      if (!trigger || conflict(*trigger, h)) go.insert(h.block[0]);
+      if (!trigger || conflict(*trigger, h)) go.insert(size_class(h));
     for (auto& h : held) {
-      if (go.count(h.block[0])) by_block[h.block[0]].push_back(std::move(h));
+      if (go.count(size_class(h))) by_block[size_class(h)].push_back(std::move(h));
       else stay.push_back(std::move(h));
     }
     held = std::move(stay);
     for (auto& kv : by_block) {
       for (size_t q = next; q < in.size(); ++q) {
-        if (taken[q] || in[q].block[0] != kv.first || !mergeable(in[q])) continue;
+        if (taken[q] || !mergeable(in[q]) || size_class(in[q]) != kv.first) continue;
         bool free_to_move = true;
         for (size_t p = next; p < q && free_to_move; ++p) free_to_move = taken[p] || !conflict(in[q], in[p]);
         for (const auto& h : held) free_to_move = free_to_move && !conflict(in[q], h);
@@ -254,50 +265,80 @@ void assign_lanes(ProgramPlan* plan, const std::vector<const Node*>& kernels, co
 }
 
 
-LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions& opt) {
+LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts_in, const GenOptions& opt) {
   LaunchSpec out;
   const std::string head = hdr(opt);
+  // template kernels: the longest first, so that the launch ends on its short parts
+  std::vector<LaunchSpec> parts = parts_in;
+  const bool templates = !parts.front().part_params.empty();
+  if (templates)
+    std::stable_sort(parts.begin(), parts.end(), [](const LaunchSpec& x, const LaunchSpec& y) { return x.flops > y.flops; });
   unsigned block = 0;
   for (const auto& p : parts) block = std::max(block, p.block[0]);
   out.entry = parts.front().entry + "_and_" + std::to_string(parts.size() - 1);
   out.tune_key = parts.front().tune_key;
-  std::ostringstream os, sig, body;
+  std::ostringstream os, sig, body, lds;
   os << head;
   unsigned first = 0;
   for (size_t i = 0; i < parts.size(); ++i) {
     const LaunchSpec& p = parts[i];
-    if (p.source.rfind(head, 0) != 0 || p.grid[1] != 1 || p.grid[2] != 1 || p.block[1] != 1 || p.block[2] != 1 || p.block[0] % 64 || p.lds_bytes)
-      throw Error("internal: launch '" + p.entry + "' cannot be merged");
-    std::string text = p.source.substr(head.size());
-    const std::string open = "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(p.block[0]) + ") " + p.entry + "(";
-    const size_t at = text.find(open);
-    const size_t close = at == std::string::npos ? at : text.find(") {\n", at);
-    if (close == std::string::npos) throw Error("internal: launch '" + p.entry + "' has no entry point to merge");
-    const std::string params = text.substr(at + open.size(), close - at - open.size());
-    text.replace(at, open.size(), "__device__ __forceinline__ void eh_run(const unsigned eh_bx, ");
-    for (size_t q = text.find("blockIdx.x"); q != std::string::npos; q = text.find("blockIdx.x", q)) text.replace(q, 10, "eh_bx");
-    const std::string own_grid = std::to_string(p.grid[0]) + "u";
-    for (size_t q = text.find("gridDim.x"); q != std::string::npos; q = text.find("gridDim.x", q)) text.replace(q, 9, own_grid);
     const std::string ns = "eh_part" + std::to_string(i);
-    os << "namespace " << ns << " {\n" << text << "}  // namespace " << ns << "\n";
+    std::string params;
+    unsigned blocks = p.grid[0];
+    if (templates) {
+      // the template's EH_PART mode: a device function eh_run(linear workgroup id, LDS block, parameters...)
+      if (p.part_params.empty() || p.block[0] != block || p.block[1] != 1 || p.block[2] != 1 || p.lds_bytes)
+        throw Error("internal: launch '" + p.entry + "' cannot be merged");
+      blocks = p.grid[0] * p.grid[1] * p.grid[2];
+      os << "#define EH_PART 1\n#define EH_PART_GX " << p.grid[0] << "u\n#define EH_PART_GY " << p.grid[1] << "u\n";
+      os << "namespace " << ns << " {\n" << p.source << "}  // namespace " << ns << "\n";
+      // every macro the part defined goes again: the next part defines its own
+      std::set<std::string> macros = {"EH_PART", "EH_PART_GX", "EH_PART_GY"};
+      for (size_t q = p.source.find("#define "); q != std::string::npos; q = p.source.find("#define ", q + 8)) {
+        if (q > 0 && p.source[q - 1] != '\n') continue;
+        size_t e = q + 8;
+        while (e < p.source.size() && (std::isalnum(static_cast<unsigned char>(p.source[e])) || p.source[e] == '_')) ++e;
+        macros.insert(p.source.substr(q + 8, e - q - 8));
+      }
+      for (const auto& m : macros) os << "#undef " << m << "\n";
+      params = p.part_params;
+      lds << "eh_max2(" << ns << "::eh_lds_floats, ";
+    } else {
+      if (p.source.rfind(head, 0) != 0 || p.grid[1] != 1 || p.grid[2] != 1 || p.block[1] != 1 || p.block[2] != 1 || p.block[0] % 64 || p.lds_bytes)
+        throw Error("internal: launch '" + p.entry + "' cannot be merged");
+      std::string text = p.source.substr(head.size());
+      const std::string open = "extern \"C\" __global__ void __launch_bounds__(" + std::to_string(p.block[0]) + ") " + p.entry + "(";
+      const size_t at = text.find(open);
+      const size_t close = at == std::string::npos ? at : text.find(") {\n", at);
+      if (close == std::string::npos) throw Error("internal: launch '" + p.entry + "' has no entry point to merge");
+      params = text.substr(at + open.size(), close - at - open.size());
+      text.replace(at, open.size(), "__device__ __forceinline__ void eh_run(const unsigned eh_bx, ");
+      for (size_t q = text.find("blockIdx.x"); q != std::string::npos; q = text.find("blockIdx.x", q)) text.replace(q, 10, "eh_bx");
+      const std::string own_grid = std::to_string(p.grid[0]) + "u";
+      for (size_t q = text.find("gridDim.x"); q != std::string::npos; q = text.find("gridDim.x", q)) text.replace(q, 9, own_grid);
+      os << "namespace " << ns << " {\n" << text << "}  // namespace " << ns << "\n";
+    }
     // the part's parameters, renamed, in the merged signature; the same names in the call
     std::string call;
     size_t from = 0, n = 0;
     while (from < params.size()) {
       size_t comma = params.find(", ", from);
       if (comma == std::string::npos) comma = params.size();
-      const std::string one = params.substr(from, comma - from);
+      std::string one = params.substr(from, comma - from);
+      while (!one.empty() && one.front() == ' ') one.erase(one.begin());
+      while (!one.empty() && one.back() == ' ') one.pop_back();
+      from = comma + 2;
+      if (one.empty()) continue;
       const size_t sp = one.rfind(' ');
       const std::string name = "p" + std::to_string(i) + "_" + one.substr(sp + 1);
       sig << (sig.tellp() > 0 ? ", " : "") << one.substr(0, sp + 1) << name;
       call += ", " + name;
-      from = comma + 2;
       ++n;
     }
     if (n != p.arg_bufs.size()) throw Error("internal: launch '" + p.entry + "' lists " + std::to_string(p.arg_bufs.size()) + " buffers for " + std::to_string(n) + " parameters");
-    body << "  if (blockIdx.x < " << first + p.grid[0] << "u) {\n    if (threadIdx.x < " << p.block[0] << "u) " << ns << "::eh_run(blockIdx.x - "
-         << first << "u" << call << ");\n    return;\n  }\n";
-    first += p.grid[0];
+    body << "  if (blockIdx.x < " << first + blocks << "u) {\n    if (threadIdx.x < " << p.block[0] << "u) " << ns << "::eh_run(blockIdx.x - "
+         << first << "u" << (templates ? ", eh_lds" : "") << call << ");\n    return;\n  }\n";
+    first += blocks;
     for (size_t a = 0; a < p.arg_bufs.size(); ++a) {
       out.arg_bufs.push_back(p.arg_bufs[a]);
       out.arg_min_bytes.push_back(a < p.arg_min_bytes.size() ? p.arg_min_bytes[a] : 0);
@@ -308,7 +349,14 @@ LaunchSpec merge_launches(const std::vector<LaunchSpec>& parts, const GenOptions
     out.schedule += (i ? " + " : "together(") + p.schedule;
   }
   out.schedule += ")";
-  os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << out.entry << "(" << sig.str() << ") {\n" << body.str() << "}\n";
+  if (templates) {
+    os << "namespace {\nconstexpr int eh_max2(int a, int b) { return a > b ? a : b; }\n}\n";
+  }
+  os << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << out.entry << "(" << sig.str() << ") {\n";
+  if (templates)
+    os << "  // the parts' tiles, one part at a time: a workgroup runs exactly one part\n"
+       << "  __shared__ __attribute__((aligned(16))) float eh_lds[" << lds.str() << "4" << std::string(parts.size(), ')') << "];\n";
+  os << body.str() << "}\n";
   out.source = os.str();
   out.grid[0] = first;
   out.block[0] = block;

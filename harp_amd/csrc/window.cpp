@@ -589,6 +589,8 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   }
   os << kWindowSource;
   ls.source = os.str();
+  ls.part_params = std::string("const float* __restrict__ A, const float* __restrict__ F") +
+                   (epilogue && !epilogue->store_c ? "" : ", float* __restrict__ C") + (epilogue ? epilogue->params : "");
   ls.schedule = "mfma16x16x4(window,group=" + std::to_string(NG) + ",M=" + std::to_string(M) + ",K=" + std::to_string(K) +
                 ",waves=" + std::to_string(lay.waves_m) + "x" + std::to_string(lay.waves_n) + ",blocks=" + std::to_string(lay.mb) +
                 "x" + std::to_string(lay.nb) + ",steps=" + std::to_string(ksteps) + ",patterns=" + std::to_string(patterns.size()) +

@@ -55,7 +55,7 @@ GEMM_TILES = [  # (bm, bn, bk, wm, wn): macro tile, k step, wave tile; LDS 2*bk*
 
 def suggest_gemm(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
     """Tile shapes, register budget (waves per SIMD) and K split of the MFMA contraction."""
-    if not any(s.startswith("mfma") for s in schedules):
+    if not any("mfma" in s for s in schedules):
         return
     cur = tuple(state.get(k, 0) for k in ("gemm_bm", "gemm_bn", "gemm_bk", "gemm_wm", "gemm_wn"))
     for t in GEMM_TILES:
@@ -112,7 +112,7 @@ def suggest_pipeline(state: Dict[str, int], schedules: Sequence[str]) -> Iterabl
     """How far ahead of their use a contraction's tiles are loaded (register stages), whether they
     go through registers or straight into LDS, and how many streams a program's independent
     launches are spread over: the register, LDS and queue budgets of a plan."""
-    if any(s.startswith("mfma") for s in schedules):
+    if any("mfma" in s for s in schedules):
         for p in (1, 3, 5):
             if p != state.get("gemm_prefetch", 0):
                 yield {**state, "gemm_prefetch": p}
@@ -128,7 +128,7 @@ def suggest_pipeline(state: Dict[str, int], schedules: Sequence[str]) -> Iterabl
 def suggest_window(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Dict[str, int]]:
     """Passes over k of the LDS-staged window contractions (stores of one pass drain behind the
     next), their interleaving of LDS reads with MFMAs, or the tile-loader schedule instead."""
-    if not any(s.startswith("mfma16x16x4(window,") for s in schedules) and not state.get("gemm_window", 1) == 0:
+    if not any("mfma16x16x4(window," in s for s in schedules) and not state.get("gemm_window", 1) == 0:
         return
     for p in (1, 2, 3, 4):
         if p != state.get("window_passes", 0):

@@ -153,3 +153,31 @@ def test_lanes_change_nothing_but_the_timing(hip):
             assert np.array_equal(g, w), options
         del graph, prog, sets
         dev.trim()
+
+
+def test_contractions_issued_together_change_nothing_but_the_timing(hip):
+    """A layer's input gradient and weight gradient as one launch (the kernel templates compiled
+    as parts that share the launch's block of LDS) and as launches of their own: the same
+    arithmetic on the same inputs, so every output of the CNN training step is equal bit for bit
+    -- also on back-to-back executes and as a recorded graph."""
+    hb = hip
+    dev = hb.HipDevice(0)
+    want = None
+    for options in ("merge_templates=0", None):
+        prog, sets, arg_names, outs, arrays = _cnn_sets(hb, dev, 32, seed=95, options=options)
+        pairs = [l for l in prog.launches if l["schedule"].startswith("together(mfma")]
+        assert len(pairs) == (0 if options else 3), [l["schedule"] for l in prog.launches]
+        for _ in range(2):
+            prog.run(sets[0][0], sync=False)
+        dev.sync()
+        got = _read_outputs(sets[0][1], outs)
+        if want is None:
+            want = got
+        for g, w in zip(got, want):
+            assert np.array_equal(g, w), options
+        graph = prog.record(sets[1][0])
+        graph.replay()
+        for g, w in zip(_read_outputs(sets[1][1], outs), want):
+            assert np.array_equal(g, w), options
+        del graph, prog, sets
+        dev.trim()

@@ -99,9 +99,34 @@ def test_join_shifted_sums_with_their_contraction(cnn_ast):
     """The second convolution's input gradient: dY x W, then eight kernels adding up nine shifted,
     guarded reads of the product.  One window contraction over (channel, shift) covers all nine
     kernels; gemm_window=0 keeps the product and the sums apart."""
-    plan = _plan(cnn_ast)
+    plan = _plan(cnn_ast, "merge_templates=0")
     dx = _covering(plan, "R_256_196_1_288_59")
     assert dx["kernels"][1:] == ["E_256_32_16_16_%d" % q for q in range(60, 68)] and "shifts=9" in dx["schedule"]
-    off = _plan(cnn_ast, "gemm_window=0")
+    off = _plan(cnn_ast, "gemm_window=0,merge_templates=0")
     assert _covering(off, "R_256_196_1_288_59")["kernels"] == ["R_256_196_1_288_59"]
     assert len(off.launches) == len(plan.launches) + 1
+
+
+def test_issue_independent_contractions_together(cnn_ast):
+    """A layer's input gradient and weight gradient are contractions that read the same dY and
+    nothing of each other.  Each is an instance of a kernel template; compiled as parts (a device
+    function of the launch's linear workgroup id and of the launch's one block of LDS) they go out
+    as one launch, the longer part first: the second convolution's, and both fully connected
+    layers'.  merge_templates=0 launches them one by one."""
+    from harp_amd import backend as hb
+    plan = _plan(cnn_ast)
+    pairs = [l for l in plan.launches if l["schedule"].startswith("together(mfma")]
+    assert [sorted(k for k in l["kernels"] if k.startswith("R_")) for l in pairs] == [
+        ["R_1_128_10_103", "R_256_128_1_44"], ["R_1_3136_128_97", "R_256_3136_1_47"], ["R_256_196_1_288_59", "R_256_1_64_288_88"]]
+    conv = pairs[2]
+    assert conv["grid"] == [512, 1, 1] and conv["block"] == [256, 1, 1]
+    src = conv["source"]
+    assert src.count("#define EH_PART 1") == 2 and src.count("#undef EW_ENTRY") == 2
+    assert "float eh_lds[eh_max2(eh_part0::eh_lds_floats, eh_max2(eh_part1::eh_lds_floats, 4))];" in src
+    assert src.index("eh_part0::eh_run(blockIdx.x - 0u, eh_lds") < src.index("eh_part1::eh_run(blockIdx.x - 256u, eh_lds")
+    assert len(hb.compile_source(src)) > 1000
+    # split K over the second grid axis: the part decodes it from the linear id
+    fc = pairs[1]
+    assert "split-k=2" in fc["schedule"] and fc["grid"] == [196 + 98 * 2, 1, 1] and "#define EH_PART_GY 2u" in fc["source"]
+    apart = _plan(cnn_ast, "merge_templates=0")
+    assert len(apart.launches) == len(plan.launches) + 3 and not any(l["schedule"].startswith("together(mfma") for l in apart.launches)
