@@ -118,11 +118,16 @@ bool choose(const GemmShape& s, const GenOptions& opt, Choice* out, bool compute
     for (int split : {1, 2, 4, 8, 16, 32, 64, 128, 256}) {
       if (split > 1 && (opt.gemm_split_k == 0 || opt.gemm_split_k == 1)) break;
       if (opt.gemm_split_k > 1 && split != 1) break;
-      // a requested split is capped so that every chunk keeps at least eight k-steps
+      // a split of the planner's own keeps at least eight k-steps per chunk -- two where the
+      // whole result is at most four small tiles, K is split anyway and the k-steps' dependent
+      // loads are all there is to wait for (a 128 x 10 weight gradient over a batch of 256: 7.9 us in two chunks, 4 us in
+      // eight) -- and a requested one two
+      const bool few = s.M * s.N * s.batch <= 4 * 64 * 64 && ksteps >= 16;
+      const int64_t least = opt.gemm_split_k > 1 || few ? 2 : 8;
       int sp = opt.gemm_split_k > 1
-                   ? static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(opt.gemm_split_k, ksteps / 8)))
+                   ? static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(opt.gemm_split_k, ksteps / 2)))
                    : split;
-      if (sp > 1 && ksteps / sp < 8) break;
+      if (sp > 1 && ksteps / sp < least) break;
       double us = estimate_us(s, c, sp);
       if (!have || us < best_us) {
         have = true;
