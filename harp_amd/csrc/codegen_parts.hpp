@@ -242,7 +242,8 @@ std::string gather_fn_name(const std::string& buf);
 std::string gather_call(const NestKernel& g, const std::string& src, const Node& index, const std::vector<Loop>& caller,
                         const std::string& idx_type);
 std::string gather_fn_text(const NestKernel& g, const std::string& src, const NestKernel* inner, const std::string& idx_type);
-std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems);
+// (`computing`: any expression of that one buffer, not only a load under an index-only guard)
+std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems, bool computing = false);
 std::optional<Affine> relayout(const NestKernel& g, const NestKernel& sk, const Affine& read);
 
 // ---- rewrites.cpp -----------------------------------------------------------------------------

@@ -1216,6 +1216,44 @@ void read_windows_through_their_gathers(Planning& st) {
         buf = gl[0].load->args[0]->name;
       }
       if (chain.empty()) continue;
+      // The source itself may be a cheap elementwise function of a buffer that stays in memory
+      // anyway (the activation max(z, 0) of a pre-activation z that the backward pass reads): the
+      // windows then read z and apply the function, and the activation is never stored.
+      if (opt.rematerialize && chain.size() < 3) {
+        auto w = writer.find(buf);
+        if (w != writer.end() && role_of(buf) == "temp" && readers[buf] == std::vector<size_t>{chain.back()}) {
+          const size_t q = w->second;
+          const NestKernel& e = *nests[q];
+          std::function<size_t(const Node&)> size_of = [&](const Node& n) {
+            size_t c = 1;
+            for (const auto& a : n.args)
+              if (a && n.op != Op::Load) c += size_of(*a);
+            return c;
+          };
+          std::vector<LoadRef> el;
+          if (e.rkind == ReduceKind::None && e.value) collect_loads(*e.value, el);
+          bool ok_e = !el.empty() && el.size() <= 2 && size_of(*e.value) <= 8 && e.out_aff && make_fold(e, elems, true).has_value();
+          std::string z;
+          for (const auto& lr : el) {
+            if (!ok_e) break;
+            auto a = affine_of(*lr.load->args[1]);
+            ok_e = a && *a == *e.out_aff && !lr.guarded && lr.load->args[0]->op == Op::Var;    // element for element
+            if (ok_e) z = lr.load->args[0]->name;
+          }
+          if (ok_e) {
+            // z is kept: an input or output of the program, or a temp that a kernel behind r reads
+            bool kept = role_of(z) != "temp";
+            for (size_t c : readers[z]) kept = kept || c > r;
+            // ... and nothing between its writer and r overwrites it
+            for (size_t m = q + 1; m <= r && kept; ++m)
+              if (nests[m] && nests[m]->out_buf == z && !folded_kernels.count(m) && !absorbed.count(m)) kept = false;
+            if (kept) {
+              chain.push_back(q);
+              buf = z;
+            }
+          }
+        }
+      }
       windows[r] = chain;
       for (size_t q : chain) {
         folded_kernels.insert(q);

@@ -247,7 +247,7 @@ std::string gather_fn_text(const NestKernel& g, const std::string& src, const Ne
 
 // An elementwise kernel as a function of the linear index of its (dense, row-major) output, for
 // contractions that evaluate it in their tile loader.  Only kernels reading one f32 buffer.
-std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems) {
+std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::string, size_t>& elems, bool computing) {
   if (k.rkind != ReduceKind::None || k.out_dtype.ty != Ty::F32 || !k.out_aff || k.out_aff->c != 0) return std::nullopt;
   int64_t stride = 1, numel = 1;
   std::vector<int64_t> strides(k.loops.size(), 0);
@@ -280,7 +280,7 @@ std::optional<FoldedOperand> make_fold(const NestKernel& k, const std::map<std::
   if (src == k.out_buf) return std::nullopt;
   // pure gathers only (a load, possibly under an index-only guard with a constant default):
   // anything that computes is cheaper done once than once per tile that reads it
-  {
+  if (!computing) {
     const Node* v = k.value.get();
     if (v->op == Op::Select && v->args[2]->op == Op::Const) {
       std::vector<LoadRef> in_cond;

@@ -85,11 +85,20 @@ def test_fold_gathers_into_contractions(cnn_ast):
 
 def test_read_windows_through_their_gathers(cnn_ast):
     """Max pooling is lowered as unfold, copy, reduce over the window axis.  The reduce reads the
-    convolution's output through the gathers' index maps: one launch, no window buffer.
-    window=0 launches the gather."""
+    convolution's output through the gathers' index maps: one launch, no window buffer.  What the
+    gather reads is max(z, 0) of a pre-activation z that the backward pass needs anyway: the
+    reduce applies that as well, and the convolution stores z only.  window=0 launches the
+    gather; rematerialize=0 keeps the stored activation."""
     plan = _plan(cnn_ast)
     pool = _covering(plan, "R_256_32_14_14_1_7")
-    assert "E_256_32_14_14_2_2_6" in pool["kernels"] and "window-reduce(window=4,gathers=1)" in pool["schedule"]
+    assert pool["kernels"][:3] == ["E_256_32_28_28_5", "E_256_32_14_14_2_2_6", "R_256_32_14_14_1_7"]
+    assert "window-reduce(window=4,gathers=2)" in pool["schedule"] and "fmaxf(buf31[" in pool["source"]
+    conv = _covering(plan, "R_256_784_32_1_1")
+    assert "E_256_32_28_28_5" not in conv["kernels"] and sum(conv["written"]) == 1
+    assert any(b["name"] == "buf37" and b["elided"] for b in plan.buffers)
+    stored = _plan(cnn_ast, "rematerialize=0")
+    assert "E_256_32_28_28_5" in _covering(stored, "R_256_784_32_1_1")["kernels"]
+    assert "window-reduce(window=4,gathers=1)" in _covering(stored, "R_256_32_14_14_1_7")["schedule"]
     off = _plan(cnn_ast, "window=0")
     assert "E_256_32_14_14_2_2_6" not in _covering(off, "R_256_32_14_14_1_7")["kernels"]
     assert len(off.launches) > len(plan.launches)
