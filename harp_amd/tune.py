@@ -67,9 +67,10 @@ def suggest_gemm(state: Dict[str, int], schedules: Sequence[str]) -> Iterable[Di
         for w in (per_simd, 2 * per_simd, 4 * per_simd):
             if w <= 8 and w != state.get("gemm_waves", 0):
                 yield {**state, "gemm_waves": w}
-        for sk in (1, 2, 4, 8):
-            if sk != state.get("gemm_split_k", 1):
-                yield {**state, "gemm_split_k": sk}
+    # (1: never; a requested split goes down to two k-steps a chunk; unset leaves it to the planner)
+    for sk in (1, 2, 4, 8, 16, 32):
+        if sk != state.get("gemm_split_k", -1):
+            yield {**state, "gemm_split_k": sk}
     for p in (0, 1):
         if p != state.get("gemm_setprio", 0):
             yield {**state, "gemm_setprio": p}
