@@ -1378,19 +1378,34 @@ def test_softmax_over_two_rows_of_millions(frontend, hip):
     assert np.allclose(ref.reshape(shape), exact, rtol=1e-3, atol=0)
 
 
-@pytest.mark.parametrize("seed", range(64))
+def _held_to_error_bounds(frontend, seed, desc, fn, fn64, arrays, fuses=(True,)):
+    """HIP against the oracle and against float64, per element, by what float32 rounding can do to
+    the graph (tests/np_frontend.py): two float32 evaluations may differ by twice the bound."""
+    import np_frontend
+    exact, bound = np_frontend.evaluate(fn64, arrays)
+    for fuse in fuses:
+        ref, got = both(frontend, fn, arrays, fuse)
+        assert ref.shape == got.shape and ref.size == exact.size, desc
+        exact, bound = exact.reshape(ref.shape), bound.reshape(ref.shape)
+        tol = 2.0 * bound + 4 * np_frontend.U * np.abs(exact)
+        assert np.all(np.abs(got.astype(np.float64) - ref) <= tol), (desc, fuse, float(np.max(np.abs(got.astype(np.float64) - ref) / tol)))
+        assert np.all(np.abs(got.astype(np.float64) - exact) <= 0.5 * tol + 2 * np_frontend.U * np.abs(exact)), (desc, fuse)
+
+
+@pytest.mark.parametrize("seed", list(range(64)) + [1211])
 def test_random_graphs_match_the_oracle(frontend, hip, seed):
     """Differential test on seeded random graphs (tests/graph_fuzz.py): elementwise chains,
-    views, reductions over any axis, row normalisations, small contractions.  Held to the
-    reduction tolerance (every graph may contain a sum)."""
-    import graph_fuzz
+    views, reductions over any axis, row normalisations, small contractions.  Held per element to
+    the running error bound of a float64 evaluation of the same graph: seed 1211 ends in an
+    element of 0.0033 that the graph computes as a difference of values near one -- the oracle is
+    3.7e-6 off the float64 value there, more than a relative 2e-5 plus 2e-6 allows either side,
+    and the bound says 1.3e-4 is what float32 can do."""
+    import graph_fuzz, np_frontend
     shapes, fn, desc = graph_fuzz.build(seed, frontend)
+    _, fn64, _ = graph_fuzz.build(seed, np_frontend.Frontend)
     rng = RNG(seed)
     arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
-    ref, got = both(frontend, fn, arrays, True)
-    assert ref.shape == got.shape, desc
-    scale = max(1.0, float(np.abs(ref).max()))
-    assert np.allclose(got, ref, rtol=2e-5, atol=2e-6 * scale), desc
+    _held_to_error_bounds(frontend, seed, desc, fn, fn64, arrays)
 
 
 @pytest.mark.parametrize("seed", range(600, 624))
@@ -1441,14 +1456,7 @@ def test_random_large_graphs_match_the_oracle(frontend, hip, seed):
     _, fn64, _ = graph_fuzz.build(seed, np_frontend.Frontend, dims=graph_fuzz.LARGE_DIMS, max_rank=2)
     rng = RNG(seed)
     arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
-    exact, bound = np_frontend.evaluate(fn64, arrays)
-    for fuse in (True, False):
-        ref, got = both(frontend, fn, arrays, fuse)
-        assert ref.shape == got.shape and ref.size == exact.size, desc
-        exact, bound = exact.reshape(ref.shape), bound.reshape(ref.shape)
-        tol = 2.0 * bound + 4 * np_frontend.U * np.abs(exact)
-        assert np.all(np.abs(got.astype(np.float64) - ref) <= tol), (desc, fuse, float(np.max(np.abs(got.astype(np.float64) - ref) / tol)))
-        assert np.all(np.abs(got.astype(np.float64) - exact) <= 0.5 * tol + 2 * np_frontend.U * np.abs(exact)), (desc, fuse)
+    _held_to_error_bounds(frontend, seed, desc, fn, fn64, arrays, fuses=(True, False))
 
 
 LONG_LINE_SEEDS = [(7007, 0), (7052, 0), (7084, 0), (7092, 0), (7229, 0), (7264, 0), (7282, 0), (7284, 0), (7296, 0),
