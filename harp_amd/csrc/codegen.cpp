@@ -978,6 +978,7 @@ void apply_options(GenOptions* out, const std::string& text) {
     else if (k == "rematerialize") o.rematerialize = as_int() != 0;
     else if (k == "merge_launches") o.merge_launches = as_int() != 0;
     else if (k == "merge_templates") o.merge_templates = as_int() != 0;
+    else if (k == "gemm_tail") o.gemm_tail = as_int() != 0;
     else if (k == "lanes") o.lanes = std::max(1, as_int());
     else if (k == "lane_us") o.lane_us = std::max(0, as_int());
     else if (k == "gemm_epilogue") o.gemm_epilogue = as_int() != 0;

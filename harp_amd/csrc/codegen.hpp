@@ -34,6 +34,7 @@ struct GenOptions {
   int lane_us = 100;                  // launches estimated longer than this many microseconds stay on lane 0 (0: no limit)
   bool reindex = true;                // elementwise producers evaluated in a reader that walks another index space
   bool merge_launches = true;         // independent final reductions of a program (parameter updates) are issued as one launch
+  bool gemm_tail = true;               // a pooling reduce over a convolution's stored result runs in the convolution's launch
   bool merge_templates = true;        // ... and independent small MFMA contractions (template kernels) as one launch among themselves
   bool rematerialize = true;          // a cheap elementwise temp is evaluated again by a far reader of the same index space instead of being stored for it
   bool ranged_loads = true;           // a folded gather reads its source through a buffer resource: a guarded load is one load at an out-of-range offset where the guard fails

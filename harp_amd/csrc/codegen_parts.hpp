@@ -311,6 +311,8 @@ LaunchSpec emit_group(const Group& g, const GenOptions& opt, const std::map<std:
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan, const EpilogueSpec* epi = nullptr);
 LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestKernel*>& chain, const GenOptions& opt,
                               const std::map<std::string, size_t>& elems);
+bool window_reduce_tail(const NestKernel& r, const std::vector<const NestKernel*>& chain,
+                        const std::map<std::string, size_t>& elems, EpilogueSpec* epi);
 
 // ---- launches.cpp -----------------------------------------------------------------------------
 void mark_written(ProgramPlan* plan, const std::vector<const Node*>& kernels);

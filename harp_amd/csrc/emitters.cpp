@@ -1,4 +1,5 @@
 // Source text of the elementwise / reduce schedules.
+#include <cctype>
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -1039,6 +1040,192 @@ LaunchSpec emit_window_reduce(const NestKernel& r, const std::vector<const NestK
     if (e != elems.end() && counted.insert(b).second) ls.algo_bytes += 4.0 * static_cast<double>(e->second);
   }
   return ls;
+}
+
+// The same reduce as a function of an output's position, for the launch that produces its source
+// to call once a workgroup has stored what that output reads (EpilogueSpec's tail).  Only the
+// plain case: r reads nothing but the window buffer, no gather of the chain is guarded, and the
+// source is a buffer the epilogue stores.  False when it does not apply.
+bool window_reduce_tail(const NestKernel& r, const std::vector<const NestKernel*>& chain,
+                        const std::map<std::string, size_t>& elems, EpilogueSpec* epi) {
+  if (chain.empty() || !r.out_aff || r.acc_dtype.ty != Ty::F32 || r.out_dtype.ty != Ty::F32) return false;
+  std::vector<LoadRef> deep;
+  collect_loads(*chain.back()->value, deep);
+  if (deep.empty() || deep[0].load->args[0]->op != Op::Var) return false;
+  const std::string src = deep[0].load->args[0]->name;
+  if (std::find(epi->bufs.begin(), epi->bufs.end(), src) == epi->bufs.end()) return false;
+  const std::string T = chain[0]->out_buf;
+  std::vector<LoadRef> rloads;
+  collect_loads(*r.value, rloads);
+  for (const auto& lr : rloads)
+    if (lr.load->args[0]->op != Op::Var || lr.load->args[0]->name != T || lr.guarded || !affine_of(*lr.load->args[1])) return false;
+  for (const auto* g : chain) {
+    std::vector<LoadRef> gl;
+    collect_loads(*g->value, gl);
+    for (const auto& lr : gl)
+      if (lr.guarded || lr.load->args[0]->op != Op::Var || !affine_of(*lr.load->args[1]) || !g->out_aff) return false;
+  }
+  int64_t N = 1;
+  std::vector<Loop> live;
+  for (const auto& l : r.loops) {
+    N *= l.extent;
+    if (l.extent > 1) live.push_back(l);
+  }
+  auto big = [&](const std::string& b) {
+    auto it = elems.find(b);
+    return it == elems.end() || it->second >= static_cast<size_t>(kIndex32Limit);
+  };
+  if (N >= kIndex32Limit || big(src) || big(r.out_buf)) return false;
+  for (const auto* g : chain)
+    if (big(g->out_buf)) return false;
+  // dense output in the order of r's loops: a workgroup's share is a run of positions
+  {
+    int64_t stride = 1;
+    for (size_t i = r.loops.size(); i-- > 0;) {
+      if (r.loops[i].extent > 1 && r.out_aff->of(r.loops[i].var) != stride) return false;
+      stride *= r.loops[i].extent;
+    }
+    if (r.out_aff->c != 0 || r.out_aff->of(r.rloop.var) != 0) return false;
+  }
+  std::ostringstream os;
+  os << "// the reduce " << r.name << " over windows of " << src << ", by the position of its output\nnamespace eh_tail_ns {\ntypedef int idx_t;\n";
+  for (size_t j = chain.size(); j-- > 0;)
+    os << gather_fn_text(*chain[j], src, j + 1 < chain.size() ? chain[j + 1] : nullptr, "idx_t");
+  std::string sig;
+  epi->tail_params.clear();
+  epi->tail_args.clear();
+  epi->tail_bufs.clear();
+  epi->tail_min_bytes.clear();
+  bool src_listed = false;
+  for (const auto& p : r.params) {
+    std::string name = p.name;
+    if (name == T) name = src;
+    if (name == src) {
+      if (src_listed) continue;
+      src_listed = true;
+    }
+    if (name != src && name != r.out_buf) return false;
+    const std::string decl = std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + name;
+    sig += ", " + decl;
+    epi->tail_args += ", " + (name == src ? std::string("eh_tail_lds") : name);
+    if (name != src) {
+      if (std::find(epi->bufs.begin(), epi->bufs.end(), name) != epi->bufs.end()) return false;
+      epi->tail_params += ", " + decl;
+      epi->tail_bufs.push_back(name);
+      epi->tail_min_bytes.push_back(static_cast<size_t>(N) * 4);
+    }
+  }
+  if (!src_listed || epi->tail_bufs.size() != 1) return false;
+  os << "__device__ __forceinline__ void eh_tail(const idx_t eh_o" << sig << ") {\n";
+  os << "  idx_t eh_rem = eh_o;\n  __builtin_assume(eh_rem >= 0);\n";
+  for (size_t q = live.size(); q-- > 0;) {
+    os << "  const idx_t " << live[q].var << " = eh_rem % " << live[q].extent << ";\n";
+    if (q) os << "  eh_rem /= " << live[q].extent << ";\n";
+  }
+  for (const auto& l : r.loops)
+    if (l.extent == 1) os << "  const idx_t " << l.var << " = 0;\n";
+  ExprRenderer er;
+  std::vector<Loop> rvars = r.loops;
+  rvars.push_back(r.rloop);
+  er.load_hook = [&](const Node& ld, std::string* out) {
+    if (ld.args[0]->op != Op::Var || ld.args[0]->name != T) return false;
+    *out = gather_call(*chain[0], src, *ld.args[1], rvars, "idx_t");
+    return true;
+  };
+  os << "  float acc = " << literal(*r.identity) << ";\n#pragma unroll\n";
+  os << "  for (idx_t " << r.rloop.var << " = 0; " << r.rloop.var << " < " << r.rloop.extent << "; ++" << r.rloop.var << ") {\n";
+  os << "    acc = " << combine_text(r.rkind, r.acc_dtype, "acc", "(float)(" + er.expr(*r.value) + ")") << ";\n  }\n";
+  os << "  " << r.out_buf << "[eh_o] = acc;\n}\n}  // namespace eh_tail_ns\n";
+  epi->tail_function = os.str();
+  // The launch keeps its workgroup's share of the source in LDS (eh_tail_lds, element e of the
+  // source at e - EH_TAIL_BASE): the tail reads it there, and wherever the epilogue stores the
+  // source it stores into LDS as well.
+  {
+    std::string& t = epi->tail_function;
+    const std::string from = src + "[", to = src + "[-(idx_t)EH_TAIL_BASE + ";
+    size_t n_loads = 0;
+    for (size_t q = t.find(from); q != std::string::npos; q = t.find(from, q + to.size())) {
+      if (q > 0 && (std::isalnum(static_cast<unsigned char>(t[q - 1])) || t[q - 1] == '_')) continue;
+      t.replace(q, from.size(), to);
+      ++n_loads;
+    }
+    if (n_loads == 0) return false;
+    size_t n_stores = 0;
+    auto twin = [&](std::string* text) {
+      const std::string scalar = "    " + src + "[eh_e] = eh_v_" + src + ";\n";
+      for (size_t q = text->find(scalar); q != std::string::npos; q = text->find(scalar, q)) {
+        const std::string add = scalar + "#ifdef EH_TAIL\n    eh_tail_lds[eh_e - EH_TAIL_BASE] = eh_v_" + src + ";\n#endif\n";
+        text->replace(q, scalar.size(), add);
+        q += add.size();
+        ++n_stores;
+      }
+      const std::string quad = "    *reinterpret_cast<EhQ<float>*>(" + src + " + eh_e) = ";
+      for (size_t q = text->find(quad); q != std::string::npos; q = text->find(quad, q)) {
+        const size_t end = text->find(";\n", q);
+        if (end == std::string::npos) break;
+        const std::string value = text->substr(q + quad.size(), end - q - quad.size());
+        const std::string add = "#ifdef EH_TAIL\n    *reinterpret_cast<EhQ<float>*>(eh_tail_lds + (eh_e - EH_TAIL_BASE)) = " + value + ";\n#endif\n";
+        text->insert(end + 2, add);
+        q = end + 2 + add.size();
+        ++n_stores;
+      }
+    };
+    twin(&epi->function);
+    twin(&epi->split_functions);
+    twin(&epi->quad_functions);
+    if (n_stores == 0) return false;
+  }
+  epi->tail_source = src;
+  epi->tail_outputs = N;
+  epi->tail_bytes = 4.0 * static_cast<double>(N);
+  epi->tail_tag = "window-reduce(window=" + std::to_string(r.rloop.extent) + ",gathers=" + std::to_string(chain.size()) + ")";
+  epi->tail_kernels.clear();
+  for (size_t j = chain.size(); j-- > 0;) epi->tail_kernels.push_back(chain[j]->name);
+  epi->tail_kernels.push_back(r.name);
+  // which elements of the source an output reads: the chain's index maps, evaluated on the host
+  const NestKernel rk = r;
+  std::vector<NestKernel> gs;
+  for (const auto* g : chain) gs.push_back(*g);
+  epi->tail_reads = [rk, gs, T](int64_t o, std::vector<int64_t>* out) {
+    std::map<std::string, int64_t> val;
+    int64_t rem = o;
+    for (size_t q = rk.loops.size(); q-- > 0;) {
+      val[rk.loops[q].var] = rem % rk.loops[q].extent;
+      rem /= rk.loops[q].extent;
+    }
+    auto eval = [](const Affine& a, const std::map<std::string, int64_t>& v) {
+      int64_t x = a.c;
+      for (const auto& kv : a.coef) {
+        auto it = v.find(kv.first);
+        x += kv.second * (it == v.end() ? 0 : it->second);
+      }
+      return x;
+    };
+    std::vector<LoadRef> rl;
+    collect_loads(*rk.value, rl);
+    for (int64_t j = 0; j < rk.rloop.extent; ++j) {
+      val[rk.rloop.var] = j;
+      std::vector<int64_t> at;                       // positions in the current buffer
+      for (const auto& lr : rl) at.push_back(eval(*affine_of(*lr.load->args[1]), val));
+      for (const auto& g : gs) {
+        std::vector<LoadRef> gl;
+        collect_loads(*g.value, gl);
+        std::vector<int64_t> next;
+        for (int64_t pos : at) {
+          std::map<std::string, int64_t> gv;         // g's loops from a position in its dense output
+          int64_t pr = pos;
+          for (size_t q = g.loops.size(); q-- > 0;) {
+            gv[g.loops[q].var] = pr % g.loops[q].extent;
+            pr /= g.loops[q].extent;
+          }
+          for (const auto& lr : gl) next.push_back(eval(*affine_of(*lr.load->args[1]), gv));
+        }
+        at = std::move(next);
+      }
+      out->insert(out->end(), at.begin(), at.end());
+    }
+  };
+  return true;
 }
 
 void emit_serial_reduce(const NestKernel& k, const GenOptions& opt, ProgramPlan* plan, const EpilogueSpec* epi) {

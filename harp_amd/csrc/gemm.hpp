@@ -7,6 +7,7 @@
 #pragma once
 
 #include <map>
+#include <functional>
 #include <optional>
 
 #include "analysis.hpp"
@@ -87,6 +88,22 @@ struct EpilogueSpec {
   //   void eh_epilogue_apply4(long long eh_e, const float (&eh_acc)[4], const EhEpiLoads4&, [C,] <params>);
   std::string quad_functions;
   int quad_regs = 0;                   // registers EhEpiLoads4 takes
+  // A tail: a short reduce over windows of a buffer this epilogue stores (the pooling behind a
+  // convolution), offered to schedules whose workgroup stores a closed share of that buffer -- the
+  // workgroup then also computes the reduce's outputs that read its share, once its stores are
+  // done.  Filled by window_reduce_tail; a schedule that takes it lists tail_kernels in its launch.
+  //   namespace eh_tail_ns { void eh_tail(idx_t output, <tail's own parameters>); }
+  std::string tail_function;
+  std::string tail_params;             // parameters the launch does not have yet, ", float* __restrict__ buf41"
+  std::string tail_args;               // ", buf31, buf41": every parameter of eh_tail, by buffer name
+  std::string tail_source;             // the stored buffer it reads
+  std::string tail_tag;                // for the schedule string
+  std::vector<std::string> tail_bufs;  // buffers of tail_params, in order
+  std::vector<size_t> tail_min_bytes;
+  std::vector<std::string> tail_kernels;
+  int64_t tail_outputs = 0;            // outputs of the reduce; a workgroup's share is a run of them
+  double tail_bytes = 0;
+  std::function<void(int64_t, std::vector<int64_t>*)> tail_reads;   // elements of tail_source that output o reads
 };
 
 // True when element (b, m, n) of C sits at (b*M + m)*N + n, the index an epilogue is written for.

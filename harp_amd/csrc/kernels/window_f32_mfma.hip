@@ -100,6 +100,13 @@ __device__ __forceinline__ long long ew_c_b(long long bz) { (void)bz; return 0; 
 #define EH_EPI_PARAMS
 #define EH_EPI_ARGS
 #endif
+// EH_TAIL: a short reduce over windows of a buffer the epilogue stores (the pooling behind a
+// convolution).  Group g's EH_TAIL_PER_GROUP outputs read only what workgroup g stores, which the
+// epilogue also keeps in LDS (eh_tail_lds): the workgroup computes those outputs itself at the
+// end, eh_tail_ns::eh_tail(output, buffers...).  Not with EH_PART (the block is found by blockIdx).
+#ifndef EH_TAIL
+#define EH_TAIL_PARAMS
+#endif
 #ifdef EH_NO_C
 #define EH_C_PARAM
 #define EH_C_ARG
@@ -132,14 +139,14 @@ template <int V> struct EwInt { static constexpr int value = V; };
 // launch's one block of LDS, which the parts use in turn; eh_lds_floats says how much it needs.
 #ifdef EH_PART
 constexpr int eh_lds_floats = ((EW_PATCH_FLOATS + 3) & ~3) + EW_WAVES_M * EW_MB * 16 * EW_A_LDS;
-__device__ __forceinline__ void eh_run(const unsigned eh_bx, float* const eh_lds, const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS) {
+__device__ __forceinline__ void eh_run(const unsigned eh_bx, float* const eh_lds, const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS EH_TAIL_PARAMS) {
   constexpr int MROWS = EW_WAVES_M * EW_MB * 16;
   float* const patch = eh_lds;
   float* const As = eh_lds + ((EW_PATCH_FLOATS + 3) & ~3);
   const long long g = eh_bx % EH_PART_GX, bz = eh_bx / EH_PART_GX;
 #else
 extern "C" __global__ void __launch_bounds__(EW_NT)
-EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS) {
+EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_EPI_PARAMS EH_TAIL_PARAMS) {
   constexpr int MROWS = EW_WAVES_M * EW_MB * 16;        // rows of A a workgroup multiplies (padding rows are zero)
   __shared__ __attribute__((aligned(16))) float patch[EW_PATCH_FLOATS];
   __shared__ __attribute__((aligned(16))) float As[MROWS * EW_A_LDS];
@@ -408,5 +415,16 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
 #endif
 #if EW_PASSES > 3
   pass(EwInt<3>{});
+#endif
+#ifdef EH_TAIL
+  // The epilogue has put this workgroup's results into eh_tail_lds as well.  The barrier waits for
+  // those LDS stores only, not for the stores to memory; the waves that only fetched have left,
+  // the multiplying waves share the outputs.  Unrolled: a work-item's outputs are independent.
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  constexpr int EW_TT = EW_WAVES_M * EW_WAVES_N * 64;
+  constexpr int EW_TAIL_FULL = EH_TAIL_PER_GROUP / EW_TT;
+#pragma unroll 8
+  for (int q = 0; q < EW_TAIL_FULL; ++q) eh_tail_ns::eh_tail((int)g * EH_TAIL_PER_GROUP + tid + q * EW_TT EH_TAIL_ARGS);
+  if (EW_TAIL_FULL * EW_TT + tid < EH_TAIL_PER_GROUP) eh_tail_ns::eh_tail((int)g * EH_TAIL_PER_GROUP + EW_TAIL_FULL * EW_TT + tid EH_TAIL_ARGS);
 #endif
 }

@@ -70,7 +70,7 @@ void issue_independent_launches_together(ProgramPlan* plan, const std::vector<co
   // launch's, so these go out among themselves, never with kernels that want many workgroups a CU.
   auto template_part = [&](const LaunchSpec& ls) {
     return !ls.part_params.empty() && ls.block[0] == 256 && ls.block[1] == 1 && ls.block[2] == 1 && !ls.lds_bytes &&
-           ls.flops <= 4e9 && !ls.kernels.empty() && opt.merge_templates;
+           ls.flops <= 4e9 && !ls.kernels.empty() && opt.merge_templates && ls.schedule.find(",tail=") == std::string::npos;
   };
   auto size_class = [&](const LaunchSpec& ls) { return ls.block[0] * 2 + (template_part(ls) ? 1u : 0u); };
   auto mergeable = [&](const LaunchSpec& ls) {

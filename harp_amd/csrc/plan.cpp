@@ -581,7 +581,38 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
           have_epi = build_epilogue(i, k0, gs->batch * gs->M * gs->N, true, k0r, epi, after);
         }
       }
+      // A pooling reduce over what the epilogue stores (read through its gathers) is offered to the
+      // contraction as a tail: a schedule whose workgroups each store a closed share of that buffer
+      // lets them compute the reduce's outputs over their share, and the reduce's launch goes.
+      size_t tail_of = kernels.size();
+      if (have_epi && opt.fuse && opt.window && opt.reindex && opt.gemm_tail) {
+        for (const auto& w : windows) {
+          const size_t ri = w.first;
+          if (ri < after || folded_kernels.count(ri) || absorbed.count(ri) || !nests[ri]) continue;
+          std::vector<const NestKernel*> chain;
+          for (size_t q : w.second) chain.push_back(&*nests[q]);
+          // nothing between here and the reduce may write what it writes or read it
+          bool free_to_move = true;
+          for (size_t m = after; m < ri && free_to_move; ++m) {
+            if (folded_kernels.count(m) || absorbed.count(m)) continue;
+            for (const auto& pm : kernels[m]->params) free_to_move = free_to_move && pm.name != nests[ri]->out_buf;
+          }
+          if (!free_to_move) continue;
+          if (window_reduce_tail(*nests[ri], chain, elems, &epi)) {
+            tail_of = ri;
+            break;
+          }
+        }
+      }
       auto gl = try_emit_gemm(have_epi ? k0r : k0, lopt, &plan.buffers, &folded, have_epi ? &epi : nullptr);
+      if (!gl.empty() && tail_of < kernels.size()) {
+        // taken when the launch lists the reduce among its kernels
+        const auto& ks = gl.back().kernels;
+        if (std::find(ks.begin(), ks.end(), nests[tail_of]->name) != ks.end()) {
+          folded_kernels.insert(tail_of);
+          windows.erase(tail_of);
+        }
+      }
       if (!gl.empty()) {
         if (absorbed_name.count(i)) gl.back().kernels.push_back(absorbed_name[i]);
         // K was split and the next kernel only sums the (dense) result over the batch axis: it

@@ -476,12 +476,62 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
      << "\n#define EW_KPAD " << kpad << "\n#define EW_A_LDS " << a_lds << "\n";
   os << "#define EW_SRC_BYTES " << p.f_bytes << "u\n";
   os << "#define EW_MIX " << (opt.gemm_mix ? 1 : 0) << "\n#define EW_C_VEC " << (c_quad ? 4 : 1) << "\n#define EW_PASSES " << passes << "\n";
+  // The epilogue's tail (a pooling reduce over what this launch stores): taken when the outputs
+  // split evenly over the groups, group g's outputs read nothing outside the block of the stored
+  // buffer that workgroup g writes -- checked on the first two groups and the last by walking
+  // every address either side touches -- and that block fits into LDS beside the tiles: the
+  // epilogue then stores its results there as well, and the tail reads them back from LDS behind
+  // a barrier that does not wait for the stores to memory.
+  bool tail = false;
+  int64_t tail_per_group = 0, tail_block = 0, tail_lo = 0;
+  if (epilogue && !epilogue->tail_function.empty() && epilogue->tail_reads && batch == 1 && groups > 0 &&
+      epilogue->tail_outputs % groups == 0 && !epilogue->store_c) {
+    tail_per_group = epilogue->tail_outputs / groups;
+    tail_block = M * NG;
+    auto digit_sum = [&](const std::vector<size_t>& which, int64_t v) {
+      int64_t o = 0;
+      for (size_t q : which) o += ((v / loops[q].unit) % loops[q].w.extent) * loops[q].w.c;
+      return o;
+    };
+    tail = tail_block <= (int64_t{1} << 16) && tail_block % 4 == 0 &&
+           (patch_floats + mrows * a_lds + tail_block) * 4 + 64 <= 160 * 1024;
+    std::set<int64_t> gs = {0, std::min<int64_t>(1, groups - 1), groups - 1};
+    for (int64_t g : gs) {
+      if (!tail) break;
+      int64_t lo = INT64_MAX, hi = INT64_MIN;
+      for (int64_t m = 0; m < M; ++m) {
+        const int64_t cm = digit_sum(m_loops, m);
+        for (int64_t n = g * NG; n < (g + 1) * NG; ++n) {
+          const int64_t at = p.c_c0 + cm + digit_sum(row_loops, n);
+          lo = std::min(lo, at);
+          hi = std::max(hi, at);
+        }
+      }
+      if (g == 0) tail_lo = lo;
+      // a closed block, every element written, group g's right behind group g - 1's
+      tail = hi - lo + 1 == tail_block && lo == tail_lo + g * tail_block && tail_lo % 4 == 0;
+      std::vector<int64_t> reads;
+      for (int64_t o = g * tail_per_group; o < (g + 1) * tail_per_group && tail; ++o) {
+        reads.clear();
+        epilogue->tail_reads(o, &reads);
+        for (int64_t at : reads) tail = tail && at >= lo && at <= hi;
+      }
+    }
+  }
+  if (tail) {
+    os << "#define EH_TAIL 1\n#define EH_TAIL_PER_GROUP " << tail_per_group << "\n#define EH_TAIL_BLOCK " << tail_block
+       << "\n#define EH_TAIL_BASE ((long long)blockIdx.x * " << tail_block << "LL + " << tail_lo << "LL)\n"
+       << "#define EH_TAIL_PARAMS " << epilogue->tail_params << "\n#define EH_TAIL_ARGS " << epilogue->tail_args << "\n"
+       << "// the workgroup's share of " << epilogue->tail_source << ", kept for the tail\n"
+       << "__shared__ __attribute__((aligned(16))) float eh_tail_lds[EH_TAIL_BLOCK];\n";
+  }
   if (epilogue) {
     os << "#define EH_EPILOGUE 1\n#define EH_EPI_PARAMS " << epilogue->params << "\n#define EH_EPI_ARGS " << epilogue->args << "\n";
     if (!epilogue->store_c) os << "#define EH_NO_C 1\n";
     os << epilogue->function;
     if (!epilogue->split_functions.empty()) os << "#define EH_EPILOGUE_SPLIT " << epilogue->n_loads << "\n" << epilogue->split_functions;
     if (c_quad) os << "#define EH_EPILOGUE_QUAD " << std::max(1, epilogue->quad_regs) << "\n" << epilogue->quad_functions;
+    if (tail) os << epilogue->tail_function;
   }
   auto table = [&](const char* name, const std::vector<int64_t>& vals) {
     os << "constexpr int " << name << "[" << vals.size() << "] = {";
@@ -590,12 +640,13 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
   os << kWindowSource;
   ls.source = os.str();
   ls.part_params = std::string("const float* __restrict__ A, const float* __restrict__ F") +
-                   (epilogue && !epilogue->store_c ? "" : ", float* __restrict__ C") + (epilogue ? epilogue->params : "");
+                   (epilogue && !epilogue->store_c ? "" : ", float* __restrict__ C") + (epilogue ? epilogue->params : "") +
+                   (tail ? epilogue->tail_params : "");
   ls.schedule = "mfma16x16x4(window,group=" + std::to_string(NG) + ",M=" + std::to_string(M) + ",K=" + std::to_string(K) +
                 ",waves=" + std::to_string(lay.waves_m) + "x" + std::to_string(lay.waves_n) + ",blocks=" + std::to_string(lay.mb) +
                 "x" + std::to_string(lay.nb) + ",steps=" + std::to_string(ksteps) + ",patterns=" + std::to_string(patterns.size()) +
-                ",lds=" + std::to_string((patch_floats + mrows * a_lds) * 4) + "B" + (c_quad ? ",C:x4" : "") + (passes > 1 ? ",passes=" + std::to_string(passes) : std::string()) + p.tag +
-                (epilogue ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + ")";
+                ",lds=" + std::to_string((patch_floats + mrows * a_lds + (tail ? tail_block : 0)) * 4) + "B" + (c_quad ? ",C:x4" : "") + (passes > 1 ? ",passes=" + std::to_string(passes) : std::string()) + p.tag +
+                (epilogue ? ",epilogue=" + std::to_string(epilogue->kernels.size()) : "") + (tail ? ",tail=" + epilogue->tail_tag : "") + ")";
   ls.grid[0] = static_cast<unsigned>(groups);
   ls.grid[1] = 1;
   ls.grid[2] = static_cast<unsigned>(batch);
@@ -618,6 +669,13 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
       ls.arg_min_bytes.push_back(epilogue->min_bytes[i]);
     }
     for (const auto& n : epilogue->kernels) ls.kernels.push_back(n);
+    if (tail) {
+      for (size_t i = 0; i < epilogue->tail_bufs.size(); ++i) {
+        ls.arg_bufs.push_back(epilogue->tail_bufs[i]);
+        ls.arg_min_bytes.push_back(epilogue->tail_min_bytes[i]);
+      }
+      for (const auto& n : epilogue->tail_kernels) ls.kernels.push_back(n);
+    }
   }
   ls.flops = 2.0 * static_cast<double>(M) * static_cast<double>(N) * static_cast<double>(K) * static_cast<double>(batch);
   {
@@ -627,7 +685,8 @@ std::vector<LaunchSpec> emit_window(const WindowProblem& p, const GenOptions& op
     const double a_bytes = 4.0 * static_cast<double>(M) * K * (a_moves ? nb : 1.0);
     const double f_bytes = p.f_algo_bytes > 0 ? p.f_algo_bytes : 4.0 * static_cast<double>(K) * N * nb;
     const double c_bytes = 4.0 * nb * static_cast<double>(M) * N;
-    ls.algo_bytes = a_bytes + f_bytes + (epilogue && !epilogue->store_c ? 0.0 : c_bytes) + (epilogue ? epilogue->bytes : 0.0);
+    ls.algo_bytes = a_bytes + f_bytes + (epilogue && !epilogue->store_c ? 0.0 : c_bytes) + (epilogue ? epilogue->bytes : 0.0) +
+                    (tail ? epilogue->tail_bytes : 0.0);
   }
   return {ls};
 }

@@ -157,16 +157,19 @@ def test_lanes_change_nothing_but_the_timing(hip):
 
 def test_contractions_issued_together_change_nothing_but_the_timing(hip):
     """A layer's input gradient and weight gradient as one launch (the kernel templates compiled
-    as parts that share the launch's block of LDS) and as launches of their own: the same
-    arithmetic on the same inputs, so every output of the CNN training step is equal bit for bit
-    -- also on back-to-back executes and as a recorded graph."""
+    as parts that share the launch's block of LDS) and as launches of their own; the poolings as
+    tails of their convolutions' launches and as launches of their own: the same arithmetic on
+    the same inputs, so every output of the CNN training step is equal bit for bit -- also on
+    back-to-back executes and as a recorded graph."""
     hb = hip
     dev = hb.HipDevice(0)
     want = None
-    for options in ("merge_templates=0", None):
+    for options in ("merge_templates=0,gemm_tail=0", "gemm_tail=0", None):
         prog, sets, arg_names, outs, arrays = _cnn_sets(hb, dev, 32, seed=95, options=options)
         pairs = [l for l in prog.launches if l["schedule"].startswith("together(mfma")]
-        assert len(pairs) == (0 if options else 3), [l["schedule"] for l in prog.launches]
+        assert len(pairs) == (0 if options and "merge_templates" in options else 3), [l["schedule"] for l in prog.launches]
+        # (and the poolings in their convolutions' launches, reading the workgroup's results from LDS)
+        assert sum(",tail=" in l["schedule"] for l in prog.launches) == (0 if options else 2)
         for _ in range(2):
             prog.run(sets[0][0], sync=False)
         dev.sync()

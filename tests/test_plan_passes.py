@@ -88,18 +88,19 @@ def test_read_windows_through_their_gathers(cnn_ast):
     convolution's output through the gathers' index maps: one launch, no window buffer.  What the
     gather reads is max(z, 0) of a pre-activation z that the backward pass needs anyway: the
     reduce applies that as well, and the convolution stores z only.  window=0 launches the
-    gather; rematerialize=0 keeps the stored activation."""
-    plan = _plan(cnn_ast)
+    gather; rematerialize=0 keeps the stored activation.  (gemm_tail=0: the pooling as a launch
+    of its own.)"""
+    plan = _plan(cnn_ast, "gemm_tail=0")
     pool = _covering(plan, "R_256_32_14_14_1_7")
     assert pool["kernels"][:3] == ["E_256_32_28_28_5", "E_256_32_14_14_2_2_6", "R_256_32_14_14_1_7"]
     assert "window-reduce(window=4,gathers=2)" in pool["schedule"] and "fmaxf(buf31[" in pool["source"]
     conv = _covering(plan, "R_256_784_32_1_1")
     assert "E_256_32_28_28_5" not in conv["kernels"] and sum(conv["written"]) == 1
     assert any(b["name"] == "buf37" and b["elided"] for b in plan.buffers)
-    stored = _plan(cnn_ast, "rematerialize=0")
+    stored = _plan(cnn_ast, "rematerialize=0,gemm_tail=0")
     assert "E_256_32_28_28_5" in _covering(stored, "R_256_784_32_1_1")["kernels"]
     assert "window-reduce(window=4,gathers=1)" in _covering(stored, "R_256_32_14_14_1_7")["schedule"]
-    off = _plan(cnn_ast, "window=0")
+    off = _plan(cnn_ast, "window=0,gemm_tail=0")
     assert "E_256_32_14_14_2_2_6" not in _covering(off, "R_256_32_14_14_1_7")["kernels"]
     assert len(off.launches) > len(plan.launches)
 
@@ -108,7 +109,7 @@ def test_join_shifted_sums_with_their_contraction(cnn_ast):
     """The second convolution's input gradient: dY x W, then eight kernels adding up nine shifted,
     guarded reads of the product.  One window contraction over (channel, shift) covers all nine
     kernels; gemm_window=0 keeps the product and the sums apart."""
-    plan = _plan(cnn_ast, "merge_templates=0")
+    plan = _plan(cnn_ast, "merge_templates=0,gemm_tail=0")
     dx = _covering(plan, "R_256_196_1_288_59")
     assert dx["kernels"][1:] == ["E_256_32_16_16_%d" % q for q in range(60, 68)] and "shifts=9" in dx["schedule"]
     off = _plan(cnn_ast, "gemm_window=0,merge_templates=0")
@@ -139,3 +140,28 @@ def test_issue_independent_contractions_together(cnn_ast):
     assert "split-k=2" in fc["schedule"] and fc["grid"] == [196 + 98 * 2, 1, 1] and "#define EH_PART_GY 2u" in fc["source"]
     apart = _plan(cnn_ast, "merge_templates=0")
     assert len(apart.launches) == len(plan.launches) + 3 and not any(l["schedule"].startswith("together(mfma") for l in apart.launches)
+
+
+def test_pooling_runs_in_the_convolution_launch(cnn_ast):
+    """The pooling reduce reads the convolution's stored pre-activation through its gathers, and one
+    image's pooled outputs read only that image's block, which is what one workgroup of the window
+    schedule stores.  The reduce is offered to the contraction as a tail: the epilogue keeps the
+    block in LDS as well (beside the tiles: 158 812 of 163 840 bytes for the second convolution),
+    and behind a barrier that waits for LDS only the workgroup computes its image's pooled outputs.
+    Two launches less; gemm_tail=0 keeps the poolings as launches."""
+    from harp_amd import backend as hb
+    plan = _plan(cnn_ast)
+    for conv, pool, z, per_image, block in (("R_256_784_32_1_1", "R_256_32_14_14_1_7", "buf31", 6272, 25088),
+                                            ("R_256_196_64_1_9", "R_256_64_7_7_1_15", "buf47", 3136, 12544)):
+        l = _covering(plan, conv)
+        assert l is _covering(plan, pool) and ",tail=window-reduce(window=4,gathers=2)" in l["schedule"]
+        src = l["source"]
+        assert "#define EH_TAIL_PER_GROUP %d\n" % per_image in src and "#define EH_TAIL_BLOCK %d\n" % block in src
+        # every store of the pre-activation has its twin into LDS, and the tail reads LDS
+        assert src.count("eh_tail_lds[eh_e - EH_TAIL_BASE] = eh_v_" + z) == 2
+        assert src.count("*reinterpret_cast<EhQ<float>*>(eh_tail_lds + (eh_e - EH_TAIL_BASE))") == 1
+        assert "fmaxf(%s[-(idx_t)EH_TAIL_BASE + " % z in src and "#define EH_TAIL_ARGS , eh_tail_lds, " in src
+        assert int(l["schedule"].split("lds=")[1].split("B")[0]) <= 160 * 1024
+        assert len(hb.compile_source(src)) > 1000
+    apart = _plan(cnn_ast, "gemm_tail=0")
+    assert len(apart.launches) == len(plan.launches) + 2 and not any(",tail=" in l["schedule"] for l in apart.launches)
