@@ -99,11 +99,12 @@ int eh_buffer_device_ptr(eh_buffer* buf, void** ptr);
  *      arch, fuse, vectorize, transpose, window, row_threads, row_elems, flat_block, flat_iters, gemm, gemm_bm,
  *      gemm_bn, gemm_bk, gemm_wm, gemm_wn, gemm_split_k, gemm_waves, gemm_setprio, gemm_fold, gemm_window, window_passes,
  *      gemm_epilogue, gemm_dma, gemm_mix, gemm_prefetch, gemm_transpose, gemm_merge_batch, nontemporal,
- *      normalize, allow_serial, reindex, rematerialize, merge_launches, merge_templates, guard_branches, ranged_loads,
+ *      normalize, allow_serial, reindex, rematerialize, merge_launches, merge_templates, gemm_tail, guard_branches, ranged_loads,
  *      lanes, lane_us.
  *      merge_launches (default 1): launches of a program that do not depend on each other go out as one launch;
  *      merge_templates (default 1): so do small MFMA contractions among themselves (a layer's input and weight
- *      gradient), each a part of the launch that uses the launch's LDS in turn.
+ *      gradient), each a part of the launch that uses the launch's LDS in turn; gemm_tail (default 1): a pooling
+ *      reduce over a convolution's stored result is computed by the convolution's workgroups from LDS.
  *      lanes (default 1; 2 or more): launches of a program that do not depend on each other are spread
  *      over that many streams (lane 0 is the device's stream; a program's execute forks the side
  *      lanes off it and joins them back, so callers still see one stream); launches estimated
