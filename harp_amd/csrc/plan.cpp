@@ -716,7 +716,9 @@ ProgramPlan plan_program(const Node& program, const GenOptions& opt) {
       if (pick.ok && (!aligned_with_group(g, pick.stage) || g.producer(pick.stage.out_buf))) pick.ok = false;
       return pick;
     };
-    while (opt.fuse && i < kernels.size() && nests[i] && !folded_kernels.count(i)) {
+    // (a reduce that reads through its gathers, or a contraction with its shifted sums, has a
+    // launch of its own planned: its operands are not in memory for a stage of this group to read)
+    while (opt.fuse && i < kernels.size() && nests[i] && !folded_kernels.count(i) && !windows.count(i) && !scattered.count(i)) {
       if (absorbed.count(i)) {
         ++i;
         continue;
