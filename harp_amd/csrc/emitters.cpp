@@ -1116,12 +1116,27 @@ bool window_reduce_tail(const NestKernel& r, const std::vector<const NestKernel*
     }
   }
   if (!src_listed || epi->tail_bufs.size() != 1) return false;
-  os << "__device__ __forceinline__ void eh_tail(const idx_t eh_o" << sig << ") {\n";
-  os << "  idx_t eh_rem = eh_o;\n  __builtin_assume(eh_rem >= 0);\n";
-  for (size_t q = live.size(); q-- > 0;) {
-    os << "  const idx_t " << live[q].var << " = eh_rem % " << live[q].extent << ";\n";
-    if (q) os << "  eh_rem /= " << live[q].extent << ";\n";
+  // output eh_l of group eh_g.  Where a group is one step of the outermost loop, only the inner
+  // loops are decoded, from the small number (the workgroup has its SIMDs to itself: every
+  // integer division of the decode is time nothing else hides).
+  os << "__device__ __forceinline__ void eh_tail(const idx_t eh_g, const idx_t eh_l" << sig << ") {\n";
+  os << "  const idx_t eh_o = eh_g * EH_TAIL_PER_GROUP + eh_l;\n";
+  int64_t inner = 1;
+  for (size_t q = 1; q < live.size(); ++q) inner *= live[q].extent;
+  if (!live.empty()) {
+    os << "#if EH_TAIL_PER_GROUP == " << inner << "\n  unsigned eh_rem = (unsigned)eh_l;\n";
+    for (size_t q = live.size(); q-- > 1;) {
+      os << "  const idx_t " << live[q].var << " = (idx_t)(eh_rem % " << live[q].extent << "u);\n";
+      if (q > 1) os << "  eh_rem /= " << live[q].extent << "u;\n";
+    }
+    os << "  const idx_t " << live[0].var << " = eh_g;\n#else\n";
   }
+  os << "  unsigned eh_rem = (unsigned)eh_o;\n";
+  for (size_t q = live.size(); q-- > 0;) {
+    os << "  const idx_t " << live[q].var << " = (idx_t)(eh_rem % " << live[q].extent << "u);\n";
+    if (q) os << "  eh_rem /= " << live[q].extent << "u;\n";
+  }
+  if (!live.empty()) os << "#endif\n";
   for (const auto& l : r.loops)
     if (l.extent == 1) os << "  const idx_t " << l.var << " = 0;\n";
   ExprRenderer er;

@@ -424,7 +424,7 @@ EW_ENTRY(const float* __restrict__ A, const float* __restrict__ F EH_C_PARAM EH_
   constexpr int EW_TT = EW_WAVES_M * EW_WAVES_N * 64;
   constexpr int EW_TAIL_FULL = EH_TAIL_PER_GROUP / EW_TT;
 #pragma unroll 8
-  for (int q = 0; q < EW_TAIL_FULL; ++q) eh_tail_ns::eh_tail((int)g * EH_TAIL_PER_GROUP + tid + q * EW_TT EH_TAIL_ARGS);
-  if (EW_TAIL_FULL * EW_TT + tid < EH_TAIL_PER_GROUP) eh_tail_ns::eh_tail((int)g * EH_TAIL_PER_GROUP + EW_TAIL_FULL * EW_TT + tid EH_TAIL_ARGS);
+  for (int q = 0; q < EW_TAIL_FULL; ++q) eh_tail_ns::eh_tail((int)g, tid + q * EW_TT EH_TAIL_ARGS);
+  if (EW_TAIL_FULL * EW_TT + tid < EH_TAIL_PER_GROUP) eh_tail_ns::eh_tail((int)g, EW_TAIL_FULL * EW_TT + tid EH_TAIL_ARGS);
 #endif
 }
