@@ -725,11 +725,14 @@ struct SerialReduce {
     std::string t;
     for (const auto& p : k.params) {
       if (p.mut_ && (!with_out || (epi && !epi->store_c))) continue;
+      // what the epilogue reads as well comes in once, with the epilogue's parameters
+      if (!p.mut_ && with_out && epi && std::find(epi->bufs.begin(), epi->bufs.end(), p.name) != epi->bufs.end()) continue;
       t += (t.empty() ? "" : ", ") + std::string(p.mut_ ? "" : "const ") + ctype(p.dtype.elem()) + "* __restrict__ " + p.name;
       ls->arg_bufs.push_back(p.name);
     }
     if (!extra.empty()) t += (t.empty() ? "" : ", ") + extra;
-    if (with_out && epi) t += epi->params;        // (bound by finish_epilogue, after the reduce's own buffers)
+    // (bound by finish_epilogue, after the reduce's own buffers; the text starts with ", ")
+    if (with_out && epi) t += t.empty() && epi->params.size() > 2 ? epi->params.substr(2) : epi->params;
     return t;
   }
 

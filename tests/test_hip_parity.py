@@ -1632,6 +1632,27 @@ def test_random_graph_gradients_match_the_oracle(frontend, hip, seed):
         assert int((~close).sum()) <= allowed, desc
 
 
+@pytest.mark.parametrize("seed", sorted(set(range(22100, 22124)) | {22112, 22119}))
+def test_random_gradients_of_graphs_with_scans_selects_and_windows(frontend, hip, seed):
+    """The generator's other final stages (prefix scans, selects on comparisons, sliding windows,
+    batched contractions), differentiated where exact VJPs exist.  Seeds 22112 and 22119: a reduce
+    whose epilogue reads a buffer the reduce reads as well listed that buffer twice among its
+    kernel's parameters, and the launch did not compile."""
+    import graph_fuzz
+    shapes, fn, desc = graph_fuzz.build(seed, frontend, kinds=(8, 12))
+    rng = RNG(seed)
+    arrays = [rng.uniform(-1.5, 1.5, s).astype(np.float32) for s in shapes]
+    ref = _grads_on(frontend, "c-exactdiv", shapes, fn, arrays)
+    if ref is None:
+        pytest.skip("graph uses an op without an exact VJP: " + desc)
+    got = _grads_on(frontend, "hip", shapes, fn, arrays)
+    assert len(ref) == len(got), desc
+    for r, g in zip(ref, got):
+        assert r.shape == g.shape, desc
+        scale = max(1.0, float(np.abs(r).max()))
+        assert np.allclose(g, r, rtol=2e-4, atol=2e-5 * scale), desc
+
+
 def test_producers_read_through_another_index_space(frontend, hip):
     """A squared tensor, permuted, made contiguous and regrouped, feeding a kernel over the new
     axes: planned as one launch (the producers are evaluated where they are read), as three with
