@@ -233,7 +233,20 @@ struct StmtRenderer {
       case Op::Block: {
         std::string s;
         for (const auto& d : n.decls) s += ind() + ctype(d.second) + " " + d.first + ";\n";
-        for (const auto& a : n.args) s += stmt(*a);
+        for (const auto& a : n.args) {
+          // A block with declarations inside a block gets braces: the reference prints it without
+          // (src/backend/renderer.rs:604-624), and an unrolled loop around a reduction -- the same
+          // block with its accumulator several times over -- is then a redefinition in C.
+          if (a->op == Op::Block && !a->decls.empty()) {
+            s += ind() + "{\n";
+            ++level;
+            s += stmt(*a);
+            --level;
+            s += ind() + "}\n";
+          } else {
+            s += stmt(*a);
+          }
+        }
         return s;
       }
       case Op::Range: {
