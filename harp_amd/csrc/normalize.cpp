@@ -288,6 +288,32 @@ struct Normalizer {
   // in arithmetic progression (what full unrolling leaves, src/opt/ast/transforms.rs:238-361)
   // becomes `for u in 0..k { the p statements over u }`.  Variables the block declares move into
   // the loop body, which is sound when every repetition assigns them before it reads them.
+  // `n` with the loops named in `m` (and every use of their variables) renamed
+  static NodePtr rename_loops(const NodePtr& n, const std::map<std::string, std::string>& m) {
+    if (n->op == Op::Var) {
+      auto it = m.find(n->name);
+      return it == m.end() ? n : make_var(it->second);
+    }
+    bool changed = false;
+    std::vector<NodePtr> args;
+    args.reserve(n->args.size());
+    for (const auto& a : n->args) {
+      NodePtr r = rename_loops(a, m);
+      changed = changed || r != a;
+      args.push_back(std::move(r));
+    }
+    auto it = n->op == Op::Range ? m.find(n->name) : m.end();
+    if (!changed && it == m.end()) return n;
+    auto c = std::make_shared<Node>(*n);
+    c->args = std::move(args);
+    if (it != m.end()) c->name = it->second;
+    return c;
+  }
+  void rolled_loops_in(const Node& n, std::vector<std::string>* out) const {
+    if (n.op == Op::Range && rolled.count(n.name)) out->push_back(n.name);
+    for (const auto& a : n.args) rolled_loops_in(*a, out);
+  }
+
   NodePtr reroll(const std::vector<NodePtr>& stmts, const std::vector<std::pair<std::string, DType>>& decls) {
     const size_t n = stmts.size();
     // the smallest period of the statements' forms (failure function over their hashes); a
@@ -515,6 +541,25 @@ struct Normalizer {
   NodePtr block(std::vector<NodePtr> stmts, std::vector<std::pair<std::string, DType>> decls) {
     stmts.erase(std::remove_if(stmts.begin(), stmts.end(), [](const NodePtr& s) { return is_empty_stmt(*s); }),
                 stmts.end());
+    // Loops that an inner roll made carry fresh names, one per repetition of an enclosing unrolled
+    // loop (or of a loop and its remainder): each statement's are renamed by their order in it, so
+    // that the repetitions compare equal below.
+    if (stmts.size() >= 2) {
+      const int id = fresh++;
+      for (auto& st : stmts) {
+        std::vector<std::string> inner;
+        rolled_loops_in(*st, &inner);
+        if (inner.empty()) continue;
+        std::map<std::string, std::string> m;
+        for (size_t k = 0; k < inner.size(); ++k) {
+          const std::string to = "eh_c" + std::to_string(id) + "_" + std::to_string(k);
+          if (!m.emplace(inner[k], to).second) { m.clear(); break; }     // (a name bound twice in one statement: left alone)
+          int_vars.insert(to);
+          rolled.insert(to);
+        }
+        if (!m.empty()) st = rename_loops(st, m);
+      }
+    }
     // neighbouring loops with the same body over adjoining ranges are one loop; so are two whose
     // ranges adjoin once the second one's variable is shifted (a remainder loop that was moved to
     // start at 0, its offset now inside its body): bodies are compared with their integer
@@ -569,6 +614,22 @@ struct Normalizer {
     }
   }
 
+  // `for v in [0, e) { if (v < c) S }` is `for v in [0, min(e, c)) S`: what is left of a guarded
+  // tiling once its tile loops were unrolled and rolled back into one loop over the padded extent.
+  NodePtr unguard(const NodePtr& loop) const {
+    int64_t s = 0, step = 0, e = 0, c = 0;
+    if (loop->op != Op::Range || !int_const(*loop->args[0], &s) || !int_const(*loop->args[1], &step) ||
+        !int_const(*loop->args[2], &e) || s != 0 || step != 1)
+      return loop;
+    const Node* body = loop->args[3].get();
+    while (body->op == Op::Block && body->args.size() == 1 && body->decls.empty()) body = body->args[0].get();
+    if (body->op != Op::If || body->args.size() != 2) return loop;
+    const Node& cond = *body->args[0];
+    if (cond.op != Op::Lt || cond.args[0]->op != Op::Var || cond.args[0]->name != loop->name || !int_const(*cond.args[1], &c)) return loop;
+    if (assigns(*body->args[1], loop->name)) return loop;
+    return make_loop(*loop, loop->name, make_i64(0), make_i64(1), make_i64(std::max<int64_t>(0, std::min(e, c))), body->args[1]);
+  }
+
   // ---- second pass: what the first left behind ------------------------------------------------
 
   // Integer block variables assigned once from an affine expression are substituted into the
@@ -614,9 +675,9 @@ struct Normalizer {
           a.c = s;
           a.coef[n->name] = step;
           body = substitute_vars(body, {{n->name, affine_to_node(a)}});
-          return make_loop(*n, n->name, make_i64(0), make_i64(1), make_i64(count), settle(body));
+          return unguard(make_loop(*n, n->name, make_i64(0), make_i64(1), make_i64(count), settle(body)));
         }
-        return make_loop(*n, n->name, n->args[0], n->args[1], n->args[2], settle(body));
+        return unguard(make_loop(*n, n->name, n->args[0], n->args[1], n->args[2], settle(body)));
       }
       case Op::If: {
         std::vector<NodePtr> args = {n->args[0]};
